@@ -1,0 +1,235 @@
+/*
+ * torsh_hipq - C-ABI of the MI355X (gfx950) quantized-inference kernels that
+ * sit behind ToRSh's quantization API.
+ *
+ * Every entry point returns an int32_t status using the numbering of the
+ * reference's own C error enum (crates/torsh-core/src/ffi.rs:196-220) and
+ * records a thread-local message readable through hipq_get_last_error(), the
+ * convention of crates/torsh-ffi/src/c_api/utils.rs:162-190.  Pointers are
+ * null-checked first (crates/torsh-ffi/src/c_api/neural.rs:106-113).
+ *
+ * Unless a parameter is documented as "host", data pointers are DEVICE
+ * pointers valid on the context's GPU.  Work is enqueued on the context's HIP
+ * stream and is asynchronous; hipq_ctx_synchronize() waits for it.  Inputs are
+ * only read, outputs are caller-allocated, nothing is retained across calls
+ * (the reference's functions borrow inputs and return fresh outputs,
+ * crates/torsh-tensor/src/advanced_ops.rs:624-629).  A context must not be
+ * used from two threads at once; distinct contexts are independent.
+ *
+ * Layouts: matrices are row-major and dense.  Linear weights are [N,K]
+ * (output channel major, K contiguous) - the transpose of the [K,N] operand of
+ * crates/torsh-backend/src/quantization/specialized.rs:191-193, same integers.
+ * Conv tensors are NCHW / [OC,IC,KH,KW].
+ */
+#ifndef TORSH_HIPQ_H
+#define TORSH_HIPQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPQ_API __attribute__((visibility("default")))
+
+typedef struct hipq_ctx hipq_ctx;
+
+/* crates/torsh-core/src/ffi.rs:196-220 */
+enum {
+    HIPQ_SUCCESS = 0,
+    HIPQ_INVALID_ARGUMENT = 1,
+    HIPQ_SHAPE_ERROR = 2,
+    HIPQ_DIMENSION_MISMATCH = 3,
+    HIPQ_DEVICE_ERROR = 4,
+    HIPQ_ALLOCATION_ERROR = 5,
+    HIPQ_SYNCHRONIZATION_ERROR = 6,
+    HIPQ_UNKNOWN_ERROR = 7
+};
+
+/* `mode` bit field of the quantizing entry points.
+ * Rounding: the reference rounds with Rust f32::round, half away from zero
+ * (crates/torsh-quantization/src/simd_ops.rs:44); half-to-even is offered as a
+ * variant.  Form: multiply by 1/scale (simd_ops.rs:36-46, the len > 64 branch
+ * of algorithms.rs:292) or divide by scale (algorithms.rs:302-305, 230-233). */
+enum {
+    HIPQ_ROUND_HALF_AWAY = 0,
+    HIPQ_ROUND_HALF_EVEN = 1,
+    HIPQ_FORM_MUL_INV = 0,
+    HIPQ_FORM_DIV = 2
+};
+
+/* Quantized integer types, ranges per get_dtype_range
+ * (crates/torsh-quantization/src/algorithms.rs:425-433). */
+enum { HIPQ_DTYPE_I8 = 0, HIPQ_DTYPE_U8 = 1 };
+
+/* Which reference formula turns (min,max) into (scale, zero_point). */
+enum {
+    /* calculate_symmetric_quantization_params, algorithms.rs:397-422 */
+    HIPQ_PARAMS_SYMMETRIC = 0,
+    /* calculate_affine_quantization_params, algorithms.rs:358-394 */
+    HIPQ_PARAMS_AFFINE = 1,
+    /* torsh-backend from_statistics, symmetric: params.rs:323-340 */
+    HIPQ_PARAMS_BACKEND_SYMMETRIC = 2,
+    /* torsh-backend from_statistics, asymmetric: params.rs:343-363 */
+    HIPQ_PARAMS_BACKEND_ASYMMETRIC = 3
+};
+
+/* Device-resident quantization parameters, written by the kernels that derive
+ * them so that a dynamic quantize never round-trips to the host.  `status` is
+ * HIPQ_SUCCESS or HIPQ_INVALID_ARGUMENT (non-finite or inverted range, where
+ * the reference returns InvalidArgument, algorithms.rs:363-373,403-407). */
+typedef struct hipq_qparams {
+    float scale;
+    int32_t zero_point;
+    float min_val;
+    float max_val;
+    int32_t status;
+    int32_t reserved[3];
+} hipq_qparams;
+
+/* ---- library, context, errors ---------------------------------------- */
+HIPQ_API const char *hipq_version(void);
+/* torsh_get_last_error / torsh_clear_last_error / torsh_has_error,
+ * crates/torsh-ffi/src/c_api/utils.rs:162-190. */
+HIPQ_API const char *hipq_get_last_error(void);
+HIPQ_API void hipq_clear_last_error(void);
+HIPQ_API int32_t hipq_has_error(void);
+
+/* Creates a context on `device` with its own non-blocking stream. */
+HIPQ_API int32_t hipq_ctx_create(int32_t device, hipq_ctx **out_ctx);
+/* Creates a context that enqueues on a caller-owned hipStream_t (0 = the
+ * legacy default stream). */
+HIPQ_API int32_t hipq_ctx_create_on_stream(int32_t device, void *hip_stream, hipq_ctx **out_ctx);
+HIPQ_API int32_t hipq_ctx_destroy(hipq_ctx *ctx);
+HIPQ_API int32_t hipq_ctx_synchronize(hipq_ctx *ctx);
+HIPQ_API void *hipq_ctx_stream(hipq_ctx *ctx);
+
+/* Device-buffer helpers for callers whose tensors live on the host (the
+ * reference's Tensor has no ROCm device, crates/torsh-core/src/device/types.rs:39-48). */
+HIPQ_API int32_t hipq_device_malloc(hipq_ctx *ctx, size_t bytes, void **out_ptr);
+HIPQ_API int32_t hipq_device_free(hipq_ctx *ctx, void *ptr);
+HIPQ_API int32_t hipq_memcpy_h2d(hipq_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+HIPQ_API int32_t hipq_memcpy_d2h(hipq_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+
+/* ---- range reduction and parameters ---------------------------------- */
+/* find_min_max_simd, crates/torsh-quantization/src/simd_ops.rs:84-121.
+ * out_minmax: 2 floats {min, max}; NaNs are ignored as f32::min/max do.
+ * n == 0 is InvalidArgument as in the reference. */
+HIPQ_API int32_t hipq_minmax_f32(hipq_ctx *ctx, const float *x, size_t n, float *out_minmax);
+/* max |x| (the symmetric-scheme reduction: max(|min|,|max|), algorithms.rs:410). */
+HIPQ_API int32_t hipq_absmax_f32(hipq_ctx *ctx, const float *x, size_t n, float *out_absmax);
+/* (min,max) -> (scale, zero_point) on the device; `flavor` is HIPQ_PARAMS_*.
+ * qmin/qmax: -128/127 for I8, 0/255 for U8. */
+HIPQ_API int32_t hipq_qparams_from_minmax(hipq_ctx *ctx, const float *minmax, int32_t flavor, int32_t qmin,
+                                          int32_t qmax, hipq_qparams *out_params);
+
+/* ---- per-tensor quantize / dequantize -------------------------------- */
+/* quantize_to_int8_simd / quantize_per_tensor_affine_i8,
+ * crates/torsh-quantization/src/simd_ops.rs:196-227, algorithms.rs:245-274:
+ * q = clamp(round(x * (1/scale) | x / scale) + zp, -128, 127) as i8.
+ * scale <= 0 is InvalidArgument (algorithms.rs:284-288). */
+HIPQ_API int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                                 int32_t zero_point, int32_t mode, int8_t *out);
+/* CpuQuantizationOps::quantize_f32 for UInt8,
+ * crates/torsh-backend/src/quantization/ops.rs:185-195,295-364:
+ * q = clamp(round(x / scale) + zp, 0, 255). */
+HIPQ_API int32_t hipq_quantize_per_tensor_f32_u8(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                                 int32_t zero_point, int32_t mode, uint8_t *out);
+/* quantize_per_tensor_affine_simd, simd_ops.rs:18-49: same arithmetic, result
+ * kept in an f32 carrier clamped to [qmin,qmax] (NaN stays NaN), the form
+ * torsh-quantization hands back (algorithms.rs:291,304-312). */
+HIPQ_API int32_t hipq_quantize_per_tensor_f32_carrier(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                                      int32_t zero_point, int32_t mode, int32_t qmin,
+                                                      int32_t qmax, float *out);
+/* As hipq_quantize_per_tensor_f32_i8 / _u8 with scale and zero point read from
+ * a device hipq_qparams (no host round trip). */
+HIPQ_API int32_t hipq_quantize_with_params_f32_i8(hipq_ctx *ctx, const float *x, size_t n,
+                                                  const hipq_qparams *params, int32_t mode, int8_t *out);
+HIPQ_API int32_t hipq_quantize_with_params_f32_u8(hipq_ctx *ctx, const float *x, size_t n,
+                                                  const hipq_qparams *params, int32_t mode, uint8_t *out);
+/* quantize_tensor_auto, algorithms.rs:85-123: min/max -> params (`flavor`) ->
+ * quantize, all on the device.  dtype is HIPQ_DTYPE_I8 (out is int8_t*) or
+ * HIPQ_DTYPE_U8 (out is uint8_t*).  out_params receives the parameters. */
+HIPQ_API int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor,
+                                                      int32_t dtype, int32_t mode, void *out,
+                                                      hipq_qparams *out_params);
+/* dequantize_per_tensor_affine, algorithms.rs:318-355: y = (q - zp) * scale. */
+HIPQ_API int32_t hipq_dequantize_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t n, float scale, int32_t zero_point,
+                                        float *out);
+HIPQ_API int32_t hipq_dequantize_u8_f32(hipq_ctx *ctx, const uint8_t *q, size_t n, float scale,
+                                        int32_t zero_point, float *out);
+/* The same on the f32 carrier form (simd_ops.rs:52-81). */
+HIPQ_API int32_t hipq_dequantize_carrier_f32(hipq_ctx *ctx, const float *q, size_t n, float scale,
+                                             int32_t zero_point, float *out);
+/* Scale / zero point from a device hipq_qparams. */
+HIPQ_API int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t n,
+                                                    const hipq_qparams *params, float *out);
+
+/* ---- per-channel quantize / dequantize ------------------------------- */
+/* quantize_per_channel_auto with axis 0 on a [rows, cols] view
+ * (algorithms.rs:126-242): per row min/max -> params (`flavor`
+ * HIPQ_PARAMS_SYMMETRIC or HIPQ_PARAMS_AFFINE) -> clamp(round(x / s) + zp,
+ * qmin, qmax).  Used per output channel for weights and per token for
+ * activations.  out_scales[rows], out_zero_points[rows] (may be NULL).
+ * out_status: device int32, set non-zero if any row had a non-finite range. */
+HIPQ_API int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
+                                              int32_t flavor, int32_t mode, int8_t *out, float *out_scales,
+                                              int32_t *out_zero_points, int32_t *out_status);
+/* quantize_per_channel_auto for any axis of a dense tensor viewed as
+ * [outer, channels, inner] (algorithms.rs:126-242). */
+HIPQ_API int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer,
+                                                       size_t channels, size_t inner, int32_t flavor,
+                                                       int32_t mode, int8_t *out, float *out_scales,
+                                                       int32_t *out_zero_points, int32_t *out_status);
+/* quantize_per_channel_affine, explicit parameters,
+ * crates/torsh-quantization/src/quantize.rs:287-331 (HIPQ_FORM_DIV) and
+ * quantize_per_channel_simd, simd_ops.rs:124-169 (HIPQ_FORM_MUL_INV, inner
+ * contiguous). */
+HIPQ_API int32_t hipq_quantize_per_channel_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels,
+                                                  size_t inner, const float *scales,
+                                                  const int32_t *zero_points, int32_t mode, int8_t *out);
+/* dequantize_per_channel_affine, crates/torsh-quantization/src/dequantize.rs:46-89:
+ * y = scale[c] * (q - zp[c]). */
+HIPQ_API int32_t hipq_dequantize_per_channel_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t outer,
+                                                    size_t channels, size_t inner, const float *scales,
+                                                    const int32_t *zero_points, float *out);
+
+/* ---- integer GEMM and the quantized Linear forward ------------------- */
+/* vnni_matmul_kernel, crates/torsh-backend/src/quantization/specialized.rs:175-201:
+ * acc[m,n] = sum_k a[m,k] * w[n,k] in int32 (raw accumulators, no clamp). */
+HIPQ_API int32_t hipq_gemm_i8_i32(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size_t m, size_t n, size_t k,
+                                  int32_t *out);
+/* Quantized Linear with dequantizing epilogue:
+ *   out[m,n] = (acc as f32) * (s_a * s_w[n]) + bias[n]
+ * (acc*(s_in*s_w): crates/torsh-backend/src/quantization/operations.rs:669,722;
+ * f32 bias add: crates/torsh-backend/src/quantization/ops.rs:561).
+ * a_scale: device, 1 float (per tensor) or m floats (per token) as
+ * a_scale_per_row says; w_scales: device [n]; bias: device [n] or NULL. */
+HIPQ_API int32_t hipq_linear_i8_f32(hipq_ctx *ctx, const int8_t *a, const float *a_scale,
+                                    int32_t a_scale_per_row, const int8_t *w, const float *w_scales,
+                                    const float *bias, size_t m, size_t n, size_t k, float *out);
+/* Same accumulators, requantizing epilogue (tail of operations.rs:716-724 with
+ * a supplied output scale): q = clamp(round(v / s_out) + zp_out, -128, 127). */
+HIPQ_API int32_t hipq_linear_i8_i8(hipq_ctx *ctx, const int8_t *a, const float *a_scale, int32_t a_scale_per_row,
+                                   const int8_t *w, const float *w_scales, const float *bias, size_t m, size_t n,
+                                   size_t k, float out_scale, int32_t out_zero_point, int32_t mode,
+                                   int8_t *out);
+/* Stand-alone requantize of int32 accumulators [rows, cols]; the weight
+ * channel is the column. */
+HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_t rows, size_t cols,
+                                        const float *a_scale, int32_t a_scale_per_row, const float *w_scales,
+                                        const float *bias, float out_scale, int32_t out_zero_point,
+                                        int32_t mode, int8_t *out);
+/* Whole forward of a quantized Linear on fp32 activations: dynamic activation
+ * quantization (per tensor: algorithms.rs:85-123; per token: algorithms.rs:126-242
+ * on axis 0), int8 GEMM, dequantizing epilogue.  Uses context-owned scratch
+ * for the int8 activations and their scales. */
+HIPQ_API int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w,
+                                         const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
+                                         int32_t mode, float *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORSH_HIPQ_H */

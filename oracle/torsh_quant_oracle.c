@@ -170,7 +170,7 @@ int tq_calculate_affine_params(float mn, float mx, int dtype, float *scale, int3
     float s = (mx - mn) / (qmax - qmin);
     float zp_fp = qmin - mn / s;
     *scale = s;
-    *zp = f32_as_i32(clampf_rust(rnd(zp_fp), qmin, qmax));
+    *zp = f32_as_i32(clampf_rust(roundf(zp_fp), qmin, qmax)); /* always f32::round */
     return TQ_OK;
 }
 
@@ -438,7 +438,7 @@ int tq_backend_params_asymmetric(float mn, float mx, int32_t qmin, int32_t qmax,
     float s = (mx - mn) / (fqmax - fqmin);
     float z = fqmin - mn / s;
     *scale = s;
-    *zp = f32_as_i32(clampf_rust(rnd(z), fqmin, fqmax));
+    *zp = f32_as_i32(clampf_rust(roundf(z), fqmin, fqmax)); /* always f32::round */
     return TQ_OK;
 }
 

@@ -27,3 +27,23 @@ def golden():
 
     with open(os.path.join(ROOT, "tests", "golden", "reference_vectors.json")) as f:
         return json.load(f)
+
+
+@pytest.fixture(scope="session")
+def hipq():
+    from torsh_amd import hipq as mod
+
+    mod.load()
+    return mod
+
+
+@pytest.fixture(scope="session")
+def ctx(hipq):
+    import torch
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    c = hipq.Context(0)
+    yield c
+    torch.cuda.synchronize()
+    c.close()

@@ -1,0 +1,57 @@
+"""CPU-side checks of the C-ABI: the library loads and exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "torsh_hipq.h")).read()
+    return sorted(set(re.findall(r"HIPQ_API[^;()]*?\b(hipq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_entry_points():
+    names = _declared_symbols()
+    assert "hipq_ctx_create" in names and "hipq_linear_i8_f32" in names and len(names) >= 30
+
+
+def test_library_exports_every_declared_symbol():
+    from torsh_amd import hipq
+
+    assert os.path.exists(hipq.lib_path()), "build with `python -m torsh_amd.build`"
+    lib = ctypes.CDLL(hipq.lib_path())
+    missing = [n for n in _declared_symbols() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_python_binding_covers_the_header():
+    from torsh_amd import hipq
+
+    assert sorted(hipq.exported_symbols()) == _declared_symbols()
+
+
+def test_error_string_api_without_gpu():
+    from torsh_amd import hipq
+
+    lib = hipq.load()
+    lib.hipq_clear_last_error()
+    assert lib.hipq_has_error() == 0
+    assert lib.hipq_version().startswith(b"torsh_hipq")
+    # null out-pointer is rejected before any device call
+    rc = lib.hipq_ctx_create(0, None)
+    assert rc == hipq.INVALID_ARGUMENT
+    assert lib.hipq_has_error() == 1 and b"null pointer" in lib.hipq_get_last_error()
+    lib.hipq_clear_last_error()
+    assert lib.hipq_has_error() == 0
+
+
+def test_no_silent_fallback_when_library_missing(monkeypatch):
+    from torsh_amd import hipq
+
+    monkeypatch.setattr(hipq, "_lib", None)
+    monkeypatch.setattr(hipq, "_LIB_PATH", "/nonexistent/libtorsh_hipq.so")
+    with pytest.raises(FileNotFoundError):
+        hipq.load()

@@ -1,0 +1,282 @@
+"""Parity of the HBM-streaming kernels (through the C-ABI) with the CPU oracle: bit-exact."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def normal(seed, shape, std=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * std).astype(np.float32)
+
+
+def test_golden_vectors_through_the_cabi(ctx, hipq, golden):
+    for case in golden["quantize_per_tensor"] + golden["proptest_regressions"]:
+        x = np.array(case["x"], np.float32)
+        want = np.array(case["q"], np.int8)[: x.size]
+        for mode in (hipq.FORM_MUL_INV, hipq.FORM_DIV):
+            got = host(ctx.quantize_per_tensor_i8(dev(x), case["scale"], case["zp"], mode))
+            np.testing.assert_array_equal(got, want, case["src"])
+    for case in golden["dequantize_per_tensor"]:
+        q = np.array(case["q"], np.float32)
+        got = host(ctx.dequantize(dev(q), case["scale"], case["zp"]))
+        np.testing.assert_allclose(got, np.array(case["y"], np.float32), atol=case["atol"], rtol=0)
+    for case in golden["min_max"]:
+        got = host(ctx.minmax(dev(np.array(case["x"], np.float32))))
+        assert got[0] == np.float32(case["min"]) and got[1] == np.float32(case["max"])
+
+
+def test_error_cases_match_the_reference(ctx, hipq):
+    x = dev(np.array([1.0, 2.0], np.float32))
+    for bad in (-1.0, 0.0):
+        with pytest.raises(hipq.HipqError) as e:
+            ctx.quantize_per_tensor_i8(x, bad, 0)
+        assert e.value.code == hipq.INVALID_ARGUMENT and "Scale must be positive" in e.value.message
+        with pytest.raises(hipq.HipqError):
+            ctx.dequantize(x, bad, 0)
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.minmax(torch.empty(0, dtype=torch.float32, device="cuda"))
+    assert e.value.code == hipq.INVALID_ARGUMENT
+    with pytest.raises(hipq.HipqError):
+        ctx.quantize_dynamic_per_tensor(torch.empty(0, dtype=torch.float32, device="cuda"))
+    with pytest.raises(hipq.HipqError):
+        ctx.quantize_per_tensor_i8(x, 1.0, 0, mode=64)
+    # empty input with a valid scale is a no-op, as the reference's loop over zero elements
+    ctx.quantize_per_tensor_i8(torch.empty(0, dtype=torch.float32, device="cuda"), 1.0, 0)
+
+
+@pytest.mark.parametrize("n", [1, 3, 63, 64, 65, 1000, 4096, 4097, 65536 + 5, 1 << 20])
+def test_minmax_absmax(ctx, oracle, n):
+    x = normal(n, n) * 3
+    got = host(ctx.minmax(dev(x)))
+    mn, mx = oracle.find_min_max(x)
+    assert (got[0], got[1]) == (np.float32(mn), np.float32(mx))
+    assert host(ctx.absmax(dev(x)))[0] == np.float32(max(abs(mn), abs(mx)))
+
+
+def test_minmax_ignores_nan_and_handles_unaligned(ctx, oracle):
+    x = normal(7, 5000)
+    x[17] = np.nan
+    x[4000] = np.nan
+    t = dev(x)
+    got = host(ctx.minmax(t))
+    assert tuple(got) == tuple(np.float32(v) for v in oracle.find_min_max(x))
+    got = host(ctx.minmax(t[1:]))  # base pointer no longer 16-byte aligned
+    assert tuple(got) == tuple(np.float32(v) for v in oracle.find_min_max(x[1:]))
+
+
+@pytest.mark.parametrize("n", [1, 5, 64, 65, 4095, 4096, 100_003, 1 << 20])
+@pytest.mark.parametrize("mode_name", ["mul", "div", "mul_even", "div_even"])
+def test_quantize_per_tensor_bit_exact(ctx, hipq, oracle, n, mode_name):
+    x = normal(100 + n, n) * 2
+    # plant exact ties and saturating values
+    x[: min(n, 6)] = np.array([0.5, -0.5, 1.5, -2.5, 1000.0, -1000.0], np.float32)[: min(n, 6)]
+    scale, zp = np.float32(0.03125 if n % 2 else 0.0173), 3
+    x[: min(n, 4)] *= scale  # ties in units of the scale when scale is a power of two
+    mode = (hipq.FORM_DIV if "div" in mode_name else 0) | (hipq.ROUND_HALF_EVEN if "even" in mode_name else 0)
+    oracle.set_round_mode(1 if "even" in mode_name else 0)
+    try:
+        if "div" in mode_name:
+            want = oracle.quantize_per_tensor_affine_i8(x, scale, zp)
+        else:
+            want = oracle.quantize_to_int8_simd(x, scale, zp)
+        want_carrier = oracle.quantize_per_tensor_affine_simd(x, scale, zp) if "div" not in mode_name else None
+    finally:
+        oracle.set_round_mode(0)
+    got = host(ctx.quantize_per_tensor_i8(dev(x), scale, zp, mode))
+    np.testing.assert_array_equal(got, want)
+    if want_carrier is not None:
+        got_c = host(ctx.quantize_per_tensor_carrier(dev(x), scale, zp, mode))
+        np.testing.assert_array_equal(got_c, want_carrier)
+
+
+def test_quantize_ties_follow_the_rounding_mode(ctx, hipq):
+    x = dev(np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, -128.5], np.float32))
+    away = host(ctx.quantize_per_tensor_i8(x, 1.0, 0, hipq.ROUND_HALF_AWAY))
+    even = host(ctx.quantize_per_tensor_i8(x, 1.0, 0, hipq.ROUND_HALF_EVEN))
+    np.testing.assert_array_equal(away, [1, 2, 3, -1, -2, -3, 127, 127, -128])
+    np.testing.assert_array_equal(even, [0, 2, 2, 0, -2, -2, 126, 127, -128])
+
+
+def test_quantize_nan_inf(ctx, oracle):
+    x = np.array([np.nan, np.inf, -np.inf, 1.0, -3.0] * 30, np.float32)
+    got = host(ctx.quantize_per_tensor_i8(dev(x), 0.5, 0))
+    np.testing.assert_array_equal(got, oracle.quantize_to_int8_simd(x, 0.5, 0))
+    car = host(ctx.quantize_per_tensor_carrier(dev(x), 0.5, 0))
+    want = oracle.quantize_per_tensor_affine_simd(x, 0.5, 0)
+    np.testing.assert_array_equal(np.isnan(car), np.isnan(want))
+    np.testing.assert_array_equal(car[~np.isnan(car)], want[~np.isnan(want)])
+
+
+def test_quantize_unaligned_views(ctx, oracle):
+    x = normal(5, 10_007)
+    t = dev(x)
+    out = torch.empty(10_007 + 8, dtype=torch.int8, device="cuda")
+    for off_in, off_out in [(1, 0), (0, 1), (3, 2), (2, 3)]:
+        ctx.quantize_per_tensor_i8(t[off_in:], 0.02, -1, out=out[off_out: off_out + x.size - off_in])
+        got = host(out[off_out: off_out + x.size - off_in])
+        np.testing.assert_array_equal(got, oracle.quantize_to_int8_simd(x[off_in:], 0.02, -1))
+
+
+@pytest.mark.parametrize("n", [2, 64, 65, 4096, 1 << 20, (1 << 20) + 7])
+def test_u8_quantize_backend_flavour(ctx, hipq, oracle, n):
+    x = np.maximum(normal(n, n), 0)
+    mn, mx = oracle.find_min_max(x)
+    scale, zp = oracle.backend_params_asymmetric(mn, mx, 0, 255)
+    want = oracle.backend_quantize_f32(x, scale, zp, 0, 255)
+    got = host(ctx.quantize_per_tensor_u8(dev(x), scale, zp, hipq.FORM_DIV))
+    np.testing.assert_array_equal(got, want)
+    # fully on-device: min/max -> asymmetric params -> quantize
+    q, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_BACKEND_ASYMMETRIC, hipq.DTYPE_U8, hipq.FORM_DIV)
+    p = ctx.read_qparams(params)
+    assert p.status == 0 and p.scale == np.float32(scale) and p.zero_point == zp
+    np.testing.assert_array_equal(host(q), want)
+    deq = host(ctx.dequantize(q, scale, zp))
+    np.testing.assert_array_equal(deq, oracle.backend_dequantize_f32(want, scale, zp, False))
+
+
+@pytest.mark.parametrize("flavor_name", ["symmetric", "affine", "backend_symmetric", "backend_asymmetric"])
+def test_qparams_from_minmax(ctx, hipq, oracle, flavor_name):
+    cases = [(-1.0, 1.0), (0.0, 0.0), (1.0, 1.0), (-3.5, 0.25), (0.0, 6.0), (1.0, 2.0), (-1e-9, 1e-9), (2.0, 1.0),
+             (float("nan"), 1.0), (0.0, float("inf"))]
+    flavor = {"symmetric": hipq.PARAMS_SYMMETRIC, "affine": hipq.PARAMS_AFFINE,
+              "backend_symmetric": hipq.PARAMS_BACKEND_SYMMETRIC,
+              "backend_asymmetric": hipq.PARAMS_BACKEND_ASYMMETRIC}[flavor_name]
+    for qmin, qmax, dt in ((-128, 127, 0), (0, 255, 1)):
+        for mn, mx in cases:
+            p = ctx.read_qparams(ctx.qparams_from_minmax(dev(np.array([mn, mx], np.float32)), flavor, qmin, qmax))
+            try:
+                if flavor_name == "symmetric":
+                    want = oracle.calculate_symmetric_params(mn, mx, dt)
+                elif flavor_name == "affine":
+                    want = oracle.calculate_affine_params(mn, mx, dt)
+                elif flavor_name == "backend_symmetric":
+                    want = oracle.backend_params_symmetric(mn, mx, qmin, qmax)
+                else:
+                    want = oracle.backend_params_asymmetric(mn, mx, qmin, qmax)
+            except oracle.OracleError:
+                assert p.status == hipq.INVALID_ARGUMENT, (flavor_name, mn, mx)
+                continue
+            assert p.status == 0 and (p.scale, p.zero_point) == (np.float32(want[0]), want[1]), (flavor_name, mn, mx)
+
+
+@pytest.mark.parametrize("shape", [(4, 4), (256, 256), (1000, 37), (1024, 1024)])
+def test_config1_round_trip(ctx, hipq, oracle, shape):
+    """Symmetric per-tensor int8 quantize -> dequantize of N(0,1) data (BASELINE config 1, small sizes)."""
+    x = normal(1, shape)
+    want_q, scale, zp = oracle.quantize_tensor_auto(x, 0, oracle.PER_TENSOR_SYMMETRIC)
+    want_y = oracle.dequantize_per_tensor_affine(want_q, scale, zp)
+    mode = hipq.FORM_MUL_INV if x.size > 64 else hipq.FORM_DIV  # the reference's len > 64 branch
+    q, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_SYMMETRIC, hipq.DTYPE_I8, mode)
+    p = ctx.read_qparams(params)
+    assert p.status == 0 and p.scale == np.float32(scale) and p.zero_point == zp
+    np.testing.assert_array_equal(host(q), want_q.astype(np.int8))
+    y = host(ctx.dequantize_with_params(q, params))
+    np.testing.assert_array_equal(y, want_y)  # (q - 0) * scale has one rounding: bit-exact
+    np.testing.assert_allclose(y, want_y, rtol=1e-5, atol=0)
+    assert np.abs(y - x).max() <= 0.5 * scale * (1 + 1e-4)
+
+
+def test_config1_full_size_properties(ctx, hipq):
+    """Full BASELINE size [4096,4096]: size-independent properties instead of a CPU pass."""
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(4096, 4096, generator=g, device="cuda", dtype=torch.float32)
+    q, params = ctx.quantize_dynamic_per_tensor(x, hipq.PARAMS_SYMMETRIC, hipq.DTYPE_I8, hipq.FORM_MUL_INV)
+    p = ctx.read_qparams(params)
+    absmax = x.abs().max().item()
+    assert p.status == 0 and p.zero_point == 0
+    assert p.scale == np.float32(absmax) / np.float32(127.0)
+    assert (p.min_val, p.max_val) == (x.min().item(), x.max().item())
+    assert int(q.abs().max().item()) == 127 and int(q.min().item()) >= -127
+    y = ctx.dequantize_with_params(q, params)
+    torch.cuda.synchronize()
+    assert (y - x).abs().max().item() <= 0.5 * p.scale * (1 + 1e-4)
+    # idempotence: quantizing the dequantized tensor with the same scale returns the same codes
+    q2 = ctx.quantize_per_tensor_i8(y, p.scale, 0, hipq.FORM_MUL_INV)
+    torch.cuda.synchronize()
+    assert torch.equal(q2, q)
+    # checksum against an independent torch formulation of the same f32 arithmetic
+    inv = torch.tensor(1.0, device="cuda") / torch.tensor(p.scale, device="cuda")
+    t = x * inv
+    ref = torch.clamp(torch.sign(t) * torch.floor(t.abs().double() + 0.5).float(), -128, 127).to(torch.int8)
+    assert torch.equal(q, ref)
+
+
+def test_non_finite_range_sets_status_and_skips(ctx, hipq):
+    x = torch.tensor([1.0, float("inf"), 2.0] * 50, device="cuda")
+    out = torch.full((150,), 77, dtype=torch.int8, device="cuda")
+    _, params = ctx.quantize_dynamic_per_tensor(x, out=out)
+    assert ctx.read_qparams(params).status == hipq.INVALID_ARGUMENT
+    assert bool((out == 77).all())
+
+
+@pytest.mark.parametrize("shape", [(1, 8), (3, 33), (16, 4096), (5, 1024), (7, 1025), (4, 4100), (2, 20000), (64, 768)])
+@pytest.mark.parametrize("flavor_name", ["symmetric", "affine"])
+def test_per_row_quantize(ctx, hipq, oracle, shape, flavor_name):
+    x = normal(shape[0] * 7 + shape[1], shape)
+    if shape[0] > 2:
+        x[2] = 0.0  # degenerate row -> (1.0, 0) / (1.0, -128)
+    flavor = hipq.PARAMS_SYMMETRIC if flavor_name == "symmetric" else hipq.PARAMS_AFFINE
+    scheme = oracle.PER_CHANNEL_SYMMETRIC if flavor_name == "symmetric" else oracle.PER_CHANNEL_AFFINE
+    want_q, want_s, want_z = oracle.quantize_per_channel_auto(x, 0, 0, scheme)
+    q, s, z, status = ctx.quantize_per_row(dev(x), flavor)
+    assert host(status)[0] == 0
+    np.testing.assert_array_equal(host(s), want_s)
+    np.testing.assert_array_equal(host(z), want_z)
+    np.testing.assert_array_equal(host(q), want_q.astype(np.int8))
+
+
+def test_per_row_status_on_non_finite_row(ctx, hipq):
+    x = normal(3, (4, 128))
+    x[1, 5] = np.inf
+    _, _, _, status = ctx.quantize_per_row(dev(x))
+    assert host(status)[0] == hipq.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_per_channel_any_axis(ctx, hipq, oracle, axis):
+    x = normal(21 + axis, (5, 6, 7))
+    want_q, want_s, want_z = oracle.quantize_per_channel_auto(x, axis, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    q, s, z, status = ctx.quantize_per_channel_auto(dev(x), axis)
+    assert host(status)[0] == 0
+    np.testing.assert_array_equal(host(s), want_s)
+    np.testing.assert_array_equal(host(q), want_q.astype(np.int8))
+    # explicit parameters, both forms, and per-channel dequantize
+    zps = np.arange(x.shape[axis], dtype=np.int32) - 2
+    got = host(ctx.quantize_per_channel(dev(x), dev(want_s), dev(zps), axis, hipq.FORM_DIV))
+    np.testing.assert_array_equal(got, oracle.quantize_per_channel_affine(x, want_s, zps, axis).astype(np.int8))
+    deq = host(ctx.dequantize_per_channel(dev(got), dev(want_s), dev(zps), axis))
+    np.testing.assert_array_equal(deq, oracle.dequantize_per_channel_affine(got.astype(np.float32), want_s, zps, axis))
+    if axis == 0:
+        got = host(ctx.quantize_per_channel(dev(x), dev(want_s), dev(zps), 0, hipq.FORM_MUL_INV))
+        want = oracle.quantize_per_channel_simd(x.reshape(5, -1), want_s, zps, 42).reshape(x.shape)
+        np.testing.assert_array_equal(got, want.astype(np.int8))
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (5, 9), (64, 256), (100, 333)])
+def test_requantize(ctx, hipq, oracle, shape):
+    rng = np.random.default_rng(shape[1])
+    acc = rng.integers(-3_000_000, 3_000_000, size=shape, dtype=np.int32)
+    sw = rng.uniform(1e-4, 1e-3, shape[1]).astype(np.float32)
+    bias = (rng.standard_normal(shape[1]) * 0.01).astype(np.float32)
+    for sa in (np.array([0.02], np.float32), rng.uniform(0.01, 0.03, shape[0]).astype(np.float32)):
+        want = oracle.requantize_epilogue(acc, sa, sw, bias, 0.31, -3)
+        got = host(ctx.requantize(dev(acc), dev(sa), dev(sw), dev(bias), 0.31, -3))
+        np.testing.assert_array_equal(got, want)
+    want = oracle.requantize_epilogue(acc, sa, sw, None, 0.31, 0)
+    got = host(ctx.requantize(dev(acc), dev(sa), dev(sw), None, 0.31, 0))
+    np.testing.assert_array_equal(got, want)

@@ -1,0 +1,153 @@
+"""Parity of the int8 MFMA GEMM and the quantized Linear forward with the CPU oracle.
+
+int32 accumulators and int8 outputs are bit-exact; fp32 outputs are held to 1e-5
+relative (and are in practice bit-exact, since the epilogue is the same sequence of
+individually rounded f32 operations).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rand_i8(rng, shape):
+    return rng.integers(-128, 128, size=shape, dtype=np.int8)
+
+
+SHAPES = [
+    (1, 1, 16), (1, 16, 64), (16, 16, 64), (17, 33, 128), (64, 64, 256), (128, 64, 128), (130, 70, 144),
+    (127, 129, 4096), (512, 256, 1024), (5, 300, 48), (256, 512, 16), (33, 1000, 2048),
+]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_i32_bit_exact(ctx, oracle, m, n, k):
+    rng = np.random.default_rng(m * 1000003 + n * 1009 + k)
+    a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+    got = host(ctx.gemm_i8_i32(dev(a), dev(w)))
+    np.testing.assert_array_equal(got, oracle.gemm_i8_nk(a, w))
+
+
+@pytest.mark.parametrize("m,n,k", [(3, 5, 7), (16, 16, 20), (9, 40, 1001), (1, 1, 1)])
+def test_gemm_generic_path_for_odd_k(ctx, oracle, m, n, k):
+    rng = np.random.default_rng(k)
+    a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+    np.testing.assert_array_equal(host(ctx.gemm_i8_i32(dev(a), dev(w))), oracle.gemm_i8_nk(a, w))
+
+
+def test_gemm_matches_reference_kn_layout(ctx, oracle):
+    """The reference's B operand is [K,N]; the kernel takes its transpose and must give the same integers."""
+    rng = np.random.default_rng(77)
+    a, b_kn = rand_i8(rng, (20, 64)), rand_i8(rng, (64, 24))
+    acc, _ = oracle.backend_matmul_i32(a, b_kn)
+    got = host(ctx.gemm_i8_i32(dev(a), dev(np.ascontiguousarray(b_kn.T))))
+    np.testing.assert_array_equal(got, acc)
+
+
+def test_gemm_extreme_values_and_identity(ctx):
+    a = np.full((32, 4096), -128, np.int8)
+    got = host(ctx.gemm_i8_i32(dev(a), dev(a)))
+    np.testing.assert_array_equal(got, np.full((32, 32), 4096 * 16384, np.int32))
+    eye = np.eye(64, dtype=np.int8)
+    rng = np.random.default_rng(1)
+    x = rand_i8(rng, (48, 64))
+    np.testing.assert_array_equal(host(ctx.gemm_i8_i32(dev(x), dev(eye))), x.astype(np.int32))
+
+
+def test_gemm_linearity_full_size(ctx):
+    """M=512, K=N=4096: (a1 + a2) W^T == a1 W^T + a2 W^T, checked against torch's int64 matmul on a slice."""
+    g = torch.Generator(device="cuda").manual_seed(2)
+    a1 = torch.randint(-60, 60, (512, 4096), generator=g, device="cuda", dtype=torch.int8)
+    a2 = torch.randint(-60, 60, (512, 4096), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (4096, 4096), generator=g, device="cuda", dtype=torch.int8)
+    c1, c2, c12 = ctx.gemm_i8_i32(a1, w), ctx.gemm_i8_i32(a2, w), ctx.gemm_i8_i32(a1 + a2, w)
+    torch.cuda.synchronize()
+    assert torch.equal(c12, c1 + c2)
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 511], device="cuda")
+    ref = (a1[rows].double() @ w.double().T).to(torch.int32)  # exact: |acc| < 2^53
+    assert torch.equal(c1[rows], ref)
+
+
+def _quantized_linear_case(oracle, m, n, k, per_token, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wf = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    wq, sw, _ = oracle.quantize_per_channel_auto(wf, 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    if per_token:
+        aq, sa, _ = oracle.quantize_per_channel_auto(x, 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    else:
+        aq, s, _ = oracle.quantize_tensor_auto(x, 0, oracle.PER_TENSOR_SYMMETRIC)
+        sa = np.array([s], np.float32)
+    acc = oracle.gemm_i8_nk(aq.astype(np.int8), wq.astype(np.int8))
+    out = oracle.linear_dequant_epilogue(acc, sa, sw, bias)
+    return x, wf, bias, wq.astype(np.int8), sw, aq.astype(np.int8), sa, acc, out
+
+
+@pytest.mark.parametrize("m,n,k", [(4, 8, 16), (64, 128, 256), (100, 200, 304), (512, 512, 512), (33, 65, 1040)])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_quantized_linear_forward(ctx, hipq, oracle, m, n, k, per_token):
+    x, wf, bias, wq, sw, aq, sa, acc, want = _quantized_linear_case(oracle, m, n, k, per_token, m + n + k)
+    # weights quantized on the device (offline step), bit-exact with the oracle
+    dwq, dsw, _, _ = ctx.quantize_per_row(dev(wf))
+    np.testing.assert_array_equal(host(dwq), wq)
+    np.testing.assert_array_equal(host(dsw), sw)
+    # separate steps
+    got = host(ctx.linear_i8_f32(dev(aq), dev(sa), dwq, dsw, dev(bias)))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=0)
+    np.testing.assert_array_equal(got, want)
+    # whole forward from fp32 activations
+    got = host(ctx.linear_dynamic(dev(x), dwq, dsw, dev(bias), per_token=per_token,
+                                  mode=hipq.FORM_MUL_INV if x.size > 64 else hipq.FORM_DIV))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=0)
+    np.testing.assert_array_equal(got, want)
+    # no bias
+    got = host(ctx.linear_i8_f32(dev(aq), dev(sa), dwq, dsw, None))
+    np.testing.assert_array_equal(got, oracle.linear_dequant_epilogue(acc, sa, sw, None))
+
+
+@pytest.mark.parametrize("m,n,k", [(7, 24, 64), (128, 96, 512), (50, 130, 272)])
+def test_quantized_linear_requant_epilogue(ctx, hipq, oracle, m, n, k):
+    x, wf, bias, wq, sw, aq, sa, acc, out = _quantized_linear_case(oracle, m, n, k, False, 5 * m + k)
+    s_out, _ = oracle.calculate_symmetric_params(*oracle.find_min_max(out), 0)
+    for mode, rm in ((hipq.ROUND_HALF_AWAY, 0), (hipq.ROUND_HALF_EVEN, 1)):
+        oracle.set_round_mode(rm)
+        try:
+            want = oracle.requantize_epilogue(acc, sa, sw, bias, s_out, 2)
+        finally:
+            oracle.set_round_mode(0)
+        got = host(ctx.linear_i8_i8(dev(aq), dev(sa), dev(wq), dev(sw), dev(bias), s_out, 2, mode))
+        np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_decode_shapes_small_n(ctx, hipq, oracle, m):
+    """Config-3 shaped (per-token activations, K=4096) at an N the oracle finishes quickly."""
+    x, wf, bias, wq, sw, aq, sa, acc, want = _quantized_linear_case(oracle, m, 344, 4096, True, 40 + m)
+    got = host(ctx.linear_dynamic(dev(x), dev(wq), dev(sw), dev(bias), per_token=True))
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(host(ctx.gemm_i8_i32(dev(aq), dev(wq))), acc)
+
+
+def test_gemm_error_cases(ctx, hipq):
+    a = torch.zeros((4, 16), dtype=torch.int8, device="cuda")
+    w = torch.zeros((4, 32), dtype=torch.int8, device="cuda")
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.gemm_i8_i32(a, w)
+    assert e.value.code == hipq.DIMENSION_MISMATCH
+    with pytest.raises(hipq.HipqError):
+        ctx.call("hipq_gemm_i8_i32", a.data_ptr(), None, 4, 4, 16, a.data_ptr())
+    # empty M or N is a no-op
+    ctx.call("hipq_gemm_i8_i32", a.data_ptr(), w.data_ptr(), 0, 4, 16, None)

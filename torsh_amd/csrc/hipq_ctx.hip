@@ -1,0 +1,181 @@
+// Context, error reporting and device-memory helpers of the torsh_hipq C-ABI.
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "hipq_internal.h"
+
+namespace {
+thread_local char g_last_error[512] = {0};
+thread_local bool g_has_error = false;
+}  // namespace
+
+namespace hipq {
+
+int32_t fail(int32_t code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    g_has_error = true;
+    return code;
+}
+
+void clear_error() {
+    g_last_error[0] = 0;
+    g_has_error = false;
+}
+
+int32_t enter(hipq_ctx *ctx) {
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e != hipSuccess) return fail(HIPQ_DEVICE_ERROR, "hipSetDevice(%d): %s", ctx->device, hipGetErrorString(e));
+    return HIPQ_SUCCESS;
+}
+
+int32_t scratch(hipq_ctx *ctx, size_t bytes, void **out) {
+    if (bytes > ctx->scratch_bytes) {
+        // Round up so a sequence of slightly growing requests reallocates rarely.
+        size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        if (ctx->scratch) {
+            hipError_t e = hipStreamSynchronize(ctx->stream);
+            if (e != hipSuccess) return fail(HIPQ_SYNCHRONIZATION_ERROR, "scratch: %s", hipGetErrorString(e));
+            (void)hipFree(ctx->scratch);
+            ctx->scratch = nullptr;
+            ctx->scratch_bytes = 0;
+        }
+        hipError_t e = hipMalloc(&ctx->scratch, want);
+        if (e != hipSuccess) {
+            ctx->scratch = nullptr;
+            return fail(HIPQ_ALLOCATION_ERROR, "scratch: hipMalloc(%zu): %s", want, hipGetErrorString(e));
+        }
+        ctx->scratch_bytes = want;
+    }
+    *out = ctx->scratch;
+    return HIPQ_SUCCESS;
+}
+
+int32_t check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HIPQ_DEVICE_ERROR, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+    return HIPQ_SUCCESS;
+}
+
+}  // namespace hipq
+
+extern "C" {
+
+const char *hipq_version(void) { return "torsh_hipq 0.1.0 (gfx950)"; }
+
+const char *hipq_get_last_error(void) { return g_last_error; }
+
+void hipq_clear_last_error(void) { hipq::clear_error(); }
+
+int32_t hipq_has_error(void) { return g_has_error ? 1 : 0; }
+
+static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **out_ctx) {
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0)
+        return hipq::fail(HIPQ_DEVICE_ERROR, "hipq_ctx_create: no HIP device available (%s)",
+                          e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    if (device < 0 || device >= count)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "hipq_ctx_create: device %d out of range [0,%d)", device, count);
+    HIPQ_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIPQ_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return hipq::fail(HIPQ_DEVICE_ERROR, "hipq_ctx_create: device %d is %s; this library is built for gfx950 only",
+                          device, prop.gcnArchName);
+    hipq_ctx *ctx = new (std::nothrow) hipq_ctx();
+    if (!ctx) return hipq::fail(HIPQ_ALLOCATION_ERROR, "hipq_ctx_create: out of host memory");
+    ctx->device = device;
+    ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    if (own) {
+        e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            delete ctx;
+            return hipq::fail(HIPQ_DEVICE_ERROR, "hipq_ctx_create: hipStreamCreate: %s", hipGetErrorString(e));
+        }
+        ctx->owns_stream = true;
+    } else {
+        ctx->stream = stream;
+    }
+    void *p = nullptr;
+    int32_t rc = hipq::scratch(ctx, size_t(8) << 20, &p);
+    if (rc != HIPQ_SUCCESS) {
+        if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return rc;
+    }
+    *out_ctx = ctx;
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_ctx_create(int32_t device, hipq_ctx **out_ctx) {
+    HIPQ_REQUIRE_PTR(out_ctx);
+    return ctx_new(device, nullptr, true, out_ctx);
+}
+
+int32_t hipq_ctx_create_on_stream(int32_t device, void *hip_stream, hipq_ctx **out_ctx) {
+    HIPQ_REQUIRE_PTR(out_ctx);
+    return ctx_new(device, static_cast<hipStream_t>(hip_stream), false, out_ctx);
+}
+
+int32_t hipq_ctx_destroy(hipq_ctx *ctx) {
+    HIPQ_ENTER(ctx);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_ctx_synchronize(hipq_ctx *ctx) {
+    HIPQ_ENTER(ctx);
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess)
+        return hipq::fail(HIPQ_SYNCHRONIZATION_ERROR, "hipq_ctx_synchronize: %s", hipGetErrorString(e));
+    return HIPQ_SUCCESS;
+}
+
+void *hipq_ctx_stream(hipq_ctx *ctx) { return ctx ? static_cast<void *>(ctx->stream) : nullptr; }
+
+int32_t hipq_device_malloc(hipq_ctx *ctx, size_t bytes, void **out_ptr) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(out_ptr);
+    *out_ptr = nullptr;
+    if (bytes == 0) return HIPQ_SUCCESS;
+    hipError_t e = hipMalloc(out_ptr, bytes);
+    if (e != hipSuccess)
+        return hipq::fail(HIPQ_ALLOCATION_ERROR, "hipq_device_malloc(%zu): %s", bytes, hipGetErrorString(e));
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_device_free(hipq_ctx *ctx, void *ptr) {
+    HIPQ_ENTER(ctx);
+    if (!ptr) return HIPQ_SUCCESS;
+    HIPQ_HIP(hipFree(ptr));
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_memcpy_h2d(hipq_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    HIPQ_ENTER(ctx);
+    if (bytes == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(dst_dev);
+    HIPQ_REQUIRE_PTR(src_host);
+    HIPQ_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIPQ_HIP(hipStreamSynchronize(ctx->stream));
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_memcpy_d2h(hipq_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    HIPQ_ENTER(ctx);
+    if (bytes == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(dst_host);
+    HIPQ_REQUIRE_PTR(src_dev);
+    HIPQ_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIPQ_HIP(hipStreamSynchronize(ctx->stream));
+    return HIPQ_SUCCESS;
+}
+
+}  // extern "C"

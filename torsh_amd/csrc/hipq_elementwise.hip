@@ -1,0 +1,761 @@
+// HBM-streaming kernels of the quantized path: min/max reduction, per-tensor and
+// per-row quantize, dequantize, requantize.  All are bandwidth bound; the design
+// rule is one coalesced 16-byte load per lane per instruction (a wavefront reads
+// 1 KiB contiguous), enough independent loads in flight per lane to cover HBM
+// latency, and wave-level shuffles for the reductions.
+#include "hipq_internal.h"
+#include "hipq_math.h"
+
+namespace hipq {
+
+constexpr int kBlock = 256;
+constexpr int kVecPerThread = 4;                         // float4 loads in flight per lane
+constexpr int kTileVec = kBlock * kVecPerThread;         // float4s per block iteration
+constexpr int kTileElems = kTileVec * 4;                 // 4096 elements
+
+struct MinMax {
+    float mn, mx;
+};
+
+__device__ __forceinline__ void acc_minmax(MinMax &m, float v) {
+    m.mn = fminf(m.mn, v);
+    m.mx = fmaxf(m.mx, v);
+}
+
+// Block-wide min/max; result valid in every thread.
+__device__ __forceinline__ MinMax block_minmax(MinMax m, float *lds /* 2 * kBlock/kWave + 2 floats */) {
+    m.mn = wave_min(m.mn);
+    m.mx = wave_max(m.mx);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    constexpr int nw = kBlock / kWave;
+    __syncthreads();
+    if (lane == 0) {
+        lds[wave] = m.mn;
+        lds[nw + wave] = m.mx;
+    }
+    __syncthreads();
+    MinMax r{lds[0], lds[nw]};
+#pragma unroll
+    for (int w = 1; w < nw; ++w) {
+        r.mn = fminf(r.mn, lds[w]);
+        r.mx = fmaxf(r.mx, lds[nw + w]);
+    }
+    return r;
+}
+
+// Stage 1 of the range reduction: each block folds a strided set of 4096-element
+// tiles and writes one (min,max) partial.
+__global__ __launch_bounds__(kBlock) void minmax_partial_kernel(const float *__restrict__ x, size_t n,
+                                                                 float2 *__restrict__ partials) {
+    __shared__ float lds[2 * kBlock / kWave];
+    MinMax m{INFINITY, -INFINITY};
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    const size_t nvec = aligned ? n / 4 : 0;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * kTileVec + threadIdx.x;
+        float4 v[kVecPerThread];
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) {
+            const size_t idx = base + size_t(i) * kBlock;
+            v[i] = idx < nvec ? x4[idx] : make_float4(INFINITY, INFINITY, -INFINITY, -INFINITY);
+        }
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) {
+            const size_t idx = base + size_t(i) * kBlock;
+            if (idx < nvec) {
+                acc_minmax(m, v[i].x);
+                acc_minmax(m, v[i].y);
+                acc_minmax(m, v[i].z);
+                acc_minmax(m, v[i].w);
+            }
+        }
+    }
+    for (size_t i = nvec * 4 + size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += size_t(gridDim.x) * kBlock)
+        acc_minmax(m, x[i]);
+    MinMax r = block_minmax(m, lds);
+    if (threadIdx.x == 0) partials[blockIdx.x] = make_float2(r.mn, r.mx);
+}
+
+// Stage 2: one block folds the partials and writes what the caller asked for:
+// {min,max}, max|x|, and/or a hipq_qparams derived with `flavor`.
+__global__ __launch_bounds__(kBlock) void minmax_final_kernel(const float2 *__restrict__ partials, int nparts,
+                                                               float *__restrict__ out_minmax,
+                                                               float *__restrict__ out_absmax,
+                                                               hipq_qparams *__restrict__ out_params, int flavor,
+                                                               int qmin, int qmax) {
+    __shared__ float lds[2 * kBlock / kWave];
+    MinMax m{INFINITY, -INFINITY};
+    for (int i = threadIdx.x; i < nparts; i += kBlock) {
+        float2 p = partials[i];
+        m.mn = fminf(m.mn, p.x);
+        m.mx = fmaxf(m.mx, p.y);
+    }
+    MinMax r = block_minmax(m, lds);
+    if (threadIdx.x == 0) {
+        if (out_minmax) {
+            out_minmax[0] = r.mn;
+            out_minmax[1] = r.mx;
+        }
+        if (out_absmax) *out_absmax = fmaxf(fabsf(r.mn), fabsf(r.mx));
+        if (out_params) {
+            float s;
+            int zp;
+            int st = params_from_minmax(r.mn, r.mx, flavor, qmin, qmax, &s, &zp);
+            out_params->scale = s;
+            out_params->zero_point = zp;
+            out_params->min_val = r.mn;
+            out_params->max_val = r.mx;
+            out_params->status = st;
+        }
+    }
+}
+
+__global__ void qparams_kernel(const float *__restrict__ minmax, int flavor, int qmin, int qmax,
+                               hipq_qparams *__restrict__ out) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        float s;
+        int zp;
+        const float mn = minmax[0], mx = minmax[1];
+        int st = params_from_minmax(mn, mx, flavor, qmin, qmax, &s, &zp);
+        out->scale = s;
+        out->zero_point = zp;
+        out->min_val = mn;
+        out->max_val = mx;
+        out->status = st;
+    }
+}
+
+__global__ void fill_i32_kernel(int32_t *p, int32_t v, size_t n) {
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+template <typename OutT>
+__device__ __forceinline__ OutT to_out(float q) {
+    if constexpr (sizeof(OutT) == 4)
+        return q;  // f32 carrier keeps NaN
+    else
+        return static_cast<OutT>(to_int_nan0(q));
+}
+
+// Per-tensor quantize.  Scale and zero point come from the launch arguments or,
+// when `params` is non-null, from device memory (dynamic quantization).
+template <typename OutT, bool DIV, bool EVEN>
+__global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restrict__ x, size_t n, float scale,
+                                                           int zp, const hipq_qparams *__restrict__ params,
+                                                           float lo, float hi, OutT *__restrict__ out) {
+    if (params) {
+        if (params->status != HIPQ_SUCCESS) return;  // the reference errors before quantizing
+        scale = params->scale;
+        zp = params->zero_point;
+    }
+    const float inv = 1.0f / scale;
+    const float zpf = static_cast<float>(zp);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) &&
+                         ((reinterpret_cast<uintptr_t>(out) & (4 * sizeof(OutT) - 1)) == 0);
+    const size_t nvec = aligned ? n / 4 : 0;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * kTileVec + threadIdx.x;
+        float4 v[kVecPerThread];
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) {
+            const size_t idx = base + size_t(i) * kBlock;
+            if (idx < nvec) v[i] = x4[idx];
+        }
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) {
+            const size_t idx = base + size_t(i) * kBlock;
+            if (idx < nvec) {
+                const float a = quantize_value<DIV, EVEN>(v[i].x, scale, inv, zpf, lo, hi);
+                const float b = quantize_value<DIV, EVEN>(v[i].y, scale, inv, zpf, lo, hi);
+                const float c = quantize_value<DIV, EVEN>(v[i].z, scale, inv, zpf, lo, hi);
+                const float d = quantize_value<DIV, EVEN>(v[i].w, scale, inv, zpf, lo, hi);
+                if constexpr (sizeof(OutT) == 4) {
+                    reinterpret_cast<float4 *>(out)[idx] = make_float4(a, b, c, d);
+                } else {
+                    reinterpret_cast<uint32_t *>(out)[idx] =
+                        pack4(to_int_nan0(a), to_int_nan0(b), to_int_nan0(c), to_int_nan0(d));
+                }
+            }
+        }
+    }
+    for (size_t i = nvec * 4 + size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += size_t(gridDim.x) * kBlock)
+        out[i] = to_out<OutT>(quantize_value<DIV, EVEN>(x[i], scale, inv, zpf, lo, hi));
+}
+
+template <typename InT>
+__device__ __forceinline__ float4 unpack4(uint32_t w) {
+    if constexpr (sizeof(InT) == 1 && InT(-1) < InT(0)) {
+        return make_float4(static_cast<float>(static_cast<int8_t>(w & 0xff)),
+                           static_cast<float>(static_cast<int8_t>((w >> 8) & 0xff)),
+                           static_cast<float>(static_cast<int8_t>((w >> 16) & 0xff)),
+                           static_cast<float>(static_cast<int8_t>(w >> 24)));
+    } else {
+        return make_float4(static_cast<float>(w & 0xff), static_cast<float>((w >> 8) & 0xff),
+                           static_cast<float>((w >> 16) & 0xff), static_cast<float>(w >> 24));
+    }
+}
+
+// Per-tensor dequantize: y = (q - zp) * scale.
+template <typename InT>
+__global__ __launch_bounds__(kBlock) void dequantize_kernel(const InT *__restrict__ q, size_t n, float scale, int zp,
+                                                             const hipq_qparams *__restrict__ params,
+                                                             float *__restrict__ out) {
+    if (params) {
+        if (params->status != HIPQ_SUCCESS) return;
+        scale = params->scale;
+        zp = params->zero_point;
+    }
+    const float zpf = static_cast<float>(zp);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(q) & (4 * sizeof(InT) - 1)) == 0) &&
+                         ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
+    const size_t nvec = aligned ? n / 4 : 0;
+    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * kTileVec + threadIdx.x;
+        float4 v[kVecPerThread];
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) {
+            const size_t idx = base + size_t(i) * kBlock;
+            if (idx < nvec) {
+                if constexpr (sizeof(InT) == 4)
+                    v[i] = reinterpret_cast<const float4 *>(q)[idx];
+                else
+                    v[i] = unpack4<InT>(reinterpret_cast<const uint32_t *>(q)[idx]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) {
+            const size_t idx = base + size_t(i) * kBlock;
+            if (idx < nvec)
+                reinterpret_cast<float4 *>(out)[idx] = make_float4((v[i].x - zpf) * scale, (v[i].y - zpf) * scale,
+                                                                   (v[i].z - zpf) * scale, (v[i].w - zpf) * scale);
+        }
+    }
+    for (size_t i = nvec * 4 + size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += size_t(gridDim.x) * kBlock)
+        out[i] = (static_cast<float>(q[i]) - zpf) * scale;
+}
+
+// Per-row (axis 0 of [rows, cols]) dynamic quantize: TPR threads own one row,
+// read it once (rows up to TPR*16 floats stay in registers), reduce min/max
+// across the row with wave shuffles, derive the row's parameters and quantize
+// with the division form.
+template <int TPR, bool EVEN>
+__global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *__restrict__ x, size_t rows,
+                                                                   size_t cols, int flavor, int qmin, int qmax,
+                                                                   int8_t *__restrict__ out,
+                                                                   float *__restrict__ out_scales,
+                                                                   int32_t *__restrict__ out_zps,
+                                                                   int32_t *__restrict__ out_status) {
+    constexpr int kRowsPerBlock = kBlock / TPR;
+    constexpr int kCache = 4;
+    __shared__ float lds[2 * kBlock / kWave];
+    const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
+    const size_t row = size_t(blockIdx.x) * kRowsPerBlock + sub;
+    const bool active = row < rows;
+    const float *xr = x + (active ? row : 0) * cols;
+    int8_t *qr = out + (active ? row : 0) * cols;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (cols % 4 == 0) &&
+                         ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
+    const size_t nvec = aligned ? cols / 4 : 0;
+    const float4 *x4 = reinterpret_cast<const float4 *>(xr);
+
+    MinMax m{INFINITY, -INFINITY};
+    float4 cache[kCache];
+    if (active) {
+#pragma unroll
+        for (int i = 0; i < kCache; ++i) {
+            const size_t v = size_t(lane) + size_t(i) * TPR;
+            if (v < nvec) cache[i] = x4[v];
+        }
+#pragma unroll
+        for (int i = 0; i < kCache; ++i) {
+            const size_t v = size_t(lane) + size_t(i) * TPR;
+            if (v < nvec) {
+                acc_minmax(m, cache[i].x);
+                acc_minmax(m, cache[i].y);
+                acc_minmax(m, cache[i].z);
+                acc_minmax(m, cache[i].w);
+            }
+        }
+        for (size_t v = size_t(lane) + size_t(kCache) * TPR; v < nvec; v += TPR) {
+            float4 t = x4[v];
+            acc_minmax(m, t.x);
+            acc_minmax(m, t.y);
+            acc_minmax(m, t.z);
+            acc_minmax(m, t.w);
+        }
+        for (size_t c = nvec * 4 + lane; c < cols; c += TPR) acc_minmax(m, xr[c]);
+    }
+    if constexpr (TPR == kWave) {
+        m.mn = wave_min(m.mn);
+        m.mx = wave_max(m.mx);
+    } else {
+        static_assert(TPR == kBlock, "a row is owned by one wave or by the whole block");
+        m = block_minmax(m, lds);
+    }
+    if (!active) return;
+
+    float scale;
+    int zp;
+    const int st = params_from_minmax(m.mn, m.mx, flavor, qmin, qmax, &scale, &zp);
+    if (lane == 0) {
+        if (out_scales) out_scales[row] = scale;
+        if (out_zps) out_zps[row] = zp;
+        if (st != HIPQ_SUCCESS && out_status) *out_status = st;
+    }
+    if (st != HIPQ_SUCCESS) return;
+    const float zpf = static_cast<float>(zp), lo = static_cast<float>(qmin), hi = static_cast<float>(qmax);
+    uint32_t *q4 = reinterpret_cast<uint32_t *>(qr);
+    auto quant4 = [&](float4 t) {
+        const float a = quantize_value<true, EVEN>(t.x, scale, 0.0f, zpf, lo, hi);
+        const float b = quantize_value<true, EVEN>(t.y, scale, 0.0f, zpf, lo, hi);
+        const float c = quantize_value<true, EVEN>(t.z, scale, 0.0f, zpf, lo, hi);
+        const float d = quantize_value<true, EVEN>(t.w, scale, 0.0f, zpf, lo, hi);
+        return pack4(to_int_nan0(a), to_int_nan0(b), to_int_nan0(c), to_int_nan0(d));
+    };
+#pragma unroll
+    for (int i = 0; i < kCache; ++i) {
+        const size_t v = size_t(lane) + size_t(i) * TPR;
+        if (v < nvec) q4[v] = quant4(cache[i]);
+    }
+    for (size_t v = size_t(lane) + size_t(kCache) * TPR; v < nvec; v += TPR) q4[v] = quant4(x4[v]);
+    for (size_t c = nvec * 4 + lane; c < cols; c += TPR)
+        qr[c] = static_cast<int8_t>(to_int_nan0(quantize_value<true, EVEN>(xr[c], scale, 0.0f, zpf, lo, hi)));
+}
+
+// quantize_per_channel_auto for a channel axis that is not the leading one:
+// one block per channel walks its [outer, inner] slices twice.
+template <bool EVEN>
+__global__ __launch_bounds__(kBlock) void quantize_per_channel_auto_kernel(
+    const float *__restrict__ x, size_t outer, size_t channels, size_t inner, int flavor, int qmin, int qmax,
+    int8_t *__restrict__ out, float *__restrict__ out_scales, int32_t *__restrict__ out_zps,
+    int32_t *__restrict__ out_status) {
+    __shared__ float lds[2 * kBlock / kWave];
+    const size_t ch = blockIdx.x;
+    const size_t per = outer * inner;
+    MinMax m{INFINITY, -INFINITY};
+    for (size_t i = threadIdx.x; i < per; i += kBlock) {
+        const size_t o = i / inner, in = i % inner;
+        acc_minmax(m, x[(o * channels + ch) * inner + in]);
+    }
+    m = block_minmax(m, lds);
+    float scale;
+    int zp;
+    const int st = params_from_minmax(m.mn, m.mx, flavor, qmin, qmax, &scale, &zp);
+    if (threadIdx.x == 0) {
+        if (out_scales) out_scales[ch] = scale;
+        if (out_zps) out_zps[ch] = zp;
+        if (st != HIPQ_SUCCESS && out_status) *out_status = st;
+    }
+    if (st != HIPQ_SUCCESS) return;
+    const float zpf = static_cast<float>(zp), lo = static_cast<float>(qmin), hi = static_cast<float>(qmax);
+    for (size_t i = threadIdx.x; i < per; i += kBlock) {
+        const size_t o = i / inner, in = i % inner;
+        const size_t idx = (o * channels + ch) * inner + in;
+        out[idx] = static_cast<int8_t>(to_int_nan0(quantize_value<true, EVEN>(x[idx], scale, 0.0f, zpf, lo, hi)));
+    }
+}
+
+// Explicit per-channel parameters over a dense [outer, channels, inner] view.
+template <bool DIV, bool EVEN>
+__global__ __launch_bounds__(kBlock) void quantize_per_channel_kernel(const float *__restrict__ x, size_t total,
+                                                                       size_t channels, size_t inner,
+                                                                       const float *__restrict__ scales,
+                                                                       const int32_t *__restrict__ zps,
+                                                                       int8_t *__restrict__ out) {
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += size_t(gridDim.x) * kBlock) {
+        const size_t c = (i / inner) % channels;
+        const float s = scales[c];
+        const float inv = 1.0f / s;
+        const float q = quantize_value<DIV, EVEN>(x[i], s, inv, static_cast<float>(zps[c]), -128.0f, 127.0f);
+        out[i] = static_cast<int8_t>(to_int_nan0(q));
+    }
+}
+
+// y = scale[c] * (q - zp[c])
+__global__ __launch_bounds__(kBlock) void dequantize_per_channel_kernel(const int8_t *__restrict__ q, size_t total,
+                                                                         size_t channels, size_t inner,
+                                                                         const float *__restrict__ scales,
+                                                                         const int32_t *__restrict__ zps,
+                                                                         float *__restrict__ out) {
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += size_t(gridDim.x) * kBlock) {
+        const size_t c = (i / inner) % channels;
+        out[i] = scales[c] * (static_cast<float>(q[i]) - static_cast<float>(zps[c]));
+    }
+}
+
+// int32 accumulators -> int8: v = acc*(s_a*s_w[c]) (+bias[c]); q = clamp(round(v/s_out)+zp_out).
+template <bool EVEN>
+__global__ __launch_bounds__(kBlock) void requantize_kernel(const int32_t *__restrict__ acc, size_t rows, size_t cols,
+                                                             const float *__restrict__ sa, int sa_per_row,
+                                                             const float *__restrict__ sw,
+                                                             const float *__restrict__ bias, float s_out, int zp_out,
+                                                             int8_t *__restrict__ out) {
+    const size_t total = rows * cols;
+    const float zpf = static_cast<float>(zp_out);
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += size_t(gridDim.x) * kBlock) {
+        const size_t r = i / cols, c = i % cols;
+        const float s = (sa_per_row ? sa[r] : sa[0]) * sw[c];
+        float v = static_cast<float>(acc[i]) * s;
+        if (bias) v = v + bias[c];
+        const float q = clamp_keep_nan(round_mode<EVEN>(v / s_out) + zpf, -128.0f, 127.0f);
+        out[i] = static_cast<int8_t>(to_int_nan0(q));
+    }
+}
+
+static inline int grid_for_tiles(hipq_ctx *ctx, size_t n) {
+    size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
+    if (tiles == 0) tiles = 1;
+    const size_t cap = size_t(ctx->num_cus) * 16;
+    return static_cast<int>(tiles < cap ? tiles : cap);
+}
+
+static inline int grid_for_elems(hipq_ctx *ctx, size_t n) {
+    size_t blocks = (n + kBlock - 1) / kBlock;
+    if (blocks == 0) blocks = 1;
+    const size_t cap = size_t(ctx->num_cus) * 16;
+    return static_cast<int>(blocks < cap ? blocks : cap);
+}
+
+// Launches the two-stage range reduction.
+static int32_t launch_minmax(hipq_ctx *ctx, const float *x, size_t n, float *out_minmax, float *out_absmax,
+                             hipq_qparams *out_params, int flavor, int qmin, int qmax) {
+    const int grid = grid_for_tiles(ctx, n);
+    void *s = nullptr;
+    int32_t rc = scratch(ctx, kScratchHeader + size_t(grid) * sizeof(float2), &s);
+    if (rc != HIPQ_SUCCESS) return rc;
+    float2 *partials = reinterpret_cast<float2 *>(static_cast<char *>(s) + kScratchHeader);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, partials);
+    hipLaunchKernelGGL(minmax_final_kernel, dim3(1), dim3(kBlock), 0, ctx->stream, partials, grid, out_minmax,
+                       out_absmax, out_params, flavor, qmin, qmax);
+    return check_launch("minmax");
+}
+
+template <typename OutT>
+static int32_t launch_quantize(hipq_ctx *ctx, const float *x, size_t n, float scale, int zp,
+                               const hipq_qparams *params, int mode, float lo, float hi, OutT *out) {
+    const int grid = grid_for_tiles(ctx, n);
+    const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+#define HIPQ_LAUNCH_Q(D, E)                                                                                   \
+    hipLaunchKernelGGL((quantize_kernel<OutT, D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, scale, zp, \
+                       params, lo, hi, out)
+    if (div && even)
+        HIPQ_LAUNCH_Q(true, true);
+    else if (div)
+        HIPQ_LAUNCH_Q(true, false);
+    else if (even)
+        HIPQ_LAUNCH_Q(false, true);
+    else
+        HIPQ_LAUNCH_Q(false, false);
+#undef HIPQ_LAUNCH_Q
+    return check_launch("quantize");
+}
+
+static int32_t check_mode(const char *fn, int32_t mode) {
+    if (mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV)) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits 0x%x", fn, mode);
+    return HIPQ_SUCCESS;
+}
+
+static int32_t check_scale(const char *fn, float scale) {
+    // `scale <= 0.0` in the reference: NaN passes that test there too.
+    if (scale <= 0.0f) return fail(HIPQ_INVALID_ARGUMENT, "%s: Scale must be positive", fn);
+    return HIPQ_SUCCESS;
+}
+
+template <typename InT>
+static int32_t dequant_common(const char *fn, hipq_ctx *ctx, const InT *q, size_t n, float scale, int32_t zp,
+                              const hipq_qparams *params, float *out) {
+    if (!params) {
+        int32_t rc = check_scale(fn, scale);
+        if (rc) return rc;
+    }
+    if (n == 0) return HIPQ_SUCCESS;
+    if (!q || !out) return fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer", fn);
+    const int grid = grid_for_tiles(ctx, n);
+    hipLaunchKernelGGL((dequantize_kernel<InT>), dim3(grid), dim3(kBlock), 0, ctx->stream, q, n, scale, zp, params,
+                       out);
+    return check_launch(fn);
+}
+
+static int32_t check_row_flavor(const char *fn, int32_t flavor) {
+    if (flavor != HIPQ_PARAMS_SYMMETRIC && flavor != HIPQ_PARAMS_AFFINE)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: Unsupported scheme for per-channel quantization (flavor %d)", fn, flavor);
+    return HIPQ_SUCCESS;
+}
+
+}  // namespace hipq
+
+using namespace hipq;
+
+extern "C" {
+
+int32_t hipq_minmax_f32(hipq_ctx *ctx, const float *x, size_t n, float *out_minmax) {
+    HIPQ_ENTER(ctx);
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "hipq_minmax_f32: Cannot find min/max of empty array");
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out_minmax);
+    return launch_minmax(ctx, x, n, out_minmax, nullptr, nullptr, 0, 0, 0);
+}
+
+int32_t hipq_absmax_f32(hipq_ctx *ctx, const float *x, size_t n, float *out_absmax) {
+    HIPQ_ENTER(ctx);
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "hipq_absmax_f32: Cannot find min/max of empty array");
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out_absmax);
+    return launch_minmax(ctx, x, n, nullptr, out_absmax, nullptr, 0, 0, 0);
+}
+
+int32_t hipq_qparams_from_minmax(hipq_ctx *ctx, const float *minmax, int32_t flavor, int32_t qmin, int32_t qmax,
+                                 hipq_qparams *out_params) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(minmax);
+    HIPQ_REQUIRE_PTR(out_params);
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_BACKEND_ASYMMETRIC)
+        return fail(HIPQ_INVALID_ARGUMENT, "hipq_qparams_from_minmax: unknown flavor %d", flavor);
+    if (qmin >= qmax) return fail(HIPQ_INVALID_ARGUMENT, "hipq_qparams_from_minmax: qmin %d >= qmax %d", qmin, qmax);
+    hipLaunchKernelGGL(qparams_kernel, dim3(1), dim3(64), 0, ctx->stream, minmax, flavor, qmin, qmax, out_params);
+    return check_launch("qparams");
+}
+
+int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n, float scale, int32_t zero_point,
+                                        int32_t mode, int8_t *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_scale(__func__, scale);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    return launch_quantize<int8_t>(ctx, x, n, scale, zero_point, nullptr, mode, -128.0f, 127.0f, out);
+}
+
+int32_t hipq_quantize_per_tensor_f32_u8(hipq_ctx *ctx, const float *x, size_t n, float scale, int32_t zero_point,
+                                        int32_t mode, uint8_t *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_scale(__func__, scale);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    return launch_quantize<uint8_t>(ctx, x, n, scale, zero_point, nullptr, mode, 0.0f, 255.0f, out);
+}
+
+int32_t hipq_quantize_per_tensor_f32_carrier(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                             int32_t zero_point, int32_t mode, int32_t qmin, int32_t qmax,
+                                             float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_scale(__func__, scale);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    if (qmin > qmax) return fail(HIPQ_INVALID_ARGUMENT, "%s: qmin %d > qmax %d", __func__, qmin, qmax);
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    return launch_quantize<float>(ctx, x, n, scale, zero_point, nullptr, mode, static_cast<float>(qmin),
+                                  static_cast<float>(qmax), out);
+}
+
+int32_t hipq_quantize_with_params_f32_i8(hipq_ctx *ctx, const float *x, size_t n, const hipq_qparams *params,
+                                         int32_t mode, int8_t *out) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(params);
+    int32_t rc = check_mode(__func__, mode);
+    if (rc) return rc;
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    return launch_quantize<int8_t>(ctx, x, n, 1.0f, 0, params, mode, -128.0f, 127.0f, out);
+}
+
+int32_t hipq_quantize_with_params_f32_u8(hipq_ctx *ctx, const float *x, size_t n, const hipq_qparams *params,
+                                         int32_t mode, uint8_t *out) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(params);
+    int32_t rc = check_mode(__func__, mode);
+    if (rc) return rc;
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    return launch_quantize<uint8_t>(ctx, x, n, 1.0f, 0, params, mode, 0.0f, 255.0f, out);
+}
+
+int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor, int32_t dtype,
+                                             int32_t mode, void *out, hipq_qparams *out_params) {
+    HIPQ_ENTER(ctx);
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    HIPQ_REQUIRE_PTR(out_params);
+    int32_t rc = check_mode(__func__, mode);
+    if (rc) return rc;
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_BACKEND_ASYMMETRIC)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", __func__, flavor);
+    if (dtype != HIPQ_DTYPE_I8 && dtype != HIPQ_DTYPE_U8)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", __func__, dtype);
+    const int qmin = dtype == HIPQ_DTYPE_I8 ? -128 : 0, qmax = dtype == HIPQ_DTYPE_I8 ? 127 : 255;
+    rc = launch_minmax(ctx, x, n, nullptr, nullptr, out_params, flavor, qmin, qmax);
+    if (rc) return rc;
+    if (dtype == HIPQ_DTYPE_I8)
+        return launch_quantize<int8_t>(ctx, x, n, 1.0f, 0, out_params, mode, -128.0f, 127.0f,
+                                       static_cast<int8_t *>(out));
+    return launch_quantize<uint8_t>(ctx, x, n, 1.0f, 0, out_params, mode, 0.0f, 255.0f, static_cast<uint8_t *>(out));
+}
+
+int32_t hipq_dequantize_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t n, float scale, int32_t zero_point, float *out) {
+    HIPQ_ENTER(ctx);
+    return dequant_common<int8_t>(__func__, ctx, q, n, scale, zero_point, nullptr, out);
+}
+
+int32_t hipq_dequantize_u8_f32(hipq_ctx *ctx, const uint8_t *q, size_t n, float scale, int32_t zero_point,
+                               float *out) {
+    HIPQ_ENTER(ctx);
+    return dequant_common<uint8_t>(__func__, ctx, q, n, scale, zero_point, nullptr, out);
+}
+
+int32_t hipq_dequantize_carrier_f32(hipq_ctx *ctx, const float *q, size_t n, float scale, int32_t zero_point,
+                                    float *out) {
+    HIPQ_ENTER(ctx);
+    return dequant_common<float>(__func__, ctx, q, n, scale, zero_point, nullptr, out);
+}
+
+int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t n, const hipq_qparams *params,
+                                           float *out) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(params);
+    return dequant_common<int8_t>(__func__, ctx, q, n, 1.0f, 0, params, out);
+}
+
+int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t flavor,
+                                     int32_t mode, int8_t *out, float *out_scales, int32_t *out_zero_points,
+                                     int32_t *out_status) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_row_flavor(__func__, flavor);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
+    if (rows == 0) return check_launch(__func__);
+    if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length have no range", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    if (rows >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many rows", __func__);
+    if (cols > 1024) {
+        const int grid = static_cast<int>(rows);
+        if (even)
+            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+        else
+            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+    } else {
+        const int grid = static_cast<int>((rows + 3) / 4);
+        if (even)
+            hipLaunchKernelGGL((quantize_per_row_kernel<kWave, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+        else
+            hipLaunchKernelGGL((quantize_per_row_kernel<kWave, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+    }
+    return check_launch(__func__);
+}
+
+int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels,
+                                              size_t inner, int32_t flavor, int32_t mode, int8_t *out,
+                                              float *out_scales, int32_t *out_zero_points, int32_t *out_status) {
+    HIPQ_ENTER(ctx);
+    if (outer == 1)
+        return hipq_quantize_per_row_f32_i8(ctx, x, channels, inner, flavor, mode, out, out_scales, out_zero_points,
+                                            out_status);
+    int32_t rc = check_row_flavor(__func__, flavor);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
+    if (channels == 0) return check_launch(__func__);
+    if (outer == 0 || inner == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: channels of zero length have no range", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    if (channels >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many channels", __func__);
+    const int grid = static_cast<int>(channels);
+    if (mode & HIPQ_ROUND_HALF_EVEN)
+        hipLaunchKernelGGL((quantize_per_channel_auto_kernel<true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, outer,
+                           channels, inner, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+    else
+        hipLaunchKernelGGL((quantize_per_channel_auto_kernel<false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                           outer, channels, inner, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+    return check_launch(__func__);
+}
+
+int32_t hipq_quantize_per_channel_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels, size_t inner,
+                                         const float *scales, const int32_t *zero_points, int32_t mode,
+                                         int8_t *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_mode(__func__, mode);
+    if (rc) return rc;
+    const size_t total = outer * channels * inner;
+    if (total == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(scales);
+    HIPQ_REQUIRE_PTR(zero_points);
+    HIPQ_REQUIRE_PTR(out);
+    const int grid = grid_for_elems(ctx, total);
+    const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+#define HIPQ_LAUNCH_PC(D, E)                                                                                       \
+    hipLaunchKernelGGL((quantize_per_channel_kernel<D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, total,     \
+                       channels, inner, scales, zero_points, out)
+    if (div && even)
+        HIPQ_LAUNCH_PC(true, true);
+    else if (div)
+        HIPQ_LAUNCH_PC(true, false);
+    else if (even)
+        HIPQ_LAUNCH_PC(false, true);
+    else
+        HIPQ_LAUNCH_PC(false, false);
+#undef HIPQ_LAUNCH_PC
+    return check_launch(__func__);
+}
+
+int32_t hipq_dequantize_per_channel_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t outer, size_t channels,
+                                           size_t inner, const float *scales, const int32_t *zero_points,
+                                           float *out) {
+    HIPQ_ENTER(ctx);
+    const size_t total = outer * channels * inner;
+    if (total == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(q);
+    HIPQ_REQUIRE_PTR(scales);
+    HIPQ_REQUIRE_PTR(zero_points);
+    HIPQ_REQUIRE_PTR(out);
+    const int grid = grid_for_elems(ctx, total);
+    hipLaunchKernelGGL(dequantize_per_channel_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, q, total, channels,
+                       inner, scales, zero_points, out);
+    return check_launch(__func__);
+}
+
+int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_t rows, size_t cols, const float *a_scale,
+                               int32_t a_scale_per_row, const float *w_scales, const float *bias, float out_scale,
+                               int32_t out_zero_point, int32_t mode, int8_t *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_scale(__func__, out_scale);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    if (rows * cols == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(acc);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    const int grid = grid_for_elems(ctx, rows * cols);
+    if (mode & HIPQ_ROUND_HALF_EVEN)
+        hipLaunchKernelGGL((requantize_kernel<true>), dim3(grid), dim3(kBlock), 0, ctx->stream, acc, rows, cols,
+                           a_scale, a_scale_per_row, w_scales, bias, out_scale, out_zero_point, out);
+    else
+        hipLaunchKernelGGL((requantize_kernel<false>), dim3(grid), dim3(kBlock), 0, ctx->stream, acc, rows, cols,
+                           a_scale, a_scale_per_row, w_scales, bias, out_scale, out_zero_point, out);
+    return check_launch(__func__);
+}
+
+}  // extern "C"

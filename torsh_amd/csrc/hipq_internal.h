@@ -1,0 +1,60 @@
+// Internal declarations shared by the torsh_hipq translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+
+#include "torsh_hipq.h"
+
+struct hipq_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    // Scratch owned by the context: partial reductions, device-side parameters,
+    // int8 activations of the fused Linear forward.  Grown on demand, freed with
+    // the context.
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    int num_cus = 256;
+};
+
+namespace hipq {
+
+// Records `msg` (printf style) as the calling thread's last error and returns `code`.
+int32_t fail(int32_t code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+// Makes the context's device current; returns HIPQ_SUCCESS or a recorded error.
+int32_t enter(hipq_ctx *ctx);
+// Ensures ctx->scratch holds at least `bytes`; returns pointer via out.
+int32_t scratch(hipq_ctx *ctx, size_t bytes, void **out);
+// Checks the sticky launch error after a kernel launch.
+int32_t check_launch(const char *what);
+
+// Bytes reserved at the head of the context scratch for small device records
+// (hipq_qparams, min/max pairs, status words); bulk scratch starts after it.
+constexpr size_t kScratchHeader = 4096;
+
+}  // namespace hipq
+
+#define HIPQ_REQUIRE_PTR(p)                                                              \
+    do {                                                                                 \
+        if ((p) == nullptr) return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer '%s'", __func__, #p); \
+    } while (0)
+
+#define HIPQ_ENTER(ctx)                                   \
+    do {                                                  \
+        HIPQ_REQUIRE_PTR(ctx);                            \
+        int32_t _rc = hipq::enter(ctx);                   \
+        if (_rc != HIPQ_SUCCESS) return _rc;              \
+    } while (0)
+
+#define HIPQ_HIP(call)                                                                              \
+    do {                                                                                            \
+        hipError_t _e = (call);                                                                     \
+        if (_e != hipSuccess)                                                                       \
+            return hipq::fail(HIPQ_DEVICE_ERROR, "%s: %s failed: %s", __func__, #call, hipGetErrorString(_e)); \
+    } while (0)

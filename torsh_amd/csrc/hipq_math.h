@@ -1,0 +1,129 @@
+// Device-side scalar arithmetic of the quantized path.  Each helper states the
+// Rust semantics it reproduces; the translation units are compiled with
+// -ffp-contract=off so no multiply-add is fused and every f32 operation rounds
+// exactly as the reference's CPU code does.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <cstdint>
+
+#include "torsh_hipq.h"
+
+namespace hipq {
+
+constexpr int kWave = 64;
+
+// f32::round (half away from zero) or IEEE nearest-even.
+template <bool EVEN>
+__device__ __forceinline__ float round_mode(float v) {
+    if constexpr (EVEN)
+        return rintf(v);
+    else
+        return roundf(v);
+}
+
+// f32::clamp: NaN passes through.
+__device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
+    v = (v < lo) ? lo : v;
+    v = (v > hi) ? hi : v;
+    return v;
+}
+
+// `f32 as i32` on a value already clamped to a small range: NaN -> 0.
+__device__ __forceinline__ int to_int_nan0(float v) { return (v != v) ? 0 : static_cast<int>(v); }
+
+// `f32 as i32`, saturating, NaN -> 0.
+__device__ __forceinline__ int f32_as_i32(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return static_cast<int>(v);
+}
+
+// round(x * inv | x / scale) + zp, clamped; result still a float (the carrier).
+template <bool DIV, bool EVEN>
+__device__ __forceinline__ float quantize_value(float x, float scale, float inv, float zpf, float lo, float hi) {
+    float t;
+    if constexpr (DIV)
+        t = x / scale;
+    else
+        t = x * inv;
+    float q = round_mode<EVEN>(t) + zpf;
+    return clamp_keep_nan(q, lo, hi);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// (min,max) -> (scale, zero_point) with the reference formula `flavor` selects.
+// Returns HIPQ_SUCCESS or HIPQ_INVALID_ARGUMENT.
+//   HIPQ_PARAMS_SYMMETRIC          crates/torsh-quantization/src/algorithms.rs:397-422
+//   HIPQ_PARAMS_AFFINE             crates/torsh-quantization/src/algorithms.rs:358-394
+//   HIPQ_PARAMS_BACKEND_SYMMETRIC  crates/torsh-backend/src/quantization/params.rs:323-340
+//   HIPQ_PARAMS_BACKEND_ASYMMETRIC crates/torsh-backend/src/quantization/params.rs:343-363
+__device__ __forceinline__ int params_from_minmax(float mn, float mx, int flavor, int qmin_i, int qmax_i,
+                                                  float *scale, int *zp) {
+    const bool finite = (fabsf(mn) <= FLT_MAX) && (fabsf(mx) <= FLT_MAX);  // false for NaN and Inf
+    const float qmin = static_cast<float>(qmin_i), qmax = static_cast<float>(qmax_i);
+    *scale = 1.0f;
+    *zp = 0;
+    switch (flavor) {
+    case HIPQ_PARAMS_SYMMETRIC: {
+        if (!finite) return HIPQ_INVALID_ARGUMENT;
+        float abs_max = fmaxf(fabsf(mn), fabsf(mx));
+        if (abs_max < FLT_EPSILON) return HIPQ_SUCCESS;
+        *scale = abs_max / qmax;
+        return HIPQ_SUCCESS;
+    }
+    case HIPQ_PARAMS_AFFINE: {
+        if (!finite || mn > mx) return HIPQ_INVALID_ARGUMENT;
+        if (fabsf(mx - mn) < FLT_EPSILON) {
+            *zp = qmin_i;
+            return HIPQ_SUCCESS;
+        }
+        float s = (mx - mn) / (qmax - qmin);
+        float z = qmin - mn / s;
+        *scale = s;
+        *zp = f32_as_i32(clamp_keep_nan(roundf(z), qmin, qmax));
+        return HIPQ_SUCCESS;
+    }
+    case HIPQ_PARAMS_BACKEND_SYMMETRIC: {
+        if (!finite || mn > mx) return HIPQ_INVALID_ARGUMENT;
+        float r = fmaxf(fabsf(mx), fabsf(mn));
+        if (r != 0.0f) *scale = (2.0f * r) / (qmax - qmin);
+        return HIPQ_SUCCESS;
+    }
+    case HIPQ_PARAMS_BACKEND_ASYMMETRIC: {
+        if (!finite || mn > mx) return HIPQ_INVALID_ARGUMENT;
+        if (mx == mn) {
+            *zp = qmin_i;
+            return HIPQ_SUCCESS;
+        }
+        float s = (mx - mn) / (qmax - qmin);
+        float z = qmin - mn / s;
+        *scale = s;
+        *zp = f32_as_i32(clamp_keep_nan(roundf(z), qmin, qmax));
+        return HIPQ_SUCCESS;
+    }
+    default:
+        return HIPQ_INVALID_ARGUMENT;
+    }
+}
+
+}  // namespace hipq

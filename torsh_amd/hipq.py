@@ -1,0 +1,320 @@
+"""ctypes binding of ``libtorsh_hipq.so`` for tests, the smoke check and the benchmark.
+
+The binding is deliberately thin: every function forwards raw device pointers
+(``torch.Tensor.data_ptr()``) to the C-ABI entry point of the same name and turns
+a non-zero status into :class:`HipqError` carrying the library's last-error
+string.  torch is used for device memory and streams only.  There is no
+fallback: if the shared library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtorsh_hipq.so")
+
+SUCCESS, INVALID_ARGUMENT, SHAPE_ERROR, DIMENSION_MISMATCH, DEVICE_ERROR, ALLOCATION_ERROR, SYNCHRONIZATION_ERROR, UNKNOWN_ERROR = range(8)
+ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
+FORM_MUL_INV, FORM_DIV = 0, 2
+DTYPE_I8, DTYPE_U8 = 0, 1
+PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC = range(4)
+
+
+class HipqError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[hipq status {code}] {message}")
+        self.code = code
+        self.message = message
+
+
+class QParams(C.Structure):
+    _fields_ = [("scale", C.c_float), ("zero_point", C.c_int32), ("min_val", C.c_float), ("max_val", C.c_float),
+                ("status", C.c_int32), ("reserved", C.c_int32 * 3)]
+
+
+_lib: Optional[C.CDLL] = None
+
+_vp, _sz, _i32, _f32 = C.c_void_p, C.c_size_t, C.c_int32, C.c_float
+
+# name -> argtypes (all return int32 status unless listed in _SPECIAL)
+_SIGNATURES = {
+    "hipq_ctx_create": [_i32, C.POINTER(_vp)],
+    "hipq_ctx_create_on_stream": [_i32, _vp, C.POINTER(_vp)],
+    "hipq_ctx_destroy": [_vp],
+    "hipq_ctx_synchronize": [_vp],
+    "hipq_device_malloc": [_vp, _sz, C.POINTER(_vp)],
+    "hipq_device_free": [_vp, _vp],
+    "hipq_memcpy_h2d": [_vp, _vp, _vp, _sz],
+    "hipq_memcpy_d2h": [_vp, _vp, _vp, _sz],
+    "hipq_minmax_f32": [_vp, _vp, _sz, _vp],
+    "hipq_absmax_f32": [_vp, _vp, _sz, _vp],
+    "hipq_qparams_from_minmax": [_vp, _vp, _i32, _i32, _i32, _vp],
+    "hipq_quantize_per_tensor_f32_i8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp],
+    "hipq_quantize_per_tensor_f32_u8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp],
+    "hipq_quantize_per_tensor_f32_carrier": [_vp, _vp, _sz, _f32, _i32, _i32, _i32, _i32, _vp],
+    "hipq_quantize_with_params_f32_i8": [_vp, _vp, _sz, _vp, _i32, _vp],
+    "hipq_quantize_with_params_f32_u8": [_vp, _vp, _sz, _vp, _i32, _vp],
+    "hipq_quantize_dynamic_per_tensor_f32": [_vp, _vp, _sz, _i32, _i32, _i32, _vp, _vp],
+    "hipq_dequantize_i8_f32": [_vp, _vp, _sz, _f32, _i32, _vp],
+    "hipq_dequantize_u8_f32": [_vp, _vp, _sz, _f32, _i32, _vp],
+    "hipq_dequantize_carrier_f32": [_vp, _vp, _sz, _f32, _i32, _vp],
+    "hipq_dequantize_with_params_i8_f32": [_vp, _vp, _sz, _vp, _vp],
+    "hipq_quantize_per_row_f32_i8": [_vp, _vp, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
+    "hipq_quantize_per_channel_auto_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
+    "hipq_quantize_per_channel_f32_i8": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _i32, _vp],
+    "hipq_dequantize_per_channel_i8_f32": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp],
+    "hipq_gemm_i8_i32": [_vp, _vp, _vp, _sz, _sz, _sz, _vp],
+    "hipq_linear_i8_f32": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
+    "hipq_linear_i8_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _f32, _i32, _i32, _vp],
+    "hipq_requantize_i32_i8": [_vp, _vp, _sz, _sz, _vp, _i32, _vp, _vp, _f32, _i32, _i32, _vp],
+    "hipq_linear_dynamic_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
+}
+
+_SPECIAL = {
+    "hipq_version": (C.c_char_p, []),
+    "hipq_get_last_error": (C.c_char_p, []),
+    "hipq_clear_last_error": (None, []),
+    "hipq_has_error": (_i32, []),
+    "hipq_ctx_stream": (_vp, [_vp]),
+}
+
+
+def exported_symbols() -> list[str]:
+    """Every entry point ``include/torsh_hipq.h`` declares."""
+    return sorted(list(_SIGNATURES) + list(_SPECIAL))
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> C.CDLL:
+    """Loads the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise FileNotFoundError(
+                f"{_LIB_PATH} is missing: build it with `python -m torsh_amd.build` (there is no CPU fallback)")
+        lib = C.CDLL(_LIB_PATH)
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = _i32
+        for name, (restype, argtypes) in _SPECIAL.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return (load().hipq_get_last_error() or b"").decode()
+
+
+def _check(code: int) -> None:
+    if code != SUCCESS:
+        raise HipqError(code, last_error())
+
+
+def _ptr(t) -> Optional[int]:
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    if not t.is_contiguous():
+        raise ValueError("hipq entry points take dense row-major tensors")
+    return t.data_ptr()
+
+
+class Context:
+    """A ``hipq_ctx`` bound to a device; by default it enqueues on torch's current stream."""
+
+    def __init__(self, device: int = 0, stream: Optional[torch.cuda.Stream] = None, own_stream: bool = False):
+        self._lib = load()
+        self.handle = _vp()
+        self.device = device
+        if own_stream:
+            _check(self._lib.hipq_ctx_create(device, C.byref(self.handle)))
+        else:
+            st = stream if stream is not None else torch.cuda.current_stream(device)
+            _check(self._lib.hipq_ctx_create_on_stream(device, _vp(st.cuda_stream), C.byref(self.handle)))
+
+    def close(self) -> None:
+        if self.handle:
+            self._lib.hipq_ctx_destroy(self.handle)
+            self.handle = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def call(self, name: str, *args) -> None:
+        _check(getattr(self._lib, name)(self.handle, *args))
+
+    def synchronize(self) -> None:
+        self.call("hipq_ctx_synchronize")
+
+    @property
+    def stream_handle(self) -> int:
+        return self._lib.hipq_ctx_stream(self.handle) or 0
+
+    # ---- convenience wrappers over torch tensors (device memory only) -------------
+    def _dev(self):
+        return torch.device("cuda", self.device)
+
+    def minmax(self, x: torch.Tensor) -> torch.Tensor:
+        out = torch.empty(2, dtype=torch.float32, device=self._dev())
+        self.call("hipq_minmax_f32", _ptr(x), x.numel(), _ptr(out))
+        return out
+
+    def absmax(self, x: torch.Tensor) -> torch.Tensor:
+        out = torch.empty(1, dtype=torch.float32, device=self._dev())
+        self.call("hipq_absmax_f32", _ptr(x), x.numel(), _ptr(out))
+        return out
+
+    def new_qparams(self) -> torch.Tensor:
+        return torch.zeros(C.sizeof(QParams), dtype=torch.uint8, device=self._dev())
+
+    @staticmethod
+    def read_qparams(buf: torch.Tensor) -> QParams:
+        return QParams.from_buffer_copy(bytes(buf.cpu().numpy().tobytes()))
+
+    def qparams_from_minmax(self, minmax: torch.Tensor, flavor: int, qmin: int, qmax: int) -> torch.Tensor:
+        out = self.new_qparams()
+        self.call("hipq_qparams_from_minmax", _ptr(minmax), flavor, qmin, qmax, _ptr(out))
+        return out
+
+    def quantize_per_tensor_i8(self, x, scale, zp, mode=0, out=None):
+        out = out if out is not None else torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        self.call("hipq_quantize_per_tensor_f32_i8", _ptr(x), x.numel(), float(scale), int(zp), mode, _ptr(out))
+        return out
+
+    def quantize_per_tensor_u8(self, x, scale, zp, mode=FORM_DIV, out=None):
+        out = out if out is not None else torch.empty(x.shape, dtype=torch.uint8, device=self._dev())
+        self.call("hipq_quantize_per_tensor_f32_u8", _ptr(x), x.numel(), float(scale), int(zp), mode, _ptr(out))
+        return out
+
+    def quantize_per_tensor_carrier(self, x, scale, zp, mode=0, qmin=-128, qmax=127):
+        out = torch.empty(x.shape, dtype=torch.float32, device=self._dev())
+        self.call("hipq_quantize_per_tensor_f32_carrier", _ptr(x), x.numel(), float(scale), int(zp), mode, qmin, qmax,
+                  _ptr(out))
+        return out
+
+    def quantize_dynamic_per_tensor(self, x, flavor=PARAMS_SYMMETRIC, dtype=DTYPE_I8, mode=0, out=None, params=None):
+        tdt = torch.int8 if dtype == DTYPE_I8 else torch.uint8
+        out = out if out is not None else torch.empty(x.shape, dtype=tdt, device=self._dev())
+        params = params if params is not None else self.new_qparams()
+        self.call("hipq_quantize_dynamic_per_tensor_f32", _ptr(x), x.numel(), flavor, dtype, mode, _ptr(out),
+                  _ptr(params))
+        return out, params
+
+    def dequantize(self, q, scale, zp, out=None):
+        out = out if out is not None else torch.empty(q.shape, dtype=torch.float32, device=self._dev())
+        name = {torch.int8: "hipq_dequantize_i8_f32", torch.uint8: "hipq_dequantize_u8_f32",
+                torch.float32: "hipq_dequantize_carrier_f32"}[q.dtype]
+        self.call(name, _ptr(q), q.numel(), float(scale), int(zp), _ptr(out))
+        return out
+
+    def dequantize_with_params(self, q, params, out=None):
+        out = out if out is not None else torch.empty(q.shape, dtype=torch.float32, device=self._dev())
+        self.call("hipq_dequantize_with_params_i8_f32", _ptr(q), q.numel(), _ptr(params), _ptr(out))
+        return out
+
+    def quantize_per_row(self, x, flavor=PARAMS_SYMMETRIC, mode=0):
+        rows, cols = x.shape
+        out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
+        scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
+        zps = torch.empty(rows, dtype=torch.int32, device=self._dev())
+        status = torch.empty(1, dtype=torch.int32, device=self._dev())
+        self.call("hipq_quantize_per_row_f32_i8", _ptr(x), rows, cols, flavor, mode, _ptr(out), _ptr(scales),
+                  _ptr(zps), _ptr(status))
+        return out, scales, zps, status
+
+    def quantize_per_channel_auto(self, x, axis, flavor=PARAMS_SYMMETRIC, mode=0):
+        shape = list(x.shape)
+        outer = 1
+        for s in shape[:axis]:
+            outer *= s
+        inner = 1
+        for s in shape[axis + 1:]:
+            inner *= s
+        ch = shape[axis]
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        scales = torch.empty(ch, dtype=torch.float32, device=self._dev())
+        zps = torch.empty(ch, dtype=torch.int32, device=self._dev())
+        status = torch.empty(1, dtype=torch.int32, device=self._dev())
+        self.call("hipq_quantize_per_channel_auto_f32_i8", _ptr(x), outer, ch, inner, flavor, mode, _ptr(out),
+                  _ptr(scales), _ptr(zps), _ptr(status))
+        return out, scales, zps, status
+
+    def quantize_per_channel(self, x, scales, zps, axis, mode=FORM_DIV):
+        shape = list(x.shape)
+        outer = 1
+        for s in shape[:axis]:
+            outer *= s
+        inner = 1
+        for s in shape[axis + 1:]:
+            inner *= s
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        self.call("hipq_quantize_per_channel_f32_i8", _ptr(x), outer, shape[axis], inner, _ptr(scales), _ptr(zps),
+                  mode, _ptr(out))
+        return out
+
+    def dequantize_per_channel(self, q, scales, zps, axis):
+        shape = list(q.shape)
+        outer = 1
+        for s in shape[:axis]:
+            outer *= s
+        inner = 1
+        for s in shape[axis + 1:]:
+            inner *= s
+        out = torch.empty(q.shape, dtype=torch.float32, device=self._dev())
+        self.call("hipq_dequantize_per_channel_i8_f32", _ptr(q), outer, shape[axis], inner, _ptr(scales), _ptr(zps),
+                  _ptr(out))
+        return out
+
+    def gemm_i8_i32(self, a, w, out=None):
+        m, k = a.shape
+        n, k2 = w.shape
+        if k != k2:
+            raise HipqError(DIMENSION_MISMATCH, f"gemm dimension mismatch: a has K={k} but w has K={k2}")
+        out = out if out is not None else torch.empty((m, n), dtype=torch.int32, device=self._dev())
+        self.call("hipq_gemm_i8_i32", _ptr(a), _ptr(w), m, n, k, _ptr(out))
+        return out
+
+    def linear_i8_f32(self, a, a_scale, w, w_scales, bias=None, out=None):
+        m, k = a.shape
+        n, _ = w.shape
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_i8_f32", _ptr(a), _ptr(a_scale), int(a_scale.numel() > 1), _ptr(w), _ptr(w_scales),
+                  _ptr(bias), m, n, k, _ptr(out))
+        return out
+
+    def linear_i8_i8(self, a, a_scale, w, w_scales, bias, out_scale, out_zp, mode=0, out=None):
+        m, k = a.shape
+        n, _ = w.shape
+        out = out if out is not None else torch.empty((m, n), dtype=torch.int8, device=self._dev())
+        self.call("hipq_linear_i8_i8", _ptr(a), _ptr(a_scale), int(a_scale.numel() > 1), _ptr(w), _ptr(w_scales),
+                  _ptr(bias), m, n, k, float(out_scale), int(out_zp), mode, _ptr(out))
+        return out
+
+    def requantize(self, acc, a_scale, w_scales, bias, out_scale, out_zp, mode=0):
+        rows, cols = acc.shape
+        out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
+        self.call("hipq_requantize_i32_i8", _ptr(acc), rows, cols, _ptr(a_scale), int(a_scale.numel() > 1),
+                  _ptr(w_scales), _ptr(bias), float(out_scale), int(out_zp), mode, _ptr(out))
+        return out
+
+    def linear_dynamic(self, x, w, w_scales, bias=None, per_token=False, mode=0, out=None):
+        m, k = x.shape
+        n, _ = w.shape
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_dynamic_f32", _ptr(x), int(per_token), _ptr(w), _ptr(w_scales), _ptr(bias), m, n, k,
+                  mode, _ptr(out))
+        return out
