@@ -1,0 +1,253 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference hot path on one MI355X.
+
+One "step" is one QuantizedLinear forward of the headline workload
+(BASELINE.json configs[1]): fp32 activations [512,4096] -> dynamic per-tensor
+int8 quantize (min/max, scale, quantize) -> int8 x int8 -> int32 MFMA GEMM
+against per-output-channel int8 weights [4096,4096] -> dequantize + bias epilogue
+-> fp32 [512,4096].  All inputs are resident in HBM before the timed region.
+Activations, weights and outputs rotate through pools larger than the 256 MB
+memory-side cache, so every step streams its operands from HBM as successive
+layers of a model would.
+
+Prints ONE JSON line.  `value` is int8 TOP/s of the whole step (2*M*N*K per
+step time); `roofline` describes the dominant kernel (the GEMM) timed on its
+own with HIP events on the launch stream; `extra` carries the quantize /
+dequantize GB/s of configs[0] and the other shapes.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA, 5.0 POP/s
+PEAK_HBM_GBPS = 8000.0   # MI355X HBM3E, 8 TB/s
+
+# HBM bytes per GEMM launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None until measured.
+GEMM_TRAFFIC_BYTES = None
+
+
+def event_time_ms(fn, reps: int, warmup: int) -> float:
+    """Average duration of fn() in ms, HIP events on torch's current stream (the stream the kernels use)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def cpu_baseline(m: int, n: int, k: int):
+    """Times the CPU oracle (reference loop structure) on a bounded sample of the same workload."""
+    import numpy as np
+
+    from oracle import pyoracle
+
+    rng = np.random.default_rng(2)
+    m_sample = 4
+    a = rng.integers(-127, 128, size=(m_sample, k), dtype=np.int8)
+    b_kn = rng.integers(-127, 128, size=(k, n), dtype=np.int8)  # the reference's [K,N] operand
+    t = pyoracle.time_matmul_rows(a, b_kn, m_sample)
+    # widen the sample until it is a few seconds of work, capped at 32 rows
+    while t < 2.0 and m_sample < 32:
+        m_sample *= 2
+        a = rng.integers(-127, 128, size=(m_sample, k), dtype=np.int8)
+        t = pyoracle.time_matmul_rows(a, b_kn, m_sample)
+    tops = 2.0 * m_sample * n * k / t / 1e12
+    # configs[0] round trip on all host cores (the reference's rayon loops)
+    x = rng.standard_normal(4096 * 4096, dtype=np.float32)
+    t_rt = pyoracle.time_roundtrip_c1(x, reps=2)
+    return {
+        "value": tops,
+        "unit": "TOP/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"first {m_sample} of {m} activation rows through the reference's single-threaded i,j,l int32 "
+                  f"loop with [K,N] weights ({t:.2f} s); extrapolated full forward {t * m / m_sample:.1f} s",
+        "roundtrip_4096x4096": {
+            "seconds": t_rt,
+            "GB/s": 14.0 * 4096 * 4096 / t_rt / 1e9,
+            "cores": pyoracle.num_threads(),
+            "note": "min/max + symmetric params + quantize + dequantize, 14 algorithmic B/elem, OpenMP over all host "
+                    "cores like the reference's rayon loops",
+        },
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (no collectives are part of it).",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    from torsh_amd import hipq
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        return 3
+    hipq.load()
+    ctx = hipq.Context(0)
+    M, N, K = 512, 4096, 4096
+    g = torch.Generator(device="cuda").manual_seed(2)
+    pool = 32  # 32 x 16.8 MB weights = 537 MB > 256 MB memory-side cache
+    xs = [torch.randn(M, K, generator=g, device="cuda") for _ in range(pool)]
+    wq, sw = [], []
+    for i in range(pool):
+        wf = torch.randn(N, K, generator=g, device="cuda") * 0.02
+        q, s, _, _ = ctx.quantize_per_row(wf)
+        wq.append(q)
+        sw.append(s)
+        del wf
+    bias = torch.randn(N, generator=g, device="cuda") * 0.01
+    outs = [torch.empty(M, N, device="cuda") for _ in range(pool)]
+    torch.cuda.synchronize()
+
+    it = [0]
+
+    def step():
+        i = it[0] % pool
+        it[0] += 1
+        ctx.linear_dynamic(xs[i], wq[i], sw[i], bias, per_token=False, mode=hipq.FORM_MUL_INV, out=outs[i])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ops = 2.0 * M * N * K
+    value = ops / (ms_per_step * 1e-3) / 1e12
+
+    # dominant kernel on its own: the GEMM + dequant epilogue on pre-quantized activations
+    aq = [ctx.quantize_dynamic_per_tensor(x)[0] for x in xs]
+    sa = torch.full((1,), 0.03, device="cuda")
+    jt = [0]
+
+    def gemm_only():
+        i = jt[0] % pool
+        jt[0] += 1
+        ctx.linear_i8_f32(aq[i], sa, wq[i], sw[i], bias, out=outs[i])
+
+    gemm_ms = event_time_ms(gemm_only, reps=max(args.steps, 100), warmup=args.warmup)
+    gemm_tops = ops / (gemm_ms * 1e-3) / 1e12
+    algo_bytes = M * K + N * K + 4 * N + 4 * N + 4 * M * N
+
+    result = {
+        "metric": "int8 TOPS & % MFMA peak, QuantizedLinear M=512 K=N=4096; quantize GB/s",
+        "value": value,
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: QuantizedLinear forward, fp32 act [512,4096] dynamic per-tensor int8, "
+                        "per-channel int8 W [4096,4096], fp32 bias, int32 accumulate, fp32 out",
+            "M": M, "N": N, "K": K,
+            "rounding": "half-away-from-zero (reference f32::round)",
+            "operand_pool": f"{pool} rotating weight/activation/output sets (HBM-cold)",
+        },
+        "roofline": {
+            "kernel": "gemm_i8_pipe_kernel (int8 MFMA GEMM + dequant/bias epilogue)",
+            "bound": "mfma",
+            "achieved": gemm_tops,
+            "peak": PEAK_INT8_TOPS,
+            "unit": "TOP/s",
+            "frac": gemm_tops / PEAK_INT8_TOPS,
+            "traffic": GEMM_TRAFFIC_BYTES,
+            "ops_per_launch": ops,
+            "algorithmic_bytes_per_launch": algo_bytes,
+            "avg_launch_us": gemm_ms * 1e3,
+        },
+    }
+
+    if not args.no_extra:
+        extra = {}
+        n = 4096 * 4096
+        npool = 10  # 10 x (64 + 16 + 64) MiB > memory-side cache
+        fx = [torch.randn(n, generator=g, device="cuda") for _ in range(npool)]
+        fq = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(npool)]
+        fy = [torch.empty(n, device="cuda") for _ in range(npool)]
+        params = ctx.new_qparams()
+        mm = torch.empty(2, device="cuda")
+        kt = [0]
+
+        def rot():
+            i = kt[0] % npool
+            kt[0] += 1
+            return i
+
+        def run_quant():
+            i = rot()
+            ctx.quantize_per_tensor_i8(fx[i], 0.04, 0, hipq.FORM_MUL_INV, out=fq[i])
+
+        def run_dequant():
+            i = rot()
+            ctx.dequantize(fq[i], 0.04, 0, out=fy[i])
+
+        def run_minmax():
+            i = rot()
+            ctx.call("hipq_minmax_f32", fx[i].data_ptr(), n, mm.data_ptr())
+
+        def run_dynamic():
+            i = rot()
+            ctx.quantize_dynamic_per_tensor(fx[i], out=fq[i], params=params)
+
+        for name, fn, bytes_per in (("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
+                                    ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9)):
+            ms = event_time_ms(fn, reps=50, warmup=5)
+            gbps = bytes_per * n / (ms * 1e-3) / 1e9
+            extra[name] = {"us": ms * 1e3, "GB/s": gbps, "frac_hbm_peak": gbps / PEAK_HBM_GBPS,
+                           "algorithmic_bytes_per_elem": bytes_per, "elements": n}
+        del fx, fq, fy
+        result["extra"] = extra
+        result["roofline_quantize"] = {
+            "kernel": "quantize_kernel<int8> on fp32 [4096,4096] (configs[0])",
+            "bound": "hbm",
+            "achieved": extra["quantize_f32_i8"]["GB/s"],
+            "peak": PEAK_HBM_GBPS,
+            "unit": "GB/s",
+            "frac": extra["quantize_f32_i8"]["frac_hbm_peak"],
+            "traffic": None,
+        }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(M, N, K)
+        result["speedup_vs_cpu_baseline"] = value / result["cpu_baseline"]["value"]
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -11,7 +11,6 @@ namespace hipq {
 constexpr int kBlock = 256;
 constexpr int kVecPerThread = 4;                         // float4 loads in flight per lane
 constexpr int kTileVec = kBlock * kVecPerThread;         // float4s per block iteration
-constexpr int kTileElems = kTileVec * 4;                 // 4096 elements
 
 struct MinMax {
     float mn, mx;
