@@ -151,3 +151,24 @@ def test_gemm_error_cases(ctx, hipq):
         ctx.call("hipq_gemm_i8_i32", a.data_ptr(), None, 4, 4, 16, a.data_ptr())
     # empty M or N is a no-op
     ctx.call("hipq_gemm_i8_i32", a.data_ptr(), w.data_ptr(), 0, 4, 16, None)
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 17, 40, 64])
+def test_config3_full_size_weight_streaming(ctx, hipq, m):
+    """Llama-7B up-proj shape N=11008, K=4096 (BASELINE config 3): int32 accumulators against an exact
+    float64 product computed by torch, and the fused per-token epilogue against the same f32 expression."""
+    g = torch.Generator(device="cuda").manual_seed(5 + m)
+    n, k = 11008, 4096
+    a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    acc = ctx.gemm_i8_i32(a, w)
+    ref = (a.double() @ w.double().T).to(torch.int32)  # exact: |acc| < 2^53
+    torch.cuda.synchronize()
+    assert torch.equal(acc, ref)
+    sa = torch.rand(m, generator=g, device="cuda") * 0.05 + 0.01
+    sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(n, generator=g, device="cuda") * 0.01
+    out = ctx.linear_i8_f32(a, sa, w, sw, bias)
+    want = ref.float() * (sa[:, None] * sw[None, :]) + bias[None, :]  # same individually rounded f32 ops
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)

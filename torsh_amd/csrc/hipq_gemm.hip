@@ -557,6 +557,136 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     HIPQ_TS_FLUSH();
 }
 
+// ---------------------------------------------------------------------------
+// Skinny GEMM (M <= 16: decode-shaped Linear).  The weight matrix is read exactly
+// once and nothing else matters: 16 weight rows per workgroup, the K range split
+// between the four waves, each lane loading 16 bytes of "its" weight row straight
+// into the MFMA operand layout (no LDS staging: there is no reuse to stage for).
+// Vector-memory loads return in order, so the (L2-resident) activation fragments
+// are requested first and all weight loads of the batch follow back to back; the
+// MFMAs then run off registers while the next batch is already in flight.  The
+// four partial 16x16 accumulators are summed through LDS (integer adds: order
+// independent).
+template <int G, int EPI, bool EVEN>
+__global__ __launch_bounds__(kGemmThreads) void gemv_i8_kernel(const int8_t *__restrict__ A,
+                                                               const int8_t *__restrict__ W, int M, int N, int K,
+                                                               GemmEpilogue ep) {
+    constexpr int NW = kGemmThreads / kWave;
+    constexpr int BATCH = 16;  // k-steps of 64 bytes per batch: 16 KiB of weights per wave in flight
+    __shared__ v4i red[NW][G][kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int n0 = blockIdx.x * (16 * G);
+    const int frow = lane % 16, g = lane / 16;
+    const int kw = K / NW;  // bytes of K per wave, a multiple of 64
+    const int kbeg = wave * kw;
+    const int mrow = frow < M ? frow : M - 1;
+    const int8_t *ap = A + size_t(mrow) * K + kbeg + g * 16;
+    const int8_t *wp[G];
+#pragma unroll
+    for (int r = 0; r < G; ++r) {
+        int nrow = n0 + r * 16 + frow;
+        nrow = nrow < N ? nrow : N - 1;  // rows past the edge are computed and discarded
+        wp[r] = W + size_t(nrow) * K + kbeg + g * 16;
+    }
+    // Epilogue operands of the wave that will store row group `wave` (requested first, so
+    // they are back long before they are needed).
+    float4 sw4 = make_float4(1.f, 1.f, 1.f, 1.f), b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float s_a = 1.0f;
+    const int n_out = n0 + wave * 16 + 4 * g;
+    if constexpr (EPI != EPI_I32) {
+        if (wave < G && n_out < N) {
+            const int n1 = n_out + 1 < N ? n_out + 1 : N - 1, n2 = n_out + 2 < N ? n_out + 2 : N - 1,
+                      n3 = n_out + 3 < N ? n_out + 3 : N - 1;
+            sw4 = make_float4(ep.sw[n_out], ep.sw[n1], ep.sw[n2], ep.sw[n3]);
+            if (ep.bias) b4 = make_float4(ep.bias[n_out], ep.bias[n1], ep.bias[n2], ep.bias[n3]);
+            s_a = ep.sa_per_row ? ep.sa[mrow] : ep.sa[0];
+        }
+    }
+    v4i acc[G];
+#pragma unroll
+    for (int r = 0; r < G; ++r) acc[r] = v4i{0, 0, 0, 0};
+    for (int k0 = 0; k0 < kw; k0 += BATCH * 64) {
+        v4i fa[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+            if (k0 + u * 64 < kw) fa[u] = *reinterpret_cast<const v4i *>(ap + k0 + u * 64);
+#pragma unroll
+        for (int r = 0; r < G; ++r) {
+            v4i fw[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+                if (k0 + u * 64 < kw) fw[u] = *reinterpret_cast<const v4i *>(wp[r] + k0 + u * 64);
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+                if (k0 + u * 64 < kw) acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[u], fa[u], acc[r], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < G; ++r) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    // Wave r finishes row group r.  D = Wfrag (rows n) x Afrag (cols m): a lane holds
+    // m = lane%16 and the four consecutive channels n = 4*(lane/16) + i.
+    if (wave >= G) return;
+    v4i sum = red[0][wave][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[w][wave][lane];
+    const int m = frow;
+    if (m >= M || n_out >= N) return;
+    const size_t off = size_t(m) * N + n_out;
+    constexpr unsigned kAlignMask = (EPI == EPI_I8) ? 3u : 15u;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(ep.out) & kAlignMask) == 0);
+    if constexpr (EPI == EPI_I32) {
+        int32_t *o = static_cast<int32_t *>(ep.out);
+        if (vec) {
+            *reinterpret_cast<v4i *>(o + off) = sum;
+        } else {
+            for (int i = 0; i < 4; ++i)
+                if (n_out + i < N) o[off + i] = sum[i];
+        }
+    } else {
+        const float swa[4] = {sw4.x, sw4.y, sw4.z, sw4.w}, ba[4] = {b4.x, b4.y, b4.z, b4.w};
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float s = s_a * swa[i];
+            v[i] = static_cast<float>(sum[i]) * s;
+            if (ep.bias) v[i] = v[i] + ba[i];
+        }
+        if constexpr (EPI == EPI_F32) {
+            float *o = static_cast<float *>(ep.out);
+            if (vec) {
+                *reinterpret_cast<float4 *>(o + off) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+                for (int i = 0; i < 4; ++i)
+                    if (n_out + i < N) o[off + i] = v[i];
+            }
+        } else {
+            int8_t *o = static_cast<int8_t *>(ep.out);
+            int q[4];
+            const float zpf = static_cast<float>(ep.zp_out);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                q[i] = to_int_nan0(clamp_keep_nan(round_mode<EVEN>(v[i] / ep.s_out) + zpf, -128.0f, 127.0f));
+            if (vec) {
+                *reinterpret_cast<uint32_t *>(o + off) = pack4(q[0], q[1], q[2], q[3]);
+            } else {
+                for (int i = 0; i < 4; ++i)
+                    if (n_out + i < N) o[off + i] = static_cast<int8_t>(q[i]);
+            }
+        }
+    }
+}
+
+template <int EPI, bool EVEN>
+static int32_t launch_gemv(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, int N, int K,
+                           const GemmEpilogue &ep) {
+    // One weight row group per workgroup measured fastest for every M <= 16 (more row groups
+    // per workgroup save activation re-reads from L2 but leave fewer loads in flight).
+    hipLaunchKernelGGL((gemv_i8_kernel<1, EPI, EVEN>), dim3((N + 15) / 16), dim3(kGemmThreads), 0, ctx->stream, a, w,
+                       M, N, K, ep);
+    return check_launch("gemv_i8");
+}
+
 // Any shape, any alignment: one thread per output, plain integer dot product.
 // Used when K is not a multiple of 16 or an operand is not 16-byte aligned.
 template <int EPI, bool EVEN>
@@ -647,6 +777,7 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
     const GemmEpilogue &epd = ep;
 #endif
     int variant = gemm_variant_override();
+    if (variant == 0 && M <= 16 && K % 256 == 0) return launch_gemv<EPI, EVEN>(ctx, a, w, M, N, K, ep);
     const bool pipe_ok = (K % 128 == 0) && K >= 256;
     if (variant == 0) variant = pipe_ok ? 2 : 10;
     if (variant < 10 && !pipe_ok) variant = 10;
