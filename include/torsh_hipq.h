@@ -229,6 +229,36 @@ HIPQ_API int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t 
                                          const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
                                          int32_t mode, float *out);
 
+/* ---- quantized Conv2d forward (NCHW, filters [OC,IC,KH,KW]) ------------ */
+/* Integer part of perform_quantized_convolution,
+ * crates/torsh-backend/src/quantization/operations.rs:637-713:
+ *   acc[n,oc,oh,ow] = sum over kh,kw,ic of (x_q - zp_in) * w_q   (int32)
+ * with padded taps contributing nothing (the real value 0), output size
+ * (H + 2p - k)/s + 1 (crates/torsh-backend/src/quantization/ops.rs:513-514). */
+HIPQ_API int32_t hipq_conv2d_u8i8_i32(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, const int8_t *w, size_t nb,
+                                      size_t c, size_t h, size_t wd, size_t oc, size_t kh, size_t kw, size_t stride_h,
+                                      size_t stride_w, size_t pad_h, size_t pad_w, int32_t *out);
+/* The same accumulators followed by the fused bias + requantize tail
+ * (operations.rs:716-724 with a supplied output scale):
+ *   v = acc * (s_in * s_w[oc]) + bias[oc];  q = clamp(round(v / s_out) + zp_out, -128, 127).
+ * s_in and s_out are host scalars; w_scales [oc] and bias [oc] (may be NULL) are device. */
+HIPQ_API int32_t hipq_conv2d_u8i8_i8(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in, const int8_t *w,
+                                     const float *w_scales, const float *bias, size_t nb, size_t c, size_t h, size_t wd,
+                                     size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
+                                     size_t pad_w, float out_scale, int32_t out_zero_point, int32_t mode, int8_t *out);
+/* One-time filter preparation for the stride-1 fast path: int8 [OC,IC,KH,KW]
+ * -> [OC,KH*KW,IC] (same byte count) and the per-filter sums w_sums[oc]
+ * (offline weight preparation; no reference counterpart, the reference keeps
+ * filters as stored). */
+HIPQ_API int32_t hipq_conv2d_pack_weights_i8(hipq_ctx *ctx, const int8_t *w, size_t oc, size_t ic, size_t kh, size_t kw,
+                                             int8_t *packed, int32_t *w_sums);
+/* hipq_conv2d_u8i8_i8 on prepared filters (stride 1, channels a multiple of 128). */
+HIPQ_API int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in,
+                                            const int8_t *w_packed, const int32_t *w_sums, const float *w_scales,
+                                            const float *bias, size_t nb, size_t c, size_t h, size_t wd, size_t oc,
+                                            size_t kh, size_t kw, size_t pad_h, size_t pad_w, float out_scale,
+                                            int32_t out_zero_point, int32_t mode, int8_t *out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,121 @@
+"""Parity of the quantized Conv2d forward (u8 x i8 -> i32 -> requantized i8) with the CPU oracle: bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+GEOMS = [
+    # nb, c, h, w, oc, k, stride, pad, zp      (fast path: stride 1 and c % 128 == 0)
+    (1, 128, 5, 5, 8, 3, (1, 1), (1, 1), 0),
+    (2, 128, 7, 6, 130, 3, (1, 1), (1, 1), 17),
+    (1, 256, 6, 6, 64, 1, (1, 1), (0, 0), 3),
+    (2, 128, 9, 8, 40, 5, (1, 1), (2, 2), 200),
+    (1, 256, 14, 14, 32, 3, (1, 1), (0, 0), 128),
+    # direct path
+    (2, 3, 8, 8, 4, 3, (1, 1), (1, 1), 5),
+    (1, 16, 9, 9, 6, 3, (2, 2), (1, 1), 0),
+    (2, 128, 8, 8, 8, 3, (2, 1), (0, 1), 9),
+    (1, 1, 3, 3, 1, 1, (1, 1), (0, 0), 0),
+]
+
+
+@pytest.mark.parametrize("nb,c,h,w,oc,k,stride,pad,zp", GEOMS)
+def test_conv_accumulators_bit_exact(ctx, oracle, nb, c, h, w, oc, k, stride, pad, zp):
+    rng = np.random.default_rng(nb * 7 + c + h * 3 + oc)
+    x = rng.integers(0, 256, size=(nb, c, h, w), dtype=np.uint8)
+    wq = rng.integers(-128, 128, size=(oc, c, k, k), dtype=np.int8)
+    want = oracle.backend_conv2d_i32(x, zp, wq, stride, pad)
+    got = host(ctx.conv2d_i32(dev(x), zp, dev(wq), stride, pad))
+    np.testing.assert_array_equal(got, want)
+
+
+def _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, seed):
+    rng = np.random.default_rng(seed)
+    x = np.maximum(rng.standard_normal((nb, c, h, w)), 0).astype(np.float32)  # ReLU(N(0,1))
+    wf = (rng.standard_normal((oc, c, k, k)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(oc) * 0.01).astype(np.float32)
+    mn, mx = oracle.find_min_max(x)
+    s_in, zp_in = oracle.backend_params_asymmetric(mn, mx, 0, 255)
+    xq = oracle.backend_quantize_f32(x, s_in, zp_in, 0, 255)
+    wq, sw, _ = oracle.quantize_per_channel_auto(wf.reshape(oc, -1), 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    wq = wq.astype(np.int8).reshape(wf.shape)
+    acc = oracle.backend_conv2d_i32(xq, zp_in, wq, (1, 1), (pad, pad))
+    ho, wo = acc.shape[2:]
+    acc2d = acc.reshape(nb * oc, ho * wo)
+    out_f = (acc2d.astype(np.float32) * np.tile(np.float32(s_in) * sw, nb)[:, None]) + np.tile(bias, nb)[:, None]
+    s_out, _ = oracle.calculate_symmetric_params(float(out_f.min()), float(out_f.max()), 0)
+    return x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out
+
+
+@pytest.mark.parametrize("nb,c,h,w,oc,k,pad", [(2, 128, 14, 14, 64, 3, 1), (1, 256, 7, 7, 33, 3, 1), (3, 16, 10, 10, 8, 3, 1)])
+def test_quantized_conv2d_forward(ctx, hipq, oracle, nb, c, h, w, oc, k, pad):
+    """BASELINE config 4 at reduced size: asymmetric u8 activations, per-channel int8 filters, fused bias + requant."""
+    x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out = _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, c + oc)
+    # activations quantized on the device: min/max -> asymmetric params -> u8
+    dq, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_BACKEND_ASYMMETRIC, hipq.DTYPE_U8, hipq.FORM_DIV)
+    p = ctx.read_qparams(params)
+    assert (p.scale, p.zero_point) == (np.float32(s_in), zp_in)
+    np.testing.assert_array_equal(host(dq), xq)
+    # filters quantized per output channel on the device
+    dwq, dsw, _, _ = ctx.quantize_per_row(dev(wf.reshape(oc, -1)))
+    np.testing.assert_array_equal(host(dwq).reshape(wq.shape), wq)
+    dwq = dwq.reshape(wq.shape)
+    for mode, rm in ((hipq.ROUND_HALF_AWAY, 0), (hipq.ROUND_HALF_EVEN, 1)):
+        oracle.set_round_mode(rm)
+        try:
+            want = oracle.requantize_epilogue(acc2d, s_in, sw, bias, s_out, -2, channel_axis_is_row=True, inner=oc)
+        finally:
+            oracle.set_round_mode(0)
+        got = host(ctx.conv2d_i8(dq, zp_in, s_in, dwq, dsw, dev(bias), s_out, -2, (1, 1), (pad, pad), mode))
+        np.testing.assert_array_equal(got.reshape(acc2d.shape), want)
+        if c % 128 == 0:
+            packed, sums = ctx.conv2d_pack_weights(dwq)
+            got = host(ctx.conv2d_i8_packed(dq, zp_in, s_in, packed, sums, (k, k), dsw, dev(bias), s_out, -2, (pad, pad), mode))
+            np.testing.assert_array_equal(got.reshape(acc2d.shape), want)
+    want = oracle.requantize_epilogue(acc2d, s_in, sw, None, s_out, 0, channel_axis_is_row=True, inner=oc)
+    got = host(ctx.conv2d_i8(dq, zp_in, s_in, dwq, dsw, None, s_out, 0, (1, 1), (pad, pad)))
+    np.testing.assert_array_equal(got.reshape(acc2d.shape), want)
+
+
+def test_config4_full_size_against_direct_kernel_and_torch(ctx, hipq):
+    """[32,256,14,14] (*) [256,256,3,3], stride 1, pad 1: the implicit-GEMM accumulators must equal an exact
+    float64 convolution computed by torch (|acc| < 2^53), for a non-zero input zero point as well."""
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randint(0, 256, (32, 256, 14, 14), generator=g, device="cuda", dtype=torch.uint8)
+    w = torch.randint(-128, 128, (256, 256, 3, 3), generator=g, device="cuda", dtype=torch.int8)
+    for zp in (0, 37):
+        acc = ctx.conv2d_i32(x, zp, w, (1, 1), (1, 1))
+        ref = torch.nn.functional.conv2d(x.double() - zp, w.double(), padding=0)
+        # zero padding of the real values: pad the shifted input with zeros
+        ref = torch.nn.functional.conv2d(torch.nn.functional.pad(x.double() - zp, (1, 1, 1, 1)), w.double())
+        torch.cuda.synchronize()
+        assert torch.equal(acc, ref.to(torch.int32))
+
+
+def test_conv_error_cases(ctx, hipq):
+    x = torch.zeros((1, 4, 5, 5), dtype=torch.uint8, device="cuda")
+    w = torch.zeros((2, 3, 3, 3), dtype=torch.int8, device="cuda")
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.conv2d_i32(x, 0, w)
+    assert e.value.code == hipq.DIMENSION_MISMATCH
+    w = torch.zeros((2, 4, 7, 7), dtype=torch.int8, device="cuda")
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.conv2d_i32(x, 0, w)
+    assert e.value.code == hipq.SHAPE_ERROR
+    w = torch.zeros((2, 4, 3, 3), dtype=torch.int8, device="cuda")
+    sw = torch.ones(2, device="cuda")
+    with pytest.raises(hipq.HipqError):
+        ctx.conv2d_i8(x, 0, -1.0, w, sw, None, 1.0, 0)
+    with pytest.raises(hipq.HipqError):
+        ctx.conv2d_i8(x, 300, 1.0, w, sw, None, 1.0, 0)

@@ -1,0 +1,287 @@
+// Quantized Conv2d forward: u8 activations (NCHW) x per-channel int8 filters ->
+// int32 accumulators -> requantized int8 (NCHW), bias fused.
+//
+// Fast path (stride 1, channels a multiple of 128): an im2col-free implicit GEMM
+// on the pipelined MFMA kernel.  The activations are rewritten once as signed
+// bytes (x - 128) in a zero-point-padded NHWC image, so that for every filter tap
+// the K-slice of the "window matrix" is a plain strided matrix (consecutive
+// windows start one pixel apart) and the kernel's global->LDS fills need no
+// gather.  Shifting by 128 lets the signed int8 MFMA multiply unsigned
+// activations; the shift and the zero point are undone in the epilogue with the
+// per-filter weight sum:  sum (x - zp) w = sum (x - 128) w + (128 - zp) sum w,
+// and a border pixel holds exactly zp so padded taps contribute nothing.
+// Everything else runs through a direct per-output kernel (correct, not fast).
+#include "hipq_gemm_kernels.h"
+
+namespace hipq {
+
+constexpr int kConvThreads = 256;
+
+// u8 NCHW -> i8 NHWC with a border of `pad` pixels holding (zp - 128).
+__global__ __launch_bounds__(kConvThreads) void conv_pack_input_kernel(const uint8_t *__restrict__ x, int C, int H, int W,
+                                                                         int pad_h, int pad_w, int zp,
+                                                                         int8_t *__restrict__ out) {
+    const int hp_count = H + 2 * pad_h, wp_count = W + 2 * pad_w;
+    const int n = blockIdx.x / hp_count, hp = blockIdx.x % hp_count;
+    const int h = hp - pad_h;
+    int8_t *orow = out + (size_t(n) * hp_count + hp) * wp_count * C;
+    const int8_t border = static_cast<int8_t>(zp - 128);
+    for (int wp = 0; wp < wp_count; ++wp) {
+        const int w = wp - pad_w;
+        const bool inside = h >= 0 && h < H && w >= 0 && w < W;
+        for (int c = threadIdx.x; c < C; c += kConvThreads) {
+            int8_t v = border;
+            if (inside) v = static_cast<int8_t>(static_cast<int>(x[((size_t(n) * C + c) * H + h) * W + w]) - 128);
+            orow[size_t(wp) * C + c] = v;
+        }
+    }
+}
+
+__global__ void conv_fill_i8_kernel(int8_t *p, int8_t v, size_t n) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) p[i] = v;
+}
+
+// int8 [OC, IC, KH*KW] -> [OC, KH*KW, IC] and wsum[oc] = sum of the filter's weights.
+__global__ __launch_bounds__(kConvThreads) void conv_pack_weights_kernel(const int8_t *__restrict__ w, int IC, int taps,
+                                                                           int8_t *__restrict__ packed,
+                                                                           int32_t *__restrict__ wsum) {
+    __shared__ int part[kConvThreads / kWave];
+    const int oc = blockIdx.x;
+    const size_t base = size_t(oc) * IC * taps;
+    int s = 0;
+    for (int i = threadIdx.x; i < IC * taps; i += kConvThreads) {
+        const int t = i / IC, c = i % IC;  // destination order
+        const int8_t v = w[base + size_t(c) * taps + t];
+        packed[base + i] = v;
+        s += v;
+    }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+    if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int i = 0; i < kConvThreads / kWave; ++i) t += part[i];
+        wsum[oc] = t;
+    }
+}
+
+struct ConvGeom {
+    int nb, c, h, w, oc, kh, kw, sh, sw, ph, pw, ho, wo;
+};
+
+// Direct convolution, one thread per output: acc = sum over valid taps (x - zp_in) * w.
+template <int EPI, bool EVEN>
+__global__ __launch_bounds__(kConvThreads) void conv_direct_kernel(const uint8_t *__restrict__ x, int zp_in,
+                                                                    const int8_t *__restrict__ w, ConvGeom g,
+                                                                    float s_in, const float *__restrict__ sw,
+                                                                    const float *__restrict__ bias, float s_out,
+                                                                    int zp_out, void *__restrict__ out) {
+    const size_t total = size_t(g.nb) * g.oc * g.ho * g.wo;
+    for (size_t idx = size_t(blockIdx.x) * kConvThreads + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * kConvThreads) {
+        const int ow = static_cast<int>(idx % g.wo);
+        const int oh = static_cast<int>((idx / g.wo) % g.ho);
+        const int oc = static_cast<int>((idx / (size_t(g.wo) * g.ho)) % g.oc);
+        const int n = static_cast<int>(idx / (size_t(g.wo) * g.ho * g.oc));
+        int acc = 0;
+        for (int r = 0; r < g.kh; ++r) {
+            const int ih = oh * g.sh + r - g.ph;
+            if (ih < 0 || ih >= g.h) continue;
+            for (int s = 0; s < g.kw; ++s) {
+                const int iw = ow * g.sw + s - g.pw;
+                if (iw < 0 || iw >= g.w) continue;
+                for (int c = 0; c < g.c; ++c) {
+                    const int xv = static_cast<int>(x[((size_t(n) * g.c + c) * g.h + ih) * g.w + iw]) - zp_in;
+                    const int wv = w[((size_t(oc) * g.c + c) * g.kh + r) * g.kw + s];
+                    acc += xv * wv;
+                }
+            }
+        }
+        if constexpr (EPI == EPI_I32) {
+            static_cast<int32_t *>(out)[idx] = acc;
+        } else {
+            float v = static_cast<float>(acc) * (s_in * sw[oc]);
+            if (bias) v = v + bias[oc];
+            const float q = clamp_keep_nan(round_mode<EVEN>(v / s_out) + static_cast<float>(zp_out), -128.0f, 127.0f);
+            static_cast<int8_t *>(out)[idx] = static_cast<int8_t>(to_int_nan0(q));
+        }
+    }
+}
+
+static int32_t check_geom(const char *fn, const ConvGeom &g) {
+    if (g.sh <= 0 || g.sw <= 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: stride must be positive", fn);
+    if (g.kh <= 0 || g.kw <= 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: empty kernel", fn);
+    if (g.h + 2 * g.ph < g.kh || g.w + 2 * g.pw < g.kw)
+        return fail(HIPQ_SHAPE_ERROR, "%s: kernel larger than the padded input", fn);
+    if (size_t(g.c) * g.kh * g.kw > (size_t(1) << 16))
+        return fail(HIPQ_SHAPE_ERROR, "%s: c*kh*kw = %zu could overflow the int32 accumulator", fn,
+                    size_t(g.c) * g.kh * g.kw);
+    return HIPQ_SUCCESS;
+}
+
+static bool fast_path_ok(const ConvGeom &g) {
+    return g.sh == 1 && g.sw == 1 && g.c % 128 == 0 && g.c * g.kh * g.kw >= 256 && g.oc >= 1;
+}
+
+// Runs the implicit GEMM on an already packed image / filter pair.
+template <int EPI, bool EVEN>
+static int32_t run_implicit_gemm(hipq_ctx *ctx, const int8_t *ximg, const int8_t *wpacked, const int32_t *wsum,
+                                 int zp_in, const ConvGeom &g, float s_in, const float *sw, const float *bias,
+                                 float s_out, int zp_out, void *out) {
+    const int hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw;
+    GemmEpilogue ep{nullptr, 0, sw, bias, s_out, zp_out, out};
+    ep.sa_scalar = s_in;
+    ep.cv_tiles_per_tap = g.c / 128;
+    ep.cv_kw = g.kw;
+    ep.cv_wp = wp;
+    ep.cv_hp = hp;
+    ep.cv_c = g.c;
+    ep.cv_ho = g.ho;
+    ep.cv_wo = g.wo;
+    ep.cv_oc = g.oc;
+    ep.cv_wsum = wsum;
+    ep.cv_corr_mul = 128 - zp_in;
+    const int M = g.oc, N = g.nb * hp * wp, K = g.c * g.kh * g.kw;
+    return launch_pipe<128, 64, 6, 4, 2, 1, 2, EPI, EVEN, 1>(ctx, wpacked, ximg, M, N, K, ep);
+}
+
+static size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+template <int EPI, bool EVEN>
+static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int zp_in, float s_in, const int8_t *w,
+                            const int8_t *wpacked, const int32_t *wsum, const float *sw, const float *bias,
+                            const ConvGeom &g, float s_out, int zp_out, void *out) {
+    if (!fast_path_ok(g)) {
+        if (!w) return fail(HIPQ_INVALID_ARGUMENT, "%s: this geometry needs the unpacked filters", fn);
+        const size_t total = size_t(g.nb) * g.oc * g.ho * g.wo;
+        size_t blocks = (total + kConvThreads - 1) / kConvThreads;
+        const size_t cap = size_t(ctx->num_cus) * 32;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL((conv_direct_kernel<EPI, EVEN>), dim3(static_cast<int>(blocks)), dim3(kConvThreads), 0,
+                           ctx->stream, x, zp_in, w, g, s_in, sw, bias, s_out, zp_out, out);
+        return check_launch(fn);
+    }
+    const int hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw, taps = g.kh * g.kw;
+    // Windows near the end of the last image read up to (kh-1)*wp + kw-1 pixels past it.
+    const size_t img_bytes = size_t(g.nb) * hp * wp * g.c;
+    const size_t slack = (size_t(g.kh - 1) * wp + g.kw) * g.c + 1024;
+    const size_t w_bytes = size_t(g.oc) * g.c * taps;
+    void *s = nullptr;
+    int32_t rc = scratch(ctx, kScratchHeader + align256(img_bytes + slack) + align256(w_bytes) + align256(g.oc * 4), &s);
+    if (rc) return rc;
+    int8_t *ximg = reinterpret_cast<int8_t *>(static_cast<char *>(s) + kScratchHeader);
+    int8_t *wbuf = ximg + align256(img_bytes + slack);
+    int32_t *wsbuf = reinterpret_cast<int32_t *>(wbuf + align256(w_bytes));
+    hipLaunchKernelGGL(conv_pack_input_kernel, dim3(g.nb * hp), dim3(kConvThreads), 0, ctx->stream, x, g.c, g.h, g.w, g.ph,
+                       g.pw, zp_in, ximg);
+    hipLaunchKernelGGL(conv_fill_i8_kernel, dim3(8), dim3(256), 0, ctx->stream, ximg + img_bytes, int8_t(0), slack);
+    if (!wpacked) {
+        hipLaunchKernelGGL(conv_pack_weights_kernel, dim3(g.oc), dim3(kConvThreads), 0, ctx->stream, w, g.c, taps, wbuf,
+                           wsbuf);
+        wpacked = wbuf;
+        wsum = wsbuf;
+    }
+    rc = check_launch(fn);
+    if (rc) return rc;
+    return run_implicit_gemm<EPI, EVEN>(ctx, ximg, wpacked, wsum, zp_in, g, s_in, sw, bias, s_out, zp_out, out);
+}
+
+static int32_t make_geom(const char *fn, size_t nb, size_t c, size_t h, size_t w, size_t oc, size_t kh, size_t kw,
+                         size_t sh, size_t sw, size_t ph, size_t pw, ConvGeom *g) {
+    const size_t lim = size_t(1) << 24;
+    if (nb >= lim || c >= lim || h >= lim || w >= lim || oc >= lim || kh >= lim || kw >= lim || sh >= lim || sw >= lim ||
+        ph >= lim || pw >= lim)
+        return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", fn);
+    *g = ConvGeom{int(nb), int(c), int(h), int(w), int(oc), int(kh), int(kw), int(sh), int(sw), int(ph), int(pw), 0, 0};
+    int32_t rc = check_geom(fn, *g);
+    if (rc) return rc;
+    // (H + 2p - k) / s + 1, crates/torsh-backend/src/quantization/ops.rs:513-514
+    g->ho = (g->h + 2 * g->ph - g->kh) / g->sh + 1;
+    g->wo = (g->w + 2 * g->pw - g->kw) / g->sw + 1;
+    if (size_t(g->nb) * (g->h + 2 * g->ph) * (g->w + 2 * g->pw) >= (size_t(1) << 31))
+        return fail(HIPQ_SHAPE_ERROR, "%s: too many pixels", fn);
+    return HIPQ_SUCCESS;
+}
+
+}  // namespace hipq
+
+using namespace hipq;
+
+extern "C" {
+
+int32_t hipq_conv2d_pack_weights_i8(hipq_ctx *ctx, const int8_t *w, size_t oc, size_t ic, size_t kh, size_t kw,
+                                    int8_t *packed, int32_t *wsum) {
+    HIPQ_ENTER(ctx);
+    if (oc == 0 || ic * kh * kw == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(w);
+    HIPQ_REQUIRE_PTR(packed);
+    HIPQ_REQUIRE_PTR(wsum);
+    if (oc >> 24 || ic >> 24 || (kh * kw) >> 16) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    hipLaunchKernelGGL(conv_pack_weights_kernel, dim3(static_cast<int>(oc)), dim3(kConvThreads), 0, ctx->stream, w,
+                       static_cast<int>(ic), static_cast<int>(kh * kw), packed, wsum);
+    return check_launch(__func__);
+}
+
+int32_t hipq_conv2d_u8i8_i32(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, const int8_t *w, size_t nb, size_t c,
+                             size_t h, size_t wd, size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                             size_t pad_h, size_t pad_w, int32_t *out) {
+    HIPQ_ENTER(ctx);
+    ConvGeom g;
+    int32_t rc = make_geom(__func__, nb, c, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w, &g);
+    if (rc) return rc;
+    if (zp_in < 0 || zp_in > 255) return fail(HIPQ_INVALID_ARGUMENT, "%s: zero point %d outside [0,255]", __func__, zp_in);
+    if (nb == 0 || oc == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(w);
+    HIPQ_REQUIRE_PTR(out);
+    return conv_forward<EPI_I32, false>(__func__, ctx, x, zp_in, 1.0f, w, nullptr, nullptr, nullptr, nullptr, g, 1.0f, 0,
+                                        out);
+}
+
+static int32_t conv_i8_common(const char *fn, hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in,
+                              const int8_t *w, const int8_t *wpacked, const int32_t *wsum, const float *sw,
+                              const float *bias, const ConvGeom &g, float s_out, int32_t zp_out, int32_t mode,
+                              int8_t *out) {
+    if (s_in <= 0.0f || s_out <= 0.0f) return fail(HIPQ_INVALID_ARGUMENT, "%s: Scale must be positive", fn);
+    if (zp_in < 0 || zp_in > 255) return fail(HIPQ_INVALID_ARGUMENT, "%s: zero point %d outside [0,255]", fn, zp_in);
+    if (mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV)) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", fn);
+    if (g.nb == 0 || g.oc == 0) return HIPQ_SUCCESS;
+    if (!x || !sw || !out) return fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer", fn);
+    if (mode & HIPQ_ROUND_HALF_EVEN)
+        return conv_forward<EPI_I8, true>(fn, ctx, x, zp_in, s_in, w, wpacked, wsum, sw, bias, g, s_out, zp_out, out);
+    return conv_forward<EPI_I8, false>(fn, ctx, x, zp_in, s_in, w, wpacked, wsum, sw, bias, g, s_out, zp_out, out);
+}
+
+int32_t hipq_conv2d_u8i8_i8(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in, const int8_t *w,
+                            const float *w_scales, const float *bias, size_t nb, size_t c, size_t h, size_t wd,
+                            size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
+                            size_t pad_w, float out_scale, int32_t out_zero_point, int32_t mode, int8_t *out) {
+    HIPQ_ENTER(ctx);
+    ConvGeom g;
+    int32_t rc = make_geom(__func__, nb, c, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w, &g);
+    if (rc) return rc;
+    if (nb != 0 && oc != 0) HIPQ_REQUIRE_PTR(w);
+    return conv_i8_common(__func__, ctx, x, zp_in, s_in, w, nullptr, nullptr, w_scales, bias, g, out_scale,
+                          out_zero_point, mode, out);
+}
+
+int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in, const int8_t *w_packed,
+                                   const int32_t *w_sums, const float *w_scales, const float *bias, size_t nb, size_t c,
+                                   size_t h, size_t wd, size_t oc, size_t kh, size_t kw, size_t pad_h, size_t pad_w,
+                                   float out_scale, int32_t out_zero_point, int32_t mode, int8_t *out) {
+    HIPQ_ENTER(ctx);
+    ConvGeom g;
+    int32_t rc = make_geom(__func__, nb, c, h, wd, oc, kh, kw, 1, 1, pad_h, pad_w, &g);
+    if (rc) return rc;
+    if (!fast_path_ok(g))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: packed filters need stride 1 and channels a multiple of 128", __func__);
+    if (nb != 0 && oc != 0) {
+        HIPQ_REQUIRE_PTR(w_packed);
+        HIPQ_REQUIRE_PTR(w_sums);
+    }
+    return conv_i8_common(__func__, ctx, x, zp_in, s_in, nullptr, w_packed, w_sums, w_scales, bias, g, out_scale,
+                          out_zero_point, mode, out);
+}
+
+}  // extern "C"

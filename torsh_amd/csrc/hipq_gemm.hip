@@ -7,555 +7,10 @@
 // accumulators in registers.  The weight fragment is the MFMA's row operand so
 // that each lane ends up with four consecutive output channels of one
 // activation row: 16-byte stores, 16-byte loads of the per-channel scales.
-#include <cstdlib>
 
-#include "hipq_internal.h"
-#include "hipq_math.h"
+#include "hipq_gemm_kernels.h"
 
 namespace hipq {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-
-enum { EPI_I32 = 0, EPI_F32 = 1, EPI_I8 = 2 };
-
-struct GemmEpilogue {
-    const float *sa;    // activation scale(s)
-    int sa_per_row;     // 0: sa[0], 1: sa[m]
-    const float *sw;    // [N]
-    const float *bias;  // [N] or null
-    float s_out;        // requantize only
-    int zp_out;
-    void *out;  // int32 / float / int8 [M,N]
-#ifdef HIPQ_GEMM_TRACE
-    long long *ts = nullptr;  // per-wave phase timestamps
-#endif
-};
-
-constexpr int kGemmThreads = 256;
-
-template <int EPI, bool EVEN>
-__device__ __forceinline__ void epilogue_store4(const GemmEpilogue &ep, int m, int n, int N, v4i acc, float s_a) {
-    const size_t off = size_t(m) * N + n;
-    constexpr unsigned kAlignMask = (EPI == EPI_I8) ? 3u : 15u;
-    const bool vec = (N % 4 == 0) && (n + 3 < N) && ((reinterpret_cast<uintptr_t>(ep.out) & kAlignMask) == 0);
-    if constexpr (EPI == EPI_I32) {
-        int32_t *o = static_cast<int32_t *>(ep.out);
-        if (vec) {
-            *reinterpret_cast<v4i *>(o + off) = acc;
-        } else {
-            for (int r = 0; r < 4; ++r)
-                if (n + r < N) o[off + r] = acc[r];
-        }
-    } else {
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int nn = (n + r < N) ? n + r : N - 1;
-            const float s = s_a * ep.sw[nn];
-            float t = static_cast<float>(acc[r]) * s;
-            if (ep.bias) t = t + ep.bias[nn];
-            v[r] = t;
-        }
-        if constexpr (EPI == EPI_F32) {
-            float *o = static_cast<float *>(ep.out);
-            if (vec) {
-                *reinterpret_cast<float4 *>(o + off) = make_float4(v[0], v[1], v[2], v[3]);
-            } else {
-                for (int r = 0; r < 4; ++r)
-                    if (n + r < N) o[off + r] = v[r];
-            }
-        } else {
-            int8_t *o = static_cast<int8_t *>(ep.out);
-            int q[4];
-            const float zpf = static_cast<float>(ep.zp_out);
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                q[r] = to_int_nan0(clamp_keep_nan(round_mode<EVEN>(v[r] / ep.s_out) + zpf, -128.0f, 127.0f));
-            if (vec) {
-                *reinterpret_cast<uint32_t *>(o + off) = pack4(q[0], q[1], q[2], q[3]);
-            } else {
-                for (int r = 0; r < 4; ++r)
-                    if (n + r < N) o[off + r] = static_cast<int8_t>(q[r]);
-            }
-        }
-    }
-}
-
-// Maps the linear workgroup id to a tile so that the workgroups one XCD receives
-// (ids congruent modulo 8) cover a contiguous band of weight panels: a panel of
-// W is then pulled from HBM into one XCD's L2 only.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) {
-    const int nblk = tiles_m * tiles_n;
-    int b = blockIdx.x;
-    if (nblk % 8 == 0) b = (b % 8) * (nblk / 8) + b / 8;
-    *tm = b % tiles_m;
-    *tn = b / tiles_m;
-}
-
-// BM x BN output tile per workgroup, BK = 128 bytes of K per stage, WM x WN
-// waves each owning a (BM/WM) x (BN/WN) sub-tile.
-template <int BM, int BN, int WM, int WN, int EPI, bool EVEN>
-__global__ __launch_bounds__(kGemmThreads) void gemm_i8_mfma_kernel(const int8_t *__restrict__ A,
-                                                                     const int8_t *__restrict__ W, int M, int N,
-                                                                     int K, GemmEpilogue ep) {
-    constexpr int BK = 128;
-    constexpr int CPR = BK / 16;  // 16-byte chunks per tile row
-    static_assert(WM * WN * kWave == kGemmThreads, "wave grid must use the whole workgroup");
-    constexpr int TM = BM / WM, TN = BN / WN;
-    constexpr int FM = TM / 16, FN = TN / 16;
-    static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile is made of 16x16 MFMA blocks");
-    constexpr int A_CHUNKS = BM * CPR, W_CHUNKS = BN * CPR;
-    static_assert(A_CHUNKS % kGemmThreads == 0 && W_CHUNKS % kGemmThreads == 0, "tile loads divide evenly");
-    constexpr int A_PER_T = A_CHUNKS / kGemmThreads, W_PER_T = W_CHUNKS / kGemmThreads;
-    constexpr int STAGE = (BM + BN) * BK;
-
-    __shared__ __attribute__((aligned(16))) int8_t lds[2 * STAGE];
-
-    int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    const int wm = wave % WM, wn = wave / WM;
-
-    v4i acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
-
-    v4i ra[A_PER_T], rw[W_PER_T];
-    const v4i zero = v4i{0, 0, 0, 0};
-
-    auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < A_PER_T; ++i) {
-            const int c = tid + i * kGemmThreads;
-            const int row = c / CPR, col = c % CPR;
-            const int gm = m0 + row, gk = k0 + col * 16;
-            ra[i] = (gm < M && gk < K) ? *reinterpret_cast<const v4i *>(A + size_t(gm) * K + gk) : zero;
-        }
-#pragma unroll
-        for (int i = 0; i < W_PER_T; ++i) {
-            const int c = tid + i * kGemmThreads;
-            const int row = c / CPR, col = c % CPR;
-            const int gn = n0 + row, gk = k0 + col * 16;
-            rw[i] = (gn < N && gk < K) ? *reinterpret_cast<const v4i *>(W + size_t(gn) * K + gk) : zero;
-        }
-    };
-    auto store_lds = [&](int stage) {
-        int8_t *sa = lds + stage * STAGE;
-        int8_t *sw = sa + BM * BK;
-#pragma unroll
-        for (int i = 0; i < A_PER_T; ++i) {
-            const int c = tid + i * kGemmThreads;
-            const int row = c / CPR, col = c % CPR;
-            *reinterpret_cast<v4i *>(sa + row * BK + ((col ^ (row & (CPR - 1))) * 16)) = ra[i];
-        }
-#pragma unroll
-        for (int i = 0; i < W_PER_T; ++i) {
-            const int c = tid + i * kGemmThreads;
-            const int row = c / CPR, col = c % CPR;
-            *reinterpret_cast<v4i *>(sw + row * BK + ((col ^ (row & (CPR - 1))) * 16)) = rw[i];
-        }
-    };
-
-    const int nk = (K + BK - 1) / BK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-
-    const int frow = lane % 16, fcol = lane / 16;
-    for (int kt = 0; kt < nk; ++kt) {
-        if (kt + 1 < nk) load_global((kt + 1) * BK);
-        const int8_t *sa = lds + (kt & 1) * STAGE;
-        const int8_t *sw = sa + BM * BK;
-#pragma unroll
-        for (int ks = 0; ks < BK / 64; ++ks) {
-            v4i fa[FM], fw[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const int row = wm * TM + i * 16 + frow;
-                const int col = ks * 4 + fcol;
-                fa[i] = *reinterpret_cast<const v4i *>(sa + row * BK + ((col ^ (row & (CPR - 1))) * 16));
-            }
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const int row = wn * TN + j * 16 + frow;
-                const int col = ks * 4 + fcol;
-                fw[j] = *reinterpret_cast<const v4i *>(sw + row * BK + ((col ^ (row & (CPR - 1))) * 16));
-            }
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[j], fa[i], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) store_lds((kt + 1) & 1);
-        __syncthreads();
-    }
-
-    // D = Wfrag (rows: n) x Afrag (cols: m): lane holds m = lane%16, n = 4*(lane/16)+r.
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        const int m = m0 + wm * TM + i * 16 + (lane % 16);
-        if (m >= M) continue;
-        float s_a = 1.0f;
-        if constexpr (EPI != EPI_I32) s_a = ep.sa_per_row ? ep.sa[m] : ep.sa[0];
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int n = n0 + wn * TN + j * 16 + 4 * (lane / 16);
-            if (n >= N) continue;
-            epilogue_store4<EPI, EVEN>(ep, m, n, N, acc[i][j], s_a);
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Deep-pipelined kernel for K % 128 == 0 (the shapes that matter).
-//
-// Occupancy for the headline shape is one workgroup per CU (256 tiles on 256
-// CUs), so all latency hiding happens inside the workgroup:
-//   * STAGES K-tiles of 128 bytes live in LDS (up to 144 KiB of the CU's 160 KiB)
-//     and are filled by global_load_lds_dwordx4, which moves 16 bytes per lane
-//     from global memory straight into LDS without passing through VGPRs.  A
-//     wave instruction fills 1 KiB of contiguous LDS, so the XOR swizzle is
-//     applied on the global side: lane l fetches the chunk that belongs in slot l.
-//   * the MFMA fragments of stage kt+1 are read from LDS into a second register
-//     set while the MFMAs of stage kt run, so LDS latency is off the MFMA path
-//     even with a single wave per SIMD.
-//   * vmcnt counts a wave's outstanding fills in order; waiting until only the
-//     newest stages are outstanding, then a bare workgroup barrier, publishes a
-//     stage to every wave and frees the buffer that the next fill reuses.
-// v_mfma_i32_32x32x32_i8 is used (it sustains a higher rate than the 16x16x64
-// form with one wave per SIMD).  The activation fragment is the row operand and
-// the weight fragment the column operand, so a lane owns one output channel n
-// and a wave-wide dword store writes 128 contiguous bytes of two output rows.
-//
-// Wave roles: WM x WN x WK.  WK > 1 splits the four k-steps of a stage between
-// waves; the partial accumulators are summed through LDS after the main loop.
-// Integer addition is associative, so the result is bit-identical for every WK.
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    // gfx9 s_waitcnt encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
-}
-
-__device__ __forceinline__ void wait_lgkmcnt0() {
-    __builtin_amdgcn_s_waitcnt(0xF | (0x3 << 14) | (0x7 << 4) | (0x0 << 8));
-}
-
-template <int PER_STAGE, int MAX_STAGES>
-__device__ __forceinline__ void wait_stages_outstanding(int stages) {
-    // `stages` is wave-uniform; the immediate of s_waitcnt must be a constant.
-    if constexpr (MAX_STAGES > 0) {
-        if (stages >= MAX_STAGES) {
-            wait_vmcnt<PER_STAGE * MAX_STAGES>();
-            return;
-        }
-        wait_stages_outstanding<PER_STAGE, MAX_STAGES - 1>(stages);
-    } else {
-        wait_vmcnt<0>();
-    }
-}
-
-// PW producer waves do nothing but issue the fills; WM*WN*WK consumer waves do
-// nothing but LDS reads and MFMAs.  A wave issues in order, and a fill blocks its
-// wave while the texture path is busy, so mixing fills and MFMAs in one wave
-// serialises the two pipes; with the roles split, MFMA issue never waits behind a
-// memory instruction.  All waves meet at one barrier per K-tile.
-template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN>
-__global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kernel(const int8_t *__restrict__ A,
-                                                                                    const int8_t *__restrict__ W,
-                                                                                    int M, int N, int K,
-                                                                                    GemmEpilogue ep) {
-    constexpr int BK = 128;
-    constexpr int CPR = BK / 16;   // 16-byte chunks per tile row
-    constexpr int RPI = 1024 / BK;  // tile rows filled by one wave-wide 1 KiB load
-    constexpr int IPS = (BM + BN) / RPI;  // load instructions per stage
-    static_assert(BM % RPI == 0 && IPS % PW == 0, "stage loads divide evenly between producer waves");
-    constexpr int IPW = IPS / PW;
-    static_assert(IPW * STAGES < 64, "outstanding loads must fit vmcnt");
-    constexpr int STAGE = (BM + BN) * BK;
-    constexpr int TM = BM / WM, TN = BN / WN;
-    constexpr int FM = TM / 32, FN = TN / 32;
-    static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
-    constexpr int KS = BK / 32;  // MFMA k-steps per stage
-    static_assert(KS % WK == 0, "k-steps of a stage divide between the K-split waves");
-    constexpr int KSW = KS / WK;
-    static_assert(FM % WK == 0, "after the K-split reduction each wave owns FM/WK row blocks");
-    constexpr int RED_BYTES = WM * WN * FM * (WK - 1) * FN * 4 * kWave * 16;
-    static_assert(RED_BYTES <= STAGES * STAGE, "partial sums fit the pipeline buffers");
-
-    extern __shared__ __attribute__((aligned(1024))) int8_t lds[];
-
-    int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    const int nk = K / BK;
-
-#ifdef HIPQ_GEMM_TRACE
-    long long tr[5] = {clock64(), 0, 0, 0, 0};
-#define HIPQ_TS(i) tr[i] = clock64()
-#define HIPQ_TS_FLUSH() if (ep.ts && lane == 0) { long long *o = ep.ts + (size_t(blockIdx.x) * 16 + wave) * 5; for (int q = 0; q < 5; ++q) o[q] = tr[q]; }
-#else
-#define HIPQ_TS(i)
-#define HIPQ_TS_FLUSH()
-#endif
-    if (wave < PW) {
-        // ---------------- producer ----------------
-        const int8_t *src[IPW];
-#pragma unroll
-        for (int j = 0; j < IPW; ++j) {
-            const int q = wave * IPW + j;
-            const int trow = q * RPI + lane / CPR;  // row in the stacked [A rows | W rows] tile
-            const int col = (lane % CPR) ^ ((trow >> 1) & 7);
-            if (trow < BM) {
-                int gm = m0 + trow;
-                gm = gm < M ? gm : M - 1;  // rows past the edge are computed and discarded
-                src[j] = A + size_t(gm) * K + col * 16;
-            } else {
-                int gn = n0 + (trow - BM);
-                gn = gn < N ? gn : N - 1;
-                src[j] = W + size_t(gn) * K + col * 16;
-            }
-        }
-        auto issue_stage = [&](int kt, int buf) {
-            int8_t *base = lds + buf * STAGE + wave * (IPW * 1024);
-#pragma unroll
-            for (int j = 0; j < IPW; ++j)
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void *)(src[j] + size_t(kt) * BK),
-                    (__attribute__((address_space(3))) void *)(base + j * 1024), 16, 0, 0);
-        };
-        // Two stages before the first barrier so the consumers start after one memory
-        // latency; the remaining buffers are requested while they work on stage 0.
-        int issued = 0;  // stages [0, issued) have been requested
-        for (; issued < 2 && issued < nk; ++issued) issue_stage(issued, issued);
-        wait_stages_outstanding<IPW, STAGES - 1>(issued - 1);  // stage 0 has landed
-        __builtin_amdgcn_s_barrier();
-        HIPQ_TS(1);
-        for (; issued < STAGES && issued < nk; ++issued) issue_stage(issued, issued);
-        for (int kt = 0; kt < nk; ++kt) {
-            // Requests so far cover stages <= kt+STAGES-1; stage kt+1 must have landed.
-            int newer = nk - 2 - kt;
-            if (newer > STAGES - 2) newer = STAGES - 2;
-            if (newer < 0) newer = 0;
-            wait_stages_outstanding<IPW, STAGES - 2>(newer);
-            // A bare barrier: __syncthreads() carries a release fence that would drain every
-            // outstanding fill (vmcnt(0)) and serialise the pipeline.
-            __builtin_amdgcn_s_barrier();
-            // Every consumer holds stage kt in registers: its buffer is free for stage kt+STAGES.
-            if (kt + STAGES < nk) issue_stage(kt + STAGES, kt % STAGES);
-        }
-        HIPQ_TS(2);
-        if constexpr (WK > 1) {
-            __syncthreads();
-            __syncthreads();
-        }
-        HIPQ_TS(3);
-        HIPQ_TS_FLUSH();
-        return;
-    }
-
-    // ---------------- consumer ----------------
-    const int cw = wave - PW;
-    const int wk = cw / (WM * WN), wmn = cw % (WM * WN);
-    const int wm = wmn % WM, wn = wmn / WM;
-
-    // Epilogue operands are fetched now so their latency hides behind the main loop.
-    float swv[FN], bv[FN], sa0 = 1.0f;
-    int nn[FN];
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-        nn[j] = n0 + wn * TN + j * 32 + lane % 32;
-        const int nc = nn[j] < N ? nn[j] : N - 1;
-        swv[j] = 1.0f;
-        bv[j] = 0.0f;
-        if constexpr (EPI != EPI_I32) {
-            swv[j] = ep.sw[nc];
-            if (ep.bias) bv[j] = ep.bias[nc];
-        }
-    }
-    if constexpr (EPI != EPI_I32)
-        if (!ep.sa_per_row) sa0 = ep.sa[0];
-
-    // LDS byte offsets (within a stage) of this lane's fragment reads.
-    int offA[FM][KSW], offW[FN][KSW];
-#pragma unroll
-    for (int s = 0; s < KSW; ++s) {
-        const int col = (s * WK + wk) * 2 + lane / 32;
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            const int row = wm * TM + i * 32 + lane % 32;
-            offA[i][s] = row * BK + ((col ^ ((row >> 1) & 7)) * 16);
-        }
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int row = BM + wn * TN + j * 32 + lane % 32;  // stacked-tile row
-            offW[j][s] = row * BK + ((col ^ ((row >> 1) & 7)) * 16);
-        }
-    }
-    v4i fa[2][KSW][FM], fw[2][KSW][FN];
-    auto read_frags = [&](int buf, int set) {
-        const int8_t *st = lds + buf * STAGE;
-#pragma unroll
-        for (int s = 0; s < KSW; ++s) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i) fa[set][s][i] = *reinterpret_cast<const v4i *>(st + offA[i][s]);
-#pragma unroll
-            for (int j = 0; j < FN; ++j) fw[set][s][j] = *reinterpret_cast<const v4i *>(st + offW[j][s]);
-        }
-    };
-
-    v16i acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    auto compute = [&](int set) {
-#pragma unroll
-        for (int s = 0; s < KSW; ++s)
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][s][i], fw[set][s][j], acc[i][j], 0, 0, 0);
-    };
-    auto iteration = [&](int kt, int set) {
-        wait_lgkmcnt0();  // this wave's fragment reads of stage kt are in registers
-        asm volatile("" ::: "memory");  // compiler-only fence: keep LDS reads on their side of the barrier
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        // Unconditional: after the last stage this re-reads a resident buffer whose values are
-        // never used, which keeps reads and MFMAs in one basic block for the interleave below.
-        read_frags((kt + 1) % STAGES, set ^ 1);
-        compute(set);
-        // Issue order: one MFMA, then one fragment read, ...: the reads slip into the issue
-        // slots between MFMAs (an MFMA occupies the matrix pipe for 32 cycles) instead of
-        // delaying the first MFMA of the stage.
-#pragma unroll
-        for (int q = 0; q < KSW * FM * FN; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (q < KSW * (FM + FN)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-    };
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();  // stage 0 published
-    asm volatile("" ::: "memory");
-    read_frags(0, 0);
-    HIPQ_TS(1);
-    int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-        iteration(kt, 0);
-        iteration(kt + 1, 1);
-    }
-    if (kt < nk) iteration(kt, 0);
-    HIPQ_TS(2);
-
-    if constexpr (WK > 1) {
-        // Sum the K-split partials through LDS.  Row block i of a wave-group tile is owned
-        // by wave (i % WK); every other wave of the group parks its partial for it.
-        __syncthreads();
-        v4i *red = reinterpret_cast<v4i *>(lds);
-        auto slot = [&](int i, int srcw, int j, int g) {
-            const int owner = i % WK;
-            const int sidx = (srcw - owner - 1 + WK) % WK;  // 0 .. WK-2
-            return ((((wmn * FM + i) * (WK - 1) + sidx) * FN + j) * 4 + g) * kWave + lane;
-        };
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            if (i % WK == wk) continue;
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int g = 0; g < 4; ++g)
-                    red[slot(i, wk, j, g)] =
-                        v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            if (i % WK != wk) continue;
-#pragma unroll
-            for (int p = 1; p < WK; ++p) {
-                const int srcw = (wk + p) % WK;
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const v4i t = red[slot(i, srcw, j, g)];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] += t[r];
-                    }
-            }
-        }
-    }
-
-    HIPQ_TS(3);
-    // Epilogue.  32x32 accumulator block: lane holds column n = lane%32 and rows
-    // m = 8*(r/4) + 4*(lane/32) + r%4 for r = 0..15.
-    const float zpf = static_cast<float>(ep.zp_out);
-    const bool has_bias = ep.bias != nullptr;
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        if (WK > 1 && i % WK != wk) continue;
-        // All loads of the row block first, then arithmetic and stores only: a load between
-        // stores would wait for every earlier store to retire (stores count in vmcnt too).
-        float s_row[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s_row[r] = sa0;
-        if constexpr (EPI != EPI_I32) {
-            if (ep.sa_per_row) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-                    s_row[r] = ep.sa[m < M ? m : M - 1];
-                }
-            }
-        }
-        // Combined scales for the whole row block, computed before the first store so that no
-        // loaded value is first touched between stores.
-        float s_comb[16][FN];
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-#pragma unroll
-            for (int j = 0; j < FN; ++j) s_comb[r][j] = s_row[r] * swv[j];
-        // Every load of this wave has landed (and the compiler's wait tracking knows it), so
-        // the stores below are issued back to back without waiting on one another.
-        wait_vmcnt<0>();
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-            if (m >= M) continue;
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                if (nn[j] >= N) continue;
-                const size_t off = size_t(m) * N + nn[j];
-                if constexpr (EPI == EPI_I32) {
-                    static_cast<int32_t *>(ep.out)[off] = acc[i][j][r];
-                } else {
-                    float v = static_cast<float>(acc[i][j][r]) * s_comb[r][j];
-                    if (has_bias) v = v + bv[j];
-                    if constexpr (EPI == EPI_F32) {
-                        static_cast<float *>(ep.out)[off] = v;
-                    } else {
-                        const float q = clamp_keep_nan(round_mode<EVEN>(v / ep.s_out) + zpf, -128.0f, 127.0f);
-                        static_cast<int8_t *>(ep.out)[off] = static_cast<int8_t>(to_int_nan0(q));
-                    }
-                }
-            }
-        }
-    }
-    HIPQ_TS(4);
-    HIPQ_TS_FLUSH();
-}
 
 // ---------------------------------------------------------------------------
 // Skinny GEMM (M <= 16: decode-shaped Linear).  The weight matrix is read exactly
@@ -723,25 +178,6 @@ static void launch_tile(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, 
     const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     hipLaunchKernelGGL((gemm_i8_mfma_kernel<BM, BN, WM, WN, EPI, EVEN>), dim3(tiles), dim3(kGemmThreads), 0,
                        ctx->stream, a, w, M, N, K, ep);
-}
-
-template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN>
-static int32_t launch_pipe(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, int N, int K,
-                           const GemmEpilogue &ep) {
-    constexpr int kLds = STAGES * (BM + BN) * 128;
-    constexpr int kThreads = (PW + WM * WN * WK) * kWave;
-    auto kernel = gemm_i8_pipe_kernel<BM, BN, STAGES, PW, WM, WN, WK, EPI, EVEN>;
-    static bool configured[16] = {false};  // per device: raise the dynamic LDS limit once
-    if (ctx->device < 16 && !configured[ctx->device]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        if (e != hipSuccess)
-            return fail(HIPQ_DEVICE_ERROR, "gemm_i8: cannot reserve %d bytes of LDS: %s", kLds, hipGetErrorString(e));
-        configured[ctx->device] = true;
-    }
-    const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    hipLaunchKernelGGL(kernel, dim3(tiles), dim3(kThreads), kLds, ctx->stream, a, w, M, N, K, ep);
-    return check_launch("gemm_i8 (pipelined)");
 }
 
 // Tuning hook: HIPQ_GEMM_VARIANT=<n> forces one kernel configuration (0 = automatic).

@@ -71,6 +71,10 @@ _SIGNATURES = {
     "hipq_linear_i8_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _f32, _i32, _i32, _vp],
     "hipq_requantize_i32_i8": [_vp, _vp, _sz, _sz, _vp, _i32, _vp, _vp, _f32, _i32, _i32, _vp],
     "hipq_linear_dynamic_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
+    "hipq_conv2d_u8i8_i32": [_vp, _vp, _i32, _vp] + [_sz] * 11 + [_vp],
+    "hipq_conv2d_u8i8_i8": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_f32, _i32, _i32, _vp],
+    "hipq_conv2d_pack_weights_i8": [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp],
+    "hipq_conv2d_u8i8_i8_packed": [_vp, _vp, _i32, _f32, _vp, _vp, _vp, _vp] + [_sz] * 9 + [_f32, _i32, _i32, _vp],
 }
 
 _SPECIAL = {
@@ -317,4 +321,50 @@ class Context:
         out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
         self.call("hipq_linear_dynamic_f32", _ptr(x), int(per_token), _ptr(w), _ptr(w_scales), _ptr(bias), m, n, k,
                   mode, _ptr(out))
+        return out
+
+    def conv2d_i32(self, x_u8, zp_in, w_i8, stride=(1, 1), padding=(0, 0)):
+        nb, c, h, wd = x_u8.shape
+        oc, c2, kh, kw = w_i8.shape
+        if c != c2:
+            raise HipqError(DIMENSION_MISMATCH, f"qconv2d channel mismatch: input C_in={c} but weight C_in={c2}")
+        ho = max((h + 2 * padding[0] - kh) // stride[0] + 1, 0)  # the library rejects impossible geometry
+        wo = max((wd + 2 * padding[1] - kw) // stride[1] + 1, 0)
+        out = torch.empty((nb, oc, ho, wo), dtype=torch.int32, device=self._dev())
+        self.call("hipq_conv2d_u8i8_i32", _ptr(x_u8), int(zp_in), _ptr(w_i8), nb, c, h, wd, oc, kh, kw, stride[0],
+                  stride[1], padding[0], padding[1], _ptr(out))
+        return out
+
+    def conv2d_i8(self, x_u8, zp_in, s_in, w_i8, w_scales, bias, s_out, zp_out, stride=(1, 1), padding=(0, 0), mode=0,
+                  out=None):
+        nb, c, h, wd = x_u8.shape
+        oc, c2, kh, kw = w_i8.shape
+        if c != c2:
+            raise HipqError(DIMENSION_MISMATCH, f"qconv2d channel mismatch: input C_in={c} but weight C_in={c2}")
+        ho = max((h + 2 * padding[0] - kh) // stride[0] + 1, 0)  # the library rejects impossible geometry
+        wo = max((wd + 2 * padding[1] - kw) // stride[1] + 1, 0)
+        out = out if out is not None else torch.empty((nb, oc, ho, wo), dtype=torch.int8, device=self._dev())
+        self.call("hipq_conv2d_u8i8_i8", _ptr(x_u8), int(zp_in), float(s_in), _ptr(w_i8), _ptr(w_scales), _ptr(bias), nb,
+                  c, h, wd, oc, kh, kw, stride[0], stride[1], padding[0], padding[1], float(s_out), int(zp_out), mode,
+                  _ptr(out))
+        return out
+
+    def conv2d_pack_weights(self, w_i8):
+        oc, ic, kh, kw = w_i8.shape
+        packed = torch.empty((oc, kh * kw, ic), dtype=torch.int8, device=self._dev())
+        sums = torch.empty(oc, dtype=torch.int32, device=self._dev())
+        self.call("hipq_conv2d_pack_weights_i8", _ptr(w_i8), oc, ic, kh, kw, _ptr(packed), _ptr(sums))
+        return packed, sums
+
+    def conv2d_i8_packed(self, x_u8, zp_in, s_in, w_packed, w_sums, kernel, w_scales, bias, s_out, zp_out,
+                         padding=(0, 0), mode=0, out=None):
+        nb, c, h, wd = x_u8.shape
+        oc = w_packed.shape[0]
+        kh, kw = kernel
+        ho = h + 2 * padding[0] - kh + 1
+        wo = wd + 2 * padding[1] - kw + 1
+        out = out if out is not None else torch.empty((nb, oc, ho, wo), dtype=torch.int8, device=self._dev())
+        self.call("hipq_conv2d_u8i8_i8_packed", _ptr(x_u8), int(zp_in), float(s_in), _ptr(w_packed), _ptr(w_sums),
+                  _ptr(w_scales), _ptr(bias), nb, c, h, wd, oc, kh, kw, padding[0], padding[1], float(s_out),
+                  int(zp_out), mode, _ptr(out))
         return out
