@@ -176,6 +176,12 @@ HIPQ_API int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t 
 HIPQ_API int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
                                               int32_t flavor, int32_t mode, int8_t *out, float *out_scales,
                                               int32_t *out_zero_points, int32_t *out_status);
+/* The same for rows that are `ld` elements apart in memory (a column slice of
+ * a wider matrix); the int8 output is dense [rows, cols]. */
+HIPQ_API int32_t hipq_quantize_per_row_strided_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
+                                                      size_t ld, int32_t flavor, int32_t mode, int8_t *out,
+                                                      float *out_scales, int32_t *out_zero_points,
+                                                      int32_t *out_status);
 /* quantize_per_channel_auto for any axis of a dense tensor viewed as
  * [outer, channels, inner] (algorithms.rs:126-242). */
 HIPQ_API int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer,
@@ -209,6 +215,13 @@ HIPQ_API int32_t hipq_gemm_i8_i32(hipq_ctx *ctx, const int8_t *a, const int8_t *
 HIPQ_API int32_t hipq_linear_i8_f32(hipq_ctx *ctx, const int8_t *a, const float *a_scale,
                                     int32_t a_scale_per_row, const int8_t *w, const float *w_scales,
                                     const float *bias, size_t m, size_t n, size_t k, float *out);
+/* hipq_linear_i8_f32 with a residual added after the bias:
+ * out = acc * (s_a * s_w[n]) + bias[n] + residual[m,n]; out may alias residual
+ * (Linear followed by the `.add()` of a skip connection). */
+HIPQ_API int32_t hipq_linear_i8_f32_residual(hipq_ctx *ctx, const int8_t *a, const float *a_scale,
+                                             int32_t a_scale_per_row, const int8_t *w, const float *w_scales,
+                                             const float *bias, const float *residual, size_t m, size_t n, size_t k,
+                                             float *out);
 /* Same accumulators, requantizing epilogue (tail of operations.rs:716-724 with
  * a supplied output scale): q = clamp(round(v / s_out) + zp_out, -128, 127). */
 HIPQ_API int32_t hipq_linear_i8_i8(hipq_ctx *ctx, const int8_t *a, const float *a_scale, int32_t a_scale_per_row,
@@ -258,6 +271,49 @@ HIPQ_API int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int
                                             const float *bias, size_t nb, size_t c, size_t h, size_t wd, size_t oc,
                                             size_t kh, size_t kw, size_t pad_h, size_t pad_w, float out_scale,
                                             int32_t out_zero_point, int32_t mode, int8_t *out);
+
+/* ---- fp32 helpers of the int8 transformer stack ------------------------- */
+/* LayerNorm over the last dimension (biased variance, eps inside the square
+ * root, eps 1e-5 by default: crates/torsh-nn/src/layers/normalization/layer_group/mod.rs:130-166,660).
+ * gamma / beta [cols] may be NULL.  cols % 4 == 0, cols <= 8192. */
+HIPQ_API int32_t hipq_layer_norm_f32(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
+                                     const float *beta, float eps, float *out);
+/* LayerNorm followed by the per-token symmetric int8 quantizer
+ * (quantize_per_channel_auto on axis 0, algorithms.rs:126-242) in one pass. */
+HIPQ_API int32_t hipq_layer_norm_quantize_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
+                                                 const float *gamma, const float *beta, float eps, int32_t mode,
+                                                 int8_t *out, float *out_scales);
+/* tanh-form GELU, crates/torsh-nn/src/layers/activation/modern.rs:124-136. */
+HIPQ_API int32_t hipq_gelu_tanh_f32(hipq_ctx *ctx, const float *x, size_t n, float *out);
+/* GELU followed by the per-token symmetric int8 quantizer in one pass. */
+HIPQ_API int32_t hipq_gelu_tanh_quantize_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
+                                                int8_t *out, float *out_scales);
+/* out = a + b (skip connection; Tensor::add). */
+HIPQ_API int32_t hipq_add_f32(hipq_ctx *ctx, const float *a, const float *b, size_t n, float *out);
+
+/* Device pointers of one block of the projection stack: every Linear is
+ * per-output-channel int8 ([out,in] weights, [out] scales, [out] fp32 bias). */
+typedef struct hipq_block_weights {
+    const float *ln1_gamma, *ln1_beta, *ln2_gamma, *ln2_beta;
+    const int8_t *w_qkv;
+    const float *s_qkv, *b_qkv; /* [3d, d] */
+    const int8_t *w_out;
+    const float *s_out, *b_out; /* [d, d] */
+    const int8_t *w_fc1;
+    const float *s_fc1, *b_fc1; /* [d_ff, d] */
+    const int8_t *w_fc2;
+    const float *s_fc2, *b_fc2; /* [d, d_ff] */
+} hipq_block_weights;
+/* Bytes of device workspace hipq_transformer_stack_forward_f32 needs. */
+HIPQ_API size_t hipq_transformer_stack_workspace_bytes(size_t tokens, size_t d_model, size_t d_ff);
+/* Forward of n_layers blocks on x [tokens, d_model] in place: per block
+ *   x += Linear_out(quant(V(Linear_qkv(quant(LN1(x))))));  x += Linear_fc2(quant(GELU(Linear_fc1(quant(LN2(x))))))
+ * with per-token dynamic int8 activations, LayerNorm and GELU in fp32, and the
+ * attention mixing replaced by a pass-through of the value slice (it is not part
+ * of the quantized path).  `blocks` is a HOST array of n_layers records. */
+HIPQ_API int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_block_weights *blocks, size_t n_layers,
+                                                    size_t tokens, size_t d_model, size_t d_ff, float eps,
+                                                    int32_t mode, float *x, void *workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -245,7 +245,8 @@ __global__ __launch_bounds__(kBlock) void dequantize_kernel(const InT *__restric
 // with the division form.
 template <int TPR, bool EVEN>
 __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *__restrict__ x, size_t rows,
-                                                                   size_t cols, int flavor, int qmin, int qmax,
+                                                                   size_t cols, size_t ld, int flavor, int qmin,
+                                                                   int qmax,
                                                                    int8_t *__restrict__ out,
                                                                    float *__restrict__ out_scales,
                                                                    int32_t *__restrict__ out_zps,
@@ -256,9 +257,9 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
     const size_t row = size_t(blockIdx.x) * kRowsPerBlock + sub;
     const bool active = row < rows;
-    const float *xr = x + (active ? row : 0) * cols;
+    const float *xr = x + (active ? row : 0) * ld;  // input rows are ld elements apart, output is dense
     int8_t *qr = out + (active ? row : 0) * cols;
-    const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (cols % 4 == 0) &&
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (cols % 4 == 0) && (ld % 4 == 0) &&
                          ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
     const size_t nvec = aligned ? cols / 4 : 0;
     const float4 *x4 = reinterpret_cast<const float4 *>(xr);
@@ -630,9 +631,9 @@ int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t *q, size_
     return dequant_common<int8_t>(__func__, ctx, q, n, 1.0f, 0, params, out);
 }
 
-int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t flavor,
-                                     int32_t mode, int8_t *out, float *out_scales, int32_t *out_zero_points,
-                                     int32_t *out_status) {
+int32_t hipq_quantize_per_row_strided_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
+                                             int32_t flavor, int32_t mode, int8_t *out, float *out_scales,
+                                             int32_t *out_zero_points, int32_t *out_status) {
     HIPQ_ENTER(ctx);
     int32_t rc = check_row_flavor(__func__, flavor);
     if (rc) return rc;
@@ -640,6 +641,7 @@ int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows,
     if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
     if (rows == 0) return check_launch(__func__);
     if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length have no range", __func__);
+    if (ld < cols) return fail(HIPQ_INVALID_ARGUMENT, "%s: row stride %zu smaller than the row length %zu", __func__, ld, cols);
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
     const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
@@ -648,20 +650,27 @@ int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows,
         const int grid = static_cast<int>(rows);
         if (even)
             hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
         else
             hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
     } else {
         const int grid = static_cast<int>((rows + 3) / 4);
         if (even)
             hipLaunchKernelGGL((quantize_per_row_kernel<kWave, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
         else
             hipLaunchKernelGGL((quantize_per_row_kernel<kWave, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
     }
     return check_launch(__func__);
+}
+
+int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t flavor,
+                                     int32_t mode, int8_t *out, float *out_scales, int32_t *out_zero_points,
+                                     int32_t *out_status) {
+    return hipq_quantize_per_row_strided_f32_i8(ctx, x, rows, cols, cols, flavor, mode, out, out_scales,
+                                                out_zero_points, out_status);
 }
 
 int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels,

@@ -1,0 +1,275 @@
+// fp32 helpers of the int8 transformer stack: LayerNorm, tanh-GELU, residual add,
+// and the fused forms that hand their result straight to the per-token int8
+// quantizer (the normalised / activated row never makes a round trip through HBM
+// as fp32).  One wavefront or one workgroup owns a row and keeps it in registers:
+// a single HBM read per element, wave shuffles for the row statistics.
+#include "hipq_internal.h"
+#include "hipq_math.h"
+
+namespace hipq {
+
+constexpr int kRowBlock = 256;
+constexpr int kRowCache = 8;  // float4 per thread kept in registers
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float *lds) {
+    v = wave_sum(v);
+    if constexpr (TPR == kWave) {
+        return v;
+    } else {
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        __syncthreads();
+        if (lane == 0) lds[wave] = v;
+        __syncthreads();
+        float r = 0.0f;
+#pragma unroll
+        for (int w = 0; w < TPR / kWave; ++w) r += lds[w];
+        return r;
+    }
+}
+
+template <int TPR>
+__device__ __forceinline__ float row_max(float v, float *lds) {
+    v = wave_max(v);
+    if constexpr (TPR == kWave) {
+        return v;
+    } else {
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        __syncthreads();
+        if (lane == 0) lds[wave] = v;
+        __syncthreads();
+        float r = lds[0];
+#pragma unroll
+        for (int w = 1; w < TPR / kWave; ++w) r = fmaxf(r, lds[w]);
+        return r;
+    }
+}
+
+// tanh-form GELU, crates/torsh-nn/src/layers/activation/modern.rs:124-136.
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float x3 = x * x * x;
+    const float inner = (x + x3 * 0.044715f) * 0.7978845608028654f;  // sqrt(2/pi)
+    return (x * 0.5f) * (tanhf(inner) + 1.0f);
+}
+
+enum { ROW_LAYERNORM = 0, ROW_GELU = 1 };
+
+// OP: LayerNorm over the row (biased variance, eps inside the square root) or GELU.
+// QUANT: write the row as per-token symmetric int8 (scale = absmax/127,
+// q = clamp(round(y / scale)), the division form of
+// crates/torsh-quantization/src/algorithms.rs:126-242) instead of fp32.
+// Rows are TPR threads wide and at most TPR * kRowCache * 4 columns long; cols % 4 == 0.
+template <int TPR, int OP, bool QUANT, bool EVEN>
+__global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restrict__ x, size_t rows, size_t cols,
+                                                            const float *__restrict__ gamma,
+                                                            const float *__restrict__ beta, float eps,
+                                                            float *__restrict__ out_f, int8_t *__restrict__ out_q,
+                                                            float *__restrict__ out_scales) {
+    constexpr int kRowsPerBlock = kRowBlock / TPR;
+    __shared__ float lds[kRowBlock / kWave];
+    const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
+    const size_t row = size_t(blockIdx.x) * kRowsPerBlock + sub;
+    const bool active = row < rows;
+    const size_t nvec = cols / 4;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x + (active ? row : 0) * cols);
+    float4 v[kRowCache];
+#pragma unroll
+    for (int i = 0; i < kRowCache; ++i) {
+        const size_t idx = size_t(lane) + size_t(i) * TPR;
+        v[i] = (active && idx < nvec) ? x4[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if constexpr (OP == ROW_LAYERNORM) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        const float mean = row_sum<TPR>(s, lds) / static_cast<float>(cols);
+        float sq = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            if (idx < nvec) {
+                const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+                sq += (a * a + b * b) + (c * c + d * d);
+            }
+        }
+        const float var = row_sum<TPR>(sq, lds) / static_cast<float>(cols);
+        const float rstd = 1.0f / sqrtf(var + eps);
+        const float4 *g4 = reinterpret_cast<const float4 *>(gamma), *b4 = reinterpret_cast<const float4 *>(beta);
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            if (idx < nvec) {
+                float4 y = make_float4((v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
+                                       (v[i].w - mean) * rstd);
+                if (gamma) {
+                    const float4 g = g4[idx];
+                    y = make_float4(y.x * g.x, y.y * g.y, y.z * g.z, y.w * g.w);
+                }
+                if (beta) {
+                    const float4 b = b4[idx];
+                    y = make_float4(y.x + b.x, y.y + b.y, y.z + b.z, y.w + b.w);
+                }
+                v[i] = y;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i)
+            v[i] = make_float4(gelu_tanh(v[i].x), gelu_tanh(v[i].y), gelu_tanh(v[i].z), gelu_tanh(v[i].w));
+    }
+    if constexpr (!QUANT) {
+        if (!active) return;
+        float4 *o4 = reinterpret_cast<float4 *>(out_f + row * cols);
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            if (idx < nvec) o4[idx] = v[i];
+        }
+    } else {
+        float am = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            if (idx < nvec) am = fmaxf(fmaxf(am, fmaxf(fabsf(v[i].x), fabsf(v[i].y))), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
+        }
+        am = row_max<TPR>(am, lds);
+        if (!active) return;
+        // calculate_symmetric_quantization_params, algorithms.rs:397-422 (a non-finite row
+        // yields a NaN scale, which the caller can test for).
+        float scale = am < FLT_EPSILON ? 1.0f : am / 127.0f;
+        if (!(fabsf(am) <= FLT_MAX)) scale = NAN;
+        if (lane == 0) out_scales[row] = scale;
+        uint32_t *q4 = reinterpret_cast<uint32_t *>(out_q + row * cols);
+#pragma unroll
+        for (int i = 0; i < kRowCache; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            if (idx < nvec) {
+                const float a = quantize_value<true, EVEN>(v[i].x, scale, 0.0f, 0.0f, -128.0f, 127.0f);
+                const float b = quantize_value<true, EVEN>(v[i].y, scale, 0.0f, 0.0f, -128.0f, 127.0f);
+                const float c = quantize_value<true, EVEN>(v[i].z, scale, 0.0f, 0.0f, -128.0f, 127.0f);
+                const float d = quantize_value<true, EVEN>(v[i].w, scale, 0.0f, 0.0f, -128.0f, 127.0f);
+                q4[idx] = pack4(to_int_nan0(a), to_int_nan0(b), to_int_nan0(c), to_int_nan0(d));
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void gelu_kernel(const float *__restrict__ x, size_t n, float *__restrict__ out) {
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += size_t(gridDim.x) * 256) out[i] = gelu_tanh(x[i]);
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, const float *__restrict__ b, size_t n,
+                                                   float *__restrict__ out) {
+    const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                           reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    const size_t nvec = aligned ? n / 4 : 0;
+    const float4 *a4 = reinterpret_cast<const float4 *>(a), *b4 = reinterpret_cast<const float4 *>(b);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < nvec; i += size_t(gridDim.x) * 256) {
+        const float4 p = a4[i], q = b4[i];
+        o4[i] = make_float4(p.x + q.x, p.y + q.y, p.z + q.z, p.w + q.w);
+    }
+    for (size_t i = nvec * 4 + size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += size_t(gridDim.x) * 256)
+        out[i] = a[i] + b[i];
+}
+
+template <int OP, bool QUANT>
+static int32_t launch_row_op(const char *fn, hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
+                             const float *beta, float eps, int32_t mode, float *out_f, int8_t *out_q,
+                             float *out_scales) {
+    if (rows == 0) return HIPQ_SUCCESS;
+    if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length", fn);
+    if (cols % 4 != 0 || cols > size_t(kRowBlock) * kRowCache * 4)
+        return fail(HIPQ_SHAPE_ERROR, "%s: row length %zu must be a multiple of 4 and at most %d", fn, cols,
+                    kRowBlock * kRowCache * 4);
+    uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gamma) |
+                     reinterpret_cast<uintptr_t>(beta) | reinterpret_cast<uintptr_t>(out_f);
+    if ((bits & 15u) || (reinterpret_cast<uintptr_t>(out_q) & 3u))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", fn);
+    if (rows >> 31) return fail(HIPQ_SHAPE_ERROR, "%s: too many rows", fn);
+    const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    const bool wave_rows = cols <= size_t(kWave) * kRowCache * 4;
+#define HIPQ_ROW(TPR, E)                                                                                          \
+    hipLaunchKernelGGL((row_op_kernel<TPR, OP, QUANT, E>), dim3(static_cast<int>((rows + kRowBlock / TPR - 1) / (kRowBlock / TPR))), \
+                       dim3(kRowBlock), 0, ctx->stream, x, rows, cols, gamma, beta, eps, out_f, out_q, out_scales)
+    if (wave_rows) {
+        if (even) HIPQ_ROW(kWave, true); else HIPQ_ROW(kWave, false);
+    } else {
+        if (even) HIPQ_ROW(kRowBlock, true); else HIPQ_ROW(kRowBlock, false);
+    }
+#undef HIPQ_ROW
+    return check_launch(fn);
+}
+
+}  // namespace hipq
+
+using namespace hipq;
+
+extern "C" {
+
+int32_t hipq_layer_norm_f32(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
+                            const float *beta, float eps, float *out) {
+    HIPQ_ENTER(ctx);
+    if (rows * cols != 0) {
+        HIPQ_REQUIRE_PTR(x);
+        HIPQ_REQUIRE_PTR(out);
+    }
+    return launch_row_op<ROW_LAYERNORM, false>(__func__, ctx, x, rows, cols, gamma, beta, eps, 0, out, nullptr, nullptr);
+}
+
+int32_t hipq_layer_norm_quantize_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
+                                        const float *beta, float eps, int32_t mode, int8_t *out, float *out_scales) {
+    HIPQ_ENTER(ctx);
+    if (rows * cols != 0) {
+        HIPQ_REQUIRE_PTR(x);
+        HIPQ_REQUIRE_PTR(out);
+        HIPQ_REQUIRE_PTR(out_scales);
+    }
+    return launch_row_op<ROW_LAYERNORM, true>(__func__, ctx, x, rows, cols, gamma, beta, eps, mode, nullptr, out,
+                                              out_scales);
+}
+
+int32_t hipq_gelu_tanh_f32(hipq_ctx *ctx, const float *x, size_t n, float *out) {
+    HIPQ_ENTER(ctx);
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    size_t blocks = (n + 255) / 256;
+    const size_t cap = size_t(ctx->num_cus) * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(gelu_kernel, dim3(static_cast<int>(blocks)), dim3(256), 0, ctx->stream, x, n, out);
+    return check_launch(__func__);
+}
+
+int32_t hipq_gelu_tanh_quantize_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
+                                       int8_t *out, float *out_scales) {
+    HIPQ_ENTER(ctx);
+    if (rows * cols != 0) {
+        HIPQ_REQUIRE_PTR(x);
+        HIPQ_REQUIRE_PTR(out);
+        HIPQ_REQUIRE_PTR(out_scales);
+    }
+    return launch_row_op<ROW_GELU, true>(__func__, ctx, x, rows, cols, nullptr, nullptr, 0.0f, mode, nullptr, out,
+                                         out_scales);
+}
+
+int32_t hipq_add_f32(hipq_ctx *ctx, const float *a, const float *b, size_t n, float *out) {
+    HIPQ_ENTER(ctx);
+    if (n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(a);
+    HIPQ_REQUIRE_PTR(b);
+    HIPQ_REQUIRE_PTR(out);
+    size_t blocks = (n / 4 + 255) / 256 + 1;
+    const size_t cap = size_t(ctx->num_cus) * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(add_kernel, dim3(static_cast<int>(blocks)), dim3(256), 0, ctx->stream, a, b, n, out);
+    return check_launch(__func__);
+}
+
+}  // extern "C"

@@ -109,6 +109,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemv_i8_kernel(const int8_t *__r
         }
         if constexpr (EPI == EPI_F32) {
             float *o = static_cast<float *>(ep.out);
+            if (ep.residual)
+                for (int i = 0; i < 4; ++i)
+                    if (n_out + i < N) v[i] = v[i] + ep.residual[off + i];
             if (vec) {
                 *reinterpret_cast<float4 *>(o + off) = make_float4(v[0], v[1], v[2], v[3]);
             } else {
@@ -162,6 +165,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_i8_generic_kernel(const int
             float v = static_cast<float>(acc) * s;
             if (ep.bias) v = v + ep.bias[n];
             if constexpr (EPI == EPI_F32) {
+                if (ep.residual) v = v + ep.residual[idx];
                 static_cast<float *>(ep.out)[idx] = v;
             } else {
                 const float q = clamp_keep_nan(round_mode<EVEN>(v / ep.s_out) + static_cast<float>(ep.zp_out), -128.0f,
@@ -276,6 +280,26 @@ int32_t hipq_linear_i8_f32(hipq_ctx *ctx, const int8_t *a, const float *a_scale,
         HIPQ_REQUIRE_PTR(w);
     }
     GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, 1.0f, 0, out};
+    return launch_gemm<EPI_F32, false>(ctx, a, w, m, n, k, ep);
+}
+
+int32_t hipq_linear_i8_f32_residual(hipq_ctx *ctx, const int8_t *a, const float *a_scale, int32_t a_scale_per_row,
+                                    const int8_t *w, const float *w_scales, const float *bias, const float *residual,
+                                    size_t m, size_t n, size_t k, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_gemm_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(out);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(residual);
+    if (k > 0) {
+        HIPQ_REQUIRE_PTR(a);
+        HIPQ_REQUIRE_PTR(w);
+    }
+    GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, 1.0f, 0, out};
+    ep.residual = residual;
     return launch_gemm<EPI_F32, false>(ctx, a, w, m, n, k, ep);
 }
 

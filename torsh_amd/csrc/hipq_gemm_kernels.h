@@ -21,6 +21,7 @@ struct GemmEpilogue {
     float s_out;        // requantize only
     int zp_out;
     void *out;  // int32 / float / int8 [M,N]
+    const float *residual = nullptr;  // fp32 epilogue only: added after the bias, [M,N]; may alias out
     // Implicit-GEMM convolution (pipelined kernel, CONV = 1): the column operand is a padded
     // NHWC int8 image [nb, hp, wp, c]; column q is the window whose top-left tap is padded
     // pixel q, and K runs over (tap, channel).  The row operand holds the packed filters.
@@ -58,6 +59,7 @@ __device__ __forceinline__ void epilogue_store4(const GemmEpilogue &ep, int m, i
             const float s = s_a * ep.sw[nn];
             float t = static_cast<float>(acc[r]) * s;
             if (ep.bias) t = t + ep.bias[nn];
+            if (ep.residual && n + r < N) t = t + ep.residual[off + r];
             v[r] = t;
         }
         if constexpr (EPI == EPI_F32) {
@@ -596,11 +598,25 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
         }
         // Combined scales for the whole row block, computed before the first store so that no
         // loaded value is first touched between stores.
-        float s_comb[16][FN];
+        float s_comb[16][FN], res[16][FN];
 #pragma unroll
         for (int r = 0; r < 16; ++r)
 #pragma unroll
-            for (int j = 0; j < FN; ++j) s_comb[r][j] = s_row[r] * swv[j];
+            for (int j = 0; j < FN; ++j) {
+                s_comb[r][j] = s_row[r] * swv[j];
+                res[r][j] = 0.0f;
+            }
+        if constexpr (EPI == EPI_F32) {
+            if (ep.residual) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        if (m < M && nn[j] < N) res[r][j] = ep.residual[size_t(m) * N + nn[j]];
+                }
+            }
+        }
         // Every load of this wave has landed (and the compiler's wait tracking knows it), so
         // the stores below are issued back to back without waiting on one another.
         wait_vmcnt<0>();
@@ -618,6 +634,7 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
                     float v = static_cast<float>(acc[i][j][r]) * s_comb[r][j];
                     if (has_bias) v = v + bv[j];
                     if constexpr (EPI == EPI_F32) {
+                        if (ep.residual) v = v + res[r][j];
                         static_cast<float *>(ep.out)[off] = v;
                     } else {
                         const float q = clamp_keep_nan(round_mode<EVEN>(v / ep.s_out) + zpf, -128.0f, 127.0f);

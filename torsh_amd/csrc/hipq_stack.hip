@@ -1,0 +1,74 @@
+// Forward of the int8 transformer projection stack (LayerNorm -> per-token int8 ->
+// QKV Linear -> stand-in attention -> output Linear + residual -> LayerNorm ->
+// per-token int8 -> fc1 -> GELU -> per-token int8 -> fc2 + residual), composed
+// from the library's own entry points.  Eight kernels per layer; the fp32
+// intermediates that only feed a quantizer are never written to memory.
+#include "hipq_internal.h"
+
+namespace {
+size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+}  // namespace
+
+extern "C" {
+
+size_t hipq_transformer_stack_workspace_bytes(size_t tokens, size_t d_model, size_t d_ff) {
+    const size_t widest = d_model > d_ff ? d_model : d_ff;
+    return align256(tokens * widest)                          // int8 activations
+           + align256(tokens * sizeof(float))                 // per-token scales
+           + align256(tokens * 3 * d_model * sizeof(float))   // qkv
+           + align256(tokens * d_ff * sizeof(float));         // fc1 output
+}
+
+int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_block_weights *blocks, size_t n_layers,
+                                           size_t tokens, size_t d_model, size_t d_ff, float eps, int32_t mode,
+                                           float *x, void *workspace, size_t workspace_bytes) {
+    HIPQ_ENTER(ctx);
+    if (n_layers == 0 || tokens == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(blocks);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(workspace);
+    if (d_model == 0 || d_ff == 0) return hipq::fail(HIPQ_SHAPE_ERROR, "%s: empty model dimension", __func__);
+    if (workspace_bytes < hipq_transformer_stack_workspace_bytes(tokens, d_model, d_ff))
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: workspace of %zu bytes is smaller than the %zu needed", __func__,
+                          workspace_bytes, hipq_transformer_stack_workspace_bytes(tokens, d_model, d_ff));
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", __func__);
+    const size_t widest = d_model > d_ff ? d_model : d_ff;
+    char *p = static_cast<char *>(workspace);
+    int8_t *q8 = reinterpret_cast<int8_t *>(p);
+    p += align256(tokens * widest);
+    float *scales = reinterpret_cast<float *>(p);
+    p += align256(tokens * sizeof(float));
+    float *qkv = reinterpret_cast<float *>(p);
+    p += align256(tokens * 3 * d_model * sizeof(float));
+    float *hidden = reinterpret_cast<float *>(p);
+    const int32_t round_bits = mode & HIPQ_ROUND_HALF_EVEN;
+
+    for (size_t l = 0; l < n_layers; ++l) {
+        const hipq_block_weights &b = blocks[l];
+        int32_t rc;
+        // attention half: x += W_out * quant(V(LN1(x)))
+        rc = hipq_layer_norm_quantize_f32_i8(ctx, x, tokens, d_model, b.ln1_gamma, b.ln1_beta, eps, round_bits, q8, scales);
+        if (rc) return rc;
+        rc = hipq_linear_i8_f32(ctx, q8, scales, 1, b.w_qkv, b.s_qkv, b.b_qkv, tokens, 3 * d_model, d_model, qkv);
+        if (rc) return rc;
+        // Stand-in for the attention mixing, which is outside this path: the value slice passes through.
+        rc = hipq_quantize_per_row_strided_f32_i8(ctx, qkv + 2 * d_model, tokens, d_model, 3 * d_model,
+                                                  HIPQ_PARAMS_SYMMETRIC, round_bits, q8, scales, nullptr, nullptr);
+        if (rc) return rc;
+        rc = hipq_linear_i8_f32_residual(ctx, q8, scales, 1, b.w_out, b.s_out, b.b_out, x, tokens, d_model, d_model, x);
+        if (rc) return rc;
+        // MLP half: x += W_fc2 * quant(GELU(W_fc1 * quant(LN2(x))))
+        rc = hipq_layer_norm_quantize_f32_i8(ctx, x, tokens, d_model, b.ln2_gamma, b.ln2_beta, eps, round_bits, q8, scales);
+        if (rc) return rc;
+        rc = hipq_linear_i8_f32(ctx, q8, scales, 1, b.w_fc1, b.s_fc1, b.b_fc1, tokens, d_ff, d_model, hidden);
+        if (rc) return rc;
+        rc = hipq_gelu_tanh_quantize_f32_i8(ctx, hidden, tokens, d_ff, round_bits, q8, scales);
+        if (rc) return rc;
+        rc = hipq_linear_i8_f32_residual(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, x, tokens, d_model, d_ff, x);
+        if (rc) return rc;
+    }
+    return HIPQ_SUCCESS;
+}
+
+}  // extern "C"

@@ -30,6 +30,13 @@ class HipqError(RuntimeError):
         self.message = message
 
 
+class BlockWeights(C.Structure):
+    """hipq_block_weights: device pointers of one block of the projection stack."""
+    _fields_ = [(n, C.c_void_p) for n in (
+        "ln1_gamma", "ln1_beta", "ln2_gamma", "ln2_beta", "w_qkv", "s_qkv", "b_qkv", "w_out", "s_out", "b_out",
+        "w_fc1", "s_fc1", "b_fc1", "w_fc2", "s_fc2", "b_fc2")]
+
+
 class QParams(C.Structure):
     _fields_ = [("scale", C.c_float), ("zero_point", C.c_int32), ("min_val", C.c_float), ("max_val", C.c_float),
                 ("status", C.c_int32), ("reserved", C.c_int32 * 3)]
@@ -71,6 +78,14 @@ _SIGNATURES = {
     "hipq_linear_i8_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _f32, _i32, _i32, _vp],
     "hipq_requantize_i32_i8": [_vp, _vp, _sz, _sz, _vp, _i32, _vp, _vp, _f32, _i32, _i32, _vp],
     "hipq_linear_dynamic_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
+    "hipq_quantize_per_row_strided_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
+    "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
+    "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
+    "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
+    "hipq_gelu_tanh_f32": [_vp, _vp, _sz, _vp],
+    "hipq_gelu_tanh_quantize_f32_i8": [_vp, _vp, _sz, _sz, _i32, _vp, _vp],
+    "hipq_add_f32": [_vp, _vp, _vp, _sz, _vp],
+    "hipq_transformer_stack_forward_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
     "hipq_conv2d_u8i8_i32": [_vp, _vp, _i32, _vp] + [_sz] * 11 + [_vp],
     "hipq_conv2d_u8i8_i8": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_f32, _i32, _i32, _vp],
     "hipq_conv2d_pack_weights_i8": [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp],
@@ -83,6 +98,7 @@ _SPECIAL = {
     "hipq_clear_last_error": (None, []),
     "hipq_has_error": (_i32, []),
     "hipq_ctx_stream": (_vp, [_vp]),
+    "hipq_transformer_stack_workspace_bytes": (_sz, [_sz, _sz, _sz]),
 }
 
 
@@ -368,3 +384,65 @@ class Context:
                   _ptr(w_scales), _ptr(bias), nb, c, h, wd, oc, kh, kw, padding[0], padding[1], float(s_out),
                   int(zp_out), mode, _ptr(out))
         return out
+
+    def quantize_per_row_strided(self, x_base, rows, cols, ld, elem_offset=0, flavor=PARAMS_SYMMETRIC, mode=0):
+        out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
+        scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
+        self.call("hipq_quantize_per_row_strided_f32_i8", x_base.data_ptr() + 4 * elem_offset, rows, cols, ld, flavor,
+                  mode, _ptr(out), _ptr(scales), None, None)
+        return out, scales
+
+    def linear_i8_f32_residual(self, a, a_scale, w, w_scales, bias, residual, out=None):
+        m, k = a.shape
+        n, _ = w.shape
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_i8_f32_residual", _ptr(a), _ptr(a_scale), int(a_scale.numel() > 1), _ptr(w),
+                  _ptr(w_scales), _ptr(bias), _ptr(residual), m, n, k, _ptr(out))
+        return out
+
+    def layer_norm(self, x, gamma=None, beta=None, eps=1e-5):
+        rows, cols = x.shape
+        out = torch.empty_like(x)
+        self.call("hipq_layer_norm_f32", _ptr(x), rows, cols, _ptr(gamma), _ptr(beta), float(eps), _ptr(out))
+        return out
+
+    def layer_norm_quantize(self, x, gamma=None, beta=None, eps=1e-5, mode=0):
+        rows, cols = x.shape
+        out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
+        scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
+        self.call("hipq_layer_norm_quantize_f32_i8", _ptr(x), rows, cols, _ptr(gamma), _ptr(beta), float(eps), mode,
+                  _ptr(out), _ptr(scales))
+        return out, scales
+
+    def gelu_tanh(self, x):
+        out = torch.empty_like(x)
+        self.call("hipq_gelu_tanh_f32", _ptr(x), x.numel(), _ptr(out))
+        return out
+
+    def gelu_tanh_quantize(self, x, mode=0):
+        rows, cols = x.shape
+        out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
+        scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
+        self.call("hipq_gelu_tanh_quantize_f32_i8", _ptr(x), rows, cols, mode, _ptr(out), _ptr(scales))
+        return out, scales
+
+    def add(self, a, b):
+        out = torch.empty_like(a)
+        self.call("hipq_add_f32", _ptr(a), _ptr(b), a.numel(), _ptr(out))
+        return out
+
+    def stack_workspace(self, tokens, d_model, d_ff):
+        nbytes = self._lib.hipq_transformer_stack_workspace_bytes(tokens, d_model, d_ff)
+        return torch.empty(nbytes, dtype=torch.uint8, device=self._dev())
+
+    def stack_forward(self, blocks, x, d_ff, workspace, eps=1e-5, mode=0):
+        """blocks: list of dicts of device tensors keyed like BlockWeights; x [tokens, d_model] is updated in place."""
+        arr = (BlockWeights * len(blocks))()
+        for rec, blk in zip(arr, blocks):
+            for name, _ in BlockWeights._fields_:
+                t = blk.get(name)
+                setattr(rec, name, None if t is None else t.data_ptr())
+        tokens, d_model = x.shape
+        self.call("hipq_transformer_stack_forward_f32", C.cast(arr, C.c_void_p), len(blocks), tokens, d_model, d_ff,
+                  float(eps), mode, _ptr(x), _ptr(workspace), workspace.numel())
+        return x
