@@ -280,3 +280,40 @@ def test_requantize(ctx, hipq, oracle, shape):
     want = oracle.requantize_epilogue(acc, sa, sw, None, 0.31, 0)
     got = host(ctx.requantize(dev(acc), dev(sa), dev(sw), None, 0.31, 0))
     np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("n", [4, 1024, 8192, 8196, 1 << 20, 4096 * 4096, 4096 * 4096 + 8192])
+@pytest.mark.parametrize("dtype_name", ["i8", "u8"])
+def test_dynamic_quantize_equals_explicit_steps(ctx, hipq, n, dtype_name):
+    """The dynamic entry point (range reduction, then quantize from the device-resident parameters) must agree
+    bit for bit with min/max, parameter and quantize calls made one by one."""
+    g = torch.Generator(device="cuda").manual_seed(n % 1000)
+    x = torch.randn(n, generator=g, device="cuda")
+    if dtype_name == "i8":
+        flavor, dtype, qmin, qmax, mode = hipq.PARAMS_SYMMETRIC, hipq.DTYPE_I8, -128, 127, hipq.FORM_MUL_INV
+    else:
+        flavor, dtype, qmin, qmax, mode = hipq.PARAMS_BACKEND_ASYMMETRIC, hipq.DTYPE_U8, 0, 255, hipq.FORM_DIV
+    q, params = ctx.quantize_dynamic_per_tensor(x, flavor, dtype, mode)
+    p = ctx.read_qparams(params)
+    mm = ctx.minmax(x)
+    params2 = ctx.qparams_from_minmax(mm, flavor, qmin, qmax)
+    q2 = torch.empty_like(q)
+    name = "hipq_quantize_with_params_f32_i8" if dtype_name == "i8" else "hipq_quantize_with_params_f32_u8"
+    ctx.call(name, x.data_ptr(), n, params2.data_ptr(), mode, q2.data_ptr())
+    p2 = ctx.read_qparams(params2)
+    ctx.synchronize()
+    assert (p.scale, p.zero_point, p.min_val, p.max_val, p.status) == (p2.scale, p2.zero_point, p2.min_val, p2.max_val, 0)
+    assert torch.equal(q, q2)
+
+
+def test_dynamic_quantize_back_to_back(ctx, hipq):
+    """Many calls in a row share the context's scratch (partials, parameters); stream order keeps them apart."""
+    g = torch.Generator(device="cuda").manual_seed(3)
+    xs = [torch.randn(512 * 4096, generator=g, device="cuda") * (i + 1) for i in range(6)]
+    outs = [ctx.quantize_dynamic_per_tensor(x) for x in xs * 5]
+    ctx.synchronize()
+    for i, (q, params) in enumerate(outs):
+        x = xs[i % len(xs)]
+        p = ctx.read_qparams(params)
+        assert p.status == 0 and p.scale == np.float32(x.abs().max().item()) / np.float32(127.0)
+        assert int(q.abs().max().item()) == 127

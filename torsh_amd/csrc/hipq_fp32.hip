@@ -150,11 +150,10 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restri
         for (int i = 0; i < kRowCache; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
             if (idx < nvec) {
-                const float a = quantize_value<true, EVEN>(v[i].x, scale, 0.0f, 0.0f, -128.0f, 127.0f);
-                const float b = quantize_value<true, EVEN>(v[i].y, scale, 0.0f, 0.0f, -128.0f, 127.0f);
-                const float c = quantize_value<true, EVEN>(v[i].z, scale, 0.0f, 0.0f, -128.0f, 127.0f);
-                const float d = quantize_value<true, EVEN>(v[i].w, scale, 0.0f, 0.0f, -128.0f, 127.0f);
-                q4[idx] = pack4(to_int_nan0(a), to_int_nan0(b), to_int_nan0(c), to_int_nan0(d));
+                q4[idx] = pack4(quantize_int<true, EVEN>(v[i].x, scale, 0.0f, 0.0f, -128, 127),
+                                quantize_int<true, EVEN>(v[i].y, scale, 0.0f, 0.0f, -128, 127),
+                                quantize_int<true, EVEN>(v[i].z, scale, 0.0f, 0.0f, -128, 127),
+                                quantize_int<true, EVEN>(v[i].w, scale, 0.0f, 0.0f, -128, 127));
             }
         }
     }

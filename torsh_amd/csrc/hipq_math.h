@@ -15,6 +15,23 @@ namespace hipq {
 
 constexpr int kWave = 64;
 
+// Streaming (non-temporal) 16-byte and 4-byte accesses for data touched once.  Measured on
+// MI355X over 16 Mi elements: quantize (64 MiB read, 16 MiB written) 19.8 us with ordinary
+// accesses, 17.6 us with both streams non-temporal; dequantize (16 MiB read, 64 MiB written)
+// 19.3 us ordinary, 13.4 us with ordinary loads and non-temporal stores (non-temporal loads
+// of the small side cost 4 us there, so dequantize keeps ordinary loads).
+typedef float hipq_vf4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load_stream(const float4 *p) {
+    const hipq_vf4 t = __builtin_nontemporal_load(reinterpret_cast<const hipq_vf4 *>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint32_t load_stream(const uint32_t *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void store_stream(float4 *p, float4 v) {
+    const hipq_vf4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<hipq_vf4 *>(p));
+}
+__device__ __forceinline__ void store_stream(uint32_t *p, uint32_t v) { __builtin_nontemporal_store(v, p); }
+
 // f32::round (half away from zero) or IEEE nearest-even.
 template <bool EVEN>
 __device__ __forceinline__ float round_mode(float v) {
@@ -54,9 +71,38 @@ __device__ __forceinline__ float quantize_value(float x, float scale, float inv,
     return clamp_keep_nan(q, lo, hi);
 }
 
+// Saturating f32 -> i32 with NaN -> 0: exactly Rust's `as i32`, and exactly what
+// v_cvt_i32_f32 does.  Inline asm so the conversion is never treated as undefined for
+// out-of-range inputs.
+__device__ __forceinline__ int cvt_i32_sat(float v) {
+    int r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+
+// Integer form of quantize_value for int8/uint8 outputs: the clamp is done after the
+// conversion, on integers (round(..)+zp is integral, so converting first changes nothing;
+// a NaN becomes 0 as `NaN.clamp(..) as i8` does, and +-Inf saturate).  About half the
+// vector instructions of the float-clamp form.
+template <bool DIV, bool EVEN>
+__device__ __forceinline__ int quantize_int(float x, float scale, float inv, float zpf, int lo, int hi) {
+    float t;
+    if constexpr (DIV)
+        t = x / scale;
+    else
+        t = x * inv;
+    const int q = cvt_i32_sat(round_mode<EVEN>(t) + zpf);
+    return min(max(q, lo), hi);
+}
+
+// clamp(round(v) ...) already formed as a float: convert and clamp on integers.
+__device__ __forceinline__ int clamp_to_int(float q, int lo, int hi) { return min(max(cvt_i32_sat(q), lo), hi); }
+
+// Low bytes of four ints -> one dword (three v_perm_b32 / v_or).
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
-    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
-           ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+    const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c), 0x04000c0cu);
+    return lo | hi;
 }
 
 __device__ __forceinline__ float wave_min(float v) {
