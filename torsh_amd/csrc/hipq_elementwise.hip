@@ -148,14 +148,44 @@ __device__ __forceinline__ OutT to_out(float q) {
         return static_cast<OutT>(cvt_i32_sat(q));  // q is already clamped; NaN -> 0
 }
 
-// Per-tensor quantize.  Scale and zero point come from the launch arguments or,
-// when `params` is non-null, from device memory (dynamic quantization).
+// What a dynamic quantize folds in front of its element loop: the range partials of
+// minmax_partial_kernel, the parameter formula, and where to publish the result.
+struct DynamicRange {
+    const float2 *partials;  // null: not a dynamic call
+    int nparts;
+    int flavor, qmin, qmax;
+    hipq_qparams *out_params;
+};
+
+// Per-tensor quantize.  Scale and zero point come from the launch arguments, from device
+// memory when `params` is non-null, or (dynamic quantization) from the range partials: then
+// every workgroup folds the same few hundred partials in the same order, derives the same
+// parameters, and workgroup 0 publishes them, which saves the launch of a finalize kernel.
 template <typename OutT, bool DIV, bool EVEN>
 __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restrict__ x, size_t n, float scale,
                                                            int zp, const hipq_qparams *__restrict__ params,
-                                                           float lo, float hi, OutT *__restrict__ out) {
-    if (params) {
-        if (params->status != HIPQ_SUCCESS) return;  // the reference errors before quantizing
+                                                           DynamicRange dyn, float lo, float hi,
+                                                           OutT *__restrict__ out) {
+    if (dyn.partials) {
+        __shared__ float lds[2 * kBlock / kWave];
+        MinMax m{INFINITY, -INFINITY};
+        for (int i = threadIdx.x; i < dyn.nparts; i += kBlock) {
+            const float2 p = dyn.partials[i];
+            m.mn = fminf(m.mn, p.x);
+            m.mx = fmaxf(m.mx, p.y);
+        }
+        const MinMax r = block_minmax(m, lds);
+        const int st = params_from_minmax(r.mn, r.mx, dyn.flavor, dyn.qmin, dyn.qmax, &scale, &zp);
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            dyn.out_params->scale = scale;
+            dyn.out_params->zero_point = zp;
+            dyn.out_params->min_val = r.mn;
+            dyn.out_params->max_val = r.mx;
+            dyn.out_params->status = st;
+        }
+        if (st != HIPQ_SUCCESS) return;  // the reference errors before quantizing
+    } else if (params) {
+        if (params->status != HIPQ_SUCCESS) return;
         scale = params->scale;
         zp = params->zero_point;
     }
@@ -467,14 +497,28 @@ static int32_t launch_minmax(hipq_ctx *ctx, const float *x, size_t n, float *out
     return check_launch("minmax");
 }
 
+// First stage only; the quantize kernel that follows folds the partials itself.
+static int32_t launch_minmax_partials(hipq_ctx *ctx, const float *x, size_t n, DynamicRange *dyn) {
+    const int grid = grid_for_minmax(ctx, n);
+    void *s = nullptr;
+    int32_t rc = scratch(ctx, kScratchHeader + size_t(grid) * sizeof(float2), &s);
+    if (rc != HIPQ_SUCCESS) return rc;
+    float2 *partials = reinterpret_cast<float2 *>(static_cast<char *>(s) + kScratchHeader);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, partials);
+    dyn->partials = partials;
+    dyn->nparts = grid;
+    return check_launch("minmax");
+}
+
 template <typename OutT>
 static int32_t launch_quantize(hipq_ctx *ctx, const float *x, size_t n, float scale, int zp,
-                               const hipq_qparams *params, int mode, float lo, float hi, OutT *out) {
+                               const hipq_qparams *params, int mode, float lo, float hi, OutT *out,
+                               DynamicRange dyn = DynamicRange{nullptr, 0, 0, 0, 0, nullptr}) {
     const int grid = grid_for_tiles(ctx, n);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
 #define HIPQ_LAUNCH_Q(D, E)                                                                                   \
     hipLaunchKernelGGL((quantize_kernel<OutT, D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, scale, zp, \
-                       params, lo, hi, out)
+                       params, dyn, lo, hi, out)
     if (div && even)
         HIPQ_LAUNCH_Q(true, true);
     else if (div)
@@ -630,12 +674,14 @@ int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size
     if (dtype != HIPQ_DTYPE_I8 && dtype != HIPQ_DTYPE_U8)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", __func__, dtype);
     const int qmin = dtype == HIPQ_DTYPE_I8 ? -128 : 0, qmax = dtype == HIPQ_DTYPE_I8 ? 127 : 255;
-    rc = launch_minmax(ctx, x, n, nullptr, nullptr, out_params, flavor, qmin, qmax);
+    DynamicRange dyn{nullptr, 0, flavor, qmin, qmax, out_params};
+    rc = launch_minmax_partials(ctx, x, n, &dyn);
     if (rc) return rc;
     if (dtype == HIPQ_DTYPE_I8)
-        return launch_quantize<int8_t>(ctx, x, n, 1.0f, 0, out_params, mode, -128.0f, 127.0f,
-                                       static_cast<int8_t *>(out));
-    return launch_quantize<uint8_t>(ctx, x, n, 1.0f, 0, out_params, mode, 0.0f, 255.0f, static_cast<uint8_t *>(out));
+        return launch_quantize<int8_t>(ctx, x, n, 1.0f, 0, nullptr, mode, -128.0f, 127.0f,
+                                       static_cast<int8_t *>(out), dyn);
+    return launch_quantize<uint8_t>(ctx, x, n, 1.0f, 0, nullptr, mode, 0.0f, 255.0f, static_cast<uint8_t *>(out),
+                                    dyn);
 }
 
 int32_t hipq_dequantize_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t n, float scale, int32_t zero_point, float *out) {

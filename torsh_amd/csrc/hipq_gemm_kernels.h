@@ -629,16 +629,16 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
                 if (nn[j] >= N) continue;
                 const size_t off = size_t(m) * N + nn[j];
                 if constexpr (EPI == EPI_I32) {
-                    static_cast<int32_t *>(ep.out)[off] = acc[i][j][r];
+                    __builtin_nontemporal_store(acc[i][j][r], static_cast<int32_t *>(ep.out) + off);
                 } else {
                     float v = static_cast<float>(acc[i][j][r]) * s_comb[r][j];
                     if (has_bias) v = v + bv[j];
                     if constexpr (EPI == EPI_F32) {
                         if (ep.residual) v = v + res[r][j];
-                        static_cast<float *>(ep.out)[off] = v;
+                        __builtin_nontemporal_store(v, static_cast<float *>(ep.out) + off);
                     } else {
-                        const float q = clamp_keep_nan(round_mode<EVEN>(v / ep.s_out) + zpf, -128.0f, 127.0f);
-                        static_cast<int8_t *>(ep.out)[off] = static_cast<int8_t>(to_int_nan0(q));
+                        const int q = clamp_to_int(round_mode<EVEN>(v / ep.s_out) + zpf, -128, 127);
+                        __builtin_nontemporal_store(static_cast<int8_t>(q), static_cast<int8_t *>(ep.out) + off);
                     }
                 }
             }
