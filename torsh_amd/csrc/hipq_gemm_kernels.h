@@ -304,8 +304,13 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     const int nk = K / BK;
 
 #ifdef HIPQ_GEMM_TRACE
-    long long tr[5] = {clock64(), 0, 0, 0, 0};
-#define HIPQ_TS(i) tr[i] = clock64()
+#ifdef HIPQ_GEMM_TRACE_WALL
+#define HIPQ_CLK() wall_clock64()
+#else
+#define HIPQ_CLK() clock64()
+#endif
+    long long tr[5] = {HIPQ_CLK(), 0, 0, 0, 0};
+#define HIPQ_TS(i) tr[i] = HIPQ_CLK()
 #define HIPQ_TS_FLUSH() if (ep.ts && lane == 0) { long long *o = ep.ts + (size_t(blockIdx.x) * 16 + wave) * 5; for (int q = 0; q < 5; ++q) o[q] = tr[q]; }
 #else
 #define HIPQ_TS(i)
