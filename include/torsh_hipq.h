@@ -242,6 +242,7 @@ HIPQ_API int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t 
                                          const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
                                          int32_t mode, float *out);
 
+
 /* ---- quantized Conv2d forward (NCHW, filters [OC,IC,KH,KW]) ------------ */
 /* Integer part of perform_quantized_convolution,
  * crates/torsh-backend/src/quantization/operations.rs:637-713:
@@ -259,6 +260,14 @@ HIPQ_API int32_t hipq_conv2d_u8i8_i8(hipq_ctx *ctx, const uint8_t *x, int32_t zp
                                      const float *w_scales, const float *bias, size_t nb, size_t c, size_t h, size_t wd,
                                      size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
                                      size_t pad_w, float out_scale, int32_t out_zero_point, int32_t mode, int8_t *out);
+/* Convolution with the dequantize-with-bias epilogue: out[n,oc,oh,ow] = acc * (s_in * w_scales[oc]) + bias[oc], fp32
+ * NCHW.  This is the fp32 result the reference forms before it derives output parameters from its range
+ * (crates/torsh-backend/src/quantization/ops.rs:479-580; integer accumulation as in
+ * crates/torsh-quantization/src/operations.rs:672-713 with zero-contribution padding). */
+HIPQ_API int32_t hipq_conv2d_u8i8_f32(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in, const int8_t *w,
+                                      const float *w_scales, const float *bias, size_t nb, size_t c, size_t h, size_t wd,
+                                      size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
+                                      size_t pad_w, float *out);
 /* One-time filter preparation for the stride-1 fast path: int8 [OC,IC,KH,KW]
  * -> [OC,KH*KW,IC] (same byte count) and the per-filter sums w_sums[oc]
  * (offline weight preparation; no reference counterpart, the reference keeps

@@ -1,0 +1,668 @@
+// Tests of the C++ host layer (torsh_amd/host/include/torsh_hipq/*.hpp).  The first group
+// restates the reference's own unit tests against the mirrored API
+// (crates/torsh-quantization/src/algorithms.rs:736-893, simd_ops.rs:475-582,
+//  crates/torsh-backend/src/quantization/params.rs tests); the second group compares the
+// device results with the CPU oracle on seeded random inputs, bit for bit.
+//
+// Output: one line per case, "ok <name>", "FAIL <name>: <why>" or "skip <name>"; exit status 1
+// if any case failed.  `--cpu-only` runs the cases that never reach the device.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <random>
+#include <sstream>
+
+#include "torsh_hipq/backend.hpp"
+#include "torsh_hipq/nn.hpp"
+#include "torsh_hipq/quantization.hpp"
+#include "torsh_quant_oracle.h"
+
+using namespace torsh;
+using namespace torsh::quantization;
+namespace bq = torsh::backend::quantization;
+
+namespace {
+
+struct Case {
+    const char *name;
+    bool needs_gpu;
+    std::function<void()> fn;
+};
+std::vector<Case> &cases() {
+    static std::vector<Case> c;
+    return c;
+}
+struct Reg {
+    Reg(const char *n, bool g, std::function<void()> f) { cases().push_back({n, g, std::move(f)}); }
+};
+struct Failure {
+    std::string why;
+};
+#define CPU_TEST(name) \
+    void name();       \
+    Reg reg_##name(#name, false, name); \
+    void name()
+#define GPU_TEST(name) \
+    void name();       \
+    Reg reg_##name(#name, true, name); \
+    void name()
+#define CHECK(cond)                                                                    \
+    do {                                                                               \
+        if (!(cond)) {                                                                 \
+            std::ostringstream o;                                                      \
+            o << __LINE__ << ": " #cond;                                               \
+            throw Failure{o.str()};                                                    \
+        }                                                                              \
+    } while (0)
+#define CHECK_EQ(a, b)                                                                 \
+    do {                                                                               \
+        if (!((a) == (b))) {                                                           \
+            std::ostringstream o;                                                      \
+            o << __LINE__ << ": " #a " == " #b " (" << (a) << " vs " << (b) << ")";    \
+            throw Failure{o.str()};                                                    \
+        }                                                                              \
+    } while (0)
+
+std::vector<float> normal(size_t n, unsigned seed, float sigma = 1.0f, bool relu = false) {
+    std::mt19937 g(seed);
+    std::normal_distribution<float> d(0.0f, sigma);
+    std::vector<float> v(n);
+    for (auto &x : v) {
+        x = d(g);
+        if (relu && x < 0) x = 0;
+    }
+    return v;
+}
+template <typename A, typename B>
+void check_same(const std::vector<A> &a, const std::vector<B> &b, int line) {
+    if (a.size() != b.size()) throw Failure{std::to_string(line) + ": size mismatch"};
+    for (size_t i = 0; i < a.size(); ++i)
+        if (!(static_cast<double>(a[i]) == static_cast<double>(b[i]))) {
+            std::ostringstream o;
+            o << line << ": element " << i << ": " << static_cast<double>(a[i]) << " vs " << static_cast<double>(b[i]);
+            throw Failure{o.str()};
+        }
+}
+#define CHECK_SAME(a, b) check_same(a, b, __LINE__)
+
+// ---------------------------------------------------------------- host logic (no device)
+
+CPU_TEST(test_calculate_affine_quantization_params) {  // algorithms.rs:742-760
+    auto [scale, zp] = calculate_affine_quantization_params(-1.0f, 1.0f, DType::I8).unwrap();
+    CHECK(scale > 0.0f);
+    CHECK(zp >= -128 && zp <= 127);
+    float s_ref;
+    int32_t z_ref;
+    CHECK_EQ(tq_calculate_affine_params(-1.0f, 1.0f, TQ_DTYPE_I8, &s_ref, &z_ref), 0);
+    CHECK_EQ(scale, s_ref);
+    CHECK_EQ(zp, z_ref);
+    auto [s2, z2] = calculate_affine_quantization_params(1.0f, 1.0f, DType::I8).unwrap();
+    CHECK_EQ(s2, 1.0f);
+    CHECK_EQ(z2, -128);
+    CHECK(calculate_affine_quantization_params(2.0f, 1.0f, DType::I8).is_err());
+    CHECK(calculate_affine_quantization_params(NAN, 1.0f, DType::I8).is_err());
+}
+
+CPU_TEST(test_calculate_symmetric_quantization_params) {  // algorithms.rs:763-776
+    auto [scale, zp] = calculate_symmetric_quantization_params(-2.0f, 1.0f, DType::I8).unwrap();
+    CHECK_EQ(scale, 2.0f / 127.0f);
+    CHECK_EQ(zp, 0);
+    auto [s0, z0] = calculate_symmetric_quantization_params(0.0f, 0.0f, DType::I8).unwrap();
+    CHECK_EQ(s0, 1.0f);
+    CHECK_EQ(z0, 0);
+    auto [su, zu] = calculate_symmetric_quantization_params(-2.0f, 1.0f, DType::U8).unwrap();
+    CHECK_EQ(su, 2.0f / 255.0f);  // qmax of the dtype, algorithms.rs:417-419
+    CHECK_EQ(zu, 0);
+    CHECK(calculate_symmetric_quantization_params(-INFINITY, 1.0f, DType::I8).is_err());
+}
+
+CPU_TEST(test_params_match_oracle_on_random_ranges) {
+    std::mt19937 g(5);
+    std::uniform_real_distribution<float> d(-50.0f, 50.0f);
+    for (int i = 0; i < 2000; ++i) {
+        float a = d(g), b = d(g);
+        if (a > b) std::swap(a, b);
+        for (int dt = 0; dt < 2; ++dt) {
+            const DType dtype = dt ? DType::U8 : DType::I8;
+            float s;
+            int32_t z;
+            CHECK_EQ(tq_calculate_affine_params(a, b, dt, &s, &z), 0);
+            auto p = calculate_affine_quantization_params(a, b, dtype).unwrap();
+            CHECK_EQ(p.first, s);
+            CHECK_EQ(p.second, z);
+            CHECK_EQ(tq_calculate_symmetric_params(a, b, dt, &s, &z), 0);
+            auto q = calculate_symmetric_quantization_params(a, b, dtype).unwrap();
+            CHECK_EQ(q.first, s);
+            CHECK_EQ(q.second, z);
+            bq::QuantizationParams bp;
+            bp.dtype = dt ? bq::QuantizedDType::UInt8 : bq::QuantizedDType::Int8;
+            bp.scheme = bq::QuantizationScheme::Asymmetric;
+            CHECK(bp.from_statistics(a, b).is_ok());
+            CHECK_EQ(tq_backend_params_asymmetric(a, b, dt ? 0 : -128, dt ? 255 : 127, &s, &z), 0);
+            CHECK_EQ(bp.scale[0], s);
+            CHECK_EQ(bp.zero_point[0], z);
+            bp.scheme = bq::QuantizationScheme::Symmetric;
+            CHECK(bp.from_statistics(a, b).is_ok());
+            CHECK_EQ(tq_backend_params_symmetric(a, b, dt ? 0 : -128, dt ? 255 : 127, &s, &z), 0);
+            CHECK_EQ(bp.scale[0], s);
+            CHECK_EQ(bp.zero_point[0], z);
+        }
+    }
+}
+
+CPU_TEST(test_get_dtype_range) {  // algorithms.rs:779-784
+    CHECK(get_dtype_range(DType::I8) == std::make_pair(-128, 127));
+    CHECK(get_dtype_range(DType::U8) == std::make_pair(0, 255));
+    CHECK(get_dtype_range(DType::I16) == std::make_pair(-32768, 32767));
+}
+
+CPU_TEST(test_quant_config) {  // config.rs:158-409
+    CHECK(QuantConfig::int8().validate().is_ok());
+    CHECK(QuantConfig::int8().scheme == QScheme::PerTensorAffine);
+    CHECK(QuantConfig::int8().get_qint_range() == std::make_pair(-128, 127));
+    CHECK(QuantConfig::uint8().get_qint_range() == std::make_pair(0, 255));
+    CHECK(QuantConfig::int8().with_reduce_range(ReduceRange::Reduce).get_qint_range() == std::make_pair(-63, 63));
+    QuantConfig c;
+    c.scheme = QScheme::PerChannelSymmetric;
+    CHECK(c.validate().is_err());  // no channel axis
+    CHECK(QuantConfig::int8().with_scheme(QScheme::PerChannelSymmetric).validate().is_ok());
+    CHECK(*QuantConfig::int8().with_scheme(QScheme::PerChannelSymmetric).ch_axis == 0);
+    c = QuantConfig::int8();
+    c.eps = 0.0f;
+    CHECK(c.validate().is_err());
+    c = QuantConfig::int8();
+    c.averaging_constant = 1.0f;
+    CHECK(c.validate().is_err());
+    c = QuantConfig::int8().with_scheme(QScheme::MixedPrecision);
+    CHECK(c.validate().is_err());  // needs a KL / entropy observer
+}
+
+CPU_TEST(test_error_cases_before_the_device) {  // algorithms.rs:876-893, simd_ops.rs:538-552
+    auto tensor = tensor_1d({1.0f, 2.0f}).unwrap();
+    auto r = quantize_per_tensor_affine(tensor, -1.0f, 0);
+    CHECK(r.is_err());
+    CHECK(r.unwrap_err().kind == TorshError::InvalidArgument);
+    CHECK_EQ(r.unwrap_err().message, std::string("Scale must be positive"));
+    CHECK(dequantize_per_tensor_affine(tensor, 0.0f, 0).is_err());
+    CHECK(quantize_per_tensor_affine_i8(tensor, 0.0f, 0).is_err());
+    auto empty = tensor_1d({}).unwrap();
+    auto e = quantize_tensor_auto(empty, DType::I8, QScheme::PerTensorAffine);
+    CHECK(e.is_err());
+    CHECK_EQ(e.unwrap_err().message, std::string("Cannot quantize empty tensor"));
+    std::vector<float> in{1.0f, 2.0f}, out(1);
+    CHECK(quantize_per_tensor_affine_simd(in, 0.1f, 0, out).is_err());  // length mismatch
+    out.resize(2);
+    CHECK(quantize_per_tensor_affine_simd(in, -0.1f, 0, out).is_err());
+    CHECK(dequantize_per_tensor_affine_simd(in, 0.0f, 0, out).is_err());
+    CHECK(find_min_max_simd({}).is_err());
+    auto t3 = Tensor::from_data(std::vector<float>(24, 1.0f), {2, 3, 4}).unwrap();
+    auto ax = quantize_per_channel_auto(t3, 3, DType::I8, QScheme::PerChannelSymmetric);
+    CHECK(ax.is_err());
+    CHECK_EQ(ax.unwrap_err().message, std::string("Axis out of bounds"));
+    CHECK(quantize_per_channel_auto(t3, 0, DType::I8, QScheme::PerTensorAffine).is_err());
+    CHECK(Tensor::from_data({1.0f, 2.0f}, {3}).is_err());
+    QuantConfig bad;
+    bad.scheme = QScheme::PerChannelAffine;
+    CHECK(quantize_with_config(tensor, bad).is_err());
+}
+
+CPU_TEST(test_backend_params_and_tensor) {  // params.rs / tensor.rs tests
+    auto p = bq::QuantizationParams{};
+    CHECK(p.dtype == bq::QuantizedDType::UInt8 && p.scale[0] == 1.0f && p.zero_point[0] == 0);
+    CHECK(bq::QuantizationParams::int8_symmetric().validate().is_ok());
+    CHECK(bq::QuantizationParams::uint8_asymmetric().zero_point[0] == 128);
+    auto bad = bq::QuantizationParams::int8_symmetric();
+    bad.zero_point[0] = 3;
+    CHECK(bad.validate().is_err());
+    bad = bq::QuantizationParams::int8_symmetric();
+    bad.scale[0] = 0.0f;
+    CHECK(bad.validate().is_err());
+    bad = bq::QuantizationParams::uint8_asymmetric();
+    bad.zero_point[0] = 300;
+    CHECK(bad.validate().is_err());
+    CHECK(bq::QuantizationParams::channel_wise(1, bq::QuantizedDType::Int8).validate().is_err());
+    CHECK(bq::QuantizationParams::channel_wise(4, bq::QuantizedDType::Int8).validate().is_ok());
+    auto u = bq::QuantizationParams::uint8_asymmetric();
+    CHECK(u.from_statistics(2.0f, 1.0f).is_err());
+    CHECK(u.from_statistics(0.0f, INFINITY).is_err());
+    CHECK(u.from_statistics(-1.0f, 1.0f).is_ok());
+    CHECK_EQ(u.scale[0], 2.0f / 255.0f);
+    CHECK(u.zero_point[0] == 127 || u.zero_point[0] == 128);
+    CHECK(u.from_statistics(3.0f, 3.0f).is_ok());
+    CHECK(u.scale[0] == 1.0f && u.zero_point[0] == 0);
+    auto s = bq::QuantizationParams::int8_symmetric();
+    CHECK(s.from_statistics(-2.0f, 1.0f).is_ok());
+    CHECK_EQ(s.scale[0], 4.0f / 255.0f);  // 2*max_range/(qmax-qmin), params.rs:331-337
+    CHECK(bq::QuantizedTensor::from_data(std::vector<uint8_t>(5), {2, 3}, bq::QuantizationParams{}).is_err());
+    CHECK(bq::QuantizedTensor::from_data(std::vector<uint8_t>(6), {2, 3}, bq::QuantizationParams{}).is_ok());
+    bq::HipQuantizationOps ops;
+    auto a = bq::QuantizedTensor::from_data(std::vector<uint8_t>(6), {2, 3}, bq::QuantizationParams::int8_symmetric()).unwrap();
+    auto b = bq::QuantizedTensor::from_data(std::vector<uint8_t>(8), {4, 2}, bq::QuantizationParams::int8_symmetric()).unwrap();
+    CHECK(ops.qmatmul(a, b).is_err());            // K mismatch
+    CHECK(ops.vnni_qmatmul_int8(a, b).is_err());
+    CHECK(ops.vnni_qmatmul_int8(a, b).unwrap_err().kind == TorshError::BackendError);
+    auto v = bq::QuantizedTensor::from_data(std::vector<uint8_t>(6), {6}, bq::QuantizationParams::int8_symmetric()).unwrap();
+    CHECK(ops.qmatmul(v, b).is_err());            // not 2D
+    CHECK(ops.qconv2d(a, b, nullptr, {1, 1}, {0, 0}).is_err());
+    CHECK(ops.calibrate({}, bq::QuantizedDType::UInt8).is_err());
+    CHECK(ops.quantize_f32({}, bq::QuantizationParams::int8_symmetric()).unwrap().empty());
+    CHECK(ops.quantize_f32({1.0f}, bad).is_err());
+    CHECK(ops.qadd(a, a).unwrap_err().kind == TorshError::NotImplemented);
+}
+
+CPU_TEST(test_module_shapes_before_the_device) {
+    nn::Linear lin(4, 3, true);
+    CHECK(lin.parameters().count("weight") == 1 && lin.parameters().count("bias") == 1);
+    CHECK(lin.parameters().at("weight").shape().dims() == (std::vector<size_t>{4, 3}));
+    CHECK(lin.set_weight(Tensor::from_data(std::vector<float>(12, 0.f), {3, 4}).unwrap()).is_err());
+    CHECK(lin.training());
+    lin.eval();
+    CHECK(!lin.training());
+    auto w1 = tensor_1d({1.0f, 2.0f}).unwrap();
+    CHECK(nn::QuantizedLinear::from_weight_nk(w1, nullptr).is_err());
+    CHECK(nn::QuantizedConv2d::from_weight(w1, nullptr, {1, 1}, {0, 0}, 0.1f, 0).is_err());
+    auto w4 = Tensor::from_data(std::vector<float>(2 * 3 * 1 * 1, 0.5f), {2, 3, 1, 1}).unwrap();
+    CHECK(nn::QuantizedConv2d::from_weight(w4, nullptr, {1, 1}, {0, 0}, 0.0f, 0).is_err());
+    CHECK(nn::QuantizedConv2d::from_weight(w4, nullptr, {0, 1}, {0, 0}, 0.1f, 0).is_err());
+}
+
+// ---------------------------------------------------------------- the reference's tests, on the device
+
+GPU_TEST(test_quantize_per_tensor_affine) {  // algorithms.rs:787-800
+    auto tensor = tensor_1d({1.0f, 2.0f, 3.0f, 4.0f}).unwrap();
+    auto [quantized, scale, zero_point] = quantize_per_tensor_affine(tensor, 0.1f, 0).unwrap();
+    auto q = quantized.data().unwrap();
+    CHECK_EQ(q[0], 10.0f);
+    CHECK_EQ(q[1], 20.0f);
+    CHECK_EQ(q[2], 30.0f);
+    CHECK_EQ(q[3], 40.0f);
+    CHECK_EQ(scale, 0.1f);
+    CHECK_EQ(zero_point, 0);
+    auto [q8, s8, z8] = quantize_per_tensor_affine_i8(tensor, 0.1f, 0).unwrap();  // simd_ops.rs:525-535 values
+    CHECK_SAME(q8.as_slice(), (std::vector<int>{10, 20, 30, 40}));
+    CHECK_EQ(s8, 0.1f);
+    CHECK_EQ(z8, 0);
+}
+
+GPU_TEST(test_dequantize_per_tensor_affine) {  // algorithms.rs:803-813
+    auto qt = tensor_1d({10.0f, 20.0f, 30.0f, 40.0f}).unwrap();
+    auto d = dequantize_per_tensor_affine(qt, 0.1f, 0).unwrap().data().unwrap();
+    for (int i = 0; i < 4; ++i) CHECK(std::fabs(d[i] - float(i + 1)) < 1e-6f);
+}
+
+GPU_TEST(test_quantize_tensor_auto) {  // algorithms.rs:816-829
+    auto tensor = tensor_1d({-1.0f, 0.0f, 1.0f, 2.0f}).unwrap();
+    auto [quantized, scale, zp] = quantize_tensor_auto(tensor, DType::I8, QScheme::PerTensorAffine).unwrap();
+    CHECK(scale > 0.0f);
+    CHECK(zp >= -128 && zp <= 127);
+    CHECK_EQ(quantized.data().unwrap().size(), size_t(4));
+}
+
+GPU_TEST(test_quantize_with_config) {  // algorithms.rs:832-845
+    auto tensor = tensor_1d({1.0f, 2.0f, 3.0f, 4.0f}).unwrap();
+    auto result = quantize_with_config(tensor, QuantConfig::int8());
+    CHECK(result.is_ok());
+    auto [quantized, scale, zp] = result.unwrap();
+    CHECK(scale > 0.0f);
+    CHECK(zp >= -128 && zp <= 127);
+    CHECK(quantized.shape().dims() == tensor.shape().dims());
+}
+
+GPU_TEST(test_dequantize) {  // algorithms.rs:847-859
+    auto qt = tensor_1d({64.0f, 128.0f, -64.0f, 0.0f}).unwrap();
+    auto d = dequantize(qt, 0.5f, 0).unwrap().data().unwrap();
+    CHECK(std::fabs(d[0] - 32.0f) < 1e-6f);
+    CHECK(std::fabs(d[1] - 64.0f) < 1e-6f);
+    CHECK(std::fabs(d[2] + 32.0f) < 1e-6f);
+    CHECK(std::fabs(d[3] - 0.0f) < 1e-6f);
+}
+
+GPU_TEST(test_quantize_auto) {  // algorithms.rs:862-873
+    auto tensor = tensor_1d({0.5f, 1.0f, 1.5f, 2.0f}).unwrap();
+    auto result = quantize_auto(tensor, QuantConfig::int8());
+    CHECK(result.is_ok());
+    CHECK(std::get<1>(result.unwrap()) > 0.0f);
+}
+
+GPU_TEST(test_simd_slice_functions) {  // simd_ops.rs:479-511, 570-582
+    std::vector<float> in{1.0f, 2.0f, 3.0f, 4.0f}, out(4);
+    CHECK(quantize_per_tensor_affine_simd(in, 0.1f, 0, out).is_ok());
+    CHECK_SAME(out, (std::vector<float>{10, 20, 30, 40}));
+    std::vector<float> deq(4);
+    CHECK(dequantize_per_tensor_affine_simd(out, 0.1f, 0, deq).is_ok());
+    for (int i = 0; i < 4; ++i) CHECK(std::fabs(deq[i] - in[i]) < 1e-6f);
+    auto mm = find_min_max_simd({-1.5f, 0.0f, 2.3f, -0.8f, 4.7f, 1.2f}).unwrap();
+    CHECK_EQ(mm.first, -1.5f);
+    CHECK_EQ(mm.second, 4.7f);
+    std::vector<float> mob{1.0f, 2.0f, 3.0f, 4.0f, -1.0f, -2.0f};
+    std::vector<int8_t> q8(6);
+    CHECK(quantize_to_int8_simd(mob, 0.1f, 0, q8).is_ok());
+    CHECK_SAME(q8, (std::vector<int>{10, 20, 30, 40, -10, -20}));
+}
+
+// ---------------------------------------------------------------- parity with the oracle
+
+GPU_TEST(parity_quantize_tensor_auto_and_round_trip) {
+    for (size_t n : {size_t(7), size_t(64), size_t(65), size_t(5000), size_t(1 << 18)}) {
+        auto x = normal(n, 11 + unsigned(n));
+        auto t = tensor_1d(x).unwrap();
+        for (int dt = 0; dt < 2; ++dt)
+            for (int sch = 0; sch < 2; ++sch) {
+                std::vector<float> want(n);
+                float s;
+                int32_t z;
+                CHECK_EQ(tq_quantize_tensor_auto(x.data(), n, dt, sch ? TQ_PER_TENSOR_SYMMETRIC : TQ_PER_TENSOR_AFFINE,
+                                                 want.data(), &s, &z), 0);
+                auto [q, scale, zp] = quantize_tensor_auto(t, dt ? DType::U8 : DType::I8,
+                                                           sch ? QScheme::PerTensorSymmetric : QScheme::PerTensorAffine)
+                                          .unwrap();
+                CHECK_EQ(scale, s);
+                CHECK_EQ(zp, z);
+                CHECK_SAME(q.as_slice(), want);
+                std::vector<float> back(n);
+                CHECK_EQ(tq_dequantize_per_tensor_affine(want.data(), n, s, z, back.data()), 0);
+                CHECK_SAME(dequantize(q, scale, zp).unwrap().as_slice(), back);
+            }
+    }
+}
+
+GPU_TEST(parity_quantize_per_channel_auto) {
+    const std::vector<size_t> shape{6, 5, 7};
+    auto x = normal(6 * 5 * 7, 3);
+    auto t = Tensor::from_data(x, shape).unwrap();
+    for (size_t axis = 0; axis < 3; ++axis)
+        for (int sch = 0; sch < 2; ++sch) {
+            std::vector<float> want(x.size()), ws(shape[axis]);
+            std::vector<int32_t> wz(shape[axis]);
+            CHECK_EQ(tq_quantize_per_channel_auto(x.data(), shape.data(), 3, axis, TQ_DTYPE_I8,
+                                                  sch ? TQ_PER_CHANNEL_SYMMETRIC : TQ_PER_CHANNEL_AFFINE, want.data(),
+                                                  ws.data(), wz.data()), 0);
+            auto [q, s, z] = quantize_per_channel_auto(t, axis, DType::I8,
+                                                       sch ? QScheme::PerChannelSymmetric : QScheme::PerChannelAffine)
+                                 .unwrap();
+            CHECK_SAME(s, ws);
+            CHECK_SAME(z, wz);
+            CHECK_SAME(q.as_slice(), want);
+        }
+    auto cfg = QuantConfig::int8().with_scheme(QScheme::PerChannelSymmetric);
+    auto [q, s0, z0] = quantize_with_config(t, cfg).unwrap();
+    float mn, mx, s_ref;
+    int32_t z_ref;
+    tq_find_min_max(x.data(), 35, &mn, &mx);  // channel 0 of axis 0 is the first 35 values
+    tq_calculate_symmetric_params(mn, mx, TQ_DTYPE_I8, &s_ref, &z_ref);
+    CHECK_EQ(s0, s_ref);
+    CHECK_EQ(z0, 0);
+}
+
+GPU_TEST(parity_backend_quantize_dequantize) {
+    bq::HipQuantizationOps ops;
+    const size_t n = 4096 + 12;
+    auto x = normal(n, 21, 3.0f);
+    for (int dt = 0; dt < 2; ++dt) {
+        bq::QuantizationParams p = dt ? bq::QuantizationParams::uint8_asymmetric() : bq::QuantizationParams::int8_symmetric();
+        if (dt) p.from_statistics(-7.5f, 9.0f).unwrap();
+        else p.from_statistics(-9.0f, 9.0f).unwrap();
+        std::vector<uint8_t> want(n);
+        CHECK_EQ(tq_backend_quantize_f32(x.data(), n, p.scale.data(), p.zero_point.data(), 1, dt ? 0 : -128,
+                                         dt ? 255 : 127, want.data()), 0);
+        auto got = ops.quantize_f32(x, p).unwrap();
+        CHECK_SAME(got, want);
+        std::vector<float> back(n);
+        CHECK_EQ(tq_backend_dequantize_f32(want.data(), n, p.scale.data(), p.zero_point.data(), 1, dt ? 0 : 1,
+                                           back.data()), 0);
+        CHECK_SAME(ops.dequantize_f32(got, p).unwrap(), back);
+    }
+    // channel-wise: contiguous equal chunks
+    const size_t ch = 8, m = 8 * 515;
+    auto y = normal(m, 22);
+    for (int dt = 0; dt < 2; ++dt) {
+        auto p = bq::QuantizationParams::channel_wise(ch, dt ? bq::QuantizedDType::UInt8 : bq::QuantizedDType::Int8);
+        for (size_t c = 0; c < ch; ++c) {
+            p.scale[c] = 0.01f * float(c + 1);
+            p.zero_point[c] = dt ? int32_t(100 + c) : int32_t(c) - 4;
+        }
+        std::vector<uint8_t> want(m);
+        CHECK_EQ(tq_backend_quantize_f32(y.data(), m, p.scale.data(), p.zero_point.data(), ch, dt ? 0 : -128,
+                                         dt ? 255 : 127, want.data()), 0);
+        auto got = ops.quantize_f32(y, p).unwrap();
+        CHECK_SAME(got, want);
+        std::vector<float> back(m);
+        CHECK_EQ(tq_backend_dequantize_f32(want.data(), m, p.scale.data(), p.zero_point.data(), ch, dt ? 0 : 1,
+                                           back.data()), 0);
+        CHECK_SAME(ops.dequantize_f32(got, p).unwrap(), back);
+    }
+    auto cal = ops.calibrate({normal(1000, 1), normal(3000, 2, 2.0f)}, bq::QuantizedDType::UInt8).unwrap();
+    float mn = INFINITY, mx = -INFINITY;
+    for (auto &s : {normal(1000, 1), normal(3000, 2, 2.0f)})
+        for (float v : s) mn = std::fmin(mn, v), mx = std::fmax(mx, v);
+    float s_ref;
+    int32_t z_ref;
+    tq_backend_params_asymmetric(mn, mx, 0, 255, &s_ref, &z_ref);
+    CHECK_EQ(cal.scale[0], s_ref);
+    CHECK_EQ(cal.zero_point[0], z_ref);
+}
+
+GPU_TEST(parity_backend_matmul) {
+    bq::HipQuantizationOps ops;
+    for (auto [m, k, n] : {std::make_tuple(size_t(5), size_t(7), size_t(3)), std::make_tuple(size_t(33), size_t(256), size_t(70)),
+                           std::make_tuple(size_t(128), size_t(512), size_t(64))}) {
+        std::mt19937 g(unsigned(m * 31 + k));
+        std::uniform_int_distribution<int> d(-128, 127);
+        std::vector<uint8_t> a(m * k), b(k * n);
+        for (auto &v : a) v = uint8_t(int8_t(d(g)));
+        for (auto &v : b) v = uint8_t(int8_t(d(g)));
+        auto pa = bq::QuantizationParams::int8_symmetric(), pb = bq::QuantizationParams::int8_symmetric();
+        pa.scale[0] = 0.031f;
+        pb.scale[0] = 0.0007f;
+        auto ta = bq::QuantizedTensor::from_data(a, {m, k}, pa).unwrap();
+        auto tb = bq::QuantizedTensor::from_data(b, {k, n}, pb).unwrap();
+        std::vector<int32_t> acc(m * n);
+        std::vector<uint8_t> clamped(m * n);
+        CHECK_EQ(tq_backend_matmul_i32(a.data(), b.data(), m, k, n, acc.data(), clamped.data()), 0);
+        CHECK_SAME(ops.qmatmul_i32(ta, tb).unwrap(), acc);
+        auto v = ops.vnni_qmatmul_int8(ta, tb).unwrap();
+        CHECK_SAME(v.data, clamped);
+        CHECK(v.shape == (std::vector<size_t>{m, n}));
+        CHECK_EQ(v.params.scale[0], pa.scale[0]);
+        // qmatmul: acc * (s_a * s_b) -> range -> symmetric params of `a`'s kind -> requantize
+        std::vector<float> out_f(m * n);
+        const float sab = pa.scale[0] * pb.scale[0];
+        float mn = INFINITY, mx = -INFINITY;
+        for (size_t i = 0; i < m * n; ++i) {
+            out_f[i] = float(acc[i]) * sab;
+            mn = std::fmin(mn, out_f[i]);
+            mx = std::fmax(mx, out_f[i]);
+        }
+        float s_out;
+        int32_t z_out;
+        tq_backend_params_symmetric(mn, mx, -128, 127, &s_out, &z_out);
+        std::vector<uint8_t> want(m * n);
+        tq_backend_quantize_f32(out_f.data(), m * n, &s_out, &z_out, 1, -128, 127, want.data());
+        auto r = ops.qmatmul(ta, tb).unwrap();
+        CHECK_EQ(r.params.scale[0], s_out);
+        CHECK_EQ(r.params.zero_point[0], 0);
+        CHECK_SAME(r.data, want);
+        // and against the reference's own f32 loop (dequantize, accumulate in k order): the two
+        // differ only by f32 summation error, at most one output step
+        std::vector<float> af(m * k), bf(k * n);
+        tq_backend_dequantize_f32(a.data(), m * k, pa.scale.data(), pa.zero_point.data(), 1, 1, af.data());
+        tq_backend_dequantize_f32(b.data(), k * n, pb.scale.data(), pb.zero_point.data(), 1, 1, bf.data());
+        for (size_t i = 0; i < m; ++i)
+            for (size_t j = 0; j < n; ++j) {
+                float s = 0.0f;
+                for (size_t l = 0; l < k; ++l) s += af[i * k + l] * bf[l * n + j];
+                CHECK(std::fabs(s - out_f[i * n + j]) <= 1e-4f * std::fmax(1.0f, std::fabs(s)) + 0.51f * s_out);
+            }
+    }
+}
+
+GPU_TEST(parity_backend_qconv2d) {
+    bq::HipQuantizationOps ops;
+    struct G { size_t nb, c, h, w, oc, k, stride, pad; };
+    for (G g : {G{2, 3, 8, 8, 4, 3, 1, 1}, G{1, 128, 7, 7, 16, 3, 1, 1}, G{1, 16, 9, 9, 6, 3, 2, 1}}) {
+        auto xf = normal(g.nb * g.c * g.h * g.w, unsigned(g.c), 1.0f, true);
+        auto in_p = bq::QuantizationParams::uint8_asymmetric();
+        float mn, mx;
+        tq_find_min_max(xf.data(), xf.size(), &mn, &mx);
+        in_p.from_statistics(mn, mx).unwrap();
+        auto xq = ops.quantize_f32(xf, in_p).unwrap();
+        const size_t per = g.c * g.k * g.k;
+        auto wf = normal(g.oc * per, 77, 0.02f);
+        auto w_p = bq::QuantizationParams::channel_wise(g.oc, bq::QuantizedDType::Int8);
+        for (size_t o = 0; o < g.oc; ++o) {
+            float a = 0.0f;
+            for (size_t i = 0; i < per; ++i) a = std::fmax(a, std::fabs(wf[o * per + i]));
+            w_p.scale[o] = a / 127.0f;
+        }
+        auto wq = ops.quantize_f32(wf, w_p).unwrap();
+        auto bias_f = normal(g.oc, 5, 0.01f);
+        auto b_p = bq::QuantizationParams::int8_symmetric();
+        b_p.scale[0] = 0.0005f;
+        auto bq8 = ops.quantize_f32(bias_f, b_p).unwrap();
+        auto tin = bq::QuantizedTensor::from_data(xq, {g.nb, g.c, g.h, g.w}, in_p).unwrap();
+        auto tw = bq::QuantizedTensor::from_data(wq, {g.oc, g.c, g.k, g.k}, w_p).unwrap();
+        auto tb = bq::QuantizedTensor::from_data(bq8, {g.oc}, b_p).unwrap();
+        const size_t ho = (g.h + 2 * g.pad - g.k) / g.stride + 1, wo = (g.w + 2 * g.pad - g.k) / g.stride + 1;
+        std::vector<int32_t> acc(g.nb * g.oc * ho * wo);
+        CHECK_EQ(tq_backend_conv2d_i32(xq.data(), 0, in_p.zero_point[0], reinterpret_cast<const int8_t *>(wq.data()), g.nb,
+                                       g.c, g.h, g.w, g.oc, g.k, g.k, g.stride, g.stride, g.pad, g.pad, acc.data()), 0);
+        std::vector<float> bias_dq(g.oc);
+        tq_backend_dequantize_f32(bq8.data(), g.oc, b_p.scale.data(), b_p.zero_point.data(), 1, 1, bias_dq.data());
+        std::vector<float> out_f(acc.size());
+        mn = INFINITY, mx = -INFINITY;
+        for (size_t i = 0; i < acc.size(); ++i) {
+            const size_t oc = (i / (ho * wo)) % g.oc;
+            out_f[i] = float(acc[i]) * (in_p.scale[0] * w_p.scale[oc]) + bias_dq[oc];
+            mn = std::fmin(mn, out_f[i]);
+            mx = std::fmax(mx, out_f[i]);
+        }
+        float s_out;
+        int32_t z_out;
+        tq_backend_params_asymmetric(mn, mx, 0, 255, &s_out, &z_out);
+        std::vector<uint8_t> want(acc.size());
+        tq_backend_quantize_f32(out_f.data(), out_f.size(), &s_out, &z_out, 1, 0, 255, want.data());
+        auto r = ops.qconv2d(tin, tw, &tb, {g.stride, g.stride}, {g.pad, g.pad}).unwrap();
+        CHECK(r.shape == (std::vector<size_t>{g.nb, g.oc, ho, wo}));
+        CHECK_EQ(r.params.scale[0], s_out);
+        CHECK_EQ(r.params.zero_point[0], z_out);
+        CHECK_SAME(r.data, want);
+    }
+}
+
+GPU_TEST(parity_quantized_linear_module) {
+    for (int per_token = 0; per_token < 2; ++per_token) {
+        const size_t m = 48, k = 256, n = 96;
+        nn::Linear lin(k, n, true);
+        auto w_in_out = normal(k * n, 31, 0.02f);
+        auto bias = normal(n, 32, 0.01f);
+        lin.set_weight(Tensor::from_data(w_in_out, {k, n}).unwrap()).unwrap();
+        lin.set_bias(Tensor::from_data(bias, {n}).unwrap()).unwrap();
+        auto qlin = nn::QuantizedLinear::from_linear(lin, per_token ? nn::ActivationQuant::PerToken
+                                                                    : nn::ActivationQuant::PerTensor)
+                        .unwrap();
+        auto x = normal(m * k, 33);
+        auto y = qlin.forward(Tensor::from_data(x, {4, 12, k}).unwrap()).unwrap();
+        CHECK(y.shape().dims() == (std::vector<size_t>{4, 12, n}));
+        // oracle composition
+        std::vector<float> wnk(n * k);
+        for (size_t i = 0; i < k; ++i)
+            for (size_t j = 0; j < n; ++j) wnk[j * k + i] = w_in_out[i * n + j];
+        const size_t wshape[2] = {n, k};
+        std::vector<float> wq_f(n * k), sw(n);
+        std::vector<int32_t> wz(n);
+        tq_quantize_per_channel_auto(wnk.data(), wshape, 2, 0, TQ_DTYPE_I8, TQ_PER_CHANNEL_SYMMETRIC, wq_f.data(),
+                                     sw.data(), wz.data());
+        std::vector<int8_t> wq(n * k), aq(m * k);
+        for (size_t i = 0; i < n * k; ++i) wq[i] = int8_t(wq_f[i]);
+        std::vector<float> sa(per_token ? m : 1), aq_f(m * k);
+        if (per_token) {
+            const size_t ashape[2] = {m, k};
+            std::vector<int32_t> az(m);
+            tq_quantize_per_channel_auto(x.data(), ashape, 2, 0, TQ_DTYPE_I8, TQ_PER_CHANNEL_SYMMETRIC, aq_f.data(),
+                                         sa.data(), az.data());
+        } else {
+            int32_t z;
+            tq_quantize_tensor_auto(x.data(), m * k, TQ_DTYPE_I8, TQ_PER_TENSOR_SYMMETRIC, aq_f.data(), &sa[0], &z);
+        }
+        for (size_t i = 0; i < m * k; ++i) aq[i] = int8_t(aq_f[i]);
+        std::vector<int32_t> acc(m * n);
+        tq_gemm_i8_nk(aq.data(), wq.data(), m, n, k, acc.data());
+        std::vector<float> want(m * n);
+        tq_linear_dequant_epilogue(acc.data(), m, n, sa.data(), per_token, sw.data(), bias.data(), want.data());
+        CHECK_SAME(y.as_slice(), want);
+        auto params = qlin.parameters();
+        CHECK(params.count("weight") && params.count("bias") && params.count("weight_scale"));
+        CHECK_SAME(params.at("weight").as_slice(), wq_f);
+        CHECK_SAME(params.at("weight_scale").as_slice(), sw);
+        CHECK(qlin.forward(Tensor::from_data(std::vector<float>(10, 0.f), {2, 5}).unwrap()).is_err());
+    }
+}
+
+GPU_TEST(parity_quantized_conv2d_module) {
+    const size_t nb = 2, c = 128, h = 9, w = 9, oc = 24, k = 3, pad = 1;
+    auto wf = normal(oc * c * k * k, 41, 0.02f);
+    auto bias = normal(oc, 42, 0.01f);
+    auto x = normal(nb * c * h * w, 43, 1.0f, true);
+    const float s_out = 0.013f;
+    const int32_t zp_out = -3;
+    auto bt = Tensor::from_data(bias, {oc}).unwrap();
+    auto conv = nn::QuantizedConv2d::from_weight(Tensor::from_data(wf, {oc, c, k, k}).unwrap(), &bt, {1, 1}, {pad, pad},
+                                                 s_out, zp_out)
+                    .unwrap();
+    auto xt = Tensor::from_data(x, {nb, c, h, w}).unwrap();
+    auto q = conv.forward_quantized(xt).unwrap();
+    // oracle composition
+    float mn, mx, s_in;
+    int32_t zp_in;
+    tq_find_min_max(x.data(), x.size(), &mn, &mx);
+    tq_backend_params_asymmetric(mn, mx, 0, 255, &s_in, &zp_in);
+    std::vector<uint8_t> xq(x.size());
+    tq_backend_quantize_f32(x.data(), x.size(), &s_in, &zp_in, 1, 0, 255, xq.data());
+    const size_t wshape[2] = {oc, c * k * k};
+    std::vector<float> wq_f(wf.size()), sw(oc);
+    std::vector<int32_t> wz(oc);
+    tq_quantize_per_channel_auto(wf.data(), wshape, 2, 0, TQ_DTYPE_I8, TQ_PER_CHANNEL_SYMMETRIC, wq_f.data(), sw.data(),
+                                 wz.data());
+    std::vector<int8_t> wq(wf.size());
+    for (size_t i = 0; i < wf.size(); ++i) wq[i] = int8_t(wq_f[i]);
+    std::vector<int32_t> acc(nb * oc * h * w);
+    tq_backend_conv2d_i32(xq.data(), 0, zp_in, wq.data(), nb, c, h, w, oc, k, k, 1, 1, pad, pad, acc.data());
+    std::vector<int8_t> want(acc.size());
+    // rows of the [nb*oc, h*w] view cycle through the output channels
+    tq_requantize_epilogue(acc.data(), nb * oc, h * w, &s_in, 0, sw.data(), bias.data(), s_out, zp_out, -128, 127, 1, oc,
+                           want.data());
+    CHECK(q.shape().dims() == (std::vector<size_t>{nb, oc, h, w}));
+    CHECK_SAME(q.as_slice(), want);
+    auto y = conv.forward(xt).unwrap();
+    for (size_t i = 0; i < want.size(); ++i) CHECK_EQ(y.as_slice()[i], float(int(want[i]) - zp_out) * s_out);
+    CHECK(conv.forward(Tensor::from_data(std::vector<float>(6, 0.f), {2, 3}).unwrap()).is_err());
+    CHECK(conv.forward(Tensor::from_data(std::vector<float>(2 * 3 * 4 * 4, 0.f), {2, 3, 4, 4}).unwrap()).is_err());
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    const bool cpu_only = argc > 1 && std::strcmp(argv[1], "--cpu-only") == 0;
+    int failed = 0;
+    for (const Case &c : cases()) {
+        if (c.needs_gpu && cpu_only) {
+            std::printf("skip %s\n", c.name);
+            continue;
+        }
+        std::printf("run %s\n", c.name);
+        std::fflush(stdout);
+        try {
+            c.fn();
+            std::printf("ok %s\n", c.name);
+        } catch (const Failure &f) {
+            std::printf("FAIL %s: line %s\n", c.name, f.why.c_str());
+            ++failed;
+        } catch (const std::exception &e) {
+            std::printf("FAIL %s: %s\n", c.name, e.what());
+            ++failed;
+        }
+        std::fflush(stdout);
+    }
+    return failed ? 1 : 0;
+}

@@ -55,13 +55,13 @@ def _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, seed):
     acc2d = acc.reshape(nb * oc, ho * wo)
     out_f = (acc2d.astype(np.float32) * np.tile(np.float32(s_in) * sw, nb)[:, None]) + np.tile(bias, nb)[:, None]
     s_out, _ = oracle.calculate_symmetric_params(float(out_f.min()), float(out_f.max()), 0)
-    return x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out
+    return x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out, out_f
 
 
 @pytest.mark.parametrize("nb,c,h,w,oc,k,pad", [(2, 128, 14, 14, 64, 3, 1), (1, 256, 7, 7, 33, 3, 1), (3, 16, 10, 10, 8, 3, 1)])
 def test_quantized_conv2d_forward(ctx, hipq, oracle, nb, c, h, w, oc, k, pad):
     """BASELINE config 4 at reduced size: asymmetric u8 activations, per-channel int8 filters, fused bias + requant."""
-    x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out = _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, c + oc)
+    x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out, out_f = _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, c + oc)
     # activations quantized on the device: min/max -> asymmetric params -> u8
     dq, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_BACKEND_ASYMMETRIC, hipq.DTYPE_U8, hipq.FORM_DIV)
     p = ctx.read_qparams(params)
@@ -83,6 +83,9 @@ def test_quantized_conv2d_forward(ctx, hipq, oracle, nb, c, h, w, oc, k, pad):
             packed, sums = ctx.conv2d_pack_weights(dwq)
             got = host(ctx.conv2d_i8_packed(dq, zp_in, s_in, packed, sums, (k, k), dsw, dev(bias), s_out, -2, (pad, pad), mode))
             np.testing.assert_array_equal(got.reshape(acc2d.shape), want)
+    # dequantize-with-bias epilogue: the same f32 expression in the same order -> identical bits
+    got = host(ctx.conv2d_f32(dq, zp_in, s_in, dwq, dsw, dev(bias), (1, 1), (pad, pad)))
+    np.testing.assert_array_equal(got.reshape(acc2d.shape), out_f)
     want = oracle.requantize_epilogue(acc2d, s_in, sw, None, s_out, 0, channel_axis_is_row=True, inner=oc)
     got = host(ctx.conv2d_i8(dq, zp_in, s_in, dwq, dsw, None, s_out, 0, (1, 1), (pad, pad)))
     np.testing.assert_array_equal(got.reshape(acc2d.shape), want)

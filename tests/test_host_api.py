@@ -1,0 +1,99 @@
+"""Runs the C++ host-layer test program (tests/host/host_api_test.cpp): the reference's own unit tests restated
+against the mirrored C++ API, and parity of the device results with the CPU oracle.
+
+The program is built ahead of time (``make -C tests/host``, also done by ``__graft_entry__.build()``); it is built
+here only when no binary exists.  It runs once per session; each case is reported as its own pytest test."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "host", "bin", "host_api_test")
+
+CPU_CASES = [
+    "test_calculate_affine_quantization_params",
+    "test_calculate_symmetric_quantization_params",
+    "test_params_match_oracle_on_random_ranges",
+    "test_get_dtype_range",
+    "test_quant_config",
+    "test_error_cases_before_the_device",
+    "test_backend_params_and_tensor",
+    "test_module_shapes_before_the_device",
+]
+GPU_CASES = [
+    "test_quantize_per_tensor_affine",
+    "test_dequantize_per_tensor_affine",
+    "test_quantize_tensor_auto",
+    "test_quantize_with_config",
+    "test_dequantize",
+    "test_quantize_auto",
+    "test_simd_slice_functions",
+    "parity_quantize_tensor_auto_and_round_trip",
+    "parity_quantize_per_channel_auto",
+    "parity_backend_quantize_dequantize",
+    "parity_backend_matmul",
+    "parity_backend_qconv2d",
+    "parity_quantized_linear_module",
+    "parity_quantized_conv2d_module",
+]
+
+
+def _binary():
+    if not os.path.exists(BIN):
+        from oracle import pyoracle
+        from torsh_amd import hipq
+
+        hipq.load()
+        pyoracle.lib()
+        subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "host")], check=True, capture_output=True)
+    return BIN
+
+
+def _run(args):
+    proc = subprocess.run([_binary(), *args], capture_output=True, text=True, timeout=300)
+    results = {}
+    for line in proc.stdout.splitlines():
+        word, _, rest = line.partition(" ")
+        if word in ("ok", "skip"):
+            results[rest.strip()] = (word, "")
+        elif word == "FAIL":
+            name, _, why = rest.partition(":")
+            results[name.strip()] = ("FAIL", why.strip())
+        elif word == "run":
+            results.setdefault(rest.strip(), ("crashed", proc.stderr[-2000:]))
+    return results, proc
+
+
+@pytest.fixture(scope="module")
+def cpu_results():
+    return _run(["--cpu-only"])
+
+
+@pytest.fixture(scope="module")
+def gpu_results():
+    import torch
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return _run([])
+
+
+@pytest.mark.parametrize("case", CPU_CASES)
+def test_host_logic(cpu_results, case):
+    results, proc = cpu_results
+    assert case in results, f"case did not run; stderr: {proc.stderr[-1000:]}"
+    assert results[case][0] == "ok", results[case][1]
+
+
+def test_cpu_only_run_skips_every_device_case(cpu_results):
+    results, _ = cpu_results
+    assert all(results[c][0] == "skip" for c in GPU_CASES)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CPU_CASES + GPU_CASES)
+def test_host_api_on_device(gpu_results, case):
+    results, proc = gpu_results
+    assert case in results, f"case did not run; stderr: {proc.stderr[-1000:]}"
+    assert results[case][0] == "ok", results[case][1]

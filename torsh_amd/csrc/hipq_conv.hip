@@ -103,8 +103,13 @@ __global__ __launch_bounds__(kConvThreads) void conv_direct_kernel(const uint8_t
         } else {
             float v = static_cast<float>(acc) * (s_in * sw[oc]);
             if (bias) v = v + bias[oc];
-            const float q = clamp_keep_nan(round_mode<EVEN>(v / s_out) + static_cast<float>(zp_out), -128.0f, 127.0f);
-            static_cast<int8_t *>(out)[idx] = static_cast<int8_t>(to_int_nan0(q));
+            if constexpr (EPI == EPI_F32) {
+                static_cast<float *>(out)[idx] = v;
+            } else {
+                const float q =
+                    clamp_keep_nan(round_mode<EVEN>(v / s_out) + static_cast<float>(zp_out), -128.0f, 127.0f);
+                static_cast<int8_t *>(out)[idx] = static_cast<int8_t>(to_int_nan0(q));
+            }
         }
     }
 }
@@ -264,6 +269,25 @@ int32_t hipq_conv2d_u8i8_i8(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, floa
     if (nb != 0 && oc != 0) HIPQ_REQUIRE_PTR(w);
     return conv_i8_common(__func__, ctx, x, zp_in, s_in, w, nullptr, nullptr, w_scales, bias, g, out_scale,
                           out_zero_point, mode, out);
+}
+
+int32_t hipq_conv2d_u8i8_f32(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in, const int8_t *w,
+                             const float *w_scales, const float *bias, size_t nb, size_t c, size_t h, size_t wd,
+                             size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
+                             size_t pad_w, float *out) {
+    HIPQ_ENTER(ctx);
+    ConvGeom g;
+    int32_t rc = make_geom(__func__, nb, c, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w, &g);
+    if (rc) return rc;
+    if (s_in <= 0.0f) return fail(HIPQ_INVALID_ARGUMENT, "%s: Scale must be positive", __func__);
+    if (zp_in < 0 || zp_in > 255) return fail(HIPQ_INVALID_ARGUMENT, "%s: zero point %d outside [0,255]", __func__, zp_in);
+    if (nb == 0 || oc == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(w);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    return conv_forward<EPI_F32, false>(__func__, ctx, x, zp_in, s_in, w, nullptr, nullptr, w_scales, bias, g, 1.0f, 0,
+                                        out);
 }
 
 int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in, const int8_t *w_packed,

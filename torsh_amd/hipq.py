@@ -88,6 +88,7 @@ _SIGNATURES = {
     "hipq_transformer_stack_forward_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
     "hipq_conv2d_u8i8_i32": [_vp, _vp, _i32, _vp] + [_sz] * 11 + [_vp],
     "hipq_conv2d_u8i8_i8": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_f32, _i32, _i32, _vp],
+    "hipq_conv2d_u8i8_f32": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_vp],
     "hipq_conv2d_pack_weights_i8": [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp],
     "hipq_conv2d_u8i8_i8_packed": [_vp, _vp, _i32, _f32, _vp, _vp, _vp, _vp] + [_sz] * 9 + [_f32, _i32, _i32, _vp],
 }
@@ -363,6 +364,18 @@ class Context:
         self.call("hipq_conv2d_u8i8_i8", _ptr(x_u8), int(zp_in), float(s_in), _ptr(w_i8), _ptr(w_scales), _ptr(bias), nb,
                   c, h, wd, oc, kh, kw, stride[0], stride[1], padding[0], padding[1], float(s_out), int(zp_out), mode,
                   _ptr(out))
+        return out
+
+    def conv2d_f32(self, x_u8, zp_in, s_in, w_i8, w_scales, bias, stride=(1, 1), padding=(0, 0), out=None):
+        nb, c, h, wd = x_u8.shape
+        oc, c2, kh, kw = w_i8.shape
+        if c != c2:
+            raise HipqError(DIMENSION_MISMATCH, f"qconv2d channel mismatch: input C_in={c} but weight C_in={c2}")
+        ho = max((h + 2 * padding[0] - kh) // stride[0] + 1, 0)
+        wo = max((wd + 2 * padding[1] - kw) // stride[1] + 1, 0)
+        out = out if out is not None else torch.empty((nb, oc, ho, wo), dtype=torch.float32, device=self._dev())
+        self.call("hipq_conv2d_u8i8_f32", _ptr(x_u8), int(zp_in), float(s_in), _ptr(w_i8), _ptr(w_scales), _ptr(bias), nb,
+                  c, h, wd, oc, kh, kw, stride[0], stride[1], padding[0], padding[1], _ptr(out))
         return out
 
     def conv2d_pack_weights(self, w_i8):
