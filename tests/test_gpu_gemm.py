@@ -132,6 +132,35 @@ def test_quantized_linear_requant_epilogue(ctx, hipq, oracle, m, n, k):
         np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k", [(4096, 1024, 512), (4100, 1000, 256), (8192, 768, 768)])
+def test_many_tile_shapes_persistent_kernel(ctx, hipq, oracle, m, n, k):
+    """Shapes with at least two 128x64 tiles per compute unit run on the persistent kernel: accumulators, the
+    dequantize epilogue with per-token scales, the residual add and the requantize epilogue against the oracle."""
+    rng = np.random.default_rng(m + n + k)
+    a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+    acc = oracle.gemm_i8_nk(a, w)
+    np.testing.assert_array_equal(host(ctx.gemm_i8_i32(dev(a), dev(w))), acc)
+    sa = (rng.random(m) * 0.05 + 0.001).astype(np.float32)
+    sw = (rng.random(n) * 0.002 + 0.0001).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    want = oracle.linear_dequant_epilogue(acc, sa, sw, bias)
+    np.testing.assert_array_equal(host(ctx.linear_i8_f32(dev(a), dev(sa), dev(w), dev(sw), dev(bias))), want)
+    s1 = np.array([0.021], np.float32)
+    want1 = oracle.linear_dequant_epilogue(acc, s1, sw, None)
+    np.testing.assert_array_equal(host(ctx.linear_i8_f32(dev(a), dev(s1), dev(w), dev(sw), None)), want1)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    got = host(ctx.linear_i8_f32_residual(dev(a), dev(sa), dev(w), dev(sw), dev(bias), dev(res)))
+    np.testing.assert_array_equal(got, want + res)
+    s_out, _ = oracle.calculate_symmetric_params(*oracle.find_min_max(want), 0)
+    for mode, rm in ((hipq.ROUND_HALF_AWAY, 0), (hipq.ROUND_HALF_EVEN, 1)):
+        oracle.set_round_mode(rm)
+        try:
+            wantq = oracle.requantize_epilogue(acc, sa, sw, bias, s_out, -5)
+        finally:
+            oracle.set_round_mode(0)
+        np.testing.assert_array_equal(host(ctx.linear_i8_i8(dev(a), dev(sa), dev(w), dev(sw), dev(bias), s_out, -5, mode)), wantq)
+
+
 @pytest.mark.parametrize("m", [1, 4, 16])
 def test_decode_shapes_small_n(ctx, hipq, oracle, m):
     """Config-3 shaped (per-token activations, K=4096) at an N the oracle finishes quickly."""

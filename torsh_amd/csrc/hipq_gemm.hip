@@ -9,6 +9,7 @@
 // activation row: 16-byte stores, 16-byte loads of the per-channel scales.
 
 #include "hipq_gemm_kernels.h"
+#include "hipq_gemm_persist.h"
 
 namespace hipq {
 
@@ -210,21 +211,38 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
     }
     const size_t cus = static_cast<size_t>(ctx->num_cus);
     auto tiles = [&](size_t bm, size_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-#ifdef HIPQ_GEMM_TRACE
-    GemmEpilogue epd = ep;
-    if (const char *e = getenv("HIPQ_GEMM_TS")) epd.ts = reinterpret_cast<long long *>(strtoull(e, nullptr, 0));
-#else
-    const GemmEpilogue &epd = ep;
-#endif
     int variant = gemm_variant_override();
     if (variant == 0 && M <= 16 && K % 256 == 0) return launch_gemv<EPI, EVEN>(ctx, a, w, M, N, K, ep);
     const bool pipe_ok = (K % 128 == 0) && K >= 256;
-    if (variant == 0) variant = pipe_ok ? 2 : 10;
-    if (variant < 10 && !pipe_ok) variant = 10;
+    if (variant == 0 && pipe_ok) {
+        variant = 2;
+        if (tiles(128, 64) >= 2 * cus) {
+            // Many more tiles than CUs: the persistent kernel.  Its tile shape is picked with a
+            // cost model fitted to measurements: a tile costs nk * L + E cycles, where the main
+            // loop is bound by LDS traffic (L per K-tile: fills plus fragment reads) and the
+            // epilogue by the CU's share of HBM write bandwidth (E per tile of 4-byte outputs);
+            // a workgroup runs ceil(tiles / CUs) tiles.  Bigger tiles move fewer LDS bytes per MAC
+            // but quantise worse.  The 256x128 form has no room for residual values in registers.
+            const double nk = double(K / 128), out_scale = (EPI == EPI_I8) ? 0.25 : 1.0;
+            auto cost = [&](size_t bm, size_t bn, double L, double E) {
+                const size_t t = tiles(bm, bn);
+                return double((t + cus - 1) / cus) * (nk * L + E * out_scale);
+            };
+            const double c5 = cost(128, 64, 900.0, 2700.0), c6 = cost(128, 128, 1350.0, 4700.0);
+            const double c7 = (EPI == EPI_F32 && ep.residual) ? 1e30 : cost(256, 128, 1950.0, 9600.0);
+            variant = (c7 <= c6 && c7 <= c5) ? 7 : (c6 <= c5 ? 6 : 5);
+        }
+    }
+    if (variant == 0 || (variant < 10 && !pipe_ok)) variant = 10;
     switch (variant) {
-    case 1: return launch_pipe<128, 64, 6, 4, 1, 1, 4, EPI, EVEN>(ctx, a, w, M, N, K, epd);
-    case 2: return launch_pipe<128, 64, 6, 4, 2, 1, 2, EPI, EVEN>(ctx, a, w, M, N, K, epd);
-    case 3: return launch_pipe<128, 64, 6, 4, 2, 2, 1, EPI, EVEN>(ctx, a, w, M, N, K, epd);
+    case 1: return launch_pipe<128, 64, 6, 4, 1, 1, 4, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+    case 2: return launch_pipe<128, 64, 6, 4, 2, 1, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+    case 3: return launch_pipe<128, 64, 6, 4, 2, 2, 1, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+    case 5: return launch_persist<128, 64, 6, 4, 2, 2, 4, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+    case 6: return launch_persist<128, 128, 4, 4, 2, 2, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+    case 7:
+        if (!(EPI == EPI_F32 && ep.residual)) return launch_persist<256, 128, 3, 4, 2, 2, 1, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+        return launch_persist<128, 128, 4, 4, 2, 2, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
     default: break;
     }
     // Register-staged kernel: any K that is a multiple of 16.

@@ -31,9 +31,6 @@ struct GemmEpilogue {
     const int32_t *cv_wsum = nullptr;  // [oc] sum of the filter's int8 weights
     int cv_corr_mul = 0;               // 128 - zp_in: accumulator += cv_corr_mul * cv_wsum[oc]
     float sa_scalar = 1.0f;            // activation scale used when sa is null
-#ifdef HIPQ_GEMM_TRACE
-    long long *ts = nullptr;  // per-wave phase timestamps
-#endif
 };
 
 constexpr int kGemmThreads = 256;
@@ -303,19 +300,6 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int nk = K / BK;
 
-#ifdef HIPQ_GEMM_TRACE
-#ifdef HIPQ_GEMM_TRACE_WALL
-#define HIPQ_CLK() wall_clock64()
-#else
-#define HIPQ_CLK() clock64()
-#endif
-    long long tr[5] = {HIPQ_CLK(), 0, 0, 0, 0};
-#define HIPQ_TS(i) tr[i] = HIPQ_CLK()
-#define HIPQ_TS_FLUSH() if (ep.ts && lane == 0) { long long *o = ep.ts + (size_t(blockIdx.x) * 16 + wave) * 5; for (int q = 0; q < 5; ++q) o[q] = tr[q]; }
-#else
-#define HIPQ_TS(i)
-#define HIPQ_TS_FLUSH()
-#endif
     if (wave < PW) {
         // ---------------- producer ----------------
         const int8_t *src[IPW];
@@ -357,7 +341,6 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
         for (; issued < 2 && issued < nk; ++issued) issue_stage(issued, issued);
         wait_stages_outstanding<IPW, STAGES - 1>(issued - 1);  // stage 0 has landed
         __builtin_amdgcn_s_barrier();
-        HIPQ_TS(1);
         for (; issued < STAGES && issued < nk; ++issued) issue_stage(issued, issued);
         for (int kt = 0; kt < nk; ++kt) {
             // Requests so far cover stages <= kt+STAGES-1; stage kt+1 must have landed.
@@ -371,13 +354,10 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
             // Every consumer holds stage kt in registers: its buffer is free for stage kt+STAGES.
             if (kt + STAGES < nk) issue_stage(kt + STAGES, kt % STAGES);
         }
-        HIPQ_TS(2);
         if constexpr (WK > 1) {
             __syncthreads();
             __syncthreads();
         }
-        HIPQ_TS(3);
-        HIPQ_TS_FLUSH();
         return;
     }
 
@@ -470,14 +450,12 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     __builtin_amdgcn_s_barrier();  // stage 0 published
     asm volatile("" ::: "memory");
     read_frags(0, 0);
-    HIPQ_TS(1);
     int kt = 0;
     for (; kt + 1 < nk; kt += 2) {
         iteration(kt, 0);
         iteration(kt + 1, 1);
     }
     if (kt < nk) iteration(kt, 0);
-    HIPQ_TS(2);
 
     if constexpr (WK > 1) {
         // Sum the K-split partials through LDS.  Row block i of a wave-group tile is owned
@@ -517,8 +495,6 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
             }
         }
     }
-
-    HIPQ_TS(3);
     // Epilogue.  32x32 accumulator block: lane holds column n = lane%32 and rows
     // m = 8*(r/4) + 4*(lane/32) + r%4 for r = 0..15.
     const float zpf = static_cast<float>(ep.zp_out);
@@ -580,8 +556,6 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
                 }
             }
         }
-        HIPQ_TS(4);
-        HIPQ_TS_FLUSH();
         return;
     }
 #pragma unroll
@@ -649,8 +623,6 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
             }
         }
     }
-    HIPQ_TS(4);
-    HIPQ_TS_FLUSH();
 }
 
 template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN, int CONV = 0>
