@@ -136,6 +136,7 @@ static int32_t run_implicit_gemm(hipq_ctx *ctx, const int8_t *ximg, const int8_t
                                  float s_out, int zp_out, void *out) {
     const int hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw;
     GemmEpilogue ep{nullptr, 0, sw, bias, s_out, zp_out, out};
+    ep.s_out_inv = host_recip_for_div(s_out);
     ep.sa_scalar = s_in;
     ep.cv_tiles_per_tap = g.c / 128;
     ep.cv_kw = g.kw;

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
         scale = params->scale;
         zp = params->zero_point;
     }
-    const float inv = 1.0f / scale;
+    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
     const float zpf = static_cast<float>(zp);
     const int ilo = static_cast<int>(lo), ihi = static_cast<int>(hi);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) &&
@@ -362,12 +362,13 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     }
     if (st != HIPQ_SUCCESS) return;
     const float zpf = static_cast<float>(zp);
+    const float inv = recip_for_div(scale);  // once per row; each element then divides with two FMAs
     uint32_t *q4 = reinterpret_cast<uint32_t *>(qr);
     auto quant4 = [&](float4 t) {
-        return pack4(quantize_int<true, EVEN>(t.x, scale, 0.0f, zpf, qmin, qmax),
-                     quantize_int<true, EVEN>(t.y, scale, 0.0f, zpf, qmin, qmax),
-                     quantize_int<true, EVEN>(t.z, scale, 0.0f, zpf, qmin, qmax),
-                     quantize_int<true, EVEN>(t.w, scale, 0.0f, zpf, qmin, qmax));
+        return pack4(quantize_int<true, EVEN>(t.x, scale, inv, zpf, qmin, qmax),
+                     quantize_int<true, EVEN>(t.y, scale, inv, zpf, qmin, qmax),
+                     quantize_int<true, EVEN>(t.z, scale, inv, zpf, qmin, qmax),
+                     quantize_int<true, EVEN>(t.w, scale, inv, zpf, qmin, qmax));
     };
 #pragma unroll
     for (int i = 0; i < kCache; ++i) {
@@ -376,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     }
     for (size_t v = size_t(lane) + size_t(kCache) * TPR; v < nvec; v += TPR) q4[v] = quant4(x4[v]);
     for (size_t c = nvec * 4 + lane; c < cols; c += TPR)
-        qr[c] = static_cast<int8_t>(quantize_int<true, EVEN>(xr[c], scale, 0.0f, zpf, qmin, qmax));
+        qr[c] = static_cast<int8_t>(quantize_int<true, EVEN>(xr[c], scale, inv, zpf, qmin, qmax));
 }
 
 // quantize_per_channel_auto for a channel axis that is not the leading one:
@@ -405,10 +406,11 @@ __global__ __launch_bounds__(kBlock) void quantize_per_channel_auto_kernel(
     }
     if (st != HIPQ_SUCCESS) return;
     const float zpf = static_cast<float>(zp), lo = static_cast<float>(qmin), hi = static_cast<float>(qmax);
+    const float inv = recip_for_div(scale);
     for (size_t i = threadIdx.x; i < per; i += kBlock) {
         const size_t o = i / inner, in = i % inner;
         const size_t idx = (o * channels + ch) * inner + in;
-        out[idx] = static_cast<int8_t>(to_int_nan0(quantize_value<true, EVEN>(x[idx], scale, 0.0f, zpf, lo, hi)));
+        out[idx] = static_cast<int8_t>(to_int_nan0(quantize_value<true, EVEN>(x[idx], scale, inv, zpf, lo, hi)));
     }
 }
 
@@ -422,7 +424,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_channel_kernel(const floa
     for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += size_t(gridDim.x) * kBlock) {
         const size_t c = (i / inner) % channels;
         const float s = scales[c];
-        const float inv = 1.0f / s;
+        const float inv = DIV ? 0.0f : 1.0f / s;  // a scale per element: the division form divides directly
         const float q = quantize_value<DIV, EVEN>(x[i], s, inv, static_cast<float>(zps[c]), -128.0f, 127.0f);
         out[i] = static_cast<int8_t>(to_int_nan0(q));
     }
@@ -449,12 +451,13 @@ __global__ __launch_bounds__(kBlock) void requantize_kernel(const int32_t *__res
                                                              int8_t *__restrict__ out) {
     const size_t total = rows * cols;
     const float zpf = static_cast<float>(zp_out);
+    const float inv_out = recip_for_div(s_out);
     for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += size_t(gridDim.x) * kBlock) {
         const size_t r = i / cols, c = i % cols;
         const float s = (sa_per_row ? sa[r] : sa[0]) * sw[c];
         float v = static_cast<float>(acc[i]) * s;
         if (bias) v = v + bias[c];
-        const float q = clamp_keep_nan(round_mode<EVEN>(v / s_out) + zpf, -128.0f, 127.0f);
+        const float q = clamp_keep_nan(round_mode<EVEN>(div_rn(v, s_out, inv_out)) + zpf, -128.0f, 127.0f);
         out[i] = static_cast<int8_t>(to_int_nan0(q));
     }
 }

@@ -9,7 +9,7 @@
 namespace hipq {
 
 constexpr int kRowBlock = 256;
-constexpr int kRowCache = 8;  // float4 per thread kept in registers
+constexpr int kRowCacheMax = 12;  // most float4 a thread keeps in registers (RC template parameter)
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -51,11 +51,20 @@ __device__ __forceinline__ float row_max(float v, float *lds) {
     }
 }
 
-// tanh-form GELU, crates/torsh-nn/src/layers/activation/modern.rs:124-136.
+// tanh-form GELU, crates/torsh-nn/src/layers/activation/modern.rs:124-136:
+//   0.5 * x * (1 + tanh(u)),  u = sqrt(2/pi) * (x + 0.044715 x^3).
+// Evaluated as x / (1 + exp(-2u)), which is the same function (1 + tanh(u) = 2 / (1 + exp(-2u)))
+// without the cancellation of 1 + tanh(u) for negative x, and costs one v_exp_f32 and one
+// v_rcp_f32 instead of a tanhf call: the fused GELU + quantize kernel was bound by tanhf, not by
+// HBM.  Against the reference's evaluation order in f32 the difference stays below 2e-6
+// relative + 1e-7 absolute (the reference form itself carries up to |x| * 3e-8 of cancellation
+// error).
 __device__ __forceinline__ float gelu_tanh(float x) {
     const float x3 = x * x * x;
     const float inner = (x + x3 * 0.044715f) * 0.7978845608028654f;  // sqrt(2/pi)
-    return (x * 0.5f) * (tanhf(inner) + 1.0f);
+    // exp(-2u) as exp2(u * -2*log2(e)); clamp keeps the exponent finite (result 0 or x either way).
+    const float e = __builtin_amdgcn_exp2f(fminf(fmaxf(inner * -2.8853900817779268f, -126.0f), 126.0f));
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 enum { ROW_LAYERNORM = 0, ROW_GELU = 1 };
@@ -64,34 +73,23 @@ enum { ROW_LAYERNORM = 0, ROW_GELU = 1 };
 // QUANT: write the row as per-token symmetric int8 (scale = absmax/127,
 // q = clamp(round(y / scale)), the division form of
 // crates/torsh-quantization/src/algorithms.rs:126-242) instead of fp32.
-// Rows are TPR threads wide and at most TPR * kRowCache * 4 columns long; cols % 4 == 0.
-template <int TPR, int OP, bool QUANT, bool EVEN>
-__global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restrict__ x, size_t rows, size_t cols,
-                                                            const float *__restrict__ gamma,
-                                                            const float *__restrict__ beta, float eps,
-                                                            float *__restrict__ out_f, int8_t *__restrict__ out_q,
-                                                            float *__restrict__ out_scales) {
-    constexpr int kRowsPerBlock = kRowBlock / TPR;
-    __shared__ float lds[kRowBlock / kWave];
-    const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
-    const size_t row = size_t(blockIdx.x) * kRowsPerBlock + sub;
-    const bool active = row < rows;
+// Rows are TPR threads wide and at most TPR * RC * 4 columns long (RC float4 per thread, all
+// requested before the first is used); cols % 4 == 0.  The row is read once and written once,
+// so both streams bypass the caches.
+template <int TPR, int RC, int OP, bool QUANT, bool EVEN>
+__device__ __forceinline__ void row_op_body(float4 (&v)[RC], size_t row, bool active, int lane, size_t cols,
+                                            const float *__restrict__ gamma, const float *__restrict__ beta,
+                                            float eps, float *__restrict__ out_f, int8_t *__restrict__ out_q,
+                                            float *__restrict__ out_scales, float *lds) {
     const size_t nvec = cols / 4;
-    const float4 *x4 = reinterpret_cast<const float4 *>(x + (active ? row : 0) * cols);
-    float4 v[kRowCache];
-#pragma unroll
-    for (int i = 0; i < kRowCache; ++i) {
-        const size_t idx = size_t(lane) + size_t(i) * TPR;
-        v[i] = (active && idx < nvec) ? x4[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
     if constexpr (OP == ROW_LAYERNORM) {
         float s = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        for (int i = 0; i < RC; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
         const float mean = row_sum<TPR>(s, lds) / static_cast<float>(cols);
         float sq = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i) {
+        for (int i = 0; i < RC; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
             if (idx < nvec) {
                 const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
@@ -102,7 +100,7 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restri
         const float rstd = 1.0f / sqrtf(var + eps);
         const float4 *g4 = reinterpret_cast<const float4 *>(gamma), *b4 = reinterpret_cast<const float4 *>(beta);
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i) {
+        for (int i = 0; i < RC; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
             if (idx < nvec) {
                 float4 y = make_float4((v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
@@ -120,21 +118,23 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restri
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i)
-            v[i] = make_float4(gelu_tanh(v[i].x), gelu_tanh(v[i].y), gelu_tanh(v[i].z), gelu_tanh(v[i].w));
+        for (int i = 0; i < RC; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            if (idx < nvec) v[i] = make_float4(gelu_tanh(v[i].x), gelu_tanh(v[i].y), gelu_tanh(v[i].z), gelu_tanh(v[i].w));
+        }
     }
     if constexpr (!QUANT) {
         if (!active) return;
         float4 *o4 = reinterpret_cast<float4 *>(out_f + row * cols);
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i) {
+        for (int i = 0; i < RC; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
-            if (idx < nvec) o4[idx] = v[i];
+            if (idx < nvec) store_stream(o4 + idx, v[i]);
         }
     } else {
         float am = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i) {
+        for (int i = 0; i < RC; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
             if (idx < nvec) am = fmaxf(fmaxf(am, fmaxf(fabsf(v[i].x), fabsf(v[i].y))), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
         }
@@ -145,17 +145,57 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restri
         float scale = am < FLT_EPSILON ? 1.0f : am / 127.0f;
         if (!(fabsf(am) <= FLT_MAX)) scale = NAN;
         if (lane == 0) out_scales[row] = scale;
+        const float inv = recip_for_div(scale);  // once per row
         uint32_t *q4 = reinterpret_cast<uint32_t *>(out_q + row * cols);
 #pragma unroll
-        for (int i = 0; i < kRowCache; ++i) {
+        for (int i = 0; i < RC; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
             if (idx < nvec) {
-                q4[idx] = pack4(quantize_int<true, EVEN>(v[i].x, scale, 0.0f, 0.0f, -128, 127),
-                                quantize_int<true, EVEN>(v[i].y, scale, 0.0f, 0.0f, -128, 127),
-                                quantize_int<true, EVEN>(v[i].z, scale, 0.0f, 0.0f, -128, 127),
-                                quantize_int<true, EVEN>(v[i].w, scale, 0.0f, 0.0f, -128, 127));
+                store_stream(q4 + idx, pack4(quantize_int<true, EVEN>(v[i].x, scale, inv, 0.0f, -128, 127),
+                                             quantize_int<true, EVEN>(v[i].y, scale, inv, 0.0f, -128, 127),
+                                             quantize_int<true, EVEN>(v[i].z, scale, inv, 0.0f, -128, 127),
+                                             quantize_int<true, EVEN>(v[i].w, scale, inv, 0.0f, -128, 127)));
             }
         }
+    }
+}
+
+// Workgroups walk the row groups with a grid stride; the next group's row is requested before
+// the current one is processed, so loads, arithmetic and stores of different rows overlap in
+// every wave (with one row per wave and a single generation of workgroups the three phases ran
+// one after the other across the whole chip).
+template <int TPR, int RC, int OP, bool QUANT, bool EVEN>
+__global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restrict__ x, size_t rows, size_t cols,
+                                                            const float *__restrict__ gamma,
+                                                            const float *__restrict__ beta, float eps,
+                                                            float *__restrict__ out_f, int8_t *__restrict__ out_q,
+                                                            float *__restrict__ out_scales) {
+    constexpr int kRowsPerBlock = kRowBlock / TPR;
+    __shared__ float lds[kRowBlock / kWave];
+    const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
+    const size_t nvec = cols / 4;
+    const size_t groups = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    auto load_row = [&](size_t g, float4(&dst)[RC]) {
+        const size_t row = g * kRowsPerBlock + sub;
+        const bool active = row < rows;
+        const float4 *x4 = reinterpret_cast<const float4 *>(x + (active ? row : 0) * cols);
+#pragma unroll
+        for (int i = 0; i < RC; ++i) {
+            const size_t idx = size_t(lane) + size_t(i) * TPR;
+            dst[i] = (active && idx < nvec) ? load_stream(x4 + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    float4 v[RC], nx[RC];
+    size_t g = blockIdx.x;
+    if (g < groups) load_row(g, v);
+    for (; g < groups; g += gridDim.x) {
+        const size_t gn = g + gridDim.x;
+        if (gn < groups) load_row(gn, nx);
+        const size_t row = g * kRowsPerBlock + sub;
+        row_op_body<TPR, RC, OP, QUANT, EVEN>(v, row, row < rows, lane, cols, gamma, beta, eps, out_f, out_q, out_scales,
+                                              lds);
+#pragma unroll
+        for (int i = 0; i < RC; ++i) v[i] = nx[i];
     }
 }
 
@@ -178,30 +218,44 @@ __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, c
         out[i] = a[i] + b[i];
 }
 
+// Enough workgroups to fill the chip a few times over, few enough that each walks several
+// row groups and overlaps their phases.
+static int row_grid(hipq_ctx *ctx, size_t rows, int rows_per_block) {
+    const size_t groups = (rows + rows_per_block - 1) / rows_per_block;
+    constexpr int per_cu = 8;  // measured best of 1, 2, 4, 8 on [8192, 768] and [8192, 3072]
+    const size_t cap = size_t(ctx->num_cus) * per_cu;
+    return static_cast<int>(groups < cap ? groups : cap);
+}
+
 template <int OP, bool QUANT>
 static int32_t launch_row_op(const char *fn, hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
                              const float *beta, float eps, int32_t mode, float *out_f, int8_t *out_q,
                              float *out_scales) {
     if (rows == 0) return HIPQ_SUCCESS;
     if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length", fn);
-    if (cols % 4 != 0 || cols > size_t(kRowBlock) * kRowCache * 4)
+    if (cols % 4 != 0 || cols > size_t(kRowBlock) * kRowCacheMax * 4)
         return fail(HIPQ_SHAPE_ERROR, "%s: row length %zu must be a multiple of 4 and at most %d", fn, cols,
-                    kRowBlock * kRowCache * 4);
+                    kRowBlock * kRowCacheMax * 4);
     uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gamma) |
                      reinterpret_cast<uintptr_t>(beta) | reinterpret_cast<uintptr_t>(out_f);
     if ((bits & 15u) || (reinterpret_cast<uintptr_t>(out_q) & 3u))
         return fail(HIPQ_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", fn);
     if (rows >> 31) return fail(HIPQ_SHAPE_ERROR, "%s: too many rows", fn);
     const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
-    const bool wave_rows = cols <= size_t(kWave) * kRowCache * 4;
-#define HIPQ_ROW(TPR, E)                                                                                          \
-    hipLaunchKernelGGL((row_op_kernel<TPR, OP, QUANT, E>), dim3(static_cast<int>((rows + kRowBlock / TPR - 1) / (kRowBlock / TPR))), \
+    // A wavefront per row while the row fits 12 float4 per lane (no workgroup barrier in the row
+    // reductions), else the whole workgroup; the register cache is sized to the row.
+    const size_t vec_per_wave_lane = (cols / 4 + kWave - 1) / kWave, vec_per_block_lane = (cols / 4 + kRowBlock - 1) / kRowBlock;
+#define HIPQ_ROW(TPR, RC, E)                                                                                      \
+    hipLaunchKernelGGL((row_op_kernel<TPR, RC, OP, QUANT, E>), dim3(row_grid(ctx, rows, kRowBlock / TPR)), \
                        dim3(kRowBlock), 0, ctx->stream, x, rows, cols, gamma, beta, eps, out_f, out_q, out_scales)
-    if (wave_rows) {
-        if (even) HIPQ_ROW(kWave, true); else HIPQ_ROW(kWave, false);
-    } else {
-        if (even) HIPQ_ROW(kRowBlock, true); else HIPQ_ROW(kRowBlock, false);
-    }
+#define HIPQ_ROW_E(TPR, RC) do { if (even) HIPQ_ROW(TPR, RC, true); else HIPQ_ROW(TPR, RC, false); } while (0)
+    if (vec_per_wave_lane <= 4) HIPQ_ROW_E(kWave, 4);
+    else if (vec_per_wave_lane <= 8) HIPQ_ROW_E(kWave, 8);
+    else if (vec_per_wave_lane <= 12) HIPQ_ROW_E(kWave, 12);
+    else if (vec_per_block_lane <= 4) HIPQ_ROW_E(kRowBlock, 4);
+    else if (vec_per_block_lane <= 8) HIPQ_ROW_E(kRowBlock, 8);
+    else HIPQ_ROW_E(kRowBlock, 12);
+#undef HIPQ_ROW_E
 #undef HIPQ_ROW
     return check_launch(fn);
 }

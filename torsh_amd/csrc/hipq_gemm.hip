@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemv_i8_kernel(const int8_t *__r
             const float zpf = static_cast<float>(ep.zp_out);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                q[i] = to_int_nan0(clamp_keep_nan(round_mode<EVEN>(v[i] / ep.s_out) + zpf, -128.0f, 127.0f));
+                q[i] = to_int_nan0(clamp_keep_nan(round_mode<EVEN>(div_rn(v[i], ep.s_out, ep.s_out_inv)) + zpf, -128.0f, 127.0f));
             if (vec) {
                 *reinterpret_cast<uint32_t *>(o + off) = pack4(q[0], q[1], q[2], q[3]);
             } else {
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_i8_generic_kernel(const int
                 if (ep.residual) v = v + ep.residual[idx];
                 static_cast<float *>(ep.out)[idx] = v;
             } else {
-                const float q = clamp_keep_nan(round_mode<EVEN>(v / ep.s_out) + static_cast<float>(ep.zp_out), -128.0f,
+                const float q = clamp_keep_nan(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + static_cast<float>(ep.zp_out), -128.0f,
                                                127.0f);
                 static_cast<int8_t *>(ep.out)[idx] = static_cast<int8_t>(to_int_nan0(q));
             }
@@ -338,6 +338,7 @@ int32_t hipq_linear_i8_i8(hipq_ctx *ctx, const int8_t *a, const float *a_scale, 
         HIPQ_REQUIRE_PTR(w);
     }
     GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, out_scale, out_zero_point, out};
+    ep.s_out_inv = host_recip_for_div(out_scale);
     if (mode & HIPQ_ROUND_HALF_EVEN) return launch_gemm<EPI_I8, true>(ctx, a, w, m, n, k, ep);
     return launch_gemm<EPI_I8, false>(ctx, a, w, m, n, k, ep);
 }

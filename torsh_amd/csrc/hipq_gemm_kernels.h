@@ -31,7 +31,15 @@ struct GemmEpilogue {
     const int32_t *cv_wsum = nullptr;  // [oc] sum of the filter's int8 weights
     int cv_corr_mul = 0;               // 128 - zp_in: accumulator += cv_corr_mul * cv_wsum[oc]
     float sa_scalar = 1.0f;            // activation scale used when sa is null
+    float s_out_inv = 0.0f;            // recip_for_div(s_out), or 0 to divide directly (requantize only)
 };
+
+// Host-side twin of recip_for_div: the correctly rounded 1/b if it is a normal number, else 0.
+static inline float host_recip_for_div(float b) {
+    const float y = 1.0f / b;
+    const float ay = y < 0.0f ? -y : y;
+    return (ay >= 1.17549435e-38f && ay <= 3.40282347e+38f) ? y : 0.0f;
+}
 
 constexpr int kGemmThreads = 256;
 
@@ -73,7 +81,7 @@ __device__ __forceinline__ void epilogue_store4(const GemmEpilogue &ep, int m, i
             const float zpf = static_cast<float>(ep.zp_out);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                q[r] = to_int_nan0(clamp_keep_nan(round_mode<EVEN>(v[r] / ep.s_out) + zpf, -128.0f, 127.0f));
+                q[r] = to_int_nan0(clamp_keep_nan(round_mode<EVEN>(div_rn(v[r], ep.s_out, ep.s_out_inv)) + zpf, -128.0f, 127.0f));
             if (vec) {
                 *reinterpret_cast<uint32_t *>(o + off) = pack4(q[0], q[1], q[2], q[3]);
             } else {
@@ -549,7 +557,7 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
                         if constexpr (EPI == EPI_F32) {
                             static_cast<float *>(ep.out)[off] = v;
                         } else {
-                            const float qv = clamp_keep_nan(round_mode<EVEN>(v / ep.s_out) + zpf, -128.0f, 127.0f);
+                            const float qv = clamp_keep_nan(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128.0f, 127.0f);
                             static_cast<int8_t *>(ep.out)[off] = static_cast<int8_t>(to_int_nan0(qv));
                         }
                     }
@@ -616,7 +624,7 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
                         if (ep.residual) v = v + res[r][j];
                         __builtin_nontemporal_store(v, static_cast<float *>(ep.out) + off);
                     } else {
-                        const int q = clamp_to_int(round_mode<EVEN>(v / ep.s_out) + zpf, -128, 127);
+                        const int q = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
                         __builtin_nontemporal_store(static_cast<int8_t>(q), static_cast<int8_t *>(ep.out) + off);
                     }
                 }

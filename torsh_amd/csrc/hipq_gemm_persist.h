@@ -398,7 +398,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                             int q[4];
 #pragma unroll
                             for (int c = 0; c < 4; ++c)
-                                q[c] = clamp_to_int(round_mode<EVEN>(v[c] / ep.s_out) + zpf, -128, 127);
+                                q[c] = clamp_to_int(round_mode<EVEN>(div_rn(v[c], ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
                             store_stream(reinterpret_cast<uint32_t *>(static_cast<int8_t *>(ep.out) + off),
                                          pack4(q[0], q[1], q[2], q[3]));
                         }
@@ -490,7 +490,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                                 if constexpr (RESIDUAL) v = v + res[RES_ALL ? i : 0][r][j];
                                 __builtin_nontemporal_store(v, reinterpret_cast<float *>(p));
                             } else {
-                                const int q = clamp_to_int(round_mode<EVEN>(v / ep.s_out) + zpf, -128, 127);
+                                const int q = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
                                 __builtin_nontemporal_store(static_cast<int8_t>(q), reinterpret_cast<int8_t *>(p));
                             }
                         }

