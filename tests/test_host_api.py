@@ -50,6 +50,18 @@ def _binary():
     return BIN
 
 
+def test_two_fma_division_equals_ieee_division():
+    """The kernels divide by a per-row / per-tensor scale as fma(fma(-q0, b, a), y, q0) with y = 1/b; this sweeps every
+    numerator significand for a few dozen denominators on the CPU and demands equality with a / b."""
+    _binary()
+    exe = os.path.join(ROOT, "tests", "host", "bin", "div_rn_check")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "host"), "bin/div_rn_check"], check=True, capture_output=True)
+    proc = subprocess.run([exe, "200"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert " 0 mismatches" in proc.stdout
+
+
 def _run(args):
     proc = subprocess.run([_binary(), *args], capture_output=True, text=True, timeout=300)
     results = {}
