@@ -17,28 +17,43 @@ namespace hipq {
 
 constexpr int kConvThreads = 256;
 
-// u8 NCHW -> i8 NHWC with a border of `pad` pixels holding (zp - 128).
+// u8 NCHW -> i8 NHWC with a border of `pad` pixels holding (zp - 128).  One workgroup per
+// padded image row: the C x W source bytes of that row (W-byte runs, one per channel) are
+// transposed through LDS so that the NHWC row is written as 16-byte pieces; one extra
+// workgroup clears the slack behind the last image that the last windows read into.
+// C % 16 == 0.  Dynamic LDS: W * (C + 16) bytes.
 __global__ __launch_bounds__(kConvThreads) void conv_pack_input_kernel(const uint8_t *__restrict__ x, int C, int H, int W,
-                                                                         int pad_h, int pad_w, int zp,
-                                                                         int8_t *__restrict__ out) {
+                                                                         int pad_h, int pad_w, int zp, int nb,
+                                                                         int8_t *__restrict__ out, size_t slack) {
+    extern __shared__ __attribute__((aligned(16))) int8_t tile[];  // [W][C + 16]
     const int hp_count = H + 2 * pad_h, wp_count = W + 2 * pad_w;
+    const uint32_t border4 = static_cast<uint32_t>(static_cast<uint8_t>(zp - 128)) * 0x01010101u;
+    if (static_cast<int>(blockIdx.x) == nb * hp_count) {
+        int8_t *tail = out + size_t(nb) * hp_count * wp_count * C;
+        for (size_t i = threadIdx.x; i < slack; i += kConvThreads) tail[i] = 0;
+        return;
+    }
     const int n = blockIdx.x / hp_count, hp = blockIdx.x % hp_count;
     const int h = hp - pad_h;
-    int8_t *orow = out + (size_t(n) * hp_count + hp) * wp_count * C;
-    const int8_t border = static_cast<int8_t>(zp - 128);
-    for (int wp = 0; wp < wp_count; ++wp) {
-        const int w = wp - pad_w;
-        const bool inside = h >= 0 && h < H && w >= 0 && w < W;
-        for (int c = threadIdx.x; c < C; c += kConvThreads) {
-            int8_t v = border;
-            if (inside) v = static_cast<int8_t>(static_cast<int>(x[((size_t(n) * C + c) * H + h) * W + w]) - 128);
-            orow[size_t(wp) * C + c] = v;
+    const bool row_inside = h >= 0 && h < H;
+    const int pitch = C + 16;
+    if (row_inside) {
+        const uint8_t *src = x + (size_t(n) * C * H + h) * W;  // + c * H * W + w
+        for (int e = threadIdx.x; e < C * W; e += kConvThreads) {
+            const int c = e / W, w = e % W;
+            tile[w * pitch + c] = static_cast<int8_t>(static_cast<int>(src[size_t(c) * H * W + w]) - 128);
         }
     }
-}
-
-__global__ void conv_fill_i8_kernel(int8_t *p, int8_t v, size_t n) {
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) p[i] = v;
+    __syncthreads();
+    uint4 *orow = reinterpret_cast<uint4 *>(out + (size_t(n) * hp_count + hp) * wp_count * C);
+    const int vec_per_pixel = C / 16;
+    for (int i = threadIdx.x; i < wp_count * vec_per_pixel; i += kConvThreads) {
+        const int wp = i / vec_per_pixel, cv = i % vec_per_pixel;
+        const int w = wp - pad_w;
+        uint4 v = make_uint4(border4, border4, border4, border4);
+        if (row_inside && w >= 0 && w < W) v = *reinterpret_cast<const uint4 *>(tile + w * pitch + cv * 16);
+        orow[i] = v;
+    }
 }
 
 // int8 [OC, IC, KH*KW] -> [OC, KH*KW, IC] and wsum[oc] = sum of the filter's weights.
@@ -126,7 +141,9 @@ static int32_t check_geom(const char *fn, const ConvGeom &g) {
 }
 
 static bool fast_path_ok(const ConvGeom &g) {
-    return g.sh == 1 && g.sw == 1 && g.c % 128 == 0 && g.c * g.kh * g.kw >= 256 && g.oc >= 1;
+    // (the layout pass stages one image row, w * (c + 16) bytes, in the default 64 KiB of LDS)
+    return g.sh == 1 && g.sw == 1 && g.c % 128 == 0 && g.c * g.kh * g.kw >= 256 && g.oc >= 1 &&
+           size_t(g.w) * (g.c + 16) <= 64 * 1024;
 }
 
 // Runs the implicit GEMM on an already packed image / filter pair.
@@ -179,9 +196,9 @@ static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int
     int8_t *ximg = reinterpret_cast<int8_t *>(static_cast<char *>(s) + kScratchHeader);
     int8_t *wbuf = ximg + align256(img_bytes + slack);
     int32_t *wsbuf = reinterpret_cast<int32_t *>(wbuf + align256(w_bytes));
-    hipLaunchKernelGGL(conv_pack_input_kernel, dim3(g.nb * hp), dim3(kConvThreads), 0, ctx->stream, x, g.c, g.h, g.w, g.ph,
-                       g.pw, zp_in, ximg);
-    hipLaunchKernelGGL(conv_fill_i8_kernel, dim3(8), dim3(256), 0, ctx->stream, ximg + img_bytes, int8_t(0), slack);
+    const size_t pack_lds = size_t(g.w) * (g.c + 16);
+    hipLaunchKernelGGL(conv_pack_input_kernel, dim3(g.nb * hp + 1), dim3(kConvThreads), pack_lds, ctx->stream, x, g.c, g.h,
+                       g.w, g.ph, g.pw, zp_in, g.nb, ximg, slack);
     if (!wpacked) {
         hipLaunchKernelGGL(conv_pack_weights_kernel, dim3(g.oc), dim3(kConvThreads), 0, ctx->stream, w, g.c, taps, wbuf,
                            wsbuf);
