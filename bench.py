@@ -63,9 +63,10 @@ def cpu_baseline(m: int, n: int, k: int):
     a = rng.integers(-127, 128, size=(m_sample, k), dtype=np.int8)
     b_kn = rng.integers(-127, 128, size=(k, n), dtype=np.int8)  # the reference's [K,N] operand
     t = pyoracle.time_matmul_rows(a, b_kn, m_sample)
-    # widen the sample until it is a few seconds of work, capped at 32 rows
-    while t < 2.0 and m_sample < 32:
-        m_sample *= 2
+    # one more run sized from that rate to about 12 s of work (the bounded sample asked of this leg)
+    rows = int(max(m_sample, min(m, round(12.0 / (t / m_sample)))))
+    if rows > m_sample:
+        m_sample = rows
         a = rng.integers(-127, 128, size=(m_sample, k), dtype=np.int8)
         t = pyoracle.time_matmul_rows(a, b_kn, m_sample)
     tops = 2.0 * m_sample * n * k / t / 1e12
@@ -241,6 +242,31 @@ def main() -> int:
 
     if not args.no_extra:
         extra = {}
+        # The same step with two independent batches in flight (two contexts, each with its own stream): the
+        # latency-bound activation quantize of one batch runs beside the GEMM of the other.  Reported next to
+        # `value`, which stays the one-stream figure.
+        ctx2 = hipq.Context(0, own_stream=True)
+        ctx3 = hipq.Context(0, own_stream=True)
+        pt = [0]
+
+        def step_two_streams():
+            i = pt[0] % pool
+            pt[0] += 1
+            (ctx2 if i % 2 == 0 else ctx3).linear_dynamic(xs[i], wq[i], sw[i], bias, per_token=False,
+                                                        mode=hipq.FORM_MUL_INV, out=outs[i])
+
+        for _ in range(args.warmup):
+            step_two_streams()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_two_streams()
+        torch.cuda.synchronize()
+        ms2 = (time.perf_counter() - t0) * 1e3 / args.steps
+        extra["linear_step_two_batches_in_flight"] = {"ms_per_step": ms2, "TOP/s": ops / (ms2 * 1e-3) / 1e12,
+                                                      "note": "alternating batches on two contexts/streams"}
+        ctx2.close()
+        ctx3.close()
         n = 4096 * 4096
         npool = 10  # 10 x (64 + 16 + 64) MiB > memory-side cache
         fx = [torch.randn(n, generator=g, device="cuda") for _ in range(npool)]
