@@ -297,8 +297,38 @@ def main() -> int:
             i = rot()
             ctx.quantize_dynamic_per_tensor(fx[i], out=fq[i], params=params)
 
+        # calibration / quality kernels on the same 16 Mi-element tensors
+        metrics_rec = ctx.quantization_metrics(fx[0], fy[0])
+        observe_rec = ctx.observe(fx[0])
+        hist = torch.zeros(256, dtype=torch.int64, device="cuda")
+
+        def run_metrics():
+            i = rot()
+            ctx.quantization_metrics(fx[i], fy[i], out=metrics_rec)
+
+        def run_fused_metrics():
+            i = rot()
+            ctx.fake_quantize_metrics(fx[i], 0.04, 0, out=metrics_rec)
+
+        def run_fake_quant():
+            i = rot()
+            ctx.fake_quantize(fx[i], 0.04, 0, out=fy[i])
+
+        def run_observe():
+            i = rot()
+            ctx.observe(fx[i], out=observe_rec)
+
+        def run_histogram():
+            i = rot()
+            ctx.histogram(fx[i], -6.0, 6.0, 256, counts=hist)
+
         for name, fn, bytes_per in (("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
-                                    ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9)):
+                                    ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9),
+                                    ("quality_metrics_two_tensors_f32", run_metrics, 8),
+                                    ("fake_quantize_metrics_fused_f32", run_fused_metrics, 4),
+                                    ("fake_quantize_f32", run_fake_quant, 8),
+                                    ("observe_minmax_nonfinite_f32", run_observe, 4),
+                                    ("histogram_256_bins_f32", run_histogram, 4)):
             ms = event_time_ms(fn, reps=50, warmup=5)
             gbps = bytes_per * n / (ms * 1e-3) / 1e9
             extra[name] = {"us": ms * 1e3, "GB/s": gbps, "frac_hbm_peak": gbps / PEAK_HBM_GBPS,

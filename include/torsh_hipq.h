@@ -300,6 +300,73 @@ HIPQ_API int32_t hipq_gelu_tanh_quantize_f32_i8(hipq_ctx *ctx, const float *x, s
 /* out = a + b (skip connection; Tensor::add). */
 HIPQ_API int32_t hipq_add_f32(hipq_ctx *ctx, const float *a, const float *b, size_t n, float *out);
 
+/* ---- calibration observers and quality metrics ------------------------ */
+/* Extra `mode` bit of the fake-quantizing entry points: the clamped value goes
+ * through `as i32` before it is dequantized (NaN becomes 0), as
+ * ModelQuantizer::quantize_value does (crates/torsh-models/src/quantization.rs:336-342);
+ * without it the value stays in its f32 carrier and a NaN stays a NaN
+ * (crates/torsh-quantization/src/simd_ops.rs:36-46). */
+enum { HIPQ_FAKE_INT_CAST = 4 };
+
+/* QuantizationMetrics, crates/torsh-quantization/src/metrics.rs:30-48 (same
+ * fields, same order). */
+typedef struct hipq_quant_metrics {
+    float mse;
+    float psnr;
+    float snr;
+    float mae;
+    float max_error;
+    float zero_error_percentage;
+    float cosine_similarity;
+    float compression_ratio;
+} hipq_quant_metrics;
+
+/* calculate_quantization_metrics, crates/torsh-quantization/src/metrics.rs:67-175,
+ * over two f32 tensors of n elements in one pass; out_metrics is a device
+ * record.  n == 0 yields QuantizationMetrics::default() (metrics.rs:50-63).
+ * The sums are carried in f64 (the reference adds f32 terms in element
+ * order); max_error and the zero-error count are exact. */
+HIPQ_API int32_t hipq_quantization_metrics_f32(hipq_ctx *ctx, const float *original, const float *quantized, size_t n,
+                                               uint32_t original_bits, uint32_t quantized_bits,
+                                               hipq_quant_metrics *out_metrics);
+/* The quantize -> dequantize -> metrics sequence of compare_quantization_configs
+ * (metrics.rs:178-240) and of ModelQuantizer::calculate_quantization_stats
+ * (crates/torsh-models/src/quantization.rs:504-533) fused into one pass over x:
+ * the dequantized image is formed in registers and never written.  Quantizer:
+ * q = clamp(round(x * (1/scale) | x / scale) + zp, qmin, qmax), y = (q - zp) * scale;
+ * `mode` = HIPQ_ROUND_* | HIPQ_FORM_* | HIPQ_FAKE_INT_CAST.  `params` (device,
+ * may be NULL) overrides scale and zero_point. */
+HIPQ_API int32_t hipq_fake_quantize_metrics_f32(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                                int32_t zero_point, const hipq_qparams *params, int32_t qmin,
+                                                int32_t qmax, int32_t mode, uint32_t original_bits,
+                                                uint32_t quantized_bits, hipq_quant_metrics *out_metrics);
+/* ModelQuantizer::quantize_tensor, crates/torsh-models/src/quantization.rs:309-332:
+ * out = dequantize(quantize(x)) as f32 ("fake quantization"); same quantizer
+ * and `mode` as above. */
+HIPQ_API int32_t hipq_fake_quantize_f32(hipq_ctx *ctx, const float *x, size_t n, float scale, int32_t zero_point,
+                                        const hipq_qparams *params, int32_t qmin, int32_t qmax, int32_t mode,
+                                        float *out);
+
+/* What Observer::update derives from one batch before it touches its state
+ * (crates/torsh-quantization/src/observers.rs:122-150): the batch range (NaN
+ * ignoring f32::min/max folds from +inf/-inf) and how many values are NaN or
+ * infinite (the reference rejects the batch when this is not 0). */
+typedef struct hipq_observe_stats {
+    float min_val;
+    float max_val;
+    uint64_t nonfinite;
+} hipq_observe_stats;
+HIPQ_API int32_t hipq_observe_f32(hipq_ctx *ctx, const float *x, size_t n, hipq_observe_stats *out_stats);
+
+/* Histogram update of the Histogram observer (observers.rs:186-225) with the
+ * bin rule of Observer::value_to_bin_index (observers.rs:313-333) over the
+ * range [range_min, range_max]: counts[bin] += occurrences, counts is a device
+ * array of num_bins uint64 that the caller zeroes once and keeps across
+ * batches.  Exact integer counts. */
+#define HIPQ_HISTOGRAM_MAX_BINS 16384
+HIPQ_API int32_t hipq_histogram_f32(hipq_ctx *ctx, const float *x, size_t n, float range_min, float range_max,
+                                    size_t num_bins, uint64_t *counts);
+
 /* Device pointers of one block of the projection stack: every Linear is
  * per-output-channel int8 ([out,in] weights, [out] scales, [out] fp32 bias). */
 typedef struct hipq_block_weights {

@@ -60,6 +60,35 @@ def _declare(l: C.CDLL) -> None:
     l.tq_quint8_quantize.restype = C.c_uint8
     for name in ("tq_nn_quantize_value_symmetric", "tq_nn_quantize_value_asymmetric", "tq_backend_quantize_value"):
         getattr(l, name).restype = C.c_int32
+    l.tq_observer_new.restype = C.c_void_p
+    l.tq_observer_new.argtypes = [C.c_int, C.c_size_t, C.c_float]
+    for name in ("tq_observer_free", "tq_observer_reset"):
+        getattr(l, name).restype = None
+        getattr(l, name).argtypes = [C.c_void_p]
+    l.tq_observer_update.argtypes = [C.c_void_p, _f32p, C.c_size_t]
+    l.tq_observer_calculate_qparams.argtypes = [C.c_void_p, C.c_int, _f32p, _i32p]
+    for name in ("tq_observer_get_min_max", "tq_observer_get_avg", "tq_observer_get_hist_range",
+                 "tq_observer_histogram_range", "tq_observer_percentile_range"):
+        getattr(l, name).restype = None
+        getattr(l, name).argtypes = [C.c_void_p, _f32p, _f32p]
+    for name in ("tq_observer_num_batches", "tq_observer_num_bins", "tq_observer_num_values"):
+        getattr(l, name).restype = C.c_size_t
+        getattr(l, name).argtypes = [C.c_void_p]
+    l.tq_observer_histogram.restype = C.POINTER(C.c_uint64)
+    l.tq_observer_histogram.argtypes = [C.c_void_p]
+    l.tq_observer_values.restype = _f32p
+    l.tq_observer_values.argtypes = [C.c_void_p]
+    l.tq_value_to_bin_index.restype = C.c_size_t
+    l.tq_value_to_bin_index.argtypes = [C.c_float, C.c_float, C.c_float, C.c_size_t]
+    l.tq_histogram_accumulate.restype = None
+    l.tq_histogram_accumulate.argtypes = [_f32p, C.c_size_t, C.c_float, C.c_float, C.c_size_t, C.POINTER(C.c_uint64)]
+    l.tq_model_calculate_quantization_params.restype = None
+    l.tq_model_calculate_quantization_params.argtypes = [C.c_float, C.c_float, C.c_int32, C.c_int32, _f32p, _i32p,
+                                                         _f32p, _f32p]
+    l.tq_model_fake_quantize.restype = None
+    l.tq_model_fake_quantize.argtypes = [_f32p, C.c_size_t, C.c_float, C.c_int32, C.c_int32, C.c_int32, _f32p]
+    l.tq_model_mse_error.restype = C.c_double
+    l.tq_model_mse_error.argtypes = [_f32p, _f32p, C.c_size_t]
 
 
 def _p(a: np.ndarray, ty):
@@ -399,3 +428,131 @@ def time_matmul_rows(a_bytes, b_kn_bytes, m_sample):
     acc = np.empty((m_sample, n), dtype=np.int32)
     return float(lib().tq_time_matmul_rows(_p(a, _u8p), _p(b, _u8p), C.c_size_t(m_sample), C.c_size_t(k),
                                            C.c_size_t(n), _p(acc, _i32p)))
+
+
+# ---- calibration observers, quality metrics, model-level fake quantization ----------------
+
+OBS_MINMAX, OBS_MOVING_AVERAGE, OBS_HISTOGRAM, OBS_PERCENTILE, OBS_KL_DIVERGENCE, OBS_ENTROPY = range(6)
+
+METRIC_FIELDS = ("mse", "psnr", "snr", "mae", "max_error", "zero_error_percentage", "cosine_similarity",
+                 "compression_ratio")
+
+
+class _Metrics(C.Structure):
+    _fields_ = [(name, C.c_float) for name in METRIC_FIELDS]
+
+
+def calculate_quantization_metrics(original, quantized, original_bits=32, quantized_bits=8) -> dict:
+    """calculate_quantization_metrics (metrics.rs:67-175): sequential f32 sums, f32 results."""
+    a, b = _f32(original).ravel(), _f32(quantized).ravel()
+    if a.size != b.size:
+        raise OracleError("calculate_quantization_metrics: shape mismatch")
+    m = _Metrics()
+    lib().tq_calculate_quantization_metrics(_p(a, _f32p), _p(b, _f32p), C.c_size_t(a.size), C.c_uint32(original_bits),
+                                            C.c_uint32(quantized_bits), C.byref(m))
+    return {name: np.float32(getattr(m, name)) for name in METRIC_FIELDS}
+
+
+def calculate_quantization_metrics_f64(original, quantized, original_bits=32, quantized_bits=8) -> dict:
+    """The same quantities with the sums carried in f64."""
+    a, b = _f32(original).ravel(), _f32(quantized).ravel()
+    out = (C.c_double * 8)()
+    lib().tq_calculate_quantization_metrics_f64(_p(a, _f32p), _p(b, _f32p), C.c_size_t(a.size),
+                                                C.c_uint32(original_bits), C.c_uint32(quantized_bits), out)
+    return {name: float(out[i]) for i, name in enumerate(METRIC_FIELDS)}
+
+
+class Observer:
+    """Observer (observers.rs:36-556) driven through the C restatement."""
+
+    def __init__(self, observer_type=OBS_MINMAX, num_bins=0, percentile=0.0):
+        self._l = lib()
+        self._h = self._l.tq_observer_new(int(observer_type), C.c_size_t(num_bins), C.c_float(percentile))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._l.tq_observer_free(self._h)
+            self._h = None
+
+    def update(self, x) -> None:
+        x = _f32(x).ravel()
+        _check(self._l.tq_observer_update(self._h, _p(x, _f32p), C.c_size_t(x.size)), "Observer::update")
+
+    def calculate_qparams(self, dtype=DTYPE_I8):
+        s, z = C.c_float(), C.c_int32()
+        _check(self._l.tq_observer_calculate_qparams(self._h, int(dtype), C.byref(s), C.byref(z)),
+               "Observer::calculate_qparams")
+        return np.float32(s.value), z.value
+
+    def reset(self) -> None:
+        self._l.tq_observer_reset(self._h)
+
+    def _pair(self, fn):
+        a, b = C.c_float(), C.c_float()
+        fn(self._h, C.byref(a), C.byref(b))
+        return np.float32(a.value), np.float32(b.value)
+
+    def get_min_max(self):
+        return self._pair(self._l.tq_observer_get_min_max)
+
+    def get_avg(self):
+        return self._pair(self._l.tq_observer_get_avg)
+
+    def get_hist_range(self):
+        return self._pair(self._l.tq_observer_get_hist_range)
+
+    def histogram_range(self):
+        return self._pair(self._l.tq_observer_histogram_range)
+
+    def percentile_range(self):
+        return self._pair(self._l.tq_observer_percentile_range)
+
+    def num_batches(self) -> int:
+        return int(self._l.tq_observer_num_batches(self._h))
+
+    def num_bins(self) -> int:
+        return int(self._l.tq_observer_num_bins(self._h))
+
+    def histogram(self) -> np.ndarray:
+        n = self.num_bins()
+        return np.ctypeslib.as_array(self._l.tq_observer_histogram(self._h), shape=(n,)).copy()
+
+    def values(self) -> np.ndarray:
+        n = int(self._l.tq_observer_num_values(self._h))
+        if n == 0:
+            return np.empty(0, dtype=np.float32)
+        return np.ctypeslib.as_array(self._l.tq_observer_values(self._h), shape=(n,)).copy()
+
+
+def value_to_bin_index(value, range_min, range_max, num_bins) -> int:
+    return int(lib().tq_value_to_bin_index(C.c_float(value), C.c_float(range_min), C.c_float(range_max),
+                                           C.c_size_t(num_bins)))
+
+
+def histogram_accumulate(x, range_min, range_max, num_bins, counts=None) -> np.ndarray:
+    x = _f32(x).ravel()
+    counts = np.zeros(num_bins, dtype=np.uint64) if counts is None else np.ascontiguousarray(counts, dtype=np.uint64)
+    lib().tq_histogram_accumulate(_p(x, _f32p), C.c_size_t(x.size), C.c_float(range_min), C.c_float(range_max),
+                                  C.c_size_t(num_bins), _p(counts, C.POINTER(C.c_uint64)))
+    return counts
+
+
+def model_calculate_quantization_params(min_val, max_val, qmin=-128, qmax=127):
+    """ModelQuantizer::calculate_quantization_params -> (scale, zero_point, adjusted_min, adjusted_max)."""
+    s, z, a, b = C.c_float(), C.c_int32(), C.c_float(), C.c_float()
+    lib().tq_model_calculate_quantization_params(C.c_float(min_val), C.c_float(max_val), qmin, qmax, C.byref(s),
+                                                 C.byref(z), C.byref(a), C.byref(b))
+    return np.float32(s.value), z.value, np.float32(a.value), np.float32(b.value)
+
+
+def model_fake_quantize(x, scale, zp, qmin=-128, qmax=127) -> np.ndarray:
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().tq_model_fake_quantize(_p(x, _f32p), C.c_size_t(x.size), C.c_float(scale), int(zp), qmin, qmax,
+                                 _p(out, _f32p))
+    return out
+
+
+def model_mse_error(original, quantized) -> float:
+    a, b = _f32(original).ravel(), _f32(quantized).ravel()
+    return float(lib().tq_model_mse_error(_p(a, _f32p), _p(b, _f32p), C.c_size_t(a.size)))

@@ -1,0 +1,92 @@
+/*
+ * CPU oracle, second part: calibration observers, quality metrics and the
+ * model-level fake quantization of ToRSh.  TEST INFRASTRUCTURE ONLY, like
+ * torsh_quant_oracle.h: a plain-C restatement of the reference's CPU formulas
+ * used as the checker by the parity tests.  Nothing in the shipped library
+ * links, loads or calls it.
+ *
+ * Every function names the reference lines it restates (paths relative to the
+ * reference root).
+ */
+#ifndef TORSH_CALIB_ORACLE_H
+#define TORSH_CALIB_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- quality metrics: crates/torsh-quantization/src/metrics.rs:30-175 ---- */
+typedef struct {
+    float mse, psnr, snr, mae, max_error, zero_error_percentage, cosine_similarity, compression_ratio;
+} tq_metrics;
+
+/* calculate_quantization_metrics, metrics.rs:67-175: sequential f32 sums in element order. */
+int tq_calculate_quantization_metrics(const float *original, const float *quantized, size_t n,
+                                      uint32_t original_bits, uint32_t quantized_bits, tq_metrics *out);
+/* The same eight quantities with every sum carried in f64 (elementwise terms still f32, as
+ * in the reference): the value the f32 formulas approach without the rounding a long
+ * sequential f32 sum accumulates.  Used to separate kernel error from that rounding. */
+int tq_calculate_quantization_metrics_f64(const float *original, const float *quantized, size_t n,
+                                          uint32_t original_bits, uint32_t quantized_bits, double out[8]);
+
+/* ---- observers: crates/torsh-quantization/src/observers.rs -------------- */
+/* ObserverType, crates/torsh-quantization/src/config.rs:78-91 */
+enum {
+    TQ_OBS_MINMAX = 0,
+    TQ_OBS_MOVING_AVERAGE = 1,
+    TQ_OBS_HISTOGRAM = 2,
+    TQ_OBS_PERCENTILE = 3,
+    TQ_OBS_KL_DIVERGENCE = 4,
+    TQ_OBS_ENTROPY = 5
+};
+
+typedef struct tq_observer tq_observer;
+
+/* Observer::new / new_histogram / new_percentile, observers.rs:57-109.  num_bins 0 -> 256,
+ * percentile <= 0 -> 99.99 (the defaults of Observer::new). */
+tq_observer *tq_observer_new(int observer_type, size_t num_bins, float percentile);
+void tq_observer_free(tq_observer *o);
+/* Observer::update, observers.rs:112-260. */
+int tq_observer_update(tq_observer *o, const float *x, size_t n);
+/* Observer::calculate_qparams, observers.rs:263-310 (dtype: TQ_DTYPE_I8 = 0, TQ_DTYPE_U8 = 1). */
+int tq_observer_calculate_qparams(const tq_observer *o, int dtype, float *scale, int32_t *zp);
+/* Observer::reset, observers.rs:522-532. */
+void tq_observer_reset(tq_observer *o);
+/* State readers (get_min_max, num_batches, the histogram, the retained values). */
+void tq_observer_get_min_max(const tq_observer *o, float *mn, float *mx);
+void tq_observer_get_avg(const tq_observer *o, float *avg_min, float *avg_max);
+void tq_observer_get_hist_range(const tq_observer *o, float *hist_min, float *hist_max);
+size_t tq_observer_num_batches(const tq_observer *o);
+size_t tq_observer_num_bins(const tq_observer *o);
+const uint64_t *tq_observer_histogram(const tq_observer *o);
+size_t tq_observer_num_values(const tq_observer *o);
+const float *tq_observer_values(const tq_observer *o);
+/* calculate_histogram_range / calculate_percentile_range, observers.rs:336-423. */
+void tq_observer_histogram_range(const tq_observer *o, float *mn, float *mx);
+void tq_observer_percentile_range(const tq_observer *o, float *mn, float *mx);
+
+/* value_to_bin_index, observers.rs:313-333, as a free function of the range. */
+size_t tq_value_to_bin_index(float value, float range_min, float range_max, size_t num_bins);
+/* Histogram of x over [range_min, range_max] added into counts[num_bins]. */
+void tq_histogram_accumulate(const float *x, size_t n, float range_min, float range_max, size_t num_bins,
+                             uint64_t *counts);
+
+/* ---- model-level quantizer: crates/torsh-models/src/quantization.rs ------ */
+/* ModelQuantizer::calculate_quantization_params, quantization.rs:365-392.
+ * Writes the adjusted range too (it is stored in QuantizationParams). */
+void tq_model_calculate_quantization_params(float min_val, float max_val, int32_t qmin, int32_t qmax, float *scale,
+                                            int32_t *zp, float *adj_min, float *adj_max);
+/* ModelQuantizer::quantize_tensor, quantization.rs:309-349: quantize_value then
+ * dequantize_value per element ("fake quantization"). */
+void tq_model_fake_quantize(const float *x, size_t n, float scale, int32_t zp, int32_t qmin, int32_t qmax,
+                            float *out);
+/* ModelQuantizer::calculate_mse_error, quantization.rs:548-566 (f32 sum, result widened). */
+double tq_model_mse_error(const float *original, const float *quantized, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -14,13 +14,18 @@
 #include <sstream>
 
 #include "torsh_hipq/backend.hpp"
+#include "torsh_hipq/calibration.hpp"
+#include "torsh_hipq/models.hpp"
 #include "torsh_hipq/nn.hpp"
 #include "torsh_hipq/quantization.hpp"
+#include "torsh_hipq/serialize.hpp"
+#include "torsh_calib_oracle.h"
 #include "torsh_quant_oracle.h"
 
 using namespace torsh;
 using namespace torsh::quantization;
 namespace bq = torsh::backend::quantization;
+namespace mq = torsh::models::quantization;
 
 namespace {
 
@@ -638,6 +643,392 @@ GPU_TEST(parity_quantized_conv2d_module) {
     for (size_t i = 0; i < want.size(); ++i) CHECK_EQ(y.as_slice()[i], float(int(want[i]) - zp_out) * s_out);
     CHECK(conv.forward(Tensor::from_data(std::vector<float>(6, 0.f), {2, 3}).unwrap()).is_err());
     CHECK(conv.forward(Tensor::from_data(std::vector<float>(2 * 3 * 4 * 4, 0.f), {2, 3, 4, 4}).unwrap()).is_err());
+}
+
+
+// ---- calibration, metrics, model quantizer, persistence ----------------------------------------
+
+bool close_rel(double a, double b, double rel, double abs_tol = 1e-9) {
+    if (std::isinf(a) || std::isinf(b)) return a == b;
+    return std::fabs(a - b) <= abs_tol + rel * std::fabs(b);
+}
+
+CPU_TEST(test_observer_creation_and_host_logic) {  // observers.rs:577-591, 654-662, 706-716
+    CHECK(Observer::min_max().observer_type() == ObserverType::MinMax);
+    Observer h = Observer::histogram_with_bins(128);
+    CHECK(h.observer_type() == ObserverType::Histogram);
+    CHECK_EQ(h.num_bins(), size_t(128));
+    Observer p = Observer::percentile_with_value(95.0f);
+    CHECK(p.observer_type() == ObserverType::Percentile);
+    CHECK_EQ(p.percentile_value(), 95.0f);
+    auto [cleaned, removed] = Observer::min_max().detect_outliers({1.f, 2.f, 3.f, 4.f, 5.f, 100.f}, 1.5f);
+    CHECK(removed > 0 && cleaned.size() < 6);
+    CHECK(std::find(cleaned.begin(), cleaned.end(), 100.0f) == cleaned.end());
+    CHECK(Observer::min_max().calculate_qparams(DType::F32).is_err());
+    // an empty batch is counted and touches nothing else (observers.rs:694-703)
+    Observer e = Observer::min_max();
+    CHECK(e.update(Tensor::from_data({}, {0}).unwrap()).is_ok());
+    CHECK_EQ(e.num_batches(), size_t(1));
+    CHECK(std::isinf(e.get_min_max().first) && e.get_min_max().first > 0);
+}
+
+CPU_TEST(test_config_json_round_trip) {  // utils.rs:322-347
+    QuantConfig c = QuantConfig::per_channel(1).with_reduce_range(ReduceRange::Reduce);
+    c.dtype = DType::U8;
+    c.observer_type = ObserverType::Histogram;
+    c.qint_min = -5;
+    c.eps = 1e-6f;
+    c.averaging_constant = 0.05f;
+    const std::string json = export_config_to_json(c).unwrap();
+    CHECK(json.find("\"scheme\": \"PerChannelAffine\"") != std::string::npos);
+    CHECK(json.find("\"qint_max\": null") != std::string::npos);
+    CHECK(json.find("\"ch_axis\": 1") != std::string::npos);
+    const QuantConfig d = import_config_from_json(json).unwrap();
+    CHECK(d.dtype == c.dtype && d.scheme == c.scheme && d.observer_type == c.observer_type);
+    CHECK(d.reduce_range == c.reduce_range && d.backend == c.backend && d.enable_fake_quant == c.enable_fake_quant);
+    CHECK(d.qint_min == c.qint_min && !d.qint_max && d.ch_axis == c.ch_axis && !d.group_size);
+    CHECK_EQ(d.eps, c.eps);
+    CHECK_EQ(d.averaging_constant, c.averaging_constant);
+    // compact single-line form, as serde_json::to_string writes it
+    const char *compact =
+        "{\"dtype\":\"I8\",\"scheme\":\"PerTensorSymmetric\",\"enable_fake_quant\":true,\"observer_type\":\"MinMax\","
+        "\"backend\":\"Native\",\"reduce_range\":\"None\",\"qint_min\":null,\"qint_max\":null,\"eps\":1e-8,"
+        "\"averaging_constant\":0.01,\"ch_axis\":null,\"group_size\":64}";
+    const QuantConfig g = import_config_from_json(compact).unwrap();
+    CHECK(g.scheme == QScheme::PerTensorSymmetric && g.enable_fake_quant && g.group_size == size_t(64));
+    CHECK(import_config_from_json("{\"dtype\":\"I8\"}").is_err());          // missing fields
+    CHECK(import_config_from_json("not json").is_err());
+    CHECK(import_config_from_json(std::string(compact).replace(10, 2, "Q9")).is_err());  // unknown variant
+}
+
+CPU_TEST(test_weight_file_round_trip_and_corruption) {
+    QuantizedWeights w;
+    w.kind = QuantizedWeights::Conv2d;
+    w.dims = {3, 2, 2, 2};
+    for (int i = 0; i < 24; ++i) w.weight.push_back(static_cast<int8_t>(i * 11 - 128));
+    w.scales = {0.5f, 0.25f, 1e-3f};
+    w.bias = {1.f, -2.f, 3.f};
+    const std::string path = "/tmp/torsh_hipq_weights_test.bin";
+    CHECK(save_quantized_weights(w, path).is_ok());
+    const QuantizedWeights r = load_quantized_weights(path).unwrap();
+    CHECK(r.kind == w.kind && r.dims == w.dims && r.weight == w.weight && r.scales == w.scales && r.bias == w.bias);
+    // flipped payload byte -> checksum error; truncated file -> length error; wrong sections -> validate error
+    std::vector<char> bytes;
+    {
+        std::ifstream f(path, std::ios::binary);
+        bytes.assign((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    }
+    CHECK(bytes.size() % 256 == 0 && bytes.size() >= 1024);
+    auto write = [&](const std::vector<char> &b) {
+        std::ofstream f(path, std::ios::binary | std::ios::trunc);
+        f.write(b.data(), static_cast<std::streamsize>(b.size()));
+    };
+    auto flipped = bytes;
+    flipped[256 + 5] ^= 1;
+    write(flipped);
+    CHECK(load_quantized_weights(path).is_err());
+    CHECK(load_quantized_weights(path).unwrap_err().message.find("checksum") != std::string::npos);
+    write(std::vector<char>(bytes.begin(), bytes.begin() + 512));
+    CHECK(load_quantized_weights(path).is_err());
+    write(std::vector<char>(300, 'x'));
+    CHECK(load_quantized_weights(path).is_err());
+    QuantizedWeights bad = w;
+    bad.scales.pop_back();
+    CHECK(save_quantized_weights(bad, path).is_err());
+    std::remove(path.c_str());
+    CHECK(load_quantized_weights(path).is_err());
+}
+
+CPU_TEST(test_model_quantizer_scalar_logic) {  // crates/torsh-models/src/quantization.rs:726-822
+    mq::ModelQuantizer quantizer{mq::QuantizationConfig{}};
+    const mq::QuantizationParams p = quantizer.calculate_quantization_params(-1.0f, 1.0f, mq::QuantizationDType::Int8);
+    CHECK(p.scale > 0.0f && p.zero_point >= -128 && p.zero_point <= 127);
+    CHECK(quantizer.get_quantization_range(mq::QuantizationDType::Int8) == std::make_pair(-128, 127));
+    CHECK(quantizer.get_quantization_range(mq::QuantizationDType::Uint8) == std::make_pair(0, 255));
+    std::mt19937 g(3);
+    std::uniform_real_distribution<float> d(-50.f, 50.f);
+    for (int i = 0; i < 2000; ++i) {
+        float a = d(g), b = i % 17 == 0 ? a : d(g);
+        if (a > b) std::swap(a, b);
+        const auto got = quantizer.calculate_quantization_params(a, b, i % 2 ? mq::QuantizationDType::Int8
+                                                                             : mq::QuantizationDType::Uint8);
+        float s, amin, amax;
+        int32_t z;
+        tq_model_calculate_quantization_params(a, b, i % 2 ? -128 : 0, i % 2 ? 127 : 255, &s, &z, &amin, &amax);
+        CHECK(got.scale == s && got.zero_point == z && got.min_val == amin && got.max_val == amax);
+    }
+    const auto [ratio, savings] = mq::quantization_utils::calculate_memory_savings(1000, 250);
+    CHECK_EQ(ratio, 4.0);
+    CHECK_EQ(savings, 75.0);
+    CHECK(mq::quantization_utils::estimate_inference_speedup(mq::QuantizationDType::Int8, "cpu") > 1.0);
+    CHECK(mq::quantization_utils::post_training_quantization_config(mq::QuantizationDType::Int8).strategy.kind ==
+          mq::QuantizationStrategyKind::PostTraining);
+    // layer filter by substring and by type (quantization.rs:411-457)
+    std::map<std::string, Tensor> params;
+    for (const char *n : {"encoder.fc1.weight", "encoder.conv.weight", "embed.weight", "attn.q.weight"})
+        params.emplace(n, Tensor::from_data({1.f}, {1}).unwrap());
+    mq::QuantizationConfig cfg;
+    cfg.layer_filter.kind = mq::LayerQuantizationFilter::Exclude;
+    cfg.layer_filter.names = {"embed"};
+    CHECK_EQ(mq::ModelQuantizer{cfg}.filter_parameters(params).size(), size_t(3));
+    cfg.layer_filter.kind = mq::LayerQuantizationFilter::LayerTypes;
+    cfg.layer_filter.types = {mq::QuantizableLayerType::Linear, mq::QuantizableLayerType::Attention};
+    const auto kept = mq::ModelQuantizer{cfg}.filter_parameters(params);
+    CHECK(kept.size() == 2 && kept.count("encoder.fc1.weight") && kept.count("attn.q.weight"));
+}
+
+GPU_TEST(test_calculate_quantization_metrics) {  // metrics.rs:588-621
+    const Tensor original = tensor_1d({1.0f, 2.0f, 3.0f, 4.0f}).unwrap();
+    const Tensor quantized = tensor_1d({1.1f, 2.1f, 2.9f, 3.9f}).unwrap();
+    const QuantizationMetrics m = calculate_quantization_metrics(original, quantized, 32, 8).unwrap();
+    CHECK(m.mse > 0.0f && m.mse < 1.0f && m.mae > 0.0f && m.mae < 1.0f && m.psnr > 0.0f && m.snr > 0.0f);
+    CHECK(m.max_error >= 0.0f && m.zero_error_percentage >= 0.0f && m.zero_error_percentage <= 100.0f);
+    CHECK(m.cosine_similarity > 0.8f);
+    CHECK_EQ(m.compression_ratio, 4.0f);
+    const QuantizationMetrics p = calculate_quantization_metrics(original, original, 32, 16).unwrap();
+    CHECK(p.mse == 0.0f && p.mae == 0.0f && p.max_error == 0.0f && p.zero_error_percentage == 100.0f);
+    CHECK(std::fabs(p.cosine_similarity - 1.0f) < 1e-6f && std::isinf(p.psnr) && std::isinf(p.snr));
+    CHECK_EQ(p.compression_ratio, 2.0f);
+    CHECK(calculate_quantization_metrics(original, tensor_1d({1.f, 2.f}).unwrap(), 32, 8).is_err());
+    const Tensor empty = Tensor::from_data({}, {0}).unwrap();
+    CHECK_EQ(calculate_quantization_metrics(empty, empty, 32, 8).unwrap().zero_error_percentage, 100.0f);
+}
+
+GPU_TEST(test_compare_quantization_configs) {  // metrics.rs:623-661
+    const Tensor tensor = tensor_1d({1.0f, 2.0f, 3.0f, 4.0f, 5.0f}).unwrap();
+    QuantConfig binary;
+    binary.scheme = QScheme::Binary;
+    const std::vector<QuantConfig> configs{QuantConfig::int8(), binary,
+                                           QuantConfig::int8().with_scheme(QScheme::PerTensorSymmetric)};
+    const auto results = compare_quantization_configs(tensor, configs).unwrap();
+    CHECK_EQ(results.size(), size_t(3));
+    for (size_t i = 1; i < results.size(); ++i) {
+        const float a = results[i - 1].metrics.psnr, b = results[i].metrics.psnr;
+        if (std::isfinite(a) && std::isfinite(b)) CHECK(a >= b);
+    }
+    // the scheme outside the int8 path is reported with the worst-case record and sorts last
+    CHECK(results.back().config.scheme == QScheme::Binary && std::isinf(results.back().metrics.mse));
+    for (const auto &r : results)
+        if (std::isfinite(r.metrics.psnr)) CHECK(r.metrics.psnr > 0.0f && r.metrics.compression_ratio >= 1.0f);
+}
+
+GPU_TEST(parity_metrics_and_compare_configs) {
+    const std::vector<float> x = normal(200003, 31, 1.7f);
+    const Tensor tx = tensor_1d(x).unwrap();
+    for (QScheme scheme : {QScheme::PerTensorAffine, QScheme::PerTensorSymmetric}) {
+        const QuantConfig cfg = QuantConfig::int8().with_scheme(scheme);
+        const auto res = compare_quantization_configs(tx, {cfg}).unwrap();
+        // oracle: quantize_tensor_auto -> dequantize -> metrics
+        std::vector<float> q(x.size()), y(x.size());
+        float s;
+        int32_t z;
+        CHECK_EQ(tq_quantize_tensor_auto(x.data(), x.size(), TQ_DTYPE_I8,
+                                         scheme == QScheme::PerTensorAffine ? TQ_PER_TENSOR_AFFINE : TQ_PER_TENSOR_SYMMETRIC,
+                                         q.data(), &s, &z), 0);
+        CHECK_EQ(tq_dequantize_per_tensor_affine(q.data(), q.size(), s, z, y.data()), 0);
+        double want[8];
+        tq_calculate_quantization_metrics_f64(x.data(), y.data(), x.size(), 32, 8, want);
+        const QuantizationMetrics &m = res[0].metrics;
+        CHECK(close_rel(m.mse, want[0], 1e-6) && close_rel(m.psnr, want[1], 1e-6) && close_rel(m.snr, want[2], 1e-6));
+        CHECK(close_rel(m.mae, want[3], 1e-6) && m.max_error == static_cast<float>(want[4]));
+        CHECK(m.zero_error_percentage == static_cast<float>(want[5]) && close_rel(m.cosine_similarity, want[6], 1e-6));
+        // and the two-tensor form on the materialised image
+        const QuantizationMetrics two = calculate_quantization_metrics(tx, tensor_1d(y).unwrap(), 32, 8).unwrap();
+        CHECK(close_rel(two.mse, m.mse, 1e-6) && two.max_error == m.max_error);
+    }
+}
+
+GPU_TEST(test_observers) {  // observers.rs:594-651, 665-703
+    Observer mm = Observer::min_max();
+    CHECK(mm.update(tensor_1d({1.0f, 2.0f, 3.0f, 4.0f}).unwrap()).is_ok());
+    CHECK(mm.get_min_max() == std::make_pair(1.0f, 4.0f));
+    CHECK(mm.update(tensor_1d({0.5f, 5.0f}).unwrap()).is_ok());
+    CHECK(mm.get_min_max() == std::make_pair(0.5f, 5.0f));
+    Observer h = Observer::histogram_with_bins(10);
+    CHECK(h.update(tensor_1d({1.0f, 2.0f, 3.0f, 4.0f, 5.0f}).unwrap()).is_ok());
+    auto stats = h.get_statistics();
+    CHECK_EQ(stats.at("total_samples"), 5.0f);
+    CHECK_EQ(stats.at("num_bins"), 10.0f);
+    Observer p = Observer::percentile_with_value(90.0f);
+    std::vector<float> ramp(100);
+    for (int i = 0; i < 100; ++i) ramp[i] = static_cast<float>(i);
+    CHECK(p.update(tensor_1d(ramp).unwrap()).is_ok());
+    CHECK_EQ(p.get_statistics().at("total_values"), 100.0f);
+    CHECK_EQ(p.get_statistics().at("percentile"), 90.0f);
+    Observer q = Observer::min_max();
+    CHECK(q.update(tensor_1d({-2.0f, -1.0f, 0.0f, 1.0f, 2.0f}).unwrap()).is_ok());
+    const auto qp = q.calculate_qparams(DType::I8).unwrap();
+    CHECK(qp.first > 0.0f && qp.second >= -128 && qp.second <= 127);
+    Observer r = Observer::min_max();
+    CHECK(r.update(tensor_1d({1.0f, 2.0f, 3.0f}).unwrap()).is_ok());
+    CHECK_EQ(r.num_batches(), size_t(1));
+    r.reset();
+    CHECK_EQ(r.num_batches(), size_t(0));
+    CHECK(std::isinf(r.get_min_max().first) && r.get_min_max().first > 0 && r.get_min_max().second < 0);
+    Observer bad = Observer::min_max();
+    auto err = bad.update(tensor_1d({NAN, 1.0f, 2.0f}).unwrap());
+    CHECK(err.is_err() && err.unwrap_err().kind == TorshError::InvalidArgument);
+    CHECK_EQ(bad.num_batches(), size_t(1));
+}
+
+GPU_TEST(parity_observers_against_the_oracle) {
+    struct Kind {
+        ObserverType type;
+        int tq;
+    };
+    for (Kind k : {Kind{ObserverType::MinMax, TQ_OBS_MINMAX}, Kind{ObserverType::MovingAverage, TQ_OBS_MOVING_AVERAGE},
+                   Kind{ObserverType::Histogram, TQ_OBS_HISTOGRAM}, Kind{ObserverType::Percentile, TQ_OBS_PERCENTILE}}) {
+        Observer ob(k.type);
+        tq_observer *ref = tq_observer_new(k.tq, 0, 0.0f);
+        for (unsigned b = 0; b < 4; ++b) {
+            const std::vector<float> x = normal(60000 + 1111 * b, 900 + b, 0.5f + b);
+            CHECK(ob.update(tensor_1d(x).unwrap()).is_ok());
+            CHECK_EQ(tq_observer_update(ref, x.data(), x.size()), 0);
+            float mn, mx;
+            tq_observer_get_min_max(ref, &mn, &mx);
+            CHECK(ob.get_min_max() == std::make_pair(mn, mx));
+            for (DType dt : {DType::I8, DType::U8}) {
+                float s;
+                int32_t z;
+                CHECK_EQ(tq_observer_calculate_qparams(ref, dt == DType::I8 ? 0 : 1, &s, &z), 0);
+                const auto got = ob.calculate_qparams(dt).unwrap();
+                CHECK(got.first == s && got.second == z);
+            }
+        }
+        float a, b;
+        tq_observer_get_avg(ref, &a, &b);
+        CHECK(ob.get_moving_average() == std::make_pair(a, b));
+        tq_observer_get_hist_range(ref, &a, &b);
+        CHECK(ob.get_histogram_bounds() == std::make_pair(a, b));
+        if (k.type == ObserverType::Histogram) {
+            const uint64_t *h = tq_observer_histogram(ref);
+            check_same(ob.histogram_counts(), std::vector<uint64_t>(h, h + 256), __LINE__);
+            tq_observer_histogram_range(ref, &a, &b);
+            CHECK(ob.calculate_histogram_range() == std::make_pair(a, b));
+        }
+        if (k.type == ObserverType::Percentile) {
+            const float *v = tq_observer_values(ref);
+            check_same(ob.values(), std::vector<float>(v, v + tq_observer_num_values(ref)), __LINE__);
+            CHECK(ob.values().size() < 60000u * 4 + 7000);  // sampling kicked in above 100k values
+            tq_observer_percentile_range(ref, &a, &b);
+            CHECK(ob.calculate_percentile_range() == std::make_pair(a, b));
+        }
+        tq_observer_free(ref);
+    }
+}
+
+GPU_TEST(parity_quantize_batch_consistent) {  // utils.rs:153-180
+    const std::vector<float> a = normal(5000, 41, 1.0f), b = normal(300, 42, 3.0f), c = normal(70, 43, 0.2f);
+    const Tensor ta = tensor_1d(a).unwrap(), tb = tensor_1d(b).unwrap(), tc = tensor_1d(c).unwrap();
+    const auto res = quantize_batch_consistent({&ta, &tb, &tc}, QuantConfig::int8()).unwrap();
+    CHECK_EQ(res.size(), size_t(3));
+    tq_observer *ref = tq_observer_new(TQ_OBS_MINMAX, 0, 0.0f);
+    for (const auto *v : {&a, &b, &c}) tq_observer_update(ref, v->data(), v->size());
+    float s;
+    int32_t z;
+    tq_observer_calculate_qparams(ref, 0, &s, &z);
+    tq_observer_free(ref);
+    const std::vector<float> *inputs[3] = {&a, &b, &c};
+    for (int i = 0; i < 3; ++i) {
+        CHECK(std::get<1>(res[i]) == s && std::get<2>(res[i]) == z);
+        std::vector<float> want(inputs[i]->size());
+        CHECK_EQ(tq_quantize_per_tensor_affine(inputs[i]->data(), want.size(), s, z, want.data()), 0);
+        check_same(std::get<0>(res[i]).as_slice(), want, __LINE__);
+    }
+    CHECK(quantize_batch_consistent({}, QuantConfig::int8()).unwrap().empty());
+}
+
+GPU_TEST(parity_model_quantizer) {  // crates/torsh-models/src/quantization.rs:260-332, 491-566
+    std::map<std::string, Tensor> params;
+    params.emplace("block.fc1.weight", Tensor::from_data(normal(64 * 48, 51, 0.05f), {64, 48}).unwrap());
+    params.emplace("block.fc1.bias", Tensor::from_data(normal(64, 52, 0.01f), {64}).unwrap());
+    params.emplace("block.conv.weight", Tensor::from_data(normal(8 * 4 * 3 * 3, 53, 0.2f), {8, 4, 3, 3}).unwrap());
+    params.emplace("norm.gamma", Tensor::from_data(std::vector<float>(48, 1.0f), {48}).unwrap());  // constant tensor
+    for (mq::QuantizationDType dt : {mq::QuantizationDType::Int8, mq::QuantizationDType::Uint8}) {
+        mq::QuantizationConfig cfg = mq::quantization_utils::post_training_quantization_config(dt);
+        mq::ModelQuantizer quantizer{cfg};
+        const mq::QuantizationStats stats = quantizer.quantize_parameters(params).unwrap();
+        size_t total = 0;
+        for (const auto &[name, t] : params) total += t.numel();
+        CHECK_EQ(stats.original_size, total * 4);
+        CHECK_EQ(stats.quantized_size, total);
+        CHECK_EQ(stats.compression_ratio, 4.0);
+        CHECK_EQ(stats.theoretical_speedup, 2.0);
+        const int32_t qmin = dt == mq::QuantizationDType::Int8 ? -128 : 0, qmax = qmin + 255;
+        for (const auto &[name, t] : params) {
+            const std::vector<float> &x = t.as_slice();
+            float mn, mx, s, amin, amax;
+            int32_t z;
+            tq_min_max_fold(x.data(), x.size(), &mn, &mx);
+            tq_model_calculate_quantization_params(mn, mx, qmin, qmax, &s, &z, &amin, &amax);
+            const mq::QuantizationParams &p = quantizer.quantization_params().at(name);
+            CHECK(p.scale == s && p.zero_point == z && p.min_val == amin && p.max_val == amax);
+            std::vector<float> want(x.size());
+            tq_model_fake_quantize(x.data(), x.size(), s, z, qmin, qmax, want.data());
+            check_same(quantizer.quantize_tensor(t, p).unwrap().as_slice(), want, __LINE__);
+            CHECK(close_rel(stats.layer_stats.at(name).quantization_error, tq_model_mse_error(x.data(), want.data(), x.size()), 1e-5, 1e-12));
+            CHECK_EQ(stats.layer_stats.at(name).original_params, x.size());
+            CHECK_EQ(int(stats.layer_stats.at(name).bits_per_param), 8);
+        }
+        // parameters survive a save / load through JSON bit for bit
+        const std::string path = "/tmp/torsh_hipq_qparams_test.json";
+        CHECK(quantizer.save_quantization_params(path).is_ok());
+        mq::ModelQuantizer other{cfg};
+        CHECK(other.load_quantization_params(path).is_ok());
+        CHECK_EQ(other.quantization_params().size(), params.size());
+        for (const auto &[name, p] : quantizer.quantization_params()) {
+            const mq::QuantizationParams &o = other.quantization_params().at(name);
+            CHECK(o.scale == p.scale && o.zero_point == p.zero_point && o.min_val == p.min_val &&
+                  o.max_val == p.max_val && o.dtype == p.dtype);
+        }
+        std::remove(path.c_str());
+    }
+    // the layer filter restricts calibration, not the size statistics
+    mq::QuantizationConfig cfg;
+    cfg.layer_filter.kind = mq::LayerQuantizationFilter::Include;
+    cfg.layer_filter.names = {"fc1"};
+    mq::ModelQuantizer filtered{cfg};
+    const auto st = filtered.quantize_parameters(params).unwrap();
+    CHECK_EQ(filtered.quantization_params().size(), size_t(2));
+    CHECK_EQ(st.layer_stats.size(), size_t(4));
+    CHECK_EQ(st.layer_stats.at("norm.gamma").quantization_error, 0.0);
+    mq::MinMaxObserver obs;  // quantization.rs:756-768
+    CHECK(obs.observe(Tensor::from_data({1.f, 2.f, 3.f}, {3}).unwrap()).is_ok());
+    CHECK(obs.observe(Tensor::from_data({-1.f, 0.f, 4.f}, {3}).unwrap()).is_ok());
+    CHECK(obs.get_min_max() == std::make_pair(-1.0f, 4.0f));
+}
+
+GPU_TEST(test_quantized_modules_survive_a_weight_file) {
+    const size_t n = 96, k = 256, m = 7;
+    const Tensor w = Tensor::from_data(normal(n * k, 61, 0.03f), {n, k}).unwrap();
+    const Tensor b = Tensor::from_data(normal(n, 62, 0.01f), {n}).unwrap();
+    const Tensor x = Tensor::from_data(normal(m * k, 63), {m, k}).unwrap();
+    auto lin = nn::QuantizedLinear::from_weight_nk(w, &b, nn::ActivationQuant::PerToken).unwrap();
+    const std::string path = "/tmp/torsh_hipq_linear_test.bin";
+    CHECK(lin.save(path).is_ok());
+    auto back = nn::QuantizedLinear::load(path, nn::ActivationQuant::PerToken).unwrap();
+    CHECK(back.in_features() == k && back.out_features() == n);
+    check_same(back.forward(x).unwrap().as_slice(), lin.forward(x).unwrap().as_slice(), __LINE__);
+    // the file holds exactly what quantize_per_channel_auto produces on axis 0
+    const QuantizedWeights file = load_quantized_weights(path).unwrap();
+    std::vector<float> carrier(n * k), scales(n);
+    std::vector<int32_t> zps(n);
+    const size_t shape[2] = {n, k};
+    CHECK_EQ(tq_quantize_per_channel_auto(w.as_slice().data(), shape, 2, 0, TQ_DTYPE_I8, TQ_PER_CHANNEL_SYMMETRIC,
+                                          carrier.data(), scales.data(), zps.data()), 0);
+    check_same(file.scales, scales, __LINE__);
+    for (size_t i = 0; i < n * k; ++i) CHECK(static_cast<float>(file.weight[i]) == carrier[i]);
+    check_same(file.bias, b.as_slice(), __LINE__);
+    std::remove(path.c_str());
+    // conv: same round trip
+    const Tensor cw = Tensor::from_data(normal(8 * 4 * 3 * 3, 64, 0.1f), {8, 4, 3, 3}).unwrap();
+    const Tensor cx = Tensor::from_data(normal(2 * 4 * 6 * 6, 65, 1.0f, true), {2, 4, 6, 6}).unwrap();
+    auto conv = nn::QuantizedConv2d::from_weight(cw, nullptr, {1, 1}, {1, 1}, 0.05f, 3).unwrap();
+    CHECK(conv.save(path).is_ok());
+    auto conv2 = nn::QuantizedConv2d::from_quantized(load_quantized_weights(path).unwrap(), {1, 1}, {1, 1}, 0.05f, 3).unwrap();
+    check_same(conv2.forward_quantized(cx).unwrap().as_slice(), conv.forward_quantized(cx).unwrap().as_slice(), __LINE__);
+    CHECK(nn::QuantizedLinear::load(path).is_err());  // a conv file is not a linear layer
+    std::remove(path.c_str());
 }
 
 }  // namespace

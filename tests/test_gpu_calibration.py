@@ -1,0 +1,268 @@
+"""Parity of the calibration / metrics kernels (through the C-ABI) with the CPU oracle.
+
+Integer results (histogram counts, non-finite counts, zero-error counts) and order-independent
+float results (min, max, max error, the fake-quantized image) are bit-exact.  Sums are compared
+with a stated tolerance: the reference adds f32 terms in element order, the kernels carry f64, so
+against the oracle's f64-sum variant the tolerance is 1e-6 relative, and against the faithful f32
+sequential sums it is 1e-5 on inputs short enough (<= 4096 elements) that the sequential f32 sum
+itself is that accurate.
+"""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXACT_FIELDS = ("max_error", "zero_error_percentage", "compression_ratio")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def normal(seed, shape, std=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * std).astype(np.float32)
+
+
+@pytest.fixture(scope="module")
+def cal():
+    with open(os.path.join(ROOT, "tests", "golden", "calibration_vectors.json")) as f:
+        return json.load(f)
+
+
+def check_metrics(got, want32, want64, rel32=None):
+    for k in EXACT_FIELDS:
+        assert np.float32(got[k]) == np.float32(want64[k]), (k, got[k], want64[k])
+    for k in ("mse", "psnr", "snr", "mae", "cosine_similarity"):
+        g, w = float(got[k]), float(want64[k])
+        if math.isinf(w):
+            assert g == w, (k, g, w)
+        else:
+            assert g == pytest.approx(w, rel=1e-6, abs=1e-7), (k, g, w)
+        if rel32 is not None and not math.isinf(float(want32[k])):
+            assert g == pytest.approx(float(want32[k]), rel=rel32, abs=1e-7), (k, g, want32[k])
+
+
+def test_metrics_golden_vectors(ctx, oracle, cal):
+    for case in cal["metrics"]:
+        a, b = np.float32(case["original"]), np.float32(case["quantized"])
+        got = ctx.read_metrics(ctx.quantization_metrics(dev(a), dev(b), case["original_bits"], case["quantized_bits"]))
+        want32 = oracle.calculate_quantization_metrics(a, b, case["original_bits"], case["quantized_bits"])
+        want64 = oracle.calculate_quantization_metrics_f64(a, b, case["original_bits"], case["quantized_bits"])
+        check_metrics(got, want32, want64, rel32=1e-5)
+        assert got["compression_ratio"] == case["assert"]["compression_ratio"]
+    empty = torch.empty(0, dtype=torch.float32, device="cuda")
+    got = ctx.read_metrics(ctx.quantization_metrics(empty, empty))
+    assert got == dict(mse=0, psnr=0, snr=0, mae=0, max_error=0, zero_error_percentage=100, cosine_similarity=1,
+                       compression_ratio=1)
+
+
+@pytest.mark.parametrize("n", [1, 3, 64, 1000, 4096, 4099, 65536 + 7, 1 << 20])
+def test_metrics_two_tensors(ctx, oracle, n):
+    a = normal(n, n)
+    b = (a + normal(n + 1, n, 0.02)).astype(np.float32)
+    b[:: 7] = a[:: 7]                                  # some exact matches
+    got = ctx.read_metrics(ctx.quantization_metrics(dev(a), dev(b), 32, 8))
+    check_metrics(got, oracle.calculate_quantization_metrics(a, b), oracle.calculate_quantization_metrics_f64(a, b),
+                  rel32=1e-5 if n <= 4096 else None)
+
+
+def test_metrics_unaligned_views(ctx, oracle):
+    a = normal(21, 10000)
+    b = (a * np.float32(1.01)).astype(np.float32)
+    da, db = dev(a), dev(b)
+    for off in (1, 2, 3):
+        got = ctx.read_metrics(ctx.quantization_metrics(da[off:], db[off:]))
+        check_metrics(got, None, oracle.calculate_quantization_metrics_f64(a[off:], b[off:]))
+
+
+def test_metrics_closed_forms_on_device(ctx):
+    n = 1 << 16
+    got = ctx.read_metrics(ctx.quantization_metrics(dev(np.full(n, 4.0, np.float32)), dev(np.full(n, 4.5, np.float32)), 32, 4))
+    assert got["mse"] == 0.25 and got["mae"] == 0.5 and got["max_error"] == 0.5 and got["zero_error_percentage"] == 0
+    assert got["psnr"] == pytest.approx(20 * math.log10(8.0), rel=1e-6)
+    assert got["snr"] == pytest.approx(10 * math.log10(64.0), rel=1e-6)
+    assert got["cosine_similarity"] == pytest.approx(1.0, abs=1e-6) and got["compression_ratio"] == 8.0
+    got = ctx.read_metrics(ctx.quantization_metrics(dev(np.float32([2.0, 0.0])), dev(np.float32([0.0, 4.0]))))
+    assert got["mse"] == 10.0 and got["mae"] == 3.0 and got["cosine_similarity"] == 0.0
+    assert got["psnr"] == pytest.approx(20 * math.log10(2.0 / math.sqrt(10.0)), rel=1e-6)
+    assert got["snr"] == pytest.approx(10 * math.log10(0.2), rel=1e-6)
+
+
+@pytest.mark.parametrize("form", ["mul_inv", "div"])
+@pytest.mark.parametrize("n", [5, 4096, 100003, 1 << 20])
+def test_fused_fake_quantize_metrics_equal_the_three_step_path(ctx, hipq, oracle, n, form):
+    # compare_quantization_configs: quantize (x * 1/scale form for len > 64) -> dequantize -> metrics.
+    x = normal(100 + n, n, 2.0)
+    mn, mx = oracle.find_min_max(x)
+    scale, zp = oracle.calculate_affine_params(mn, mx, oracle.DTYPE_I8)
+    mode = hipq.FORM_DIV if form == "div" else hipq.FORM_MUL_INV
+    if form == "div":
+        y = oracle.model_fake_quantize(x, scale, zp)
+    else:
+        y = oracle.dequantize_per_tensor_affine(oracle.quantize_per_tensor_affine_simd(x, scale, zp), scale, zp)
+    got = ctx.read_metrics(ctx.fake_quantize_metrics(dev(x), scale, zp, -128, 127, mode))
+    check_metrics(got, oracle.calculate_quantization_metrics(x, y), oracle.calculate_quantization_metrics_f64(x, y),
+                  rel32=1e-5 if n <= 4096 else None)
+    # and the image itself, bit for bit
+    img = host(ctx.fake_quantize(dev(x), scale, zp, -128, 127, mode | (hipq.FAKE_INT_CAST if form == "div" else 0)))
+    np.testing.assert_array_equal(img, y)
+    # two-tensor kernel on the materialised image gives the same record as the fused kernel
+    two = ctx.read_metrics(ctx.quantization_metrics(dev(x), dev(y)))
+    for k in two:
+        assert two[k] == pytest.approx(got[k], rel=1e-6, abs=1e-9) or (math.isinf(two[k]) and two[k] == got[k])
+
+
+def test_fake_quantize_metrics_with_device_params(ctx, hipq, oracle):
+    x = normal(77, 50000)
+    q, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_AFFINE)
+    p = ctx.read_qparams(params)
+    got = ctx.read_metrics(ctx.fake_quantize_metrics(dev(x), 0.0, 0, -128, 127, 0, params=params))
+    want = ctx.read_metrics(ctx.fake_quantize_metrics(dev(x), p.scale, p.zero_point, -128, 127, 0))
+    assert got == want
+
+
+def test_fake_quantize_nan_semantics_and_errors(ctx, hipq, oracle):
+    x = np.float32([float("nan"), 1.2, float("inf"), -float("inf"), 1.25, -1.25])
+    want = oracle.model_fake_quantize(x, 0.5, 3)
+    got = host(ctx.fake_quantize(dev(x), 0.5, 3, -128, 127, hipq.FORM_DIV | hipq.FAKE_INT_CAST))
+    np.testing.assert_array_equal(got, want)
+    carrier = host(ctx.fake_quantize(dev(x), 0.5, 3, -128, 127, hipq.FORM_DIV))
+    assert np.isnan(carrier[0])
+    np.testing.assert_array_equal(carrier[1:], want[1:])
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.fake_quantize(dev(x), 0.0, 0)
+    assert e.value.code == hipq.INVALID_ARGUMENT and "Scale must be positive" in e.value.message
+    with pytest.raises(hipq.HipqError):
+        ctx.fake_quantize_metrics(dev(x), 1.0, 0, 5, -5)
+    with pytest.raises(hipq.HipqError):
+        ctx.fake_quantize(dev(x), 1.0, 0, mode=64)
+
+
+# ---- observers -------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 63, 4096, 4097, 1 << 20, (1 << 22) + 5])
+def test_observe_range_and_nonfinite_count(ctx, oracle, n):
+    x = normal(n + 9, n, 3.0)
+    st = ctx.read_observe(ctx.observe(dev(x)))
+    mn, mx = oracle.min_max_fold(x)
+    assert (st.min_val, st.max_val, st.nonfinite) == (mn, mx, 0)
+    if n >= 63:
+        x[5], x[n // 2], x[n - 1] = np.nan, np.inf, -np.inf
+        st = ctx.read_observe(ctx.observe(dev(x)))
+        assert st.nonfinite == 3
+
+
+def test_observe_empty(ctx):
+    st = ctx.read_observe(ctx.observe(torch.empty(0, dtype=torch.float32, device="cuda")))
+    assert st.min_val == float("inf") and st.max_val == -float("inf") and st.nonfinite == 0
+
+
+@pytest.mark.parametrize("bins", [1, 10, 256, 1000, 2048, 5000, 16384])
+def test_histogram_counts_are_exact(ctx, oracle, bins):
+    n = 300000
+    x = normal(bins, n, 1.5)
+    lo, hi = oracle.min_max_fold(x)
+    got = host(ctx.histogram(dev(x), lo, hi, bins)).astype(np.uint64)
+    want = oracle.histogram_accumulate(x, lo, hi, bins)
+    np.testing.assert_array_equal(got, want)
+    assert int(got.sum()) == n
+
+
+def test_histogram_edges_clamping_and_accumulation(ctx, oracle):
+    x = np.float32([-5.0, 0.0, 0.999, 1.0, 9.999, 10.0, 11.0, 1e30, float("nan"), float("inf"), -float("inf")])
+    counts = ctx.histogram(dev(x), 0.0, 10.0, 10)
+    want = oracle.histogram_accumulate(x, 0.0, 10.0, 10)
+    np.testing.assert_array_equal(host(counts).astype(np.uint64), want)
+    # second batch adds into the same counters; a narrower range than the data clamps to the end bins
+    y = normal(4, 70001, 4.0)
+    counts = ctx.histogram(dev(y), -1.0, 1.0, 10, counts=counts)
+    want = oracle.histogram_accumulate(y, -1.0, 1.0, 10, counts=want)
+    np.testing.assert_array_equal(host(counts).astype(np.uint64), want)
+    # degenerate ranges: everything in bin 0
+    for lo, hi in ((3.0, 3.0), (4.0, 3.0)):
+        got = host(ctx.histogram(dev(y), lo, hi, 16))
+        assert got[0] == y.size and got[1:].sum() == 0
+
+
+def test_histogram_awkward_ranges_bit_exact(ctx, oracle):
+    # Ranges whose width is not a power of two and values sitting on bin edges: the bin index depends on the
+    # correctly rounded quotient, so this fails if the division is replaced by a multiplication.
+    rng = np.random.default_rng(8)
+    for lo, hi, bins in ((-0.7, 2.9, 256), (1e-3, 3e-3, 100), (-1e6, 3.3e6, 777), (0.1, 0.7, 6)):
+        edges = (np.float32(lo) + (np.float32(hi) - np.float32(lo)) * (np.arange(bins + 1, dtype=np.float32) / np.float32(bins)))
+        x = np.concatenate([edges, np.nextafter(edges, np.float32(-np.inf)), np.nextafter(edges, np.float32(np.inf)),
+                            rng.uniform(lo, hi, 50000).astype(np.float32)]).astype(np.float32)
+        got = host(ctx.histogram(dev(x), lo, hi, bins)).astype(np.uint64)
+        np.testing.assert_array_equal(got, oracle.histogram_accumulate(x, lo, hi, bins), err_msg=str((lo, hi, bins)))
+
+
+def test_histogram_unaligned_and_errors(ctx, hipq, oracle):
+    x = normal(31, 100001)
+    dx = dev(x)
+    for off in (1, 2, 3):
+        got = host(ctx.histogram(dx[off:], -4.0, 4.0, 64)).astype(np.uint64)
+        np.testing.assert_array_equal(got, oracle.histogram_accumulate(x[off:], -4.0, 4.0, 64))
+    with pytest.raises(hipq.HipqError):
+        ctx.histogram(dx, 0.0, 1.0, 0, counts=torch.zeros(1, dtype=torch.int64, device="cuda"))
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.histogram(dx, 0.0, 1.0, hipq.HISTOGRAM_MAX_BINS + 1)
+    assert "exceeds" in e.value.message
+
+
+def test_histogram_observer_sequence_matches_the_oracle(ctx, oracle):
+    # The observer's own update order: range first (grown by the batch), then the batch is binned over it.
+    ob = oracle.Observer(oracle.OBS_HISTOGRAM)
+    counts = torch.zeros(256, dtype=torch.int64, device="cuda")
+    hmin, hmax = np.float32(np.inf), np.float32(-np.inf)
+    for i, std in enumerate((1.0, 0.5, 3.0, 2.0)):
+        x = normal(500 + i, 123457, std)
+        ob.update(x)
+        st = ctx.read_observe(ctx.observe(dev(x)))
+        assert st.nonfinite == 0
+        hmin, hmax = min(hmin, np.float32(st.min_val)), max(hmax, np.float32(st.max_val))
+        ctx.histogram(dev(x), hmin, hmax, 256, counts=counts)
+        np.testing.assert_array_equal(host(counts).astype(np.uint64), ob.histogram())
+    assert ob.get_hist_range() == (hmin, hmax)
+
+
+def test_full_size_properties(ctx, hipq, oracle):
+    # 4096 x 4096 (the streaming configuration): size-independent properties.
+    n = 4096 * 4096
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(n, dtype=torch.float32, device="cuda", generator=g)
+    mm = host(ctx.minmax(x))
+    st = ctx.read_observe(ctx.observe(x))
+    assert (st.min_val, st.max_val, st.nonfinite) == (mm[0], mm[1], 0)
+    counts = host(ctx.histogram(x, mm[0], mm[1], 256))
+    assert counts.sum() == n and counts.min() >= 0
+    # histogram of a concatenation = sum of histograms
+    c2 = ctx.histogram(x[: n // 2], mm[0], mm[1], 256)
+    c2 = host(ctx.histogram(x[n // 2:], mm[0], mm[1], 256, counts=c2))
+    np.testing.assert_array_equal(c2, counts)
+    # torch.histc bins by the same rule up to rounding of the quotient: totals per coarse region agree
+    absmax = max(abs(mm[0]), abs(mm[1]))
+    scale = float(np.float32(absmax) / np.float32(127.0))
+    fused = ctx.read_metrics(ctx.fake_quantize_metrics(x, scale, 0))
+    y = ctx.dequantize(ctx.quantize_per_tensor_i8(x, scale, 0), scale, 0)
+    two = ctx.read_metrics(ctx.quantization_metrics(x, y))
+    for k in fused:
+        assert fused[k] == pytest.approx(two[k], rel=1e-6), k
+    # uniform-quantizer noise model: mse ~ scale^2 / 12 for a fine grid, and SNR = 10 log10(var / mse)
+    assert fused["mse"] == pytest.approx(scale * scale / 12.0, rel=0.02)
+    assert fused["snr"] == pytest.approx(10 * math.log10(1.0 / fused["mse"]), abs=0.05)
+    assert fused["max_error"] <= scale / 2 * (1 + 1e-6)
+    # a tensor against itself
+    same = ctx.read_metrics(ctx.quantization_metrics(x, x))
+    assert same["mse"] == 0 and same["zero_error_percentage"] == 100 and math.isinf(same["psnr"])
+    assert same["cosine_similarity"] == pytest.approx(1.0, abs=1e-6)

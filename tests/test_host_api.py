@@ -20,6 +20,10 @@ CPU_CASES = [
     "test_error_cases_before_the_device",
     "test_backend_params_and_tensor",
     "test_module_shapes_before_the_device",
+    "test_observer_creation_and_host_logic",
+    "test_config_json_round_trip",
+    "test_weight_file_round_trip_and_corruption",
+    "test_model_quantizer_scalar_logic",
 ]
 GPU_CASES = [
     "test_quantize_per_tensor_affine",
@@ -36,6 +40,14 @@ GPU_CASES = [
     "parity_backend_qconv2d",
     "parity_quantized_linear_module",
     "parity_quantized_conv2d_module",
+    "test_calculate_quantization_metrics",
+    "test_compare_quantization_configs",
+    "parity_metrics_and_compare_configs",
+    "test_observers",
+    "parity_observers_against_the_oracle",
+    "parity_quantize_batch_consistent",
+    "parity_model_quantizer",
+    "test_quantized_modules_survive_a_weight_file",
 ]
 
 

@@ -21,6 +21,8 @@ ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
 FORM_MUL_INV, FORM_DIV = 0, 2
 DTYPE_I8, DTYPE_U8 = 0, 1
 PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC = range(4)
+FAKE_INT_CAST = 4
+HISTOGRAM_MAX_BINS = 16384
 
 
 class HipqError(RuntimeError):
@@ -40,6 +42,19 @@ class BlockWeights(C.Structure):
 class QParams(C.Structure):
     _fields_ = [("scale", C.c_float), ("zero_point", C.c_int32), ("min_val", C.c_float), ("max_val", C.c_float),
                 ("status", C.c_int32), ("reserved", C.c_int32 * 3)]
+
+
+class QuantMetrics(C.Structure):
+    """hipq_quant_metrics: the fields of the reference's QuantizationMetrics, in its order."""
+    _fields_ = [(n, C.c_float) for n in ("mse", "psnr", "snr", "mae", "max_error", "zero_error_percentage",
+                                         "cosine_similarity", "compression_ratio")]
+
+    def as_dict(self) -> dict:
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+class ObserveStats(C.Structure):
+    _fields_ = [("min_val", C.c_float), ("max_val", C.c_float), ("nonfinite", C.c_uint64)]
 
 
 _lib: Optional[C.CDLL] = None
@@ -86,6 +101,11 @@ _SIGNATURES = {
     "hipq_gelu_tanh_quantize_f32_i8": [_vp, _vp, _sz, _sz, _i32, _vp, _vp],
     "hipq_add_f32": [_vp, _vp, _vp, _sz, _vp],
     "hipq_transformer_stack_forward_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
+    "hipq_quantization_metrics_f32": [_vp, _vp, _vp, _sz, C.c_uint32, C.c_uint32, _vp],
+    "hipq_fake_quantize_metrics_f32": [_vp, _vp, _sz, _f32, _i32, _vp, _i32, _i32, _i32, C.c_uint32, C.c_uint32, _vp],
+    "hipq_fake_quantize_f32": [_vp, _vp, _sz, _f32, _i32, _vp, _i32, _i32, _i32, _vp],
+    "hipq_observe_f32": [_vp, _vp, _sz, _vp],
+    "hipq_histogram_f32": [_vp, _vp, _sz, _f32, _f32, _sz, _vp],
     "hipq_conv2d_u8i8_i32": [_vp, _vp, _i32, _vp] + [_sz] * 11 + [_vp],
     "hipq_conv2d_u8i8_i8": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_f32, _i32, _i32, _vp],
     "hipq_conv2d_u8i8_f32": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_vp],
@@ -210,6 +230,54 @@ class Context:
         out = self.new_qparams()
         self.call("hipq_qparams_from_minmax", _ptr(minmax), flavor, qmin, qmax, _ptr(out))
         return out
+
+    # ---- calibration observers and quality metrics --------------------------------
+    def _record(self, ty):
+        return torch.zeros(C.sizeof(ty), dtype=torch.uint8, device=self._dev())
+
+    @staticmethod
+    def _read(buf: torch.Tensor, ty):
+        return ty.from_buffer_copy(bytes(buf.cpu().numpy().tobytes()))
+
+    def quantization_metrics(self, original, quantized, original_bits=32, quantized_bits=8, out=None) -> torch.Tensor:
+        """Device record (QuantMetrics); read it with read_metrics()."""
+        out = out if out is not None else self._record(QuantMetrics)
+        self.call("hipq_quantization_metrics_f32", _ptr(original), _ptr(quantized), original.numel(), original_bits,
+                  quantized_bits, _ptr(out))
+        return out
+
+    def fake_quantize_metrics(self, x, scale, zp, qmin=-128, qmax=127, mode=0, params=None, original_bits=32,
+                              quantized_bits=8, out=None) -> torch.Tensor:
+        out = out if out is not None else self._record(QuantMetrics)
+        self.call("hipq_fake_quantize_metrics_f32", _ptr(x), x.numel(), float(scale), int(zp), _ptr(params), qmin,
+                  qmax, mode, original_bits, quantized_bits, _ptr(out))
+        return out
+
+    def read_metrics(self, buf: torch.Tensor) -> dict:
+        return self._read(buf, QuantMetrics).as_dict()
+
+    def fake_quantize(self, x, scale, zp, qmin=-128, qmax=127, mode=0, params=None, out=None) -> torch.Tensor:
+        out = out if out is not None else torch.empty(x.shape, dtype=torch.float32, device=self._dev())
+        self.call("hipq_fake_quantize_f32", _ptr(x), x.numel(), float(scale), int(zp), _ptr(params), qmin, qmax,
+                  mode, _ptr(out))
+        return out
+
+    def observe(self, x, out=None) -> torch.Tensor:
+        """Device record (ObserveStats): batch min, max and the number of non-finite values."""
+        out = out if out is not None else self._record(ObserveStats)
+        self.call("hipq_observe_f32", _ptr(x), x.numel(), _ptr(out))
+        return out
+
+    def read_observe(self, buf: torch.Tensor) -> ObserveStats:
+        return self._read(buf, ObserveStats)
+
+    def histogram(self, x, range_min, range_max, num_bins, counts=None) -> torch.Tensor:
+        """counts[num_bins] (int64 tensor holding the uint64 counters) += histogram of x."""
+        if counts is None:
+            counts = torch.zeros(num_bins, dtype=torch.int64, device=self._dev())
+        self.call("hipq_histogram_f32", _ptr(x), x.numel(), float(range_min), float(range_max), num_bins,
+                  _ptr(counts))
+        return counts
 
     def quantize_per_tensor_i8(self, x, scale, zp, mode=0, out=None):
         out = out if out is not None else torch.empty(x.shape, dtype=torch.int8, device=self._dev())

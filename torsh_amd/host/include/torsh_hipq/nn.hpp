@@ -19,6 +19,7 @@
 #include <map>
 
 #include "core.hpp"
+#include "serialize.hpp"
 
 namespace torsh {
 namespace nn {
@@ -134,6 +135,55 @@ class QuantizedLinear : public Module {
         return from_weight_nk(wnk, nullptr, act);
     }
 
+    // From prepared int8 weights (already quantized per output channel): one copy per section,
+    // no arithmetic.  The counterpart of to_quantized_weights() / save().
+    static Result<QuantizedLinear> from_quantized(const quantization::QuantizedWeights &w,
+                                                  ActivationQuant act = ActivationQuant::PerTensor) {
+        TORSH_CHECK(w.validate());
+        if (w.kind != quantization::QuantizedWeights::Linear)
+            return TorshError::invalid_argument("QuantizedLinear needs weights of kind Linear");
+        QuantizedLinear q;
+        q.out_ = w.dims[0];
+        q.in_ = w.dims[1];
+        q.act_ = act;
+        if (q.in_ == 0 || q.out_ == 0)
+            return TorshError::invalid_argument("QuantizedLinear weight must be a non-empty 2D tensor");
+        TORSH_TRY(ctx, hip::Runtime::ctx());
+        q.ctx_ = ctx;
+        TORSH_TRY(dw, hip::DeviceBuffer::from_host(ctx, w.weight.data(), w.weight.size()));
+        TORSH_TRY(ds, hip::DeviceBuffer::from_host(ctx, w.scales.data(), w.scales.size()));
+        q.w_ = std::move(dw);
+        q.sw_ = std::move(ds);
+        if (!w.bias.empty()) {
+            TORSH_TRY(db, hip::DeviceBuffer::from_host(ctx, w.bias.data(), w.bias.size()));
+            q.bias_ = std::move(db);
+            q.has_bias_ = true;
+        }
+        return std::move(q);
+    }
+    Result<quantization::QuantizedWeights> to_quantized_weights() const {
+        quantization::QuantizedWeights w;
+        w.kind = quantization::QuantizedWeights::Linear;
+        w.dims = {out_, in_};
+        TORSH_TRY(wq, w_.to_host<int8_t>(out_ * in_));
+        TORSH_TRY(sw, sw_.to_host<float>(out_));
+        w.weight = std::move(wq);
+        w.scales = std::move(sw);
+        if (has_bias_) {
+            TORSH_TRY(b, bias_.to_host<float>(out_));
+            w.bias = std::move(b);
+        }
+        return w;
+    }
+    Result<Unit> save(const std::string &path) const {
+        TORSH_TRY(w, to_quantized_weights());
+        return quantization::save_quantized_weights(w, path);
+    }
+    static Result<QuantizedLinear> load(const std::string &path, ActivationQuant act = ActivationQuant::PerTensor) {
+        TORSH_TRY(w, quantization::load_quantized_weights(path));
+        return from_quantized(w, act);
+    }
+
     // input [..., in_features] -> [..., out_features]
     Result<Tensor> forward(const Tensor &input) const override {
         const auto &d = input.shape().dims();
@@ -225,6 +275,54 @@ class QuantizedConv2d : public Module {
             q.has_bias_ = true;
         }
         return std::move(q);
+    }
+
+    // From prepared int8 weights; stride, padding and the output parameters are not part of the
+    // weight file (they belong to the layer's configuration).
+    static Result<QuantizedConv2d> from_quantized(const quantization::QuantizedWeights &w,
+                                                  std::pair<size_t, size_t> stride, std::pair<size_t, size_t> padding,
+                                                  float out_scale, int32_t out_zero_point) {
+        TORSH_CHECK(w.validate());
+        if (w.kind != quantization::QuantizedWeights::Conv2d)
+            return TorshError::invalid_argument("QuantizedConv2d needs weights of kind Conv2d");
+        if (!(out_scale > 0.0f)) return TorshError::invalid_argument("Scale must be positive");
+        if (out_zero_point < -128 || out_zero_point > 127)
+            return TorshError::invalid_argument("Zero point is outside valid range [-128, 127]");
+        if (stride.first == 0 || stride.second == 0) return TorshError::invalid_argument("stride must be positive");
+        QuantizedConv2d q;
+        q.oc_ = w.dims[0], q.ic_ = w.dims[1], q.kh_ = w.dims[2], q.kw_ = w.dims[3];
+        q.stride_ = stride, q.padding_ = padding;
+        q.s_out_ = out_scale, q.zp_out_ = out_zero_point;
+        TORSH_TRY(ctx, hip::Runtime::ctx());
+        q.ctx_ = ctx;
+        TORSH_TRY(dw, hip::DeviceBuffer::from_host(ctx, w.weight.data(), w.weight.size()));
+        TORSH_TRY(ds, hip::DeviceBuffer::from_host(ctx, w.scales.data(), w.scales.size()));
+        q.w_ = std::move(dw);
+        q.sw_ = std::move(ds);
+        if (!w.bias.empty()) {
+            TORSH_TRY(db, hip::DeviceBuffer::from_host(ctx, w.bias.data(), w.bias.size()));
+            q.bias_ = std::move(db);
+            q.has_bias_ = true;
+        }
+        return std::move(q);
+    }
+    Result<quantization::QuantizedWeights> to_quantized_weights() const {
+        quantization::QuantizedWeights w;
+        w.kind = quantization::QuantizedWeights::Conv2d;
+        w.dims = {oc_, ic_, kh_, kw_};
+        TORSH_TRY(wq, w_.to_host<int8_t>(oc_ * ic_ * kh_ * kw_));
+        TORSH_TRY(sw, sw_.to_host<float>(oc_));
+        w.weight = std::move(wq);
+        w.scales = std::move(sw);
+        if (has_bias_) {
+            TORSH_TRY(b, bias_.to_host<float>(oc_));
+            w.bias = std::move(b);
+        }
+        return w;
+    }
+    Result<Unit> save(const std::string &path) const {
+        TORSH_TRY(w, to_quantized_weights());
+        return quantization::save_quantized_weights(w, path);
     }
 
     // int8 NCHW output and the input parameters the activations were quantized with.
