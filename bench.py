@@ -121,6 +121,24 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
             ctx.quantize_per_tensor_i8(xs[i % 8], 0.04, 0, hipq.FORM_MUL_INV, out=qs[i % 8])
         for i in range(reps):
             ctx.dequantize(qs[i % 8], 0.04, 0, out=ys[i % 8])
+    elif which == "calib":
+        n = 4096 * 4096
+        xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
+        ys = [x + 0.01 * torch.randn(n, generator=g, device="cuda") for x in xs]
+        rec = ctx.quantization_metrics(xs[0], ys[0])
+        obs = ctx.observe(xs[0])
+        hist = torch.zeros(256, dtype=torch.int64, device="cuda")
+        torch.cuda.synchronize()
+        for i in range(reps):
+            ctx.quantization_metrics(xs[i % 8], ys[i % 8], out=rec)
+        for i in range(reps):
+            ctx.fake_quantize_metrics(xs[i % 8], 0.04, 0, out=rec)
+        for i in range(reps):
+            ctx.observe(xs[i % 8], out=obs)
+        for i in range(reps):
+            ctx.histogram(xs[i % 8], -6.0, 6.0, 256, counts=hist)
+        for i in range(reps):
+            ctx.fake_quantize(xs[i % 8], 0.04, 0, out=ys[i % 8])
     else:
         n = 4096 * 4096
         xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
@@ -139,7 +157,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "quantize", "copy"], default=None,
+    ap.add_argument("--profile", choices=["gemm", "quantize", "calib", "copy"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
