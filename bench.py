@@ -1,8 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-inference hot path on one MI355X.
 
-One "step" is one QuantizedLinear forward of the headline workload
-(BASELINE.json configs[1]): fp32 activations [512,4096] -> dynamic per-tensor
+One "step" is one QuantizedLinear forward of the headline workload:
+fp32 activations [512,4096] -> dynamic per-tensor
 int8 quantize (min/max, scale, quantize) -> int8 x int8 -> int32 MFMA GEMM
 against per-output-channel int8 weights [4096,4096] -> dequantize + bias epilogue
 -> fp32 [512,4096].  All inputs are resident in HBM before the timed region.

@@ -60,7 +60,7 @@ def _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, seed):
 
 @pytest.mark.parametrize("nb,c,h,w,oc,k,pad", [(2, 128, 14, 14, 64, 3, 1), (1, 256, 7, 7, 33, 3, 1), (3, 16, 10, 10, 8, 3, 1)])
 def test_quantized_conv2d_forward(ctx, hipq, oracle, nb, c, h, w, oc, k, pad):
-    """BASELINE config 4 at reduced size: asymmetric u8 activations, per-channel int8 filters, fused bias + requant."""
+    """The Conv2d configuration ([32,256,14,14], 3x3) at reduced size: asymmetric u8 activations, per-channel int8 filters, fused bias + requant."""
     x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out, out_f = _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, c + oc)
     # activations quantized on the device: min/max -> asymmetric params -> u8
     dq, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_BACKEND_ASYMMETRIC, hipq.DTYPE_U8, hipq.FORM_DIV)

@@ -176,7 +176,7 @@ def test_qparams_from_minmax(ctx, hipq, oracle, flavor_name):
 
 @pytest.mark.parametrize("shape", [(4, 4), (256, 256), (1000, 37), (1024, 1024)])
 def test_config1_round_trip(ctx, hipq, oracle, shape):
-    """Symmetric per-tensor int8 quantize -> dequantize of N(0,1) data (BASELINE config 1, small sizes)."""
+    """Symmetric per-tensor int8 quantize -> dequantize of N(0,1) data (the round-trip configuration at small sizes)."""
     x = normal(1, shape)
     want_q, scale, zp = oracle.quantize_tensor_auto(x, 0, oracle.PER_TENSOR_SYMMETRIC)
     want_y = oracle.dequantize_per_tensor_affine(want_q, scale, zp)
@@ -192,7 +192,7 @@ def test_config1_round_trip(ctx, hipq, oracle, shape):
 
 
 def test_config1_full_size_properties(ctx, hipq):
-    """Full BASELINE size [4096,4096]: size-independent properties instead of a CPU pass."""
+    """Full size [4096,4096]: size-independent properties instead of a CPU pass."""
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn(4096, 4096, generator=g, device="cuda", dtype=torch.float32)
     q, params = ctx.quantize_dynamic_per_tensor(x, hipq.PARAMS_SYMMETRIC, hipq.DTYPE_I8, hipq.FORM_MUL_INV)

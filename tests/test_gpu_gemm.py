@@ -184,7 +184,7 @@ def test_gemm_error_cases(ctx, hipq):
 
 @pytest.mark.parametrize("m", [1, 4, 16, 17, 40, 64])
 def test_config3_full_size_weight_streaming(ctx, hipq, m):
-    """Llama-7B up-proj shape N=11008, K=4096 (BASELINE config 3): int32 accumulators against an exact
+    """Llama-7B up-proj shape N=11008, K=4096: int32 accumulators against an exact
     float64 product computed by torch, and the fused per-token epilogue against the same f32 expression."""
     g = torch.Generator(device="cuda").manual_seed(5 + m)
     n, k = 11008, 4096

@@ -1,4 +1,4 @@
-"""fp32 helpers (LayerNorm, GELU, residual) and the int8 projection stack (BASELINE config 5 at reduced size).
+"""fp32 helpers (LayerNorm, GELU, residual) and the int8 projection stack (12 x 768 x 3072 configuration at reduced size).
 
 Integer steps are bit-exact given identical fp32 inputs; LayerNorm and GELU are fp32 transcendentals / reductions
 whose last bits differ from the CPU's, so they are held to a stated tolerance and the end-to-end drift is reported."""
