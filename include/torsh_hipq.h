@@ -72,7 +72,12 @@ enum {
     /* torsh-backend from_statistics, symmetric: params.rs:323-340 */
     HIPQ_PARAMS_BACKEND_SYMMETRIC = 2,
     /* torsh-backend from_statistics, asymmetric: params.rs:343-363 */
-    HIPQ_PARAMS_BACKEND_ASYMMETRIC = 3
+    HIPQ_PARAMS_BACKEND_ASYMMETRIC = 3,
+    /* The range is first widened to contain 0, a zero scale becomes 1:
+     * Observer::calculate_qparams (crates/torsh-quantization/src/observers.rs:263-310),
+     * quantize_int4_per_tensor / _per_channel and quantize_group_wise
+     * (crates/torsh-quantization/src/specialized.rs:39-48, 126-133, 322-335). */
+    HIPQ_PARAMS_ZERO_INCLUDED = 4
 };
 
 /* Device-resident quantization parameters, written by the kernels that derive
@@ -188,6 +193,29 @@ HIPQ_API int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const floa
                                                        size_t channels, size_t inner, int32_t flavor,
                                                        int32_t mode, int8_t *out, float *out_scales,
                                                        int32_t *out_zero_points, int32_t *out_status);
+/* Generalisation to groups of `group_size` consecutive channels that share
+ * one (scale, zero point) - the last group may be shorter - with a caller-chosen
+ * integer range [qmin, qmax] inside [-128, 127] and any HIPQ_PARAMS_* flavor:
+ * quantize_group_wise (crates/torsh-quantization/src/specialized.rs:241-377) and,
+ * with group_size 1 and range -8..7, quantize_int4_per_channel (specialized.rs:68-160).
+ * out_scales / out_zero_points hold ceil(channels / group_size) entries.  Values
+ * are stored one per int8. */
+HIPQ_API int32_t hipq_quantize_per_group_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels,
+                                                     size_t inner, size_t group_size, int32_t flavor, int32_t qmin,
+                                                     int32_t qmax, int32_t mode, int8_t *out, float *out_scales,
+                                                     int32_t *out_zero_points, int32_t *out_status);
+/* quantize_binary, crates/torsh-quantization/src/specialized.rs:163-188:
+ * out = x >= 0 ? 1 : -1 (int8), scale = mean |x| (1 if that is 0), zero point 0.
+ * quantize_ternary, specialized.rs:191-238: threshold = 0.7 * max |x|;
+ * out = 0 where |x| <= threshold, else sign(x); scale = mean of |x| over the
+ * values above the threshold (1 if there are none).  out_params is a device
+ * record; min_val / max_val hold the threshold (0 for binary) and max |x|.
+ * n == 0 is InvalidArgument as in the reference.  The means are formed from
+ * f64 sums (the reference adds f32 terms in element order). */
+HIPQ_API int32_t hipq_quantize_binary_f32_i8(hipq_ctx *ctx, const float *x, size_t n, int8_t *out,
+                                             hipq_qparams *out_params);
+HIPQ_API int32_t hipq_quantize_ternary_f32_i8(hipq_ctx *ctx, const float *x, size_t n, int8_t *out,
+                                              hipq_qparams *out_params);
 /* quantize_per_channel_affine, explicit parameters,
  * crates/torsh-quantization/src/quantize.rs:287-331 (HIPQ_FORM_DIV) and
  * quantize_per_channel_simd, simd_ops.rs:124-169 (HIPQ_FORM_MUL_INV, inner

@@ -87,6 +87,12 @@ def _declare(l: C.CDLL) -> None:
                                                          _f32p, _f32p]
     l.tq_model_fake_quantize.restype = None
     l.tq_model_fake_quantize.argtypes = [_f32p, C.c_size_t, C.c_float, C.c_int32, C.c_int32, C.c_int32, _f32p]
+    l.tq_quantize_int4_per_tensor.argtypes = [_f32p, C.c_size_t, _f32p, _f32p, _i32p]
+    l.tq_quantize_int4_per_channel.argtypes = [_f32p, _szp, C.c_size_t, C.c_size_t, _f32p, _f32p, _i32p, _f32p, _i32p]
+    l.tq_quantize_binary.argtypes = [_f32p, C.c_size_t, _f32p, _f32p, C.POINTER(C.c_double)]
+    l.tq_quantize_ternary.argtypes = [_f32p, C.c_size_t, _f32p, _f32p, C.POINTER(C.c_double), _f32p]
+    l.tq_quantize_group_wise.argtypes = [_f32p, _szp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int32, C.c_int32, _f32p,
+                                         _f32p, _i32p, _f32p, _i32p]
     l.tq_model_mse_error.restype = C.c_double
     l.tq_model_mse_error.argtypes = [_f32p, _f32p, C.c_size_t]
 
@@ -556,3 +562,66 @@ def model_fake_quantize(x, scale, zp, qmin=-128, qmax=127) -> np.ndarray:
 def model_mse_error(original, quantized) -> float:
     a, b = _f32(original).ravel(), _f32(quantized).ravel()
     return float(lib().tq_model_mse_error(_p(a, _f32p), _p(b, _f32p), C.c_size_t(a.size)))
+
+
+# ---- special schemes (specialized.rs) ---------------------------------------------------------
+
+def _shape(x):
+    return (C.c_size_t * x.ndim)(*x.shape)
+
+
+def quantize_int4_per_tensor(x):
+    """-> (carrier, scale, zero_point)"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    s, z = C.c_float(), C.c_int32()
+    lib().tq_quantize_int4_per_tensor(_p(x, _f32p), C.c_size_t(x.size), _p(out, _f32p), C.byref(s), C.byref(z))
+    return out, np.float32(s.value), z.value
+
+
+def quantize_int4_per_channel(x, axis):
+    """-> (carrier, scales, zero_points, avg_scale, avg_zero_point)"""
+    x = _f32(x)
+    if axis >= x.ndim:
+        raise OracleError("quantize_int4_per_channel: Axis out of bounds")
+    ch = x.shape[axis]
+    out = np.empty_like(x)
+    scales, zps = np.empty(ch, np.float32), np.empty(ch, np.int32)
+    s, z = C.c_float(), C.c_int32()
+    _check(lib().tq_quantize_int4_per_channel(_p(x, _f32p), _shape(x), x.ndim, axis, _p(out, _f32p), _p(scales, _f32p),
+                                              _p(zps, _i32p), C.byref(s), C.byref(z)), "quantize_int4_per_channel")
+    return out, scales, zps, np.float32(s.value), z.value
+
+
+def quantize_binary(x):
+    """-> (carrier, scale, scale from an f64 sum)"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    s, d = C.c_float(), C.c_double()
+    _check(lib().tq_quantize_binary(_p(x, _f32p), C.c_size_t(x.size), _p(out, _f32p), C.byref(s), C.byref(d)),
+           "quantize_binary")
+    return out, np.float32(s.value), d.value
+
+
+def quantize_ternary(x):
+    """-> (carrier, scale, scale from an f64 sum, threshold)"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    s, d, t = C.c_float(), C.c_double(), C.c_float()
+    _check(lib().tq_quantize_ternary(_p(x, _f32p), C.c_size_t(x.size), _p(out, _f32p), C.byref(s), C.byref(d),
+                                     C.byref(t)), "quantize_ternary")
+    return out, np.float32(s.value), d.value, np.float32(t.value)
+
+
+def quantize_group_wise(x, axis, group_size, qmin=-128, qmax=127):
+    """-> (carrier, group_scales, group_zero_points, avg_scale, avg_zero_point)"""
+    x = _f32(x)
+    if axis >= x.ndim or group_size == 0:
+        raise OracleError("quantize_group_wise: invalid axis or group size")
+    groups = -(-x.shape[axis] // group_size)
+    out = np.empty_like(x)
+    scales, zps = np.empty(groups, np.float32), np.empty(groups, np.int32)
+    s, z = C.c_float(), C.c_int32()
+    _check(lib().tq_quantize_group_wise(_p(x, _f32p), _shape(x), x.ndim, axis, group_size, qmin, qmax, _p(out, _f32p),
+                                        _p(scales, _f32p), _p(zps, _i32p), C.byref(s), C.byref(z)), "quantize_group_wise")
+    return out, scales, zps, np.float32(s.value), z.value

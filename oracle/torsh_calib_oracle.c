@@ -391,3 +391,159 @@ double tq_model_mse_error(const float *original, const float *quantized, size_t 
     }
     return (double)(sum / (float)n);
 }
+
+/* ---- special schemes ------------------------------------------------------ */
+
+/* specialized.rs:33-65 */
+int tq_quantize_int4_per_tensor(const float *x, size_t n, float *out, float *scale, int32_t *zp) {
+    float mn = INFINITY, mx = -INFINITY;
+    for (size_t i = 0; i < n; ++i) {
+        mn = fminf(mn, x[i]);
+        mx = fmaxf(mx, x[i]);
+    }
+    mn = fminf(mn, 0.0f);
+    mx = fmaxf(mx, 0.0f);
+    float s = (mx - mn) / 15.0f;
+    if (s == 0.0f) s = 1.0f;
+    const int32_t z = f32_as_i32(clamp_keep_nan(roundf(-8.0f - mn / s), -8.0f, 7.0f));
+    for (size_t i = 0; i < n; ++i) out[i] = clamp_keep_nan(roundf(x[i] / s) + (float)z, -8.0f, 7.0f);
+    *scale = s;
+    *zp = z;
+    return 0;
+}
+
+/* Channel coordinate of flat index i along `axis` (the stride walk of specialized.rs:106-117). */
+static size_t channel_of(size_t i, const size_t *shape, size_t ndim, size_t axis) {
+    size_t inner = 1;
+    for (size_t d = axis + 1; d < ndim; ++d) inner *= shape[d];
+    return (i / inner) % shape[axis];
+}
+
+/* specialized.rs:68-160 */
+int tq_quantize_int4_per_channel(const float *x, const size_t *shape, size_t ndim, size_t axis, float *out,
+                                 float *scales, int32_t *zps, float *avg_scale, int32_t *avg_zp) {
+    if (axis >= ndim) return 1;
+    size_t n = 1;
+    for (size_t d = 0; d < ndim; ++d) n *= shape[d];
+    const size_t channels = shape[axis];
+    for (size_t i = 0; i < n; ++i) out[i] = 0.0f;
+    for (size_t ch = 0; ch < channels; ++ch) {
+        float mn = INFINITY, mx = -INFINITY;
+        for (size_t i = 0; i < n; ++i)
+            if (channel_of(i, shape, ndim, axis) == ch) {
+                mn = fminf(mn, x[i]);
+                mx = fmaxf(mx, x[i]);
+            }
+        mn = fminf(mn, 0.0f);
+        mx = fmaxf(mx, 0.0f);
+        float s = (mx - mn) / 15.0f;
+        if (s == 0.0f) s = 1.0f;
+        const int32_t z = f32_as_i32(clamp_keep_nan(roundf(-8.0f - mn / s), -8.0f, 7.0f));
+        scales[ch] = s;
+        zps[ch] = z;
+        for (size_t i = 0; i < n; ++i)
+            if (channel_of(i, shape, ndim, axis) == ch)
+                out[i] = clamp_keep_nan(roundf(x[i] / s) + (float)z, -8.0f, 7.0f);
+    }
+    float ssum = 0.0f;
+    int32_t zsum = 0;
+    for (size_t ch = 0; ch < channels; ++ch) {
+        ssum += scales[ch];
+        zsum += zps[ch];
+    }
+    *avg_scale = ssum / (float)channels;                           /* :154 */
+    *avg_zp = f32_as_i32(roundf((float)zsum / (float)channels));   /* :155-156 */
+    return 0;
+}
+
+/* specialized.rs:163-188 */
+int tq_quantize_binary(const float *x, size_t n, float *out, float *scale, double *scale_f64) {
+    if (n == 0) return 1;
+    float sum = 0.0f;
+    double dsum = 0.0;
+    for (size_t i = 0; i < n; ++i) {
+        sum += fabsf(x[i]);
+        dsum += (double)fabsf(x[i]);
+    }
+    float s = sum / (float)n;
+    if (s == 0.0f) s = 1.0f;
+    for (size_t i = 0; i < n; ++i) out[i] = x[i] >= 0.0f ? 1.0f : -1.0f;
+    *scale = s;
+    if (scale_f64) *scale_f64 = dsum == 0.0 ? 1.0 : dsum / (double)n;
+    return 0;
+}
+
+/* specialized.rs:191-238 */
+int tq_quantize_ternary(const float *x, size_t n, float *out, float *scale, double *scale_f64, float *threshold) {
+    if (n == 0) return 1;
+    float max_abs = 0.0f;
+    for (size_t i = 0; i < n; ++i) max_abs = fmaxf(max_abs, fabsf(x[i]));
+    const float thr = max_abs * 0.7f;
+    float sum = 0.0f;
+    double dsum = 0.0;
+    size_t count = 0;
+    for (size_t i = 0; i < n; ++i)
+        if (fabsf(x[i]) > thr) {
+            sum += fabsf(x[i]);
+            dsum += (double)fabsf(x[i]);
+            ++count;
+        }
+    *scale = count > 0 ? sum / (float)count : 1.0f;
+    if (scale_f64) *scale_f64 = count > 0 ? dsum / (double)count : 1.0;
+    if (threshold) *threshold = thr;
+    for (size_t i = 0; i < n; ++i) out[i] = fabsf(x[i]) <= thr ? 0.0f : (x[i] > 0.0f ? 1.0f : -1.0f);
+    return 0;
+}
+
+/* specialized.rs:241-377 */
+int tq_quantize_group_wise(const float *x, const size_t *shape, size_t ndim, size_t axis, size_t group_size,
+                           int32_t qmin, int32_t qmax, float *out, float *group_scales, int32_t *group_zps,
+                           float *avg_scale, int32_t *avg_zp) {
+    if (axis >= ndim || group_size == 0) return 1;
+    size_t n = 1;
+    for (size_t d = 0; d < ndim; ++d) n *= shape[d];
+    const size_t channels = shape[axis];
+    const size_t groups = (channels + group_size - 1) / group_size;
+    for (size_t i = 0; i < n; ++i) out[i] = 0.0f;
+    size_t produced = 0;
+    for (size_t g = 0; g < groups; ++g) {
+        const size_t c0 = g * group_size, c1 = c0 + group_size < channels ? c0 + group_size : channels;
+        float mn = INFINITY, mx = -INFINITY;
+        size_t members = 0;
+        for (size_t i = 0; i < n; ++i) {
+            const size_t c = channel_of(i, shape, ndim, axis);
+            if (c >= c0 && c < c1) {
+                mn = fminf(mn, x[i]);
+                mx = fmaxf(mx, x[i]);
+                ++members;
+            }
+        }
+        if (members == 0) continue; /* :301-303 */
+        mn = fminf(mn, 0.0f);
+        mx = fmaxf(mx, 0.0f);
+        float s = (mx - mn) / (float)(qmax - qmin);
+        if (s == 0.0f) s = 1.0f;
+        const int32_t z = f32_as_i32(fminf(fmaxf(roundf((float)qmin - mn / s), (float)qmin), (float)qmax));
+        group_scales[produced] = s;
+        group_zps[produced] = z;
+        ++produced;
+        for (size_t i = 0; i < n; ++i) {
+            const size_t c = channel_of(i, shape, ndim, axis);
+            if (c >= c0 && c < c1) out[i] = fminf(fmaxf(roundf(x[i] / s) + (float)z, (float)qmin), (float)qmax);
+        }
+    }
+    if (produced == 0) {
+        *avg_scale = 1.0f;
+        *avg_zp = 0;
+        return 0;
+    }
+    float ssum = 0.0f;
+    int32_t zsum = 0;
+    for (size_t g = 0; g < produced; ++g) {
+        ssum += group_scales[g];
+        zsum += group_zps[g];
+    }
+    *avg_scale = ssum / (float)produced;
+    *avg_zp = f32_as_i32(roundf((float)zsum / (float)produced));
+    return 0;
+}

@@ -86,6 +86,24 @@ void tq_model_fake_quantize(const float *x, size_t n, float scale, int32_t zp, i
 /* ModelQuantizer::calculate_mse_error, quantization.rs:548-566 (f32 sum, result widened). */
 double tq_model_mse_error(const float *original, const float *quantized, size_t n);
 
+/* ---- special schemes: crates/torsh-quantization/src/specialized.rs -------- */
+/* quantize_int4_per_tensor, specialized.rs:33-65 (f32 carrier, range -8..7). */
+int tq_quantize_int4_per_tensor(const float *x, size_t n, float *out, float *scale, int32_t *zp);
+/* quantize_int4_per_channel, specialized.rs:68-160.  scales / zps (num_channels each) receive the
+ * per-channel parameters; avg_scale / avg_zp are what the function returns. */
+int tq_quantize_int4_per_channel(const float *x, const size_t *shape, size_t ndim, size_t axis, float *out,
+                                 float *scales, int32_t *zps, float *avg_scale, int32_t *avg_zp);
+/* quantize_binary, specialized.rs:163-188; scale_f64 (may be NULL) receives the mean of |x| from an
+ * f64 sum. */
+int tq_quantize_binary(const float *x, size_t n, float *out, float *scale, double *scale_f64);
+/* quantize_ternary, specialized.rs:191-238; threshold (may be NULL) receives 0.7 * max|x|. */
+int tq_quantize_ternary(const float *x, size_t n, float *out, float *scale, double *scale_f64, float *threshold);
+/* quantize_group_wise, specialized.rs:241-377 with the integer range [qmin, qmax] of
+ * config.get_qint_range().  group_scales / group_zps hold num_groups = ceil(shape[axis]/group_size). */
+int tq_quantize_group_wise(const float *x, const size_t *shape, size_t ndim, size_t axis, size_t group_size,
+                           int32_t qmin, int32_t qmax, float *out, float *group_scales, int32_t *group_zps,
+                           float *avg_scale, int32_t *avg_zp);
+
 #ifdef __cplusplus
 }
 #endif

@@ -796,20 +796,27 @@ GPU_TEST(test_calculate_quantization_metrics) {  // metrics.rs:588-621
 
 GPU_TEST(test_compare_quantization_configs) {  // metrics.rs:623-661
     const Tensor tensor = tensor_1d({1.0f, 2.0f, 3.0f, 4.0f, 5.0f}).unwrap();
-    QuantConfig binary;
-    binary.scheme = QScheme::Binary;
-    const std::vector<QuantConfig> configs{QuantConfig::int8(), binary,
-                                           QuantConfig::int8().with_scheme(QScheme::PerTensorSymmetric)};
+    const std::vector<QuantConfig> configs{QuantConfig::int8(), QuantConfig::binary(), QuantConfig::ternary()};
     const auto results = compare_quantization_configs(tensor, configs).unwrap();
     CHECK_EQ(results.size(), size_t(3));
+    for (const auto &r : results) {
+        bool known = false;
+        for (const auto &c : configs) known = known || c.scheme == r.config.scheme;
+        CHECK(known && r.seconds >= 0.0);
+        if (std::isfinite(r.metrics.psnr))
+            CHECK(r.metrics.psnr > 0.0f && r.metrics.compression_ratio >= 1.0f && r.metrics.mae >= 0.0f &&
+                  r.metrics.mse >= 0.0f);
+    }
     for (size_t i = 1; i < results.size(); ++i) {
         const float a = results[i - 1].metrics.psnr, b = results[i].metrics.psnr;
         if (std::isfinite(a) && std::isfinite(b)) CHECK(a >= b);
     }
-    // the scheme outside the int8 path is reported with the worst-case record and sorts last
-    CHECK(results.back().config.scheme == QScheme::Binary && std::isinf(results.back().metrics.mse));
-    for (const auto &r : results)
-        if (std::isfinite(r.metrics.psnr)) CHECK(r.metrics.psnr > 0.0f && r.metrics.compression_ratio >= 1.0f);
+    // a configuration that cannot be quantized gets the worst-case record and sorts last (metrics.rs:231-245)
+    QuantConfig mixed;
+    mixed.scheme = QScheme::MixedPrecision;
+    const auto with_bad = compare_quantization_configs(tensor, {mixed, QuantConfig::int8()}).unwrap();
+    CHECK(with_bad.back().config.scheme == QScheme::MixedPrecision && std::isinf(with_bad.back().metrics.mse));
+    CHECK(with_bad.back().metrics.psnr < 0 && with_bad.back().metrics.zero_error_percentage == 0.0f);
 }
 
 GPU_TEST(parity_metrics_and_compare_configs) {
@@ -1029,6 +1036,103 @@ GPU_TEST(test_quantized_modules_survive_a_weight_file) {
     check_same(conv2.forward_quantized(cx).unwrap().as_slice(), conv.forward_quantized(cx).unwrap().as_slice(), __LINE__);
     CHECK(nn::QuantizedLinear::load(path).is_err());  // a conv file is not a linear layer
     std::remove(path.c_str());
+}
+
+
+GPU_TEST(test_special_schemes) {  // specialized.rs:577-654, 743-761
+    {
+        const std::vector<float> data{1.0f, 2.0f, 3.0f, 4.0f, 5.0f};
+        const auto [q, scale, zp] = quantize_int4_per_tensor(tensor_1d(data).unwrap(), QuantConfig::int4()).unwrap();
+        CHECK(scale > 0.0f && zp >= -8 && zp <= 7);
+        CHECK_EQ(q.numel(), data.size());
+        for (float v : q.as_slice()) CHECK(v >= -8.0f && v <= 7.0f);
+    }
+    {
+        const auto [q, scale, zp] = quantize_binary(tensor_1d({-2.0f, -1.0f, 0.0f, 1.0f, 2.0f}).unwrap()).unwrap();
+        CHECK(scale > 0.0f && zp == 0);
+        for (float v : q.as_slice()) CHECK(v == -1.0f || v == 1.0f);
+    }
+    {
+        const auto [q, scale, zp] = quantize_ternary(tensor_1d({-3.0f, -1.0f, 0.1f, 1.0f, 3.0f}).unwrap()).unwrap();
+        CHECK(scale > 0.0f && zp == 0);
+        for (float v : q.as_slice()) CHECK(v == -1.0f || v == 0.0f || v == 1.0f);
+    }
+    {
+        const Tensor t = Tensor::from_data({1.0f, 2.0f, 3.0f, 4.0f, 5.0f, 6.0f}, {2, 3}).unwrap();
+        const auto [q, scale, zp] = quantize_group_wise(t, 1, 2, QuantConfig::group_wise(1, 2)).unwrap();
+        CHECK(scale > 0.0f && q.shape().dims() == t.shape().dims());
+    }
+    const Tensor empty = tensor_1d({}).unwrap();
+    CHECK(quantize_binary(empty).is_err() && quantize_ternary(empty).is_err());
+    const Tensor t3 = tensor_1d({1.0f, 2.0f, 3.0f}).unwrap();
+    CHECK(quantize_group_wise(t3, 5, 2, QuantConfig::group_wise(0, 2)).is_err());
+    CHECK(quantize_group_wise(t3, 0, 0, QuantConfig::group_wise(0, 2)).is_err());
+    // through the dispatcher (algorithms.rs:47-57)
+    CHECK(quantize_with_config(t3, QuantConfig::int4()).is_ok());
+    CHECK(quantize_with_config(t3, QuantConfig::binary()).is_ok());
+    CHECK(quantize_with_config(t3, QuantConfig::ternary()).is_ok());
+    CHECK(quantize_with_config(t3, QuantConfig::group_wise(0, 2)).is_ok());
+}
+
+GPU_TEST(parity_special_schemes) {
+    const std::vector<float> x = normal(24 * 50 * 6, 71, 1.3f);
+    const std::vector<size_t> dims{24, 50, 6};
+    const Tensor t = Tensor::from_data(x, dims).unwrap();
+    std::vector<float> want(x.size());
+    float s;
+    int32_t z;
+    {
+        const auto [q, scale, zp] = quantize_int4_per_tensor(t, QuantConfig::int4()).unwrap();
+        CHECK_EQ(tq_quantize_int4_per_tensor(x.data(), x.size(), want.data(), &s, &z), 0);
+        CHECK(scale == s && zp == z);
+        check_same(q.as_slice(), want, __LINE__);
+    }
+    for (size_t axis : {size_t(0), size_t(1), size_t(2)}) {
+        std::vector<float> scales(dims[axis]);
+        std::vector<int32_t> zps(dims[axis]);
+        const auto [q, scale, zp] = quantize_int4_per_channel(t, axis, QuantConfig::int4()).unwrap();
+        CHECK_EQ(tq_quantize_int4_per_channel(x.data(), dims.data(), 3, axis, want.data(), scales.data(), zps.data(), &s, &z), 0);
+        CHECK(scale == s && zp == z);
+        check_same(q.as_slice(), want, __LINE__);
+    }
+    {
+        double s64;
+        const auto [q, scale, zp] = quantize_binary(t).unwrap();
+        CHECK_EQ(tq_quantize_binary(x.data(), x.size(), want.data(), &s, &s64), 0);
+        check_same(q.as_slice(), want, __LINE__);
+        CHECK(close_rel(scale, s64, 1e-6) && close_rel(scale, s, 1e-4) && zp == 0);
+    }
+    {
+        double s64;
+        float thr;
+        const auto [q, scale, zp] = quantize_ternary(t).unwrap();
+        CHECK_EQ(tq_quantize_ternary(x.data(), x.size(), want.data(), &s, &s64, &thr), 0);
+        check_same(q.as_slice(), want, __LINE__);
+        CHECK(close_rel(scale, s64, 1e-6) && close_rel(scale, s, 1e-4) && zp == 0);
+    }
+    struct G {
+        size_t axis, group;
+    };
+    for (G g : {G{0, 4}, G{0, 5}, G{0, 24}, G{0, 100}, G{1, 10}, G{1, 50}, G{1, 7}, G{2, 3}, G{2, 1}, G{2, 4}}) {
+        const QuantConfig cfg = QuantConfig::group_wise(g.axis, g.group);
+        const size_t groups = (dims[g.axis] + g.group - 1) / g.group;
+        std::vector<float> gs(groups);
+        std::vector<int32_t> gz(groups);
+        const auto [q, scale, zp] = quantize_group_wise(t, g.axis, g.group, cfg).unwrap();
+        CHECK_EQ(tq_quantize_group_wise(x.data(), dims.data(), 3, g.axis, g.group, -128, 127, want.data(), gs.data(),
+                                        gz.data(), &s, &z), 0);
+        CHECK(scale == s && zp == z);
+        check_same(q.as_slice(), want, __LINE__);
+    }
+    // reduced integer range through the configuration (config.rs:304-328)
+    const QuantConfig reduced = QuantConfig::group_wise(0, 4).with_reduce_range(ReduceRange::Reduce);
+    const auto [qmin, qmax] = reduced.get_qint_range();
+    std::vector<float> gs(6);
+    std::vector<int32_t> gz(6);
+    const auto [q, scale, zp] = quantize_group_wise(t, 0, 4, reduced).unwrap();
+    CHECK_EQ(tq_quantize_group_wise(x.data(), dims.data(), 3, 0, 4, qmin, qmax, want.data(), gs.data(), gz.data(), &s, &z), 0);
+    CHECK(scale == s && zp == z);
+    check_same(q.as_slice(), want, __LINE__);
 }
 
 }  // namespace

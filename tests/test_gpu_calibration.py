@@ -266,3 +266,118 @@ def test_full_size_properties(ctx, hipq, oracle):
     same = ctx.read_metrics(ctx.quantization_metrics(x, x))
     assert same["mse"] == 0 and same["zero_error_percentage"] == 100 and math.isinf(same["psnr"])
     assert same["cosine_similarity"] == pytest.approx(1.0, abs=1e-6)
+
+
+# ---- special schemes (int4, group-wise, binary, ternary) -----------------------------------------
+
+def _view(shape, axis):
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return outer, shape[axis], inner
+
+
+@pytest.mark.parametrize("shape,axis,group", [((24, 50, 6), 0, 4), ((24, 50, 6), 0, 5), ((24, 50, 6), 1, 10),
+                                               ((24, 50, 6), 1, 7), ((24, 50, 6), 2, 4), ((64, 2048), 0, 1),
+                                               ((64, 2048), 0, 8), ((3, 4096), 1, 128), ((7, 1000), 1, 32),
+                                               ((5,), 0, 2)])
+def test_group_wise_is_bit_exact(ctx, hipq, oracle, shape, axis, group):
+    x = normal(sum(shape) + axis + group, shape, 1.7)
+    outer, channels, inner = _view(shape, axis)
+    for qmin, qmax in ((-128, 127), (-8, 7), (-63, 63)):
+        q, scales, zps, status = ctx.quantize_per_group_auto(dev(x), outer, channels, inner, group,
+                                                             hipq.PARAMS_ZERO_INCLUDED, qmin, qmax, hipq.FORM_DIV)
+        want, ws, wz, _, _ = oracle.quantize_group_wise(x, axis, group, qmin, qmax)
+        assert int(host(status)[0]) == 0
+        np.testing.assert_array_equal(host(scales), ws)
+        np.testing.assert_array_equal(host(zps), wz)
+        np.testing.assert_array_equal(host(q).astype(np.float32), want)
+
+
+def test_int4_per_tensor_and_per_channel_are_bit_exact(ctx, hipq, oracle, cal):
+    for case in cal["special_schemes"]:
+        if case["fn"] != "quantize_int4_per_tensor":
+            continue
+        x = np.float32(case["x"])
+        q, scales, zps, _ = ctx.quantize_per_group_auto(dev(x), 1, 1, x.size, 1, hipq.PARAMS_ZERO_INCLUDED, -8, 7, hipq.FORM_DIV)
+        want, s, z = oracle.quantize_int4_per_tensor(x)
+        np.testing.assert_array_equal(host(q).astype(np.float32), want)
+        assert host(scales)[0] == s and host(zps)[0] == z and case["zp_range"][0] <= z <= case["zp_range"][1]
+    x = normal(13, (16, 33, 9), 0.8)
+    for axis in range(3):
+        outer, channels, inner = _view(x.shape, axis)
+        q, scales, zps, _ = ctx.quantize_per_group_auto(dev(x), outer, channels, inner, 1, hipq.PARAMS_ZERO_INCLUDED, -8, 7,
+                                                        hipq.FORM_DIV)
+        want, ws, wz, _, _ = oracle.quantize_int4_per_channel(x, axis)
+        np.testing.assert_array_equal(host(q).astype(np.float32), want)
+        np.testing.assert_array_equal(host(scales), ws)
+        np.testing.assert_array_equal(host(zps), wz)
+    big = normal(14, 1 << 20, 2.0)
+    q, scales, zps, _ = ctx.quantize_per_group_auto(dev(big), 1, 1, big.size, 1, hipq.PARAMS_ZERO_INCLUDED, -8, 7, hipq.FORM_DIV)
+    want, s, z = oracle.quantize_int4_per_tensor(big)
+    np.testing.assert_array_equal(host(q).astype(np.float32), want)
+    assert host(scales)[0] == s and host(zps)[0] == z
+
+
+def test_group_wise_argument_errors(ctx, hipq):
+    x = dev(normal(1, (4, 8)))
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.quantize_per_group_auto(x, 1, 4, 8, 0, hipq.PARAMS_ZERO_INCLUDED, -128, 127)
+    assert "Group size must be greater than 0" in e.value.message
+    with pytest.raises(hipq.HipqError):
+        ctx.quantize_per_group_auto(x, 1, 4, 8, 2, hipq.PARAMS_ZERO_INCLUDED, -200, 127)
+    with pytest.raises(hipq.HipqError):
+        ctx.quantize_per_group_auto(x, 1, 4, 8, 2, 9, -128, 127)
+    # a non-finite range is reported through the status word, not as garbage parameters
+    bad = normal(2, (4, 8))
+    bad[1, 3] = np.inf
+    _, _, _, status = ctx.quantize_per_group_auto(dev(bad), 1, 4, 8, 2, hipq.PARAMS_ZERO_INCLUDED, -128, 127)
+    assert int(host(status)[0]) == hipq.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("n", [1, 5, 63, 4096, 100003, 1 << 20])
+def test_binary_and_ternary(ctx, hipq, oracle, n):
+    x = normal(40 + n, n, 1.1)
+    if n >= 63:
+        x[::9] = 0.0            # zeros are +1 for the binary scheme and 0 for the ternary one
+    q, params = ctx.quantize_binary(dev(x))
+    want, s32, s64 = oracle.quantize_binary(x)
+    p = ctx.read_qparams(params)
+    np.testing.assert_array_equal(host(q).astype(np.float32), want)
+    assert p.zero_point == 0 and p.status == 0
+    assert p.scale == pytest.approx(s64, rel=1e-6) and p.scale == pytest.approx(float(s32), rel=1e-4)
+    q, params = ctx.quantize_ternary(dev(x))
+    want, s32, s64, thr = oracle.quantize_ternary(x)
+    p = ctx.read_qparams(params)
+    np.testing.assert_array_equal(host(q).astype(np.float32), want)
+    assert p.min_val == thr and p.zero_point == 0
+    assert p.scale == pytest.approx(s64, rel=1e-6) and p.scale == pytest.approx(float(s32), rel=1e-4)
+
+
+def test_binary_ternary_golden_edges_and_errors(ctx, hipq, oracle, cal):
+    for case in cal["special_schemes"]:
+        if case["fn"] not in ("quantize_binary", "quantize_ternary"):
+            continue
+        x = np.float32(case["x"])
+        fn = ctx.quantize_binary if case["fn"] == "quantize_binary" else ctx.quantize_ternary
+        q, params = fn(dev(x))
+        p = ctx.read_qparams(params)
+        assert p.scale > 0 and p.zero_point == case["zp"] and set(host(q).tolist()) <= set(case["values_in"])
+    zeros = torch.zeros(1000, device="cuda")
+    q, params = ctx.quantize_binary(zeros)
+    assert ctx.read_qparams(params).scale == 1.0 and (host(q) == 1).all()
+    q, params = ctx.quantize_ternary(zeros)
+    assert ctx.read_qparams(params).scale == 1.0 and (host(q) == 0).all()
+    x = np.float32([10, 7, -7, 7.5, -10, float("nan")])
+    np.testing.assert_array_equal(host(ctx.quantize_ternary(dev(x))[0]).astype(np.float32), oracle.quantize_ternary(x)[0])
+    np.testing.assert_array_equal(host(ctx.quantize_binary(dev(x))[0]).astype(np.float32), oracle.quantize_binary(x)[0])
+    empty = torch.empty(0, device="cuda")
+    for fn in (ctx.quantize_binary, ctx.quantize_ternary):
+        with pytest.raises(hipq.HipqError) as e:
+            fn(empty)
+        assert e.value.code == hipq.INVALID_ARGUMENT and "Cannot quantize empty tensor" in e.value.message
+    # unaligned views
+    base = normal(77, 10007)
+    d = dev(base)
+    for off in (1, 2, 3):
+        np.testing.assert_array_equal(host(ctx.quantize_ternary(d[off:])[0]).astype(np.float32),
+                                      oracle.quantize_ternary(base[off:])[0])

@@ -48,6 +48,8 @@ GPU_CASES = [
     "parity_quantize_batch_consistent",
     "parity_model_quantizer",
     "test_quantized_modules_survive_a_weight_file",
+    "test_special_schemes",
+    "parity_special_schemes",
 ]
 
 

@@ -318,3 +318,121 @@ def test_model_fake_quantize_closed_form(oracle):
     np.testing.assert_array_equal(y, x)
     np.testing.assert_array_equal(oracle.model_fake_quantize(y, 0.25, 0), y)
     assert oracle.model_mse_error(x, x + np.float32(0.5)) == 0.25
+
+
+# ---- special schemes (specialized.rs) ------------------------------------------------------------
+
+def test_special_scheme_known_answers(oracle, cal):
+    for case in cal["special_schemes"]:
+        fn = case["fn"]
+        if fn == "quantize_int4_per_tensor":
+            q, s, z = oracle.quantize_int4_per_tensor(case["x"])
+            assert s > 0 and case["zp_range"][0] <= z <= case["zp_range"][1]
+            assert q.min() >= case["value_range"][0] and q.max() <= case["value_range"][1]
+        elif fn == "quantize_binary":
+            q, s, _ = oracle.quantize_binary(case["x"])
+            assert s > 0 and set(q.tolist()) <= set(case["values_in"])
+        elif fn == "quantize_ternary":
+            q, s, _, _ = oracle.quantize_ternary(case["x"])
+            assert s > 0 and set(q.tolist()) <= set(case["values_in"])
+        elif fn == "quantize_group_wise":
+            x = np.float32(case["x"])
+            q, _, _, s, _ = oracle.quantize_group_wise(x, case["axis"], case["group_size"])
+            assert s > 0 and q.shape == x.shape
+        else:
+            with pytest.raises(oracle.OracleError):
+                oracle.quantize_binary([])
+            with pytest.raises(oracle.OracleError):
+                oracle.quantize_ternary([])
+            with pytest.raises(oracle.OracleError):
+                oracle.quantize_group_wise(np.float32([1, 2, 3]), 5, 2)
+            with pytest.raises(oracle.OracleError):
+                oracle.quantize_group_wise(np.float32([1, 2, 3]), 0, 0)
+
+
+def test_int4_closed_form(oracle):
+    # [0, 15]: scale 1, zero point -8, value k -> k - 8.
+    q, s, z = oracle.quantize_int4_per_tensor(np.arange(16, dtype=np.float32))
+    assert (s, z) == (1.0, -8)
+    np.testing.assert_array_equal(q, np.arange(16) - 8)
+    # all-positive data away from 0: the range still starts at 0 ([0, 30] -> scale 2)
+    q, s, z = oracle.quantize_int4_per_tensor(np.float32([10, 20, 30]))
+    assert (s, z) == (2.0, -8)
+    np.testing.assert_array_equal(q, [-3, 2, 7])
+    # symmetric data [-7.5, 7.5]: scale 1, zero point round(-8 + 7.5) = round(-0.5) = -1 (half away)
+    q, s, z = oracle.quantize_int4_per_tensor(np.float32([-7.5, 0.0, 7.5]))
+    assert (s, z) == (1.0, -1)
+    np.testing.assert_array_equal(q, [-8, -1, 7])       # round(-7.5) = -8 -> -9 clamps to -8; round(7.5) = 8 -> 7
+    # all zeros: scale falls back to 1
+    q, s, z = oracle.quantize_int4_per_tensor(np.zeros(4, np.float32))
+    assert (s, z) == (1.0, -8) and (q == -8).all()
+
+
+def test_int4_per_channel_equals_per_tensor_on_each_slice(oracle):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    for axis in range(3):
+        q, scales, zps, avg_s, avg_z = oracle.quantize_int4_per_channel(x, axis)
+        for c in range(x.shape[axis]):
+            sl = np.take(x, c, axis=axis)
+            qc, sc, zc = oracle.quantize_int4_per_tensor(sl)
+            np.testing.assert_array_equal(np.take(q, c, axis=axis), qc)
+            assert (scales[c], zps[c]) == (sc, zc)
+        seq = np.float32(0)
+        for s in scales:
+            seq = np.float32(seq + s)
+        assert avg_s == np.float32(seq / np.float32(len(scales)))
+        m = float(zps.sum()) / len(zps)
+        assert avg_z == int(math.copysign(math.floor(abs(m) + 0.5), m))
+
+
+def test_binary_and_ternary_closed_form(oracle):
+    q, s, s64 = oracle.quantize_binary(np.float32([-2, -1, 0, 1, 2]))
+    np.testing.assert_array_equal(q, [-1, -1, 1, 1, 1])            # 0 counts as positive
+    assert s == np.float32(6.0 / 5.0) and s64 == pytest.approx(1.2)
+    q, s, _ = oracle.quantize_binary(np.zeros(3, np.float32))
+    assert s == 1.0 and (q == 1).all()
+    assert oracle.quantize_binary(np.float32([float("nan")]))[0][0] == -1     # NaN >= 0 is false
+    # ternary: threshold 0.7 * 3 = 2.1; only +-3 survive, scale = mean(3, 3) = 3
+    q, s, s64, thr = oracle.quantize_ternary(np.float32([-3, -1, 0.1, 1, 3]))
+    np.testing.assert_array_equal(q, [-1, 0, 0, 0, 1])
+    assert s == 3.0 and thr == np.float32(3.0) * np.float32(0.7)
+    # values exactly at the threshold become 0 (<=): max 10 -> threshold 7 exactly representable
+    q, s, _, thr = oracle.quantize_ternary(np.float32([10, 7, -7, 7.5, -10]))
+    assert thr == np.float32(10) * np.float32(0.7)
+    want = [1, 1 if np.float32(7) > thr else 0, -1 if np.float32(7) > thr else 0, 1, -1]
+    np.testing.assert_array_equal(q, want)
+    # all zeros: nothing above the threshold, scale 1
+    q, s, _, _ = oracle.quantize_ternary(np.zeros(5, np.float32))
+    assert s == 1.0 and (q == 0).all()
+
+
+def test_group_wise_equals_grouped_slices(oracle):
+    # Each group is quantized with the zero-including rule over all its members, whatever the axis.
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal((4, 7, 3)) * 2).astype(np.float32)
+    for axis, gs in ((0, 2), (1, 3), (1, 7), (2, 2), (1, 100)):
+        q, scales, zps, avg_s, avg_z = oracle.quantize_group_wise(x, axis, gs)
+        groups = -(-x.shape[axis] // gs)
+        assert len(scales) == groups
+        for g in range(groups):
+            idx = [slice(None)] * 3
+            idx[axis] = slice(g * gs, min((g + 1) * gs, x.shape[axis]))
+            sl = x[tuple(idx)]
+            mn, mx = min(float(sl.min()), 0.0), max(float(sl.max()), 0.0)
+            s = np.float32(np.float32(mx) - np.float32(mn)) / np.float32(255.0)
+            assert scales[g] == s
+            # the zero point follows from the scale by exact rational arithmetic
+            exact = Fraction(-128) - Fraction(mn) / Fraction(float(s))
+            lo, hi = math.floor(exact), math.ceil(exact)
+            assert zps[g] in (max(-128, min(127, lo)), max(-128, min(127, hi)))
+            want = np.clip(np.round(sl.astype(np.float64) / float(s)) + zps[g], -128, 127)
+            got = q[tuple(idx)]
+            assert np.abs(got - want).max() <= 1          # float64 rounding may differ on near-ties only
+            assert (got != want).mean() < 0.02
+    # group size 1 over the last axis with int4 range equals quantize_int4_per_channel
+    q4, s4, z4, _, _ = oracle.quantize_int4_per_channel(x, 2)
+    qg, sg, zg, _, _ = oracle.quantize_group_wise(x, 2, 1, -8, 7)
+    np.testing.assert_array_equal(qg, q4)
+    np.testing.assert_array_equal(sg, s4)
+    np.testing.assert_array_equal(zg, z4)

@@ -380,36 +380,40 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
         qr[c] = static_cast<int8_t>(quantize_int<true, EVEN>(xr[c], scale, inv, zpf, qmin, qmax));
 }
 
-// quantize_per_channel_auto for a channel axis that is not the leading one:
-// one block per channel walks its [outer, inner] slices twice.
+// quantize_per_channel_auto for a channel axis that is not the leading one, and its group-wise
+// form: one block per group of `group` consecutive channels (the last group may be shorter) walks
+// the group's [outer, members * inner] runs twice.
 template <bool EVEN>
 __global__ __launch_bounds__(kBlock) void quantize_per_channel_auto_kernel(
-    const float *__restrict__ x, size_t outer, size_t channels, size_t inner, int flavor, int qmin, int qmax,
-    int8_t *__restrict__ out, float *__restrict__ out_scales, int32_t *__restrict__ out_zps,
+    const float *__restrict__ x, size_t outer, size_t channels, size_t inner, size_t group, int flavor, int qmin,
+    int qmax, int8_t *__restrict__ out, float *__restrict__ out_scales, int32_t *__restrict__ out_zps,
     int32_t *__restrict__ out_status) {
     __shared__ float lds[2 * kBlock / kWave];
-    const size_t ch = blockIdx.x;
-    const size_t per = outer * inner;
+    const size_t g = blockIdx.x;
+    const size_t c0 = g * group;
+    const size_t members = (c0 + group <= channels) ? group : channels - c0;
+    const size_t run = members * inner;  // contiguous elements of this group per outer index
+    const size_t per = outer * run;
     MinMax m{INFINITY, -INFINITY};
     for (size_t i = threadIdx.x; i < per; i += kBlock) {
-        const size_t o = i / inner, in = i % inner;
-        acc_minmax(m, x[(o * channels + ch) * inner + in]);
+        const size_t o = i / run, r = i % run;
+        acc_minmax(m, x[(o * channels + c0) * inner + r]);
     }
     m = block_minmax(m, lds);
     float scale;
     int zp;
     const int st = params_from_minmax(m.mn, m.mx, flavor, qmin, qmax, &scale, &zp);
     if (threadIdx.x == 0) {
-        if (out_scales) out_scales[ch] = scale;
-        if (out_zps) out_zps[ch] = zp;
+        if (out_scales) out_scales[g] = scale;
+        if (out_zps) out_zps[g] = zp;
         if (st != HIPQ_SUCCESS && out_status) *out_status = st;
     }
     if (st != HIPQ_SUCCESS) return;
     const float zpf = static_cast<float>(zp), lo = static_cast<float>(qmin), hi = static_cast<float>(qmax);
     const float inv = recip_for_div(scale);
     for (size_t i = threadIdx.x; i < per; i += kBlock) {
-        const size_t o = i / inner, in = i % inner;
-        const size_t idx = (o * channels + ch) * inner + in;
+        const size_t o = i / run, r = i % run;
+        const size_t idx = (o * channels + c0) * inner + r;
         out[idx] = static_cast<int8_t>(to_int_nan0(quantize_value<true, EVEN>(x[idx], scale, inv, zpf, lo, hi)));
     }
 }
@@ -593,7 +597,7 @@ int32_t hipq_qparams_from_minmax(hipq_ctx *ctx, const float *minmax, int32_t fla
     HIPQ_ENTER(ctx);
     HIPQ_REQUIRE_PTR(minmax);
     HIPQ_REQUIRE_PTR(out_params);
-    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_BACKEND_ASYMMETRIC)
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
         return fail(HIPQ_INVALID_ARGUMENT, "hipq_qparams_from_minmax: unknown flavor %d", flavor);
     if (qmin >= qmax) return fail(HIPQ_INVALID_ARGUMENT, "hipq_qparams_from_minmax: qmin %d >= qmax %d", qmin, qmax);
     hipLaunchKernelGGL(qparams_kernel, dim3(1), dim3(64), 0, ctx->stream, minmax, flavor, qmin, qmax, out_params);
@@ -672,7 +676,7 @@ int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size
     HIPQ_REQUIRE_PTR(out_params);
     int32_t rc = check_mode(__func__, mode);
     if (rc) return rc;
-    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_BACKEND_ASYMMETRIC)
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", __func__, flavor);
     if (dtype != HIPQ_DTYPE_I8 && dtype != HIPQ_DTYPE_U8)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", __func__, dtype);
@@ -711,39 +715,83 @@ int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t *q, size_
     return dequant_common<int8_t>(__func__, ctx, q, n, 1.0f, 0, params, out);
 }
 
-int32_t hipq_quantize_per_row_strided_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
-                                             int32_t flavor, int32_t mode, int8_t *out, float *out_scales,
-                                             int32_t *out_zero_points, int32_t *out_status) {
-    HIPQ_ENTER(ctx);
-    int32_t rc = check_row_flavor(__func__, flavor);
+}  // extern "C"
+
+// Per-row quantize over rows `ld` apart, integer range [qmin, qmax]; `any_flavor` admits every
+// HIPQ_PARAMS_* formula (the reference's per-channel function knows two).
+static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
+                             int32_t flavor, bool any_flavor, int32_t qmin, int32_t qmax, int32_t mode, int8_t *out,
+                             float *out_scales, int32_t *out_zero_points, int32_t *out_status) {
+    int32_t rc = any_flavor ? HIPQ_SUCCESS : check_row_flavor(fn, flavor);
     if (rc) return rc;
-    if ((rc = check_mode(__func__, mode))) return rc;
+    if ((rc = check_mode(fn, mode))) return rc;
     if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
-    if (rows == 0) return check_launch(__func__);
-    if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length have no range", __func__);
-    if (ld < cols) return fail(HIPQ_INVALID_ARGUMENT, "%s: row stride %zu smaller than the row length %zu", __func__, ld, cols);
+    if (rows == 0) return check_launch(fn);
+    if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length have no range", fn);
+    if (ld < cols) return fail(HIPQ_INVALID_ARGUMENT, "%s: row stride %zu smaller than the row length %zu", fn, ld, cols);
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
     const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
-    if (rows >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many rows", __func__);
+    if (rows >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many rows", fn);
     if (cols > 1024) {
         const int grid = static_cast<int>(rows);
         if (even)
             hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
         else
             hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
     } else {
         const int grid = static_cast<int>((rows + 3) / 4);
         if (even)
             hipLaunchKernelGGL((quantize_per_row_kernel<kWave, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
         else
             hipLaunchKernelGGL((quantize_per_row_kernel<kWave, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
     }
-    return check_launch(__func__);
+    return check_launch(fn);
+}
+
+// quantize_per_channel_auto over a dense [outer, channels, inner] view with groups of `group`
+// consecutive channels sharing their parameters (1 = per channel), integer range [qmin, qmax].
+static int32_t quantize_channels(const char *fn, hipq_ctx *ctx, const float *x, size_t outer, size_t channels,
+                                 size_t inner, size_t group, int32_t flavor, bool any_flavor, int32_t qmin,
+                                 int32_t qmax, int32_t mode, int8_t *out, float *out_scales, int32_t *out_zero_points,
+                                 int32_t *out_status) {
+    if (group == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Group size must be greater than 0", fn);
+    if (outer == 1 && channels % group == 0)  // every group is one contiguous row
+        return quantize_rows(fn, ctx, x, channels / group, group * inner, group * inner, flavor, any_flavor, qmin, qmax,
+                             mode, out, out_scales, out_zero_points, out_status);
+    int32_t rc = any_flavor ? HIPQ_SUCCESS : check_row_flavor(fn, flavor);
+    if (rc) return rc;
+    if ((rc = check_mode(fn, mode))) return rc;
+    if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
+    if (channels == 0) return check_launch(fn);
+    if (outer == 0 || inner == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: channels of zero length have no range", fn);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    const size_t groups = (channels + group - 1) / group;
+    if (groups >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many channels", fn);
+    const int grid = static_cast<int>(groups);
+    if (mode & HIPQ_ROUND_HALF_EVEN)
+        hipLaunchKernelGGL((quantize_per_channel_auto_kernel<true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, outer,
+                           channels, inner, group, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
+    else
+        hipLaunchKernelGGL((quantize_per_channel_auto_kernel<false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                           outer, channels, inner, group, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                           out_status);
+    return check_launch(fn);
+}
+
+extern "C" {
+
+int32_t hipq_quantize_per_row_strided_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
+                                             int32_t flavor, int32_t mode, int8_t *out, float *out_scales,
+                                             int32_t *out_zero_points, int32_t *out_status) {
+    HIPQ_ENTER(ctx);
+    return quantize_rows(__func__, ctx, x, rows, cols, ld, flavor, false, -128, 127, mode, out, out_scales,
+                         out_zero_points, out_status);
 }
 
 int32_t hipq_quantize_per_row_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t flavor,
@@ -757,26 +805,21 @@ int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const float *x, siz
                                               size_t inner, int32_t flavor, int32_t mode, int8_t *out,
                                               float *out_scales, int32_t *out_zero_points, int32_t *out_status) {
     HIPQ_ENTER(ctx);
-    if (outer == 1)
-        return hipq_quantize_per_row_f32_i8(ctx, x, channels, inner, flavor, mode, out, out_scales, out_zero_points,
-                                            out_status);
-    int32_t rc = check_row_flavor(__func__, flavor);
-    if (rc) return rc;
-    if ((rc = check_mode(__func__, mode))) return rc;
-    if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
-    if (channels == 0) return check_launch(__func__);
-    if (outer == 0 || inner == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: channels of zero length have no range", __func__);
-    HIPQ_REQUIRE_PTR(x);
-    HIPQ_REQUIRE_PTR(out);
-    if (channels >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many channels", __func__);
-    const int grid = static_cast<int>(channels);
-    if (mode & HIPQ_ROUND_HALF_EVEN)
-        hipLaunchKernelGGL((quantize_per_channel_auto_kernel<true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, outer,
-                           channels, inner, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
-    else
-        hipLaunchKernelGGL((quantize_per_channel_auto_kernel<false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                           outer, channels, inner, flavor, -128, 127, out, out_scales, out_zero_points, out_status);
-    return check_launch(__func__);
+    return quantize_channels(__func__, ctx, x, outer, channels, inner, 1, flavor, false, -128, 127, mode, out,
+                             out_scales, out_zero_points, out_status);
+}
+
+int32_t hipq_quantize_per_group_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels,
+                                            size_t inner, size_t group_size, int32_t flavor, int32_t qmin,
+                                            int32_t qmax, int32_t mode, int8_t *out, float *out_scales,
+                                            int32_t *out_zero_points, int32_t *out_status) {
+    HIPQ_ENTER(ctx);
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", __func__, flavor);
+    if (qmin < -128 || qmax > 127 || qmin >= qmax)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: range [%d, %d] must lie inside [-128, 127]", __func__, qmin, qmax);
+    return quantize_channels(__func__, ctx, x, outer, channels, inner, group_size, flavor, true, qmin, qmax, mode, out,
+                             out_scales, out_zero_points, out_status);
 }
 
 int32_t hipq_quantize_per_channel_f32_i8(hipq_ctx *ctx, const float *x, size_t outer, size_t channels, size_t inner,

@@ -144,6 +144,7 @@ __device__ __forceinline__ float wave_max(float v) {
 //   HIPQ_PARAMS_AFFINE             crates/torsh-quantization/src/algorithms.rs:358-394
 //   HIPQ_PARAMS_BACKEND_SYMMETRIC  crates/torsh-backend/src/quantization/params.rs:323-340
 //   HIPQ_PARAMS_BACKEND_ASYMMETRIC crates/torsh-backend/src/quantization/params.rs:343-363
+//   HIPQ_PARAMS_ZERO_INCLUDED      crates/torsh-quantization/src/observers.rs:263-310, specialized.rs:39-48, 322-335
 __device__ __forceinline__ int params_from_minmax(float mn, float mx, int flavor, int qmin_i, int qmax_i,
                                                   float *scale, int *zp) {
     const bool finite = (fabsf(mn) <= FLT_MAX) && (fabsf(mx) <= FLT_MAX);  // false for NaN and Inf
@@ -186,6 +187,16 @@ __device__ __forceinline__ int params_from_minmax(float mn, float mx, int flavor
         float z = qmin - mn / s;
         *scale = s;
         *zp = f32_as_i32(clamp_keep_nan(roundf(z), qmin, qmax));
+        return HIPQ_SUCCESS;
+    }
+    case HIPQ_PARAMS_ZERO_INCLUDED: {
+        mn = fminf(mn, 0.0f);
+        mx = fmaxf(mx, 0.0f);
+        if (!((fabsf(mn) <= FLT_MAX) && (fabsf(mx) <= FLT_MAX))) return HIPQ_INVALID_ARGUMENT;
+        float s = (mx - mn) / (qmax - qmin);
+        if (s == 0.0f) s = 1.0f;
+        *scale = s;
+        *zp = f32_as_i32(fminf(fmaxf(roundf(qmin - mn / s), qmin), qmax));
         return HIPQ_SUCCESS;
     }
     default:

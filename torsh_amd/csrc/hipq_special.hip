@@ -1,0 +1,191 @@
+// Binary and ternary quantization (crates/torsh-quantization/src/specialized.rs:163-238): a sign
+// or a thresholded sign per element plus one scale for the tensor, the mean of |x| over the
+// elements that keep a sign.  One streaming pass writes the int8 codes and per-workgroup sums;
+// a one-workgroup launch folds them.  The ternary threshold needs max|x| first (one more pass).
+#include "hipq_internal.h"
+#include "hipq_math.h"
+#include "hipq_stream.h"
+
+namespace hipq {
+
+struct SignPartial {
+    double sum;                 // sum of |x| over the counted elements
+    unsigned long long count;   // counted elements
+};
+
+__device__ __forceinline__ void block_store_sign_partial(double sum, unsigned count, SignPartial *__restrict__ out) {
+    __shared__ SignPartial lds[kCalBlock / kWave];
+    SignPartial w{wave_sum(sum), wave_sum(static_cast<unsigned long long>(count))};
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) lds[wave] = w;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        SignPartial r = lds[0];
+        for (int i = 1; i < kCalBlock / kWave; ++i) {
+            r.sum += lds[i].sum;
+            r.count += lds[i].count;
+        }
+        *out = r;
+    }
+}
+
+// max|x| partial per workgroup (the fold `max(|x|)` from 0 of specialized.rs:200; NaN is ignored).
+__global__ __launch_bounds__(kCalBlock) void absmax_partial_kernel(const float *__restrict__ x, size_t n,
+                                                                    float *__restrict__ partials) {
+    float m = 0.0f;
+    stream1<kCalBlock>(
+        x, n,
+        [&](const float4 &v, size_t) {
+            m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        },
+        [&](float v, size_t) { m = fmaxf(m, fabsf(v)); });
+    __shared__ float lds[kCalBlock / kWave];
+    m = wave_max(m);
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < kCalBlock / kWave; ++i) m = fmaxf(m, lds[i]);
+        partials[blockIdx.x] = m;
+    }
+}
+
+// TERNARY false: code = x >= 0 ? 1 : -1, every element counted (specialized.rs:172-180).
+// TERNARY true:  threshold = 0.7 * max|x| folded from `absmax_partials` by every workgroup;
+//                code = |x| <= threshold ? 0 : (x > 0 ? 1 : -1); elements with |x| > threshold
+//                are counted (specialized.rs:201-227).
+template <bool TERNARY>
+__global__ __launch_bounds__(kCalBlock) void sign_quantize_kernel(const float *__restrict__ x, size_t n,
+                                                                   const float *__restrict__ absmax_partials,
+                                                                   int nparts, int8_t *__restrict__ out,
+                                                                   SignPartial *__restrict__ partials,
+                                                                   float *__restrict__ out_threshold) {
+    float threshold = 0.0f, max_abs = 0.0f;
+    if constexpr (TERNARY) {
+        __shared__ float lds[kCalBlock / kWave];
+        for (int i = threadIdx.x; i < nparts; i += kCalBlock) max_abs = fmaxf(max_abs, absmax_partials[i]);
+        max_abs = wave_max(max_abs);
+        if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = max_abs;
+        __syncthreads();
+        max_abs = lds[0];
+        for (int i = 1; i < kCalBlock / kWave; ++i) max_abs = fmaxf(max_abs, lds[i]);
+        threshold = max_abs * 0.7f;
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            out_threshold[0] = threshold;
+            out_threshold[1] = max_abs;
+        }
+    }
+    float sum4 = 0.0f;  // flushed into the f64 accumulator after every float4
+    double sum = 0.0;
+    unsigned count = 0;
+    auto code = [&](float v) {
+        const float a = fabsf(v);
+        if constexpr (TERNARY) {
+            if (a <= threshold) return 0;
+            sum4 += a;
+            ++count;
+            return v > 0.0f ? 1 : -1;
+        } else {
+            sum4 += a;
+            ++count;
+            return v >= 0.0f ? 1 : -1;
+        }
+    };
+    const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+    stream1<kCalBlock>(
+        x, n,
+        [&](const float4 &v, size_t idx) {
+            sum4 = 0.0f;
+            const int a = code(v.x), b = code(v.y), c = code(v.z), d = code(v.w);
+            sum += sum4;
+            if (out_aligned) {
+                store_stream(reinterpret_cast<uint32_t *>(out) + idx, pack4(a, b, c, d));
+            } else {
+                int8_t *o = out + idx * 4;
+                o[0] = static_cast<int8_t>(a), o[1] = static_cast<int8_t>(b);
+                o[2] = static_cast<int8_t>(c), o[3] = static_cast<int8_t>(d);
+            }
+        },
+        [&](float v, size_t i) {
+            sum4 = 0.0f;
+            out[i] = static_cast<int8_t>(code(v));
+            sum += sum4;
+        });
+    block_store_sign_partial(sum, count, partials + blockIdx.x);
+}
+
+// scale = sum / count (1 when nothing was counted, and for the binary scheme when the mean is 0).
+__global__ __launch_bounds__(kCalBlock) void sign_final_kernel(const SignPartial *__restrict__ partials, int nparts,
+                                                                int ternary, const float *__restrict__ threshold,
+                                                                hipq_qparams *__restrict__ out) {
+    double sum = 0.0;
+    unsigned long long count = 0;
+    for (int i = threadIdx.x; i < nparts; i += kCalBlock) {
+        sum += partials[i].sum;
+        count += partials[i].count;
+    }
+    __shared__ SignPartial lds[kCalBlock / kWave];
+    SignPartial w{wave_sum(sum), wave_sum(count)};
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = w;
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    SignPartial r = lds[0];
+    for (int i = 1; i < kCalBlock / kWave; ++i) {
+        r.sum += lds[i].sum;
+        r.count += lds[i].count;
+    }
+    float scale = 1.0f;
+    if (r.count > 0) {
+        scale = static_cast<float>(r.sum / static_cast<double>(r.count));
+        if (!ternary && scale == 0.0f) scale = 1.0f;  // specialized.rs:174
+    }
+    out->scale = scale;
+    out->zero_point = 0;
+    out->min_val = ternary ? threshold[0] : 0.0f;
+    out->max_val = ternary ? threshold[1] : 0.0f;
+    out->status = HIPQ_SUCCESS;
+}
+
+static int32_t sign_quantize(const char *fn, hipq_ctx *ctx, const float *x, size_t n, bool ternary, int8_t *out,
+                             hipq_qparams *out_params) {
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", fn);
+    if (!x || !out || !out_params) return fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer", fn);
+    const size_t tiles = (n + size_t(kCalTile) * 4 - 1) / (size_t(kCalTile) * 4);
+    const size_t cap = static_cast<size_t>(ctx->num_cus) * 2;
+    const int grid = static_cast<int>(tiles < cap ? tiles : cap);
+    void *scr = nullptr;
+    // header: threshold and max|x| (2 floats); then absmax partials; then sign partials
+    int32_t rc = scratch(ctx, kScratchHeader + cap * (sizeof(float) + sizeof(SignPartial)) + 64, &scr);
+    if (rc != HIPQ_SUCCESS) return rc;
+    float *threshold = reinterpret_cast<float *>(scr);
+    SignPartial *partials = reinterpret_cast<SignPartial *>(static_cast<char *>(scr) + kScratchHeader);
+    float *absmax_partials = reinterpret_cast<float *>(partials + cap);
+    if (ternary) {
+        absmax_partial_kernel<<<grid, kCalBlock, 0, ctx->stream>>>(x, n, absmax_partials);
+        if ((rc = check_launch("absmax_partial_kernel")) != HIPQ_SUCCESS) return rc;
+        sign_quantize_kernel<true><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, absmax_partials, grid, out, partials,
+                                                                          threshold);
+    } else {
+        sign_quantize_kernel<false><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, nullptr, 0, out, partials, threshold);
+    }
+    if ((rc = check_launch("sign_quantize_kernel")) != HIPQ_SUCCESS) return rc;
+    sign_final_kernel<<<1, kCalBlock, 0, ctx->stream>>>(partials, grid, ternary ? 1 : 0, threshold, out_params);
+    return check_launch("sign_final_kernel");
+}
+
+}  // namespace hipq
+
+using namespace hipq;
+
+extern "C" {
+
+int32_t hipq_quantize_binary_f32_i8(hipq_ctx *ctx, const float *x, size_t n, int8_t *out, hipq_qparams *out_params) {
+    HIPQ_ENTER(ctx);
+    return sign_quantize(__func__, ctx, x, n, false, out, out_params);
+}
+
+int32_t hipq_quantize_ternary_f32_i8(hipq_ctx *ctx, const float *x, size_t n, int8_t *out, hipq_qparams *out_params) {
+    HIPQ_ENTER(ctx);
+    return sign_quantize(__func__, ctx, x, n, true, out, out_params);
+}
+
+}  // extern "C"

@@ -20,7 +20,7 @@ SUCCESS, INVALID_ARGUMENT, SHAPE_ERROR, DIMENSION_MISMATCH, DEVICE_ERROR, ALLOCA
 ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
 FORM_MUL_INV, FORM_DIV = 0, 2
 DTYPE_I8, DTYPE_U8 = 0, 1
-PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC = range(4)
+PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC, PARAMS_ZERO_INCLUDED = range(5)
 FAKE_INT_CAST = 4
 HISTOGRAM_MAX_BINS = 16384
 
@@ -86,6 +86,9 @@ _SIGNATURES = {
     "hipq_dequantize_with_params_i8_f32": [_vp, _vp, _sz, _vp, _vp],
     "hipq_quantize_per_row_f32_i8": [_vp, _vp, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
     "hipq_quantize_per_channel_auto_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
+    "hipq_quantize_per_group_auto_f32_i8": [_vp, _vp, _sz, _sz, _sz, _sz, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
+    "hipq_quantize_binary_f32_i8": [_vp, _vp, _sz, _vp, _vp],
+    "hipq_quantize_ternary_f32_i8": [_vp, _vp, _sz, _vp, _vp],
     "hipq_quantize_per_channel_f32_i8": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _i32, _vp],
     "hipq_dequantize_per_channel_i8_f32": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp],
     "hipq_gemm_i8_i32": [_vp, _vp, _vp, _sz, _sz, _sz, _vp],
@@ -324,6 +327,29 @@ class Context:
         self.call("hipq_quantize_per_row_f32_i8", _ptr(x), rows, cols, flavor, mode, _ptr(out), _ptr(scales),
                   _ptr(zps), _ptr(status))
         return out, scales, zps, status
+
+    def quantize_per_group_auto(self, x, outer, channels, inner, group_size, flavor, qmin, qmax, mode=0):
+        """Group-wise quantize of the dense [outer, channels, inner] view of x into [qmin, qmax]; parameters per group."""
+        groups = -(-channels // group_size) if group_size > 0 else 1
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        scales = torch.empty(groups, dtype=torch.float32, device=self._dev())
+        zps = torch.empty(groups, dtype=torch.int32, device=self._dev())
+        status = torch.empty(1, dtype=torch.int32, device=self._dev())
+        self.call("hipq_quantize_per_group_auto_f32_i8", _ptr(x), outer, channels, inner, group_size, flavor, qmin,
+                  qmax, mode, _ptr(out), _ptr(scales), _ptr(zps), _ptr(status))
+        return out, scales, zps, status
+
+    def quantize_binary(self, x):
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        params = self.new_qparams()
+        self.call("hipq_quantize_binary_f32_i8", _ptr(x), x.numel(), _ptr(out), _ptr(params))
+        return out, params
+
+    def quantize_ternary(self, x):
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        params = self.new_qparams()
+        self.call("hipq_quantize_ternary_f32_i8", _ptr(x), x.numel(), _ptr(out), _ptr(params))
+        return out, params
 
     def quantize_per_channel_auto(self, x, axis, flavor=PARAMS_SYMMETRIC, mode=0):
         shape = list(x.shape)

@@ -18,8 +18,8 @@
 //   quantize_to_int8_simd             crates/torsh-quantization/src/simd_ops.rs:18,52,84,196
 //   QScheme, QuantConfig              crates/torsh-quantization/src/config.rs:31-52, 95-128, 158-409
 //
-// Schemes outside the int8/uint8 path (group-wise, int4, binary, ternary, mixed precision)
-// return NotImplemented: they stay on the reference's CPU code.
+// quantize_with_config also dispatches the special schemes (int4, binary, ternary, group-wise) to
+// specialized.hpp; mixed precision needs the reference's specialised API and is an error here too.
 #pragma once
 
 #include <cfloat>
@@ -74,6 +74,34 @@ struct QuantConfig {
         QuantConfig c;
         c.dtype = DType::U8;
         c.scheme = QScheme::PerTensorAffine;
+        return c;
+    }
+    // config.rs:173-246
+    static QuantConfig int4() {
+        QuantConfig c;
+        c.scheme = QScheme::Int4PerTensor;
+        c.qint_min = -8, c.qint_max = 7;
+        c.observer_type = ObserverType::Histogram;
+        return c;
+    }
+    static QuantConfig binary() {
+        QuantConfig c;
+        c.scheme = QScheme::Binary;
+        c.qint_min = -1, c.qint_max = 1;
+        return c;
+    }
+    static QuantConfig ternary() {
+        QuantConfig c;
+        c.scheme = QScheme::Ternary;
+        c.qint_min = -1, c.qint_max = 1;
+        return c;
+    }
+    static QuantConfig group_wise(size_t ch_axis, size_t group_size) {
+        QuantConfig c;
+        c.scheme = QScheme::GroupWise;
+        c.ch_axis = ch_axis;
+        c.group_size = group_size;
+        c.observer_type = ObserverType::Histogram;
         return c;
     }
     static QuantConfig per_channel(size_t axis) {
@@ -403,6 +431,14 @@ inline Result<PerChannelTriple> quantize_per_channel_auto(const Tensor &tensor, 
     return PerChannelTriple{std::move(t), std::move(scales), std::move(zps)};
 }
 
+// specialized.hpp (included below)
+inline Result<QuantizedTriple> quantize_int4_per_tensor(const Tensor &tensor, const QuantConfig &config);
+inline Result<QuantizedTriple> quantize_int4_per_channel(const Tensor &tensor, size_t axis, const QuantConfig &config);
+inline Result<QuantizedTriple> quantize_binary(const Tensor &tensor);
+inline Result<QuantizedTriple> quantize_ternary(const Tensor &tensor);
+inline Result<QuantizedTriple> quantize_group_wise(const Tensor &tensor, size_t axis, size_t group_size,
+                                                   const QuantConfig &config);
+
 // algorithms.rs:30-66
 inline Result<QuantizedTriple> quantize_with_config(const Tensor &tensor, const QuantConfig &config) {
     TORSH_CHECK(config.validate());
@@ -418,11 +454,16 @@ inline Result<QuantizedTriple> quantize_with_config(const Tensor &tensor, const 
         const int32_t z0 = std::get<2>(r).empty() ? 0 : std::get<2>(r)[0];
         return QuantizedTriple{std::move(std::get<0>(r)), s0, z0};
     }
+    case QScheme::GroupWise:
+        return quantize_group_wise(tensor, config.ch_axis.value_or(0), config.group_size.value_or(32), config);
+    case QScheme::Int4PerTensor: return quantize_int4_per_tensor(tensor, config);
+    case QScheme::Int4PerChannel: return quantize_int4_per_channel(tensor, config.ch_axis.value_or(0), config);
+    case QScheme::Binary: return quantize_binary(tensor);
+    case QScheme::Ternary: return quantize_ternary(tensor);
     case QScheme::MixedPrecision:
         return TorshError::invalid_argument("Mixed precision quantization requires specialized API");
-    default:
-        return TorshError::not_implemented("scheme is outside the int8 HIP path; use the CPU implementation");
     }
+    return TorshError::invalid_argument("unknown quantization scheme");
 }
 
 inline Result<QuantizedTriple> quantize_auto(const Tensor &tensor, const QuantConfig &config) {
@@ -431,3 +472,5 @@ inline Result<QuantizedTriple> quantize_auto(const Tensor &tensor, const QuantCo
 
 }  // namespace quantization
 }  // namespace torsh
+
+#include "specialized.hpp"
