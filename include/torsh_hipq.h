@@ -328,6 +328,24 @@ HIPQ_API int32_t hipq_gelu_tanh_quantize_f32_i8(hipq_ctx *ctx, const float *x, s
 /* out = a + b (skip connection; Tensor::add). */
 HIPQ_API int32_t hipq_add_f32(hipq_ctx *ctx, const float *a, const float *b, size_t n, float *out);
 
+/* ---- quantized elementwise operators of the backend trait --------------- */
+/* CpuQuantizationOps::qadd, crates/torsh-backend/src/quantization/ops.rs:582-606:
+ * out = quantize(dequantize(a) + dequantize(b)) with output parameters derived
+ * from the range of the f32 sum by from_statistics (params.rs:282-363; `flavor`
+ * = HIPQ_PARAMS_BACKEND_SYMMETRIC or _ASYMMETRIC for the scheme of `a`).
+ * Operands are per-tensor quantized bytes; *_signed says the bytes are
+ * two's-complement int8 (tensor.rs:103-143).  out_dtype: HIPQ_DTYPE_I8 / _U8
+ * (the dtype of `a` in the reference).  out_params is a device record holding
+ * the derived scale, zero point and range.  The f32 intermediate is never
+ * stored: 5 bytes of traffic per element. */
+HIPQ_API int32_t hipq_qadd_u8(hipq_ctx *ctx, const uint8_t *a, int32_t a_signed, float a_scale, int32_t a_zero_point,
+                              const uint8_t *b, int32_t b_signed, float b_scale, int32_t b_zero_point, size_t n,
+                              int32_t flavor, int32_t out_dtype, uint8_t *out, hipq_qparams *out_params);
+/* CpuQuantizationOps::qrelu, ops.rs:608-624: out = quantize(max(dequantize(q), 0))
+ * with parameters from_statistics(0, max(max_val, 0)).  3 bytes per element. */
+HIPQ_API int32_t hipq_qrelu_u8(hipq_ctx *ctx, const uint8_t *q, int32_t is_signed, float scale, int32_t zero_point,
+                               size_t n, int32_t flavor, int32_t out_dtype, uint8_t *out, hipq_qparams *out_params);
+
 /* ---- calibration observers and quality metrics ------------------------ */
 /* Extra `mode` bit of the fake-quantizing entry points: the clamped value goes
  * through `as i32` before it is dequantized (NaN becomes 0), as

@@ -625,3 +625,27 @@ def quantize_group_wise(x, axis, group_size, qmin=-128, qmax=127):
     _check(lib().tq_quantize_group_wise(_p(x, _f32p), _shape(x), x.ndim, axis, group_size, qmin, qmax, _p(out, _f32p),
                                         _p(scales, _f32p), _p(zps, _i32p), C.byref(s), C.byref(z)), "quantize_group_wise")
     return out, scales, zps, np.float32(s.value), z.value
+
+
+def backend_qadd(a, a_scale, a_zp, b, b_scale, b_zp, symmetric=False):
+    """CpuQuantizationOps::qadd on int8 / uint8 arrays -> (bytes with a's dtype, scale, zero_point)."""
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    qmin, qmax = (-128, 127) if a.dtype == np.int8 else (0, 255)
+    out = np.empty(a.shape, np.uint8)
+    s, z = C.c_float(), C.c_int32()
+    _check(lib().tq_backend_qadd_or_qrelu(a.ctypes.data_as(_u8p), int(a.dtype == np.int8), C.c_float(a_scale), int(a_zp),
+                                          b.ctypes.data_as(_u8p), int(b.dtype == np.int8), C.c_float(b_scale), int(b_zp),
+                                          C.c_size_t(a.size), int(symmetric), qmin, qmax, _p(out, _u8p), C.byref(s),
+                                          C.byref(z)), "qadd")
+    return out.view(a.dtype), np.float32(s.value), z.value
+
+
+def backend_qrelu(q, scale, zp, symmetric=False):
+    q = np.ascontiguousarray(q)
+    qmin, qmax = (-128, 127) if q.dtype == np.int8 else (0, 255)
+    out = np.empty(q.shape, np.uint8)
+    s, z = C.c_float(), C.c_int32()
+    _check(lib().tq_backend_qadd_or_qrelu(q.ctypes.data_as(_u8p), int(q.dtype == np.int8), C.c_float(scale), int(zp),
+                                          None, 0, C.c_float(1.0), 0, C.c_size_t(q.size), int(symmetric), qmin, qmax,
+                                          _p(out, _u8p), C.byref(s), C.byref(z)), "qrelu")
+    return out.view(q.dtype), np.float32(s.value), z.value

@@ -474,6 +474,38 @@ int tq_backend_dequantize_f32(const uint8_t *q, size_t n, const float *scales, c
     return TQ_OK;
 }
 
+/* crates/torsh-backend/src/quantization/ops.rs:582-606 (qadd) and :608-624 (qrelu) */
+int tq_backend_qadd_or_qrelu(const uint8_t *a, int a_signed, float a_scale, int32_t a_zp, const uint8_t *b,
+                             int b_signed, float b_scale, int32_t b_zp, size_t n, int symmetric, int32_t qmin,
+                             int32_t qmax, uint8_t *out, float *out_scale, int32_t *out_zp) {
+    float *f = (float *)malloc((n ? n : 1) * sizeof(float));
+    float *g = (float *)malloc((n ? n : 1) * sizeof(float));
+    if (!f || !g) {
+        free(f);
+        free(g);
+        return TQ_ERR_INVALID_ARGUMENT;
+    }
+    tq_backend_dequantize_f32(a, n, &a_scale, &a_zp, 1, a_signed, f);
+    float mn = INFINITY, mx = -INFINITY;
+    if (b) {
+        tq_backend_dequantize_f32(b, n, &b_scale, &b_zp, 1, b_signed, g);
+        for (size_t i = 0; i < n; ++i) f[i] = f[i] + g[i];
+        for (size_t i = 0; i < n; ++i) mn = fminf(mn, f[i]);
+        for (size_t i = 0; i < n; ++i) mx = fmaxf(mx, f[i]);
+    } else {
+        for (size_t i = 0; i < n; ++i) f[i] = fmaxf(f[i], 0.0f);
+        for (size_t i = 0; i < n; ++i) mx = fmaxf(mx, f[i]);
+        mn = 0.0f;
+        mx = fmaxf(mx, 0.0f);
+    }
+    int rc = symmetric ? tq_backend_params_symmetric(mn, mx, qmin, qmax, out_scale, out_zp)
+                       : tq_backend_params_asymmetric(mn, mx, qmin, qmax, out_scale, out_zp);
+    if (rc == TQ_OK) rc = tq_backend_quantize_f32(f, n, out_scale, out_zp, 1, qmin, qmax, out);
+    free(f);
+    free(g);
+    return rc;
+}
+
 /* crates/torsh-backend/src/quantization/specialized.rs:175-201: A [M,K] bytes
  * read as i8, B [K,N] row-major bytes read as i8, i32 accumulate in k order;
  * the reference then stores clamp(acc,-128,127) as a byte.  Both are returned

@@ -91,6 +91,13 @@ int tq_backend_conv2d_i32(const uint8_t *x, int x_signed, int32_t zp_in, const i
                           size_t c_in, size_t h, size_t wd, size_t c_out, size_t kh, size_t kw,
                           size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, int32_t *acc_out);
 
+/* CpuQuantizationOps::qadd / qrelu, crates/torsh-backend/src/quantization/ops.rs:582-624: dequantize,
+ * operate in f32, from_statistics on the result's range (symmetric != 0 selects the Symmetric
+ * formula, else the Asymmetric one), quantize into [qmin, qmax].  b == NULL means qrelu. */
+int tq_backend_qadd_or_qrelu(const uint8_t *a, int a_signed, float a_scale, int32_t a_zp, const uint8_t *b,
+                             int b_signed, float b_scale, int32_t b_zp, size_t n, int symmetric, int32_t qmin,
+                             int32_t qmax, uint8_t *out, float *out_scale, int32_t *out_zp);
+
 /* ---- compositions the device path is checked against ------------------ */
 int tq_gemm_i8_nk(const int8_t *a, const int8_t *w_nk, size_t m, size_t n, size_t k, int32_t *acc);
 int tq_linear_dequant_epilogue(const int32_t *acc, size_t m, size_t n, const float *sa, int sa_per_row,

@@ -253,7 +253,7 @@ CPU_TEST(test_backend_params_and_tensor) {  // params.rs / tensor.rs tests
     CHECK(ops.calibrate({}, bq::QuantizedDType::UInt8).is_err());
     CHECK(ops.quantize_f32({}, bq::QuantizationParams::int8_symmetric()).unwrap().empty());
     CHECK(ops.quantize_f32({1.0f}, bad).is_err());
-    CHECK(ops.qadd(a, a).unwrap_err().kind == TorshError::NotImplemented);
+    CHECK(ops.qadd(a, b).unwrap_err().kind == TorshError::InvalidArgument);  // shape mismatch, before the device
 }
 
 CPU_TEST(test_module_shapes_before_the_device) {
@@ -1133,6 +1133,58 @@ GPU_TEST(parity_special_schemes) {
     CHECK_EQ(tq_quantize_group_wise(x.data(), dims.data(), 3, 0, 4, qmin, qmax, want.data(), gs.data(), gz.data(), &s, &z), 0);
     CHECK(scale == s && zp == z);
     check_same(q.as_slice(), want, __LINE__);
+}
+
+
+GPU_TEST(parity_backend_qadd_qrelu) {  // crates/torsh-backend/src/quantization/ops.rs:582-624
+    bq::HipQuantizationOps ops;
+    std::mt19937 g(91);
+    std::uniform_int_distribution<int> byte(0, 255);
+    for (auto dtype : {bq::QuantizedDType::Int8, bq::QuantizedDType::UInt8}) {
+        for (auto scheme : {bq::QuantizationScheme::Asymmetric, bq::QuantizationScheme::Symmetric}) {
+            const size_t n = 70001;
+            std::vector<uint8_t> a(n), b(n);
+            for (auto &v : a) v = static_cast<uint8_t>(byte(g));
+            for (auto &v : b) v = static_cast<uint8_t>(byte(g));
+            bq::QuantizationParams pa, pb;
+            pa.dtype = pb.dtype = dtype;
+            pa.scheme = pb.scheme = scheme;
+            const bool is_signed = dtype == bq::QuantizedDType::Int8;
+            const bool sym = scheme == bq::QuantizationScheme::Symmetric;  // validate() demands zero point 0 then
+            pa.scale = {0.0173f}, pa.zero_point = {sym ? 0 : (is_signed ? -7 : 121)};
+            pb.scale = {0.0419f}, pb.zero_point = {sym ? 0 : (is_signed ? 12 : 99)};
+            const auto ta = bq::QuantizedTensor::from_data(a, {n}, pa).unwrap();
+            const auto tb = bq::QuantizedTensor::from_data(b, {n}, pb).unwrap();
+            const int32_t qmin = is_signed ? -128 : 0, qmax = is_signed ? 127 : 255;
+            std::vector<uint8_t> want(n);
+            float s;
+            int32_t z;
+            const auto sum = ops.qadd(ta, tb).unwrap();
+            CHECK_EQ(tq_backend_qadd_or_qrelu(a.data(), is_signed, pa.scale[0], pa.zero_point[0], b.data(), is_signed,
+                                              pb.scale[0], pb.zero_point[0], n, scheme == bq::QuantizationScheme::Symmetric,
+                                              qmin, qmax, want.data(), &s, &z), 0);
+            CHECK(sum.params.scale[0] == s && sum.params.zero_point[0] == z && sum.params.dtype == dtype);
+            check_same(sum.data, want, __LINE__);
+            const auto relu = ops.qrelu(ta).unwrap();
+            CHECK_EQ(tq_backend_qadd_or_qrelu(a.data(), is_signed, pa.scale[0], pa.zero_point[0], nullptr, 0, 1.0f, 0, n,
+                                              scheme == bq::QuantizationScheme::Symmetric, qmin, qmax, want.data(), &s, &z), 0);
+            CHECK(relu.params.scale[0] == s && relu.params.zero_point[0] == z);
+            check_same(relu.data, want, __LINE__);
+            CHECK(relu.params.min_val.value_or(-1.0f) == 0.0f);
+        }
+    }
+    // shape mismatch and unsupported operands
+    bq::QuantizationParams p;
+    p.dtype = bq::QuantizedDType::Int8;
+    p.scale = {0.1f}, p.zero_point = {0};
+    const auto t4 = bq::QuantizedTensor::from_data({1, 2, 3, 4}, {4}, p).unwrap();
+    const auto t22 = bq::QuantizedTensor::from_data({1, 2, 3, 4}, {2, 2}, p).unwrap();
+    CHECK(ops.qadd(t4, t22).is_err() && ops.qadd(t4, t22).unwrap_err().kind == TorshError::InvalidArgument);
+    // ReLU of an all-negative tensor: range (0, 0) -> asymmetric degenerate parameters (1.0, qmin)
+    const auto neg = bq::QuantizedTensor::from_data({0xF6, 0xEC}, {2}, p).unwrap();  // -10, -20
+    const auto r = ops.qrelu(neg).unwrap();
+    CHECK(r.params.scale[0] == 1.0f && r.params.zero_point[0] == -128);
+    CHECK(r.data[0] == 0x80 && r.data[1] == 0x80);
 }
 
 }  // namespace

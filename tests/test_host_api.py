@@ -50,6 +50,7 @@ GPU_CASES = [
     "test_quantized_modules_survive_a_weight_file",
     "test_special_schemes",
     "parity_special_schemes",
+    "parity_backend_qadd_qrelu",
 ]
 
 

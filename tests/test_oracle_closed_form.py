@@ -287,3 +287,22 @@ def test_determinism(oracle):
     b = oracle.quantize_tensor_auto(x, 0, oracle.PER_TENSOR_SYMMETRIC)
     np.testing.assert_array_equal(a[0], b[0])
     assert a[1:] == b[1:]
+
+
+def test_backend_qadd_qrelu_closed_form(oracle):
+    # bytes 10, 20, -30, 40 at scale 0.1 are 1, 2, -3, 4; bytes 1..4 at scale 0.5 are 0.5 .. 2.
+    a, b = np.int8([10, 20, -30, 40]), np.int8([1, 2, 3, 4])
+    out, s, z = oracle.backend_qadd(a, 0.1, 0, b, 0.5, 0)
+    # sum = [1.5, 3, -1.5, 6]: scale = 7.5 / 255, zero point = round(-128 + 1.5 / scale) = round(-77) = -77
+    assert s == np.float32(7.5) / np.float32(255.0) and z == -77
+    np.testing.assert_array_equal(out, [-26, 25, -128, 127])
+    # qrelu: [1, 2, 0, 4] with range (0, 4): scale 4 / 255, zero point -128
+    out, s, z = oracle.backend_qrelu(a, 0.1, 0)
+    assert s == np.float32(4.0) / np.float32(255.0) and z == -128
+    np.testing.assert_array_equal(out, [-64, -1, -128, 127])       # round(63.75) - 128, round(127.5) - 128
+    # symmetric scheme: scale = 2 * max|v| / 255, zero point 0
+    out, s, z = oracle.backend_qadd(a, 0.1, 0, b, 0.5, 0, symmetric=True)
+    assert s == np.float32(12.0) / np.float32(255.0) and z == 0
+    # uint8 storage with a zero point, all-negative input to relu -> degenerate range (0, 0) -> (1.0, qmin)
+    out, s, z = oracle.backend_qrelu(np.uint8([0, 50, 100]), 0.02, 128)
+    assert (s, z) == (1.0, 0) and (out == 0).all()

@@ -104,6 +104,8 @@ _SIGNATURES = {
     "hipq_gelu_tanh_quantize_f32_i8": [_vp, _vp, _sz, _sz, _i32, _vp, _vp],
     "hipq_add_f32": [_vp, _vp, _vp, _sz, _vp],
     "hipq_transformer_stack_forward_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
+    "hipq_qadd_u8": [_vp, _vp, _i32, _f32, _i32, _vp, _i32, _f32, _i32, _sz, _i32, _i32, _vp, _vp],
+    "hipq_qrelu_u8": [_vp, _vp, _i32, _f32, _i32, _sz, _i32, _i32, _vp, _vp],
     "hipq_quantization_metrics_f32": [_vp, _vp, _vp, _sz, C.c_uint32, C.c_uint32, _vp],
     "hipq_fake_quantize_metrics_f32": [_vp, _vp, _sz, _f32, _i32, _vp, _i32, _i32, _i32, C.c_uint32, C.c_uint32, _vp],
     "hipq_fake_quantize_f32": [_vp, _vp, _sz, _f32, _i32, _vp, _i32, _i32, _i32, _vp],
@@ -233,6 +235,23 @@ class Context:
         out = self.new_qparams()
         self.call("hipq_qparams_from_minmax", _ptr(minmax), flavor, qmin, qmax, _ptr(out))
         return out
+
+    # ---- quantized elementwise operators ---------------------------------------------
+    def qadd(self, a, a_scale, a_zp, b, b_scale, b_zp, flavor=PARAMS_BACKEND_ASYMMETRIC):
+        """a, b: int8 or uint8 tensors (per-tensor parameters); output has a's dtype.  -> (out, params record)"""
+        out = torch.empty(a.shape, dtype=a.dtype, device=self._dev())
+        params = self.new_qparams()
+        self.call("hipq_qadd_u8", _ptr(a), int(a.dtype == torch.int8), float(a_scale), int(a_zp), _ptr(b),
+                  int(b.dtype == torch.int8), float(b_scale), int(b_zp), a.numel(), flavor,
+                  DTYPE_I8 if a.dtype == torch.int8 else DTYPE_U8, _ptr(out), _ptr(params))
+        return out, params
+
+    def qrelu(self, q, scale, zp, flavor=PARAMS_BACKEND_ASYMMETRIC):
+        out = torch.empty(q.shape, dtype=q.dtype, device=self._dev())
+        params = self.new_qparams()
+        self.call("hipq_qrelu_u8", _ptr(q), int(q.dtype == torch.int8), float(scale), int(zp), q.numel(), flavor,
+                  DTYPE_I8 if q.dtype == torch.int8 else DTYPE_U8, _ptr(out), _ptr(params))
+        return out, params
 
     # ---- calibration observers and quality metrics --------------------------------
     def _record(self, ty):

@@ -9,9 +9,9 @@
 //   CpuQuantizationOps (what each method computes)  ops.rs:185-200, 295-660
 //   VnniQuantizationOps::vnni_qmatmul_int8          crates/torsh-backend/src/quantization/specialized.rs:82-201
 //
-// HipQuantizationOps covers Int8 and UInt8.  Sub-byte and 16-bit types return NotImplemented
-// (they stay on the CPU implementation), and so do qadd / qrelu, which are not on the
-// Linear / Conv2d forward path.
+// HipQuantizationOps covers Int8 and UInt8 with per-tensor parameters for every method of the
+// trait; sub-byte and 16-bit types, logarithmic parameters and channel-wise operands of qadd /
+// qrelu return NotImplemented (they stay on the CPU implementation).
 #pragma once
 
 #include <cmath>
@@ -384,11 +384,15 @@ class HipQuantizationOps : public QuantizationOps {
         return requantize_from_range(ctx, dout, out_n, {nb, oc, ho, wo}, input.params);
     }
 
-    BackendResult<QuantizedTensor> qadd(const QuantizedTensor &, const QuantizedTensor &) const override {
-        return TorshError::not_implemented("qadd is not on the quantized Linear/Conv2d path; use CpuQuantizationOps");
+    // ops.rs:582-606.  The f32 sum is formed twice from the bytes (once for its range, once to
+    // quantize it) and never stored.
+    BackendResult<QuantizedTensor> qadd(const QuantizedTensor &a, const QuantizedTensor &b) const override {
+        if (a.shape != b.shape) return TorshError::invalid_argument("qadd shape mismatch");
+        return elementwise(a, &b);
     }
-    BackendResult<QuantizedTensor> qrelu(const QuantizedTensor &) const override {
-        return TorshError::not_implemented("qrelu is not on the quantized Linear/Conv2d path; use CpuQuantizationOps");
+    // ops.rs:608-624
+    BackendResult<QuantizedTensor> qrelu(const QuantizedTensor &input) const override {
+        return elementwise(input, nullptr);
     }
 
     // ops.rs:616-660: global range over all samples, then asymmetric parameters.  The reference
@@ -418,6 +422,56 @@ class HipQuantizationOps : public QuantizationOps {
     }
 
   private:
+    // qadd (b != nullptr) / qrelu on per-tensor Int8 / UInt8 operands.
+    static BackendResult<QuantizedTensor> elementwise(const QuantizedTensor &a, const QuantizedTensor *b) {
+        auto supported = [](const QuantizationParams &p) {
+            return (p.dtype == QuantizedDType::Int8 || p.dtype == QuantizedDType::UInt8) && p.scale.size() == 1 &&
+                   p.zero_point.size() == 1;
+        };
+        TORSH_CHECK(a.params.validate());
+        if (b) TORSH_CHECK(b->params.validate());
+        if (!supported(a.params) || (b && !supported(b->params)))
+            return TorshError::not_implemented("qadd / qrelu on the HIP path take per-tensor Int8 or UInt8 operands");
+        if (a.params.scheme == QuantizationScheme::Logarithmic)
+            return TorshError::not_implemented("logarithmic quantization is outside the int8 HIP path");
+        const size_t n = a.data.size();
+        if (b && b->data.size() != n) return TorshError::invalid_argument("qadd shape mismatch");
+        // An empty tensor has range (+inf, -inf), which from_statistics rejects (params.rs:283-297).
+        if (n == 0) return TorshError::invalid_argument("min_val must be <= max_val");
+        TORSH_TRY(ctx, hip::Runtime::ctx());
+        TORSH_TRY(da, hip::DeviceBuffer::from_host(ctx, a.data.data(), n));
+        hip::DeviceBuffer db;
+        if (b) {
+            TORSH_TRY(tmp, hip::DeviceBuffer::from_host(ctx, b->data.data(), n));
+            db = std::move(tmp);
+        }
+        TORSH_TRY(dout, hip::DeviceBuffer::alloc(ctx, n));
+        TORSH_TRY(dp, hip::DeviceBuffer::alloc(ctx, sizeof(hipq_qparams)));
+        const int32_t flavor = a.params.scheme == QuantizationScheme::Symmetric ? HIPQ_PARAMS_BACKEND_SYMMETRIC
+                                                                               : HIPQ_PARAMS_BACKEND_ASYMMETRIC;
+        const int32_t out_dtype = a.params.dtype == QuantizedDType::Int8 ? HIPQ_DTYPE_I8 : HIPQ_DTYPE_U8;
+        const int32_t a_signed = a.params.dtype == QuantizedDType::Int8;
+        if (b)
+            TORSH_CHECK(hip::check(hipq_qadd_u8(ctx, da.as<uint8_t>(), a_signed, a.params.scale[0],
+                                                a.params.zero_point[0], db.as<uint8_t>(),
+                                                b->params.dtype == QuantizedDType::Int8, b->params.scale[0],
+                                                b->params.zero_point[0], n, flavor, out_dtype, dout.as<uint8_t>(),
+                                                dp.as<hipq_qparams>())));
+        else
+            TORSH_CHECK(hip::check(hipq_qrelu_u8(ctx, da.as<uint8_t>(), a_signed, a.params.scale[0],
+                                                 a.params.zero_point[0], n, flavor, out_dtype, dout.as<uint8_t>(),
+                                                 dp.as<hipq_qparams>())));
+        TORSH_TRY(p, dp.to_host<hipq_qparams>(1));
+        if (p[0].status != HIPQ_SUCCESS) return TorshError::invalid_argument("min_val and max_val must be finite");
+        QuantizationParams out_params = a.params;
+        out_params.scale[0] = p[0].scale;
+        out_params.zero_point[0] = p[0].zero_point;
+        out_params.min_val = p[0].min_val;
+        out_params.max_val = p[0].max_val;
+        TORSH_TRY(bytes, dout.to_host<uint8_t>(n));
+        return QuantizedTensor::from_data(std::move(bytes), a.shape, std::move(out_params));
+    }
+
     static std::vector<uint8_t> transpose_kn(const std::vector<uint8_t> &b, size_t k, size_t n) {
         std::vector<uint8_t> t(b.size());
         for (size_t l = 0; l < k; ++l)
