@@ -15,6 +15,7 @@
 
 #include "torsh_hipq/backend.hpp"
 #include "torsh_hipq/calibration.hpp"
+#include "torsh_hipq/hardware.hpp"
 #include "torsh_hipq/models.hpp"
 #include "torsh_hipq/nn.hpp"
 #include "torsh_hipq/quantization.hpp"
@@ -1185,6 +1186,36 @@ GPU_TEST(parity_backend_qadd_qrelu) {  // crates/torsh-backend/src/quantization/
     const auto r = ops.qrelu(neg).unwrap();
     CHECK(r.params.scale[0] == 1.0f && r.params.zero_point[0] == -128);
     CHECK(r.data[0] == 0x80 && r.data[1] == 0x80);
+}
+
+
+CPU_TEST(test_kernel_plugin_interface) {  // hardware.rs:213-241, 482-555
+    const HardwareQuantizer hq = HardwareQuantizer::with_hip();
+    CHECK(hq.backend == HardwareBackend::make_custom("rocm-gfx950"));
+    CHECK_EQ(hq.kernel_dispatch.size(), size_t(4));
+    const QuantizationKernel &k = *hq.kernel_dispatch.at(QScheme::PerTensorAffine);
+    CHECK(std::string(k.name()) == "HIP-gfx950");
+    CHECK(k.supported_backends().size() == 1 && k.supported_backends()[0].kind == HardwareBackend::Custom);
+    CHECK(k.performance_characteristics().throughput > GenericKernel{}.performance_characteristics().throughput);
+    CHECK_EQ(hq.get_performance_info().size(), size_t(4));
+    // errors surface through the plug-in unchanged
+    CHECK(hq.quantize(tensor_1d({}).unwrap(), QuantConfig::int8()).is_err());
+    CHECK(hq.dequantize(tensor_1d({1.f}).unwrap(), 0.0f, 0).is_err());
+}
+
+GPU_TEST(test_kernel_plugin_dispatch) {
+    const HardwareQuantizer hq = HardwareQuantizer::with_hip();
+    const std::vector<float> x = normal(5000, 77, 2.0f);
+    const Tensor t = tensor_1d(x).unwrap();
+    for (const QuantConfig &cfg : {QuantConfig::int8(), QuantConfig::int8().with_scheme(QScheme::PerTensorSymmetric),
+                                   QuantConfig::int4() /* no registered kernel: generic fallback */}) {
+        const auto [q, s, z] = hq.quantize(t, cfg).unwrap();
+        const auto [q2, s2, z2] = quantize_with_config(t, cfg).unwrap();
+        CHECK(s == s2 && z == z2);
+        check_same(q.as_slice(), q2.as_slice(), __LINE__);
+        const Tensor back = hq.dequantize(q, s, z).unwrap();
+        check_same(back.as_slice(), dequantize(q2, s2, z2).unwrap().as_slice(), __LINE__);
+    }
 }
 
 }  // namespace

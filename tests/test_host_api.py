@@ -24,6 +24,7 @@ CPU_CASES = [
     "test_config_json_round_trip",
     "test_weight_file_round_trip_and_corruption",
     "test_model_quantizer_scalar_logic",
+    "test_kernel_plugin_interface",
 ]
 GPU_CASES = [
     "test_quantize_per_tensor_affine",
@@ -51,6 +52,7 @@ GPU_CASES = [
     "test_special_schemes",
     "parity_special_schemes",
     "parity_backend_qadd_qrelu",
+    "test_kernel_plugin_dispatch",
 ]
 
 
