@@ -55,3 +55,21 @@ def test_no_silent_fallback_when_library_missing(monkeypatch):
     monkeypatch.setattr(hipq, "_LIB_PATH", "/nonexistent/libtorsh_hipq.so")
     with pytest.raises(FileNotFoundError):
         hipq.load()
+
+
+def test_generated_rust_declarations_are_in_sync_with_the_header():
+    """include/torsh_hipq_sys.rs (the extern "C" block for a torsh-hipq-sys crate) is generated from the header."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("gen_rust_bindings", os.path.join(ROOT, "include", "gen_rust_bindings.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    text = gen.generate()
+    assert open(os.path.join(ROOT, "include", "torsh_hipq_sys.rs")).read() == text, \
+        "run `python include/gen_rust_bindings.py` after changing include/torsh_hipq.h"
+    declared = re.findall(r"pub fn (hipq_\w+)\(", text)
+    assert sorted(declared) == _declared_symbols()
+    # spot checks of the type mapping
+    assert "pub fn hipq_ctx_create(device: i32, out_ctx: *mut *mut hipq_ctx) -> i32;" in text
+    assert "pub fn hipq_version() -> *const c_char;" in text
+    assert "pub nonfinite: u64," in text and "pub reserved: [i32; 3]," in text
