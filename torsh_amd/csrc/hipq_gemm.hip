@@ -278,9 +278,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_i8_generic_kernel(const int
 template <int BM, int BN, int WM, int WN, int EPI, bool EVEN>
 static void launch_tile(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, int N, int K,
                         const GemmEpilogue &ep) {
-    const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    hipLaunchKernelGGL((gemm_i8_mfma_kernel<BM, BN, WM, WN, EPI, EVEN>), dim3(tiles), dim3(kGemmThreads), 0,
-                       ctx->stream, a, w, M, N, K, ep);
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    GemmEpilogue placed = ep;
+    pick_xcd_rectangle(tiles_m, tiles_n, BM, BN, &placed.xcd_gm, &placed.xcd_gn);
+    hipLaunchKernelGGL((gemm_i8_mfma_kernel<BM, BN, WM, WN, EPI, EVEN>), dim3(tiles_m * tiles_n), dim3(kGemmThreads), 0,
+                       ctx->stream, a, w, M, N, K, placed);
 }
 
 // Tuning hook: HIPQ_GEMM_VARIANT=<n> forces one kernel configuration (0 = automatic).

@@ -32,6 +32,9 @@ struct GemmEpilogue {
     int cv_corr_mul = 0;               // 128 - zp_in: accumulator += cv_corr_mul * cv_wsum[oc]
     float sa_scalar = 1.0f;            // activation scale used when sa is null
     float s_out_inv = 0.0f;            // recip_for_div(s_out), or 0 to divide directly (requantize only)
+    // Tiles per XCD along M and N (pipelined kernel): the 8 XCDs each take a gm x gn rectangle of
+    // tiles.  0 = not set (plain id order).
+    int xcd_gm = 0, xcd_gn = 0;
 };
 
 // Host-side twin of recip_for_div: the correctly rounded 1/b if it is a normal number, else 0.
@@ -92,15 +95,45 @@ __device__ __forceinline__ void epilogue_store4(const GemmEpilogue &ep, int m, i
     }
 }
 
-// Maps the linear workgroup id to a tile so that the workgroups one XCD receives
-// (ids congruent modulo 8) cover a contiguous band of weight panels: a panel of
-// W is then pulled from HBM into one XCD's L2 only.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) {
-    const int nblk = tiles_m * tiles_n;
-    int b = blockIdx.x;
-    if (nblk % 8 == 0) b = (b % 8) * (nblk / 8) + b / 8;
+// Maps the linear workgroup id to a tile.  Workgroups are handed to the 8 XCDs round robin (ids
+// congruent modulo 8 share an XCD and its L2), so XCD x is given a gm x gn rectangle of tiles:
+// it then pulls gm row blocks of the first operand and gn panels of the second through its L2
+// once each.  The host picks the rectangle with the smallest gm*BM + gn*BN (for M = 512,
+// N = 4096: all 4 row blocks x 8 weight panels, each weight panel read from HBM by one XCD only;
+// for a tall M x 256 product: 8 row blocks x all 4 panels, instead of every XCD streaming half
+// of the tall operand).
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int gm, int gn, int *tm, int *tn) {
+    const int b = blockIdx.x;
+    if (gm > 0) {
+        const int x = b % 8, i = b / 8;     // XCD, index within the XCD's rectangle
+        const int blocks_m = tiles_m / gm;  // rectangles along M
+        *tm = (x % blocks_m) * gm + i % gm;
+        *tn = (x / blocks_m) * gn + i / gm;
+        return;
+    }
     *tm = b % tiles_m;
     *tn = b / tiles_m;
+}
+
+// Host side: the rectangle for tile_of_block, or (0, 0) when the tile grid does not split into 8
+// equal rectangles.
+static inline void pick_xcd_rectangle(int tiles_m, int tiles_n, int bm, int bn, int *gm_out, int *gn_out) {
+    *gm_out = *gn_out = 0;
+    const long nblk = static_cast<long>(tiles_m) * tiles_n;
+    if (nblk % 8 != 0) return;
+    const long per = nblk / 8;
+    long best = -1;
+    for (int gm = 1; gm <= tiles_m; ++gm) {
+        if (tiles_m % gm != 0 || per % gm != 0) continue;
+        const long gn = per / gm;
+        if (gn > tiles_n || tiles_n % gn != 0) continue;
+        const long cost = static_cast<long>(gm) * bm + gn * bn;
+        if (best < 0 || cost < best) {
+            best = cost;
+            *gm_out = gm;
+            *gn_out = static_cast<int>(gn);
+        }
+    }
 }
 
 // BM x BN output tile per workgroup, BK = 128 bytes of K per stage, WM x WN
@@ -123,7 +156,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_i8_mfma_kernel(const int8_t
     __shared__ __attribute__((aligned(16))) int8_t lds[2 * STAGE];
 
     int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, ep.xcd_gm, ep.xcd_gn, &tile_m, &tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int wm = wave % WM, wn = wave / WM;
@@ -303,7 +336,7 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     extern __shared__ __attribute__((aligned(1024))) int8_t lds[];
 
     int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, ep.xcd_gm, ep.xcd_gn, &tile_m, &tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int nk = K / BK;
@@ -522,6 +555,24 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
             out_base[j] = (size_t(img) * ep.cv_oc * ep.cv_ho + oh) * ep.cv_wo + ow;  // + oc * ho * wo
         }
         const size_t plane = size_t(ep.cv_ho) * ep.cv_wo;
+        // Per-filter operands: lane l of a row block fetches those of row l % 32 (three loads per
+        // block instead of three per accumulator register); the 16 rows a lane needs come back
+        // through shuffles.
+        float s_blk[FM], b_blk[FM];
+        int c_blk[FM];
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const int m = m0 + wm * TM + i * 32 + lane % 32;
+            const int mc = m < M ? m : M - 1;
+            c_blk[i] = ep.cv_corr_mul * ep.cv_wsum[mc];
+            s_blk[i] = 1.0f;
+            b_blk[i] = 0.0f;
+            if constexpr (EPI != EPI_I32) {
+                s_blk[i] = sa0 * ep.sw[mc];
+                if (has_bias) b_blk[i] = ep.bias[mc];
+            }
+        }
+        wait_vmcnt<0>();
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             if (WK > 1 && i % WK != wk) continue;
@@ -529,17 +580,11 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
             int c_row[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-                const int mc = m < M ? m : M - 1;
-                c_row[r] = ep.cv_corr_mul * ep.cv_wsum[mc];
-                s_row[r] = 1.0f;
-                b_row[r] = 0.0f;
-                if constexpr (EPI != EPI_I32) {
-                    s_row[r] = sa0 * ep.sw[mc];
-                    if (has_bias) b_row[r] = ep.bias[mc];
-                }
+                const int src = 8 * (r / 4) + 4 * (lane / 32) + (r % 4);  // row of the block = lane that holds it
+                c_row[r] = __shfl(c_blk[i], src, kWave);
+                s_row[r] = __shfl(s_blk[i], src, kWave);
+                b_row[r] = __shfl(b_blk[i], src, kWave);
             }
-            wait_vmcnt<0>();
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
@@ -647,8 +692,10 @@ static int32_t launch_pipe(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int 
             return fail(HIPQ_DEVICE_ERROR, "gemm_i8: cannot reserve %d bytes of LDS: %s", kLds, hipGetErrorString(e));
         configured[ctx->device] = true;
     }
-    const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    hipLaunchKernelGGL(kernel, dim3(tiles), dim3(kThreads), kLds, ctx->stream, a, w, M, N, K, ep);
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    GemmEpilogue placed = ep;
+    pick_xcd_rectangle(tiles_m, tiles_n, BM, BN, &placed.xcd_gm, &placed.xcd_gn);
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(kThreads), kLds, ctx->stream, a, w, M, N, K, placed);
     return check_launch("gemm_i8 (pipelined)");
 }
 
