@@ -652,6 +652,43 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
         // Every load of this wave has landed (and the compiler's wait tracking knows it), so
         // the stores below are issued back to back without waiting on one another.
         wait_vmcnt<0>();
+        if constexpr (EPI == EPI_I8) {
+            // int8 output as dwords.  A lane holds one column of 16 rows; the four lanes of a quad
+            // hold four consecutive columns.  Per group of four rows each lane packs its four
+            // bytes, the quad transposes the 4x4 bytes (four quad broadcasts + two byte
+            // permutes), and every lane stores one dword = four consecutive columns of one row:
+            // a quarter of the store instructions of the byte form, none of them sub-dword.
+            if (N % 4 == 0 && (reinterpret_cast<uintptr_t>(ep.out) & 3u) == 0) {
+                const int qd = lane % 4;
+                const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
+                const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const int col = nn[j] - qd;  // first column of the quad; N % 4 == 0 keeps quads whole
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        int q[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            float v = static_cast<float>(acc[i][j][4 * t + k]) * s_comb[4 * t + k][j];
+                            if (has_bias) v = v + bv[j];
+                            q[k] = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
+                        }
+                        const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));  // byte k = row 8t + 4*(lane/32) + k
+                        const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
+                        const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
+                        const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
+                        const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
+                        const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                        const int m = m0 + wm * TM + i * 32 + 8 * t + 4 * (lane / 32) + qd;
+                        if (m < M && col < N)
+                            __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(static_cast<int8_t *>(ep.out) +
+                                                                                           size_t(m) * N + col));
+                    }
+                }
+                continue;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
