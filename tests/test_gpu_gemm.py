@@ -118,7 +118,10 @@ def test_quantized_linear_forward(ctx, hipq, oracle, m, n, k, per_token):
     np.testing.assert_array_equal(got, oracle.linear_dequant_epilogue(acc, sa, sw, None))
 
 
-@pytest.mark.parametrize("m,n,k", [(7, 24, 64), (128, 96, 512), (50, 130, 272)])
+# K % 128 == 0 reaches the pipelined kernel, whose int8 epilogue stores dwords when N % 4 == 0 (ragged M and N tiles
+# included) and bytes otherwise; the other shapes reach the register-staged and the generic kernels.
+@pytest.mark.parametrize("m,n,k", [(7, 24, 64), (128, 96, 512), (50, 130, 272), (50, 100, 256), (130, 132, 384),
+                                   (67, 130, 256), (300, 260, 128), (512, 1024, 1024)])
 def test_quantized_linear_requant_epilogue(ctx, hipq, oracle, m, n, k):
     x, wf, bias, wq, sw, aq, sa, acc, out = _quantized_linear_case(oracle, m, n, k, False, 5 * m + k)
     s_out, _ = oracle.calculate_symmetric_params(*oracle.find_min_max(out), 0)
