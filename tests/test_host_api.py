@@ -79,6 +79,19 @@ def test_two_fma_division_equals_ieee_division():
     assert " 0 mismatches" in proc.stdout
 
 
+def test_three_instruction_round_half_away_equals_roundf():
+    """round(v) is computed as trunc(v + copysign(0.49999997, v)) on the device; this compares it with roundf for
+    every finite float on the CPU."""
+    _binary()
+    exe = os.path.join(ROOT, "tests", "host", "bin", "round_away_check")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "host"), "bin/round_away_check"], check=True,
+                       capture_output=True)
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "0 mismatches" in proc.stdout
+
+
 def _run(args):
     proc = subprocess.run([_binary(), *args], capture_output=True, text=True, timeout=300)
     results = {}

@@ -160,11 +160,11 @@ __device__ __forceinline__ void row_op_body(float4 (&v)[RC], size_t row, bool ac
     }
 }
 
-// Workgroups walk the row groups with a grid stride; the next group's row is requested before
-// the current one is processed, so loads, arithmetic and stores of different rows overlap in
-// every wave (with one row per wave and a single generation of workgroups the three phases ran
-// one after the other across the whole chip).
-template <int TPR, int RC, int OP, bool QUANT, bool EVEN>
+// STRIDE: workgroups walk the row groups with a grid stride and request the next group's row
+// before the current one is processed, so loads, arithmetic and stores of different rows overlap in
+// every wave.  Without it (as many workgroups as row groups) a wave handles one row and holds no
+// second row buffer: fewer registers, more waves per SIMD to overlap the phases across waves.
+template <int TPR, int RC, int OP, bool QUANT, bool EVEN, bool STRIDE>
 __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restrict__ x, size_t rows, size_t cols,
                                                             const float *__restrict__ gamma,
                                                             const float *__restrict__ beta, float eps,
@@ -185,17 +185,25 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restri
             dst[i] = (active && idx < nvec) ? load_stream(x4 + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
-    float4 v[RC], nx[RC];
+    float4 v[RC];
     size_t g = blockIdx.x;
-    if (g < groups) load_row(g, v);
-    for (; g < groups; g += gridDim.x) {
-        const size_t gn = g + gridDim.x;
-        if (gn < groups) load_row(gn, nx);
+    if (g >= groups) return;
+    load_row(g, v);
+    if constexpr (!STRIDE) {
         const size_t row = g * kRowsPerBlock + sub;
         row_op_body<TPR, RC, OP, QUANT, EVEN>(v, row, row < rows, lane, cols, gamma, beta, eps, out_f, out_q, out_scales,
                                               lds);
+    } else {
+        float4 nx[RC];
+        for (; g < groups; g += gridDim.x) {
+            const size_t gn = g + gridDim.x;
+            if (gn < groups) load_row(gn, nx);
+            const size_t row = g * kRowsPerBlock + sub;
+            row_op_body<TPR, RC, OP, QUANT, EVEN>(v, row, row < rows, lane, cols, gamma, beta, eps, out_f, out_q,
+                                                  out_scales, lds);
 #pragma unroll
-        for (int i = 0; i < RC; ++i) v[i] = nx[i];
+            for (int i = 0; i < RC; ++i) v[i] = nx[i];
+        }
     }
 }
 
@@ -245,10 +253,18 @@ static int32_t launch_row_op(const char *fn, hipq_ctx *ctx, const float *x, size
     // A wavefront per row while the row fits 12 float4 per lane (no workgroup barrier in the row
     // reductions), else the whole workgroup; the register cache is sized to the row.
     const size_t vec_per_wave_lane = (cols / 4 + kWave - 1) / kWave, vec_per_block_lane = (cols / 4 + kRowBlock - 1) / kRowBlock;
-#define HIPQ_ROW(TPR, RC, E)                                                                                      \
-    hipLaunchKernelGGL((row_op_kernel<TPR, RC, OP, QUANT, E>), dim3(row_grid(ctx, rows, kRowBlock / TPR)), \
+#define HIPQ_ROW(TPR, RC, E, S)                                                                                   \
+    hipLaunchKernelGGL((row_op_kernel<TPR, RC, OP, QUANT, E, S>), dim3(row_grid(ctx, rows, kRowBlock / TPR)), \
                        dim3(kRowBlock), 0, ctx->stream, x, rows, cols, gamma, beta, eps, out_f, out_q, out_scales)
-#define HIPQ_ROW_E(TPR, RC) do { if (even) HIPQ_ROW(TPR, RC, true); else HIPQ_ROW(TPR, RC, false); } while (0)
+#define HIPQ_ROW_E(TPR, RC)                                                                              \
+    do {                                                                                                 \
+        const size_t groups = (rows + kRowBlock / TPR - 1) / (kRowBlock / TPR);                          \
+        const bool stride = static_cast<size_t>(row_grid(ctx, rows, kRowBlock / TPR)) < groups;          \
+        if (even && stride) HIPQ_ROW(TPR, RC, true, true);                                               \
+        else if (even) HIPQ_ROW(TPR, RC, true, false);                                                   \
+        else if (stride) HIPQ_ROW(TPR, RC, false, true);                                                 \
+        else HIPQ_ROW(TPR, RC, false, false);                                                            \
+    } while (0)
     if (vec_per_wave_lane <= 4) HIPQ_ROW_E(kWave, 4);
     else if (vec_per_wave_lane <= 8) HIPQ_ROW_E(kWave, 8);
     else if (vec_per_wave_lane <= 12) HIPQ_ROW_E(kWave, 12);
