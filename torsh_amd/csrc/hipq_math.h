@@ -121,6 +121,22 @@ __device__ __forceinline__ int quantize_int(float x, float scale, float inv, flo
     return min(max(q, lo), hi);
 }
 
+// quantize_int for a symmetric per-row quantizer (zero point 0, int8 range) whose scale was derived
+// from the row's own finite maximum, scale = max|x| / 127: then |x * y| stays near 127, the
+// remainder of div_rn is never NaN for a finite x, and the select that guards it can go; a NaN
+// element still comes out as 0 (NaN propagates through both FMAs and the conversion maps it to 0).
+template <bool EVEN>
+__device__ __forceinline__ int quantize_int_sym(float x, float scale, float y) {
+    float t;
+    if (y == 0.0f) {
+        t = x / scale;
+    } else {
+        const float q0 = x * y;
+        t = fmaf(fmaf(-q0, scale, x), y, q0);
+    }
+    return min(max(cvt_i32_sat(round_mode<EVEN>(t)), -128), 127);
+}
+
 // clamp(round(v) ...) already formed as a float: convert and clamp on integers.
 __device__ __forceinline__ int clamp_to_int(float q, int lo, int hi) { return min(max(cvt_i32_sat(q), lo), hi); }
 
