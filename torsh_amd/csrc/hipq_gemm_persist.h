@@ -335,7 +335,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
             int32_t *tb = reinterpret_cast<int32_t *>(lds + STAGES * STAGE + 256) + cw * 512;
             // LDS traffic of block b+1 is issued before block b is converted and stored, so the
             // LDS round trip (long while the producers are refilling the ring) is overlapped.
-            auto lds_block = [&](int b, v4i(&t)[4]) {
+            auto lds_block = [&](int b, v4i(&t)[4], float(&sr)[4]) {
                 const int i = b / FN, j = b % FN;
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
@@ -348,10 +348,20 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                     for (int p = 0; p < 2; ++p)
                         t[2 * half + p] = *reinterpret_cast<const v4i *>(tb + (lane / 8 + 8 * p) * 32 + (lane % 8) * 4);
                 }
+                // The activation scales of the block's rows are fetched (lane shuffles, which go
+                // through the LDS pipe) together with the block, one block ahead of their use.
+                if constexpr (EPI != EPI_I32) {
+#pragma unroll
+                    for (int hp = 0; hp < 4; ++hp) {
+                        const int wrow = i * 32 + 16 * (hp / 2) + lane / 8 + 8 * (hp % 2);  // row within the wave tile
+                        sr[hp] = __shfl(s_lane[wrow / kWave], wrow % kWave, kWave);
+                    }
+                }
                 asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);  // keep this block's LDS traffic ahead of the previous block's arithmetic
             };
             float4 res4[FN][4];
-            auto out_block = [&](int b, v4i(&t)[4]) {
+            auto out_block = [&](int b, v4i(&t)[4], float(&sr)[4]) {
                 const int i = b / FN, j = b % FN;
                 if constexpr (RESIDUAL) {
                     if (j == 0) {
@@ -375,7 +385,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                     if constexpr (EPI == EPI_I32) {
                         __builtin_nontemporal_store(t[hp], reinterpret_cast<v4i *>(static_cast<int32_t *>(ep.out) + off));
                     } else {
-                        const float s_m = __shfl(s_lane[wrow / kWave], wrow % kWave, kWave);
+                        const float s_m = sr[hp];
                         const float swc[4] = {sw4[j].x, sw4[j].y, sw4[j].z, sw4[j].w};
                         const float bc[4] = {b4[j].x, b4[j].y, b4[j].z, b4[j].w};
                         float v[4];
@@ -406,11 +416,12 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                 }
             };
             v4i tbuf[2][4];
-            lds_block(0, tbuf[0]);
+            float srow[2][4];
+            lds_block(0, tbuf[0], srow[0]);
 #pragma unroll
             for (int b = 0; b < FM * FN; ++b) {
-                if (b + 1 < FM * FN) lds_block(b + 1, tbuf[(b + 1) & 1]);
-                out_block(b, tbuf[b & 1]);
+                if (b + 1 < FM * FN) lds_block(b + 1, tbuf[(b + 1) & 1], srow[(b + 1) & 1]);
+                out_block(b, tbuf[b & 1], srow[b & 1]);
             }
             continue;
         }
