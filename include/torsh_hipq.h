@@ -320,6 +320,12 @@ HIPQ_API int32_t hipq_layer_norm_f32(hipq_ctx *ctx, const float *x, size_t rows,
 HIPQ_API int32_t hipq_layer_norm_quantize_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
                                                  const float *gamma, const float *beta, float eps, int32_t mode,
                                                  int8_t *out, float *out_scales);
+/* The skip connection and the LayerNorm + quantizer that follow it in one pass: x[r, :] += delta[r, :]
+ * (Tensor::add, one rounding per element, written back over x), then the new row goes through
+ * hipq_layer_norm_quantize_f32_i8.  Same results as hipq_add_f32 followed by that call. */
+HIPQ_API int32_t hipq_add_layer_norm_quantize_f32_i8(hipq_ctx *ctx, float *x, const float *delta, size_t rows,
+                                                     size_t cols, const float *gamma, const float *beta, float eps,
+                                                     int32_t mode, int8_t *out, float *out_scales);
 /* tanh-form GELU, crates/torsh-nn/src/layers/activation/modern.rs:124-136. */
 HIPQ_API int32_t hipq_gelu_tanh_f32(hipq_ctx *ctx, const float *x, size_t n, float *out);
 /* GELU followed by the per-token symmetric int8 quantizer in one pass. */

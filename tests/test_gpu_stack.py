@@ -40,6 +40,28 @@ def test_layer_norm(ctx, oracle, shape):
     np.testing.assert_array_equal(host(q), host(q_ref))
 
 
+@pytest.mark.parametrize("shape", [(1, 4), (5, 768), (64, 768), (4100, 768), (33, 3072), (3, 8192), (9, 2052)])
+def test_add_layer_norm_quantize(ctx, oracle, shape):
+    """The skip connection fused into the LayerNorm + quantize pass: the stream row is the f32 sum (bit exact,
+    checked against numpy), and the codes equal those of the unfused kernels on that sum."""
+    rng = np.random.default_rng(shape[0] * 7 + shape[1])
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    delta = rng.standard_normal(shape).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, shape[1]).astype(np.float32)
+    beta = rng.standard_normal(shape[1]).astype(np.float32) * 0.1
+    total = x + delta
+    xd = dev(x)
+    q, s = ctx.add_layer_norm_quantize(xd, dev(delta), dev(gamma), dev(beta), 1e-5)
+    np.testing.assert_array_equal(host(xd), total)
+    q_ref, s_ref = ctx.layer_norm_quantize(dev(total), dev(gamma), dev(beta), 1e-5)
+    np.testing.assert_array_equal(host(s), host(s_ref))
+    np.testing.assert_array_equal(host(q), host(q_ref))
+    # and against the oracle's LayerNorm of the sum, within the LayerNorm tolerance expressed in codes
+    want = oracle.layer_norm(total, gamma, beta, 1e-5)
+    deq = host(q).astype(np.float32) * host(s)[:, None]
+    assert np.abs(deq - want).max() <= np.abs(want).max() / 127.0 * 0.5 + 1e-4
+
+
 @pytest.mark.parametrize("shape", [(4, 8), (16, 3072), (5, 1024)])
 def test_gelu(ctx, oracle, shape):
     rng = np.random.default_rng(shape[0])

@@ -160,12 +160,15 @@ __device__ __forceinline__ void row_op_body(float4 (&v)[RC], size_t row, bool ac
     }
 }
 
+// ADD: the row is x + delta (one rounding per element), written back over x before it is
+// normalised: the residual update of the stream and the LayerNorm that follows it in one pass.
 // STRIDE: workgroups walk the row groups with a grid stride and request the next group's row
 // before the current one is processed, so loads, arithmetic and stores of different rows overlap in
 // every wave.  Without it (as many workgroups as row groups) a wave handles one row and holds no
 // second row buffer: fewer registers, more waves per SIMD to overlap the phases across waves.
-template <int TPR, int RC, int OP, bool QUANT, bool EVEN, bool STRIDE>
-__global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restrict__ x, size_t rows, size_t cols,
+template <int TPR, int RC, int OP, bool QUANT, bool EVEN, bool STRIDE, bool ADD>
+__global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *x, const float *__restrict__ delta,
+                                                            float *sum_out, size_t rows, size_t cols,
                                                             const float *__restrict__ gamma,
                                                             const float *__restrict__ beta, float eps,
                                                             float *__restrict__ out_f, int8_t *__restrict__ out_q,
@@ -175,34 +178,56 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *__restri
     const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
     const size_t nvec = cols / 4;
     const size_t groups = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    auto load_row = [&](size_t g, float4(&dst)[RC]) {
+    constexpr int RD = ADD ? RC : 1;
+    auto load_row = [&](size_t g, float4(&dst)[RC], float4(&dd)[RD]) {
         const size_t row = g * kRowsPerBlock + sub;
         const bool active = row < rows;
         const float4 *x4 = reinterpret_cast<const float4 *>(x + (active ? row : 0) * cols);
+        const float4 *d4 = reinterpret_cast<const float4 *>(delta + (ADD && active ? row : 0) * cols);
 #pragma unroll
         for (int i = 0; i < RC; ++i) {
             const size_t idx = size_t(lane) + size_t(i) * TPR;
             dst[i] = (active && idx < nvec) ? load_stream(x4 + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if constexpr (ADD) dd[i] = (active && idx < nvec) ? load_stream(d4 + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
-    float4 v[RC];
+    // x + delta, stored back as the new row of the stream.
+    auto add_row = [&](size_t g, float4(&dst)[RC], const float4(&dd)[RD]) {
+        if constexpr (ADD) {
+            const size_t row = g * kRowsPerBlock + sub;
+            float4 *s4 = reinterpret_cast<float4 *>(sum_out + (row < rows ? row : 0) * cols);
+#pragma unroll
+            for (int i = 0; i < RC; ++i) {
+                const size_t idx = size_t(lane) + size_t(i) * TPR;
+                dst[i] = make_float4(dst[i].x + dd[i].x, dst[i].y + dd[i].y, dst[i].z + dd[i].z, dst[i].w + dd[i].w);
+                if (row < rows && idx < nvec) store_stream(s4 + idx, dst[i]);
+            }
+        }
+    };
+    float4 v[RC], d[RD];
     size_t g = blockIdx.x;
     if (g >= groups) return;
-    load_row(g, v);
+    load_row(g, v, d);
     if constexpr (!STRIDE) {
         const size_t row = g * kRowsPerBlock + sub;
+        add_row(g, v, d);
         row_op_body<TPR, RC, OP, QUANT, EVEN>(v, row, row < rows, lane, cols, gamma, beta, eps, out_f, out_q, out_scales,
                                               lds);
     } else {
-        float4 nx[RC];
+        float4 nx[RC], nd[RD];
         for (; g < groups; g += gridDim.x) {
             const size_t gn = g + gridDim.x;
-            if (gn < groups) load_row(gn, nx);
+            if (gn < groups) load_row(gn, nx, nd);
             const size_t row = g * kRowsPerBlock + sub;
+            add_row(g, v, d);
             row_op_body<TPR, RC, OP, QUANT, EVEN>(v, row, row < rows, lane, cols, gamma, beta, eps, out_f, out_q,
                                                   out_scales, lds);
 #pragma unroll
             for (int i = 0; i < RC; ++i) v[i] = nx[i];
+            if constexpr (ADD) {
+#pragma unroll
+                for (int i = 0; i < RC; ++i) d[i] = nd[i];
+            }
         }
     }
 }
@@ -235,17 +260,18 @@ static int row_grid(hipq_ctx *ctx, size_t rows, int rows_per_block) {
     return static_cast<int>(groups < cap ? groups : cap);
 }
 
-template <int OP, bool QUANT>
+template <int OP, bool QUANT, bool ADD = false>
 static int32_t launch_row_op(const char *fn, hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
                              const float *beta, float eps, int32_t mode, float *out_f, int8_t *out_q,
-                             float *out_scales) {
+                             float *out_scales, const float *delta = nullptr, float *sum_out = nullptr) {
     if (rows == 0) return HIPQ_SUCCESS;
     if (cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: rows of zero length", fn);
     if (cols % 4 != 0 || cols > size_t(kRowBlock) * kRowCacheMax * 4)
         return fail(HIPQ_SHAPE_ERROR, "%s: row length %zu must be a multiple of 4 and at most %d", fn, cols,
                     kRowBlock * kRowCacheMax * 4);
     uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gamma) |
-                     reinterpret_cast<uintptr_t>(beta) | reinterpret_cast<uintptr_t>(out_f);
+                     reinterpret_cast<uintptr_t>(beta) | reinterpret_cast<uintptr_t>(out_f) |
+                     reinterpret_cast<uintptr_t>(delta) | reinterpret_cast<uintptr_t>(sum_out);
     if ((bits & 15u) || (reinterpret_cast<uintptr_t>(out_q) & 3u))
         return fail(HIPQ_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", fn);
     if (rows >> 31) return fail(HIPQ_SHAPE_ERROR, "%s: too many rows", fn);
@@ -254,8 +280,9 @@ static int32_t launch_row_op(const char *fn, hipq_ctx *ctx, const float *x, size
     // reductions), else the whole workgroup; the register cache is sized to the row.
     const size_t vec_per_wave_lane = (cols / 4 + kWave - 1) / kWave, vec_per_block_lane = (cols / 4 + kRowBlock - 1) / kRowBlock;
 #define HIPQ_ROW(TPR, RC, E, S)                                                                                   \
-    hipLaunchKernelGGL((row_op_kernel<TPR, RC, OP, QUANT, E, S>), dim3(row_grid(ctx, rows, kRowBlock / TPR)), \
-                       dim3(kRowBlock), 0, ctx->stream, x, rows, cols, gamma, beta, eps, out_f, out_q, out_scales)
+    hipLaunchKernelGGL((row_op_kernel<TPR, RC, OP, QUANT, E, S, ADD>), dim3(row_grid(ctx, rows, kRowBlock / TPR)), \
+                       dim3(kRowBlock), 0, ctx->stream, x, delta, sum_out, rows, cols, gamma, beta, eps, out_f, out_q,   \
+                       out_scales)
 #define HIPQ_ROW_E(TPR, RC)                                                                              \
     do {                                                                                                 \
         const size_t groups = (rows + kRowBlock / TPR - 1) / (kRowBlock / TPR);                          \
@@ -302,6 +329,20 @@ int32_t hipq_layer_norm_quantize_f32_i8(hipq_ctx *ctx, const float *x, size_t ro
     }
     return launch_row_op<ROW_LAYERNORM, true>(__func__, ctx, x, rows, cols, gamma, beta, eps, mode, nullptr, out,
                                               out_scales);
+}
+
+int32_t hipq_add_layer_norm_quantize_f32_i8(hipq_ctx *ctx, float *x, const float *delta, size_t rows, size_t cols,
+                                            const float *gamma, const float *beta, float eps, int32_t mode,
+                                            int8_t *out, float *out_scales) {
+    HIPQ_ENTER(ctx);
+    if (rows * cols != 0) {
+        HIPQ_REQUIRE_PTR(x);
+        HIPQ_REQUIRE_PTR(delta);
+        HIPQ_REQUIRE_PTR(out);
+        HIPQ_REQUIRE_PTR(out_scales);
+    }
+    return launch_row_op<ROW_LAYERNORM, true, true>(__func__, ctx, x, rows, cols, gamma, beta, eps, mode, nullptr, out,
+                                                    out_scales, delta, x);
 }
 
 int32_t hipq_gelu_tanh_f32(hipq_ctx *ctx, const float *x, size_t n, float *out) {

@@ -2,7 +2,11 @@
 // QKV Linear -> stand-in attention -> output Linear + residual -> LayerNorm ->
 // per-token int8 -> fc1 -> GELU -> per-token int8 -> fc2 + residual), composed
 // from the library's own entry points.  Eight kernels per layer; the fp32
-// intermediates that only feed a quantizer are never written to memory.
+// intermediates that only feed a quantizer are never written to memory.  The fc2
+// skip connection of every layer but the last is not added in the GEMM's epilogue
+// but by the next layer's first LayerNorm kernel, which reads the row anyway: the
+// GEMM then runs in its large-tile form, whose registers have no room for
+// residual values, and the stream is read and written once less.
 #include "hipq_internal.h"
 
 namespace {
@@ -48,7 +52,12 @@ int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_block_weigh
         const hipq_block_weights &b = blocks[l];
         int32_t rc;
         // attention half: x += W_out * quant(V(LN1(x)))
-        rc = hipq_layer_norm_quantize_f32_i8(ctx, x, tokens, d_model, b.ln1_gamma, b.ln1_beta, eps, round_bits, q8, scales);
+        // (from the second layer on: x += the previous layer's fc2 output, held in the qkv buffer)
+        if (l == 0)
+            rc = hipq_layer_norm_quantize_f32_i8(ctx, x, tokens, d_model, b.ln1_gamma, b.ln1_beta, eps, round_bits, q8, scales);
+        else
+            rc = hipq_add_layer_norm_quantize_f32_i8(ctx, x, qkv, tokens, d_model, b.ln1_gamma, b.ln1_beta, eps,
+                                                     round_bits, q8, scales);
         if (rc) return rc;
         rc = hipq_linear_i8_f32(ctx, q8, scales, 1, b.w_qkv, b.s_qkv, b.b_qkv, tokens, 3 * d_model, d_model, qkv);
         if (rc) return rc;
@@ -65,7 +74,10 @@ int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_block_weigh
         if (rc) return rc;
         rc = hipq_gelu_tanh_quantize_f32_i8(ctx, hidden, tokens, d_ff, round_bits, q8, scales);
         if (rc) return rc;
-        rc = hipq_linear_i8_f32_residual(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, x, tokens, d_model, d_ff, x);
+        if (l + 1 == n_layers)
+            rc = hipq_linear_i8_f32_residual(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, x, tokens, d_model, d_ff, x);
+        else
+            rc = hipq_linear_i8_f32(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, tokens, d_model, d_ff, qkv);
         if (rc) return rc;
     }
     return HIPQ_SUCCESS;

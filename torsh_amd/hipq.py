@@ -100,6 +100,7 @@ _SIGNATURES = {
     "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
+    "hipq_add_layer_norm_quantize_f32_i8": [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_gelu_tanh_f32": [_vp, _vp, _sz, _vp],
     "hipq_gelu_tanh_quantize_f32_i8": [_vp, _vp, _sz, _sz, _i32, _vp, _vp],
     "hipq_add_f32": [_vp, _vp, _vp, _sz, _vp],
@@ -538,6 +539,15 @@ class Context:
         scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
         self.call("hipq_layer_norm_quantize_f32_i8", _ptr(x), rows, cols, _ptr(gamma), _ptr(beta), float(eps), mode,
                   _ptr(out), _ptr(scales))
+        return out, scales
+
+    def add_layer_norm_quantize(self, x, delta, gamma=None, beta=None, eps=1e-5, mode=0):
+        """x += delta in place, then LayerNorm + per-token int8 of the new x."""
+        rows, cols = x.shape
+        out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
+        scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
+        self.call("hipq_add_layer_norm_quantize_f32_i8", _ptr(x), _ptr(delta), rows, cols, _ptr(gamma), _ptr(beta),
+                  float(eps), mode, _ptr(out), _ptr(scales))
         return out, scales
 
     def gelu_tanh(self, x):
