@@ -319,21 +319,25 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
         if (tiles(128, 64) >= 2 * cus) {
             // Many more tiles than CUs: the persistent kernel.  Its tile shape is picked with a
             // cost model fitted to measurements: a tile costs nk * L + E cycles, where the main
-            // loop is bound by LDS traffic (L per K-tile: fills plus fragment reads) and the
-            // epilogue by the CU's share of HBM write bandwidth (E per tile of 4-byte outputs);
+            // loop is bound by LDS traffic (L per K-tile: fills plus fragment reads) and E is the
+            // epilogue of a tile of 4-byte outputs (conversion, transposition through LDS, stores);
             // a workgroup runs ceil(tiles / CUs) tiles.  Bigger tiles move fewer LDS bytes per MAC
-            // but quantise worse.  The 256x128 form has no room for residual values in registers.
+            // but quantise worse.  The 256x128 and 128x192 forms have no room for residual values
+            // in registers.
             const double nk = double(K / 128), out_scale = (EPI == EPI_I8) ? 0.25 : 1.0;
             auto cost = [&](size_t bm, size_t bn, double L, double E) {
                 const size_t t = tiles(bm, bn);
                 return double((t + cus - 1) / cus) * (nk * L + E * out_scale);
             };
+            const bool with_residual = EPI == EPI_F32 && ep.residual;
             const double c5 = cost(128, 64, 900.0, 2700.0), c6 = cost(128, 128, 1350.0, 4700.0);
-            const double c7 = (EPI == EPI_F32 && ep.residual) ? 1e30 : cost(256, 128, 1950.0, 9600.0);
-            variant = (c7 <= c6 && c7 <= c5) ? 7 : (c6 <= c5 ? 6 : 5);
+            const double c7 = with_residual ? 1e30 : cost(256, 128, 1950.0, 9600.0);
+            // 128x192: between the two in LDS bytes per MAC; divides N = 768 and 2304 into whole rounds.
+            const double c8 = with_residual ? 1e30 : cost(128, 192, 1600.0, 7200.0);
+            variant = (c7 <= c6 && c7 <= c5 && c7 <= c8) ? 7 : (c8 <= c6 && c8 <= c5 ? 8 : (c6 <= c5 ? 6 : 5));
         }
     }
-    if (variant == 0 || (variant < 10 && !pipe_ok)) variant = 10;
+    if (variant == 0 || (variant != 10 && !pipe_ok)) variant = 10;
     switch (variant) {
     case 1: return launch_pipe<128, 64, 6, 4, 1, 1, 4, EPI, EVEN>(ctx, a, w, M, N, K, ep);
     case 2: return launch_pipe<128, 64, 6, 4, 2, 1, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
@@ -342,6 +346,9 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
     case 6: return launch_persist<128, 128, 4, 4, 2, 2, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
     case 7:
         if (!(EPI == EPI_F32 && ep.residual)) return launch_persist<256, 128, 3, 4, 2, 2, 1, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+        return launch_persist<128, 128, 4, 4, 2, 2, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
+    case 8:
+        if (!(EPI == EPI_F32 && ep.residual)) return launch_persist<128, 192, 3, 4, 2, 2, 1, EPI, EVEN>(ctx, a, w, M, N, K, ep);
         return launch_persist<128, 128, 4, 4, 2, 2, 2, EPI, EVEN>(ctx, a, w, M, N, K, ep);
     default: break;
     }
