@@ -278,6 +278,25 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                 }
             }
         }
+        // Residual values of the whole wave tile, when they fit in registers: requested here, they
+        // arrive while the tile is multiplied, and no load is issued between the epilogue's stores
+        // (a load waits for every store issued before it: they share one counter).
+        constexpr bool RES_PRE = RESIDUAL && EPI == EPI_F32 && FM * FN * 16 <= 32;
+        float4 res_pre[RES_PRE ? FM : 1][RES_PRE ? FN : 1][4];
+        if constexpr (RES_PRE) {
+            if (fast) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int jj = 0; jj < FN; ++jj)
+#pragma unroll
+                        for (int hp = 0; hp < 4; ++hp) {
+                            const int m = m0 + wm * TM + i * 32 + 16 * (hp / 2) + lane / 8 + 8 * (hp % 2);
+                            const int nq = n0 + wn * TN + jj * 32 + (lane % 8) * 4;
+                            res_pre[i][jj][hp] = *reinterpret_cast<const float4 *>(ep.residual + size_t(m) * N + nq);
+                        }
+            }
+        }
         // Activation scales of this wave's rows, one row per lane (row block i in s_lane[i]); the
         // epilogue fetches the scale of each accumulator row with a lane shuffle.
         float s_lane[(TM + kWave - 1) / kWave];
@@ -363,7 +382,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
             float4 res4[FN][4];
             auto out_block = [&](int b, v4i(&t)[4], float(&sr)[4]) {
                 const int i = b / FN, j = b % FN;
-                if constexpr (RESIDUAL) {
+                if constexpr (RESIDUAL && !RES_PRE) {
                     if (j == 0) {
 #pragma unroll
                         for (int jj = 0; jj < FN; ++jj)
@@ -396,7 +415,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                         }
                         if constexpr (EPI == EPI_F32) {
                             if constexpr (RESIDUAL) {
-                                const float4 rv = res4[j][hp];
+                                const float4 rv = RES_PRE ? res_pre[RES_PRE ? i : 0][RES_PRE ? j : 0][hp] : res4[j][hp];
                                 v[0] = v[0] + rv.x;
                                 v[1] = v[1] + rv.y;
                                 v[2] = v[2] + rv.z;
