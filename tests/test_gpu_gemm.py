@@ -135,10 +135,13 @@ def test_quantized_linear_requant_epilogue(ctx, hipq, oracle, m, n, k):
         np.testing.assert_array_equal(got, want)
 
 
-@pytest.mark.parametrize("m,n,k", [(4096, 1024, 512), (4100, 1000, 256), (8192, 768, 768)])
+@pytest.mark.parametrize("m,n,k", [(4096, 1024, 512), (4100, 1000, 256), (8192, 768, 768), (2048, 2304, 256),
+                                   (2000, 2300, 384)])
 def test_many_tile_shapes_persistent_kernel(ctx, hipq, oracle, m, n, k):
     """Shapes with at least two 128x64 tiles per compute unit run on the persistent kernel: accumulators, the
-    dequantize epilogue with per-token scales, the residual add and the requantize epilogue against the oracle."""
+    dequantize epilogue with per-token scales, the residual add and the requantize epilogue against the oracle.
+    The shapes cover its tile forms (N = 768 and 2304 take 128x192 tiles, the ragged ones the bounds-checked
+    epilogues)."""
     rng = np.random.default_rng(m + n + k)
     a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
     acc = oracle.gemm_i8_nk(a, w)
