@@ -346,26 +346,24 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
         // m = 8*(r/4) + 4*(lane/32) + r%4 for r = 0..15.
         if (fast) {
             // Transposing epilogue.  The accumulators (lane = column) pass through a wave-private
-            // 2 KiB LDS block, half a 32x32 block at a time, and come back with lane l holding
-            // columns 4*(l%8)..+3 of rows l/8 and l/8+8: every global access is then a 16-byte piece
-            // of a fully covered 128-byte line, a quarter of the store instructions of the
+            // 1 KiB LDS block, a quarter of a 32x32 block (8 rows) at a time, and come back with
+            // lane l holding columns 4*(l%8)..+3 of row l/8: every global access is then a 16-byte
+            // piece of a fully covered 128-byte line, a quarter of the store instructions of the
             // lane-per-column layout.  A wave's LDS operations execute in order, so it needs no
             // barrier to read back what it wrote.
-            int32_t *tb = reinterpret_cast<int32_t *>(lds + STAGES * STAGE + 256) + cw * 512;
+            int32_t *tb = reinterpret_cast<int32_t *>(lds + STAGES * STAGE + 256) + cw * 256;
             // LDS traffic of block b+1 is issued before block b is converted and stored, so the
             // LDS round trip (long while the producers are refilling the ring) is overlapped.
             auto lds_block = [&](int b, v4i(&t)[4], float(&sr)[4]) {
                 const int i = b / FN, j = b % FN;
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int hp = 0; hp < 4; ++hp) {
                     asm volatile("" ::: "memory");
 #pragma unroll
-                    for (int rr = 0; rr < 8; ++rr)
-                        tb[(8 * (rr / 4) + 4 * (lane / 32) + (rr % 4)) * 32 + lane % 32] = acc[i][j][8 * half + rr];
+                    for (int rr = 0; rr < 4; ++rr)
+                        tb[(4 * (lane / 32) + rr) * 32 + lane % 32] = acc[i][j][4 * hp + rr];
                     asm volatile("" ::: "memory");  // reads stay behind the writes (other lanes' data)
-#pragma unroll
-                    for (int p = 0; p < 2; ++p)
-                        t[2 * half + p] = *reinterpret_cast<const v4i *>(tb + (lane / 8 + 8 * p) * 32 + (lane % 8) * 4);
+                    t[hp] = *reinterpret_cast<const v4i *>(tb + (lane / 8) * 32 + (lane % 8) * 4);
                 }
                 // The activation scales of the block's rows are fetched (lane shuffles, which go
                 // through the LDS pipe) together with the block, one block ahead of their use.
@@ -538,8 +536,8 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
 template <int BM, int BN, int STAGES, int PW, int WM, int WN, int KG, int EPI, bool EVEN>
 static int32_t launch_persist(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, int N, int K,
                               const GemmEpilogue &ep) {
-    // ring of K-tile buffers + the queue counters + 2 KiB per consumer wave for the epilogue's transposition
-    constexpr int kLds = STAGES * (BM + BN) * 128 + 256 + WM * WN * 2048;
+    // ring of K-tile buffers + the queue counters + 1 KiB per consumer wave for the epilogue's transposition
+    constexpr int kLds = STAGES * (BM + BN) * 128 + 256 + WM * WN * 1024;
     static_assert(kLds <= 160 * 1024, "LDS budget of one CU");
     constexpr int kThreads = (PW + WM * WN) * kWave;
     const bool with_residual = EPI == EPI_F32 && ep.residual != nullptr;
