@@ -265,17 +265,20 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
         // epilogue (lane = 4 consecutive columns of one row); the others the checked one
         // (lane = one column), which fetches its operands when it gets there.
         const bool fast = vec_ok && m0 + BM <= M && n0 + BN <= N;
+        // Only the transposing epilogue reads these, and the bias only when there is one.  The
+        // loads are nevertheless unconditional - where a value is not needed they read 16 valid
+        // bytes of the activation matrix instead - because any other form (a constant first, or a
+        // load under a condition) makes the register a merge of a loaded and a moved value, and
+        // the compiler then waits at the top of every tile until all outstanding memory
+        // operations, the previous epilogue's stores included, have completed.
         float4 sw4[FN], b4[FN];
+        if constexpr (EPI != EPI_I32) {
+            const float4 *dummy = reinterpret_cast<const float4 *>(A);
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            sw4[j] = make_float4(1.f, 1.f, 1.f, 1.f);
-            b4[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if constexpr (EPI != EPI_I32) {
-                if (fast) {
-                    const int nq = n0 + wn * TN + j * 32 + (lane % 8) * 4;
-                    sw4[j] = *reinterpret_cast<const float4 *>(ep.sw + nq);
-                    if (has_bias) b4[j] = *reinterpret_cast<const float4 *>(ep.bias + nq);
-                }
+            for (int j = 0; j < FN; ++j) {
+                const int nq = n0 + wn * TN + j * 32 + (lane % 8) * 4;
+                sw4[j] = *(fast ? reinterpret_cast<const float4 *>(ep.sw + nq) : dummy);
+                b4[j] = *((fast && has_bias) ? reinterpret_cast<const float4 *>(ep.bias + nq) : dummy);
             }
         }
         // Residual values of the whole wave tile, when they fit in registers: requested here, they
@@ -301,14 +304,12 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
         // epilogue fetches the scale of each accumulator row with a lane shuffle.
         float s_lane[(TM + kWave - 1) / kWave];
         if constexpr (EPI != EPI_I32) {
-            const float sa0 = ep.sa_per_row ? 1.0f : (ep.sa ? ep.sa[0] : ep.sa_scalar);
+            // One unconditional load per row block, for the same reason (a per-tensor scale is the
+            // same address for every lane; the launcher checks that the scale is given).
 #pragma unroll
             for (int u = 0; u < (TM + kWave - 1) / kWave; ++u) {
-                s_lane[u] = sa0;
-                if (ep.sa_per_row) {
-                    const int m = m0 + wm * TM + u * kWave + lane;
-                    s_lane[u] = ep.sa[m < M ? m : M - 1];
-                }
+                const int m = m0 + wm * TM + u * kWave + lane;
+                s_lane[u] = ep.sa[ep.sa_per_row ? (m < M ? m : M - 1) : 0];
             }
         }
 #pragma unroll
@@ -552,6 +553,7 @@ static int32_t launch_persist(hipq_ctx *ctx, const int8_t *a, const int8_t *w, i
         configured[ctx->device][with_residual] = true;
     }
     if (K % 128 != 0 || K < 128) return fail(HIPQ_INVALID_ARGUMENT, "gemm_i8 (persistent): K must be a multiple of 128");
+    if (EPI != EPI_I32 && (!ep.sa || !ep.sw)) return fail(HIPQ_INVALID_ARGUMENT, "gemm_i8 (persistent): scales must be given");
     const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     const int grid = tiles < ctx->num_cus ? tiles : ctx->num_cus;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), kLds, ctx->stream, a, w, M, N, K, ep);
