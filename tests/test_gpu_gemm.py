@@ -207,3 +207,40 @@ def test_config3_full_size_weight_streaming(ctx, hipq, m):
     want = ref.float() * (sa[:, None] * sw[None, :]) + bias[None, :]  # same individually rounded f32 ops
     torch.cuda.synchronize()
     assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("n,k", [(2304, 768), (768, 768), (3072, 768), (768, 3072)])
+def test_config5_full_size_projection_shapes(ctx, hipq, n, k):
+    """The projection stack's GEMMs at their real size (8192 tokens, d = 768, d_ff = 3072), which run on the
+    persistent kernel's large tile forms: every accumulator against an exact float64 product computed by torch in
+    row chunks, the per-token dequantize epilogue and the residual form against the same f32 expression, and the
+    requantize epilogue's bytes re-derived from the f32 output with numpy's IEEE division."""
+    m = 8192
+    g = torch.Generator(device="cuda").manual_seed(n + k)
+    a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    acc = ctx.gemm_i8_i32(a, w)
+    ref = torch.empty((m, n), dtype=torch.int32, device="cuda")
+    wd = w.double().T.contiguous()
+    for r0 in range(0, m, 1024):
+        ref[r0:r0 + 1024] = (a[r0:r0 + 1024].double() @ wd).to(torch.int32)  # exact: |acc| < 2^53
+    torch.cuda.synchronize()
+    assert torch.equal(acc, ref)
+    sa = torch.rand(m, generator=g, device="cuda") * 0.05 + 0.01
+    sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(n, generator=g, device="cuda") * 0.01
+    want = ref.float() * (sa[:, None] * sw[None, :]) + bias[None, :]  # same individually rounded f32 ops
+    assert torch.equal(ctx.linear_i8_f32(a, sa, w, sw, bias), want)
+    res = torch.randn((m, n), generator=g, device="cuda")
+    assert torch.equal(ctx.linear_i8_f32_residual(a, sa, w, sw, bias, res), want + res)
+    x = res.clone()  # in place, as the stack uses it
+    ctx.linear_i8_f32_residual(a, sa, w, sw, bias, x, out=x)
+    assert torch.equal(x, want + res)
+    s_out = np.float32(float(want.abs().max()) / 127.0)
+    q = ctx.linear_i8_i8(a, sa, w, sw, bias, float(s_out), 3)
+    torch.cuda.synchronize()
+    t = want.cpu().numpy() / s_out  # IEEE f32 division
+    r = np.trunc(t + np.copysign(np.float32(0.49999997), t))  # f32::round (tests/host/round_away_check.c)
+    assert r.dtype == np.float32
+    wantq = np.clip(r + np.float32(3), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(q.cpu().numpy(), wantq)
