@@ -161,3 +161,39 @@ def test_stack_workspace_too_small_is_rejected(ctx, hipq):
     with pytest.raises(hipq.HipqError) as e:
         ctx.stack_forward([{}], x, 512, ws)
     assert e.value.code == hipq.INVALID_ARGUMENT
+
+
+def test_projection_stack_full_size_equals_its_parts(ctx, hipq):
+    """Config 5 at its real size (8192 tokens, d = 768, d_ff = 3072; 3 layers keep the test short): the stack call,
+    which defers each fc2 skip connection into the next layer's LayerNorm kernel and picks its own GEMM tile forms,
+    is bit-identical to the same layers composed from the separately tested entry points with the residual added in
+    the fc2 epilogue."""
+    tokens, d, dff, layers = 8192, 768, 3072, 3
+    g = torch.Generator(device="cuda").manual_seed(11)
+    blocks = []
+    for _ in range(layers):
+        blk = {}
+        for name, (o, i) in {"qkv": (3 * d, d), "out": (d, d), "fc1": (dff, d), "fc2": (d, dff)}.items():
+            wf = torch.randn(o, i, generator=g, device="cuda") * 0.02
+            q, sc, _, _ = ctx.quantize_per_row(wf)
+            blk["w_" + name], blk["s_" + name] = q, sc
+            blk["b_" + name] = torch.randn(o, generator=g, device="cuda") * 0.01
+        for ln in ("ln1", "ln2"):
+            blk[ln + "_gamma"] = torch.rand(d, generator=g, device="cuda") + 0.5
+            blk[ln + "_beta"] = torch.randn(d, generator=g, device="cuda") * 0.1
+        blocks.append(blk)
+    x0 = torch.randn(tokens, d, generator=g, device="cuda")
+    got = ctx.stack_forward(blocks, x0.clone(), dff, ctx.stack_workspace(tokens, d, dff))
+    x = x0.clone()
+    for blk in blocks:
+        q, s = ctx.layer_norm_quantize(x, blk["ln1_gamma"], blk["ln1_beta"], 1e-5)
+        qkv = ctx.linear_i8_f32(q, s, blk["w_qkv"], blk["s_qkv"], blk["b_qkv"])
+        q, s = ctx.quantize_per_row_strided(qkv, tokens, d, 3 * d, elem_offset=2 * d)
+        x = ctx.linear_i8_f32_residual(q, s, blk["w_out"], blk["s_out"], blk["b_out"], x)
+        q, s = ctx.layer_norm_quantize(x, blk["ln2_gamma"], blk["ln2_beta"], 1e-5)
+        h = ctx.linear_i8_f32(q, s, blk["w_fc1"], blk["s_fc1"], blk["b_fc1"])
+        q, s = ctx.gelu_tanh_quantize(h)
+        x = ctx.linear_i8_f32_residual(q, s, blk["w_fc2"], blk["s_fc2"], blk["b_fc2"], x)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all()
+    assert torch.equal(got, x)
