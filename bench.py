@@ -285,6 +285,25 @@ def main() -> int:
                                                       "note": "alternating batches on two contexts/streams"}
         ctx2.close()
         ctx3.close()
+        # The same step with a calibrated (static) activation scale: no range pass over the input.
+        ps = [0]
+
+        def step_static():
+            i = ps[0] % pool
+            ps[0] += 1
+            ctx.linear_static(xs[i], 0.035, wq[i], sw[i], bias, mode=hipq.FORM_MUL_INV, out=outs[i])
+
+        for _ in range(args.warmup):
+            step_static()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_static()
+        torch.cuda.synchronize()
+        ms3 = (time.perf_counter() - t0) * 1e3 / args.steps
+        extra["linear_step_static_activation_scale"] = {"ms_per_step": ms3, "TOP/s": ops / (ms3 * 1e-3) / 1e12,
+                                                        "note": "activation scale from calibration instead of a "
+                                                                "min/max pass per call (two launches, not three)"}
         n = 4096 * 4096
         npool = 10  # 10 x (64 + 16 + 64) MiB > memory-side cache
         fx = [torch.randn(n, generator=g, device="cuda") for _ in range(npool)]

@@ -136,6 +136,12 @@ HIPQ_API int32_t hipq_qparams_from_minmax(hipq_ctx *ctx, const float *minmax, in
  * scale <= 0 is InvalidArgument (algorithms.rs:284-288). */
 HIPQ_API int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n, float scale,
                                                  int32_t zero_point, int32_t mode, int8_t *out);
+/* hipq_quantize_per_tensor_f32_i8 that also records the parameters it was given in a device-side
+ * hipq_qparams, for the kernels that read their scale from device memory (hipq_linear_i8_f32,
+ * hipq_dequantize_with_params_i8_f32). */
+HIPQ_API int32_t hipq_quantize_static_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                                        int32_t zero_point, int32_t mode, int8_t *out,
+                                                        hipq_qparams *out_params);
 /* CpuQuantizationOps::quantize_f32 for UInt8,
  * crates/torsh-backend/src/quantization/ops.rs:185-195,295-364:
  * q = clamp(round(x / scale) + zp, 0, 255). */
@@ -262,6 +268,13 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
                                         const float *a_scale, int32_t a_scale_per_row, const float *w_scales,
                                         const float *bias, float out_scale, int32_t out_zero_point,
                                         int32_t mode, int8_t *out);
+/* Whole forward of a quantized Linear with a static (calibrated) activation scale: the scale an
+ * observer derived beforehand (Observer::calculate_qparams, crates/torsh-quantization/src/observers.rs:263-310,
+ * symmetric: zero point 0) instead of a range pass over every input - per-tensor quantize
+ * (algorithms.rs:277-315), int8 GEMM, dequantizing epilogue.  `mode` as hipq_quantize_per_tensor_f32_i8. */
+HIPQ_API int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w,
+                                        const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
+                                        int32_t mode, float *out);
 /* Whole forward of a quantized Linear on fp32 activations: dynamic activation
  * quantization (per tensor: algorithms.rs:85-123; per token: algorithms.rs:126-242
  * on axis 0), int8 GEMM, dequantizing epilogue.  Uses context-owned scratch

@@ -602,6 +602,37 @@ GPU_TEST(parity_quantized_linear_module) {
         CHECK_SAME(params.at("weight").as_slice(), wq_f);
         CHECK_SAME(params.at("weight_scale").as_slice(), sw);
         CHECK(qlin.forward(Tensor::from_data(std::vector<float>(10, 0.f), {2, 5}).unwrap()).is_err());
+        // Static quantization: a calibrated per-tensor activation scale (MinMax observer over the same
+        // data, symmetric int8) replaces the range pass.  Per-token layers refuse it.
+        if (per_token) {
+            CHECK(qlin.set_static_activation_scale(0.05f).is_err());
+        } else {
+            quantization::Observer ob(quantization::ObserverType::MinMax);
+            CHECK(ob.update(Tensor::from_data(x, {m, k}).unwrap()).is_ok());
+            const auto [mn, mx] = ob.get_min_max();
+            float s_cal;
+            int32_t z_cal;
+            tq_calculate_symmetric_params(mn, mx, TQ_DTYPE_I8, &s_cal, &z_cal);
+            CHECK(qlin.set_static_activation_scale(s_cal, 1).is_err());
+            CHECK(qlin.set_static_activation_scale(s_cal, 0).is_ok());
+            CHECK(qlin.static_activation_scale() == s_cal);
+            auto ys = qlin.forward(Tensor::from_data(x, {m, k}).unwrap()).unwrap();
+            // with the scale of this very tensor the static path reproduces the dynamic one bit for bit
+            CHECK_SAME(ys.as_slice(), want);
+            // and with another scale it follows the oracle's per-tensor quantize (x * (1/scale) above 64 elements)
+            const float s2 = 3.0f / 127.0f;
+            CHECK(qlin.set_static_activation_scale(s2).is_ok());
+            auto y2 = qlin.forward(Tensor::from_data(x, {m, k}).unwrap()).unwrap();
+            std::vector<int8_t> aq2(m * k);
+            tq_quantize_to_int8_simd(x.data(), m * k, s2, 0, aq2.data());
+            tq_gemm_i8_nk(aq2.data(), wq.data(), m, n, k, acc.data());
+            std::vector<float> want2(m * n);
+            tq_linear_dequant_epilogue(acc.data(), m, n, &s2, 0, sw.data(), bias.data(), want2.data());
+            CHECK_SAME(y2.as_slice(), want2);
+            CHECK(qlin.set_static_activation_scale(0.0f).is_ok());  // back to dynamic
+            auto y3 = qlin.forward(Tensor::from_data(x, {m, k}).unwrap()).unwrap();
+            CHECK_SAME(y3.as_slice(), want);
+        }
     }
 }
 

@@ -244,3 +244,28 @@ def test_config5_full_size_projection_shapes(ctx, hipq, n, k):
     assert r.dtype == np.float32
     wantq = np.clip(r + np.float32(3), -128, 127).astype(np.int8)
     np.testing.assert_array_equal(q.cpu().numpy(), wantq)
+
+
+@pytest.mark.parametrize("m,n,k", [(48, 80, 256), (512, 512, 512), (2048, 768, 256), (5, 24, 48)])
+def test_linear_with_static_activation_scale(ctx, hipq, oracle, m, n, k):
+    """Static quantization: the activation scale comes from calibration (an observer), not from the input.  The
+    fused call equals the oracle's per-tensor quantize (both forms) -> int32 GEMM -> dequantize epilogue, and the
+    publishing quantize records the parameters it was given."""
+    rng = np.random.default_rng(m * 3 + n)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wq = rand_i8(rng, (n, k))
+    sw = (rng.random(n) * 0.002 + 0.0001).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    s_a = np.float32(4.0 / 127.0)  # clips the tail of N(0,1): saturation is part of the case
+    for mode, quantize in ((hipq.FORM_MUL_INV, oracle.quantize_to_int8_simd), (hipq.FORM_DIV, oracle.quantize_per_tensor_affine_i8)):
+        aq = quantize(x.ravel(), s_a, 0).reshape(m, k).astype(np.int8)
+        want = oracle.linear_dequant_epilogue(oracle.gemm_i8_nk(aq, wq), np.array([s_a], np.float32), sw, bias)
+        got = host(ctx.linear_static(dev(x), float(s_a), dev(wq), dev(sw), dev(bias), mode=mode))
+        np.testing.assert_array_equal(got, want)
+        q, params = ctx.quantize_static_per_tensor(dev(x), float(s_a), 0, mode)
+        np.testing.assert_array_equal(host(q), aq)
+        rec = ctx.read_qparams(params)
+        assert rec.scale == s_a and rec.zero_point == 0 and rec.status == hipq.SUCCESS
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.linear_static(dev(x), 0.0, dev(wq), dev(sw), dev(bias))
+    assert e.value.code == hipq.INVALID_ARGUMENT and "Scale must be positive" in str(e.value)

@@ -188,6 +188,13 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
         if (params->status != HIPQ_SUCCESS) return;
         scale = params->scale;
         zp = params->zero_point;
+    } else if (dyn.out_params && blockIdx.x == 0 && threadIdx.x == 0) {
+        // Parameters given by value, to be recorded on the device for the kernels that follow.
+        dyn.out_params->scale = scale;
+        dyn.out_params->zero_point = zp;
+        dyn.out_params->min_val = 0.0f;
+        dyn.out_params->max_val = 0.0f;
+        dyn.out_params->status = HIPQ_SUCCESS;
     }
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
     const float zpf = static_cast<float>(zp);
@@ -614,6 +621,21 @@ int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n,
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
     return launch_quantize<int8_t>(ctx, x, n, scale, zero_point, nullptr, mode, -128.0f, 127.0f, out);
+}
+
+int32_t hipq_quantize_static_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n, float scale,
+                                               int32_t zero_point, int32_t mode, int8_t *out,
+                                               hipq_qparams *out_params) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_scale(__func__, scale);
+    if (rc) return rc;
+    if ((rc = check_mode(__func__, mode))) return rc;
+    HIPQ_REQUIRE_PTR(out_params);
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out);
+    return launch_quantize<int8_t>(ctx, x, n, scale, zero_point, nullptr, mode, -128.0f, 127.0f, out,
+                                   DynamicRange{nullptr, 0, 0, 0, 0, out_params});
 }
 
 int32_t hipq_quantize_per_tensor_f32_u8(hipq_ctx *ctx, const float *x, size_t n, float scale, int32_t zero_point,

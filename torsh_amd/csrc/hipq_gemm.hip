@@ -485,4 +485,26 @@ int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t per_token
     return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
 }
 
+int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w, const float *w_scales,
+                               const float *bias, size_t m, size_t n, size_t k, int32_t mode, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_gemm_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(w);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    void *s = nullptr;
+    rc = scratch(ctx, kScratchHeader + m * k + 256, &s);
+    if (rc) return rc;
+    char *base = static_cast<char *>(s);
+    hipq_qparams *params = reinterpret_cast<hipq_qparams *>(base);
+    int8_t *qa = reinterpret_cast<int8_t *>(base + kScratchHeader);
+    rc = hipq_quantize_static_per_tensor_f32_i8(ctx, x, m * k, a_scale, 0, mode, qa, params);
+    if (rc) return rc;
+    return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
+}
+
 }  // extern "C"

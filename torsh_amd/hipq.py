@@ -99,6 +99,8 @@ _SIGNATURES = {
     "hipq_quantize_per_row_strided_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
     "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
+    "hipq_quantize_static_per_tensor_f32_i8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp, _vp],
+    "hipq_linear_static_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_add_layer_norm_quantize_f32_i8": [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_gelu_tanh_f32": [_vp, _vp, _sz, _vp],
@@ -429,6 +431,23 @@ class Context:
         out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
         self.call("hipq_linear_i8_f32", _ptr(a), _ptr(a_scale), int(a_scale.numel() > 1), _ptr(w), _ptr(w_scales),
                   _ptr(bias), m, n, k, _ptr(out))
+        return out
+
+    def quantize_static_per_tensor(self, x, scale, zp=0, mode=0, out=None, params=None):
+        """Per-tensor int8 quantize with given parameters, which are also recorded in a device-side record."""
+        out = out if out is not None else torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        params = params if params is not None else self.new_qparams()
+        self.call("hipq_quantize_static_per_tensor_f32_i8", _ptr(x), x.numel(), float(scale), int(zp), mode, _ptr(out),
+                  _ptr(params))
+        return out, params
+
+    def linear_static(self, x, a_scale, w, w_scales, bias=None, mode=0, out=None):
+        """Quantized Linear forward with a calibrated (static) per-tensor activation scale."""
+        m, k = x.shape
+        n, _ = w.shape
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_static_f32", _ptr(x), float(a_scale), _ptr(w), _ptr(w_scales), _ptr(bias), m, n, k, mode,
+                  _ptr(out))
         return out
 
     def linear_i8_i8(self, a, a_scale, w, w_scales, bias, out_scale, out_zp, mode=0, out=None):

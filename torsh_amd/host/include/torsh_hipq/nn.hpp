@@ -198,6 +198,13 @@ class QuantizedLinear : public Module {
         // Activations follow the reference's branch for their size: x*(1/scale) above 64 elements
         // (algorithms.rs:292), x/scale otherwise; per-token always divides (algorithms.rs:230).
         const int32_t mode = (act_ == ActivationQuant::PerTensor && m * in_ > 64) ? HIPQ_FORM_MUL_INV : HIPQ_FORM_DIV;
+        if (static_scale_ > 0.0f) {
+            TORSH_CHECK(hip::check(hipq_linear_static_f32(ctx_, dx.as<float>(), static_scale_, w_.as<int8_t>(),
+                                                          sw_.as<float>(), has_bias_ ? bias_.as<float>() : nullptr, m,
+                                                          out_, in_, mode, dy.as<float>())));
+            TORSH_TRY(ys, dy.to_host<float>(m * out_));
+            return Tensor::from_data(std::move(ys), std::move(out_dims));
+        }
         TORSH_CHECK(hip::check(hipq_linear_dynamic_f32(ctx_, dx.as<float>(), act_ == ActivationQuant::PerToken ? 1 : 0,
                                                        w_.as<int8_t>(), sw_.as<float>(),
                                                        has_bias_ ? bias_.as<float>() : nullptr, m, out_, in_, mode,
@@ -225,6 +232,19 @@ class QuantizedLinear : public Module {
     size_t in_features() const { return in_; }
     size_t out_features() const { return out_; }
 
+    // Static quantization: use a calibrated per-tensor activation scale (what
+    // Observer::calculate_qparams returned for a symmetric int8 scheme, zero point 0) instead of
+    // taking the range of every input.  A scale <= 0 switches back to dynamic quantization.
+    Result<bool> set_static_activation_scale(float scale, int32_t zero_point = 0) {
+        if (zero_point != 0)
+            return TorshError::invalid_argument("QuantizedLinear: a static activation scale needs a symmetric scheme (zero point 0)");
+        if (scale > 0.0f && act_ != ActivationQuant::PerTensor)
+            return TorshError::invalid_argument("QuantizedLinear: a static activation scale is per tensor");
+        static_scale_ = scale > 0.0f ? scale : 0.0f;
+        return true;
+    }
+    float static_activation_scale() const { return static_scale_; }
+
   private:
     QuantizedLinear() = default;
     hipq_ctx *ctx_ = nullptr;
@@ -232,6 +252,7 @@ class QuantizedLinear : public Module {
     ActivationQuant act_ = ActivationQuant::PerTensor;
     hip::DeviceBuffer w_, sw_, bias_;
     bool has_bias_ = false;
+    float static_scale_ = 0.0f;  // > 0: calibrated activation scale
 };
 
 class QuantizedConv2d : public Module {
