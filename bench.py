@@ -359,7 +359,14 @@ def main() -> int:
             i = rot()
             ctx.histogram(fx[i], -6.0, 6.0, 256, counts=hist)
 
-        for name, fn, bytes_per in (("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
+        def run_copy():
+            # not a kernel of this library: torch's device-to-device copy of the same tensors, as the
+            # bandwidth this box sustains on a plain stream (the yardstick beside the 8 TB/s datasheet figure)
+            i = rot()
+            fy[i].copy_(fx[i])
+
+        for name, fn, bytes_per in (("hbm_copy_reference_f32", run_copy, 8),
+                                    ("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
                                     ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9),
                                     ("quality_metrics_two_tensors_f32", run_metrics, 8),
                                     ("fake_quantize_metrics_fused_f32", run_fused_metrics, 4),
