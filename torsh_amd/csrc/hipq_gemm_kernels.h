@@ -423,6 +423,38 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     }
     if constexpr (EPI != EPI_I32)
         if (CONV || !ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
+    // Convolution: where each window's outputs go and the per-filter operands, also ahead of the
+    // main loop (the index arithmetic and the loads' latency hide behind it).  Rows are output
+    // channels, columns are padded-grid window positions; a lane owns one window.  Lane l of a
+    // row block fetches the operands of row l % 32 (three loads per block instead of three per
+    // accumulator register); the 16 rows a lane needs come back through shuffles in the epilogue.
+    size_t out_base[CONV ? FN : 1];
+    bool valid[CONV ? FN : 1];
+    float s_blk[CONV ? FM : 1], b_blk[CONV ? FM : 1];
+    int c_blk[CONV ? FM : 1];
+    if constexpr (CONV) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int q = nn[j];
+            const int per_img = ep.cv_hp * ep.cv_wp;
+            const int img = q / per_img, rem = q % per_img;
+            const int oh = rem / ep.cv_wp, ow = rem % ep.cv_wp;
+            valid[j] = q < N && oh < ep.cv_ho && ow < ep.cv_wo;
+            out_base[j] = (size_t(img) * ep.cv_oc * ep.cv_ho + oh) * ep.cv_wo + ow;  // + oc * ho * wo
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const int m = m0 + wm * TM + i * 32 + lane % 32;
+            const int mc = m < M ? m : M - 1;
+            c_blk[i] = ep.cv_corr_mul * ep.cv_wsum[mc];
+            s_blk[i] = 1.0f;
+            b_blk[i] = 0.0f;
+            if constexpr (EPI != EPI_I32) {
+                s_blk[i] = sa0 * ep.sw[mc];
+                if (ep.bias) b_blk[i] = ep.bias[mc];
+            }
+        }
+    }
 
     // LDS byte offsets (within a stage) of this lane's fragment reads.
     int offA[FM][KSW], offW[FN][KSW];
@@ -543,35 +575,7 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     if constexpr (CONV) {
         // Rows are output channels, columns are padded-grid window positions.  A lane owns one
         // window; consecutive lanes are consecutive ow, i.e. consecutive bytes of the NCHW output.
-        size_t out_base[FN];
-        bool valid[FN];
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int q = nn[j];
-            const int per_img = ep.cv_hp * ep.cv_wp;
-            const int img = q / per_img, rem = q % per_img;
-            const int oh = rem / ep.cv_wp, ow = rem % ep.cv_wp;
-            valid[j] = q < N && oh < ep.cv_ho && ow < ep.cv_wo;
-            out_base[j] = (size_t(img) * ep.cv_oc * ep.cv_ho + oh) * ep.cv_wo + ow;  // + oc * ho * wo
-        }
         const size_t plane = size_t(ep.cv_ho) * ep.cv_wo;
-        // Per-filter operands: lane l of a row block fetches those of row l % 32 (three loads per
-        // block instead of three per accumulator register); the 16 rows a lane needs come back
-        // through shuffles.
-        float s_blk[FM], b_blk[FM];
-        int c_blk[FM];
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            const int m = m0 + wm * TM + i * 32 + lane % 32;
-            const int mc = m < M ? m : M - 1;
-            c_blk[i] = ep.cv_corr_mul * ep.cv_wsum[mc];
-            s_blk[i] = 1.0f;
-            b_blk[i] = 0.0f;
-            if constexpr (EPI != EPI_I32) {
-                s_blk[i] = sa0 * ep.sw[mc];
-                if (has_bias) b_blk[i] = ep.bias[mc];
-            }
-        }
         wait_vmcnt<0>();
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
