@@ -372,6 +372,10 @@ HIPQ_API int32_t hipq_qrelu_u8(hipq_ctx *ctx, const uint8_t *q, int32_t is_signe
  * without it the value stays in its f32 carrier and a NaN stays a NaN
  * (crates/torsh-quantization/src/simd_ops.rs:36-46). */
 enum { HIPQ_FAKE_INT_CAST = 4 };
+/* Or (not both): the clamp is `.max(qmin).min(qmax)`, under which a NaN becomes qmin, and the
+ * value is dequantized as scale * (q - zp): fake_quantize_per_tensor_affine,
+ * crates/torsh-quantization/src/fake_quantize.rs:14-42 (use with HIPQ_FORM_DIV). */
+enum { HIPQ_FAKE_NAN_TO_QMIN = 8 };
 
 /* QuantizationMetrics, crates/torsh-quantization/src/metrics.rs:30-48 (same
  * fields, same order). */
@@ -399,7 +403,7 @@ HIPQ_API int32_t hipq_quantization_metrics_f32(hipq_ctx *ctx, const float *origi
  * (crates/torsh-models/src/quantization.rs:504-533) fused into one pass over x:
  * the dequantized image is formed in registers and never written.  Quantizer:
  * q = clamp(round(x * (1/scale) | x / scale) + zp, qmin, qmax), y = (q - zp) * scale;
- * `mode` = HIPQ_ROUND_* | HIPQ_FORM_* | HIPQ_FAKE_INT_CAST.  `params` (device,
+ * `mode` = HIPQ_ROUND_* | HIPQ_FORM_* | HIPQ_FAKE_INT_CAST or HIPQ_FAKE_NAN_TO_QMIN.  `params` (device,
  * may be NULL) overrides scale and zero_point. */
 HIPQ_API int32_t hipq_fake_quantize_metrics_f32(hipq_ctx *ctx, const float *x, size_t n, float scale,
                                                 int32_t zero_point, const hipq_qparams *params, int32_t qmin,

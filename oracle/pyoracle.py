@@ -85,6 +85,11 @@ def _declare(l: C.CDLL) -> None:
     l.tq_model_calculate_quantization_params.restype = None
     l.tq_model_calculate_quantization_params.argtypes = [C.c_float, C.c_float, C.c_int32, C.c_int32, _f32p, _i32p,
                                                          _f32p, _f32p]
+    l.tq_fake_quantize_per_tensor_affine.restype = None
+    l.tq_fake_quantize_per_tensor_affine.argtypes = [_f32p, C.c_size_t, C.c_float, C.c_int32, C.c_int32, C.c_int32, _f32p]
+    l.tq_fake_quantize_auto.restype = C.c_int
+    l.tq_fake_quantize_auto.argtypes = [_f32p, C.c_size_t, C.c_int, C.c_int, _f32p, C.POINTER(C.c_float),
+                                        C.POINTER(C.c_int32)]
     l.tq_model_fake_quantize.restype = None
     l.tq_model_fake_quantize.argtypes = [_f32p, C.c_size_t, C.c_float, C.c_int32, C.c_int32, C.c_int32, _f32p]
     l.tq_quantize_int4_per_tensor.argtypes = [_f32p, C.c_size_t, _f32p, _f32p, _i32p]
@@ -557,6 +562,24 @@ def model_fake_quantize(x, scale, zp, qmin=-128, qmax=127) -> np.ndarray:
     lib().tq_model_fake_quantize(_p(x, _f32p), C.c_size_t(x.size), C.c_float(scale), int(zp), qmin, qmax,
                                  _p(out, _f32p))
     return out
+
+
+def fake_quantize_per_tensor_affine(x, scale, zp, qmin=-128, qmax=127) -> np.ndarray:
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().tq_fake_quantize_per_tensor_affine(_p(x, _f32p), C.c_size_t(x.size), C.c_float(scale), int(zp), qmin, qmax,
+                                             _p(out, _f32p))
+    return out
+
+
+def fake_quantize_auto(x, dtype=DTYPE_I8, scheme=0):
+    """scheme 0 = PerTensorAffine, 1 = PerTensorSymmetric.  Returns (out, scale, zero_point)."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    s, z = C.c_float(), C.c_int32()
+    _check(lib().tq_fake_quantize_auto(_p(x, _f32p), C.c_size_t(x.size), dtype, scheme, _p(out, _f32p), C.byref(s),
+                                       C.byref(z)), "fake_quantize_auto")
+    return out, float(s.value), int(z.value)
 
 
 def model_mse_error(original, quantized) -> float:

@@ -382,6 +382,52 @@ void tq_model_fake_quantize(const float *x, size_t n, float scale, int32_t zp, i
     }
 }
 
+/* f32::max / f32::min of Rust: the operand that is not NaN. */
+static float rust_max(float a, float b) { return (a != a) ? b : ((b != b) ? a : (a > b ? a : b)); }
+static float rust_min(float a, float b) { return (a != a) ? b : ((b != b) ? a : (a < b ? a : b)); }
+
+/* crates/torsh-quantization/src/fake_quantize.rs:14-42 */
+void tq_fake_quantize_per_tensor_affine(const float *x, size_t n, float scale, int32_t zp, int32_t qmin,
+                                        int32_t qmax, float *out) {
+    for (size_t i = 0; i < n; ++i) {
+        const float quantized = roundf(x[i] / scale) + (float)zp;                     /* :27 */
+        const float clamped = rust_min(rust_max(quantized, (float)qmin), (float)qmax); /* :29 */
+        out[i] = scale * (clamped - (float)zp);                                       /* :31 */
+    }
+}
+
+/* crates/torsh-quantization/src/fake_quantize.rs:119-157; dtype TQ_DTYPE_I8 = 0 / TQ_DTYPE_U8 = 1,
+ * scheme 0 = PerTensorAffine, 1 = PerTensorSymmetric (the others are errors there). */
+int tq_fake_quantize_auto(const float *x, size_t n, int dtype, int scheme, float *out, float *out_scale,
+                          int32_t *out_zp) {
+    int32_t qmin, qmax;
+    if (dtype == 0) {
+        qmin = -128, qmax = 127;
+    } else if (dtype == 1) {
+        qmin = 0, qmax = 255;
+    } else {
+        return 1; /* "Unsupported quantization dtype" */
+    }
+    float mn = INFINITY, mx = -INFINITY;
+    for (size_t i = 0; i < n; ++i) mn = rust_min(mn, x[i]);  /* :132 */
+    mn = rust_min(mn, 0.0f);
+    for (size_t i = 0; i < n; ++i) mx = rust_max(mx, x[i]);  /* :133-136 */
+    mx = rust_max(mx, 0.0f);
+    float scale = (mx - mn) / (float)(qmax - qmin);          /* :138 */
+    if (scale == 0.0f) scale = 1.0f;                         /* :139 */
+    int32_t zp = 0;
+    if (scheme == 0) {
+        const float z = rust_min(rust_max(roundf((float)qmin - mn / scale), (float)qmin), (float)qmax); /* :143-146 */
+        zp = (int32_t)z;
+    } else if (scheme != 1) {
+        return 1; /* "Quantization scheme not yet implemented" */
+    }
+    if (out_scale) *out_scale = scale;
+    if (out_zp) *out_zp = zp;
+    tq_fake_quantize_per_tensor_affine(x, n, scale, zp, qmin, qmax, out);
+    return 0;
+}
+
 /* crates/torsh-models/src/quantization.rs:548-566 */
 double tq_model_mse_error(const float *original, const float *quantized, size_t n) {
     float sum = 0.0f;

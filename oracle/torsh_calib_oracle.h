@@ -83,6 +83,15 @@ void tq_model_calculate_quantization_params(float min_val, float max_val, int32_
  * dequantize_value per element ("fake quantization"). */
 void tq_model_fake_quantize(const float *x, size_t n, float scale, int32_t zp, int32_t qmin, int32_t qmax,
                             float *out);
+/* ---- QAT fake quantization: crates/torsh-quantization/src/fake_quantize.rs ---- */
+/* fake_quantize_per_tensor_affine, fake_quantize.rs:14-42: round(x / scale) + zp, clamped with
+ * f32::max then f32::min (a NaN becomes qmin), out = scale * (clamped - zp). */
+void tq_fake_quantize_per_tensor_affine(const float *x, size_t n, float scale, int32_t zp, int32_t qmin,
+                                        int32_t qmax, float *out);
+/* fake_quantize_auto, fake_quantize.rs:119-157 (range widened to include 0, scale 0 -> 1).
+ * Returns non-zero for a dtype or scheme the reference rejects. */
+int tq_fake_quantize_auto(const float *x, size_t n, int dtype, int scheme, float *out, float *out_scale,
+                          int32_t *out_zp);
 /* ModelQuantizer::calculate_mse_error, quantization.rs:548-566 (f32 sum, result widened). */
 double tq_model_mse_error(const float *original, const float *quantized, size_t n);
 

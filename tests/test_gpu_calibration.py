@@ -149,6 +149,31 @@ def test_fake_quantize_nan_semantics_and_errors(ctx, hipq, oracle):
         ctx.fake_quantize(dev(x), 1.0, 0, mode=64)
 
 
+@pytest.mark.parametrize("n", [1, 7, 4096, 4099, (1 << 20) + 3])
+@pytest.mark.parametrize("qrange", [(-128, 127), (0, 255)])
+def test_qat_fake_quantize_matches_reference_formula(ctx, hipq, oracle, n, qrange):
+    """fake_quantize_per_tensor_affine of the QAT module: division form, clamp by max-then-min (a NaN becomes qmin),
+    scale * (q - zp).  Bit-exact against the oracle, ties, saturation and non-finite inputs included."""
+    qmin, qmax = qrange
+    x = normal(300 + n, n, 2.0)
+    special = np.float32([np.nan, np.inf, -np.inf, 0.25, -0.25, 0.75, 1e9, -1e9])
+    x[: min(n, special.size)] = special[: min(n, special.size)]
+    scale, zp = 0.5 if n % 2 else 0.0173, 3
+    mode = hipq.FORM_DIV | hipq.FAKE_NAN_TO_QMIN
+    want = oracle.fake_quantize_per_tensor_affine(x, scale, zp, qmin, qmax)
+    got = host(ctx.fake_quantize(dev(x), scale, zp, qmin, qmax, mode))
+    np.testing.assert_array_equal(got, want)
+    assert not np.isnan(got).any()
+    # the fused form measures exactly that image
+    finite = np.where(np.isfinite(x), x, np.float32(0.0)).astype(np.float32)
+    want_m = oracle.calculate_quantization_metrics_f64(finite, oracle.fake_quantize_per_tensor_affine(finite, scale, zp, qmin, qmax))
+    got_m = ctx.read_metrics(ctx.fake_quantize_metrics(dev(finite), scale, zp, qmin, qmax, mode))
+    for key in ("mse", "mae", "max_error", "cosine_similarity"):
+        assert got_m[key] == pytest.approx(want_m[key], rel=1e-6, abs=1e-12), key
+    with pytest.raises(hipq.HipqError):
+        ctx.fake_quantize(dev(x), scale, zp, qmin, qmax, hipq.FAKE_INT_CAST | hipq.FAKE_NAN_TO_QMIN)
+
+
 # ---- observers -------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("n", [1, 63, 4096, 4097, 1 << 20, (1 << 22) + 5])

@@ -25,6 +25,7 @@ CPU_CASES = [
     "test_weight_file_round_trip_and_corruption",
     "test_model_quantizer_scalar_logic",
     "test_kernel_plugin_interface",
+    "test_fake_quantize_errors_before_the_device",
 ]
 GPU_CASES = [
     "test_quantize_per_tensor_affine",
@@ -53,6 +54,8 @@ GPU_CASES = [
     "parity_special_schemes",
     "parity_backend_qadd_qrelu",
     "test_kernel_plugin_dispatch",
+    "test_fake_quantize",
+    "parity_fake_quantize",
 ]
 
 

@@ -436,3 +436,62 @@ def test_group_wise_equals_grouped_slices(oracle):
     np.testing.assert_array_equal(qg, q4)
     np.testing.assert_array_equal(sg, s4)
     np.testing.assert_array_equal(zg, z4)
+
+
+def test_fake_quantize_known_answers(oracle, cal):
+    """What the reference's own tests assert for fake_quantize.rs (ranges and lengths)."""
+    for case in cal["fake_quantize"]:
+        x = np.array(case["x"], np.float32)
+        want = case["assert"]
+        if case["fn"] == "fake_quantize_auto":
+            y, scale, zp = oracle.fake_quantize_auto(x, oracle.DTYPE_I8, 0)
+            assert len(y) == want["len"] and scale > 0 and -128 <= zp <= 127
+            assert all(want["range"][0] <= v <= want["range"][1] for v in y)
+        else:
+            y = oracle.fake_quantize_per_tensor_affine(x, case["scale"], case.get("zero_point", 0))
+            assert len(y) == len(x)
+            if want.get("abs_error_le_scale"):
+                assert np.all(np.abs(y - x) <= np.float32(case["scale"]))
+
+
+def test_fake_quantize_closed_form(oracle):
+    """Hand values: a dropped zero point, a clamp in the wrong order, round-half-even or the multiply form each
+    change one of them."""
+    # scale 0.5, zp 3: q = round(x / 0.5) + 3 clamped to [-128, 127]; y = 0.5 * (q - 3)
+    x = np.array([0.25, -0.25, 0.75, 1e9, -1e9, np.nan, np.inf, -np.inf, 0.0], np.float32)
+    want = np.array([0.5, -0.5, 1.0, 62.0, -65.5, -65.5, 62.0, -65.5, 0.0], np.float32)  # ties away; NaN -> qmin
+    np.testing.assert_array_equal(oracle.fake_quantize_per_tensor_affine(x, 0.5, 3), want)
+    # uint8 range, zp 10: negative inputs saturate at (0 - 10) * scale
+    y = oracle.fake_quantize_per_tensor_affine(np.array([-100.0, 3.0, 1000.0], np.float32), 2.0, 10, 0, 255)
+    np.testing.assert_array_equal(y, np.array([-20.0, 4.0, 490.0], np.float32))  # 3/2 = 1.5 -> 2 -> (12 - 10) * 2
+    # division, not multiplication by the reciprocal: 3 * (1/0.3f) rounds differently from 3 / 0.3f in f32 for some x;
+    # scan for such an x and check it went through the division
+    s = np.float32(0.3)
+    xs = (np.arange(1, 20001, dtype=np.float32) * np.float32(0.05)).astype(np.float32)
+    div = np.round(xs / s)  # not used for ties here: pick non-tie disagreements
+    mul = np.round(xs * (np.float32(1.0) / s))
+    idx = np.nonzero((div != mul) & (np.abs(xs / s - np.trunc(xs / s)) != 0.5))[0]
+    assert idx.size > 0
+    pick = xs[idx[:8]]
+    got = oracle.fake_quantize_per_tensor_affine(pick, float(s), 0, -(2 ** 20), 2 ** 20)
+    np.testing.assert_array_equal(got, s * div[idx[:8]].astype(np.float32))
+
+
+def test_fake_quantize_auto_closed_form(oracle):
+    # [-2, 2] -> I8 affine: scale 4/255; zp = round(-128 + 2/scale) = round(-0.5) = -1 (half away from zero)
+    y, scale, zp = oracle.fake_quantize_auto(np.array([-2, -1, 0, 1, 2], np.float32), oracle.DTYPE_I8, 0)
+    assert scale == np.float32(4.0) / np.float32(255.0) and zp == -1
+    # the range always includes 0: all-positive data keeps min = 0 -> zp = qmin
+    y, scale, zp = oracle.fake_quantize_auto(np.array([1.0, 3.0], np.float32), oracle.DTYPE_U8, 0)
+    assert scale == np.float32(3.0) / np.float32(255.0) and zp == 0
+    np.testing.assert_array_equal(y, oracle.fake_quantize_per_tensor_affine(np.array([1.0, 3.0], np.float32), scale, 0, 0, 255))
+    # constant zero: scale 0 becomes 1
+    y, scale, zp = oracle.fake_quantize_auto(np.zeros(5, np.float32), oracle.DTYPE_I8, 0)
+    assert scale == 1.0 and np.all(y == 0)
+    # symmetric: same scale formula (not absmax / 127), zero point 0
+    y, scale, zp = oracle.fake_quantize_auto(np.array([-1.0, 3.0], np.float32), oracle.DTYPE_I8, 1)
+    assert scale == np.float32(4.0) / np.float32(255.0) and zp == 0
+    # dtypes and schemes the reference rejects
+    for dtype, scheme in ((5, 0), (oracle.DTYPE_I8, 2)):
+        with pytest.raises(Exception):
+            oracle.fake_quantize_auto(np.ones(3, np.float32), dtype, scheme)

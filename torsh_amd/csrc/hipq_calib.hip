@@ -81,16 +81,24 @@ __device__ __forceinline__ void block_store_sums(const MetricLane &m, MetricSums
 // The fake-quantized image of one value: quantize (either form), then dequantize.
 //   carrier form: clamp(round(..) + zp) stays f32, y = (q - zp) * scale
 //       (crates/torsh-quantization/src/simd_ops.rs:36-46, 52-81)
-//   INT_CAST:     the clamped value goes through `as i32` (NaN -> 0), y = (q - zp) as f32 * scale
+//   FQ_INT_CAST:  the clamped value goes through `as i32` (NaN -> 0), y = (q - zp) as f32 * scale
 //       (crates/torsh-models/src/quantization.rs:336-347)
-template <bool DIV, bool EVEN, bool INT_CAST>
+//   FQ_MAX_MIN:   the clamp is `.max(qmin).min(qmax)`, which maps NaN to qmin, y = scale * (q - zp)
+//       (crates/torsh-quantization/src/fake_quantize.rs:24-33)
+enum { FQ_CARRIER = 0, FQ_INT_CAST = 1, FQ_MAX_MIN = 2 };
+template <bool DIV, bool EVEN, int KIND>
 __device__ __forceinline__ float fake_quantize_value(float x, float scale, float inv, int zp, float zpf, float lo,
                                                      float hi) {
-    float q = quantize_value<DIV, EVEN>(x, scale, inv, zpf, lo, hi);
-    if constexpr (INT_CAST) {
-        return static_cast<float>(cvt_i32_sat(q) - zp) * scale;
+    if constexpr (KIND == FQ_MAX_MIN) {
+        const float q = quantize_value<DIV, EVEN>(x, scale, inv, zpf, -INFINITY, INFINITY);
+        return scale * (fminf(fmaxf(q, lo), hi) - zpf);  // fmaxf / fminf return the operand that is not NaN
     } else {
-        return (q - zpf) * scale;
+        const float q = quantize_value<DIV, EVEN>(x, scale, inv, zpf, lo, hi);
+        if constexpr (KIND == FQ_INT_CAST) {
+            return static_cast<float>(cvt_i32_sat(q) - zp) * scale;
+        } else {
+            return (q - zpf) * scale;
+        }
     }
 }
 
@@ -111,7 +119,7 @@ __global__ __launch_bounds__(kCalBlock) void metrics_partial_kernel(const float 
     block_store_sums(m, partials + blockIdx.x);
 }
 
-template <bool DIV, bool EVEN, bool INT_CAST>
+template <bool DIV, bool EVEN, int KIND>
 __global__ __launch_bounds__(kCalBlock) void fake_quant_metrics_partial_kernel(const float *__restrict__ x, size_t n,
                                                                                 FakeQuantArgs fq,
                                                                                 MetricSums *__restrict__ partials) {
@@ -122,7 +130,7 @@ __global__ __launch_bounds__(kCalBlock) void fake_quant_metrics_partial_kernel(c
     const float scale = fq.scale, zpf = static_cast<float>(fq.zp);
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
     MetricLane m;
-    auto fqv = [&](float v) { return fake_quantize_value<DIV, EVEN, INT_CAST>(v, scale, inv, fq.zp, zpf, fq.lo, fq.hi); };
+    auto fqv = [&](float v) { return fake_quantize_value<DIV, EVEN, KIND>(v, scale, inv, fq.zp, zpf, fq.lo, fq.hi); };
     stream1<kCalBlock>(
         x, n,
         [&](const float4 &v, size_t) { m.add4(v, make_float4(fqv(v.x), fqv(v.y), fqv(v.z), fqv(v.w))); },
@@ -190,7 +198,7 @@ __global__ __launch_bounds__(kCalBlock) void metrics_final_kernel(const MetricSu
     *out = q;
 }
 
-template <bool DIV, bool EVEN, bool INT_CAST>
+template <bool DIV, bool EVEN, int KIND>
 __global__ __launch_bounds__(kCalBlock) void fake_quantize_kernel(const float *__restrict__ x, size_t n,
                                                                    FakeQuantArgs fq, float *__restrict__ out) {
     if (fq.params) {
@@ -200,7 +208,7 @@ __global__ __launch_bounds__(kCalBlock) void fake_quantize_kernel(const float *_
     }
     const float scale = fq.scale, zpf = static_cast<float>(fq.zp);
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
-    auto fqv = [&](float v) { return fake_quantize_value<DIV, EVEN, INT_CAST>(v, scale, inv, fq.zp, zpf, fq.lo, fq.hi); };
+    auto fqv = [&](float v) { return fake_quantize_value<DIV, EVEN, KIND>(v, scale, inv, fq.zp, zpf, fq.lo, fq.hi); };
     const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     if (out_aligned) {
         stream1<kCalBlock>(
@@ -386,21 +394,29 @@ static int32_t launch_metrics_final(hipq_ctx *ctx, const MetricSums *partials, i
     return check_launch("metrics_final_kernel");
 }
 
-template <bool DIV, bool EVEN>
-static void launch_fq_metrics(bool int_cast, int grid, hipStream_t s, const float *x, size_t n, FakeQuantArgs fq,
-                              MetricSums *partials) {
-    if (int_cast)
-        fake_quant_metrics_partial_kernel<DIV, EVEN, true><<<grid, kCalBlock, 0, s>>>(x, n, fq, partials);
-    else
-        fake_quant_metrics_partial_kernel<DIV, EVEN, false><<<grid, kCalBlock, 0, s>>>(x, n, fq, partials);
+static int fq_kind(int32_t mode) {
+    return (mode & HIPQ_FAKE_INT_CAST) ? FQ_INT_CAST : ((mode & HIPQ_FAKE_NAN_TO_QMIN) ? FQ_MAX_MIN : FQ_CARRIER);
 }
 
 template <bool DIV, bool EVEN>
-static void launch_fq(bool int_cast, int grid, hipStream_t s, const float *x, size_t n, FakeQuantArgs fq, float *out) {
-    if (int_cast)
-        fake_quantize_kernel<DIV, EVEN, true><<<grid, kCalBlock, 0, s>>>(x, n, fq, out);
+static void launch_fq_metrics(int kind, int grid, hipStream_t s, const float *x, size_t n, FakeQuantArgs fq,
+                              MetricSums *partials) {
+    if (kind == FQ_INT_CAST)
+        fake_quant_metrics_partial_kernel<DIV, EVEN, FQ_INT_CAST><<<grid, kCalBlock, 0, s>>>(x, n, fq, partials);
+    else if (kind == FQ_MAX_MIN)
+        fake_quant_metrics_partial_kernel<DIV, EVEN, FQ_MAX_MIN><<<grid, kCalBlock, 0, s>>>(x, n, fq, partials);
     else
-        fake_quantize_kernel<DIV, EVEN, false><<<grid, kCalBlock, 0, s>>>(x, n, fq, out);
+        fake_quant_metrics_partial_kernel<DIV, EVEN, FQ_CARRIER><<<grid, kCalBlock, 0, s>>>(x, n, fq, partials);
+}
+
+template <bool DIV, bool EVEN>
+static void launch_fq(int kind, int grid, hipStream_t s, const float *x, size_t n, FakeQuantArgs fq, float *out) {
+    if (kind == FQ_INT_CAST)
+        fake_quantize_kernel<DIV, EVEN, FQ_INT_CAST><<<grid, kCalBlock, 0, s>>>(x, n, fq, out);
+    else if (kind == FQ_MAX_MIN)
+        fake_quantize_kernel<DIV, EVEN, FQ_MAX_MIN><<<grid, kCalBlock, 0, s>>>(x, n, fq, out);
+    else
+        fake_quantize_kernel<DIV, EVEN, FQ_CARRIER><<<grid, kCalBlock, 0, s>>>(x, n, fq, out);
 }
 
 static int32_t check_fake_quant_args(const char *fn, float scale, const hipq_qparams *params, int32_t qmin,
@@ -408,8 +424,10 @@ static int32_t check_fake_quant_args(const char *fn, float scale, const hipq_qpa
     if (!params && !(scale > 0.0f))
         return fail(HIPQ_INVALID_ARGUMENT, "%s: Scale must be positive, got %g", fn, static_cast<double>(scale));
     if (qmin > qmax) return fail(HIPQ_INVALID_ARGUMENT, "%s: qmin %d > qmax %d", fn, qmin, qmax);
-    if (mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV | HIPQ_FAKE_INT_CAST))
+    if (mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV | HIPQ_FAKE_INT_CAST | HIPQ_FAKE_NAN_TO_QMIN))
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits 0x%x", fn, mode);
+    if ((mode & HIPQ_FAKE_INT_CAST) && (mode & HIPQ_FAKE_NAN_TO_QMIN))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: HIPQ_FAKE_INT_CAST and HIPQ_FAKE_NAN_TO_QMIN exclude each other", fn);
     return HIPQ_SUCCESS;
 }
 
@@ -461,7 +479,7 @@ int32_t hipq_fake_quantize_metrics_f32(hipq_ctx *ctx, const float *x, size_t n, 
     MetricSums *partials = reinterpret_cast<MetricSums *>(static_cast<char *>(scr) + kScratchHeader);
     if (grid) {
         const FakeQuantArgs fq{scale, zero_point, static_cast<float>(qmin), static_cast<float>(qmax), params};
-        const bool ic = (mode & HIPQ_FAKE_INT_CAST) != 0;
+        const int ic = fq_kind(mode);
         const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
         if (div && even)
             launch_fq_metrics<true, true>(ic, grid, ctx->stream, x, n, fq, partials);
@@ -487,7 +505,7 @@ int32_t hipq_fake_quantize_f32(hipq_ctx *ctx, const float *x, size_t n, float sc
     HIPQ_REQUIRE_PTR(out);
     const int grid = calib_grid(ctx, n, kCalTile * 4);
     const FakeQuantArgs fq{scale, zero_point, static_cast<float>(qmin), static_cast<float>(qmax), params};
-    const bool ic = (mode & HIPQ_FAKE_INT_CAST) != 0;
+    const int ic = fq_kind(mode);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
     if (div && even)
         launch_fq<true, true>(ic, grid, ctx->stream, x, n, fq, out);

@@ -22,6 +22,7 @@ FORM_MUL_INV, FORM_DIV = 0, 2
 DTYPE_I8, DTYPE_U8 = 0, 1
 PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC, PARAMS_ZERO_INCLUDED = range(5)
 FAKE_INT_CAST = 4
+FAKE_NAN_TO_QMIN = 8
 HISTOGRAM_MAX_BINS = 16384
 
 
