@@ -268,6 +268,11 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
                                         const float *a_scale, int32_t a_scale_per_row, const float *w_scales,
                                         const float *bias, float out_scale, int32_t out_zero_point,
                                         int32_t mode, int8_t *out);
+/* Test and tuning hook with no counterpart in the reference: forces one of the GEMM kernel forms
+ * for every later call of this process wherever the shape allows it (0 = automatic choice, the
+ * default; 1-3 one-tile-per-workgroup forms, 5-8 persistent forms, 10 register-staged form).
+ * Results do not depend on it; the parity tests use it to run every form on the same inputs. */
+HIPQ_API int32_t hipq_set_gemm_kernel_variant(int32_t variant);
 /* Whole forward of a quantized Linear with a static (calibrated) activation scale: the scale an
  * observer derived beforehand (Observer::calculate_qparams, crates/torsh-quantization/src/observers.rs:263-310,
  * symmetric: zero point 0) instead of a range pass over every input - per-tensor quantize

@@ -269,3 +269,31 @@ def test_linear_with_static_activation_scale(ctx, hipq, oracle, m, n, k):
     with pytest.raises(hipq.HipqError) as e:
         ctx.linear_static(dev(x), 0.0, dev(wq), dev(sw), dev(bias))
     assert e.value.code == hipq.INVALID_ARGUMENT and "Scale must be positive" in str(e.value)
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 10])
+def test_every_gemm_kernel_form_gives_the_same_bits(ctx, hipq, oracle, variant):
+    """The kernel form is a performance choice only: each form, forced on shapes it would not be picked for, gives
+    the oracle's accumulators and epilogue outputs bit for bit (interior and ragged tiles, all four epilogues)."""
+    try:
+        ctx.set_gemm_kernel_variant(variant)
+        for (m, n, k) in ((300, 200, 256), (1024, 768, 512), (130, 2304, 256)):
+            rng = np.random.default_rng(variant * 1000 + m)
+            a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+            acc = oracle.gemm_i8_nk(a, w)
+            np.testing.assert_array_equal(host(ctx.gemm_i8_i32(dev(a), dev(w))), acc)
+            sa = (rng.random(m) * 0.05 + 0.001).astype(np.float32)
+            sw = (rng.random(n) * 0.002 + 0.0001).astype(np.float32)
+            bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+            want = oracle.linear_dequant_epilogue(acc, sa, sw, bias)
+            np.testing.assert_array_equal(host(ctx.linear_i8_f32(dev(a), dev(sa), dev(w), dev(sw), dev(bias))), want)
+            res = rng.standard_normal((m, n)).astype(np.float32)
+            got = host(ctx.linear_i8_f32_residual(dev(a), dev(sa), dev(w), dev(sw), dev(bias), dev(res)))
+            np.testing.assert_array_equal(got, want + res)
+            s_out, _ = oracle.calculate_symmetric_params(*oracle.find_min_max(want), 0)
+            wantq = oracle.requantize_epilogue(acc, sa, sw, bias, s_out, -5)
+            np.testing.assert_array_equal(host(ctx.linear_i8_i8(dev(a), dev(sa), dev(w), dev(sw), dev(bias), s_out, -5)), wantq)
+    finally:
+        ctx.set_gemm_kernel_variant(0)
+    with pytest.raises(hipq.HipqError):
+        ctx.set_gemm_kernel_variant(99)

@@ -285,14 +285,15 @@ static void launch_tile(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, 
                        ctx->stream, a, w, M, N, K, placed);
 }
 
-// Tuning hook: HIPQ_GEMM_VARIANT=<n> forces one kernel configuration (0 = automatic).
+// Tuning and test hook: HIPQ_GEMM_VARIANT=<n> in the environment, or hipq_set_gemm_kernel_variant(n),
+// forces one kernel configuration wherever the shape allows it (0 = automatic).
+static int g_gemm_variant = -1;
 static int gemm_variant_override() {
-    static int v = -1;
-    if (v < 0) {
+    if (g_gemm_variant < 0) {
         const char *e = getenv("HIPQ_GEMM_VARIANT");
-        v = e ? atoi(e) : 0;
+        g_gemm_variant = e ? atoi(e) : 0;
     }
-    return v;
+    return g_gemm_variant;
 }
 
 template <int EPI, bool EVEN>
@@ -483,6 +484,12 @@ int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t per_token
     if (rc) return rc;
     // hipq_qparams starts with the f32 scale.
     return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
+}
+
+int32_t hipq_set_gemm_kernel_variant(int32_t variant) {
+    if (variant < 0 || variant > 10) return fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..10", __func__, variant);
+    g_gemm_variant = variant;
+    return HIPQ_SUCCESS;
 }
 
 int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w, const float *w_scales,

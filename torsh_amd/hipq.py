@@ -101,6 +101,7 @@ _SIGNATURES = {
     "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
     "hipq_quantize_static_per_tensor_f32_i8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp, _vp],
+    "hipq_set_gemm_kernel_variant": [_i32],
     "hipq_linear_static_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_add_layer_norm_quantize_f32_i8": [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
@@ -206,6 +207,10 @@ class Context:
 
     def call(self, name: str, *args) -> None:
         _check(getattr(self._lib, name)(self.handle, *args))
+
+    def set_gemm_kernel_variant(self, variant: int) -> None:
+        """Test / tuning hook: force one GEMM kernel form for later calls (0 = automatic)."""
+        _check(self._lib.hipq_set_gemm_kernel_variant(int(variant)))
 
     def synchronize(self) -> None:
         self.call("hipq_ctx_synchronize")
