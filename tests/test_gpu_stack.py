@@ -197,3 +197,35 @@ def test_projection_stack_full_size_equals_its_parts(ctx, hipq):
     torch.cuda.synchronize()
     assert torch.isfinite(got).all()
     assert torch.equal(got, x)
+
+
+def test_row_kernels_with_more_rows_than_resident_workgroups(ctx, oracle):
+    """Above 8 workgroups per compute unit worth of rows the row kernels switch to a grid-stride form that
+    prefetches the next row: same results as the one-row-per-wave form, checked on 9001 rows (the last row group is
+    ragged) against the oracle and against the unfused kernels."""
+    rows = 9001
+    rng = np.random.default_rng(rows)
+    for cols in (768, 3072):
+        x = (rng.standard_normal((rows, cols)) * 2 + 0.3).astype(np.float32)
+        gamma = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+        beta = (rng.standard_normal(cols) * 0.1).astype(np.float32)
+        xd, gd, bd = dev(x), dev(gamma), dev(beta)
+        y = ctx.layer_norm(xd, gd, bd, 1e-5)
+        np.testing.assert_allclose(host(y), oracle.layer_norm(x, gamma, beta, 1e-5), rtol=1e-5, atol=LN_ATOL)
+        q_ref, s_ref, _, _ = ctx.quantize_per_row(y)
+        q, s = ctx.layer_norm_quantize(xd, gd, bd, 1e-5)
+        np.testing.assert_array_equal(host(s), host(s_ref))
+        np.testing.assert_array_equal(host(q), host(q_ref))
+        delta = rng.standard_normal((rows, cols)).astype(np.float32)
+        xs = dev(x)
+        q2, s2 = ctx.add_layer_norm_quantize(xs, dev(delta), gd, bd, 1e-5)
+        np.testing.assert_array_equal(host(xs), x + delta)
+        q3, s3 = ctx.layer_norm_quantize(dev(x + delta), gd, bd, 1e-5)
+        np.testing.assert_array_equal(host(s2), host(s3))
+        np.testing.assert_array_equal(host(q2), host(q3))
+        g = ctx.gelu_tanh(xd)
+        np.testing.assert_allclose(host(g), oracle.gelu_tanh(x), rtol=GELU_RTOL, atol=1e-7)
+        qg_ref, sg_ref, _, _ = ctx.quantize_per_row(g)
+        qg, sg = ctx.gelu_tanh_quantize(xd)
+        np.testing.assert_array_equal(host(sg), host(sg_ref))
+        np.testing.assert_array_equal(host(qg), host(qg_ref))
