@@ -330,7 +330,7 @@ HIPQ_API int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int
 /* ---- fp32 helpers of the int8 transformer stack ------------------------- */
 /* LayerNorm over the last dimension (biased variance, eps inside the square
  * root, eps 1e-5 by default: crates/torsh-nn/src/layers/normalization/layer_group/mod.rs:130-166,660).
- * gamma / beta [cols] may be NULL.  cols % 4 == 0, cols <= 8192. */
+ * gamma / beta [cols] may be NULL.  cols % 4 == 0, cols <= 12288 (a row is held in registers). */
 HIPQ_API int32_t hipq_layer_norm_f32(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, const float *gamma,
                                      const float *beta, float eps, float *out);
 /* LayerNorm followed by the per-token symmetric int8 quantizer

@@ -21,7 +21,8 @@ def host(t):
     return t.cpu().numpy()
 
 
-@pytest.mark.parametrize("shape", [(1, 4), (5, 768), (64, 768), (33, 3072), (3, 8192), (7, 1024), (9, 2052)])
+@pytest.mark.parametrize("shape", [(1, 4), (5, 768), (64, 768), (33, 3072), (3, 8192), (7, 1024), (9, 2052), (5, 4096),
+                                   (2, 12288), (3, 10000)])
 def test_layer_norm(ctx, oracle, shape):
     rng = np.random.default_rng(shape[1])
     x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
@@ -40,7 +41,8 @@ def test_layer_norm(ctx, oracle, shape):
     np.testing.assert_array_equal(host(q), host(q_ref))
 
 
-@pytest.mark.parametrize("shape", [(1, 4), (5, 768), (64, 768), (4100, 768), (33, 3072), (3, 8192), (9, 2052)])
+@pytest.mark.parametrize("shape", [(1, 4), (5, 768), (64, 768), (4100, 768), (33, 3072), (3, 8192), (9, 2052), (5, 4096),
+                                   (2, 12288)])
 def test_add_layer_norm_quantize(ctx, oracle, shape):
     """The skip connection fused into the LayerNorm + quantize pass: the stream row is the f32 sum (bit exact,
     checked against numpy), and the codes equal those of the unfused kernels on that sum."""
@@ -62,7 +64,7 @@ def test_add_layer_norm_quantize(ctx, oracle, shape):
     assert np.abs(deq - want).max() <= np.abs(want).max() / 127.0 * 0.5 + 1e-4
 
 
-@pytest.mark.parametrize("shape", [(4, 8), (16, 3072), (5, 1024)])
+@pytest.mark.parametrize("shape", [(4, 8), (16, 3072), (5, 1024), (3, 4096), (2, 12288), (7, 6000)])
 def test_gelu(ctx, oracle, shape):
     rng = np.random.default_rng(shape[0])
     x = (rng.standard_normal(shape) * 2).astype(np.float32)
