@@ -231,3 +231,17 @@ def test_row_kernels_with_more_rows_than_resident_workgroups(ctx, oracle):
         qg, sg = ctx.gelu_tanh_quantize(xd)
         np.testing.assert_array_equal(host(sg), host(sg_ref))
         np.testing.assert_array_equal(host(qg), host(qg_ref))
+
+
+def test_row_kernel_shape_errors(ctx, hipq):
+    """Rows must be a multiple of 4 long and fit the register cache; zero rows are a no-op."""
+    for cols in (6, 12292):
+        x = torch.zeros((2, cols), device="cuda")
+        for call in (lambda: ctx.layer_norm(x), lambda: ctx.layer_norm_quantize(x), lambda: ctx.gelu_tanh_quantize(x),
+                     lambda: ctx.add_layer_norm_quantize(x, x.clone())):
+            with pytest.raises(hipq.HipqError) as e:
+                call()
+            assert e.value.code == hipq.SHAPE_ERROR
+    empty = torch.zeros((0, 768), device="cuda")
+    q, s = ctx.layer_norm_quantize(empty)
+    assert q.shape == (0, 768) and s.shape == (0,)
