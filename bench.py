@@ -139,6 +139,28 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
             ctx.histogram(xs[i % 8], -6.0, 6.0, 256, counts=hist)
         for i in range(reps):
             ctx.fake_quantize(xs[i % 8], 0.04, 0, out=ys[i % 8])
+    elif which == "stack":
+        # configs[4]: three forwards of the 12-layer int8 projection stack (8192 tokens, d 768, d_ff 3072)
+        tokens, d, dff, layers = 8192, 768, 3072, 12
+        blocks = []
+        for _ in range(layers):
+            blk = {}
+            for name, (o, i) in {"qkv": (3 * d, d), "out": (d, d), "fc1": (dff, d), "fc2": (d, dff)}.items():
+                wf = torch.randn(o, i, generator=g, device="cuda") * 0.02
+                q, sc, _, _ = ctx.quantize_per_row(wf)
+                blk["w_" + name], blk["s_" + name] = q, sc
+                blk["b_" + name] = torch.randn(o, generator=g, device="cuda") * 0.01
+            for ln in ("ln1", "ln2"):
+                blk[ln + "_gamma"] = torch.ones(d, device="cuda")
+                blk[ln + "_beta"] = torch.zeros(d, device="cuda")
+            blocks.append(blk)
+        x0 = torch.randn(tokens, d, generator=g, device="cuda")
+        x = x0.clone()
+        ws = ctx.stack_workspace(tokens, d, dff)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            x.copy_(x0)
+            ctx.stack_forward(blocks, x, dff, ws)
     else:
         n = 4096 * 4096
         xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
@@ -157,7 +179,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "quantize", "calib", "copy"], default=None,
+    ap.add_argument("--profile", choices=["gemm", "quantize", "calib", "copy", "stack"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
