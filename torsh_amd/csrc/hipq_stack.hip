@@ -3,8 +3,8 @@
 // per-token int8 -> fc1 -> GELU -> per-token int8 -> fc2 + residual), composed
 // from the library's own entry points.  Eight kernels per layer; the fp32
 // intermediates that only feed a quantizer are never written to memory.  The fc2
-// skip connection of every layer but the last is not added in the GEMM's epilogue
-// but by the next layer's first LayerNorm kernel, which reads the row anyway: the
+// skip connection is not added in the GEMM's epilogue but by the next layer's first
+// LayerNorm kernel, which reads the row anyway (after the last layer: by an add): the
 // GEMM then runs in its large-tile form, whose registers have no room for
 // residual values, and the stream is read and written once less.
 #include "hipq_internal.h"
@@ -74,11 +74,14 @@ int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_block_weigh
         if (rc) return rc;
         rc = hipq_gelu_tanh_quantize_f32_i8(ctx, hidden, tokens, d_ff, round_bits, q8, scales);
         if (rc) return rc;
-        if (l + 1 == n_layers)
-            rc = hipq_linear_i8_f32_residual(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, x, tokens, d_model, d_ff, x);
-        else
-            rc = hipq_linear_i8_f32(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, tokens, d_model, d_ff, qkv);
+        rc = hipq_linear_i8_f32(ctx, q8, scales, 1, b.w_fc2, b.s_fc2, b.b_fc2, tokens, d_model, d_ff, qkv);
         if (rc) return rc;
+        if (l + 1 == n_layers) {
+            // no next LayerNorm to carry the skip connection: a plain add (still cheaper than the
+            // small-tile GEMM that has room for residual values)
+            rc = hipq_add_f32(ctx, x, qkv, tokens * d_model, x);
+            if (rc) return rc;
+        }
     }
     return HIPQ_SUCCESS;
 }
