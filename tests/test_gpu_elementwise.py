@@ -317,3 +317,61 @@ def test_dynamic_quantize_back_to_back(ctx, hipq):
         p = ctx.read_qparams(params)
         assert p.status == 0 and p.scale == np.float32(x.abs().max().item()) / np.float32(127.0)
         assert int(q.abs().max().item()) == 127
+
+
+def test_more_than_two_to_the_32_elements(ctx, hipq, oracle):
+    """2^32 + 4099 elements (16 GiB of fp32) through range reduction, quantize, dequantize and the dynamic
+    quantizer.  The input is one seeded block repeated; its length is odd, so an element index that wrapped
+    at 32 bits would land in another phase of the block, and the extremes sit beyond element 2^32, where only
+    64-bit indices reach them.  Expected values: the oracle's on the block, repeated the same way."""
+    period = (1 << 20) + 7
+    n = (1 << 32) + 4099
+    reps = -(-n // period)
+    base = normal(11, (period,))
+    scale, lo_at, hi_at = np.float32(0.03), (1 << 32) + 5, n - 2
+    x = dev(base).repeat(reps)[:n]
+    x[lo_at], x[hi_at] = -11.25, 9.5
+    mm = host(ctx.minmax(x))
+    assert (mm[0], mm[1]) == (-11.25, 9.5)
+    assert host(ctx.absmax(x))[0] == 11.25
+
+    def repeated(block, lo_val, hi_val):
+        t = dev(block).repeat(reps)[:n]
+        t[lo_at], t[hi_at] = lo_val, hi_val
+        return t
+
+    q = ctx.quantize_per_tensor_i8(x, scale, 0, hipq.FORM_MUL_INV)
+    want_q = repeated(oracle.quantize_to_int8_simd(base, scale, 0), -128, 127)
+    torch.cuda.synchronize()
+    assert torch.equal(q, want_q)
+    y = ctx.dequantize(q, scale, 0)
+    want_y_block = oracle.dequantize_per_tensor_affine(oracle.quantize_to_int8_simd(base, scale, 0).astype(np.float32),
+                                                      scale, 0)
+    want_y = repeated(want_y_block, float(np.float32(-128) * scale), float(np.float32(127) * scale))
+    torch.cuda.synchronize()
+    assert torch.equal(y, want_y)
+    del y, want_y, want_q
+    # dynamic: the planted minimum fixes the scale, 11.25 / 127
+    qd, params = ctx.quantize_dynamic_per_tensor(x, hipq.PARAMS_SYMMETRIC, hipq.DTYPE_I8, hipq.FORM_MUL_INV, out=q)
+    p = ctx.read_qparams(params)
+    s_dyn = np.float32(11.25) / np.float32(127.0)
+    assert p.status == 0 and p.scale == s_dyn and (p.min_val, p.max_val) == (-11.25, 9.5)
+    want_qd = repeated(oracle.quantize_to_int8_simd(base, s_dyn, 0), -127,
+                       int(oracle.quantize_to_int8_simd(np.full(65, 9.5, np.float32), s_dyn, 0)[0]))
+    torch.cuda.synchronize()
+    assert torch.equal(qd, want_qd)
+
+
+def test_per_row_quantize_beyond_two_to_the_32_elements(ctx, hipq, oracle):
+    """[2^20 + 3, 4100] rows (4.3 G elements): a block of 1021 rows repeated, expected codes and scales from the
+    oracle on the block; row starts beyond byte 2^34 need 64-bit offsets."""
+    rows, cols, brows = (1 << 20) + 3, 4100, 1021
+    reps = -(-rows // brows)
+    base = normal(12, (brows, cols))
+    want_q, want_s, _ = oracle.quantize_per_channel_auto(base, 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    x = dev(base).repeat(reps, 1)[:rows]
+    q, scales, zps, status = ctx.quantize_per_row(x, hipq.PARAMS_SYMMETRIC)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0 and not bool(zps.any())
+    assert torch.equal(scales, dev(want_s.astype(np.float32)).repeat(reps)[:rows])
+    assert torch.equal(q, dev(want_q.astype(np.int8)).repeat(reps, 1)[:rows])

@@ -297,3 +297,26 @@ def test_every_gemm_kernel_form_gives_the_same_bits(ctx, hipq, oracle, variant):
         ctx.set_gemm_kernel_variant(0)
     with pytest.raises(hipq.HipqError):
         ctx.set_gemm_kernel_variant(99)
+
+
+def test_output_larger_than_four_gib(ctx, hipq, oracle):
+    """[32768, 128] x [32768, 128]^T: the fp32 / int32 output is 4 GiB, so byte offsets into it pass 2^32.  Both
+    operands are a 512-row block repeated 64 times; every 512 x 512 block of the output must equal the oracle's
+    product of the two blocks (and its dequantize epilogue with the per-row and per-channel scales repeated)."""
+    blk, reps, k = 512, 64, 128
+    rng = np.random.default_rng(77)
+    a0, w0 = rand_i8(rng, (blk, k)), rand_i8(rng, (blk, k))
+    sa0 = (rng.random(blk) * 0.05 + 0.01).astype(np.float32)
+    sw0 = (rng.random(blk) * 0.002 + 0.0001).astype(np.float32)
+    b0 = (rng.standard_normal(blk) * 0.01).astype(np.float32)
+    acc0 = oracle.gemm_i8_nk(a0, w0)
+    out0 = oracle.linear_dequant_epilogue(acc0, sa0, sw0, b0)
+    a, w = dev(a0).repeat(reps, 1), dev(w0).repeat(reps, 1)
+    acc = ctx.gemm_i8_i32(a, w)
+    torch.cuda.synchronize()
+    assert acc.numel() * 4 == 1 << 32
+    assert bool((acc.view(reps, blk, reps, blk) == dev(acc0)[None, :, None, :]).all())
+    del acc
+    out = ctx.linear_i8_f32(a, dev(sa0).repeat(reps), w, dev(sw0).repeat(reps), dev(b0).repeat(reps))
+    torch.cuda.synchronize()
+    assert bool((out.view(reps, blk, reps, blk) == dev(out0)[None, :, None, :]).all())
