@@ -293,6 +293,56 @@ def test_full_size_properties(ctx, hipq, oracle):
     assert same["cosine_similarity"] == pytest.approx(1.0, abs=1e-6)
 
 
+def test_more_than_two_to_the_32_elements(ctx, hipq, oracle):
+    """(2^20 + 7) x 4097 elements, one seeded block repeated: counts, sums and images of the repeated tensor
+    follow from the oracle's on the block.  What lies beyond element 2^32 (a NaN, an infinity, the range's ends,
+    the largest error) is only seen with 64-bit indices, and every count must add up to all the elements."""
+    period, reps = (1 << 20) + 7, 4097
+    n = period * reps
+    assert n > 1 << 32
+    base = normal(21, (period,), 1.5)
+    scale, zp = np.float32(0.04), 3
+    x = dev(base).repeat(reps)
+    # observe: range ends and two non-finite values past 2^32
+    x[n - 3], x[(1 << 32) + 9] = 50.0, -60.0
+    bad = x[(1 << 32) + 100:(1 << 32) + 102].clone()
+    x[(1 << 32) + 100], x[(1 << 32) + 101] = float("nan"), float("inf")
+    st = ctx.read_observe(ctx.observe(x))
+    assert (st.min_val, st.max_val, st.nonfinite) == (-60.0, float("inf"), 2)  # NaN ignored, +inf is the maximum
+    x[(1 << 32) + 100:(1 << 32) + 102] = bad
+    st = ctx.read_observe(ctx.observe(x))
+    assert (st.min_val, st.max_val, st.nonfinite) == (-60.0, 50.0, 0)
+    # histogram: block counts x repetitions; the two planted values move from their old bins to the end bins
+    lo, hi, bins = -6.0, 6.0, 256
+    block_counts = oracle.histogram_accumulate(base, lo, hi, bins).astype(np.int64)
+    want = block_counts * reps
+    for pos in ((n - 3) % period, ((1 << 32) + 9) % period):
+        want[oracle.value_to_bin_index(base[pos], lo, hi, bins)] -= 1
+    want[bins - 1] += 1
+    want[0] += 1
+    counts = host(ctx.histogram(x, lo, hi, bins))
+    np.testing.assert_array_equal(counts, want)
+    assert host(ctx.histogram(x, lo, hi, 1))[0] == n  # one counter beyond 2^32
+    # fake quantize: the block's image repeated
+    img_block = oracle.model_fake_quantize(base, scale, zp)
+    img = ctx.fake_quantize(x, scale, zp, -128, 127, hipq.FORM_DIV | hipq.FAKE_INT_CAST)
+    want_img = dev(img_block).repeat(reps)
+    ends = oracle.model_fake_quantize(np.array([50.0, -60.0], np.float32), scale, zp)
+    want_img[n - 3], want_img[(1 << 32) + 9] = float(ends[0]), float(ends[1])
+    torch.cuda.synchronize()
+    assert torch.equal(img, want_img)
+    del want_img
+    # metrics: means over the repeated tensor = the block's, plus the two saturated values' errors
+    e = (np.array([50.0, -60.0], np.float64) - ends.astype(np.float64))
+    blk = oracle.calculate_quantization_metrics_f64(base, img_block)
+    for got in (ctx.read_metrics(ctx.quantization_metrics(x, img)),
+                ctx.read_metrics(ctx.fake_quantize_metrics(x, scale, zp, -128, 127, hipq.FORM_DIV | hipq.FAKE_INT_CAST))):
+        assert got["max_error"] == np.float32(np.abs(e).max())
+        assert got["mse"] == pytest.approx(blk["mse"] + float((e * e).sum()) / n, rel=1e-5)
+        assert got["mae"] == pytest.approx(blk["mae"] + float(np.abs(e).sum()) / n, rel=1e-5)
+        assert got["zero_error_percentage"] == pytest.approx(blk["zero_error_percentage"], rel=1e-5, abs=1e-6)
+
+
 # ---- special schemes (int4, group-wise, binary, ternary) -----------------------------------------
 
 def _view(shape, axis):
