@@ -375,3 +375,35 @@ def test_per_row_quantize_beyond_two_to_the_32_elements(ctx, hipq, oracle):
     assert int(status.item()) == 0 and not bool(zps.any())
     assert torch.equal(scales, dev(want_s.astype(np.float32)).repeat(reps)[:rows])
     assert torch.equal(q, dev(want_q.astype(np.int8)).repeat(reps, 1)[:rows])
+
+
+def test_per_channel_and_requantize_beyond_two_to_the_32_elements(ctx, hipq, oracle):
+    """Explicit-parameter per-channel quantize / dequantize over [4199, 1021, 1003] (channel axis in the middle,
+    4.3 G elements) and requantize over [2^20 + 3, 4100] accumulators: one block repeated along the outer axis,
+    expected bytes from the oracle on the block."""
+    outer, ch, inner = 4199, 1021, 1003
+    assert outer * ch * inner > 1 << 32
+    rng = np.random.default_rng(5)
+    base = normal(31, (1, ch, inner))
+    scales = rng.uniform(0.01, 0.05, ch).astype(np.float32)
+    zps = rng.integers(-5, 6, ch).astype(np.int32)
+    want_q = oracle.quantize_per_channel_affine(base, scales, zps, 1).astype(np.int8)
+    want_y = oracle.dequantize_per_channel_affine(want_q.astype(np.float32), scales, zps, 1)
+    x = dev(base).repeat(outer, 1, 1)
+    q = ctx.quantize_per_channel(x, dev(scales), dev(zps), 1, hipq.FORM_DIV)
+    torch.cuda.synchronize()
+    assert bool((q == dev(want_q)).all())  # broadcast over the outer axis
+    y = ctx.dequantize_per_channel(q, dev(scales), dev(zps), 1)
+    torch.cuda.synchronize()
+    assert bool((y == dev(want_y)).all())
+    del x, q, y
+    rows, cols, brows = (1 << 20) + 3, 4100, 1021
+    reps = -(-rows // brows)
+    acc0 = rng.integers(-3_000_000, 3_000_000, size=(brows, cols), dtype=np.int32)
+    sa0 = rng.uniform(0.01, 0.03, brows).astype(np.float32)
+    sw = rng.uniform(1e-4, 1e-3, cols).astype(np.float32)
+    bias = (rng.standard_normal(cols) * 0.01).astype(np.float32)
+    want = oracle.requantize_epilogue(acc0, sa0, sw, bias, 0.31, -3)
+    got = ctx.requantize(dev(acc0).repeat(reps, 1)[:rows], dev(sa0).repeat(reps)[:rows], dev(sw), dev(bias), 0.31, -3)
+    torch.cuda.synchronize()
+    assert torch.equal(got, dev(want).repeat(reps, 1)[:rows])
