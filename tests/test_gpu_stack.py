@@ -245,3 +245,33 @@ def test_row_kernel_shape_errors(ctx, hipq):
     empty = torch.zeros((0, 768), device="cuda")
     q, s = ctx.layer_norm_quantize(empty)
     assert q.shape == (0, 768) and s.shape == (0,)
+
+
+def test_row_kernels_beyond_two_to_the_32_elements(ctx, hipq):
+    """[2^20 + 3, 4100] fp32 (4.3 G elements) through the row kernels: a block of 1021 rows repeated, and since
+    each row is processed on its own, the result must be the block's result repeated bit for bit; rows that start
+    beyond byte 2^34 need 64-bit offsets."""
+    rows, cols, brows = (1 << 20) + 3, 4100, 1021
+    reps = -(-rows // brows)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    base = torch.randn((brows, cols), generator=g, device="cuda")
+    delta = torch.randn((brows, cols), generator=g, device="cuda")
+    gamma = torch.rand(cols, generator=g, device="cuda") + 0.5
+    beta = torch.randn(cols, generator=g, device="cuda") * 0.1
+
+    def rep(t):
+        return t.repeat(reps, *([1] * (t.dim() - 1)))[:rows]
+
+    x = rep(base)
+    for got, want in ((ctx.layer_norm_quantize(x, gamma, beta), ctx.layer_norm_quantize(base, gamma, beta)),
+                      (ctx.gelu_tanh_quantize(x), ctx.gelu_tanh_quantize(base))):
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], rep(want[0])) and torch.equal(got[1], rep(want[1]))
+    assert torch.equal(ctx.layer_norm(x, gamma, beta), rep(ctx.layer_norm(base, gamma, beta)))
+    assert torch.equal(ctx.gelu_tanh(x), rep(ctx.gelu_tanh(base)))
+    b2 = base.clone()
+    want = ctx.add_layer_norm_quantize(b2, delta, gamma, beta)
+    got = ctx.add_layer_norm_quantize(x, rep(delta), gamma, beta)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0], rep(want[0])) and torch.equal(got[1], rep(want[1]))
+    assert torch.equal(x, rep(b2))  # the sum written back
