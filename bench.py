@@ -359,6 +359,7 @@ def main() -> int:
         # calibration / quality kernels on the same 16 Mi-element tensors
         metrics_rec = ctx.quantization_metrics(fx[0], fy[0])
         observe_rec = ctx.observe(fx[0])
+        stats_rec = ctx._record(hipq.TensorStats)
         hist = torch.zeros(256, dtype=torch.int64, device="cuda")
 
         def run_metrics():
@@ -381,6 +382,14 @@ def main() -> int:
             i = rot()
             ctx.histogram(fx[i], -6.0, 6.0, 256, counts=hist)
 
+        def run_stats_one_pass():
+            i = rot()
+            ctx.tensor_stats(fx[i], one_pass=True, out=stats_rec)
+
+        def run_stats_two_pass():
+            i = rot()
+            ctx.tensor_stats(fx[i], out=stats_rec)
+
         def run_copy():
             # not a kernel of this library: torch's device-to-device copy of the same tensors, as the
             # bandwidth this box sustains on a plain stream (the yardstick beside the 8 TB/s datasheet figure)
@@ -394,7 +403,9 @@ def main() -> int:
                                     ("fake_quantize_metrics_fused_f32", run_fused_metrics, 4),
                                     ("fake_quantize_f32", run_fake_quant, 8),
                                     ("observe_minmax_nonfinite_f32", run_observe, 4),
-                                    ("histogram_256_bins_f32", run_histogram, 4)):
+                                    ("histogram_256_bins_f32", run_histogram, 4),
+                                    ("tensor_stats_raw_moments_f32", run_stats_one_pass, 4),
+                                    ("tensor_stats_two_pass_f32", run_stats_two_pass, 8)):
             ms = event_time_ms(fn, reps=50, warmup=5)
             gbps = bytes_per * n / (ms * 1e-3) / 1e9
             extra[name] = {"us": ms * 1e3, "GB/s": gbps, "frac_hbm_peak": gbps / PEAK_HBM_GBPS,

@@ -56,7 +56,10 @@ enum {
     HIPQ_ROUND_HALF_AWAY = 0,
     HIPQ_ROUND_HALF_EVEN = 1,
     HIPQ_FORM_MUL_INV = 0,
-    HIPQ_FORM_DIV = 2
+    HIPQ_FORM_DIV = 2,
+    /* floor(v + 0.5): the reduced-precision rounding of quantize_mobile_optimized
+     * (simd_ops.rs:424-431); accepted by hipq_quantize_per_tensor_f32_i8 only. */
+    HIPQ_ROUND_FLOOR_HALF_UP = 16
 };
 
 /* Quantized integer types, ranges per get_dtype_range
@@ -133,7 +136,9 @@ HIPQ_API int32_t hipq_qparams_from_minmax(hipq_ctx *ctx, const float *minmax, in
 /* quantize_to_int8_simd / quantize_per_tensor_affine_i8,
  * crates/torsh-quantization/src/simd_ops.rs:196-227, algorithms.rs:245-274:
  * q = clamp(round(x * (1/scale) | x / scale) + zp, -128, 127) as i8.
- * scale <= 0 is InvalidArgument (algorithms.rs:284-288). */
+ * scale <= 0 is InvalidArgument (algorithms.rs:284-288).  Also the arithmetic of
+ * quantize_mobile_optimized (simd_ops.rs:390-446; HIPQ_ROUND_FLOOR_HALF_UP is its
+ * reduced-precision rounding for more than 256 elements). */
 HIPQ_API int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n, float scale,
                                                  int32_t zero_point, int32_t mode, int8_t *out);
 /* hipq_quantize_per_tensor_f32_i8 that also records the parameters it was given in a device-side
@@ -420,6 +425,22 @@ HIPQ_API int32_t hipq_fake_quantize_metrics_f32(hipq_ctx *ctx, const float *x, s
 HIPQ_API int32_t hipq_fake_quantize_f32(hipq_ctx *ctx, const float *x, size_t n, float scale, int32_t zero_point,
                                         const hipq_qparams *params, int32_t qmin, int32_t qmax, int32_t mode,
                                         float *out);
+
+/* TensorStats, crates/torsh-quantization/src/simd_ops.rs:264-272 (same fields, same order). */
+typedef struct hipq_tensor_stats {
+    float min_val;
+    float max_val;
+    float mean;
+    float std_dev;
+    float variance;
+} hipq_tensor_stats;
+/* calculate_tensor_stats_simd, simd_ops.rs:230-262 (one_pass == 0: range, f64 mean, then the f64
+ * sum of squared deviations from it in a second pass over x; population variance), or
+ * calculate_tensor_stats_cache_optimized, algorithms.rs:525-578 (one_pass != 0: f64 sums of x and
+ * x^2, mean rounded to f32, variance = E[x^2] - mean^2 rounded to f32, std_dev = its f32 square
+ * root).  out_stats is a device record.  n == 0 is InvalidArgument as in both. */
+HIPQ_API int32_t hipq_tensor_stats_f32(hipq_ctx *ctx, const float *x, size_t n, int32_t one_pass,
+                                       hipq_tensor_stats *out_stats);
 
 /* What Observer::update derives from one batch before it touches its state
  * (crates/torsh-quantization/src/observers.rs:122-150): the batch range (NaN

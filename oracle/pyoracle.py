@@ -173,6 +173,40 @@ def quantize_to_int8_simd(x, scale, zp):
     return out
 
 
+def quantize_cache_aware(x, scale, zp):
+    """Element formula shared by the cache-aware, tiled, streaming and NEON quantizers (f32 carrier)."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    _check(lib().tq_quantize_cache_aware(_p(x, _f32p), C.c_size_t(x.size), C.c_float(scale), int(zp), _p(out, _f32p)),
+           "quantize_cache_aware")
+    return out
+
+
+def quantize_mobile_optimized(x, scale, zp, reduced_precision=False):
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.int8)
+    _check(lib().tq_quantize_mobile_optimized(_p(x, _f32p), C.c_size_t(x.size), C.c_float(scale), int(zp),
+                                              int(bool(reduced_precision)), _p(out, _i8p)), "quantize_mobile_optimized")
+    return out
+
+
+def calculate_tensor_stats_simd(x) -> dict:
+    x = _f32(x)
+    out = np.empty(5, dtype=np.float32)
+    _check(lib().tq_calculate_tensor_stats_simd(_p(x, _f32p), C.c_size_t(x.size), _p(out, _f32p)),
+           "calculate_tensor_stats_simd")
+    return dict(zip(("min", "max", "mean", "std_dev", "variance"), out))
+
+
+def calculate_tensor_stats_cache_optimized(x):
+    """(min, max, mean, std_dev)"""
+    x = _f32(x)
+    out = np.empty(4, dtype=np.float32)
+    _check(lib().tq_calculate_tensor_stats_cache_optimized(_p(x, _f32p), C.c_size_t(x.size), _p(out, _f32p)),
+           "calculate_tensor_stats_cache_optimized")
+    return tuple(out)
+
+
 def quantize_per_tensor_affine(x, scale, zp):
     x = _f32(x)
     out = np.empty_like(x)

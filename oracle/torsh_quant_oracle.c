@@ -692,3 +692,78 @@ double tq_time_matmul_rows(const uint8_t *a, const uint8_t *b_kn, size_t m_sampl
     tq_backend_matmul_i32(a, b_kn, m_sample, k, n, acc, NULL);
     return now_s() - t0;
 }
+
+/* crates/torsh-quantization/src/algorithms.rs:473-522 (quantize_per_tensor_affine_cache_aware), 581-635
+ * (quantize_matrix_cache_friendly), 638-674 (quantize_streaming_with_prefetch) and simd_ops.rs:302-350
+ * (quantize_neon_optimized): chunking, tiling and prefetch hints differ, the element formula does not. */
+int tq_quantize_cache_aware(const float *x, size_t n, float scale, int32_t zp, float *out) {
+    if (scale <= 0.0f) return TQ_ERR_INVALID_ARGUMENT;
+    const float inv = 1.0f / scale;
+    const float zpf = (float)zp;
+    for (size_t i = 0; i < n; ++i) out[i] = clampf_rust(roundf(x[i] * inv) + zpf, -128.0f, 127.0f);
+    return TQ_OK;
+}
+
+/* crates/torsh-quantization/src/simd_ops.rs:390-446 */
+int tq_quantize_mobile_optimized(const float *x, size_t n, float scale, int32_t zp, int reduced_precision,
+                                 int8_t *out) {
+    if (scale <= 0.0f) return TQ_ERR_INVALID_ARGUMENT;
+    const float inv = 1.0f / scale; /* both branches of :409-414 */
+    const float zpf = (float)zp;
+    const int chunked = n > 256; /* :421 */
+    for (size_t i = 0; i < n; ++i) {
+        float q;
+        if (chunked && reduced_precision)
+            q = floorf(x[i] * inv + 0.5f) + zpf; /* :426-428 */
+        else
+            q = roundf(x[i] * inv) + zpf;
+        out[i] = f32_as_i8(clampf_rust(q, -128.0f, 127.0f));
+    }
+    return TQ_OK;
+}
+
+/* crates/torsh-quantization/src/simd_ops.rs:230-262; the sums run in element order here, in
+ * rayon's tree order there (f64 terms, so the two agree to ~1e-16 relative). */
+int tq_calculate_tensor_stats_simd(const float *x, size_t n, float out[5]) {
+    if (n == 0) return TQ_ERR_INVALID_ARGUMENT;
+    float mn, mx;
+    int rc = tq_find_min_max(x, n, &mn, &mx);
+    if (rc != TQ_OK) return rc;
+    double sum = 0.0;
+    for (size_t i = 0; i < n; ++i) sum += (double)x[i];
+    const double mean = sum / (double)n;
+    double vs = 0.0;
+    for (size_t i = 0; i < n; ++i) {
+        const double d = (double)x[i] - mean;
+        vs += d * d;
+    }
+    const double variance = vs / (double)n;
+    out[0] = mn;
+    out[1] = mx;
+    out[2] = (float)mean;
+    out[3] = (float)sqrt(variance);
+    out[4] = (float)variance;
+    return TQ_OK;
+}
+
+/* crates/torsh-quantization/src/algorithms.rs:525-578 */
+int tq_calculate_tensor_stats_cache_optimized(const float *x, size_t n, float out[4]) {
+    if (n == 0) return TQ_ERR_INVALID_ARGUMENT;
+    float mn = INFINITY, mx = -INFINITY;
+    double sum = 0.0, sumsq = 0.0;
+    for (size_t i = 0; i < n; ++i) {
+        mn = fminf(mn, x[i]);
+        mx = fmaxf(mx, x[i]);
+        const double v = (double)x[i];
+        sum += v;
+        sumsq += v * v;
+    }
+    const double nd = (double)n;
+    const float mean = (float)(sum / nd);
+    const float variance = (float)(sumsq / nd - (double)mean * (double)mean); /* :573 */
+    out[0] = mn;
+    out[1] = mx;
+    out[2] = mean;
+    out[3] = sqrtf(variance);
+    return TQ_OK;
+}

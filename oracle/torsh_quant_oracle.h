@@ -60,6 +60,18 @@ int tq_quantize_per_channel_auto(const float *x, const size_t *shape, size_t ndi
                                  int scheme, float *out, float *scales, int32_t *zps);
 int tq_quantize_per_channel_simd(const float *x, size_t n, const float *scales, const int32_t *zps,
                                  size_t num_channels, size_t channel_size, float *out);
+/* The cache-aware, tiled, streaming and NEON twins of the per-tensor quantizer share one element
+ * formula, clamp(round(x * (1/scale)) + zp, -128, 127) into an f32 carrier:
+ * crates/torsh-quantization/src/algorithms.rs:473-522, 581-635, 638-674; simd_ops.rs:302-350. */
+int tq_quantize_cache_aware(const float *x, size_t n, float scale, int32_t zp, float *out);
+/* quantize_mobile_optimized, simd_ops.rs:390-446: int8 output; with reduced precision and more
+ * than 256 elements the rounding is floor(x * inv + 0.5) instead of round. */
+int tq_quantize_mobile_optimized(const float *x, size_t n, float scale, int32_t zp, int reduced_precision,
+                                 int8_t *out);
+/* calculate_tensor_stats_simd, simd_ops.rs:230-262: out = {min, max, mean, std_dev, variance}. */
+int tq_calculate_tensor_stats_simd(const float *x, size_t n, float out[5]);
+/* calculate_tensor_stats_cache_optimized, algorithms.rs:525-578: out = {min, max, mean, std_dev}. */
+int tq_calculate_tensor_stats_cache_optimized(const float *x, size_t n, float out[4]);
 int tq_quantize_per_channel_affine(const float *x, const size_t *shape, size_t ndim, size_t axis,
                                    const float *scales, const int32_t *zps, size_t nparams, float *out);
 int tq_dequantize_per_channel_affine(const float *q, const size_t *shape, size_t ndim, size_t axis,

@@ -92,6 +92,16 @@ void check_same(const std::vector<A> &a, const std::vector<B> &b, int line) {
         }
 }
 #define CHECK_SAME(a, b) check_same(a, b, __LINE__)
+// As check_same for f32 carriers that may hold NaN: a NaN must face a NaN.
+void check_same_bits(const std::vector<float> &a, const std::vector<float> &b, int line) {
+    if (a.size() != b.size()) throw Failure{std::to_string(line) + ": size mismatch"};
+    for (size_t i = 0; i < a.size(); ++i)
+        if (!(a[i] == b[i] || (std::isnan(a[i]) && std::isnan(b[i])))) {
+            std::ostringstream o;
+            o << line << ": element " << i << ": " << a[i] << " vs " << b[i];
+            throw Failure{o.str()};
+        }
+}
 
 // ---------------------------------------------------------------- host logic (no device)
 
@@ -976,6 +986,130 @@ GPU_TEST(parity_quantize_batch_consistent) {  // utils.rs:153-180
         check_same(std::get<0>(res[i]).as_slice(), want, __LINE__);
     }
     CHECK(quantize_batch_consistent({}, QuantConfig::int8()).unwrap().empty());
+}
+
+CPU_TEST(test_slice_variant_errors_before_the_device) {  // algorithms.rs:997-1020, 984-994; simd_ops.rs:620-628
+    const CacheAwareParams cp;
+    CHECK_EQ(cp.cache_line_size, size_t(64));
+    CHECK_EQ(cp.l1_cache_size, size_t(32 * 1024));
+    CHECK_EQ(cp.l2_cache_size, size_t(256 * 1024));
+    CHECK_EQ(cp.l3_cache_size, size_t(8 * 1024 * 1024));
+    CHECK_EQ(cp.prefetch_distance, size_t(16));
+    CHECK(cp.enable_chunking);
+    std::vector<float> in{1.0f, 2.0f}, out(3);
+    auto r = quantize_per_tensor_affine_cache_aware(in, 0.1f, 0, out, cp);
+    CHECK(r.is_err());
+    CHECK_EQ(r.unwrap_err().message, std::string("Input and output length mismatch"));
+    out.resize(2);
+    r = quantize_per_tensor_affine_cache_aware(in, -0.1f, 0, out, cp);
+    CHECK(r.is_err());
+    CHECK_EQ(r.unwrap_err().message, std::string("Scale must be positive"));
+    CHECK(quantize_streaming_with_prefetch(in, 0.0f, 0, out, cp).is_err());
+    CHECK(quantize_with_cache_optimization(in, -1.0f, 0, out).is_err());
+    auto m = quantize_matrix_cache_friendly(in, 2, 2, 0.1f, 0, out, cp);
+    CHECK(m.is_err());
+    CHECK_EQ(m.unwrap_err().message, std::string("Matrix dimensions don't match buffer sizes"));
+    auto st = calculate_tensor_stats_cache_optimized({}, cp);
+    CHECK(st.is_err());
+    CHECK_EQ(st.unwrap_err().message, std::string("Cannot calculate stats of empty tensor"));
+    CHECK(calculate_tensor_stats_simd({}).is_err());
+    std::vector<int8_t> q8(1);
+    CHECK(quantize_mobile_optimized(in, 0.1f, 0, q8, false).is_err());
+    q8.resize(2);
+    CHECK(quantize_mobile_optimized(in, 0.0f, 0, q8, true).is_err());
+    std::vector<std::vector<float> *> outs;
+    auto b = quantize_batch_consistent_simd({&in}, 0.1f, 0, outs);
+    CHECK(b.is_err());
+    CHECK_EQ(b.unwrap_err().message, std::string("Number of input tensors must match output tensors"));
+    const auto small = get_cache_optimization_recommendations(1000, 4, cp);
+    CHECK(!small.empty() && small[0].find("L1 cache") != std::string::npos);
+    bool streaming = false;
+    for (const auto &line : get_cache_optimization_recommendations(10000000, 4, cp))
+        streaming = streaming || line.find("streaming") != std::string::npos;
+    CHECK(streaming);
+    const MobileOptimizationHints hints = get_mobile_optimization_hints();
+    CHECK(hints.prefer_int8 && hints.optimal_chunk_size > 0 && !hints.prefer_sequential);
+    CHECK(get_simd_width() >= 1 && (!is_simd_available() || get_simd_width() > 1));
+}
+
+GPU_TEST(test_slice_variants) {  // algorithms.rs:897-982, simd_ops.rs:513-522, 569-618
+    const CacheAwareParams cp;
+    std::vector<float> in8{1, 2, 3, 4, 5, 6, 7, 8}, out8(8);
+    CHECK(quantize_per_tensor_affine_cache_aware(in8, 0.1f, 0, out8, cp).is_ok());
+    CHECK_EQ(out8[0], 10.0f);
+    CHECK_EQ(out8[7], 80.0f);
+    std::fill(out8.begin(), out8.end(), 0.0f);
+    CHECK(quantize_neon_optimized(in8, 0.1f, 0, out8).is_ok());
+    CHECK(out8[0] == 10.0f && out8[1] == 20.0f && out8[7] == 80.0f);
+    std::vector<float> m9{1, 2, 3, 4, 5, 6, 7, 8, 9}, o9(9);
+    CHECK(quantize_matrix_cache_friendly(m9, 3, 3, 0.1f, 0, o9, cp).is_ok());
+    CHECK(o9[0] == 10.0f && o9[8] == 90.0f);
+    std::vector<float> s5{0.1f, 0.2f, 0.3f, 0.4f, 0.5f}, o5(5);
+    CHECK(quantize_streaming_with_prefetch(s5, 0.01f, 10, o5, cp).is_ok());
+    CHECK_EQ(o5[0], 20.0f);
+    std::vector<float> in4{1, 2, 3, 4}, o4(4);
+    CHECK(quantize_with_cache_optimization(in4, 0.1f, 0, o4).is_ok());
+    CHECK(o4[0] == 10.0f && o4[3] == 40.0f);
+    const auto st10 = calculate_tensor_stats_cache_optimized({1, 2, 3, 4, 5, 6, 7, 8, 9, 10}, cp).unwrap();
+    CHECK(std::get<0>(st10) == 1.0f && std::get<1>(st10) == 10.0f);
+    CHECK(std::fabs(std::get<2>(st10) - 5.5f) < 0.001f && std::get<3>(st10) > 0.0f);
+    const TensorStats st5 = calculate_tensor_stats_simd({1, 2, 3, 4, 5}).unwrap();
+    CHECK(st5.min == 1.0f && st5.max == 5.0f && st5.mean == 3.0f);
+    CHECK(std::fabs(st5.std_dev - static_cast<float>(std::sqrt(2.0))) < 1e-4f);
+    std::vector<float> mob{1, 2, 3, 4, -1, -2};
+    std::vector<int8_t> q6(6);
+    CHECK(quantize_mobile_optimized(mob, 0.1f, 0, q6, false).is_ok());
+    CHECK_SAME(q6, (std::vector<int>{10, 20, 30, 40, -10, -20}));
+    std::vector<int8_t> q4(4);
+    CHECK(quantize_mobile_optimized(in4, 0.1f, 0, q4, true).is_ok());
+    CHECK(std::abs(q4[0] - 10) <= 1 && std::abs(q4[1] - 20) <= 1);
+    const auto mm = find_min_max_neon({-1.5f, 0.0f, 2.3f, -0.8f, 4.7f, 1.2f, 9.5f, -2.1f}).unwrap();
+    CHECK(mm.first == -2.1f && mm.second == 9.5f);
+}
+
+GPU_TEST(parity_slice_variants) {
+    const CacheAwareParams cp;
+    for (size_t n : {size_t(7), size_t(256), size_t(257), size_t(100003)}) {
+        std::vector<float> x = normal(n, 300 + static_cast<uint32_t>(n), 2.5f);
+        if (n > 300) {
+            x[5] = 1.25f, x[6] = -1.25f, x[7] = 0.24999999f;  // ties and the 0.49999997 edge at scale 0.5
+            x[8] = 1e9f, x[9] = -1e9f, x[10] = NAN;
+        }
+        std::vector<float> want(n), got(n);
+        CHECK_EQ(tq_quantize_cache_aware(x.data(), n, 0.5f, -7, want.data()), 0);
+        CHECK(quantize_per_tensor_affine_cache_aware(x, 0.5f, -7, got, cp).is_ok());
+        check_same_bits(got, want, __LINE__);
+        CHECK(quantize_streaming_with_prefetch(x, 0.5f, -7, got, cp).is_ok());
+        check_same_bits(got, want, __LINE__);
+        CHECK(quantize_with_cache_optimization(x, 0.5f, -7, got, &cp).is_ok());
+        check_same_bits(got, want, __LINE__);
+        for (bool reduced : {false, true}) {
+            std::vector<int8_t> q(n), wq(n);
+            CHECK_EQ(tq_quantize_mobile_optimized(x.data(), n, 0.5f, 3, reduced ? 1 : 0, wq.data()), 0);
+            CHECK(quantize_mobile_optimized(x, 0.5f, 3, q, reduced).is_ok());
+            CHECK_SAME(q, wq);
+        }
+        if (n > 300) x[8] = 3.0f, x[9] = -3.0f, x[10] = 0.0f;  // finite data for the statistics
+        for (float &v : x) v += 4.0f;
+        float w5[5], w4[4];
+        CHECK_EQ(tq_calculate_tensor_stats_simd(x.data(), n, w5), 0);
+        CHECK_EQ(tq_calculate_tensor_stats_cache_optimized(x.data(), n, w4), 0);
+        const TensorStats st = calculate_tensor_stats_simd(x).unwrap();
+        CHECK(st.min == w5[0] && st.max == w5[1]);
+        CHECK(std::fabs(st.mean - w5[2]) <= 1e-6f * std::fabs(w5[2]));
+        CHECK(std::fabs(st.std_dev - w5[3]) <= 1e-6f * w5[3] && std::fabs(st.variance - w5[4]) <= 1e-6f * w5[4]);
+        const auto co = calculate_tensor_stats_cache_optimized(x, cp).unwrap();
+        CHECK(std::get<0>(co) == w4[0] && std::get<1>(co) == w4[1]);
+        CHECK(std::fabs(std::get<2>(co) - w4[2]) <= 1e-6f * std::fabs(w4[2]));
+        CHECK(std::fabs(std::get<3>(co) - w4[3]) <= 2e-5f * w4[3]);  // raw moments cancel: E[x^2] - mean^2
+    }
+    std::vector<float> a = normal(1000, 311, 1.0f), b = normal(70, 312, 3.0f), oa(1000), ob(70), wa(1000), wb(70);
+    std::vector<std::vector<float> *> outs{&oa, &ob};
+    CHECK(quantize_batch_consistent_simd({&a, &b}, 0.02f, 4, outs).is_ok());
+    CHECK_EQ(tq_quantize_per_tensor_affine_simd(a.data(), a.size(), 0.02f, 4, wa.data()), 0);
+    CHECK_EQ(tq_quantize_per_tensor_affine_simd(b.data(), b.size(), 0.02f, 4, wb.data()), 0);
+    check_same_bits(oa, wa, __LINE__);
+    check_same_bits(ob, wb, __LINE__);
 }
 
 GPU_TEST(parity_model_quantizer) {  // crates/torsh-models/src/quantization.rs:260-332, 491-566

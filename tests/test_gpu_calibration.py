@@ -343,6 +343,52 @@ def test_more_than_two_to_the_32_elements(ctx, hipq, oracle):
         assert got["zero_error_percentage"] == pytest.approx(blk["zero_error_percentage"], rel=1e-5, abs=1e-6)
 
 
+@pytest.mark.parametrize("n", [1, 5, 63, 4096, 4099, (1 << 20) + 3, 1 << 24])
+def test_tensor_stats_both_forms(ctx, oracle, n):
+    """calculate_tensor_stats_simd (two passes, centered) and calculate_tensor_stats_cache_optimized (raw moments):
+    range exact; mean, variance and standard deviation to 1e-6 of the oracle's f64 sums (the order of f64
+    additions differs), the raw-moment variance to the cancellation it carries."""
+    x = normal(500 + (n % 1000), n, 2.0) + np.float32(3.0)
+    d = dev(x)
+    st = ctx.tensor_stats(d)
+    want = oracle.calculate_tensor_stats_simd(x)
+    assert (st.min_val, st.max_val) == (want["min"], want["max"])
+    assert st.mean == pytest.approx(want["mean"], rel=1e-6)
+    assert st.variance == pytest.approx(want["variance"], rel=1e-6, abs=1e-12)
+    assert st.std_dev == pytest.approx(want["std_dev"], rel=1e-6, abs=1e-12)
+    one = ctx.tensor_stats(d, one_pass=True)
+    mn, mx, mean, std = oracle.calculate_tensor_stats_cache_optimized(x)
+    assert (one.min_val, one.max_val) == (mn, mx)
+    assert one.mean == pytest.approx(mean, rel=1e-6)
+    if n > 1:
+        assert one.std_dev == pytest.approx(std, rel=2e-5)
+        assert one.variance == pytest.approx(np.float32(std) ** 2, rel=4e-5)
+
+
+def test_tensor_stats_known_answers_and_edges(ctx, hipq, golden):
+    sv = golden["slice_variants"]
+    c = sv["stats_simd"]
+    st = ctx.tensor_stats(dev(np.array(c["x"], np.float32)))
+    assert (st.min_val, st.max_val, st.mean) == (c["min"], c["max"], c["mean"])
+    assert abs(st.std_dev - np.float32(np.sqrt(c["std_dev_f64_sqrt_of"]))) <= c["std_eps"]
+    assert st.variance == 2.0
+    c = sv["stats_cache_optimized"]
+    st = ctx.tensor_stats(dev(np.array(c["x"], np.float32)), one_pass=True)
+    assert (st.min_val, st.max_val) == (c["min"], c["max"]) and abs(st.mean - c["mean"]) < c["mean_eps"]
+    assert st.std_dev == pytest.approx(np.sqrt(8.25), rel=1e-6)
+    with pytest.raises(hipq.HipqError, match="Cannot calculate stats of empty tensor"):
+        ctx.tensor_stats(torch.empty(0, device="cuda"))
+    # NaN is ignored by the range (f32::min / max) and poisons the sums, as in the reference
+    x = torch.tensor([1.0, float("nan"), 3.0], device="cuda")
+    st = ctx.tensor_stats(x)
+    assert (st.min_val, st.max_val) == (1.0, 3.0) and math.isnan(st.mean) and math.isnan(st.std_dev)
+    # an unaligned view
+    base = torch.arange(0, 1001, device="cuda", dtype=torch.float32)
+    st = ctx.tensor_stats(base[1:])
+    assert (st.min_val, st.max_val, st.mean) == (1.0, 1000.0, 500.5)
+    assert st.variance == pytest.approx((1000 ** 2 - 1) / 12.0, rel=1e-6)
+
+
 # ---- special schemes (int4, group-wise, binary, ternary) -----------------------------------------
 
 def _view(shape, axis):

@@ -407,3 +407,32 @@ def test_per_channel_and_requantize_beyond_two_to_the_32_elements(ctx, hipq, ora
     got = ctx.requantize(dev(acc0).repeat(reps, 1)[:rows], dev(sa0).repeat(reps)[:rows], dev(sw), dev(bias), 0.31, -3)
     torch.cuda.synchronize()
     assert torch.equal(got, dev(want).repeat(reps, 1)[:rows])
+
+
+@pytest.mark.parametrize("n", [6, 256, 257, 4099, (1 << 20) + 3])
+def test_mobile_quantizer_and_its_reduced_precision_rounding(ctx, hipq, oracle, n):
+    """quantize_mobile_optimized: round(x * inv) up to 256 elements or without reduced precision, floor(x * inv + 0.5)
+    beyond; ties, the 0.49999997 edge, saturation and NaN included."""
+    x = normal(40 + n, (n,), 3.0)
+    x[:6] = [1.25, -1.25, 0.24999999, -0.25, 1e9, np.nan]
+    for reduced in (False, True):
+        mode = hipq.FORM_MUL_INV | (hipq.ROUND_FLOOR_HALF_UP if (reduced and n > 256) else 0)
+        got = host(ctx.quantize_per_tensor_i8(dev(x), 0.5, 3, mode))
+        np.testing.assert_array_equal(got, oracle.quantize_mobile_optimized(x, 0.5, 3, reduced))
+    # the other entry points do not know the mode, and two roundings at once are refused
+    with pytest.raises(hipq.HipqError):
+        ctx.quantize_per_tensor_u8(dev(x), 0.5, 3, hipq.ROUND_FLOOR_HALF_UP)
+    with pytest.raises(hipq.HipqError):
+        ctx.quantize_per_tensor_i8(dev(x), 0.5, 3, hipq.ROUND_FLOOR_HALF_UP | hipq.ROUND_HALF_EVEN)
+
+
+def test_cache_aware_twins_share_the_carrier_kernel(ctx, hipq, oracle, golden):
+    for case in golden["slice_variants"]["carrier"]:
+        x = np.array(case["x"], np.float32)
+        got = host(ctx.quantize_per_tensor_carrier(dev(x), case["scale"], case["zp"], hipq.FORM_MUL_INV))
+        for idx, val in case["checks"]:
+            assert got[idx] == np.float32(val), case["fn"]
+    x = normal(77, (100_003,), 4.0)
+    x[:3] = [np.nan, 1e9, -1e9]
+    got = host(ctx.quantize_per_tensor_carrier(dev(x), 0.05, -3, hipq.FORM_MUL_INV))
+    np.testing.assert_array_equal(got, oracle.quantize_cache_aware(x, 0.05, -3))

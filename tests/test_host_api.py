@@ -25,6 +25,7 @@ CPU_CASES = [
     "test_weight_file_round_trip_and_corruption",
     "test_model_quantizer_scalar_logic",
     "test_kernel_plugin_interface",
+    "test_slice_variant_errors_before_the_device",
     "test_fake_quantize_errors_before_the_device",
 ]
 GPU_CASES = [
@@ -48,6 +49,8 @@ GPU_CASES = [
     "test_observers",
     "parity_observers_against_the_oracle",
     "parity_quantize_batch_consistent",
+    "test_slice_variants",
+    "parity_slice_variants",
     "parity_model_quantizer",
     "test_quantized_modules_survive_a_weight_file",
     "test_special_schemes",

@@ -223,6 +223,110 @@ __global__ __launch_bounds__(kCalBlock) void fake_quantize_kernel(const float *_
     }
 }
 
+// ---- tensor statistics ---------------------------------------------------------------------
+
+struct StatsPartial {
+    float mn, mx;
+    double s1, s2;  // sum of x and of x^2, or (CENTERED) unused and the sum of (x - mean)^2
+};
+
+__device__ __forceinline__ void stats_block_store(float mn, float mx, double s1, double s2,
+                                                  StatsPartial *__restrict__ out) {
+    __shared__ StatsPartial lds[kCalBlock / kWave];
+    StatsPartial w{wave_min(mn), wave_max(mx), wave_sum(s1), wave_sum(s2)};
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) lds[wave] = w;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        StatsPartial r = lds[0];
+        for (int i = 1; i < kCalBlock / kWave; ++i) {
+            r.mn = fminf(r.mn, lds[i].mn);
+            r.mx = fmaxf(r.mx, lds[i].mx);
+            r.s1 += lds[i].s1;
+            r.s2 += lds[i].s2;
+        }
+        *out = r;
+    }
+}
+
+// One pass of calculate_tensor_stats_simd (crates/torsh-quantization/src/simd_ops.rs:230-262) or of
+// calculate_tensor_stats_cache_optimized (algorithms.rs:525-578): every element enters the sums as
+// an f64, as there.  CENTERED = the second pass of the former, sum of (x - mean)^2 with the mean
+// the first pass left in `totals`.
+template <bool CENTERED>
+__global__ __launch_bounds__(kCalBlock) void stats_partial_kernel(const float *__restrict__ x, size_t n,
+                                                                   const StatsPartial *__restrict__ totals,
+                                                                   StatsPartial *__restrict__ partials) {
+    float mn = INFINITY, mx = -INFINITY;
+    double s1 = 0.0, s2 = 0.0;
+    double mean = 0.0;
+    if constexpr (CENTERED) mean = totals->s1 / static_cast<double>(n);
+    auto one = [&](float v) {
+        const double d = static_cast<double>(v);
+        if constexpr (CENTERED) {
+            const double c = d - mean;
+            s2 = fma(c, c, s2);
+        } else {
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
+            s1 += d;
+            s2 = fma(d, d, s2);  // d * d is exact in f64
+        }
+    };
+    stream1<kCalBlock>(
+        x, n,
+        [&](const float4 &v, size_t) {
+            one(v.x);
+            one(v.y);
+            one(v.z);
+            one(v.w);
+        },
+        [&](float v, size_t) { one(v); });
+    stats_block_store(mn, mx, s1, s2, partials + blockIdx.x);
+}
+
+// STAGE 0: fold the first pass into `totals` (and, ONE_PASS, finish with the raw-moment formulas of
+// algorithms.rs:571-575).  STAGE 1: fold the centered sums and finish as simd_ops.rs:240-261.
+template <int STAGE, bool ONE_PASS>
+__global__ __launch_bounds__(kCalBlock) void stats_final_kernel(const StatsPartial *__restrict__ partials, int nparts,
+                                                                 size_t n, StatsPartial *__restrict__ totals,
+                                                                 hipq_tensor_stats *__restrict__ out) {
+    float mn = INFINITY, mx = -INFINITY;
+    double s1 = 0.0, s2 = 0.0;
+    for (int i = threadIdx.x; i < nparts; i += kCalBlock) {
+        const StatsPartial p = partials[i];
+        mn = fminf(mn, p.mn);
+        mx = fmaxf(mx, p.mx);
+        s1 += p.s1;
+        s2 += p.s2;
+    }
+    __shared__ StatsPartial folded;
+    stats_block_store(mn, mx, s1, s2, &folded);
+    if (threadIdx.x != 0) return;
+    const StatsPartial r = folded;
+    const double nd = static_cast<double>(n);
+    if constexpr (STAGE == 0) {
+        *totals = r;
+        if constexpr (ONE_PASS) {
+            const float mean = static_cast<float>(r.s1 / nd);
+            const double md = static_cast<double>(mean);
+            const float variance = static_cast<float>(r.s2 / nd - md * md);
+            out->min_val = r.mn;
+            out->max_val = r.mx;
+            out->mean = mean;
+            out->variance = variance;
+            out->std_dev = sqrtf(variance);
+        }
+    } else {
+        const double variance = r.s2 / nd;
+        out->min_val = totals->mn;
+        out->max_val = totals->mx;
+        out->mean = static_cast<float>(totals->s1 / nd);
+        out->variance = static_cast<float>(variance);
+        out->std_dev = static_cast<float>(sqrt(variance));
+    }
+}
+
 // ---- observer statistics -------------------------------------------------------------------
 
 struct ObservePartial {
@@ -516,6 +620,28 @@ int32_t hipq_fake_quantize_f32(hipq_ctx *ctx, const float *x, size_t n, float sc
     else
         launch_fq<false, false>(ic, grid, ctx->stream, x, n, fq, out);
     return check_launch("fake_quantize_kernel");
+}
+
+int32_t hipq_tensor_stats_f32(hipq_ctx *ctx, const float *x, size_t n, int32_t one_pass, hipq_tensor_stats *out_stats) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(out_stats);
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot calculate stats of empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    const int grid = calib_grid(ctx, n, kCalTile * 4);
+    void *scr = nullptr;
+    int32_t rc = scratch(ctx, kScratchHeader + sizeof(StatsPartial) * static_cast<size_t>(ctx->num_cus) * kMaxWgPerCu, &scr);
+    if (rc != HIPQ_SUCCESS) return rc;
+    StatsPartial *totals = reinterpret_cast<StatsPartial *>(scr);  // in the scratch header
+    StatsPartial *partials = reinterpret_cast<StatsPartial *>(static_cast<char *>(scr) + kScratchHeader);
+    stats_partial_kernel<false><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, totals, partials);
+    if (one_pass) {
+        stats_final_kernel<0, true><<<1, kCalBlock, 0, ctx->stream>>>(partials, grid, n, totals, out_stats);
+        return check_launch("tensor_stats");
+    }
+    stats_final_kernel<0, false><<<1, kCalBlock, 0, ctx->stream>>>(partials, grid, n, totals, out_stats);
+    stats_partial_kernel<true><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, totals, partials);
+    stats_final_kernel<1, false><<<1, kCalBlock, 0, ctx->stream>>>(partials, grid, n, totals, out_stats);
+    return check_launch("tensor_stats");
 }
 
 int32_t hipq_observe_f32(hipq_ctx *ctx, const float *x, size_t n, hipq_observe_stats *out_stats) {

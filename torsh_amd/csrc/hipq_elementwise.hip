@@ -161,7 +161,7 @@ struct DynamicRange {
 // memory when `params` is non-null, or (dynamic quantization) from the range partials: then
 // every workgroup folds the same few hundred partials in the same order, derives the same
 // parameters, and workgroup 0 publishes them, which saves the launch of a finalize kernel.
-template <typename OutT, bool DIV, bool EVEN>
+template <typename OutT, bool DIV, int RND>
 __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restrict__ x, size_t n, float scale,
                                                            int zp, const hipq_qparams *__restrict__ params,
                                                            DynamicRange dyn, float lo, float hi,
@@ -206,16 +206,16 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
     const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
     auto emit = [&](size_t idx, const float4 &t) {
         if constexpr (sizeof(OutT) == 4) {
-            const float a = quantize_value<DIV, EVEN>(t.x, scale, inv, zpf, lo, hi);
-            const float b = quantize_value<DIV, EVEN>(t.y, scale, inv, zpf, lo, hi);
-            const float c = quantize_value<DIV, EVEN>(t.z, scale, inv, zpf, lo, hi);
-            const float d = quantize_value<DIV, EVEN>(t.w, scale, inv, zpf, lo, hi);
+            const float a = quantize_value<DIV, RND>(t.x, scale, inv, zpf, lo, hi);
+            const float b = quantize_value<DIV, RND>(t.y, scale, inv, zpf, lo, hi);
+            const float c = quantize_value<DIV, RND>(t.z, scale, inv, zpf, lo, hi);
+            const float d = quantize_value<DIV, RND>(t.w, scale, inv, zpf, lo, hi);
             store_stream(reinterpret_cast<float4 *>(out) + idx, make_float4(a, b, c, d));
         } else {
-            const int a = quantize_int<DIV, EVEN>(t.x, scale, inv, zpf, ilo, ihi);
-            const int b = quantize_int<DIV, EVEN>(t.y, scale, inv, zpf, ilo, ihi);
-            const int c = quantize_int<DIV, EVEN>(t.z, scale, inv, zpf, ilo, ihi);
-            const int d = quantize_int<DIV, EVEN>(t.w, scale, inv, zpf, ilo, ihi);
+            const int a = quantize_int<DIV, RND>(t.x, scale, inv, zpf, ilo, ihi);
+            const int b = quantize_int<DIV, RND>(t.y, scale, inv, zpf, ilo, ihi);
+            const int c = quantize_int<DIV, RND>(t.z, scale, inv, zpf, ilo, ihi);
+            const int d = quantize_int<DIV, RND>(t.w, scale, inv, zpf, ilo, ihi);
             store_stream(reinterpret_cast<uint32_t *>(out) + idx, pack4(a, b, c, d));
         }
     };
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
         }
     }
     for (size_t i = nvec * 4 + size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += size_t(gridDim.x) * kBlock)
-        out[i] = to_out<OutT>(quantize_value<DIV, EVEN>(x[i], scale, inv, zpf, lo, hi));
+        out[i] = to_out<OutT>(quantize_value<DIV, RND>(x[i], scale, inv, zpf, lo, hi));
 }
 
 template <typename InT>
@@ -530,17 +530,22 @@ static int32_t launch_quantize(hipq_ctx *ctx, const float *x, size_t n, float sc
                                DynamicRange dyn = DynamicRange{nullptr, 0, 0, 0, 0, nullptr}) {
     const int grid = grid_for_tiles(ctx, n);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    const bool half_up = (mode & HIPQ_ROUND_FLOOR_HALF_UP) != 0;
 #define HIPQ_LAUNCH_Q(D, E)                                                                                   \
     hipLaunchKernelGGL((quantize_kernel<OutT, D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, scale, zp, \
                        params, dyn, lo, hi, out)
-    if (div && even)
-        HIPQ_LAUNCH_Q(true, true);
+    if (half_up && div)
+        HIPQ_LAUNCH_Q(true, 2);
+    else if (half_up)
+        HIPQ_LAUNCH_Q(false, 2);
+    else if (div && even)
+        HIPQ_LAUNCH_Q(true, 1);
     else if (div)
-        HIPQ_LAUNCH_Q(true, false);
+        HIPQ_LAUNCH_Q(true, 0);
     else if (even)
-        HIPQ_LAUNCH_Q(false, true);
+        HIPQ_LAUNCH_Q(false, 1);
     else
-        HIPQ_LAUNCH_Q(false, false);
+        HIPQ_LAUNCH_Q(false, 0);
 #undef HIPQ_LAUNCH_Q
     return check_launch("quantize");
 }
@@ -616,7 +621,10 @@ int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n,
     HIPQ_ENTER(ctx);
     int32_t rc = check_scale(__func__, scale);
     if (rc) return rc;
-    if ((rc = check_mode(__func__, mode))) return rc;
+    // this entry point alone also knows the floor(v + 0.5) rounding of quantize_mobile_optimized
+    if ((rc = check_mode(__func__, mode & ~HIPQ_ROUND_FLOOR_HALF_UP))) return rc;
+    if ((mode & HIPQ_ROUND_FLOOR_HALF_UP) && (mode & HIPQ_ROUND_HALF_EVEN))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: two rounding modes in mode 0x%x", __func__, mode);
     if (n == 0) return HIPQ_SUCCESS;
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);

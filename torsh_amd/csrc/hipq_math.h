@@ -32,16 +32,20 @@ __device__ __forceinline__ void store_stream(float4 *p, float4 v) {
 }
 __device__ __forceinline__ void store_stream(uint32_t *p, uint32_t v) { __builtin_nontemporal_store(v, p); }
 
-// f32::round (half away from zero) or IEEE nearest-even.
+// RND 0: f32::round (half away from zero); 1: IEEE nearest-even; 2: floor(v + 0.5), the
+// "faster rounding" of quantize_mobile_optimized (crates/torsh-quantization/src/simd_ops.rs:426-428),
+// with the f32 sum rounded before the floor as there.  Callers that know two modes pass a bool.
 // Half away from zero as trunc(v + copysign(h, v)) with h the largest float below 0.5: three
 // instructions (v_bfi, v_add, v_trunc) instead of the six of the library roundf.  With 0.5 itself
 // the sum rounds up across an integer for v = +-0.49999997; with h it never does, and ties still
 // land on the integer away from zero because v + h then rounds to even = that integer.  Checked
 // against roundf for every finite float (tests/host/round_away_check.c).
-template <bool EVEN>
+template <int RND>
 __device__ __forceinline__ float round_mode(float v) {
-    if constexpr (EVEN)
+    if constexpr (RND == 1)
         return rintf(v);
+    else if constexpr (RND == 2)
+        return floorf(v + 0.5f);
     else
         return truncf(v + copysignf(0x1.fffffep-2f, v));
 }
@@ -86,14 +90,14 @@ __device__ __forceinline__ float div_rn(float a, float b, float y) {
 
 // round(x * inv | x / scale) + zp, clamped; result still a float (the carrier).
 // DIV: `inv` is recip_for_div(scale); otherwise 1.0f / scale.
-template <bool DIV, bool EVEN>
+template <bool DIV, int RND>
 __device__ __forceinline__ float quantize_value(float x, float scale, float inv, float zpf, float lo, float hi) {
     float t;
     if constexpr (DIV)
         t = div_rn(x, scale, inv);
     else
         t = x * inv;
-    float q = round_mode<EVEN>(t) + zpf;
+    float q = round_mode<RND>(t) + zpf;
     return clamp_keep_nan(q, lo, hi);
 }
 
@@ -110,14 +114,14 @@ __device__ __forceinline__ int cvt_i32_sat(float v) {
 // conversion, on integers (round(..)+zp is integral, so converting first changes nothing;
 // a NaN becomes 0 as `NaN.clamp(..) as i8` does, and +-Inf saturate).  About half the
 // vector instructions of the float-clamp form.
-template <bool DIV, bool EVEN>
+template <bool DIV, int RND>
 __device__ __forceinline__ int quantize_int(float x, float scale, float inv, float zpf, int lo, int hi) {
     float t;
     if constexpr (DIV)
         t = div_rn(x, scale, inv);
     else
         t = x * inv;
-    const int q = cvt_i32_sat(round_mode<EVEN>(t) + zpf);
+    const int q = cvt_i32_sat(round_mode<RND>(t) + zpf);
     return min(max(q, lo), hi);
 }
 

@@ -18,6 +18,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 
 SUCCESS, INVALID_ARGUMENT, SHAPE_ERROR, DIMENSION_MISMATCH, DEVICE_ERROR, ALLOCATION_ERROR, SYNCHRONIZATION_ERROR, UNKNOWN_ERROR = range(8)
 ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
+ROUND_FLOOR_HALF_UP = 16  # hipq_quantize_per_tensor_f32_i8 only
 FORM_MUL_INV, FORM_DIV = 0, 2
 DTYPE_I8, DTYPE_U8 = 0, 1
 PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC, PARAMS_ZERO_INCLUDED = range(5)
@@ -56,6 +57,11 @@ class QuantMetrics(C.Structure):
 
 class ObserveStats(C.Structure):
     _fields_ = [("min_val", C.c_float), ("max_val", C.c_float), ("nonfinite", C.c_uint64)]
+
+
+class TensorStats(C.Structure):
+    _fields_ = [("min_val", C.c_float), ("max_val", C.c_float), ("mean", C.c_float), ("std_dev", C.c_float),
+                ("variance", C.c_float)]
 
 
 _lib: Optional[C.CDLL] = None
@@ -115,6 +121,7 @@ _SIGNATURES = {
     "hipq_fake_quantize_metrics_f32": [_vp, _vp, _sz, _f32, _i32, _vp, _i32, _i32, _i32, C.c_uint32, C.c_uint32, _vp],
     "hipq_fake_quantize_f32": [_vp, _vp, _sz, _f32, _i32, _vp, _i32, _i32, _i32, _vp],
     "hipq_observe_f32": [_vp, _vp, _sz, _vp],
+    "hipq_tensor_stats_f32": [_vp, _vp, _sz, _i32, _vp],
     "hipq_histogram_f32": [_vp, _vp, _sz, _f32, _f32, _sz, _vp],
     "hipq_conv2d_u8i8_i32": [_vp, _vp, _i32, _vp] + [_sz] * 11 + [_vp],
     "hipq_conv2d_u8i8_i8": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_f32, _i32, _i32, _vp],
@@ -298,6 +305,13 @@ class Context:
         out = out if out is not None else self._record(ObserveStats)
         self.call("hipq_observe_f32", _ptr(x), x.numel(), _ptr(out))
         return out
+
+    def tensor_stats(self, x, one_pass=False, out=None):
+        """min, max, mean, std_dev, variance (population) of x; one_pass selects the raw-moment form.  Returns the
+        record read back, or with `out` (a device record) leaves it there and returns `out`."""
+        rec = out if out is not None else self._record(TensorStats)
+        self.call("hipq_tensor_stats_f32", _ptr(x), x.numel(), int(one_pass), _ptr(rec))
+        return rec if out is not None else self._read(rec, TensorStats)
 
     def read_observe(self, buf: torch.Tensor) -> ObserveStats:
         return self._read(buf, ObserveStats)

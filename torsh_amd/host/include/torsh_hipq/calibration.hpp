@@ -143,7 +143,9 @@ class Observer {
     static Observer min_max() { return Observer(ObserverType::MinMax); }
     static Observer moving_average() { return Observer(ObserverType::MovingAverage); }
     static Observer histogram() { return Observer(ObserverType::Histogram); }
-    static Observer histogram_with_bins(size_t num_bins) {  // :76-91
+    static Observer new_histogram(size_t num_bins) { return histogram_with_bins(num_bins); }    // :76-91
+    static Observer new_percentile(float percentile) { return percentile_with_value(percentile); }  // :94-109
+    static Observer histogram_with_bins(size_t num_bins) {
         Observer o(ObserverType::Histogram);
         o.num_bins_ = num_bins;
         o.histogram_.assign(num_bins, 0);

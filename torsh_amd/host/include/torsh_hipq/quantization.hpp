@@ -16,6 +16,10 @@
 //   quantize_auto                     algorithms.rs:436-438
 //   quantize_per_tensor_affine_simd, dequantize_per_tensor_affine_simd, find_min_max_simd,
 //   quantize_to_int8_simd             crates/torsh-quantization/src/simd_ops.rs:18,52,84,196
+//   CacheAwareParams and the cache-aware / tiled / streaming quantizers, tensor statistics
+//                                     algorithms.rs:440-735
+//   quantize_batch_consistent_simd, calculate_tensor_stats_simd, the NEON and mobile twins
+//                                     simd_ops.rs:170-193, 230-476
 //   QScheme, QuantConfig              crates/torsh-quantization/src/config.rs:31-52, 95-128, 158-409
 //
 // quantize_with_config also dispatches the special schemes (int4, binary, ternary, group-wise) to
@@ -25,7 +29,9 @@
 #include <cfloat>
 #include <cmath>
 #include <optional>
+#include <string>
 #include <tuple>
+#include <vector>
 
 #include "core.hpp"
 
@@ -281,6 +287,155 @@ inline Result<Unit> dequantize_per_tensor_affine_simd(const std::vector<float> &
     output = std::move(y);
     return Unit{};
 }
+
+// ---- the slice-level twins: cache-aware, tiled, streaming, NEON, mobile, batch ----
+// algorithms.rs:440-735 and simd_ops.rs:170-193, 230-476.  Their chunk sizes, tile shapes and
+// prefetch hints steer a CPU's caches; the element arithmetic is one formula, so each is one call
+// of the streaming kernel here, and the cache parameters are accepted and ignored.
+
+// algorithms.rs:443-471
+struct CacheAwareParams {
+    size_t cache_line_size = 64;
+    size_t l1_cache_size = 32 * 1024;
+    size_t l2_cache_size = 256 * 1024;
+    size_t l3_cache_size = 8 * 1024 * 1024;
+    size_t prefetch_distance = 16;
+    bool enable_chunking = true;
+};
+
+// algorithms.rs:473-522: q = clamp(round(x * (1/scale)) + zp, -128, 127), f32 carrier.
+inline Result<Unit> quantize_per_tensor_affine_cache_aware(const std::vector<float> &input, float scale,
+                                                           int32_t zero_point, std::vector<float> &output,
+                                                           const CacheAwareParams & /*cache_params*/) {
+    return quantize_per_tensor_affine_simd(input, scale, zero_point, output);  // same checks, same messages
+}
+
+// algorithms.rs:581-635
+inline Result<Unit> quantize_matrix_cache_friendly(const std::vector<float> &matrix, size_t rows, size_t cols,
+                                                   float scale, int32_t zero_point, std::vector<float> &output,
+                                                   const CacheAwareParams & /*cache_params*/) {
+    if (matrix.size() != rows * cols || output.size() != rows * cols)
+        return TorshError::invalid_argument("Matrix dimensions don't match buffer sizes");
+    return quantize_per_tensor_affine_simd(matrix, scale, zero_point, output);
+}
+
+// algorithms.rs:638-674
+inline Result<Unit> quantize_streaming_with_prefetch(const std::vector<float> &input, float scale, int32_t zero_point,
+                                                     std::vector<float> &output,
+                                                     const CacheAwareParams & /*cache_params*/) {
+    return quantize_per_tensor_affine_simd(input, scale, zero_point, output);
+}
+
+// algorithms.rs:711-735: every branch of the reference's size switch ends in the same arithmetic.
+inline Result<Unit> quantize_with_cache_optimization(const std::vector<float> &input, float scale, int32_t zero_point,
+                                                     std::vector<float> &output,
+                                                     const CacheAwareParams * /*cache_params*/ = nullptr) {
+    return quantize_per_tensor_affine_simd(input, scale, zero_point, output);
+}
+
+// algorithms.rs:677-708 (advice about a CPU's caches; kept for callers that print it).
+inline std::vector<std::string> get_cache_optimization_recommendations(size_t tensor_size, size_t element_size,
+                                                                       const CacheAwareParams &cache_params) {
+    std::vector<std::string> r;
+    const size_t total_bytes = tensor_size * element_size;
+    if (total_bytes <= cache_params.l1_cache_size) {
+        r.push_back("Tensor fits in L1 cache - use simple sequential access");
+    } else if (total_bytes <= cache_params.l2_cache_size) {
+        r.push_back("Tensor fits in L2 cache - consider blocked algorithms");
+    } else if (total_bytes <= cache_params.l3_cache_size) {
+        r.push_back("Tensor fits in L3 cache - use tiled processing with medium blocks");
+    } else {
+        r.push_back("Large tensor - use streaming algorithms with prefetching");
+        r.push_back("Consider parallel processing to utilize multiple cache hierarchies");
+    }
+    const size_t per_line = cache_params.cache_line_size / element_size;
+    if (tensor_size % per_line != 0)
+        r.push_back("Consider padding to align with cache lines (" + std::to_string(cache_params.cache_line_size) +
+                    "B boundaries)");
+    return r;
+}
+
+// simd_ops.rs:264-272
+struct TensorStats {
+    float min = 0, max = 0, mean = 0, std_dev = 0, variance = 0;
+};
+
+namespace detail {
+inline Result<hipq_tensor_stats> tensor_stats(const std::vector<float> &data, bool one_pass) {
+    if (data.empty()) return TorshError::invalid_argument("Cannot calculate stats of empty tensor");
+    TORSH_TRY(ctx, hip::Runtime::ctx());
+    TORSH_TRY(dx, hip::DeviceBuffer::from_host(ctx, data.data(), data.size()));
+    TORSH_TRY(ds, hip::DeviceBuffer::alloc(ctx, sizeof(hipq_tensor_stats)));
+    TORSH_CHECK(hip::check(hipq_tensor_stats_f32(ctx, dx.as<float>(), data.size(), one_pass ? 1 : 0,
+                                                 ds.as<hipq_tensor_stats>())));
+    TORSH_TRY(st, ds.to_host<hipq_tensor_stats>(1));
+    return st[0];
+}
+}  // namespace detail
+
+// simd_ops.rs:230-262: range, f64 mean, population variance from a second pass.
+inline Result<TensorStats> calculate_tensor_stats_simd(const std::vector<float> &data) {
+    TORSH_TRY(st, detail::tensor_stats(data, false));
+    return TensorStats{st.min_val, st.max_val, st.mean, st.std_dev, st.variance};
+}
+
+// algorithms.rs:525-578: (min, max, mean, std_dev) from the raw moments.
+inline Result<std::tuple<float, float, float, float>> calculate_tensor_stats_cache_optimized(
+    const std::vector<float> &data, const CacheAwareParams & /*cache_params*/) {
+    TORSH_TRY(st, detail::tensor_stats(data, true));
+    return std::make_tuple(st.min_val, st.max_val, st.mean, st.std_dev);
+}
+
+// simd_ops.rs:170-193: the same parameters for every tensor of the batch.
+inline Result<Unit> quantize_batch_consistent_simd(const std::vector<const std::vector<float> *> &tensors, float scale,
+                                                   int32_t zero_point, std::vector<std::vector<float> *> &outputs) {
+    if (tensors.size() != outputs.size())
+        return TorshError::invalid_argument("Number of input tensors must match output tensors");
+    for (size_t i = 0; i < tensors.size(); ++i)
+        TORSH_CHECK(quantize_per_tensor_affine_simd(*tensors[i], scale, zero_point, *outputs[i]));
+    return Unit{};
+}
+
+// simd_ops.rs:302-350 and 354-387 (compiled for aarch64 only in the reference; same arithmetic).
+inline Result<Unit> quantize_neon_optimized(const std::vector<float> &input, float scale, int32_t zero_point,
+                                            std::vector<float> &output) {
+    return quantize_per_tensor_affine_simd(input, scale, zero_point, output);
+}
+inline Result<std::pair<float, float>> find_min_max_neon(const std::vector<float> &data) {
+    return find_min_max_simd(data);
+}
+
+// simd_ops.rs:390-446: int8 output; with use_reduced_precision and more than 256 elements the
+// rounding is floor(x * inv + 0.5).
+inline Result<Unit> quantize_mobile_optimized(const std::vector<float> &input, float scale, int32_t zero_point,
+                                              std::vector<int8_t> &output, bool use_reduced_precision) {
+    if (input.size() != output.size())
+        return TorshError::invalid_argument("Input and output length mismatch");
+    if (scale <= 0.0f) return TorshError::invalid_argument("Scale must be positive");
+    if (input.empty()) return Unit{};
+    const int32_t mode = HIPQ_FORM_MUL_INV |
+                         ((use_reduced_precision && input.size() > 256) ? HIPQ_ROUND_FLOOR_HALF_UP : HIPQ_ROUND_HALF_AWAY);
+    TORSH_TRY(ctx, hip::Runtime::ctx());
+    TORSH_TRY(dx, hip::DeviceBuffer::from_host(ctx, input.data(), input.size()));
+    TORSH_TRY(dq, hip::DeviceBuffer::alloc(ctx, input.size()));
+    TORSH_CHECK(hip::check(hipq_quantize_per_tensor_f32_i8(ctx, dx.as<float>(), input.size(), scale, zero_point, mode,
+                                                           dq.as<int8_t>())));
+    TORSH_TRY(q, dq.to_host<int8_t>(input.size()));
+    output = std::move(q);
+    return Unit{};
+}
+
+// simd_ops.rs:274-298, 449-471: what the reference reports on its default x86-64 build.
+inline bool is_simd_available() { return detail::is_simd_available(); }
+inline size_t get_simd_width() { return 4; }
+struct MobileOptimizationHints {
+    bool prefer_int8 = true;
+    bool use_reduced_precision = false;
+    size_t optimal_chunk_size = 512;
+    bool enable_fast_math = true;
+    bool prefer_sequential = false;
+};
+inline MobileOptimizationHints get_mobile_optimization_hints() { return MobileOptimizationHints{}; }
 
 // ---- tensor-level functions (algorithms.rs) ----
 
