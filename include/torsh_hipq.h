@@ -227,6 +227,19 @@ HIPQ_API int32_t hipq_quantize_binary_f32_i8(hipq_ctx *ctx, const float *x, size
                                              hipq_qparams *out_params);
 HIPQ_API int32_t hipq_quantize_ternary_f32_i8(hipq_ctx *ctx, const float *x, size_t n, int8_t *out,
                                               hipq_qparams *out_params);
+/* quantize_binary_learned_threshold, crates/torsh-quantization/src/specialized.rs:439-492:
+ * threshold = the given one (has_threshold != 0) or mean |x|; out = 0 where |x| <= threshold,
+ * else x >= 0 ? 1 : -1; scale = mean of |x| over the values above the threshold (1 if none).
+ * quantize_ternary_adaptive, specialized.rs:495-552: of the ten thresholds max|x| * (i * 0.1),
+ * i = 1..10, the first with the smallest mean squared error of the unit ternary code
+ * (specialized.rs:555-570); out and scale as quantize_ternary with that threshold.
+ * out_params: scale, zero point 0, min_val = the threshold used, max_val = max |x| (adaptive)
+ * or 0.  n == 0 is InvalidArgument.  Means and errors are formed from f64 sums. */
+HIPQ_API int32_t hipq_quantize_binary_learned_threshold_f32_i8(hipq_ctx *ctx, const float *x, size_t n,
+                                                               int32_t has_threshold, float threshold, int8_t *out,
+                                                               hipq_qparams *out_params);
+HIPQ_API int32_t hipq_quantize_ternary_adaptive_f32_i8(hipq_ctx *ctx, const float *x, size_t n, int8_t *out,
+                                                       hipq_qparams *out_params);
 /* quantize_per_channel_affine, explicit parameters,
  * crates/torsh-quantization/src/quantize.rs:287-331 (HIPQ_FORM_DIV) and
  * quantize_per_channel_simd, simd_ops.rs:124-169 (HIPQ_FORM_MUL_INV, inner

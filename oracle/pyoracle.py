@@ -96,6 +96,10 @@ def _declare(l: C.CDLL) -> None:
     l.tq_quantize_int4_per_channel.argtypes = [_f32p, _szp, C.c_size_t, C.c_size_t, _f32p, _f32p, _i32p, _f32p, _i32p]
     l.tq_quantize_binary.argtypes = [_f32p, C.c_size_t, _f32p, _f32p, C.POINTER(C.c_double)]
     l.tq_quantize_ternary.argtypes = [_f32p, C.c_size_t, _f32p, _f32p, C.POINTER(C.c_double), _f32p]
+    l.tq_quantize_binary_learned_threshold.argtypes = [_f32p, C.c_size_t, C.c_int, C.c_float, C.c_int, _f32p, _f32p,
+                                                       C.POINTER(C.c_double), _f32p]
+    l.tq_quantize_ternary_adaptive.argtypes = [_f32p, C.c_size_t, C.c_int, _f32p, _f32p, C.POINTER(C.c_double), _f32p,
+                                               _f32p, C.POINTER(C.c_double)]
     l.tq_quantize_group_wise.argtypes = [_f32p, _szp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int32, C.c_int32, _f32p,
                                          _f32p, _i32p, _f32p, _i32p]
     l.tq_model_mse_error.restype = C.c_double
@@ -668,6 +672,30 @@ def quantize_ternary(x):
     _check(lib().tq_quantize_ternary(_p(x, _f32p), C.c_size_t(x.size), _p(out, _f32p), C.byref(s), C.byref(d),
                                      C.byref(t)), "quantize_ternary")
     return out, np.float32(s.value), d.value, np.float32(t.value)
+
+
+def quantize_binary_learned_threshold(x, threshold=None, f64_sums=False):
+    """-> (carrier, scale, scale from an f64 sum, threshold used)"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    s, d, t = C.c_float(), C.c_double(), C.c_float()
+    _check(lib().tq_quantize_binary_learned_threshold(_p(x, _f32p), C.c_size_t(x.size), int(threshold is not None),
+                                                      C.c_float(threshold or 0.0), int(f64_sums), _p(out, _f32p),
+                                                      C.byref(s), C.byref(d), C.byref(t)),
+           "quantize_binary_learned_threshold")
+    return out, np.float32(s.value), d.value, np.float32(t.value)
+
+
+def quantize_ternary_adaptive(x, f64_sums=False):
+    """-> (carrier, scale, scale from an f64 sum, threshold chosen, ten f32-sum errors, ten f64-sum errors)"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    s, d, t = C.c_float(), C.c_double(), C.c_float()
+    e32, e64 = np.empty(10, np.float32), np.empty(10, np.float64)
+    _check(lib().tq_quantize_ternary_adaptive(_p(x, _f32p), C.c_size_t(x.size), int(f64_sums), _p(out, _f32p),
+                                              C.byref(s), C.byref(d), C.byref(t), _p(e32, _f32p),
+                                              e64.ctypes.data_as(C.POINTER(C.c_double))), "quantize_ternary_adaptive")
+    return out, np.float32(s.value), d.value, np.float32(t.value), e32, e64
 
 
 def quantize_group_wise(x, axis, group_size, qmin=-128, qmax=127):

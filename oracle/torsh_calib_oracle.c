@@ -541,6 +541,87 @@ int tq_quantize_ternary(const float *x, size_t n, float *out, float *scale, doub
     return 0;
 }
 
+/* specialized.rs:439-492 */
+int tq_quantize_binary_learned_threshold(const float *x, size_t n, int has_threshold, float threshold, int f64_sums,
+                                         float *out, float *scale, double *scale_f64, float *threshold_out) {
+    if (n == 0) return 1;
+    float thr = threshold;
+    if (!has_threshold) { /* :452-456 */
+        float abs_sum = 0.0f;
+        double abs_dsum = 0.0;
+        for (size_t i = 0; i < n; ++i) {
+            abs_sum += fabsf(x[i]);
+            abs_dsum += (double)fabsf(x[i]);
+        }
+        thr = f64_sums ? (float)(abs_dsum / (double)n) : abs_sum / (float)n;
+    }
+    float sum = 0.0f;
+    double dsum = 0.0;
+    size_t count = 0;
+    for (size_t i = 0; i < n; ++i)
+        if (fabsf(x[i]) > thr) { /* :459-463 */
+            sum += fabsf(x[i]);
+            dsum += (double)fabsf(x[i]);
+            ++count;
+        }
+    *scale = count > 0 ? sum / (float)count : 1.0f;
+    if (scale_f64) *scale_f64 = count > 0 ? dsum / (double)count : 1.0;
+    if (threshold_out) *threshold_out = thr;
+    for (size_t i = 0; i < n; ++i) out[i] = fabsf(x[i]) <= thr ? 0.0f : (x[i] >= 0.0f ? 1.0f : -1.0f); /* :473-481 */
+    return 0;
+}
+
+/* specialized.rs:555-570 */
+static void ternary_error(const float *x, size_t n, float thr, float *err, double *err64) {
+    float s = 0.0f;
+    double d = 0.0;
+    for (size_t i = 0; i < n; ++i) {
+        const float q = fabsf(x[i]) <= thr ? 0.0f : (x[i] > 0.0f ? 1.0f : -1.0f);
+        const float diff = x[i] - q;
+        const float sq = diff * diff;
+        s += sq;
+        d += (double)sq;
+    }
+    *err = s / (float)n;
+    *err64 = d / (double)n;
+}
+
+/* specialized.rs:495-552 */
+int tq_quantize_ternary_adaptive(const float *x, size_t n, int f64_sums, float *out, float *scale, double *scale_f64,
+                                 float *threshold_out, float errors[10], double errors_f64[10]) {
+    if (n == 0) return 1;
+    float max_abs = 0.0f;
+    for (size_t i = 0; i < n; ++i) max_abs = fmaxf(max_abs, fabsf(x[i]));
+    float best_thr = 0.0f, best_err = INFINITY;
+    for (int i = 1; i <= 10; ++i) { /* :510-517 */
+        const float thr = max_abs * ((float)i * 0.1f);
+        float e;
+        double e64;
+        ternary_error(x, n, thr, &e, &e64);
+        if (errors) errors[i - 1] = e;
+        if (errors_f64) errors_f64[i - 1] = e64;
+        const float cmp = f64_sums ? (float)e64 : e;
+        if (cmp < best_err) {
+            best_err = cmp;
+            best_thr = thr;
+        }
+    }
+    float sum = 0.0f;
+    double dsum = 0.0;
+    size_t count = 0;
+    for (size_t i = 0; i < n; ++i)
+        if (fabsf(x[i]) > best_thr) {
+            sum += fabsf(x[i]);
+            dsum += (double)fabsf(x[i]);
+            ++count;
+        }
+    *scale = count > 0 ? sum / (float)count : 1.0f;
+    if (scale_f64) *scale_f64 = count > 0 ? dsum / (double)count : 1.0;
+    if (threshold_out) *threshold_out = best_thr;
+    for (size_t i = 0; i < n; ++i) out[i] = fabsf(x[i]) <= best_thr ? 0.0f : (x[i] > 0.0f ? 1.0f : -1.0f);
+    return 0;
+}
+
 /* specialized.rs:241-377 */
 int tq_quantize_group_wise(const float *x, const size_t *shape, size_t ndim, size_t axis, size_t group_size,
                            int32_t qmin, int32_t qmax, float *out, float *group_scales, int32_t *group_zps,

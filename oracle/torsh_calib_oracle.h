@@ -107,6 +107,19 @@ int tq_quantize_int4_per_channel(const float *x, const size_t *shape, size_t ndi
 int tq_quantize_binary(const float *x, size_t n, float *out, float *scale, double *scale_f64);
 /* quantize_ternary, specialized.rs:191-238; threshold (may be NULL) receives 0.7 * max|x|. */
 int tq_quantize_ternary(const float *x, size_t n, float *out, float *scale, double *scale_f64, float *threshold);
+/* quantize_binary_learned_threshold, specialized.rs:439-492.  has_threshold == 0 learns the
+ * threshold as mean |x|.  f64_sums != 0 forms that mean (and nothing else) from an f64 sum instead
+ * of the reference's sequential f32 sum: the threshold the f32 sum approaches, and the one a
+ * reduction in any other order can be compared with element by element.  scale is always the
+ * reference's f32 sum; scale_f64 (may be NULL) the f64 one.  threshold_out receives the threshold. */
+int tq_quantize_binary_learned_threshold(const float *x, size_t n, int has_threshold, float threshold, int f64_sums,
+                                         float *out, float *scale, double *scale_f64, float *threshold_out);
+/* quantize_ternary_adaptive, specialized.rs:495-552 with calculate_ternary_error, :555-570.
+ * errors (may be NULL) receives the ten mean errors as the reference forms them (f32 sums),
+ * errors_f64 (may be NULL) the same from f64 sums; f64_sums != 0 selects the threshold by the
+ * latter. */
+int tq_quantize_ternary_adaptive(const float *x, size_t n, int f64_sums, float *out, float *scale, double *scale_f64,
+                                 float *threshold_out, float errors[10], double errors_f64[10]);
 /* quantize_group_wise, specialized.rs:241-377 with the integer range [qmin, qmax] of
  * config.get_qint_range().  group_scales / group_zps hold num_groups = ceil(shape[axis]/group_size). */
 int tq_quantize_group_wise(const float *x, const size_t *shape, size_t ndim, size_t axis, size_t group_size,

@@ -1315,6 +1315,81 @@ GPU_TEST(test_special_schemes) {  // specialized.rs:577-654, 743-761
     CHECK(quantize_with_config(t3, QuantConfig::group_wise(0, 2)).is_ok());
 }
 
+GPU_TEST(test_searched_thresholds_and_mixed_precision) {  // specialized.rs:655-740
+    {
+        const std::vector<float> data{-2.0f, -0.1f, 0.1f, 0.5f, 2.0f};
+        const auto [q, scale, zp, threshold] = quantize_binary_learned_threshold(tensor_1d(data).unwrap(), 0.3f).unwrap();
+        CHECK(scale > 0.0f && zp == 0);
+        CHECK_EQ(threshold, 0.3f);
+        for (size_t i = 0; i < data.size(); ++i) {
+            const float expected = std::fabs(data[i]) <= 0.3f ? 0.0f : (data[i] >= 0.0f ? 1.0f : -1.0f);
+            CHECK_EQ(q.as_slice()[i], expected);
+        }
+    }
+    {
+        const std::vector<float> data{-3.0f, -0.5f, 0.0f, 0.5f, 3.0f};
+        const auto [q, scale, zp, threshold] = quantize_ternary_adaptive(tensor_1d(data).unwrap()).unwrap();
+        CHECK(scale > 0.0f && zp == 0 && threshold > 0.0f);
+        CHECK_EQ(q.numel(), data.size());
+        for (float v : q.as_slice()) CHECK(v == -1.0f || v == 0.0f || v == 1.0f);
+    }
+    std::map<std::string, Tensor> tensors;
+    tensors.emplace("embedding", tensor_1d({1.0f, 2.0f, 3.0f}).unwrap());
+    tensors.emplace("attention", tensor_1d({4.0f, 5.0f, 6.0f}).unwrap());
+    const MixedPrecisionConfig config;
+    const auto results = quantize_mixed_precision(tensors, config).unwrap();
+    CHECK_EQ(results.size(), size_t(2));
+    CHECK(results.count("embedding") == 1 && results.count("attention") == 1);
+    // specialized.rs:678-690
+    CHECK(determine_layer_precision("layer.embedding.weight", config) == DType::I8);
+    CHECK(determine_layer_precision("layer.attention.query", config) == DType::F16);
+    CHECK(determine_layer_precision("layer.unknown.weight", config) == DType::I8);  // default
+    CHECK(determine_layer_precision("head.output", config) == DType::F32);
+    CHECK(create_precision_config(DType::U8).dtype == DType::U8 && create_precision_config(DType::I32).dtype == DType::I8);
+    CHECK(create_precision_config(DType::F16).dtype == DType::F16 && !create_precision_config(DType::F32).enable_fake_quant);
+    const Tensor empty = tensor_1d({}).unwrap();
+    CHECK(quantize_binary_learned_threshold(empty).is_err() && quantize_ternary_adaptive(empty).is_err());
+}
+
+GPU_TEST(parity_searched_thresholds_and_mixed_precision) {
+    const std::vector<float> x = normal(20011, 91, 1.2f);
+    const Tensor t = tensor_1d(x).unwrap();
+    std::vector<float> want(x.size());
+    float s32, thr;
+    double s64;
+    for (int given = 0; given < 2; ++given) {
+        CHECK_EQ(tq_quantize_binary_learned_threshold(x.data(), x.size(), given, 0.45f, 1, want.data(), &s32, &s64, &thr), 0);
+        const auto [q, scale, zp, threshold] =
+            quantize_binary_learned_threshold(t, given ? std::optional<float>(0.45f) : std::nullopt).unwrap();
+        check_same(q.as_slice(), want, __LINE__);
+        CHECK(zp == 0 && threshold == thr);
+        CHECK(std::fabs(scale - s64) <= 1e-6 * s64);
+    }
+    CHECK_EQ(tq_quantize_ternary_adaptive(x.data(), x.size(), 1, want.data(), &s32, &s64, &thr, nullptr, nullptr), 0);
+    {
+        const auto [q, scale, zp, threshold] = quantize_ternary_adaptive(t).unwrap();
+        check_same(q.as_slice(), want, __LINE__);
+        CHECK(zp == 0 && threshold == thr);
+        CHECK(std::fabs(scale - s64) <= 1e-6 * s64);
+    }
+    // mixed precision = quantize_with_config per tensor: int8 per-tensor affine for all three default precisions
+    std::map<std::string, Tensor> tensors;
+    tensors.emplace("model.embedding.weight", Tensor::from_data(normal(600, 92, 0.7f), {20, 30}).unwrap());
+    tensors.emplace("block0.attention.q", Tensor::from_data(normal(500, 93, 0.2f), {500}).unwrap());
+    tensors.emplace("head.output", Tensor::from_data(normal(70, 94, 2.0f), {70}).unwrap());
+    const auto results = quantize_mixed_precision(tensors, MixedPrecisionConfig{}).unwrap();
+    for (const auto &[name, tensor] : tensors) {
+        const std::vector<float> &v = tensor.as_slice();
+        std::vector<float> wq(v.size());
+        float ws;
+        int32_t wz;
+        CHECK_EQ(tq_quantize_tensor_auto(v.data(), v.size(), TQ_DTYPE_I8, TQ_PER_TENSOR_AFFINE, wq.data(), &ws, &wz), 0);
+        const QuantizedTriple &r = results.at(name);
+        check_same(std::get<0>(r).as_slice(), wq, __LINE__);
+        CHECK(std::get<1>(r) == ws && std::get<2>(r) == wz);
+    }
+}
+
 GPU_TEST(parity_special_schemes) {
     const std::vector<float> x = normal(24 * 50 * 6, 71, 1.3f);
     const std::vector<size_t> dims{24, 50, 6};

@@ -474,6 +474,68 @@ def test_binary_and_ternary(ctx, hipq, oracle, n):
     assert p.scale == pytest.approx(s64, rel=1e-6) and p.scale == pytest.approx(float(s32), rel=1e-4)
 
 
+@pytest.mark.parametrize("n", [1, 5, 63, 4096, 100003, 1 << 20])
+def test_learned_threshold_binary_and_adaptive_ternary(ctx, hipq, oracle, n):
+    """quantize_binary_learned_threshold (given and learned threshold) and quantize_ternary_adaptive: codes bit for
+    bit and the threshold exactly against the oracle run with f64 sums (the order-free value of the reference's
+    sequential f32 sums, which it must also agree with to their own rounding), scales to 1e-6 of the f64 mean."""
+    x = normal(60 + n, n, 1.1)
+    if n >= 63:
+        x[::9] = 0.0
+        x[1::11] = -0.0
+    d = dev(x)
+    for given in (0.4, -1.0, None):
+        q, params = ctx.quantize_binary_learned_threshold(d, given)
+        want, s32, s64, thr = oracle.quantize_binary_learned_threshold(x, given, f64_sums=True)
+        p = ctx.read_qparams(params)
+        assert p.min_val == thr and p.max_val == 0 and p.zero_point == 0 and p.status == 0
+        np.testing.assert_array_equal(host(q).astype(np.float32), want)
+        assert p.scale == pytest.approx(s64, rel=1e-6)
+        _, s32_ref, _, thr_ref = oracle.quantize_binary_learned_threshold(x, given)  # the reference's f32 sums
+        assert p.min_val == pytest.approx(float(thr_ref), rel=1e-4) and p.scale == pytest.approx(float(s32_ref), rel=1e-3)
+    q, params = ctx.quantize_ternary_adaptive(d)
+    want, s32, s64, thr, e32, e64 = oracle.quantize_ternary_adaptive(x, f64_sums=True)
+    p = ctx.read_qparams(params)
+    assert p.min_val == thr and p.max_val == np.abs(x).max() and p.zero_point == 0
+    np.testing.assert_array_equal(host(q).astype(np.float32), want)
+    assert p.scale == pytest.approx(s64, rel=1e-6)
+    # the reference's own f32 sums pick the same threshold unless two candidates cost the same to f32 rounding
+    order = np.sort(e64)
+    if n == 1 or order[1] - order[0] > 1e-3 * order[0]:
+        assert oracle.quantize_ternary_adaptive(x)[3] == thr
+
+
+def test_learned_threshold_and_adaptive_golden_and_errors(ctx, hipq, cal):
+    for case in cal["special_schemes"]:
+        x = dev(np.float32(case["x"])) if "x" in case and case["fn"] in ("quantize_binary_learned_threshold",
+                                                                          "quantize_ternary_adaptive") else None
+        if case["fn"] == "quantize_binary_learned_threshold":
+            q, params = ctx.quantize_binary_learned_threshold(x, case["threshold"])
+            p = ctx.read_qparams(params)
+            assert p.scale > 0 and p.zero_point == case["zp"] and p.min_val == np.float32(case["threshold_out"])
+            np.testing.assert_array_equal(host(q), case["q"])
+        elif case["fn"] == "quantize_ternary_adaptive":
+            q, params = ctx.quantize_ternary_adaptive(x)
+            p = ctx.read_qparams(params)
+            assert p.scale > 0 and p.zero_point == case["zp"] and p.min_val > 0
+            assert set(host(q).tolist()) <= set(case["values_in"])
+            # by hand: every threshold from 0.3 to 2.7 costs 1.7, the first wins; +-0.5 keep their signs
+            assert p.min_val == np.float32(3) * (np.float32(1) * np.float32(0.1)) and p.scale == 1.75
+            np.testing.assert_array_equal(host(q), [-1, -1, 0, 1, 1])
+    empty = torch.empty(0, device="cuda")
+    with pytest.raises(hipq.HipqError, match="Cannot quantize empty tensor"):
+        ctx.quantize_binary_learned_threshold(empty)
+    with pytest.raises(hipq.HipqError, match="Cannot quantize empty tensor"):
+        ctx.quantize_ternary_adaptive(empty)
+    # unaligned views
+    base = dev(normal(7, 4099, 1.0))
+    for off in (1, 2, 3):
+        v = base[off:]
+        q, params = ctx.quantize_ternary_adaptive(v)
+        q2, params2 = ctx.quantize_ternary_adaptive(v.clone())
+        assert torch.equal(q, q2) and ctx.read_qparams(params).scale == ctx.read_qparams(params2).scale
+
+
 def test_binary_ternary_golden_edges_and_errors(ctx, hipq, oracle, cal):
     for case in cal["special_schemes"]:
         if case["fn"] not in ("quantize_binary", "quantize_ternary"):

@@ -55,6 +55,8 @@ GPU_CASES = [
     "test_quantized_modules_survive_a_weight_file",
     "test_special_schemes",
     "parity_special_schemes",
+    "test_searched_thresholds_and_mixed_precision",
+    "parity_searched_thresholds_and_mixed_precision",
     "parity_backend_qadd_qrelu",
     "test_kernel_plugin_dispatch",
     "test_fake_quantize",

@@ -339,6 +339,13 @@ def test_special_scheme_known_answers(oracle, cal):
             x = np.float32(case["x"])
             q, _, _, s, _ = oracle.quantize_group_wise(x, case["axis"], case["group_size"])
             assert s > 0 and q.shape == x.shape
+        elif fn == "quantize_binary_learned_threshold":
+            q, s, _, thr = oracle.quantize_binary_learned_threshold(case["x"], case["threshold"])
+            assert s > 0 and thr == np.float32(case["threshold_out"])
+            np.testing.assert_array_equal(q, case["q"])
+        elif fn == "quantize_ternary_adaptive":
+            q, s, _, thr, _, _ = oracle.quantize_ternary_adaptive(case["x"])
+            assert s > 0 and thr > 0 and set(q.tolist()) <= set(case["values_in"]) and q.size == len(case["x"])
         else:
             with pytest.raises(oracle.OracleError):
                 oracle.quantize_binary([])
@@ -405,6 +412,63 @@ def test_binary_and_ternary_closed_form(oracle):
     # all zeros: nothing above the threshold, scale 1
     q, s, _, _ = oracle.quantize_ternary(np.zeros(5, np.float32))
     assert s == 1.0 and (q == 0).all()
+
+
+def test_learned_threshold_and_adaptive_ternary_closed_form(oracle):
+    # learned threshold = mean |x| = (2 + 0.1 + 0.1 + 0.5 + 2) / 5 = 0.94: only +-2 keep a sign, scale 2
+    x = np.float32([-2, -0.1, 0.1, 0.5, 2])
+    q, s, s64, thr = oracle.quantize_binary_learned_threshold(x)
+    assert thr == pytest.approx(0.94, rel=1e-6) and s == 2.0 and s64 == 2.0
+    np.testing.assert_array_equal(q, [-1, 0, 0, 0, 1])
+    # given threshold 0.3: scale = (2 + 0.5 + 2) / 3; a value equal to the threshold becomes 0
+    q, s, _, thr = oracle.quantize_binary_learned_threshold(x, 0.3)
+    assert s == np.float32(4.5) / np.float32(3) and thr == np.float32(0.3)
+    q, _, _, _ = oracle.quantize_binary_learned_threshold(np.float32([0.5, -0.5, 0.75]), 0.5)
+    np.testing.assert_array_equal(q, [0, 0, 1])
+    # a negative threshold keeps every element, and zero (of either sign) then counts as positive: x >= 0
+    q, s, _, _ = oracle.quantize_binary_learned_threshold(np.float32([0.0, -0.0, -1.0]), -1.0)
+    np.testing.assert_array_equal(q, [1, 1, -1])
+    assert s == np.float32(1.0) / np.float32(3)
+    # nothing above the threshold: scale 1
+    q, s, _, _ = oracle.quantize_binary_learned_threshold(np.float32([0.1, -0.2]), 5.0)
+    assert s == 1.0 and (q == 0).all()
+    # adaptive, by hand for [-3, -0.5, 0, 0.5, 3]: thresholds 0.3 .. 2.7 all cost (4 + .25 + 0 + .25 + 4) / 5 = 1.7
+    # (0.5 costs 0.25 kept or dropped), threshold 3.0 costs 18.5 / 5; the first minimum wins: 3 * 0.1
+    q, s, _, thr, e32, e64 = oracle.quantize_ternary_adaptive(np.float32([-3, -0.5, 0, 0.5, 3]))
+    np.testing.assert_allclose(e32, [1.7] * 9 + [3.7], rtol=1e-6)
+    np.testing.assert_allclose(e64, [1.7] * 9 + [3.7], rtol=1e-12)
+    assert thr == np.float32(3) * (np.float32(1) * np.float32(0.1))
+    np.testing.assert_array_equal(q, [-1, -1, 0, 1, 1])
+    assert s == np.float32(7.0) / np.float32(4)
+    # values near 1 with small noise: a high threshold that zeroes the noise and keeps the ones wins
+    x = np.float32([1.0, -1.0, 0.05, -0.05, 1.0, 0.02])
+    q, s, _, thr, e32, _ = oracle.quantize_ternary_adaptive(x)
+    np.testing.assert_array_equal(q, [1, -1, 0, 0, 1, 0])
+    assert thr == np.float32(1) * (np.float32(1) * np.float32(0.1)) and s == 1.0
+    assert int(np.argmin(e32)) == 0 and e32[9] > e32[0]            # threshold 1.0 drops the ones as well
+    # zero (and -0.0) is never given a sign by the adaptive form (x > 0), whatever the threshold
+    q, _, _, _, _, _ = oracle.quantize_ternary_adaptive(np.float32([0.0, -0.0, 2.0]))
+    np.testing.assert_array_equal(q[:2], [0, 0])
+    # brute force of the search in float64 on random data: same winner wherever the margin is clear
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal(2000) * 1.3).astype(np.float32)
+    q, s, s64, thr, e32, e64 = oracle.quantize_ternary_adaptive(x)
+    mx = np.abs(x).max()
+    errs = []
+    for i in range(1, 11):
+        t = mx * (np.float32(i) * np.float32(0.1))
+        code = np.where(np.abs(x) <= t, 0.0, np.sign(x)).astype(np.float64)
+        errs.append(((x.astype(np.float64) - code) ** 2).mean())
+    np.testing.assert_allclose(e64, errs, rtol=1e-6)
+    np.testing.assert_allclose(e32, errs, rtol=1e-4)
+    best = int(np.argmin(errs))
+    assert thr == mx * (np.float32(best + 1) * np.float32(0.1))
+    keep = np.abs(x) > thr
+    assert s64 == pytest.approx(np.abs(x[keep]).astype(np.float64).mean(), rel=1e-12)
+    np.testing.assert_array_equal(q, np.where(keep, np.sign(x), 0.0))
+    for fn in (oracle.quantize_binary_learned_threshold, oracle.quantize_ternary_adaptive):
+        with pytest.raises(oracle.OracleError):
+            fn([])
 
 
 def test_group_wise_equals_grouped_slices(oracle):

@@ -96,6 +96,8 @@ _SIGNATURES = {
     "hipq_quantize_per_group_auto_f32_i8": [_vp, _vp, _sz, _sz, _sz, _sz, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "hipq_quantize_binary_f32_i8": [_vp, _vp, _sz, _vp, _vp],
     "hipq_quantize_ternary_f32_i8": [_vp, _vp, _sz, _vp, _vp],
+    "hipq_quantize_binary_learned_threshold_f32_i8": [_vp, _vp, _sz, _i32, _f32, _vp, _vp],
+    "hipq_quantize_ternary_adaptive_f32_i8": [_vp, _vp, _sz, _vp, _vp],
     "hipq_quantize_per_channel_f32_i8": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _i32, _vp],
     "hipq_dequantize_per_channel_i8_f32": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp],
     "hipq_gemm_i8_i32": [_vp, _vp, _vp, _sz, _sz, _sz, _vp],
@@ -391,6 +393,20 @@ class Context:
         out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
         params = self.new_qparams()
         self.call("hipq_quantize_ternary_f32_i8", _ptr(x), x.numel(), _ptr(out), _ptr(params))
+        return out, params
+
+    def quantize_binary_learned_threshold(self, x, threshold=None):
+        """Codes in {-1, 0, 1}; params.min_val holds the threshold used (mean |x| when none is given)."""
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        params = self.new_qparams()
+        self.call("hipq_quantize_binary_learned_threshold_f32_i8", _ptr(x), x.numel(), int(threshold is not None),
+                  float(threshold or 0.0), _ptr(out), _ptr(params))
+        return out, params
+
+    def quantize_ternary_adaptive(self, x):
+        out = torch.empty(x.shape, dtype=torch.int8, device=self._dev())
+        params = self.new_qparams()
+        self.call("hipq_quantize_ternary_adaptive_f32_i8", _ptr(x), x.numel(), _ptr(out), _ptr(params))
         return out, params
 
     def quantize_per_channel_auto(self, x, axis, flavor=PARAMS_SYMMETRIC, mode=0):

@@ -52,6 +52,7 @@ inline uint32_t dtype_bits(DType d) {  // metrics.rs:203-216
     switch (d) {
     case DType::F32:
     case DType::I32: return 32;
+    case DType::F16:
     case DType::I16: return 16;
     default: return 8;
     }

@@ -26,7 +26,7 @@
 
 namespace torsh {
 
-enum class DType { F32, I8, U8, I16, I32 };
+enum class DType { F32, I8, U8, I16, I32, F16 };  // F16 only names a precision (mixed-precision configs)
 
 struct TorshError {
     enum Kind { InvalidArgument, ShapeError, DimensionMismatch, BackendError, AllocationError, NotImplemented };

@@ -42,6 +42,7 @@ inline const char *name_of(DType d) {
     case DType::I8: return "I8";
     case DType::U8: return "U8";
     case DType::I16: return "I16";
+    case DType::F16: return "F16";
     default: return "I32";
     }
 }
@@ -189,6 +190,7 @@ inline Result<QuantConfig> import_config_from_json(const std::string &json) {
     else if (dt == "U8") c.dtype = DType::U8;
     else if (dt == "I16") c.dtype = DType::I16;
     else if (dt == "I32") c.dtype = DType::I32;
+    else if (dt == "F16") c.dtype = DType::F16;
     else return bad("unknown variant `" + dt + "` for dtype");
     if (!detail::parse_enum(detail::FlatJson::unquote(m.at("scheme")), 10, &c.scheme)) return bad("unknown scheme");
     if (!detail::parse_enum(detail::FlatJson::unquote(m.at("observer_type")), 6, &c.observer_type))

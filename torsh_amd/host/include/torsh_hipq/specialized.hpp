@@ -6,6 +6,10 @@
 //   quantize_binary              specialized.rs:163-188
 //   quantize_ternary             specialized.rs:191-238
 //   quantize_group_wise          specialized.rs:241-377
+//   quantize_mixed_precision, determine_layer_precision, create_precision_config
+//                                specialized.rs:379-436 (MixedPrecisionConfig: config.rs:131-154)
+//   quantize_binary_learned_threshold, quantize_ternary_adaptive
+//                                specialized.rs:439-552
 //
 // Values come back in the f32 carrier like the reference's.  Two documented differences, both
 // only for non-finite inputs: a NaN element quantizes to clamp(0) (the int8 conversion used by the
@@ -13,6 +17,10 @@
 // is not finite is InvalidArgument.  The scale of the binary and ternary schemes is the mean of
 // |x| formed from f64 partial sums; the reference adds f32 terms in element order.
 #pragma once
+
+#include <map>
+#include <optional>
+#include <string>
 
 #include "quantization.hpp"
 
@@ -120,6 +128,77 @@ inline Result<QuantizedTriple> quantize_binary(const Tensor &tensor) { return de
 // specialized.rs:191-238
 inline Result<QuantizedTriple> quantize_ternary(const Tensor &tensor) { return detail::sign_scheme(tensor, true); }
 
+// (tensor, scale, zero_point, threshold)
+using ThresholdQuadruple = std::tuple<Tensor, float, int32_t, float>;
+
+namespace detail {
+inline Result<ThresholdQuadruple> searched_sign_scheme(const Tensor &tensor, bool adaptive,
+                                                       std::optional<float> threshold) {
+    const std::vector<float> &data = tensor.as_slice();
+    if (data.empty()) return TorshError::invalid_argument("Cannot quantize empty tensor");
+    TORSH_TRY(ctx, hip::Runtime::ctx());
+    TORSH_TRY(dx, hip::DeviceBuffer::from_host(ctx, data.data(), data.size()));
+    TORSH_TRY(dq, hip::DeviceBuffer::alloc(ctx, data.size()));
+    TORSH_TRY(dp, hip::DeviceBuffer::alloc(ctx, sizeof(hipq_qparams)));
+    TORSH_CHECK(hip::check(
+        adaptive ? hipq_quantize_ternary_adaptive_f32_i8(ctx, dx.as<float>(), data.size(), dq.as<int8_t>(),
+                                                         dp.as<hipq_qparams>())
+                 : hipq_quantize_binary_learned_threshold_f32_i8(ctx, dx.as<float>(), data.size(),
+                                                                 threshold.has_value() ? 1 : 0, threshold.value_or(0.0f),
+                                                                 dq.as<int8_t>(), dp.as<hipq_qparams>())));
+    TORSH_TRY(q, dq.to_host<int8_t>(data.size()));
+    TORSH_TRY(p, dp.to_host<hipq_qparams>(1));
+    TORSH_TRY(t, carrier_tensor(q, tensor.shape().dims()));
+    return ThresholdQuadruple{std::move(t), p[0].scale, 0, p[0].min_val};
+}
+}  // namespace detail
+
+// specialized.rs:439-492: the threshold is the given one or mean |x|; |x| <= threshold -> 0, else the
+// sign with x >= 0 counted as positive; scale = mean |x| of the values above the threshold.
+inline Result<ThresholdQuadruple> quantize_binary_learned_threshold(const Tensor &tensor,
+                                                                    std::optional<float> threshold = std::nullopt) {
+    return detail::searched_sign_scheme(tensor, false, threshold);
+}
+
+// specialized.rs:495-552: the first of the ten thresholds max|x| * (i * 0.1) with the least mean
+// squared error of the unit ternary code.
+inline Result<ThresholdQuadruple> quantize_ternary_adaptive(const Tensor &tensor) {
+    return detail::searched_sign_scheme(tensor, true, std::nullopt);
+}
+
+// config.rs:131-154
+struct MixedPrecisionConfig {
+    std::map<std::string, DType> layer_precision{{"embedding", DType::I8}, {"attention", DType::F16},
+                                                 {"output", DType::F32}};
+    DType default_precision = DType::I8;
+    float sensitivity_threshold = 0.1f;
+};
+
+// specialized.rs:401-412: the first pattern contained in the layer name decides.  (The reference walks
+// a HashMap, so which of several matching patterns wins is unspecified there; here it is the
+// alphabetically first.)
+inline DType determine_layer_precision(const std::string &layer_name, const MixedPrecisionConfig &config) {
+    for (const auto &[pattern, precision] : config.layer_precision)
+        if (layer_name.find(pattern) != std::string::npos) return precision;
+    return config.default_precision;
+}
+
+// specialized.rs:414-436
+inline QuantConfig create_precision_config(DType precision) {
+    switch (precision) {
+    case DType::I8: return QuantConfig::int8();
+    case DType::U8: return QuantConfig::uint8();
+    case DType::F16:
+    case DType::F32: {
+        QuantConfig c;
+        c.dtype = precision;
+        c.enable_fake_quant = false;
+        return c;
+    }
+    default: return QuantConfig::int8();
+    }
+}
+
 // specialized.rs:241-377: groups of `group_size` consecutive channels along `axis` share one
 // (scale, zero point), the last group may be shorter; integer range from config.get_qint_range().
 inline Result<QuantizedTriple> quantize_group_wise(const Tensor &tensor, size_t axis, size_t group_size,
@@ -148,6 +227,20 @@ inline Result<QuantizedTriple> quantize_group_wise(const Tensor &tensor, size_t 
     const auto avg = detail::average_params(scales, zps);
     TORSH_TRY(t, detail::carrier_tensor(q, shape));
     return QuantizedTriple{std::move(t), avg.first, avg.second};
+}
+
+// specialized.rs:379-399: every tensor through quantize_with_config with the configuration of the
+// precision its layer name selects.  As in the reference, the F16 / F32 configurations still carry
+// the default per-tensor affine scheme, whose integer range falls back to int8 (algorithms.rs:425-433).
+inline Result<std::map<std::string, QuantizedTriple>> quantize_mixed_precision(
+    const std::map<std::string, Tensor> &tensors, const MixedPrecisionConfig &config) {
+    std::map<std::string, QuantizedTriple> results;
+    for (const auto &[layer_name, tensor] : tensors) {
+        const QuantConfig layer_config = create_precision_config(determine_layer_precision(layer_name, config));
+        TORSH_TRY(r, quantize_with_config(tensor, layer_config));
+        results.emplace(layer_name, std::move(r));
+    }
+    return results;
 }
 
 }  // namespace quantization
