@@ -862,6 +862,40 @@ GPU_TEST(test_compare_quantization_configs) {  // metrics.rs:623-661
     CHECK(with_bad.back().metrics.psnr < 0 && with_bad.back().metrics.zero_error_percentage == 0.0f);
 }
 
+GPU_TEST(test_auto_calibrate_quantization) {  // metrics.rs:663-686
+    const Tensor t1 = tensor_1d({1.0f, 2.0f, 3.0f, 4.0f}).unwrap(), t2 = tensor_1d({2.0f, 3.0f, 4.0f, 5.0f}).unwrap(),
+                 t3 = tensor_1d({0.5f, 1.5f, 2.5f, 3.5f}).unwrap();
+    const std::vector<const Tensor *> calibration{&t1, &t2, &t3};
+    const auto result = auto_calibrate_quantization(calibration, 20.0f, 10.0f);
+    CHECK(result.is_ok());
+    CHECK(result.unwrap().validate().is_ok());
+    CHECK(auto_calibrate_quantization(calibration, 100.0f, 1.1f).is_ok());  // impossible thresholds still yield a config
+    const auto none = auto_calibrate_quantization({}, 20.0f, 10.0f);
+    CHECK(none.is_err());
+    CHECK_EQ(none.unwrap_err().message, std::string("No calibration tensors provided"));
+    // the score rule, recomputed from compare_quantization_configs on one tensor: every candidate has
+    // compression ratio 4 (int8 carrier), so with both thresholds met the highest PSNR wins
+    const Tensor big = Tensor::from_data(normal(64 * 32, 97, 1.0f), {64, 32}).unwrap();
+    const QuantConfig chosen = auto_calibrate_quantization({&big}, 10.0f, 10.0f).unwrap();
+    const std::vector<QuantConfig> candidates{
+        QuantConfig::int8(),           QuantConfig::int8().with_observer(ObserverType::Histogram),
+        QuantConfig::per_channel(0),   QuantConfig::per_channel(1),
+        QuantConfig::group_wise(0, 8), QuantConfig::group_wise(1, 16),
+        QuantConfig::int4(),           QuantConfig::ternary()};
+    float best = -INFINITY;
+    size_t best_i = 0;
+    for (size_t i = 0; i < candidates.size(); ++i) {
+        const auto cmp = compare_quantization_configs(big, {candidates[i]}).unwrap();
+        const QuantizationMetrics &m = cmp.front().metrics;
+        if (!std::isfinite(m.psnr)) continue;
+        const float score = (m.psnr >= 10.0f && m.compression_ratio <= 10.0f) ? m.compression_ratio + m.psnr / 100.0f
+                                                                              : m.psnr / m.compression_ratio;
+        if (score > best) best = score, best_i = i;
+    }
+    CHECK(chosen.scheme == candidates[best_i].scheme && chosen.observer_type == candidates[best_i].observer_type);
+    CHECK(chosen.ch_axis == candidates[best_i].ch_axis && chosen.group_size == candidates[best_i].group_size);
+}
+
 GPU_TEST(parity_metrics_and_compare_configs) {
     const std::vector<float> x = normal(200003, 31, 1.7f);
     const Tensor tx = tensor_1d(x).unwrap();

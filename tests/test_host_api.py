@@ -45,6 +45,7 @@ GPU_CASES = [
     "parity_quantized_conv2d_module",
     "test_calculate_quantization_metrics",
     "test_compare_quantization_configs",
+    "test_auto_calibrate_quantization",
     "parity_metrics_and_compare_configs",
     "test_observers",
     "parity_observers_against_the_oracle",

@@ -7,6 +7,7 @@
 //
 //   QuantizationMetrics, calculate_quantization_metrics   crates/torsh-quantization/src/metrics.rs:30-175
 //   compare_quantization_configs                          metrics.rs:178-260
+//   auto_calibrate_quantization                           metrics.rs:252-338
 //   Observer                                              crates/torsh-quantization/src/observers.rs:36-556
 //   quantize_batch_consistent                             crates/torsh-quantization/src/utils.rs:153-180
 #pragma once
@@ -135,6 +136,51 @@ inline Result<std::vector<ConfigComparison>> compare_quantization_configs(const 
         return b.metrics.psnr < a.metrics.psnr;
     });
     return results;
+}
+
+// metrics.rs:252-338: the eight candidate configurations, each scored by its metrics averaged over the
+// calibration tensors; a candidate that meets both thresholds is ranked by compression, the others by
+// PSNR per unit of compression; the first best wins.
+inline Result<QuantConfig> auto_calibrate_quantization(const std::vector<const Tensor *> &calibration_tensors,
+                                                       float target_accuracy_threshold, float max_compression_ratio) {
+    if (calibration_tensors.empty()) return TorshError::invalid_argument("No calibration tensors provided");
+    const std::vector<QuantConfig> candidates{
+        QuantConfig::int8(),           QuantConfig::int8().with_observer(ObserverType::Histogram),
+        QuantConfig::per_channel(0),   QuantConfig::per_channel(1),
+        QuantConfig::group_wise(0, 8), QuantConfig::group_wise(1, 16),
+        QuantConfig::int4(),           QuantConfig::ternary()};
+    bool found = false;
+    QuantConfig best_config;
+    float best_score = -std::numeric_limits<float>::infinity();
+    for (const QuantConfig &config : candidates) {
+        QuantizationMetrics total;  // QuantizationMetrics::default(): zero_error 100, cosine 1, ratio 1 (metrics.rs:50-63)
+        int successful_tests = 0;
+        for (const Tensor *tensor : calibration_tensors) {
+            auto comparison = compare_quantization_configs(*tensor, {config});
+            if (comparison.is_err() || comparison.unwrap().empty()) continue;
+            const QuantizationMetrics &m = comparison.unwrap().front().metrics;
+            if (!std::isfinite(m.psnr)) continue;
+            total.mse += m.mse, total.psnr += m.psnr, total.snr += m.snr, total.mae += m.mae;
+            total.max_error = std::fmax(total.max_error, m.max_error);
+            total.zero_error_percentage += m.zero_error_percentage;
+            total.cosine_similarity += m.cosine_similarity;
+            total.compression_ratio += m.compression_ratio;
+            ++successful_tests;
+        }
+        if (successful_tests == 0) continue;
+        const float n = static_cast<float>(successful_tests);
+        const float psnr = total.psnr / n, ratio = total.compression_ratio / n;
+        const float score = (psnr >= target_accuracy_threshold && ratio <= max_compression_ratio)
+                                ? ratio + psnr / 100.0f
+                                : psnr / ratio;
+        if (score > best_score) {
+            best_score = score;
+            best_config = config;
+            found = true;
+        }
+    }
+    if (!found) return TorshError::invalid_argument("No suitable configuration found");
+    return best_config;
 }
 
 // observers.rs:36-556

@@ -126,6 +126,11 @@ struct QuantConfig {
         if (s == QScheme::GroupWise && !c.group_size) c.group_size = 32;
         return c;
     }
+    QuantConfig with_observer(ObserverType o) const {  // config.rs:264-267
+        QuantConfig c = *this;
+        c.observer_type = o;
+        return c;
+    }
     QuantConfig with_reduce_range(ReduceRange r) const {
         QuantConfig c = *this;
         c.reduce_range = r;
