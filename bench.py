@@ -139,6 +139,24 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
             ctx.histogram(xs[i % 8], -6.0, 6.0, 256, counts=hist)
         for i in range(reps):
             ctx.fake_quantize(xs[i % 8], 0.04, 0, out=ys[i % 8])
+    elif which == "special":
+        # tensor statistics and the sign schemes (binary, ternary, learned threshold, adaptive ternary)
+        n = 4096 * 4096
+        xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
+        rec = ctx._record(hipq.TensorStats)
+        torch.cuda.synchronize()
+        for i in range(reps):
+            ctx.tensor_stats(xs[i % 8], one_pass=True, out=rec)
+        for i in range(reps):
+            ctx.tensor_stats(xs[i % 8], out=rec)
+        for i in range(reps):
+            ctx.quantize_binary(xs[i % 8])
+        for i in range(reps):
+            ctx.quantize_ternary(xs[i % 8])
+        for i in range(reps):
+            ctx.quantize_binary_learned_threshold(xs[i % 8])
+        for i in range(reps):
+            ctx.quantize_ternary_adaptive(xs[i % 8])
     elif which == "stack":
         # configs[4]: three forwards of the 12-layer int8 projection stack (8192 tokens, d 768, d_ff 3072)
         tokens, d, dff, layers = 8192, 768, 3072, 12
@@ -179,7 +197,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "quantize", "calib", "copy", "stack"], default=None,
+    ap.add_argument("--profile", choices=["gemm", "quantize", "calib", "special", "copy", "stack"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
     if args.gpus != 1:

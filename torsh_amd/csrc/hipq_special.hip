@@ -245,22 +245,33 @@ __global__ __launch_bounds__(kCalBlock) void ternary_search_kernel(const float *
 }
 
 // First threshold with the strictly smallest mean error, in candidate order (specialized.rs:510-517).
-__global__ __launch_bounds__(kWave) void ternary_search_final_kernel(const SearchPartial *__restrict__ partials,
-                                                                      int nparts, size_t n,
-                                                                      float *__restrict__ out_threshold) {
-    __shared__ float mean_err[kTernaryCandidates];
-    if (threadIdx.x < kTernaryCandidates) {
-        double r = 0.0;
-        for (int p = 0; p < nparts; ++p) r += partials[p].err[threadIdx.x];
-        mean_err[threadIdx.x] = static_cast<float>(r / static_cast<double>(n));
+__global__ __launch_bounds__(kCalBlock) void ternary_search_final_kernel(const SearchPartial *__restrict__ partials,
+                                                                          int nparts, size_t n,
+                                                                          float *__restrict__ out_threshold) {
+    double err[kTernaryCandidates];
+#pragma unroll
+    for (int i = 0; i < kTernaryCandidates; ++i) err[i] = 0.0;
+    for (int p = threadIdx.x; p < nparts; p += kCalBlock) {
+#pragma unroll
+        for (int i = 0; i < kTernaryCandidates; ++i) err[i] += partials[p].err[i];
+    }
+    __shared__ SearchPartial lds[kCalBlock / kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+#pragma unroll
+    for (int i = 0; i < kTernaryCandidates; ++i) {
+        const double w = wave_sum(err[i]);
+        if (lane == 0) lds[wave].err[i] = w;
     }
     __syncthreads();
     if (threadIdx.x != 0) return;
     const float max_abs = out_threshold[1];
     float best_threshold = 0.0f, best_error = INFINITY;
     for (int i = 0; i < kTernaryCandidates; ++i) {
-        if (mean_err[i] < best_error) {
-            best_error = mean_err[i];
+        double r = lds[0].err[i];
+        for (int w = 1; w < kCalBlock / kWave; ++w) r += lds[w].err[i];
+        const float mean_err = static_cast<float>(r / static_cast<double>(n));
+        if (mean_err < best_error) {
+            best_error = mean_err;
             best_threshold = ternary_candidate(max_abs, i + 1);
         }
     }
@@ -315,7 +326,7 @@ static int32_t sign_quantize_searched(const char *fn, hipq_ctx *ctx, const float
     if (adaptive) {
         absmax_partial_kernel<<<grid, kCalBlock, 0, ctx->stream>>>(x, n, absmax_partials);
         ternary_search_kernel<<<grid, kCalBlock, 0, ctx->stream>>>(x, n, absmax_partials, grid, search, threshold);
-        ternary_search_final_kernel<<<1, kWave, 0, ctx->stream>>>(search, grid, n, threshold);
+        ternary_search_final_kernel<<<1, kCalBlock, 0, ctx->stream>>>(search, grid, n, threshold);
         if ((rc = check_launch("ternary_search")) != HIPQ_SUCCESS) return rc;
         sign_quantize_kernel<SIGN_GIVEN_GT><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, nullptr, 0, out, partials,
                                                                                    threshold, 0, 0.0f);
