@@ -283,7 +283,7 @@ static int32_t sign_quantize(const char *fn, hipq_ctx *ctx, const float *x, size
     if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", fn);
     if (!x || !out || !out_params) return fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer", fn);
     const size_t tiles = (n + size_t(kCalTile) * 4 - 1) / (size_t(kCalTile) * 4);
-    const size_t cap = static_cast<size_t>(ctx->num_cus) * 2;
+    const size_t cap = static_cast<size_t>(ctx->num_cus) * 4;
     const int grid = static_cast<int>(tiles < cap ? tiles : cap);
     void *scr = nullptr;
     // header: threshold and max|x| (2 floats); then absmax partials; then sign partials
@@ -313,7 +313,7 @@ static int32_t sign_quantize_searched(const char *fn, hipq_ctx *ctx, const float
     if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", fn);
     if (!x || !out || !out_params) return fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer", fn);
     const size_t tiles = (n + size_t(kCalTile) * 4 - 1) / (size_t(kCalTile) * 4);
-    const size_t cap = static_cast<size_t>(ctx->num_cus) * 2;
+    const size_t cap = static_cast<size_t>(ctx->num_cus) * 4;
     const int grid = static_cast<int>(tiles < cap ? tiles : cap);
     void *scr = nullptr;
     int32_t rc = scratch(ctx, kScratchHeader + cap * (sizeof(float) + sizeof(SignPartial) + sizeof(SearchPartial)) + 64,
