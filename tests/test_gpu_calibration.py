@@ -312,6 +312,28 @@ def test_more_than_two_to_the_32_elements(ctx, hipq, oracle):
     x[(1 << 32) + 100:(1 << 32) + 102] = bad
     st = ctx.read_observe(ctx.observe(x))
     assert (st.min_val, st.max_val, st.nonfinite) == (-60.0, 50.0, 0)
+    # tensor statistics: range from beyond 2^32, moments = the block's plus the two planted values
+    b64 = base.astype(np.float64)
+    pos = [(n - 3) % period, ((1 << 32) + 9) % period]
+    total = b64.sum() * reps - b64[pos].sum() + (50.0 - 60.0)
+    total_sq = (b64 * b64).sum() * reps - (b64[pos] ** 2).sum() + (50.0 ** 2 + 60.0 ** 2)
+    mean = total / n
+    for one_pass in (False, True):
+        ts = ctx.tensor_stats(x, one_pass=one_pass)
+        assert (ts.min_val, ts.max_val) == (-60.0, 50.0)
+        assert ts.mean == pytest.approx(mean, rel=1e-5, abs=1e-7)
+        assert ts.variance == pytest.approx(total_sq / n - mean * mean, rel=1e-5)
+    # adaptive ternary: the codes must follow the threshold the search chose, everywhere
+    qa, params = ctx.quantize_ternary_adaptive(x)
+    p = ctx.read_qparams(params)
+    assert p.max_val == 60.0 and 0 < p.min_val <= 60.0
+    want_codes = torch.where(x.abs() <= p.min_val, torch.zeros_like(x), torch.sign(x)).to(torch.int8)
+    torch.cuda.synchronize()
+    assert torch.equal(qa, want_codes)
+    kept = x.abs() > p.min_val
+    kept_sum = torch.where(kept, x.abs(), torch.zeros_like(x)).sum(dtype=torch.float64)
+    assert p.scale == pytest.approx(float(kept_sum) / int(kept.sum()), rel=1e-6)
+    del qa, want_codes, kept
     # histogram: block counts x repetitions; the two planted values move from their old bins to the end bins
     lo, hi, bins = -6.0, 6.0, 256
     block_counts = oracle.histogram_accumulate(base, lo, hi, bins).astype(np.int64)
