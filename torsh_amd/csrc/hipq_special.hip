@@ -117,6 +117,7 @@ __global__ __launch_bounds__(kCalBlock) void sign_quantize_kernel(const float *_
             sum4 = 0.0f;
             const int a = code(v.x), b = code(v.y), c = code(v.z), d = code(v.w);
             sum += sum4;
+            if (!out) return;  // sums only
             if (out_aligned) {
                 store_stream(reinterpret_cast<uint32_t *>(out) + idx, pack4(a, b, c, d));
             } else {
@@ -127,7 +128,8 @@ __global__ __launch_bounds__(kCalBlock) void sign_quantize_kernel(const float *_
         },
         [&](float v, size_t i) {
             sum4 = 0.0f;
-            out[i] = static_cast<int8_t>(code(v));
+            const int c = code(v);
+            if (out) out[i] = static_cast<int8_t>(c);
             sum += sum4;
         });
     block_store_sign_partial(sum, count, partials + blockIdx.x);
@@ -332,8 +334,8 @@ static int32_t sign_quantize_searched(const char *fn, hipq_ctx *ctx, const float
                                                                                    threshold, 0, 0.0f);
     } else {
         if (!has_threshold) {
-            // the codes of this pass are overwritten below; its sums give mean |x|
-            sign_quantize_kernel<SIGN_BINARY><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, nullptr, 0, out, partials,
+            // a pass for its sums only (no codes written): mean |x|
+            sign_quantize_kernel<SIGN_BINARY><<<grid, kCalBlock, 0, ctx->stream>>>(x, n, nullptr, 0, nullptr, partials,
                                                                                      threshold, 0, 0.0f);
             mean_abs_threshold_kernel<<<1, kCalBlock, 0, ctx->stream>>>(partials, grid, n, threshold);
             if ((rc = check_launch("mean_abs_threshold_kernel")) != HIPQ_SUCCESS) return rc;
