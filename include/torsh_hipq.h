@@ -305,6 +305,17 @@ HIPQ_API int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_s
 HIPQ_API int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w,
                                          const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
                                          int32_t mode, float *out);
+/* hipq_linear_dynamic_f32 for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, same kernels, same results; the int8 activations, their scales and the range
+ * partials go to a static device array of the library (about 4.3 MiB per GPU, held until the
+ * process ends) instead of the context's growable scratch, and the call performs no hipMalloc /
+ * hipFree.  Limits: m <= 16384 rows and m * k <= 4 Mi elements, else HIPQ_SHAPE_ERROR.  Every call
+ * on one GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * contexts) race; calls on one stream are ordered and safe. */
+HIPQ_API int32_t hipq_linear_dynamic_f32_noalloc(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w,
+                                                 const float *w_scales, const float *bias, size_t m, size_t n,
+                                                 size_t k, int32_t mode, float *out);
 
 
 /* ---- quantized Conv2d forward (NCHW, filters [OC,IC,KH,KW]) ------------ */

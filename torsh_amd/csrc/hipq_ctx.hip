@@ -101,7 +101,8 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
         ctx->stream = stream;
     }
     void *p = nullptr;
-    int32_t rc = hipq::scratch(ctx, size_t(8) << 20, &p);
+    int32_t rc = hipq::linear_noalloc_setup(device);
+    if (rc == HIPQ_SUCCESS) rc = hipq::scratch(ctx, size_t(8) << 20, &p);
     if (rc != HIPQ_SUCCESS) {
         if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
         delete ctx;

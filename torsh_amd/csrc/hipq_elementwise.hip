@@ -512,12 +512,18 @@ static int32_t launch_minmax(hipq_ctx *ctx, const float *x, size_t n, float *out
 }
 
 // First stage only; the quantize kernel that follows folds the partials itself.
-static int32_t launch_minmax_partials(hipq_ctx *ctx, const float *x, size_t n, DynamicRange *dyn) {
-    const int grid = grid_for_minmax(ctx, n);
-    void *s = nullptr;
-    int32_t rc = scratch(ctx, kScratchHeader + size_t(grid) * sizeof(float2), &s);
-    if (rc != HIPQ_SUCCESS) return rc;
-    float2 *partials = reinterpret_cast<float2 *>(static_cast<char *>(s) + kScratchHeader);
+static int32_t launch_minmax_partials(hipq_ctx *ctx, const float *x, size_t n, DynamicRange *dyn,
+                                      float2 *partials = nullptr, size_t partials_cap = 0) {
+    int grid = grid_for_minmax(ctx, n);
+    if (partials) {
+        // Caller-provided room for the partials (the entry point that must not allocate).
+        if (size_t(grid) > partials_cap) grid = static_cast<int>(partials_cap);
+    } else {
+        void *s = nullptr;
+        int32_t rc = scratch(ctx, kScratchHeader + size_t(grid) * sizeof(float2), &s);
+        if (rc != HIPQ_SUCCESS) return rc;
+        partials = reinterpret_cast<float2 *>(static_cast<char *>(s) + kScratchHeader);
+    }
     hipLaunchKernelGGL(minmax_partial_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, partials);
     dyn->partials = partials;
     dyn->nparts = grid;
@@ -699,20 +705,29 @@ int32_t hipq_quantize_with_params_f32_u8(hipq_ctx *ctx, const float *x, size_t n
 
 int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor, int32_t dtype,
                                              int32_t mode, void *out, hipq_qparams *out_params) {
+    return hipq::quantize_dynamic_per_tensor(ctx, x, n, flavor, dtype, mode, out, out_params, nullptr, 0);
+}
+
+}  // extern "C"
+
+int32_t hipq::quantize_dynamic_per_tensor(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor, int32_t dtype,
+                                          int32_t mode, void *out, hipq_qparams *out_params, void *partials,
+                                          size_t partials_cap) {
+    const char *fn = "hipq_quantize_dynamic_per_tensor_f32";
     HIPQ_ENTER(ctx);
-    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    if (n == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", fn);
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
     HIPQ_REQUIRE_PTR(out_params);
-    int32_t rc = check_mode(__func__, mode);
+    int32_t rc = check_mode(fn, mode);
     if (rc) return rc;
     if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
-        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", __func__, flavor);
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", fn, flavor);
     if (dtype != HIPQ_DTYPE_I8 && dtype != HIPQ_DTYPE_U8)
-        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", __func__, dtype);
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", fn, dtype);
     const int qmin = dtype == HIPQ_DTYPE_I8 ? -128 : 0, qmax = dtype == HIPQ_DTYPE_I8 ? 127 : 255;
     DynamicRange dyn{nullptr, 0, flavor, qmin, qmax, out_params};
-    rc = launch_minmax_partials(ctx, x, n, &dyn);
+    rc = launch_minmax_partials(ctx, x, n, &dyn, static_cast<float2 *>(partials), partials_cap / sizeof(float2));
     if (rc) return rc;
     if (dtype == HIPQ_DTYPE_I8)
         return launch_quantize<int8_t>(ctx, x, n, 1.0f, 0, nullptr, mode, -128.0f, 127.0f,
@@ -720,6 +735,8 @@ int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size
     return launch_quantize<uint8_t>(ctx, x, n, 1.0f, 0, nullptr, mode, 0.0f, 255.0f, static_cast<uint8_t *>(out),
                                     dyn);
 }
+
+extern "C" {
 
 int32_t hipq_dequantize_i8_f32(hipq_ctx *ctx, const int8_t *q, size_t n, float scale, int32_t zero_point, float *out) {
     HIPQ_ENTER(ctx);

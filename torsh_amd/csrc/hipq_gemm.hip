@@ -8,6 +8,8 @@
 // that each lane ends up with four consecutive output channels of one
 // activation row: 16-byte stores, 16-byte loads of the per-channel scales.
 
+#include <mutex>
+
 #include "hipq_gemm_kernels.h"
 #include "hipq_gemm_persist.h"
 
@@ -370,6 +372,73 @@ static int32_t check_gemm_shape(const char *fn, size_t m, size_t n, size_t k) {
     return HIPQ_SUCCESS;
 }
 
+static int32_t check_linear_dynamic_args(const char *fn, const float *x, const int8_t *w, const float *w_scales,
+                                         size_t m, size_t n, size_t k, float *out) {
+    int32_t rc = check_gemm_shape(fn, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", fn);
+    if (!x || !w || !w_scales || !out) return fail(HIPQ_INVALID_ARGUMENT, "%s: null pointer", fn);
+    return HIPQ_SUCCESS;
+}
+
+// Scratch layout of the fused dynamic Linear: header (hipq_qparams), the range-reduction partials,
+// per-row scales [m] floats, then the int8 activations [m,k].
+static size_t linear_dynamic_partial_bytes(int num_cus) { return size_t(num_cus) * 16 * sizeof(float2); }
+static size_t linear_dynamic_scales_bytes(size_t m) { return ((m * sizeof(float)) + 255) & ~size_t(255); }
+static size_t linear_dynamic_scratch_bytes(int num_cus, size_t m, size_t k) {
+    return kScratchHeader + linear_dynamic_partial_bytes(num_cus) + linear_dynamic_scales_bytes(m) + m * k + 256;
+}
+
+// The fused dynamic Linear on a scratch area of linear_dynamic_scratch_bytes() at `base`.  Launches
+// kernels only: no allocation, no synchronisation.
+static int32_t linear_dynamic_on(hipq_ctx *ctx, char *base, const float *x, int32_t per_token, const int8_t *w,
+                                 const float *w_scales, const float *bias, size_t m, size_t n, size_t k, int32_t mode,
+                                 float *out) {
+    const size_t partial_bytes = linear_dynamic_partial_bytes(ctx->num_cus);
+    hipq_qparams *params = reinterpret_cast<hipq_qparams *>(base);
+    void *partials = base + kScratchHeader;
+    float *row_scales = reinterpret_cast<float *>(base + kScratchHeader + partial_bytes);
+    int8_t *qa = reinterpret_cast<int8_t *>(base + kScratchHeader + partial_bytes + linear_dynamic_scales_bytes(m));
+    int32_t rc;
+    if (per_token) {
+        rc = hipq_quantize_per_row_f32_i8(ctx, x, m, k, HIPQ_PARAMS_SYMMETRIC, mode & HIPQ_ROUND_HALF_EVEN, qa,
+                                          row_scales, nullptr, nullptr);
+        if (rc) return rc;
+        return hipq_linear_i8_f32(ctx, qa, row_scales, 1, w, w_scales, bias, m, n, k, out);
+    }
+    rc = quantize_dynamic_per_tensor(ctx, x, m * k, HIPQ_PARAMS_SYMMETRIC, HIPQ_DTYPE_I8, mode, qa, params, partials,
+                                     partial_bytes);
+    if (rc) return rc;
+    // hipq_qparams starts with the f32 scale.
+    return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
+}
+
+// Scratch of hipq_linear_dynamic_f32_noalloc: device memory that exists from the moment the library is
+// loaded, so the entry point never calls an allocator.  Every GPU holds its own copy at its own address;
+// host code uses the per-device pointer from hipGetSymbolAddress, never the array's name.
+constexpr int kMaxDevices = 64;
+constexpr size_t kNoAllocMaxRows = 16384;
+constexpr size_t kNoAllocMaxElems = size_t(4) << 20;  // m * k
+constexpr size_t kNoAllocBytes = kScratchHeader + 1024 * 16 * sizeof(float2) + kNoAllocMaxRows * sizeof(float) +
+                                 kNoAllocMaxElems + 256;
+static __device__ __align__(256) unsigned char noalloc_scratch[kNoAllocBytes];
+static void *g_noalloc_ptr[kMaxDevices] = {nullptr};
+static std::mutex g_noalloc_mutex;
+
+int32_t linear_noalloc_setup(int device) {
+    if (device < 0 || device >= kMaxDevices) return HIPQ_SUCCESS;  // the no-alloc entry point reports it
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (g_noalloc_ptr[device]) return HIPQ_SUCCESS;
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(noalloc_scratch));
+    if (e != hipSuccess || !p)
+        return fail(HIPQ_DEVICE_ERROR, "hipGetSymbolAddress(noalloc_scratch) on device %d: %s", device,
+                    hipGetErrorString(e));
+    g_noalloc_ptr[device] = p;
+    return HIPQ_SUCCESS;
+}
+
 }  // namespace hipq
 
 using namespace hipq;
@@ -455,35 +524,31 @@ int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t per_token
                                 const float *w_scales, const float *bias, size_t m, size_t n, size_t k, int32_t mode,
                                 float *out) {
     HIPQ_ENTER(ctx);
-    int32_t rc = check_gemm_shape(__func__, m, n, k);
-    if (rc) return rc;
-    if (m == 0 || n == 0) return HIPQ_SUCCESS;
-    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
-    HIPQ_REQUIRE_PTR(x);
-    HIPQ_REQUIRE_PTR(w);
-    HIPQ_REQUIRE_PTR(w_scales);
-    HIPQ_REQUIRE_PTR(out);
-    // Scratch layout after the header: per-row scales [m] floats, then int8 activations [m,k].
-    const size_t scales_bytes = ((m * sizeof(float)) + 255) & ~size_t(255);
-    // The range-reduction partials live at the start of the bulk area; keep clear of them.
-    const size_t partial_bytes = size_t(ctx->num_cus) * 16 * sizeof(float2);
+    int32_t rc = check_linear_dynamic_args(__func__, x, w, w_scales, m, n, k, out);
+    if (rc || m == 0 || n == 0) return rc;
     void *s = nullptr;
-    rc = scratch(ctx, kScratchHeader + partial_bytes + scales_bytes + m * k + 256, &s);
+    rc = scratch(ctx, linear_dynamic_scratch_bytes(ctx->num_cus, m, k), &s);
     if (rc) return rc;
-    char *base = static_cast<char *>(s);
-    hipq_qparams *params = reinterpret_cast<hipq_qparams *>(base);
-    float *row_scales = reinterpret_cast<float *>(base + kScratchHeader + partial_bytes);
-    int8_t *qa = reinterpret_cast<int8_t *>(base + kScratchHeader + partial_bytes + scales_bytes);
-    if (per_token) {
-        rc = hipq_quantize_per_row_f32_i8(ctx, x, m, k, HIPQ_PARAMS_SYMMETRIC, mode & HIPQ_ROUND_HALF_EVEN, qa,
-                                          row_scales, nullptr, nullptr);
-        if (rc) return rc;
-        return hipq_linear_i8_f32(ctx, qa, row_scales, 1, w, w_scales, bias, m, n, k, out);
-    }
-    rc = hipq_quantize_dynamic_per_tensor_f32(ctx, x, m * k, HIPQ_PARAMS_SYMMETRIC, HIPQ_DTYPE_I8, mode, qa, params);
-    if (rc) return rc;
-    // hipq_qparams starts with the f32 scale.
-    return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
+    return linear_dynamic_on(ctx, static_cast<char *>(s), x, per_token, w, w_scales, bias, m, n, k, mode, out);
+}
+
+int32_t hipq_linear_dynamic_f32_noalloc(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w,
+                                        const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
+                                        int32_t mode, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_linear_dynamic_args(__func__, x, w, w_scales, m, n, k, out);
+    if (rc || m == 0 || n == 0) return rc;
+    if (m > kNoAllocMaxRows || m * k > kNoAllocMaxElems)
+        return fail(HIPQ_SHAPE_ERROR,
+                    "%s: activations [%zu,%zu] exceed the static scratch (at most %zu rows and %zu elements); "
+                    "use hipq_linear_dynamic_f32",
+                    __func__, m, k, kNoAllocMaxRows, kNoAllocMaxElems);
+    if (ctx->device < 0 || ctx->device >= kMaxDevices || !g_noalloc_ptr[ctx->device])
+        return fail(HIPQ_DEVICE_ERROR, "%s: the static scratch of device %d was not set up", __func__, ctx->device);
+    if (linear_dynamic_scratch_bytes(ctx->num_cus, m, k) > kNoAllocBytes)
+        return fail(HIPQ_SHAPE_ERROR, "%s: scratch layout does not fit the static array", __func__);
+    return linear_dynamic_on(ctx, static_cast<char *>(g_noalloc_ptr[ctx->device]), x, per_token, w, w_scales, bias, m,
+                             n, k, mode, out);
 }
 
 int32_t hipq_set_gemm_kernel_variant(int32_t variant) {

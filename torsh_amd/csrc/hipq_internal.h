@@ -34,6 +34,16 @@ int32_t scratch(hipq_ctx *ctx, size_t bytes, void **out);
 // Checks the sticky launch error after a kernel launch.
 int32_t check_launch(const char *what);
 
+// hipq_quantize_dynamic_per_tensor_f32 with the room for its range partials given by the caller
+// (`partials`, `partials_bytes` of device memory) instead of taken from the context scratch; null =
+// context scratch.
+int32_t quantize_dynamic_per_tensor(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor, int32_t dtype,
+                                    int32_t mode, void *out, hipq_qparams *out_params, void *partials,
+                                    size_t partials_bytes);
+// Looks up, once per device, the address of the static device array behind
+// hipq_linear_dynamic_f32_noalloc; called by hipq_ctx_create with the device current.
+int32_t linear_noalloc_setup(int device);
+
 // Bytes reserved at the head of the context scratch for small device records
 // (hipq_qparams, min/max pairs, status words); bulk scratch starts after it.
 constexpr size_t kScratchHeader = 4096;

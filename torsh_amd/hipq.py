@@ -105,6 +105,7 @@ _SIGNATURES = {
     "hipq_linear_i8_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _f32, _i32, _i32, _vp],
     "hipq_requantize_i32_i8": [_vp, _vp, _sz, _sz, _vp, _i32, _vp, _vp, _f32, _i32, _i32, _vp],
     "hipq_linear_dynamic_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
+    "hipq_linear_dynamic_f32_noalloc": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_quantize_per_row_strided_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
     "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
@@ -507,6 +508,16 @@ class Context:
         out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
         self.call("hipq_linear_dynamic_f32", _ptr(x), int(per_token), _ptr(w), _ptr(w_scales), _ptr(bias), m, n, k,
                   mode, _ptr(out))
+        return out
+
+    def linear_dynamic_noalloc(self, x, w, w_scales, bias=None, per_token=False, mode=0, out=None):
+        """hipq_linear_dynamic_f32_noalloc: the same forward on the library's static device scratch.  `out`
+        should be given by callers that must not allocate; it is created here only as a convenience."""
+        m, k = x.shape
+        n, _ = w.shape
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_dynamic_f32_noalloc", _ptr(x), int(per_token), _ptr(w), _ptr(w_scales), _ptr(bias), m, n,
+                  k, mode, _ptr(out))
         return out
 
     def conv2d_i32(self, x_u8, zp_in, w_i8, stride=(1, 1), padding=(0, 0)):
