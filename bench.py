@@ -5,7 +5,8 @@ One "step" is one QuantizedLinear forward of the headline workload:
 fp32 activations [512,4096] -> dynamic per-tensor
 int8 quantize (min/max, scale, quantize) -> int8 x int8 -> int32 MFMA GEMM
 against per-output-channel int8 weights [4096,4096] -> dequantize + bias epilogue
--> fp32 [512,4096].  All inputs are resident in HBM before the timed region.
+-> fp32 [512,4096].  The weights are prepared once (quantized per channel and stored
+in the operand order of the matrix cores), as a converted layer holds them.  All inputs are resident in HBM before the timed region.
 Activations, weights and outputs rotate through pools larger than the 256 MB
 memory-side cache, so every step streams its operands from HBM as successive
 layers of a model would.
@@ -30,10 +31,21 @@ if ROOT not in sys.path:
 PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA, 5.0 POP/s
 PEAK_HBM_GBPS = 8000.0   # MI355X HBM3E, 8 TB/s
 
-# HBM-side bytes per GEMM launch from rocprofv3 --pmc: FETCH_SIZE 16509 (x2.0: the same counter reads
-# 32781 for a 65536 KiB copy) + WRITE_SIZE 8192 KiB (x1.0) = 33.8 MB read + 8.4 MB written.  The reads are
-# the 16.8 MB of weights once plus the 2.1 MB of activations once per XCD (8 private L2s).
-GEMM_TRAFFIC_BYTES = 42.2e6
+# rocprofv3 summary of the dominant kernel (kernel-trace durations and the FETCH_SIZE / WRITE_SIZE counter
+# passes).  `roofline.traffic` is read from its line "hbm_traffic_bytes_per_launch = <bytes>"; no file or no
+# such line -> null, so the JSON never carries a figure that was not measured for this kernel.
+GEMM_PROFILE = os.path.join(ROOT, "profiles", "gemm_i8_packed_kernel_linear_m512_n4096_k4096.txt")
+
+
+def measured_gemm_traffic():
+    try:
+        with open(GEMM_PROFILE) as f:
+            for line in f:
+                if line.strip().startswith("hbm_traffic_bytes_per_launch"):
+                    return float(line.split("=")[1].split()[0])
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
 
 
 def event_time_ms(fn, reps: int, warmup: int) -> float:
@@ -101,16 +113,58 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
 
     g = torch.Generator(device="cuda").manual_seed(2)
     reps = 20
-    if which == "gemm":
+    if which in ("gemm", "gemm_rowmajor"):
         aq = [torch.randint(-128, 128, (M, K), generator=g, device="cuda", dtype=torch.int8) for _ in range(reps)]
         wq = [torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8) for _ in range(reps)]
         sw = torch.rand(N, generator=g, device="cuda") * 1e-3
         bias = torch.randn(N, generator=g, device="cuda") * 0.01
         sa = torch.full((1,), 0.03, device="cuda")
         outs = [torch.empty(M, N, device="cuda") for _ in range(reps)]
+        if which == "gemm":  # the packed-operand kernel the step runs
+            pa = [ctx.pack_rows(a) for a in aq]
+            pw = [ctx.pack_rows(w) for w in wq]
+            del aq, wq
+            torch.cuda.synchronize()
+            for i in range(reps):
+                ctx.linear_packed_i8_f32(pa[i], sa, pw[i], sw, bias, M, N, K, out=outs[i])
+        else:
+            torch.cuda.synchronize()
+            for i in range(reps):
+                ctx.linear_i8_f32(aq[i], sa, wq[i], sw, bias, out=outs[i])
+    elif which == "step":
+        # the whole Linear step (range pass, quantize into the packed layout, packed GEMM), HBM-cold operands
+        xs = [torch.randn(M, K, generator=g, device="cuda") for _ in range(reps)]
+        pw = [ctx.pack_rows(torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8))
+              for _ in range(reps)]
+        sw = torch.rand(N, generator=g, device="cuda") * 1e-3
+        bias = torch.randn(N, generator=g, device="cuda") * 0.01
+        outs = [torch.empty(M, N, device="cuda") for _ in range(reps)]
         torch.cuda.synchronize()
         for i in range(reps):
-            ctx.linear_i8_f32(aq[i], sa, wq[i], sw, bias, out=outs[i])
+            ctx.linear_dynamic_packed(xs[i], pw[i], sw, bias, per_token=False, mode=hipq.FORM_MUL_INV, out=outs[i])
+    elif which == "gemv":
+        # configs[2]: decode-shaped skinny GEMM, N=11008, K=4096, M = 1, 4, 16 (20 launches each)
+        n3, k3 = 11008, 4096
+        w3 = [torch.randint(-128, 128, (n3, k3), generator=g, device="cuda", dtype=torch.int8) for _ in range(8)]
+        sw3 = torch.rand(n3, generator=g, device="cuda") * 1e-3
+        for m3 in (1, 4, 16):
+            a3 = torch.randint(-128, 128, (m3, k3), generator=g, device="cuda", dtype=torch.int8)
+            sa3 = torch.rand(m3, generator=g, device="cuda") * 0.05 + 0.01
+            o3 = torch.empty(m3, n3, device="cuda")
+            torch.cuda.synchronize()
+            for i in range(reps):
+                ctx.linear_i8_f32(a3, sa3, w3[i % 8], sw3, None, out=o3)
+    elif which == "conv":
+        # configs[3]: quantized Conv2d [32,256,14,14] (*) [256,256,3,3], stride 1, pad 1, fused bias + requant
+        xc = [torch.randint(0, 256, (32, 256, 14, 14), generator=g, device="cuda", dtype=torch.uint8) for _ in range(8)]
+        wc = torch.randint(-128, 128, (256, 256, 3, 3), generator=g, device="cuda", dtype=torch.int8)
+        swc = torch.rand(256, generator=g, device="cuda") * 1e-3
+        bc = torch.randn(256, generator=g, device="cuda") * 0.01
+        packed, sums = ctx.conv2d_pack_weights(wc)
+        oc = torch.empty((32, 256, 14, 14), dtype=torch.int8, device="cuda")
+        torch.cuda.synchronize()
+        for i in range(reps):
+            ctx.conv2d_i8_packed(xc[i % 8], 0, 0.02, packed, sums, (3, 3), swc, bc, 0.05, 0, (1, 1), out=oc)
     elif which == "quantize":
         n = 4096 * 4096
         xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
@@ -197,7 +251,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "quantize", "calib", "special", "copy", "stack"], default=None,
+    ap.add_argument("--profile", choices=["gemm", "gemm_rowmajor", "step", "quantize", "calib", "special", "copy",
+                                          "stack", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -220,12 +275,13 @@ def main() -> int:
     g = torch.Generator(device="cuda").manual_seed(2)
     pool = 32  # 32 x 16.8 MB weights = 537 MB > 256 MB memory-side cache
     xs = [torch.randn(M, K, generator=g, device="cuda") for _ in range(pool)]
-    wq, sw = [], []
+    wq, sw, pw = [], [], []
     for i in range(pool):
         wf = torch.randn(N, K, generator=g, device="cuda") * 0.02
         q, s, _, _ = ctx.quantize_per_row(wf)
         wq.append(q)
         sw.append(s)
+        pw.append(ctx.pack_rows(q))  # weight preparation, once per layer: the operand order of the matrix cores
         del wf
     bias = torch.randn(N, generator=g, device="cuda") * 0.01
     outs = [torch.empty(M, N, device="cuda") for _ in range(pool)]
@@ -236,7 +292,7 @@ def main() -> int:
     def step():
         i = it[0] % pool
         it[0] += 1
-        ctx.linear_dynamic(xs[i], wq[i], sw[i], bias, per_token=False, mode=hipq.FORM_MUL_INV, out=outs[i])
+        ctx.linear_dynamic_packed(xs[i], pw[i], sw[i], bias, per_token=False, mode=hipq.FORM_MUL_INV, out=outs[i])
 
     for _ in range(args.warmup):
         step()
@@ -251,14 +307,14 @@ def main() -> int:
     value = ops / (ms_per_step * 1e-3) / 1e12
 
     # dominant kernel on its own: the GEMM + dequant epilogue on pre-quantized activations
-    aq = [ctx.quantize_dynamic_per_tensor(x)[0] for x in xs]
+    pa = [ctx.quantize_per_tensor_packed(x, dynamic=True, mode=hipq.FORM_MUL_INV)[0] for x in xs]
     sa = torch.full((1,), 0.03, device="cuda")
     jt = [0]
 
     def gemm_only():
         i = jt[0] % pool
         jt[0] += 1
-        ctx.linear_i8_f32(aq[i], sa, wq[i], sw[i], bias, out=outs[i])
+        ctx.linear_packed_i8_f32(pa[i], sa, pw[i], sw[i], bias, M, N, K, out=outs[i])
 
     gemm_ms = event_time_ms(gemm_only, reps=max(args.steps, 100), warmup=args.warmup)
     gemm_tops = ops / (gemm_ms * 1e-3) / 1e12
@@ -285,13 +341,13 @@ def main() -> int:
             "operand_pool": f"{pool} rotating weight/activation/output sets (HBM-cold)",
         },
         "roofline": {
-            "kernel": "gemm_i8_pipe_kernel (int8 MFMA GEMM + dequant/bias epilogue)",
+            "kernel": "gemm_i8_packed_kernel (int8 MFMA GEMM on fragment-packed operands + dequant/bias epilogue)",
             "bound": "mfma",
             "achieved": gemm_tops,
             "peak": PEAK_INT8_TOPS,
             "unit": "TOP/s",
             "frac": gemm_tops / PEAK_INT8_TOPS,
-            "traffic": GEMM_TRAFFIC_BYTES,
+            "traffic": measured_gemm_traffic(),
             "ops_per_launch": ops,
             "algorithmic_bytes_per_launch": algo_bytes,
             "avg_launch_us": gemm_ms * 1e3,
@@ -310,8 +366,8 @@ def main() -> int:
         def step_two_streams():
             i = pt[0] % pool
             pt[0] += 1
-            (ctx2 if i % 2 == 0 else ctx3).linear_dynamic(xs[i], wq[i], sw[i], bias, per_token=False,
-                                                        mode=hipq.FORM_MUL_INV, out=outs[i])
+            (ctx2 if i % 2 == 0 else ctx3).linear_dynamic_packed(xs[i], pw[i], sw[i], bias, per_token=False,
+                                                               mode=hipq.FORM_MUL_INV, out=outs[i])
 
         for _ in range(args.warmup):
             step_two_streams()
@@ -331,7 +387,7 @@ def main() -> int:
         def step_static():
             i = ps[0] % pool
             ps[0] += 1
-            ctx.linear_static(xs[i], 0.035, wq[i], sw[i], bias, mode=hipq.FORM_MUL_INV, out=outs[i])
+            ctx.linear_static_packed(xs[i], 0.035, pw[i], sw[i], bias, mode=hipq.FORM_MUL_INV, out=outs[i])
 
         for _ in range(args.warmup):
             step_static()
@@ -344,6 +400,24 @@ def main() -> int:
         extra["linear_step_static_activation_scale"] = {"ms_per_step": ms3, "TOP/s": ops / (ms3 * 1e-3) / 1e12,
                                                         "note": "activation scale from calibration instead of a "
                                                                 "min/max pass per call (two launches, not three)"}
+        # The same step on row-major int8 weights (no weight preparation): LDS-staged kernel.
+        pr = [0]
+
+        def step_row_major():
+            i = pr[0] % pool
+            pr[0] += 1
+            ctx.linear_dynamic(xs[i], wq[i], sw[i], bias, per_token=False, mode=hipq.FORM_MUL_INV, out=outs[i])
+
+        for _ in range(args.warmup):
+            step_row_major()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_row_major()
+        torch.cuda.synchronize()
+        ms4 = (time.perf_counter() - t0) * 1e3 / args.steps
+        extra["linear_step_row_major_weights"] = {"ms_per_step": ms4, "TOP/s": ops / (ms4 * 1e-3) / 1e12,
+                                                  "note": "hipq_linear_dynamic_f32 on unprepared [N,K] weights"}
         n = 4096 * 4096
         npool = 10  # 10 x (64 + 16 + 64) MiB > memory-side cache
         fx = [torch.randn(n, generator=g, device="cuda") for _ in range(npool)]

@@ -301,7 +301,9 @@ HIPQ_API int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_s
 /* Whole forward of a quantized Linear on fp32 activations: dynamic activation
  * quantization (per tensor: algorithms.rs:85-123; per token: algorithms.rs:126-242
  * on axis 0), int8 GEMM, dequantizing epilogue.  Uses context-owned scratch
- * for the int8 activations and their scales. */
+ * for the int8 activations and their scales.  Activations whose range is not finite (NaN / Inf
+ * present; the reference returns InvalidArgument, algorithms.rs:403-407) cannot fail an asynchronous
+ * call: the outputs that depend on them are NaN (the whole output per tensor, the row per token). */
 HIPQ_API int32_t hipq_linear_dynamic_f32(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w,
                                          const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
                                          int32_t mode, float *out);
@@ -317,6 +319,52 @@ HIPQ_API int32_t hipq_linear_dynamic_f32_noalloc(hipq_ctx *ctx, const float *x, 
                                                  const float *w_scales, const float *bias, size_t m, size_t n,
                                                  size_t k, int32_t mode, float *out);
 
+
+/* ---- fragment-packed operands: the fast Linear forward ------------------ */
+/* The int8 GEMM reads its operands fastest in the order the matrix cores consume them.  A packed
+ * int8 matrix [rows, k] is [rows/32][k/32][1 KiB]: inside a 1 KiB fragment, 16-byte slot l holds
+ * row 32*rb + l%32, bytes 32*kb + 16*(l/32) .. +15 (one operand of v_mfma_i32_32x32x32_i8).  Rows are
+ * padded to a multiple of 32, the k blocks of a row block to a multiple of 4; padding along k is
+ * zero.  This is the "tile order" of a prepared weight blob: weights are packed once when a layer
+ * is converted (where QuantizedLinear::from_linear transposes Linear's [in,out] weight,
+ * crates/torsh-nn/src/layers/linear.rs:28-31), activations are written packed by the quantize pass.
+ * Same integers as the row-major form, so every result below is bit-identical to the row-major
+ * entry point named beside it.  Packed buffers are device memory, 16-byte aligned, below 2 GiB. */
+/* Bytes of the packed form of an int8 [rows, k] matrix (host call, no device work). */
+HIPQ_API int32_t hipq_packed_size(size_t rows, size_t k, size_t *out_bytes);
+/* Row-major int8 [rows, k] -> packed (weight preparation; also for callers that hold int8 activations). */
+HIPQ_API int32_t hipq_pack_rows_i8(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_t *dst_packed);
+/* hipq_gemm_i8_i32 on packed operands: vnni_matmul_kernel,
+ * crates/torsh-backend/src/quantization/specialized.rs:175-201.  out is row-major [m, n]. */
+HIPQ_API int32_t hipq_gemm_packed_i8_i32(hipq_ctx *ctx, const int8_t *a_packed, const int8_t *w_packed, size_t m,
+                                         size_t n, size_t k, int32_t *out);
+/* hipq_linear_i8_f32 on packed operands (acc * (s_a * s_w[n]) + bias[n]:
+ * crates/torsh-backend/src/quantization/operations.rs:669,722 and ops.rs:561). */
+HIPQ_API int32_t hipq_linear_packed_i8_f32(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                           int32_t a_scale_per_row, const int8_t *w_packed, const float *w_scales,
+                                           const float *bias, size_t m, size_t n, size_t k, float *out);
+/* hipq_linear_i8_i8 on packed operands (requantizing epilogue, operations.rs:722-728). */
+HIPQ_API int32_t hipq_linear_packed_i8_i8(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                          int32_t a_scale_per_row, const int8_t *w_packed, const float *w_scales,
+                                          const float *bias, size_t m, size_t n, size_t k, float out_scale,
+                                          int32_t out_zero_point, int32_t mode, int8_t *out);
+/* Symmetric per-tensor int8 quantize of fp32 [rows, cols] into the packed layout: with `dynamic` the
+ * scale comes from the tensor's own range (quantize_tensor_auto, crates/torsh-quantization/src/algorithms.rs:85-123),
+ * otherwise `scale` is used (quantize_per_tensor_affine, algorithms.rs:277-315).  Codes are those of
+ * hipq_quantize_dynamic_per_tensor_f32 / hipq_quantize_per_tensor_f32_i8; a range that is not finite
+ * gives status HIPQ_INVALID_ARGUMENT in out_params, a NaN scale and zero codes. */
+HIPQ_API int32_t hipq_quantize_per_tensor_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
+                                                        int32_t dynamic, float scale, int32_t mode,
+                                                        int8_t *out_packed, hipq_qparams *out_params);
+/* hipq_linear_dynamic_f32 with prepared (packed) weights: range pass, quantize into the packed
+ * layout, packed GEMM with the dequantizing epilogue. */
+HIPQ_API int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t per_token,
+                                                const int8_t *w_packed, const float *w_scales, const float *bias,
+                                                size_t m, size_t n, size_t k, int32_t mode, float *out);
+/* hipq_linear_static_f32 with prepared (packed) weights. */
+HIPQ_API int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w_packed,
+                                               const float *w_scales, const float *bias, size_t m, size_t n,
+                                               size_t k, int32_t mode, float *out);
 
 /* ---- quantized Conv2d forward (NCHW, filters [OC,IC,KH,KW]) ------------ */
 /* Integer part of perform_quantized_convolution,

@@ -1,0 +1,243 @@
+"""Parity of the fragment-packed GEMM / Linear forward (the fast path of the headline shape).
+
+Packed operands hold the same integers as the row-major ones, so every result is compared bit for bit with
+the CPU oracle (int32 accumulators, int8 outputs, and in practice the fp32 outputs too, which are also held
+to the stated 1e-5 relative bar), and with the row-major entry points of the library.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rand_i8(rng, shape):
+    return rng.integers(-128, 128, size=shape, dtype=np.int8)
+
+
+def pack_reference(q: np.ndarray) -> np.ndarray:
+    """The packed layout written out in numpy: [rows/32][k blocks, padded to 4][64 slots of 16 bytes],
+    slot l = row l % 32, bytes 16 * (l // 32) .. + 15 of the 32-byte k block."""
+    rows, k = q.shape
+    rb, kb = (rows + 31) // 32, ((k + 31) // 32 + 3) // 4 * 4
+    padded = np.zeros((rb * 32, kb * 32), np.int8)
+    padded[:rows, :k] = q
+    # [rb, 32 rows, kb, 2 halves, 16 bytes] -> [rb, kb, half, row, 16]
+    t = padded.reshape(rb, 32, kb, 2, 16).transpose(0, 2, 3, 1, 4)
+    return np.ascontiguousarray(t).reshape(-1)
+
+
+@pytest.mark.parametrize("rows,k", [(1, 1), (32, 32), (33, 31), (64, 128), (100, 304), (5, 1001), (130, 4096)])
+def test_pack_rows_layout(ctx, rows, k):
+    rng = np.random.default_rng(rows * 7919 + k)
+    q = rand_i8(rng, (rows, k))
+    assert ctx.packed_size(rows, k) == pack_reference(q).size
+    np.testing.assert_array_equal(host(ctx.pack_rows(dev(q))), pack_reference(q))
+
+
+SHAPES = [
+    (1, 1, 16), (1, 16, 64), (16, 16, 64), (17, 33, 128), (64, 64, 256), (128, 64, 128), (130, 70, 144),
+    (127, 129, 4096), (512, 256, 1024), (5, 300, 48), (256, 512, 16), (33, 1000, 2048), (9, 40, 1001), (3, 5, 7),
+    (129, 65, 512), (200, 96, 768), (256, 128, 2304), (96, 200, 11008),
+]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_packed_bit_exact(ctx, oracle, m, n, k):
+    rng = np.random.default_rng(m * 1000003 + n * 1009 + k)
+    a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+    got = host(ctx.gemm_packed_i8_i32(ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w)), m, n, k))
+    np.testing.assert_array_equal(got, oracle.gemm_i8_nk(a, w))
+
+
+def test_gemm_packed_extreme_values(ctx):
+    a = np.full((32, 4096), -128, np.int8)
+    pa = ctx.pack_rows(dev(a))
+    got = host(ctx.gemm_packed_i8_i32(pa, pa, 32, 32, 4096))
+    np.testing.assert_array_equal(got, np.full((32, 32), 4096 * 16384, np.int32))
+
+
+def _linear_case(oracle, m, n, k, per_token, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wf = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    wq, sw, _ = oracle.quantize_per_channel_auto(wf, 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    if per_token:
+        aq, sa, _ = oracle.quantize_per_channel_auto(x, 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    else:
+        aq, s, _ = oracle.quantize_tensor_auto(x, 0, oracle.PER_TENSOR_SYMMETRIC)
+        sa = np.array([s], np.float32)
+    acc = oracle.gemm_i8_nk(aq.astype(np.int8), wq.astype(np.int8))
+    out = oracle.linear_dequant_epilogue(acc, sa, sw, bias)
+    return x, bias, wq.astype(np.int8), sw, aq.astype(np.int8), sa, acc, out
+
+
+@pytest.mark.parametrize("m,n,k", [(4, 8, 16), (64, 128, 256), (100, 200, 304), (512, 512, 512), (33, 65, 1040),
+                                   (130, 72, 768)])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_linear_packed_forward(ctx, hipq, oracle, m, n, k, per_token):
+    x, bias, wq, sw, aq, sa, acc, want = _linear_case(oracle, m, n, k, per_token, m + n + k)
+    pw = ctx.pack_rows(dev(wq))
+    # separate steps: packed int8 activations given by the caller
+    got = host(ctx.linear_packed_i8_f32(ctx.pack_rows(dev(aq)), dev(sa), pw, dev(sw), dev(bias), m, n, k))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=0)
+    np.testing.assert_array_equal(got, want)
+    # whole forward from fp32 activations (the reference's branch for the size: x * (1/scale) above 64 elements)
+    mode = hipq.FORM_MUL_INV if x.size > 64 else hipq.FORM_DIV
+    got = host(ctx.linear_dynamic_packed(dev(x), pw, dev(sw), dev(bias), per_token=per_token, mode=mode))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=0)
+    np.testing.assert_array_equal(got, want)
+    # the row-major entry point gives the same bits
+    np.testing.assert_array_equal(
+        got, host(ctx.linear_dynamic(dev(x), dev(wq), dev(sw), dev(bias), per_token=per_token, mode=mode)))
+    # no bias
+    got = host(ctx.linear_packed_i8_f32(ctx.pack_rows(dev(aq)), dev(sa), pw, dev(sw), None, m, n, k))
+    np.testing.assert_array_equal(got, oracle.linear_dequant_epilogue(acc, sa, sw, None))
+
+
+@pytest.mark.parametrize("m,n,k", [(7, 24, 64), (128, 96, 512), (50, 130, 272), (130, 132, 384), (67, 131, 256)])
+def test_linear_packed_requant_epilogue(ctx, hipq, oracle, m, n, k):
+    x, bias, wq, sw, aq, sa, acc, out = _linear_case(oracle, m, n, k, False, 5 * m + k)
+    s_out, _ = oracle.calculate_symmetric_params(*oracle.find_min_max(out), 0)
+    pa, pw = ctx.pack_rows(dev(aq)), ctx.pack_rows(dev(wq))
+    for mode, rm in ((hipq.ROUND_HALF_AWAY, 0), (hipq.ROUND_HALF_EVEN, 1)):
+        oracle.set_round_mode(rm)
+        try:
+            wantq = oracle.requantize_epilogue(acc, sa, sw, bias, s_out, -5)
+        finally:
+            oracle.set_round_mode(0)
+        got = host(ctx.linear_packed_i8_i8(pa, dev(sa), pw, dev(sw), dev(bias), m, n, k, s_out, -5, mode))
+        np.testing.assert_array_equal(got, wantq)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (3, 70), (64, 256), (100, 304), (33, 1001), (512, 4096)])
+def test_quantize_per_tensor_packed_matches_row_major(ctx, hipq, rows, cols):
+    """Codes and parameters of the packed quantizer = those of the row-major dynamic quantizer (itself bit-exact
+    with the oracle, tests/test_gpu_elementwise.py), then packed; both quantize forms and roundings; static scale."""
+    g = torch.Generator(device="cuda").manual_seed(rows * 31 + cols)
+    x = torch.randn(rows, cols, generator=g, device="cuda")
+    x[0, 0] = 2.5 * x.abs().max()  # makes x / scale land on ties here and there
+    for mode in (hipq.FORM_MUL_INV, hipq.FORM_DIV, hipq.FORM_DIV | hipq.ROUND_HALF_EVEN, hipq.ROUND_HALF_EVEN):
+        q, params = ctx.quantize_dynamic_per_tensor(x, mode=mode)
+        pq, pparams = ctx.quantize_per_tensor_packed(x, dynamic=True, mode=mode)
+        torch.cuda.synchronize()
+        assert torch.equal(pq, ctx.pack_rows(q))
+        a, b = ctx.read_qparams(params), ctx.read_qparams(pparams)
+        assert (a.scale, a.zero_point, a.min_val, a.max_val, a.status) == (b.scale, b.zero_point, b.min_val, b.max_val,
+                                                                        b.status)
+        qs = ctx.quantize_per_tensor_i8(x, 0.037, 0, mode)
+        pqs, sp = ctx.quantize_per_tensor_packed(x, dynamic=False, scale=0.037, mode=mode)
+        torch.cuda.synchronize()
+        assert torch.equal(pqs, ctx.pack_rows(qs))
+        assert ctx.read_qparams(sp).scale == np.float32(0.037)
+
+
+def test_linear_static_packed(ctx, hipq):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    m, n, k = 96, 160, 512
+    x = torch.randn(m, k, generator=g, device="cuda")
+    wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(n, generator=g, device="cuda") * 0.01
+    want = ctx.linear_static(x, 0.031, wq, sw, bias, mode=hipq.FORM_MUL_INV)
+    got = ctx.linear_static_packed(x, 0.031, ctx.pack_rows(wq), sw, bias, mode=hipq.FORM_MUL_INV)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("bad", [float("nan"), float("inf"), float("-inf")])
+def test_non_finite_activations_give_nan_outputs_not_stale_scratch(ctx, hipq, packed, per_token, bad):
+    """The reference refuses a range that is not finite (algorithms.rs:403-407: an Inf among the activations).
+    An asynchronous call cannot fail after the fact; it must not multiply whatever an earlier call left in the
+    scratch either: the outputs that depend on the bad range are NaN (all of them per tensor, the row per token),
+    the rest exact.  A NaN is different: f32::min / f32::max skip it (simd_ops.rs:95-108), the range stays finite
+    and the element quantizes to 0 (`NaN as i8`), i.e. the result is that of the input with a 0.0 in its place."""
+    g = torch.Generator(device="cuda").manual_seed(17)
+    m, n, k = 40, 72, 256
+    x = torch.randn(m, k, generator=g, device="cuda")
+    wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(n, generator=g, device="cuda") * 0.01
+    w_arg = ctx.pack_rows(wq) if packed else wq
+    run = ctx.linear_dynamic_packed if packed else ctx.linear_dynamic
+    good = run(x, w_arg, sw, bias, per_token=per_token, mode=hipq.FORM_MUL_INV)  # fills the scratch with real codes
+    xb = x.clone()
+    xb[7, 100] = bad
+    got = run(xb, w_arg, sw, bias, per_token=per_token, mode=hipq.FORM_MUL_INV)
+    torch.cuda.synchronize()
+    if bad != bad:
+        xz = x.clone()
+        xz[7, 100] = 0.0
+        want = run(xz, w_arg, sw, bias, per_token=per_token, mode=hipq.FORM_MUL_INV)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+    elif per_token:
+        assert torch.isnan(got[7]).all()
+        keep = [i for i in range(m) if i != 7]
+        assert torch.equal(got[keep], good[keep])
+    else:
+        assert torch.isnan(got).all()
+
+
+def test_config2_full_size_packed_forward(ctx, hipq):
+    """BASELINE configs[1] at full size through the packed forward the bench times: M=512, K=N=4096.  int8
+    activations against torch's formulation of clamp(round_half_away(x * (1/s))), accumulators against an exact
+    float64 product, fp32 output against the same individually rounded f32 expression (1e-5 relative stated;
+    equal in practice), and the row-major entry point against the packed one."""
+    g = torch.Generator(device="cuda").manual_seed(2)
+    m, n, k = 512, 4096, 4096
+    x = torch.randn(m, k, generator=g, device="cuda")
+    wf = torch.randn(n, k, generator=g, device="cuda") * 0.02
+    bias = torch.randn(n, generator=g, device="cuda") * 0.01
+    wq, sw, _, _ = ctx.quantize_per_row(wf)
+    pw = ctx.pack_rows(wq)
+    out = ctx.linear_dynamic_packed(x, pw, sw, bias, per_token=False, mode=hipq.FORM_MUL_INV)
+    # activations: a2 + a5 (len > 64 branch), restated with torch ops
+    absmax = x.abs().max()
+    s = absmax / 127.0
+    inv = 1.0 / s
+    t = x * inv
+    # f32::round = trunc(t + copysign(0.5, t)), exact except where t + 0.5 rounds up across an integer, which
+    # happens only for |t| = 0.49999997: make sure no element sits there, then the simple form is the definition
+    assert not bool(((t.abs() > 0.4999999) & (t.abs() < 0.5)).any())
+    qa = torch.clamp(torch.trunc(t + torch.copysign(torch.full_like(t, 0.5), t)), -128, 127)
+    pq, params = ctx.quantize_per_tensor_packed(x, dynamic=True, mode=hipq.FORM_MUL_INV)
+    torch.cuda.synchronize()
+    assert ctx.read_qparams(params).scale == float(s)
+    assert torch.equal(pq, ctx.pack_rows(qa.to(torch.int8)))
+    acc = (qa.double() @ wq.double().T)  # exact: |acc| < 2^53
+    assert torch.equal(ctx.gemm_packed_i8_i32(pq, pw, m, n, k), acc.to(torch.int32))
+    want = acc.float() * (s * sw[None, :]) + bias[None, :]  # same individually rounded f32 operations
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=0)
+    assert torch.equal(out, want)
+    assert torch.equal(out, ctx.linear_dynamic(x, wq, sw, bias, per_token=False, mode=hipq.FORM_MUL_INV))
+
+
+def test_packed_argument_errors(ctx, hipq):
+    a = torch.zeros(1024, dtype=torch.int8, device="cuda")
+    out = torch.zeros((4, 4), dtype=torch.int32, device="cuda")
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.call("hipq_gemm_packed_i8_i32", a.data_ptr(), None, 4, 4, 16, out.data_ptr())
+    assert e.value.code == hipq.INVALID_ARGUMENT
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.call("hipq_gemm_packed_i8_i32", a.data_ptr(), a.data_ptr(), 4, 4, 1 << 17, out.data_ptr())
+    assert e.value.code == hipq.SHAPE_ERROR
+    with pytest.raises(hipq.HipqError) as e:  # packed operand of 2 GiB or more
+        ctx.call("hipq_gemm_packed_i8_i32", a.data_ptr(), a.data_ptr(), 1 << 20, 4, 4096, out.data_ptr())
+    assert e.value.code == hipq.SHAPE_ERROR
+    ctx.call("hipq_gemm_packed_i8_i32", a.data_ptr(), a.data_ptr(), 0, 4, 16, None)  # empty M: no-op

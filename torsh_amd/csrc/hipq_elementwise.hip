@@ -155,19 +155,20 @@ struct DynamicRange {
     int nparts;
     int flavor, qmin, qmax;
     hipq_qparams *out_params;
+    // Fused Linear forward: a range that is not finite (where the reference returns InvalidArgument,
+    // algorithms.rs:403-407) still has to leave defined operands for the GEMM that follows on the
+    // stream.  With `poison` set the published scale is NaN and every code 0, so every output of that
+    // GEMM is NaN and the status word says why; without it the kernel returns without writing codes.
+    int poison = 0;
 };
 
-// Per-tensor quantize.  Scale and zero point come from the launch arguments, from device
-// memory when `params` is non-null, or (dynamic quantization) from the range partials: then
-// every workgroup folds the same few hundred partials in the same order, derives the same
-// parameters, and workgroup 0 publishes them, which saves the launch of a finalize kernel.
-template <typename OutT, bool DIV, int RND>
-__global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restrict__ x, size_t n, float scale,
-                                                           int zp, const hipq_qparams *__restrict__ params,
-                                                           DynamicRange dyn, float lo, float hi,
-                                                           OutT *__restrict__ out) {
+// Folds the range partials of a dynamic quantize, derives the parameters (identically in every
+// workgroup) and lets workgroup 0 publish them; or takes the parameters from device memory; or records
+// the ones given by value.  Returns false when the element loop must not run.  `lds` holds
+// 2 * kBlock / kWave floats.
+__device__ __forceinline__ bool resolve_quantize_params(const DynamicRange &dyn, const hipq_qparams *params,
+                                                        float *lds, float &scale, int &zp) {
     if (dyn.partials) {
-        __shared__ float lds[2 * kBlock / kWave];
         MinMax m{INFINITY, -INFINITY};
         for (int i = threadIdx.x; i < dyn.nparts; i += kBlock) {
             const float2 p = dyn.partials[i];
@@ -176,16 +177,21 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
         }
         const MinMax r = block_minmax(m, lds);
         const int st = params_from_minmax(r.mn, r.mx, dyn.flavor, dyn.qmin, dyn.qmax, &scale, &zp);
+        const bool bad = st != HIPQ_SUCCESS;
         if (blockIdx.x == 0 && threadIdx.x == 0) {
-            dyn.out_params->scale = scale;
+            dyn.out_params->scale = (bad && dyn.poison) ? __builtin_nanf("") : scale;
             dyn.out_params->zero_point = zp;
             dyn.out_params->min_val = r.mn;
             dyn.out_params->max_val = r.mx;
             dyn.out_params->status = st;
         }
-        if (st != HIPQ_SUCCESS) return;  // the reference errors before quantizing
+        if (bad) {  // the reference errors before quantizing
+            if (!dyn.poison) return false;
+            scale = INFINITY;  // x * (1/inf) and x / inf: 0 for finite x, NaN -> code 0 otherwise
+            zp = 0;
+        }
     } else if (params) {
-        if (params->status != HIPQ_SUCCESS) return;
+        if (params->status != HIPQ_SUCCESS) return false;
         scale = params->scale;
         zp = params->zero_point;
     } else if (dyn.out_params && blockIdx.x == 0 && threadIdx.x == 0) {
@@ -196,6 +202,20 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
         dyn.out_params->max_val = 0.0f;
         dyn.out_params->status = HIPQ_SUCCESS;
     }
+    return true;
+}
+
+// Per-tensor quantize.  Scale and zero point come from the launch arguments, from device
+// memory when `params` is non-null, or (dynamic quantization) from the range partials: then
+// every workgroup folds the same few hundred partials in the same order, derives the same
+// parameters, and workgroup 0 publishes them, which saves the launch of a finalize kernel.
+template <typename OutT, bool DIV, int RND>
+__global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restrict__ x, size_t n, float scale,
+                                                           int zp, const hipq_qparams *__restrict__ params,
+                                                           DynamicRange dyn, float lo, float hi,
+                                                           OutT *__restrict__ out) {
+    __shared__ float range_lds[2 * kBlock / kWave];
+    if (!resolve_quantize_params(dyn, params, range_lds, scale, zp)) return;
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
     const float zpf = static_cast<float>(zp);
     const int ilo = static_cast<int>(lo), ihi = static_cast<int>(hi);
@@ -237,6 +257,53 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
     }
     for (size_t i = nvec * 4 + size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += size_t(gridDim.x) * kBlock)
         out[i] = to_out<OutT>(quantize_value<DIV, RND>(x[i], scale, inv, zpf, lo, hi));
+}
+
+// Per-tensor quantize of a matrix [rows, cols] straight into the fragment-packed operand layout of
+// the packed GEMM (32-row x 32-byte fragments of 1 KiB, lane l = row l%32, bytes 16*(l/32)..+15;
+// k blocks per row block padded to a multiple of 4).  One wave per fragment: a lane reads the 16
+// floats of its (row, half k block) as four 16-byte loads and writes its 16 codes as one 16-byte
+// store, so a wave reads 32 whole 128-byte lines and writes 1 KiB contiguous.  Rows and columns
+// past the matrix become code 0 (zero padding along K adds nothing to a dot product).
+template <bool DIV, int RND>
+__global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__restrict__ x, size_t rows,
+                                                                  size_t cols, float scale, int zp,
+                                                                  const hipq_qparams *__restrict__ params,
+                                                                  DynamicRange dyn, int8_t *__restrict__ out) {
+    __shared__ float range_lds[2 * kBlock / kWave];
+    if (!resolve_quantize_params(dyn, params, range_lds, scale, zp)) return;
+    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
+    const float zpf = static_cast<float>(zp);
+    const size_t KB = ((cols + 31) / 32 + 3) / 4 * 4;
+    const size_t nfrag = ((rows + 31) / 32) * KB;
+    const int lane = threadIdx.x % kWave;
+    const bool vec = (cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
+    for (size_t f = size_t(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave; f < nfrag;
+         f += size_t(gridDim.x) * (kBlock / kWave)) {
+        const size_t rb = f / KB, kb = f % KB;
+        const size_t row = rb * 32 + lane % 32, k0 = kb * 32 + 16 * (lane / 32);
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (row < rows && k0 < cols) {
+            const float *p = x + row * cols + k0;
+            if (vec && k0 + 16 <= cols) {
+                float4 v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(p)[i];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    w[i] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, zpf, -128, 127),
+                                 quantize_int<DIV, RND>(v[i].y, scale, inv, zpf, -128, 127),
+                                 quantize_int<DIV, RND>(v[i].z, scale, inv, zpf, -128, 127),
+                                 quantize_int<DIV, RND>(v[i].w, scale, inv, zpf, -128, 127));
+            } else {
+                for (int b = 0; b < 16; ++b)
+                    if (k0 + b < cols)
+                        w[b / 4] |= (uint32_t(quantize_int<DIV, RND>(p[b], scale, inv, zpf, -128, 127)) & 0xffu)
+                                    << (8 * (b % 4));
+            }
+        }
+        *reinterpret_cast<uint4 *>(out + f * 1024 + size_t(lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
 }
 
 template <typename InT>
@@ -309,7 +376,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
                                                                    int8_t *__restrict__ out,
                                                                    float *__restrict__ out_scales,
                                                                    int32_t *__restrict__ out_zps,
-                                                                   int32_t *__restrict__ out_status) {
+                                                                   int32_t *__restrict__ out_status, int poison) {
     constexpr int kRowsPerBlock = kBlock / TPR;
     constexpr int kCache = 4;
     __shared__ float lds[2 * kBlock / kWave];
@@ -362,12 +429,19 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     float scale;
     int zp;
     const int st = params_from_minmax(m.mn, m.mx, flavor, qmin, qmax, &scale, &zp);
+    const bool bad = st != HIPQ_SUCCESS;
     if (lane == 0) {
-        if (out_scales) out_scales[row] = scale;
+        // poison (fused Linear forward): a row whose range is not finite gets a NaN scale and zero codes,
+        // so that every output of that row is NaN instead of a product of stale scratch.
+        if (out_scales) out_scales[row] = (bad && poison) ? __builtin_nanf("") : scale;
         if (out_zps) out_zps[row] = zp;
-        if (st != HIPQ_SUCCESS && out_status) *out_status = st;
+        if (bad && out_status) *out_status = st;
     }
-    if (st != HIPQ_SUCCESS) return;
+    if (bad) {
+        if (!poison) return;
+        scale = INFINITY;  // x / inf: 0 for finite x, NaN -> code 0 otherwise
+        zp = 0;
+    }
     const float zpf = static_cast<float>(zp);
     const float inv = recip_for_div(scale);  // once per row; each element then divides with two FMAs
     uint32_t *q4 = reinterpret_cast<uint32_t *>(qr);
@@ -768,7 +842,7 @@ int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t *q, size_
 // HIPQ_PARAMS_* formula (the reference's per-channel function knows two).
 static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
                              int32_t flavor, bool any_flavor, int32_t qmin, int32_t qmax, int32_t mode, int8_t *out,
-                             float *out_scales, int32_t *out_zero_points, int32_t *out_status) {
+                             float *out_scales, int32_t *out_zero_points, int32_t *out_status, int poison = 0) {
     int32_t rc = any_flavor ? HIPQ_SUCCESS : check_row_flavor(fn, flavor);
     if (rc) return rc;
     if ((rc = check_mode(fn, mode))) return rc;
@@ -784,18 +858,18 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
         const int grid = static_cast<int>(rows);
         if (even)
             hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
         else
             hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
     } else {
         const int grid = static_cast<int>((rows + 3) / 4);
         if (even)
             hipLaunchKernelGGL((quantize_per_row_kernel<kWave, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
         else
             hipLaunchKernelGGL((quantize_per_row_kernel<kWave, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
+                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
     }
     return check_launch(fn);
 }
@@ -829,6 +903,52 @@ static int32_t quantize_channels(const char *fn, hipq_ctx *ctx, const float *x, 
                            outer, channels, inner, group, flavor, qmin, qmax, out, out_scales, out_zero_points,
                            out_status);
     return check_launch(fn);
+}
+
+// Activation quantizers of the fused Linear forwards (declared in hipq_internal.h).  A range that is
+// not finite poisons the operands (NaN scale, zero codes) instead of leaving stale scratch.
+int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, bool dynamic,
+                                              float static_scale, int32_t mode, bool packed, int8_t *out,
+                                              hipq_qparams *out_params, void *partials, size_t partials_bytes) {
+    const char *fn = "hipq_linear (activation quantize)";
+    int32_t rc = check_mode(fn, mode);
+    if (rc) return rc;
+    DynamicRange dyn{nullptr, 0, HIPQ_PARAMS_SYMMETRIC, -128, 127, out_params};
+    dyn.poison = 1;
+    float scale = 1.0f;
+    if (dynamic) {
+        rc = launch_minmax_partials(ctx, x, rows * cols, &dyn, static_cast<float2 *>(partials),
+                                    partials_bytes / sizeof(float2));
+        if (rc) return rc;
+    } else {
+        if ((rc = check_scale(fn, static_scale))) return rc;
+        scale = static_scale;
+    }
+    if (!packed) return launch_quantize<int8_t>(ctx, x, rows * cols, scale, 0, nullptr, mode, -128.0f, 127.0f, out, dyn);
+    const size_t KB = ((cols + 31) / 32 + 3) / 4 * 4, nfrag = ((rows + 31) / 32) * KB;
+    size_t blocks = (nfrag + 3) / 4;
+    const size_t cap = size_t(ctx->num_cus) * 8;
+    const int grid = static_cast<int>(blocks < cap ? blocks : cap);
+    const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+#define HIPQ_LAUNCH_QP(D, E)                                                                                       \
+    hipLaunchKernelGGL((quantize_packed_kernel<D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, rows, cols, scale, \
+                       0, static_cast<const hipq_qparams *>(nullptr), dyn, out)
+    if (div && even)
+        HIPQ_LAUNCH_QP(true, 1);
+    else if (div)
+        HIPQ_LAUNCH_QP(true, 0);
+    else if (even)
+        HIPQ_LAUNCH_QP(false, 1);
+    else
+        HIPQ_LAUNCH_QP(false, 0);
+#undef HIPQ_LAUNCH_QP
+    return check_launch("quantize (packed)");
+}
+
+int32_t hipq::quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
+                                           int8_t *out, float *out_scales) {
+    return quantize_rows("hipq_linear (activation quantize)", ctx, x, rows, cols, cols, HIPQ_PARAMS_SYMMETRIC, false,
+                         -128, 127, mode, out, out_scales, nullptr, nullptr, /*poison=*/1);
 }
 
 extern "C" {

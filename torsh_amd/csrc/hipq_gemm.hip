@@ -368,7 +368,7 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
 static int32_t check_gemm_shape(const char *fn, size_t m, size_t n, size_t k) {
     if ((m >> 30) || (n >> 30) || (k >> 30)) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", fn);
     // |acc| <= K * 128 * 128 must fit int32.
-    if (k > (size_t(1) << 17)) return fail(HIPQ_SHAPE_ERROR, "%s: K=%zu could overflow the int32 accumulator", fn, k);
+    if (k >= (size_t(1) << 17)) return fail(HIPQ_SHAPE_ERROR, "%s: K=%zu could overflow the int32 accumulator", fn, k);
     return HIPQ_SUCCESS;
 }
 
@@ -402,13 +402,11 @@ static int32_t linear_dynamic_on(hipq_ctx *ctx, char *base, const float *x, int3
     int8_t *qa = reinterpret_cast<int8_t *>(base + kScratchHeader + partial_bytes + linear_dynamic_scales_bytes(m));
     int32_t rc;
     if (per_token) {
-        rc = hipq_quantize_per_row_f32_i8(ctx, x, m, k, HIPQ_PARAMS_SYMMETRIC, mode & HIPQ_ROUND_HALF_EVEN, qa,
-                                          row_scales, nullptr, nullptr);
+        rc = quantize_activations_per_row(ctx, x, m, k, mode & HIPQ_ROUND_HALF_EVEN, qa, row_scales);
         if (rc) return rc;
         return hipq_linear_i8_f32(ctx, qa, row_scales, 1, w, w_scales, bias, m, n, k, out);
     }
-    rc = quantize_dynamic_per_tensor(ctx, x, m * k, HIPQ_PARAMS_SYMMETRIC, HIPQ_DTYPE_I8, mode, qa, params, partials,
-                                     partial_bytes);
+    rc = quantize_activations_per_tensor(ctx, x, m, k, true, 1.0f, mode, false, qa, params, partials, partial_bytes);
     if (rc) return rc;
     // hipq_qparams starts with the f32 scale.
     return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
@@ -574,7 +572,7 @@ int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_scale, con
     char *base = static_cast<char *>(s);
     hipq_qparams *params = reinterpret_cast<hipq_qparams *>(base);
     int8_t *qa = reinterpret_cast<int8_t *>(base + kScratchHeader);
-    rc = hipq_quantize_static_per_tensor_f32_i8(ctx, x, m * k, a_scale, 0, mode, qa, params);
+    rc = quantize_activations_per_tensor(ctx, x, m, k, false, a_scale, mode, false, qa, params, nullptr, 0);
     if (rc) return rc;
     return hipq_linear_i8_f32(ctx, qa, &params->scale, 0, w, w_scales, bias, m, n, k, out);
 }

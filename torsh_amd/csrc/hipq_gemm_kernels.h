@@ -305,6 +305,166 @@ __device__ __forceinline__ void wait_stages_outstanding(int stages) {
     }
 }
 
+// Sum of the K-split partial accumulators of a workgroup through LDS (integer adds: the result
+// does not depend on the order).  Row block i of a wave-group tile is owned by wave (i % WK) of
+// the group; every other wave of the group parks its partial for it.  Needs
+// (waves / WK) * FM * (WK - 1) * FN * 4 KiB of LDS at `lds`, free of other use by the time the
+// first wave arrives (LDS_BUSY: the main loop used it, so a workgroup barrier comes first).
+template <int FM, int FN, int WK, bool LDS_BUSY = true>
+__device__ __forceinline__ void ksplit_reduce(v16i (&acc)[FM][FN], int8_t *lds, int wk, int wmn, int lane) {
+    if constexpr (WK > 1) {
+        if constexpr (LDS_BUSY) __syncthreads();
+        v4i *red = reinterpret_cast<v4i *>(lds);
+        auto slot = [&](int i, int srcw, int j, int g) {
+            const int owner = i % WK;
+            const int sidx = (srcw - owner - 1 + WK) % WK;  // 0 .. WK-2
+            return ((((wmn * FM + i) * (WK - 1) + sidx) * FN + j) * 4 + g) * kWave + lane;
+        };
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if (i % WK == wk) continue;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    red[slot(i, wk, j, g)] =
+                        v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if (i % WK != wk) continue;
+#pragma unroll
+            for (int p = 1; p < WK; ++p) {
+                const int srcw = (wk + p) % WK;
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const v4i t = red[slot(i, srcw, j, g)];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] += t[r];
+                    }
+            }
+        }
+    }
+}
+
+// Dequantize / requantize / plain int32 epilogue of a wave's FM x FN grid of 32x32 accumulator
+// blocks whose first row is `mrow0` (row blocks not owned by K-split wave `wk` are skipped).
+// 32x32 accumulator block: lane holds column n = lane%32 and rows m = 8*(r/4) + 4*(lane/32) + r%4
+// for r = 0..15.  nn / swv / bv: the lane's output channel per column block, its weight scale and
+// bias; sa0: the per-tensor activation scale.
+template <int FM, int FN, int WK, int EPI, bool EVEN>
+__device__ __forceinline__ void store_tile(v16i (&acc)[FM][FN], const GemmEpilogue &ep, int M, int N, int mrow0,
+                                           int wk, int lane, const int (&nn)[FN], const float (&swv)[FN],
+                                           const float (&bv)[FN], float sa0) {
+    const float zpf = static_cast<float>(ep.zp_out);
+    const bool has_bias = ep.bias != nullptr;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        if (WK > 1 && i % WK != wk) continue;
+        // All loads of the row block first, then arithmetic and stores only: a load between
+        // stores would wait for every earlier store to retire (stores count in vmcnt too).
+        float s_row[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_row[r] = sa0;
+        if constexpr (EPI != EPI_I32) {
+            if (ep.sa_per_row) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = mrow0 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+                    s_row[r] = ep.sa[m < M ? m : M - 1];
+                }
+            }
+        }
+        // Combined scales for the whole row block, computed before the first store so that no
+        // loaded value is first touched between stores.
+        float s_comb[16][FN], res[16][FN];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                s_comb[r][j] = s_row[r] * swv[j];
+                res[r][j] = 0.0f;
+            }
+        if constexpr (EPI == EPI_F32) {
+            if (ep.residual) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = mrow0 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        if (m < M && nn[j] < N) res[r][j] = ep.residual[size_t(m) * N + nn[j]];
+                }
+            }
+        }
+        // Every load of this wave has landed (and the compiler's wait tracking knows it), so
+        // the stores below are issued back to back without waiting on one another.
+        wait_vmcnt<0>();
+        if constexpr (EPI == EPI_I8) {
+            // int8 output as dwords.  A lane holds one column of 16 rows; the four lanes of a quad
+            // hold four consecutive columns.  Per group of four rows each lane packs its four
+            // bytes, the quad transposes the 4x4 bytes (four quad broadcasts + two byte
+            // permutes), and every lane stores one dword = four consecutive columns of one row:
+            // a quarter of the store instructions of the byte form, none of them sub-dword.
+            if (N % 4 == 0 && (reinterpret_cast<uintptr_t>(ep.out) & 3u) == 0) {
+                const int qd = lane % 4;
+                const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
+                const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const int col = nn[j] - qd;  // first column of the quad; N % 4 == 0 keeps quads whole
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        int q[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            float v = static_cast<float>(acc[i][j][4 * t + k]) * s_comb[4 * t + k][j];
+                            if (has_bias) v = v + bv[j];
+                            q[k] = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
+                        }
+                        const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));  // byte k = row 8t + 4*(lane/32) + k
+                        const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
+                        const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
+                        const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
+                        const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
+                        const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                        const int m = mrow0 + i * 32 + 8 * t + 4 * (lane / 32) + qd;
+                        if (m < M && col < N)
+                            __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(static_cast<int8_t *>(ep.out) +
+                                                                                           size_t(m) * N + col));
+                    }
+                }
+                continue;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = mrow0 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+            if (m >= M) continue;
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                if (nn[j] >= N) continue;
+                const size_t off = size_t(m) * N + nn[j];
+                if constexpr (EPI == EPI_I32) {
+                    __builtin_nontemporal_store(acc[i][j][r], static_cast<int32_t *>(ep.out) + off);
+                } else {
+                    float v = static_cast<float>(acc[i][j][r]) * s_comb[r][j];
+                    if (has_bias) v = v + bv[j];
+                    if constexpr (EPI == EPI_F32) {
+                        if (ep.residual) v = v + res[r][j];
+                        __builtin_nontemporal_store(v, static_cast<float *>(ep.out) + off);
+                    } else {
+                        const int q = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
+                        __builtin_nontemporal_store(static_cast<int8_t>(q), static_cast<int8_t *>(ep.out) + off);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // PW producer waves do nothing but issue the fills; WM*WN*WK consumer waves do
 // nothing but LDS reads and MFMAs.  A wave issues in order, and a fill blocks its
 // wave while the texture path is busy, so mixing fills and MFMAs in one wave
@@ -530,49 +690,10 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     }
     if (kt < nk) iteration(kt, 0);
 
-    if constexpr (WK > 1) {
-        // Sum the K-split partials through LDS.  Row block i of a wave-group tile is owned
-        // by wave (i % WK); every other wave of the group parks its partial for it.
-        __syncthreads();
-        v4i *red = reinterpret_cast<v4i *>(lds);
-        auto slot = [&](int i, int srcw, int j, int g) {
-            const int owner = i % WK;
-            const int sidx = (srcw - owner - 1 + WK) % WK;  // 0 .. WK-2
-            return ((((wmn * FM + i) * (WK - 1) + sidx) * FN + j) * 4 + g) * kWave + lane;
-        };
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            if (i % WK == wk) continue;
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int g = 0; g < 4; ++g)
-                    red[slot(i, wk, j, g)] =
-                        v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            if (i % WK != wk) continue;
-#pragma unroll
-            for (int p = 1; p < WK; ++p) {
-                const int srcw = (wk + p) % WK;
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const v4i t = red[slot(i, srcw, j, g)];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] += t[r];
-                    }
-            }
-        }
-    }
-    // Epilogue.  32x32 accumulator block: lane holds column n = lane%32 and rows
-    // m = 8*(r/4) + 4*(lane/32) + r%4 for r = 0..15.
-    const float zpf = static_cast<float>(ep.zp_out);
-    const bool has_bias = ep.bias != nullptr;
+    if constexpr (WK > 1) ksplit_reduce<FM, FN, WK>(acc, lds, wk, wmn, lane);
     if constexpr (CONV) {
+        const float zpf = static_cast<float>(ep.zp_out);
+        const bool has_bias = ep.bias != nullptr;
         // Rows are output channels, columns are padded-grid window positions.  A lane owns one
         // window; consecutive lanes are consecutive ow, i.e. consecutive bytes of the NCHW output.
         const size_t plane = size_t(ep.cv_ho) * ep.cv_wo;
@@ -613,109 +734,8 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
                 }
             }
         }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        if (WK > 1 && i % WK != wk) continue;
-        // All loads of the row block first, then arithmetic and stores only: a load between
-        // stores would wait for every earlier store to retire (stores count in vmcnt too).
-        float s_row[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s_row[r] = sa0;
-        if constexpr (EPI != EPI_I32) {
-            if (ep.sa_per_row) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-                    s_row[r] = ep.sa[m < M ? m : M - 1];
-                }
-            }
-        }
-        // Combined scales for the whole row block, computed before the first store so that no
-        // loaded value is first touched between stores.
-        float s_comb[16][FN], res[16][FN];
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                s_comb[r][j] = s_row[r] * swv[j];
-                res[r][j] = 0.0f;
-            }
-        if constexpr (EPI == EPI_F32) {
-            if (ep.residual) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        if (m < M && nn[j] < N) res[r][j] = ep.residual[size_t(m) * N + nn[j]];
-                }
-            }
-        }
-        // Every load of this wave has landed (and the compiler's wait tracking knows it), so
-        // the stores below are issued back to back without waiting on one another.
-        wait_vmcnt<0>();
-        if constexpr (EPI == EPI_I8) {
-            // int8 output as dwords.  A lane holds one column of 16 rows; the four lanes of a quad
-            // hold four consecutive columns.  Per group of four rows each lane packs its four
-            // bytes, the quad transposes the 4x4 bytes (four quad broadcasts + two byte
-            // permutes), and every lane stores one dword = four consecutive columns of one row:
-            // a quarter of the store instructions of the byte form, none of them sub-dword.
-            if (N % 4 == 0 && (reinterpret_cast<uintptr_t>(ep.out) & 3u) == 0) {
-                const int qd = lane % 4;
-                const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
-                const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
-#pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    const int col = nn[j] - qd;  // first column of the quad; N % 4 == 0 keeps quads whole
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        int q[4];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            float v = static_cast<float>(acc[i][j][4 * t + k]) * s_comb[4 * t + k][j];
-                            if (has_bias) v = v + bv[j];
-                            q[k] = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
-                        }
-                        const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));  // byte k = row 8t + 4*(lane/32) + k
-                        const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
-                        const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
-                        const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
-                        const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
-                        const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
-                        const int m = m0 + wm * TM + i * 32 + 8 * t + 4 * (lane / 32) + qd;
-                        if (m < M && col < N)
-                            __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(static_cast<int8_t *>(ep.out) +
-                                                                                           size_t(m) * N + col));
-                    }
-                }
-                continue;
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-            if (m >= M) continue;
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                if (nn[j] >= N) continue;
-                const size_t off = size_t(m) * N + nn[j];
-                if constexpr (EPI == EPI_I32) {
-                    __builtin_nontemporal_store(acc[i][j][r], static_cast<int32_t *>(ep.out) + off);
-                } else {
-                    float v = static_cast<float>(acc[i][j][r]) * s_comb[r][j];
-                    if (has_bias) v = v + bv[j];
-                    if constexpr (EPI == EPI_F32) {
-                        if (ep.residual) v = v + res[r][j];
-                        __builtin_nontemporal_store(v, static_cast<float *>(ep.out) + off);
-                    } else {
-                        const int q = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
-                        __builtin_nontemporal_store(static_cast<int8_t>(q), static_cast<int8_t *>(ep.out) + off);
-                    }
-                }
-            }
-        }
+    } else {
+        store_tile<FM, FN, WK, EPI, EVEN>(acc, ep, M, N, m0 + wm * TM, wk, lane, nn, swv, bv, sa0);
     }
 }
 

@@ -1,0 +1,194 @@
+// Entry points of the fragment-packed int8 GEMM / Linear forward (kernels: hipq_gemm_packed.h).
+//
+// Weights are packed once when a layer is prepared (hipq_pack_rows_i8: the "MFMA-friendly tile
+// order" of a prepared weight blob); activations are written in the packed layout by the quantize
+// pass itself, so the forward costs no extra pass over either operand.
+#include "hipq_gemm_packed.h"
+
+namespace hipq {
+
+static int32_t check_packed_shape(const char *fn, size_t m, size_t n, size_t k) {
+    if ((m >> 30) || (n >> 30) || (k >> 30)) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", fn);
+    // |acc| <= K * 128 * 128 must fit int32.
+    if (k >= (size_t(1) << 17)) return fail(HIPQ_SHAPE_ERROR, "%s: K=%zu could overflow the int32 accumulator", fn, k);
+    // fragment offsets are 32-bit
+    if (packed_bytes(m, k) >= (size_t(1) << 31) || packed_bytes(n, k) >= (size_t(1) << 31))
+        return fail(HIPQ_SHAPE_ERROR, "%s: a packed operand of 2 GiB or more is not supported", fn);
+    return HIPQ_SUCCESS;
+}
+
+static int32_t pack_rows(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_t *dst) {
+    const size_t nfrag = packed_row_blocks(rows) * packed_k_blocks(k);
+    size_t blocks = (nfrag + 3) / 4;
+    const size_t cap = size_t(ctx->num_cus) * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(static_cast<int>(blocks)), dim3(256), 0, ctx->stream, src, rows, k, k,
+                       dst);
+    return check_launch("pack_rows_i8");
+}
+
+// Scratch of the fused forward: header (hipq_qparams), range partials, per-row scales, the packed
+// activations, and (per token only) the row-major codes the pack pass reads.
+struct PackedScratch {
+    size_t partials, scales, packed, rowmajor, total;
+};
+static PackedScratch packed_scratch_layout(int num_cus, size_t m, size_t k, bool per_token) {
+    PackedScratch L;
+    auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
+    L.partials = kScratchHeader;
+    L.scales = L.partials + up(size_t(num_cus) * 16 * sizeof(float2));
+    L.packed = L.scales + up(m * sizeof(float));
+    L.rowmajor = L.packed + up(packed_bytes(m, k));
+    L.total = L.rowmajor + (per_token ? up(m * k) : 0) + 256;
+    return L;
+}
+
+}  // namespace hipq
+
+using namespace hipq;
+
+extern "C" {
+
+int32_t hipq_packed_size(size_t rows, size_t k, size_t *out_bytes) {
+    HIPQ_REQUIRE_PTR(out_bytes);
+    if ((rows >> 30) || (k >> 30)) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    *out_bytes = packed_bytes(rows, k);
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_pack_rows_i8(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_t *dst_packed) {
+    HIPQ_ENTER(ctx);
+    if ((rows >> 30) || (k >> 30)) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    if (rows == 0 || k == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(src);
+    HIPQ_REQUIRE_PTR(dst_packed);
+    if (reinterpret_cast<uintptr_t>(dst_packed) & 15u)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: the packed buffer must be 16-byte aligned", __func__);
+    return pack_rows(ctx, src, rows, k, dst_packed);
+}
+
+int32_t hipq_gemm_packed_i8_i32(hipq_ctx *ctx, const int8_t *a_packed, const int8_t *w_packed, size_t m, size_t n,
+                                size_t k, int32_t *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_packed_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: K must be positive", __func__);
+    HIPQ_REQUIRE_PTR(out);
+    HIPQ_REQUIRE_PTR(a_packed);
+    HIPQ_REQUIRE_PTR(w_packed);
+    GemmEpilogue ep{nullptr, 0, nullptr, nullptr, 1.0f, 0, out};
+    return launch_gemm_packed<EPI_I32, false>(ctx, a_packed, w_packed, m, n, k, ep);
+}
+
+int32_t hipq_linear_packed_i8_f32(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                  int32_t a_scale_per_row, const int8_t *w_packed, const float *w_scales,
+                                  const float *bias, size_t m, size_t n, size_t k, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_packed_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: K must be positive", __func__);
+    HIPQ_REQUIRE_PTR(out);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(a_packed);
+    HIPQ_REQUIRE_PTR(w_packed);
+    GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, 1.0f, 0, out};
+    return launch_gemm_packed<EPI_F32, false>(ctx, a_packed, w_packed, m, n, k, ep);
+}
+
+int32_t hipq_linear_packed_i8_i8(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale, int32_t a_scale_per_row,
+                                 const int8_t *w_packed, const float *w_scales, const float *bias, size_t m, size_t n,
+                                 size_t k, float out_scale, int32_t out_zero_point, int32_t mode, int8_t *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_packed_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (out_scale <= 0.0f) return fail(HIPQ_INVALID_ARGUMENT, "%s: Scale must be positive", __func__);
+    if (mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV)) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", __func__);
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: K must be positive", __func__);
+    HIPQ_REQUIRE_PTR(out);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(a_packed);
+    HIPQ_REQUIRE_PTR(w_packed);
+    GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, out_scale, out_zero_point, out};
+    ep.s_out_inv = host_recip_for_div(out_scale);
+    if (mode & HIPQ_ROUND_HALF_EVEN) return launch_gemm_packed<EPI_I8, true>(ctx, a_packed, w_packed, m, n, k, ep);
+    return launch_gemm_packed<EPI_I8, false>(ctx, a_packed, w_packed, m, n, k, ep);
+}
+
+int32_t hipq_quantize_per_tensor_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
+                                               int32_t dynamic, float scale, int32_t mode, int8_t *out_packed,
+                                               hipq_qparams *out_params) {
+    HIPQ_ENTER(ctx);
+    if ((rows >> 30) || (cols >> 30)) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    if (rows == 0 || cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out_packed);
+    HIPQ_REQUIRE_PTR(out_params);
+    if (reinterpret_cast<uintptr_t>(out_packed) & 15u)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: the packed buffer must be 16-byte aligned", __func__);
+    return quantize_activations_per_tensor(ctx, x, rows, cols, dynamic != 0, scale, mode, true, out_packed, out_params,
+                                           nullptr, 0);
+}
+
+int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w_packed,
+                                       const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
+                                       int32_t mode, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_packed_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k, per_token != 0);
+    void *s = nullptr;
+    rc = scratch(ctx, L.total, &s);
+    if (rc) return rc;
+    char *base = static_cast<char *>(s);
+    hipq_qparams *params = reinterpret_cast<hipq_qparams *>(base);
+    float *row_scales = reinterpret_cast<float *>(base + L.scales);
+    int8_t *pa = reinterpret_cast<int8_t *>(base + L.packed);
+    if (per_token) {
+        int8_t *qa = reinterpret_cast<int8_t *>(base + L.rowmajor);
+        rc = quantize_activations_per_row(ctx, x, m, k, mode & HIPQ_ROUND_HALF_EVEN, qa, row_scales);
+        if (rc) return rc;
+        if ((rc = pack_rows(ctx, qa, m, k, pa))) return rc;
+        return hipq_linear_packed_i8_f32(ctx, pa, row_scales, 1, w_packed, w_scales, bias, m, n, k, out);
+    }
+    rc = quantize_activations_per_tensor(ctx, x, m, k, true, 1.0f, mode, true, pa, params, base + L.partials,
+                                         L.scales - L.partials);
+    if (rc) return rc;
+    return hipq_linear_packed_i8_f32(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out);
+}
+
+int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w_packed,
+                                      const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
+                                      int32_t mode, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_packed_shape(__func__, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k, false);
+    void *s = nullptr;
+    rc = scratch(ctx, L.total, &s);
+    if (rc) return rc;
+    char *base = static_cast<char *>(s);
+    hipq_qparams *params = reinterpret_cast<hipq_qparams *>(base);
+    int8_t *pa = reinterpret_cast<int8_t *>(base + L.packed);
+    rc = quantize_activations_per_tensor(ctx, x, m, k, false, a_scale, mode, true, pa, params, nullptr, 0);
+    if (rc) return rc;
+    return hipq_linear_packed_i8_f32(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out);
+}
+
+}  // extern "C"

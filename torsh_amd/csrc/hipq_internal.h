@@ -40,6 +40,14 @@ int32_t check_launch(const char *what);
 int32_t quantize_dynamic_per_tensor(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor, int32_t dtype,
                                     int32_t mode, void *out, hipq_qparams *out_params, void *partials,
                                     size_t partials_bytes);
+// Activation quantizers of the fused Linear forwards: symmetric int8, per tensor (dynamic range or a given
+// static scale; row-major or fragment-packed output) and per row (row-major).  A range that is not finite
+// gives a NaN scale and zero codes, so the GEMM that follows turns it into NaN outputs.
+int32_t quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, bool dynamic,
+                                        float static_scale, int32_t mode, bool packed, int8_t *out,
+                                        hipq_qparams *out_params, void *partials, size_t partials_bytes);
+int32_t quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
+                                     int8_t *out, float *out_scales);
 // Looks up, once per device, the address of the static device array behind
 // hipq_linear_dynamic_f32_noalloc; called by hipq_ctx_create with the device current.
 int32_t linear_noalloc_setup(int device);

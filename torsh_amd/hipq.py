@@ -106,6 +106,13 @@ _SIGNATURES = {
     "hipq_requantize_i32_i8": [_vp, _vp, _sz, _sz, _vp, _i32, _vp, _vp, _f32, _i32, _i32, _vp],
     "hipq_linear_dynamic_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_linear_dynamic_f32_noalloc": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
+    "hipq_pack_rows_i8": [_vp, _vp, _sz, _sz, _vp],
+    "hipq_gemm_packed_i8_i32": [_vp, _vp, _vp, _sz, _sz, _sz, _vp],
+    "hipq_linear_packed_i8_f32": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
+    "hipq_linear_packed_i8_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _f32, _i32, _i32, _vp],
+    "hipq_quantize_per_tensor_packed_f32_i8": [_vp, _vp, _sz, _sz, _i32, _f32, _i32, _vp, _vp],
+    "hipq_linear_dynamic_packed_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
+    "hipq_linear_static_packed_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_quantize_per_row_strided_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
     "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
@@ -140,6 +147,7 @@ _SPECIAL = {
     "hipq_has_error": (_i32, []),
     "hipq_ctx_stream": (_vp, [_vp]),
     "hipq_transformer_stack_workspace_bytes": (_sz, [_sz, _sz, _sz]),
+    "hipq_packed_size": (_i32, [_sz, _sz, C.POINTER(C.c_size_t)]),
 }
 
 
@@ -508,6 +516,62 @@ class Context:
         out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
         self.call("hipq_linear_dynamic_f32", _ptr(x), int(per_token), _ptr(w), _ptr(w_scales), _ptr(bias), m, n, k,
                   mode, _ptr(out))
+        return out
+
+    # ---- fragment-packed operands ------------------------------------------------------
+    def packed_size(self, rows: int, k: int) -> int:
+        n = C.c_size_t(0)
+        _check(self._lib.hipq_packed_size(rows, k, C.byref(n)))
+        return int(n.value)
+
+    def pack_rows(self, q: torch.Tensor, out=None) -> torch.Tensor:
+        """int8 [rows, k] -> the packed operand of the fast GEMM (a flat int8 buffer)."""
+        rows, k = q.shape
+        out = out if out is not None else torch.empty(self.packed_size(rows, k), dtype=torch.int8, device=self._dev())
+        self.call("hipq_pack_rows_i8", _ptr(q), rows, k, _ptr(out))
+        return out
+
+    def gemm_packed_i8_i32(self, a_packed, w_packed, m, n, k, out=None):
+        out = out if out is not None else torch.empty((m, n), dtype=torch.int32, device=self._dev())
+        self.call("hipq_gemm_packed_i8_i32", _ptr(a_packed), _ptr(w_packed), m, n, k, _ptr(out))
+        return out
+
+    def linear_packed_i8_f32(self, a_packed, a_scale, w_packed, w_scales, bias, m, n, k, out=None):
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_packed_i8_f32", _ptr(a_packed), _ptr(a_scale), int(a_scale.numel() > 1), _ptr(w_packed),
+                  _ptr(w_scales), _ptr(bias), m, n, k, _ptr(out))
+        return out
+
+    def linear_packed_i8_i8(self, a_packed, a_scale, w_packed, w_scales, bias, m, n, k, out_scale, out_zp, mode=0):
+        out = torch.empty((m, n), dtype=torch.int8, device=self._dev())
+        self.call("hipq_linear_packed_i8_i8", _ptr(a_packed), _ptr(a_scale), int(a_scale.numel() > 1), _ptr(w_packed),
+                  _ptr(w_scales), _ptr(bias), m, n, k, float(out_scale), int(out_zp), mode, _ptr(out))
+        return out
+
+    def quantize_per_tensor_packed(self, x, dynamic=True, scale=1.0, mode=0, out=None, params=None):
+        """Symmetric per-tensor int8 quantize of fp32 [rows, cols] into the packed layout -> (packed, params)."""
+        rows, cols = x.shape
+        out = out if out is not None else torch.empty(self.packed_size(rows, cols), dtype=torch.int8,
+                                                      device=self._dev())
+        params = params if params is not None else self.new_qparams()
+        self.call("hipq_quantize_per_tensor_packed_f32_i8", _ptr(x), rows, cols, int(dynamic), float(scale), mode,
+                  _ptr(out), _ptr(params))
+        return out, params
+
+    def linear_dynamic_packed(self, x, w_packed, w_scales, bias=None, per_token=False, mode=0, out=None):
+        m, k = x.shape
+        n = w_scales.numel()
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_dynamic_packed_f32", _ptr(x), int(per_token), _ptr(w_packed), _ptr(w_scales), _ptr(bias),
+                  m, n, k, mode, _ptr(out))
+        return out
+
+    def linear_static_packed(self, x, a_scale, w_packed, w_scales, bias=None, mode=0, out=None):
+        m, k = x.shape
+        n = w_scales.numel()
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_static_packed_f32", _ptr(x), float(a_scale), _ptr(w_packed), _ptr(w_scales), _ptr(bias),
+                  m, n, k, mode, _ptr(out))
         return out
 
     def linear_dynamic_noalloc(self, x, w, w_scales, bias=None, per_token=False, mode=0, out=None):
