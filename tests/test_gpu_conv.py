@@ -106,6 +106,37 @@ def test_config4_full_size_against_direct_kernel_and_torch(ctx, hipq):
         assert torch.equal(acc, ref.to(torch.int32))
 
 
+def test_config4_full_size_packed_requant_forward(ctx, hipq):
+    """BASELINE configs[3] at full size through the entry point the bench times (layout pass, packed filters,
+    implicit GEMM, fused bias + requantize): every int8 output against the bytes re-derived, with torch's
+    individually rounded f32 operations, from exact accumulators (float64 convolution, |acc| < 2^53); both
+    roundings, a zero and a non-zero input zero point."""
+    g = torch.Generator(device="cuda").manual_seed(9)
+    nb, c, h, w_, oc = 32, 256, 14, 14, 256
+    x = torch.randint(0, 256, (nb, c, h, w_), generator=g, device="cuda", dtype=torch.uint8)
+    wq = torch.randint(-128, 128, (oc, c, 3, 3), generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(oc, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(oc, generator=g, device="cuda") * 0.01
+    packed, sums = ctx.conv2d_pack_weights(wq)
+    s_in, s_out = 0.02, 0.37
+    for zp_in, zp_out in ((0, 0), (37, -5)):
+        acc = torch.nn.functional.conv2d(torch.nn.functional.pad(x.double() - zp_in, (1, 1, 1, 1)), wq.double())
+        assert torch.equal(ctx.conv2d_i32(x, zp_in, wq, (1, 1), (1, 1)), acc.to(torch.int32))
+        # acc as f32 * (s_in * s_w[oc]) + bias[oc], then round(v / s_out) + zp_out clamped: operations.rs:722-728
+        s_comb = (torch.tensor(s_in, device="cuda", dtype=torch.float32) * sw)[None, :, None, None]
+        v = acc.float() * s_comb + bias[None, :, None, None]
+        t = v / torch.tensor(s_out, device="cuda", dtype=torch.float32)
+        for mode, rounded in ((hipq.ROUND_HALF_AWAY, torch.trunc(t + torch.copysign(torch.full_like(t, 0.5), t))),
+                              (hipq.ROUND_HALF_EVEN, torch.round(t))):
+            if mode == hipq.ROUND_HALF_AWAY:  # trunc(t + 0.5) is f32::round except just below 0.5
+                assert not bool(((t.abs() > 0.4999999) & (t.abs() < 0.5)).any())
+            want = torch.clamp(rounded + zp_out, -128, 127).to(torch.int8)
+            got = ctx.conv2d_i8_packed(x, zp_in, s_in, packed, sums, (3, 3), sw, bias, s_out, zp_out, (1, 1), mode)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want)
+            assert torch.equal(ctx.conv2d_i8(x, zp_in, s_in, wq, sw, bias, s_out, zp_out, (1, 1), (1, 1), mode), want)
+
+
 def test_conv_error_cases(ctx, hipq):
     x = torch.zeros((1, 4, 5, 5), dtype=torch.uint8, device="cuda")
     w = torch.zeros((2, 3, 3, 3), dtype=torch.int8, device="cuda")

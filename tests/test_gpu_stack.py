@@ -157,6 +157,62 @@ def test_projection_stack_small(ctx, hipq, oracle, tokens, d, dff, layers):
     assert rel < 2e-3
 
 
+@pytest.mark.parametrize("tokens,d,dff,layers", [(130, 256, 1024, 2)])
+def test_projection_stack_integer_steps_are_exact_on_the_device_operands(ctx, hipq, oracle, tokens, d, dff, layers):
+    """The end-to-end drift above comes from fp32 LayerNorm / GELU rounding only.  Here every quantize and every
+    GEMM inside the stack is checked on the DEVICE's own fp32 inputs: the per-token codes and scales of the
+    device's LayerNorm / GELU output equal the oracle's quantization of that same output, each int32 GEMM equals
+    the oracle GEMM of the device's int8 operands, each fp32 Linear output equals the oracle epilogue of those
+    accumulators (with the residual added after the bias), and the whole chain equals the one-call stack."""
+    rng = np.random.default_rng(tokens * 3 + d)
+    blocks_h = _make_blocks(rng, layers, d, dff, oracle)
+    for blk in blocks_h:  # non-trivial affine parameters
+        for ln in ("ln1", "ln2"):
+            blk[ln + "_gamma"] = rng.uniform(0.5, 1.5, d).astype(np.float32)
+            blk[ln + "_beta"] = (rng.standard_normal(d) * 0.1).astype(np.float32)
+    x_h = rng.standard_normal((tokens, d)).astype(np.float32)
+    blocks_d = [{k: dev(v) for k, v in blk.items()} for blk in blocks_h]
+    got = host(ctx.stack_forward(blocks_d, dev(x_h), dff, ctx.stack_workspace(tokens, d, dff)))
+
+    def check_quantizer(h_dev, q_dev, s_dev):
+        q, sa, _ = oracle.quantize_per_channel_auto(host(h_dev), 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+        np.testing.assert_array_equal(host(q_dev), q.astype(np.int8))
+        np.testing.assert_array_equal(host(s_dev), sa)
+
+    def checked_linear(q_dev, s_dev, blk_h, blk_d, name, residual=None):
+        w, sw, b = blk_h["w_" + name], blk_h["s_" + name], blk_h["b_" + name]
+        acc = oracle.gemm_i8_nk(host(q_dev), w)
+        np.testing.assert_array_equal(host(ctx.gemm_i8_i32(q_dev, blk_d["w_" + name])), acc)
+        want = oracle.linear_dequant_epilogue(acc, host(s_dev), sw, b)
+        if residual is None:
+            out = ctx.linear_i8_f32(q_dev, s_dev, blk_d["w_" + name], blk_d["s_" + name], blk_d["b_" + name])
+        else:
+            want = want + host(residual)  # one more individually rounded f32 addition
+            out = ctx.linear_i8_f32_residual(q_dev, s_dev, blk_d["w_" + name], blk_d["s_" + name], blk_d["b_" + name],
+                                             residual)
+        np.testing.assert_array_equal(host(out), want)
+        return out
+
+    x = dev(x_h)
+    for blk_h, blk_d in zip(blocks_h, blocks_d):
+        h = ctx.layer_norm(x, blk_d["ln1_gamma"], blk_d["ln1_beta"], 1e-5)
+        q, s = ctx.layer_norm_quantize(x, blk_d["ln1_gamma"], blk_d["ln1_beta"], 1e-5)
+        check_quantizer(h, q, s)
+        qkv = checked_linear(q, s, blk_h, blk_d, "qkv")
+        q, s = ctx.quantize_per_row_strided(qkv, tokens, d, 3 * d, elem_offset=2 * d)
+        check_quantizer(qkv[:, 2 * d:3 * d].contiguous(), q, s)
+        x = checked_linear(q, s, blk_h, blk_d, "out", residual=x)
+        h = ctx.layer_norm(x, blk_d["ln2_gamma"], blk_d["ln2_beta"], 1e-5)
+        q, s = ctx.layer_norm_quantize(x, blk_d["ln2_gamma"], blk_d["ln2_beta"], 1e-5)
+        check_quantizer(h, q, s)
+        f = checked_linear(q, s, blk_h, blk_d, "fc1")
+        a = ctx.gelu_tanh(f)
+        q, s = ctx.gelu_tanh_quantize(f)
+        check_quantizer(a, q, s)
+        x = checked_linear(q, s, blk_h, blk_d, "fc2", residual=x)
+    np.testing.assert_array_equal(got, host(x))
+
+
 def test_stack_workspace_too_small_is_rejected(ctx, hipq):
     x = torch.zeros((8, 128), device="cuda")
     ws = torch.empty(1024, dtype=torch.uint8, device="cuda")

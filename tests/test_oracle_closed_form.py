@@ -280,6 +280,38 @@ def test_layer_norm_and_gelu(oracle):
     np.testing.assert_allclose(g, [0.0, 0.841192, -0.158808, 2.996363], atol=1e-6)
 
 
+def test_layer_norm_with_affine_parameters_and_large_eps(oracle):
+    """crates/torsh-nn/src/layers/normalization/common.rs:389-404: (x - mean) / sqrt(var + eps) * weight + bias with
+    the biased variance.  Random gamma and beta and an eps of the size of the variance, so that a dropped beta,
+    gamma applied after beta, eps outside the square root or the unbiased variance would each miss by far more
+    than the tolerance; a hand-computed row on top."""
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((5, 48)) * rng.uniform(0.5, 3.0, (5, 1)) + rng.uniform(-2, 2, (5, 1))).astype(np.float32)
+    gamma = rng.uniform(0.5, 2.0, 48).astype(np.float32)
+    beta = rng.uniform(-1.0, 1.0, 48).astype(np.float32)
+    for eps in (0.5, 1e-5):
+        x64 = x.astype(np.float64)
+        mean = x64.mean(axis=1, keepdims=True)
+        var = ((x64 - mean) ** 2).mean(axis=1, keepdims=True)          # biased: divides by the row length
+        want = (x64 - mean) / np.sqrt(var + eps) * gamma.astype(np.float64) + beta.astype(np.float64)
+        np.testing.assert_allclose(oracle.layer_norm(x, gamma, beta, eps), want, rtol=2e-6, atol=2e-6)
+        np.testing.assert_allclose(oracle.layer_norm(x, gamma, None, eps), want - beta, rtol=2e-6, atol=2e-6)
+        np.testing.assert_allclose(oracle.layer_norm(x, None, beta, eps),
+                                   (x64 - mean) / np.sqrt(var + eps) + beta, rtol=2e-6, atol=2e-6)
+    # the wrong formulas really are far away at eps = 0.5 (the check above is not vacuous)
+    x64 = x.astype(np.float64)
+    mean = x64.mean(axis=1, keepdims=True)
+    var = ((x64 - mean) ** 2).mean(axis=1, keepdims=True)
+    good = (x64 - mean) / np.sqrt(var + 0.5) * gamma + beta
+    for wrong in ((x64 - mean) / (np.sqrt(var) + 0.5) * gamma + beta,              # eps outside the square root
+                  ((x64 - mean) / np.sqrt(var + 0.5) + beta) * gamma,              # gamma after beta
+                  (x64 - mean) / np.sqrt(var * 48 / 47 + 0.5) * gamma + beta):     # unbiased variance
+        assert np.abs(wrong - good).max() > 1e-2
+    # by hand: row [1, 2, 3, 6]: mean 3, biased variance 3.5, eps 0.5 -> divide by 2
+    y = oracle.layer_norm(np.float32([[1, 2, 3, 6]]), np.float32([1, 2, 3, 4]), np.float32([0.5, 0.5, -1, 0]), 0.5)
+    np.testing.assert_allclose(y, [[-0.5, -0.5, -1.0, 6.0]], rtol=0, atol=1e-6)
+
+
 def test_determinism(oracle):
     rng = np.random.default_rng(12)
     x = rng.standard_normal(100_000).astype(np.float32)
