@@ -110,6 +110,8 @@ HIPQ_API int32_t hipq_ctx_create(int32_t device, hipq_ctx **out_ctx);
  * legacy default stream). */
 HIPQ_API int32_t hipq_ctx_create_on_stream(int32_t device, void *hip_stream, hipq_ctx **out_ctx);
 HIPQ_API int32_t hipq_ctx_destroy(hipq_ctx *ctx);
+/* Waits for the context's stream.  Also returns HIPQ_DEVICE_ERROR (once) if a kernel since the last
+ * synchronize gave up on one of its bounded waits: its outputs are then invalid. */
 HIPQ_API int32_t hipq_ctx_synchronize(hipq_ctx *ctx);
 HIPQ_API void *hipq_ctx_stream(hipq_ctx *ctx);
 
@@ -287,10 +289,16 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
                                         const float *bias, float out_scale, int32_t out_zero_point,
                                         int32_t mode, int8_t *out);
 /* Test and tuning hook with no counterpart in the reference: forces one of the GEMM kernel forms
- * for every later call of this process wherever the shape allows it (0 = automatic choice, the
+ * for every later call on this context wherever the shape allows it (0 = automatic choice, the
  * default; 1-3 one-tile-per-workgroup forms, 5-8 persistent forms, 10 register-staged form).
  * Results do not depend on it; the parity tests use it to run every form on the same inputs. */
-HIPQ_API int32_t hipq_set_gemm_kernel_variant(int32_t variant);
+HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
+/* Test hook with no counterpart in the reference.  The persistent GEMM kernel couples its waves
+ * through counters and bounds every wait, so that a grid always drains; a wait that gives up
+ * marks the context, and the next hipq_ctx_synchronize returns HIPQ_DEVICE_ERROR once instead of
+ * handing back a wrong product silently.  `limit` is the number of polls after the first look
+ * (negative = the default, 2^20); 0 lets a test see the error path without hanging anything. */
+HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
 /* Whole forward of a quantized Linear with a static (calibrated) activation scale: the scale an
  * observer derived beforehand (Observer::calculate_qparams, crates/torsh-quantization/src/observers.rs:263-310,
  * symmetric: zero point 0) instead of a range pass over every input - per-tensor quantize

@@ -299,6 +299,31 @@ def test_every_gemm_kernel_form_gives_the_same_bits(ctx, hipq, oracle, variant):
         ctx.set_gemm_kernel_variant(99)
 
 
+def test_a_wait_that_gives_up_is_reported_not_swallowed(hipq, oracle):
+    """The persistent kernel bounds every wait so that its grid always drains.  With the spin limit forced to 0
+    the consumer waves do not wait for the first K-tile (a wait that is certain to be needed: the fills need a
+    memory round trip), run on and finish normally with a wrong product; the context must then report
+    HIPQ_DEVICE_ERROR at the next synchronize, once, and work normally again afterwards."""
+    c = hipq.Context(0)
+    try:
+        rng = np.random.default_rng(5)
+        a, w = rand_i8(rng, (1024, 512)), rand_i8(rng, (768, 512))
+        da, dw = dev(a), dev(w)
+        c.set_gemm_kernel_variant(7)  # a persistent form
+        c.set_wait_spin_limit(0)
+        c.gemm_i8_i32(da, dw)
+        with pytest.raises(hipq.HipqError) as e:
+            c.synchronize()
+        assert e.value.code == hipq.DEVICE_ERROR and "gave up" in str(e.value)
+        c.synchronize()  # reported once, then cleared
+        c.set_wait_spin_limit(-1)
+        got = c.gemm_i8_i32(da, dw)
+        c.synchronize()
+        np.testing.assert_array_equal(got.cpu().numpy(), oracle.gemm_i8_nk(a, w))
+    finally:
+        c.close()
+
+
 def test_output_larger_than_four_gib(ctx, hipq, oracle):
     """[32768, 128] x [32768, 128]^T: the fp32 / int32 output is 4 GiB, so byte offsets into it pass 2^32.  Both
     operands are a 512-row block repeated 64 times; every 512 x 512 block of the output must equal the oracle's

@@ -103,7 +103,15 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
     void *p = nullptr;
     int32_t rc = hipq::linear_noalloc_setup(device);
     if (rc == HIPQ_SUCCESS) rc = hipq::scratch(ctx, size_t(8) << 20, &p);
+    if (rc == HIPQ_SUCCESS) {
+        e = hipMalloc(reinterpret_cast<void **>(&ctx->wait_error), 256);
+        if (e == hipSuccess) e = hipMemset(ctx->wait_error, 0, 256);
+        if (e != hipSuccess)
+            rc = hipq::fail(HIPQ_ALLOCATION_ERROR, "hipq_ctx_create: status word: %s", hipGetErrorString(e));
+    }
     if (rc != HIPQ_SUCCESS) {
+        if (ctx->wait_error) (void)hipFree(ctx->wait_error);
+        if (ctx->scratch) (void)hipFree(ctx->scratch);
         if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return rc;
@@ -126,6 +134,7 @@ int32_t hipq_ctx_destroy(hipq_ctx *ctx) {
     HIPQ_ENTER(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->wait_error) (void)hipFree(ctx->wait_error);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return HIPQ_SUCCESS;
@@ -136,6 +145,31 @@ int32_t hipq_ctx_synchronize(hipq_ctx *ctx) {
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess)
         return hipq::fail(HIPQ_SYNCHRONIZATION_ERROR, "hipq_ctx_synchronize: %s", hipGetErrorString(e));
+    // A kernel whose bounded wait gave up has finished (every kernel drains) but its result is not the
+    // product that was asked for: report it here, once, and clear the word.
+    uint32_t gave_up = 0;
+    HIPQ_HIP(hipMemcpy(&gave_up, ctx->wait_error, sizeof(gave_up), hipMemcpyDeviceToHost));
+    if (gave_up) {
+        HIPQ_HIP(hipMemset(ctx->wait_error, 0, sizeof(gave_up)));
+        return hipq::fail(HIPQ_DEVICE_ERROR,
+                          "hipq_ctx_synchronize: a bounded wait inside the persistent GEMM kernel gave up "
+                          "(spin limit %d); results of the GEMM calls since the last synchronize are invalid",
+                          ctx->wait_spin_limit);
+    }
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant) {
+    HIPQ_REQUIRE_PTR(ctx);
+    if (variant < 0 || variant > 10)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..10", __func__, variant);
+    ctx->gemm_variant = variant;
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit) {
+    HIPQ_REQUIRE_PTR(ctx);
+    ctx->wait_spin_limit = limit < 0 ? (1 << 20) : limit;
     return HIPQ_SUCCESS;
 }
 

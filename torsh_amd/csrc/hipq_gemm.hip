@@ -287,15 +287,16 @@ static void launch_tile(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, 
                        ctx->stream, a, w, M, N, K, placed);
 }
 
-// Tuning and test hook: HIPQ_GEMM_VARIANT=<n> in the environment, or hipq_set_gemm_kernel_variant(n),
-// forces one kernel configuration wherever the shape allows it (0 = automatic).
-static int g_gemm_variant = -1;
-static int gemm_variant_override() {
-    if (g_gemm_variant < 0) {
+// Tuning and test hook, per context: HIPQ_GEMM_VARIANT=<n> in the environment (read when a context first
+// runs a GEMM), or hipq_set_gemm_kernel_variant(ctx, n), forces one kernel configuration wherever the shape
+// allows it (0 = automatic).
+static int gemm_variant_override(hipq_ctx *ctx) {
+    if (ctx->gemm_variant < 0) {
         const char *e = getenv("HIPQ_GEMM_VARIANT");
-        g_gemm_variant = e ? atoi(e) : 0;
+        const int v = e ? atoi(e) : 0;
+        ctx->gemm_variant = (v >= 0 && v <= 10) ? v : 0;
     }
-    return g_gemm_variant;
+    return ctx->gemm_variant;
 }
 
 template <int EPI, bool EVEN>
@@ -314,7 +315,7 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
     }
     const size_t cus = static_cast<size_t>(ctx->num_cus);
     auto tiles = [&](size_t bm, size_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    int variant = gemm_variant_override();
+    int variant = gemm_variant_override(ctx);
     if (variant == 0 && M <= 16 && K % 256 == 0) return launch_gemv<EPI, EVEN>(ctx, a, w, M, N, K, ep);
     const bool pipe_ok = (K % 128 == 0) && K >= 256;
     if (variant == 0 && pipe_ok) {
@@ -547,12 +548,6 @@ int32_t hipq_linear_dynamic_f32_noalloc(hipq_ctx *ctx, const float *x, int32_t p
         return fail(HIPQ_SHAPE_ERROR, "%s: scratch layout does not fit the static array", __func__);
     return linear_dynamic_on(ctx, static_cast<char *>(g_noalloc_ptr[ctx->device]), x, per_token, w, w_scales, bias, m,
                              n, k, mode, out);
-}
-
-int32_t hipq_set_gemm_kernel_variant(int32_t variant) {
-    if (variant < 0 || variant > 10) return fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..10", __func__, variant);
-    g_gemm_variant = variant;
-    return HIPQ_SUCCESS;
 }
 
 int32_t hipq_linear_static_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w, const float *w_scales,

@@ -35,6 +35,10 @@ struct GemmEpilogue {
     // Tiles per XCD along M and N (pipelined kernel): the 8 XCDs each take a gm x gn rectangle of
     // tiles.  0 = not set (plain id order).
     int xcd_gm = 0, xcd_gn = 0;
+    // Persistent kernel: how often a bounded wait polls before it gives up, and the device word
+    // (owned by the context) in which a give-up is recorded.
+    int spin_limit = 1 << 20;
+    uint32_t *wait_error = nullptr;
 };
 
 // Host-side twin of recip_for_div: the correctly rounded 1/b if it is a normal number, else 0.

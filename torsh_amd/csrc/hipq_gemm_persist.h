@@ -19,8 +19,10 @@
 //               registers;  buffer b may be refilled for the f-th time when empty[b] == CW * f.
 // A wave's LDS operations execute in order, and a fill's data is in LDS before vmcnt counts it,
 // so "counter seen" implies "data visible".  Every wait is a bounded spin: if a counter never
-// arrives (which would be a bug), the wave gives up after kSpinLimit polls and runs on, so the
-// grid always drains.
+// arrives (which would be a bug), the wave gives up after the spin limit, records that in a
+// device word of the context (GemmEpilogue::wait_error) and runs on, so the grid always drains;
+// the next hipq_ctx_synchronize reports the give-up as HIPQ_DEVICE_ERROR instead of returning a
+// wrong product silently.
 //
 // Tile order: tile t -> (t % tiles_m, t / tiles_m).  With 256 workgroups and tiles_m a multiple
 // of 64 a workgroup keeps one band of activation rows for its whole life and walks the weight
@@ -34,7 +36,12 @@
 
 namespace hipq {
 
-constexpr int kSpinLimit = 1 << 20;
+constexpr int kSpinLimit = 1 << 20;  // default of hipq_ctx::wait_spin_limit
+
+struct WaitPolicy {
+    int spin_limit;
+    uint32_t *error_word;  // device memory; set to 1 when a wait gives up
+};
 
 // The queue counters live in LDS.  They are read through an explicit LDS-address-space volatile
 // pointer: a volatile access through a generic pointer is compiled to a flat load, which waits
@@ -45,13 +52,21 @@ __device__ __forceinline__ uint32_t read_counter(const uint32_t *counter) {
     return *(lds_counter_t *)counter;
 }
 
-// Spins until *counter >= target (wave-uniform) or the spin limit is reached.
-__device__ __forceinline__ void wait_counter(const uint32_t *counter, uint32_t target) {
-    for (int spin = 0; spin < kSpinLimit; ++spin) {
+// Spins until *counter >= target (wave-uniform), polling at most spin_limit more times after the
+// first look; a wait that gives up is recorded in the policy's error word (one plain vector store).
+__device__ __forceinline__ void wait_counter(const uint32_t *counter, uint32_t target, const WaitPolicy &wp,
+                                             int lane) {
+    bool reached = false;
+    for (int spin = 0;; ++spin) {
         const uint32_t v = __builtin_amdgcn_readfirstlane(read_counter(counter));
-        if (static_cast<int32_t>(v - target) >= 0) break;
+        if (static_cast<int32_t>(v - target) >= 0) {
+            reached = true;
+            break;
+        }
+        if (spin >= wp.spin_limit) break;
         __builtin_amdgcn_s_sleep(1);
     }
+    if (!reached && wp.error_word && lane == 0) *reinterpret_cast<volatile uint32_t *>(wp.error_word) = 1u;
     asm volatile("" ::: "memory");  // nothing that follows may be moved above the wait
 }
 
@@ -99,6 +114,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                          static_cast<int>(gridDim.x);
     const int T = my_tiles * nk;  // K-tiles this workgroup streams, in consumption order
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const WaitPolicy wp{ep.spin_limit, ep.wait_error};
 
     if (tid < 2 * STAGES) full[tid] = 0;
     __syncthreads();  // the only workgroup barrier: counters are zero before anyone uses them
@@ -142,7 +158,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                 // The ring is full.  Nothing is lost by waiting for the fills in flight, and the
                 // consumers may be waiting for exactly those reports.
                 while (unreported > 0) report_oldest();
-                wait_counter(empty + buf, uint32_t(CW) * fill);  // consumers are done with the old contents
+                wait_counter(empty + buf, uint32_t(CW) * fill, wp, lane);  // consumers are done with the old contents
             }
             int8_t *base = lds + buf * STAGE + wave * (IPW * 1024);
             const size_t koff = size_t(kt_issue) * BK;
@@ -223,7 +239,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
                     // back with the fragments); only if it had not arrived by then is it polled.
                     const uint32_t want = uint32_t(PW) * (nxt_fill + 1);
                     if (static_cast<int32_t>(__builtin_amdgcn_readfirstlane(full_seen) - want) < 0) {
-                        wait_counter(full + nxt_buf, want);  // next K-tile has landed
+                        wait_counter(full + nxt_buf, want, wp, lane);  // next K-tile has landed
                     }
                     read_group(nxt_buf, 0, set ^ 1);
                 }
@@ -253,7 +269,7 @@ __global__ __launch_bounds__((PW + WM * WN) * kWave) void gemm_i8_persist_kernel
 
     const float zpf = static_cast<float>(ep.zp_out);
     const bool has_bias = ep.bias != nullptr;
-    wait_counter(full + 0, uint32_t(PW));  // first K-tile has landed
+    wait_counter(full + 0, uint32_t(PW), wp, lane);  // first K-tile has landed
     read_group(0, 0, 0);
     if (T > 1) full_seen = read_counter(full + nxt_buf);
 
@@ -556,7 +572,10 @@ static int32_t launch_persist(hipq_ctx *ctx, const int8_t *a, const int8_t *w, i
     if (EPI != EPI_I32 && (!ep.sa || !ep.sw)) return fail(HIPQ_INVALID_ARGUMENT, "gemm_i8 (persistent): scales must be given");
     const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     const int grid = tiles < ctx->num_cus ? tiles : ctx->num_cus;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), kLds, ctx->stream, a, w, M, N, K, ep);
+    GemmEpilogue placed = ep;
+    placed.wait_error = ctx->wait_error;
+    placed.spin_limit = ctx->wait_spin_limit;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), kLds, ctx->stream, a, w, M, N, K, placed);
     return check_launch("gemm_i8 (persistent)");
 }
 

@@ -19,6 +19,12 @@ struct hipq_ctx {
     void *scratch = nullptr;
     size_t scratch_bytes = 0;
     int num_cus = 256;
+    // Device word set by a kernel whose bounded wait gave up; read and cleared by hipq_ctx_synchronize.
+    uint32_t *wait_error = nullptr;
+    // Test and tuning hooks, per context: forced GEMM kernel form (0 = automatic, -1 = not yet read from the
+    // HIPQ_GEMM_VARIANT environment variable) and the spin limit of the persistent kernel's waits.
+    int gemm_variant = -1;
+    int wait_spin_limit = 1 << 20;
 };
 
 namespace hipq {

@@ -117,7 +117,8 @@ _SIGNATURES = {
     "hipq_linear_i8_f32_residual": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_layer_norm_f32": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _vp],
     "hipq_quantize_static_per_tensor_f32_i8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp, _vp],
-    "hipq_set_gemm_kernel_variant": [_i32],
+    "hipq_set_gemm_kernel_variant": [_vp, _i32],
+    "hipq_ctx_set_wait_spin_limit": [_vp, _i32],
     "hipq_linear_static_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_add_layer_norm_quantize_f32_i8": [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
@@ -228,7 +229,11 @@ class Context:
 
     def set_gemm_kernel_variant(self, variant: int) -> None:
         """Test / tuning hook: force one GEMM kernel form for later calls (0 = automatic)."""
-        _check(self._lib.hipq_set_gemm_kernel_variant(int(variant)))
+        self.call("hipq_set_gemm_kernel_variant", int(variant))
+
+    def set_wait_spin_limit(self, limit: int) -> None:
+        """Test hook: polls a bounded wait of the persistent GEMM kernel makes before it gives up (< 0: default)."""
+        self.call("hipq_ctx_set_wait_spin_limit", int(limit))
 
     def synchronize(self) -> None:
         self.call("hipq_ctx_synchronize")
