@@ -270,39 +270,54 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__
                                                                   size_t cols, float scale, int zp,
                                                                   const hipq_qparams *__restrict__ params,
                                                                   DynamicRange dyn, int8_t *__restrict__ out) {
-    __shared__ float range_lds[2 * kBlock / kWave];
-    if (!resolve_quantize_params(dyn, params, range_lds, scale, zp)) return;
-    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
-    const float zpf = static_cast<float>(zp);
     const size_t KB = ((cols + 31) / 32 + 3) / 4 * 4;
     const size_t nfrag = ((rows + 31) / 32) * KB;
     const int lane = threadIdx.x % kWave;
     const bool vec = (cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
-    for (size_t f = size_t(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave; f < nfrag;
-         f += size_t(gridDim.x) * (kBlock / kWave)) {
-        const size_t rb = f / KB, kb = f % KB;
-        const size_t row = rb * 32 + lane % 32, k0 = kb * 32 + 16 * (lane / 32);
+    const size_t fstep = size_t(gridDim.x) * (kBlock / kWave);
+    size_t f = size_t(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave;
+    // The first fragment's floats are requested before the parameters are resolved (a fold of the range
+    // partials and two workgroup barriers in a dynamic call): the loads do not depend on the scale, and a
+    // launch of this size is bound by latency, not by bandwidth.
+    auto whole = [&](size_t frag, size_t *row, size_t *k0) {
+        const size_t rb = frag / KB, kb = frag % KB;
+        *row = rb * 32 + lane % 32;
+        *k0 = kb * 32 + 16 * (lane / 32);
+        return vec && frag < nfrag && *row < rows && *k0 + 16 <= cols;
+    };
+    float4 v[4];
+    size_t row, k0;
+    bool have = whole(f, &row, &k0);
+    if (have) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(x + row * cols + k0)[i];
+    }
+    __shared__ float range_lds[2 * kBlock / kWave];
+    if (!resolve_quantize_params(dyn, params, range_lds, scale, zp)) return;
+    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
+    const float zpf = static_cast<float>(zp);
+    for (; f < nfrag; f += fstep) {
         uint32_t w[4] = {0u, 0u, 0u, 0u};
-        if (row < rows && k0 < cols) {
+        if (have) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, zpf, -128, 127),
+                             quantize_int<DIV, RND>(v[i].y, scale, inv, zpf, -128, 127),
+                             quantize_int<DIV, RND>(v[i].z, scale, inv, zpf, -128, 127),
+                             quantize_int<DIV, RND>(v[i].w, scale, inv, zpf, -128, 127));
+        } else if (row < rows && k0 < cols) {
             const float *p = x + row * cols + k0;
-            if (vec && k0 + 16 <= cols) {
-                float4 v[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(p)[i];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    w[i] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, zpf, -128, 127),
-                                 quantize_int<DIV, RND>(v[i].y, scale, inv, zpf, -128, 127),
-                                 quantize_int<DIV, RND>(v[i].z, scale, inv, zpf, -128, 127),
-                                 quantize_int<DIV, RND>(v[i].w, scale, inv, zpf, -128, 127));
-            } else {
-                for (int b = 0; b < 16; ++b)
-                    if (k0 + b < cols)
-                        w[b / 4] |= (uint32_t(quantize_int<DIV, RND>(p[b], scale, inv, zpf, -128, 127)) & 0xffu)
-                                    << (8 * (b % 4));
-            }
+            for (int b = 0; b < 16; ++b)
+                if (k0 + b < cols)
+                    w[b / 4] |= (uint32_t(quantize_int<DIV, RND>(p[b], scale, inv, zpf, -128, 127)) & 0xffu)
+                                << (8 * (b % 4));
         }
         *reinterpret_cast<uint4 *>(out + f * 1024 + size_t(lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        have = whole(f + fstep, &row, &k0);
+        if (have) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(x + row * cols + k0)[i];
+        }
     }
 }
 
