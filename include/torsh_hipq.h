@@ -59,7 +59,18 @@ enum {
     HIPQ_FORM_DIV = 2,
     /* floor(v + 0.5): the reduced-precision rounding of quantize_mobile_optimized
      * (simd_ops.rs:424-431); accepted by hipq_quantize_per_tensor_f32_i8 only. */
-    HIPQ_ROUND_FLOOR_HALF_UP = 16
+    HIPQ_ROUND_FLOOR_HALF_UP = 16,
+    /* round(x / scale + zero_point): the zero point enters before the rounding, as in the scalar
+     * quantized types QInt8 / QUInt8 (crates/torsh-core/src/dtype/quantized.rs:129-134, 285-290);
+     * differs from round(x / scale) + zero_point on ties when the zero point is not 0.  Implies the
+     * division form.  Accepted by hipq_quantize_per_tensor_f32_i8 / _u8. */
+    HIPQ_FORM_ZP_BEFORE_ROUND = 32,
+    /* ((x / scale).round() as i32) + zero_point: the value passes through Rust's `as i32` (NaN -> 0)
+     * before the zero point is added, as in torsh-nn's quantize_value_symmetric / _asymmetric
+     * (crates/torsh-nn/src/quantization/ops.rs:153-162), so a NaN input gives the code `zero_point`
+     * instead of a NaN carrier.  Implies the division form.  Accepted by
+     * hipq_quantize_per_tensor_f32_carrier. */
+    HIPQ_FORM_INT_CAST = 64
 };
 
 /* Quantized integer types, ranges per get_dtype_range
@@ -80,7 +91,14 @@ enum {
      * Observer::calculate_qparams (crates/torsh-quantization/src/observers.rs:263-310),
      * quantize_int4_per_tensor / _per_channel and quantize_group_wise
      * (crates/torsh-quantization/src/specialized.rs:39-48, 126-133, 322-335). */
-    HIPQ_PARAMS_ZERO_INCLUDED = 4
+    HIPQ_PARAMS_ZERO_INCLUDED = 4,
+    /* per_channel_quantize_weights of torsh-nn (crates/torsh-nn/src/quantization/ops.rs:296-373):
+     * symmetric scale = max(|min|,|max|) / 127 with no zero guard (an all-zero channel gets scale 0),
+     * asymmetric scale = (max - min) / 255 and zero_point = round(-min / scale), not clamped.  Both
+     * always report HIPQ_SUCCESS, as the reference does not validate the range.  Accepted by the
+     * per-row / per-group quantizers. */
+    HIPQ_PARAMS_NN_SYMMETRIC = 5,
+    HIPQ_PARAMS_NN_ASYMMETRIC = 6
 };
 
 /* Device-resident quantization parameters, written by the kernels that derive
@@ -208,7 +226,8 @@ HIPQ_API int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const floa
                                                        int32_t *out_zero_points, int32_t *out_status);
 /* Generalisation to groups of `group_size` consecutive channels that share
  * one (scale, zero point) - the last group may be shorter - with a caller-chosen
- * integer range [qmin, qmax] inside [-128, 127] and any HIPQ_PARAMS_* flavor:
+ * integer range [qmin, qmax] inside [-128, 127] (or inside [0, 255]: the codes are then the bytes of `out`
+ * read as uint8) and any HIPQ_PARAMS_* flavor:
  * quantize_group_wise (crates/torsh-quantization/src/specialized.rs:241-377) and,
  * with group_size 1 and range -8..7, quantize_int4_per_channel (specialized.rs:68-160).
  * out_scales / out_zero_points hold ceil(channels / group_size) entries.  Values

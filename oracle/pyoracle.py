@@ -325,6 +325,17 @@ def nn_per_channel_quantize_weights_sym_i8(w):
     return out, scales
 
 
+def nn_per_channel_quantize_weights_asym_u8(w):
+    w = _f32(w)
+    ch = w.shape[0]
+    out = np.empty_like(w)
+    scales = np.empty(ch, dtype=np.float32)
+    zps = np.empty(ch, dtype=np.int32)
+    lib().tq_nn_per_channel_quantize_weights_asym_u8(_p(w, _f32p), C.c_size_t(ch), C.c_size_t(w.size // max(ch, 1)),
+                                                     _p(out, _f32p), _p(scales, _f32p), _p(zps, _i32p))
+    return out, scales, zps
+
+
 def backend_quantize_value(v, scale, zp, qmin=-128, qmax=127):
     return int(lib().tq_backend_quantize_value(C.c_float(v), C.c_float(scale), int(zp), int(qmin), int(qmax)))
 

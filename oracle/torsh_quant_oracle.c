@@ -408,6 +408,29 @@ int tq_nn_per_channel_quantize_weights_sym_i8(const float *w, size_t channels, s
     return TQ_OK;
 }
 
+/* crates/torsh-nn/src/quantization/ops.rs:296-373, Asymmetric + U8 arm:
+ * scale = (max - min)/255, zero_point = round(-min/scale) as i32 (not clamped), value =
+ * clamp((round(v/scale) as i32) + zero_point, 0, 255) stored as the byte widened to f32. */
+int tq_nn_per_channel_quantize_weights_asym_u8(const float *w, size_t channels, size_t channel_size,
+                                               float *out_carrier, float *scales, int32_t *zps) {
+    for (size_t c = 0; c < channels; ++c) {
+        float mn = INFINITY, mx = -INFINITY;
+        for (size_t i = 0; i < channel_size; ++i) {
+            mn = fminf(mn, w[c * channel_size + i]);
+            mx = fmaxf(mx, w[c * channel_size + i]);
+        }
+        float s = (mx - mn) / 255.0f;
+        int32_t zp = f32_as_i32(roundf(-mn / s));
+        scales[c] = s;
+        zps[c] = zp;
+        for (size_t i = 0; i < channel_size; ++i) {
+            int32_t q = tq_nn_quantize_value_asymmetric(w[c * channel_size + i], s, zp, 0, 255);
+            out_carrier[c * channel_size + i] = (float)(uint8_t)q;
+        }
+    }
+    return TQ_OK;
+}
+
 /* crates/torsh-backend/src/quantization/ops.rs:185-195 */
 int32_t tq_backend_quantize_value(float v, float scale, int32_t zp, int32_t qmin, int32_t qmax) {
     float q = rnd(v / scale) + (float)zp;

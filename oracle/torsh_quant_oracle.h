@@ -87,6 +87,8 @@ int32_t tq_nn_quantize_value_asymmetric(float v, float scale, int32_t zp, int32_
 float tq_nn_dequantize_value_asymmetric(int32_t q, float scale, int32_t zp);
 int tq_nn_per_channel_quantize_weights_sym_i8(const float *w, size_t channels, size_t channel_size,
                                               float *out_carrier, float *scales);
+int tq_nn_per_channel_quantize_weights_asym_u8(const float *w, size_t channels, size_t channel_size,
+                                               float *out_carrier, float *scales, int32_t *zps);
 
 /* ---- torsh-backend::quantization -------------------------------------- */
 int32_t tq_backend_quantize_value(float v, float scale, int32_t zp, int32_t qmin, int32_t qmax);

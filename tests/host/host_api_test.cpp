@@ -19,6 +19,7 @@
 #include "torsh_hipq/hardware.hpp"
 #include "torsh_hipq/models.hpp"
 #include "torsh_hipq/nn.hpp"
+#include "torsh_hipq/nn_quantization.hpp"
 #include "torsh_hipq/quantization.hpp"
 #include "torsh_hipq/serialize.hpp"
 #include "torsh_calib_oracle.h"
@@ -775,6 +776,27 @@ CPU_TEST(test_weight_file_round_trip_and_corruption) {
     CHECK(load_quantized_weights(path).is_err());
     write(std::vector<char>(300, 'x'));
     CHECK(load_quantized_weights(path).is_err());
+    // a damaged header field is caught by the checksum, which covers the header
+    auto header = bytes;
+    header[16] ^= 4;  // dims[0]
+    write(header);
+    CHECK(load_quantized_weights(path).unwrap_err().message.find("checksum") != std::string::npos);
+    // a crafted header with a consistent checksum: offsets and dims near 2^64 must not wrap the bounds checks
+    auto craft = [&](size_t field_off, uint64_t value) {
+        auto b = bytes;
+        std::memcpy(b.data() + field_off, &value, 8);
+        std::memset(b.data() + 80, 0, 8);
+        const uint64_t sum = torsh::quantization::detail::fnv1a64(reinterpret_cast<const unsigned char *>(b.data()), b.size());
+        std::memcpy(b.data() + 80, &sum, 8);
+        write(b);
+        return load_quantized_weights(path);
+    };
+    CHECK(craft(48, ~uint64_t(0) - 15).unwrap_err().message.find("section outside") != std::string::npos);  // weights
+    CHECK(craft(56, ~uint64_t(0) - 3).unwrap_err().message.find("section outside") != std::string::npos);   // scales
+    CHECK(craft(64, uint64_t(1) << 63).unwrap_err().message.find("section outside") != std::string::npos);  // bias
+    CHECK(craft(48, 8).is_err());                                                                          // inside the header
+    CHECK(craft(16, uint64_t(1) << 62).unwrap_err().message.find("implausible") != std::string::npos);      // rows
+    CHECK(craft(24, ~uint64_t(0)).unwrap_err().message.find("implausible") != std::string::npos);           // a dim
     QuantizedWeights bad = w;
     bad.scales.pop_back();
     CHECK(save_quantized_weights(bad, path).is_err());
@@ -1055,15 +1077,6 @@ CPU_TEST(test_slice_variant_errors_before_the_device) {  // algorithms.rs:997-10
     auto b = quantize_batch_consistent_simd({&in}, 0.1f, 0, outs);
     CHECK(b.is_err());
     CHECK_EQ(b.unwrap_err().message, std::string("Number of input tensors must match output tensors"));
-    const auto small = get_cache_optimization_recommendations(1000, 4, cp);
-    CHECK(!small.empty() && small[0].find("L1 cache") != std::string::npos);
-    bool streaming = false;
-    for (const auto &line : get_cache_optimization_recommendations(10000000, 4, cp))
-        streaming = streaming || line.find("streaming") != std::string::npos;
-    CHECK(streaming);
-    const MobileOptimizationHints hints = get_mobile_optimization_hints();
-    CHECK(hints.prefer_int8 && hints.optimal_chunk_size > 0 && !hints.prefer_sequential);
-    CHECK(get_simd_width() >= 1 && (!is_simd_available() || get_simd_width() > 1));
 }
 
 GPU_TEST(test_slice_variants) {  // algorithms.rs:897-982, simd_ops.rs:513-522, 569-618
@@ -1564,6 +1577,106 @@ GPU_TEST(test_kernel_plugin_dispatch) {
         check_same(q.as_slice(), q2.as_slice(), __LINE__);
         const Tensor back = hq.dequantize(q, s, z).unwrap();
         check_same(back.as_slice(), dequantize(q2, s2, z2).unwrap().as_slice(), __LINE__);
+    }
+}
+
+// ---- torsh-core scalar quantized types and torsh-nn's quantizer ---------------------------------
+// crates/torsh-core/src/dtype/quantized.rs:126-127 (doc example), 878-892 (test_edge_cases), 865-875.
+CPU_TEST(test_scalar_quantized_types) {
+    using namespace torsh::dtype::quantized;
+    CHECK(QInt8::quantize(2.5f, 0.1f, 5).value == 30);  // round(2.5 / 0.1 + 5)
+    CHECK(QInt8::quantize(1000.0f, 1.0f, 0).value == 127);
+    CHECK(QInt8::quantize(-1000.0f, 1.0f, 0).value == -128);
+    const QInt8 q = QInt8::quantize(3.14159265f, 0.1f, 0);
+    CHECK(std::fabs(q.dequantize() - 3.14159265f) < 0.05f);
+    // the zero point enters before the rounding: -2.5 + 5 = 2.5 -> 3, not round(-2.5) + 5 = 2
+    CHECK(QInt8::quantize(-2.5f, 1.0f, 5).value == 3);
+    CHECK(QUInt8::quantize(-2.5f, 1.0f, 5).value == 3);
+    CHECK(QUInt8::quantize(-1000.0f, 1.0f, 5).value == 0 && QUInt8::quantize(1000.0f, 1.0f, 5).value == 255);
+    CHECK(QInt32::quantize(1e20f, 1.0f, 0).value == 2147483647 && QInt32::quantize(-1e20f, 1.0f, 7).value == INT32_MIN);
+    CHECK(QInt32::quantize(2.5f, 1.0f, 1).value == 4);  // f64: round(3.5) = 4
+    const QInt32 q32{10, 0.5f, 4};
+    const QUInt8 qu8{10, 0.5f, 4};
+    CHECK(q32.dequantize() == 3.0f && qu8.dequantize() == 3.0f);
+    std::mt19937 rng(7);
+    std::uniform_real_distribution<float> dv(-40.0f, 40.0f), ds(0.01f, 0.5f);
+    for (int i = 0; i < 2000; ++i) {
+        const float v = dv(rng), sc = ds(rng);
+        const int zp = static_cast<int>(rng() % 200) - 100;
+        CHECK(QInt8::quantize(v, sc, static_cast<int8_t>(zp)).value == tq_qint8_quantize(v, sc, zp));
+        if (zp >= 0) CHECK(QUInt8::quantize(v, sc, static_cast<uint8_t>(zp)).value == tq_quint8_quantize(v, sc, zp));
+    }
+}
+
+// crates/torsh-nn/src/quantization/ops.rs:380-429 (test_symmetric_quantization, test_asymmetric_quantization),
+// then every value against the oracle's restatement of quantize_value_* and per_channel_quantize_weights.
+GPU_TEST(parity_torsh_nn_quantizer_and_qtype_slices) {
+    namespace nq = torsh::nn::quantization;
+    {
+        const Tensor t = tensor_1d({1.0f, -1.0f, 0.5f, -0.5f, 2.0f, -2.0f}).unwrap();
+        const nq::QuantizationParams p = nq::QuantizationParams::symmetric(2.0f / 127.0f, DType::F32, DType::I8).unwrap();
+        const Tensor back = p.dequantize(p.quantize(t).unwrap()).unwrap();
+        for (size_t i = 0; i < 6; ++i) CHECK(std::fabs(back.as_slice()[i] - t.as_slice()[i]) < 0.1f);
+    }
+    {
+        const Tensor t = tensor_1d({0.0f, 1.0f, 2.0f, 3.0f, 4.0f, 5.0f}).unwrap();
+        const nq::QuantizationParams p = nq::QuantizationParams::asymmetric(5.0f / 255.0f, 0, DType::F32, DType::U8).unwrap();
+        const Tensor back = p.dequantize(p.quantize(t).unwrap()).unwrap();
+        for (size_t i = 0; i < 6; ++i) CHECK(std::fabs(back.as_slice()[i] - t.as_slice()[i]) < 0.1f);
+    }
+    CHECK(nq::QuantizationParams::symmetric(1.0f, DType::F32, DType::F32).is_err());
+    std::mt19937 rng(11);
+    std::normal_distribution<float> nd(0.0f, 2.0f);
+    std::vector<float> x(3000);
+    for (float &v : x) v = nd(rng);
+    x[0] = NAN, x[1] = INFINITY, x[2] = -INFINITY, x[3] = 2.5f * 0.05f, x[4] = -2.5f * 0.05f;
+    const Tensor t = tensor_1d(x).unwrap();
+    {
+        const nq::QuantizationParams p = nq::QuantizationParams::symmetric(0.05f, DType::F32, DType::I8).unwrap();
+        const Tensor q = p.quantize(t).unwrap();
+        for (size_t i = 0; i < x.size(); ++i)
+            CHECK(q.as_slice()[i] == static_cast<float>(tq_nn_quantize_value_symmetric(x[i], 0.05f, -128, 127)));
+        CHECK(q.as_slice()[0] == 0.0f);  // NaN as i32
+    }
+    {
+        const nq::QuantizationParams p = nq::QuantizationParams::asymmetric(0.05f, 77, DType::F32, DType::U8).unwrap();
+        const Tensor q = p.quantize(t).unwrap();
+        for (size_t i = 0; i < x.size(); ++i)
+            CHECK(q.as_slice()[i] == static_cast<float>(tq_nn_quantize_value_asymmetric(x[i], 0.05f, 77, 0, 255)));
+        CHECK(q.as_slice()[0] == 77.0f);  // NaN -> 0, then the zero point
+        const Tensor y = p.dequantize(q).unwrap();
+        for (size_t i = 0; i < x.size(); ++i)
+            CHECK(y.as_slice()[i] == tq_nn_dequantize_value_asymmetric(static_cast<int32_t>(q.as_slice()[i]), 0.05f, 77));
+    }
+    // per-channel weights: an all-zero channel keeps scale 0 (no guard)
+    std::vector<float> w(6 * 100);
+    for (float &v : w) v = nd(rng) * 0.01f;
+    for (size_t i = 200; i < 300; ++i) w[i] = 0.0f;
+    const Tensor wt = Tensor::from_data(w, {6, 100}).unwrap();
+    {
+        auto r = nq::per_channel_quantize_weights(wt, nq::QuantizationScheme::Symmetric, DType::I8).unwrap();
+        std::vector<float> carrier(w.size()), scales(6);
+        tq_nn_per_channel_quantize_weights_sym_i8(w.data(), 6, 100, carrier.data(), scales.data());
+        check_same(r.first.as_slice(), carrier, __LINE__);
+        for (size_t c = 0; c < 6; ++c) CHECK(r.second[c].scale == scales[c] && r.second[c].zero_point == 0);
+        CHECK(r.second[2].scale == 0.0f);
+    }
+    {
+        auto r = nq::per_channel_quantize_weights(wt, nq::QuantizationScheme::Asymmetric, DType::U8);
+        // (channel 2 has a zero range: scale 0, zero point round(-0/0) = NaN as i32 = 0, codes NaN -> 0 + 0)
+        std::vector<float> carrier(w.size()), scales(6);
+        std::vector<int32_t> zps(6);
+        tq_nn_per_channel_quantize_weights_asym_u8(w.data(), 6, 100, carrier.data(), scales.data(), zps.data());
+        check_same(r.unwrap().first.as_slice(), carrier, __LINE__);
+        for (size_t c = 0; c < 6; ++c) CHECK(r.unwrap().second[c].scale == scales[c] && r.unwrap().second[c].zero_point == zps[c]);
+    }
+    CHECK(nq::per_channel_quantize_weights(wt, nq::QuantizationScheme::Dynamic, DType::I8).is_err());
+    // slices of the scalar types on the device
+    {
+        const auto q = torsh::dtype::quantized::quantize_slice_qint8(x, 0.1f, 5).unwrap();
+        for (size_t i = 0; i < x.size(); ++i) CHECK(q[i] == tq_qint8_quantize(x[i], 0.1f, 5));
+        const auto u = torsh::dtype::quantized::quantize_slice_quint8(x, 0.1f, 130).unwrap();
+        for (size_t i = 0; i < x.size(); ++i) CHECK(u[i] == tq_quint8_quantize(x[i], 0.1f, 130));
     }
 }
 

@@ -436,3 +436,60 @@ def test_cache_aware_twins_share_the_carrier_kernel(ctx, hipq, oracle, golden):
     x[:3] = [np.nan, 1e9, -1e9]
     got = host(ctx.quantize_per_tensor_carrier(dev(x), 0.05, -3, hipq.FORM_MUL_INV))
     np.testing.assert_array_equal(got, oracle.quantize_cache_aware(x, 0.05, -3))
+
+
+def test_scalar_qtypes_form_zero_point_before_rounding(ctx, hipq, oracle):
+    """QInt8 / QUInt8::quantize (crates/torsh-core/src/dtype/quantized.rs:129-134, 285-290): round(v / scale + zp),
+    clamped to the type.  Ties where the two orders differ (v / scale = -2.5, zp = 5: 3 against 2), saturation,
+    NaN -> 0, and random data, element by element against the oracle's scalar functions."""
+    rng = np.random.default_rng(21)
+    special = np.float32([-2.5, 2.5, -0.5, 0.5, 0.0, 1e9, -1e9, np.nan, np.inf, -np.inf, 122.5, -133.5])
+    for scale, zp in ((1.0, 5), (0.1, -7), (0.37, 100)):
+        x = np.concatenate([special * np.float32(scale), rng.standard_normal(3000).astype(np.float32) * 40]).astype(np.float32)
+        got = host(ctx.quantize_per_tensor_i8(dev(x), scale, zp, hipq.FORM_ZP_BEFORE_ROUND))
+        want = np.array([oracle.qint8_quantize(float(v), scale, zp) for v in x], np.int8)
+        np.testing.assert_array_equal(got, want)
+        if zp >= 0:
+            gotu = host(ctx.quantize_per_tensor_u8(dev(x), scale, zp, hipq.FORM_ZP_BEFORE_ROUND))
+            wantu = np.array([oracle.quint8_quantize(float(v), scale, zp) for v in x], np.uint8)
+            np.testing.assert_array_equal(gotu, wantu)
+    # the order matters: the default form gives the other answer on the crafted tie
+    x = dev(np.float32([-2.5]))
+    assert int(host(ctx.quantize_per_tensor_i8(x, 1.0, 5, hipq.FORM_ZP_BEFORE_ROUND))[0]) == 3
+    assert int(host(ctx.quantize_per_tensor_i8(x, 1.0, 5, hipq.FORM_DIV))[0]) == 2
+    with pytest.raises(hipq.HipqError):  # two rounding rules at once
+        ctx.quantize_per_tensor_i8(x, 1.0, 5, hipq.FORM_ZP_BEFORE_ROUND | hipq.ROUND_FLOOR_HALF_UP)
+
+
+def test_torsh_nn_flavour(ctx, hipq, oracle):
+    """torsh-nn's own quantizer (crates/torsh-nn/src/quantization/ops.rs:153-172, 296-373): values pass through
+    `as i32` before the zero point is added (a NaN becomes the code zero_point, not a NaN carrier), per-channel
+    weight scales have no zero guard, negative int8 codes are carried as 256 + q."""
+    rng = np.random.default_rng(22)
+    x = np.concatenate([np.float32([2.5, -2.5, 1e9, -1e9, np.nan, np.inf, -np.inf, 0.0]),
+                        rng.standard_normal(2000).astype(np.float32) * 3]).astype(np.float32)
+    for scale, zp, qmin, qmax in ((0.05, 0, -128, 127), (0.02, 77, 0, 255), (0.001, 0, -32768, 32767)):
+        got = host(ctx.quantize_per_tensor_carrier(dev(x), scale, zp, hipq.FORM_INT_CAST, qmin, qmax))
+        if zp == 0:
+            want = [oracle.nn_quantize_value_symmetric(float(v), scale, qmin, qmax) for v in x]
+        else:
+            want = [oracle.nn_quantize_value_asymmetric(float(v), scale, zp, qmin, qmax) for v in x]
+        np.testing.assert_array_equal(got, np.float32(want))
+    # per-channel weights, symmetric int8: codes, unguarded scales (an all-zero and a tiny channel among them)
+    w = (rng.standard_normal((9, 200)) * 0.02).astype(np.float32)
+    w[3] = 0.0
+    w[5] *= 1e-9
+    want_carrier, want_s = oracle.nn_per_channel_quantize_weights_sym_i8(w)
+    q, s, z, st = ctx.quantize_per_group_auto(dev(w), 1, 9, 200, 1, hipq.PARAMS_NN_SYMMETRIC, -128, 127, hipq.FORM_DIV)
+    assert int(host(st)[0]) == 0
+    np.testing.assert_array_equal(host(s), want_s)
+    np.testing.assert_array_equal(host(q).view(np.uint8).astype(np.float32), want_carrier)  # 256 + q for negatives
+    assert (host(z) == 0).all()
+    # asymmetric uint8: unclamped zero point, bytes 0..255
+    w2 = (rng.standard_normal((7, 130)) * 0.5 + 1.0).astype(np.float32)
+    w2[2] = np.abs(w2[2]) + 2.0  # all positive: zero point far below 0
+    want_carrier, want_s, want_z = oracle.nn_per_channel_quantize_weights_asym_u8(w2)
+    q, s, z, st = ctx.quantize_per_group_auto(dev(w2), 1, 7, 130, 1, hipq.PARAMS_NN_ASYMMETRIC, 0, 255, hipq.FORM_DIV)
+    np.testing.assert_array_equal(host(s), want_s)
+    np.testing.assert_array_equal(host(z), want_z)
+    np.testing.assert_array_equal(host(q).view(np.uint8).astype(np.float32), want_carrier)

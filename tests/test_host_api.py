@@ -27,8 +27,10 @@ CPU_CASES = [
     "test_kernel_plugin_interface",
     "test_slice_variant_errors_before_the_device",
     "test_fake_quantize_errors_before_the_device",
+    "test_scalar_quantized_types",
 ]
 GPU_CASES = [
+    "parity_torsh_nn_quantizer_and_qtype_slices",
     "test_quantize_per_tensor_affine",
     "test_dequantize_per_tensor_affine",
     "test_quantize_tensor_auto",

@@ -178,6 +178,21 @@ def test_nn_flavour(oracle):
     assert s[0] == np.float32(2.0) / np.float32(127.0) and s[1] == np.float32(0.2) / np.float32(127.0)
     # negatives are carried as the two's-complement byte widened to f32
     np.testing.assert_array_equal(q[0], [64, 256 - 127, 32])
+    # an all-zero channel: no zero guard, scale 0, 0/0 = NaN -> `as i32` 0
+    q, s = oracle.nn_per_channel_quantize_weights_sym_i8(np.zeros((1, 4), np.float32))
+    assert s[0] == 0.0 and (q == 0).all()
+    # asymmetric uint8 arm by hand: channel [-1, 0, 1.55]: scale 2.55/255 = 0.01, zp = round(1/0.01) = 100,
+    # codes round(v/0.01) + 100 = 0, 100, 255; channel [2, 4]: scale 2/255, zp = round(-2/scale) = -255 (not
+    # clamped), codes clamp(255 - 255, 0, 255) = 0 and clamp(510 - 255) = 255
+    q, s, z = oracle.nn_per_channel_quantize_weights_asym_u8(np.float32([[-1.0, 0.0, 1.55]]))
+    assert s[0] == np.float32(2.55) / np.float32(255.0) and z[0] == 100
+    np.testing.assert_array_equal(q[0], [0, 100, 255])
+    q, s, z = oracle.nn_per_channel_quantize_weights_asym_u8(np.float32([[2.0, 4.0]]))
+    assert z[0] == -255
+    np.testing.assert_array_equal(q[0], [0, 255])
+    # the scalar quantized types (zero point before rounding), unsigned: round(-2.5 + 5) = 3, not round(-2.5) + 5 = 2
+    assert oracle.quint8_quantize(-2.5, 1.0, 5) == 3
+    assert oracle.quint8_quantize(1000.0, 1.0, 5) == 255 and oracle.quint8_quantize(-1000.0, 1.0, 5) == 0
 
 
 def test_int_gemm_vs_int64_bruteforce(oracle):

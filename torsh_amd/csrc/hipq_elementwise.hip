@@ -209,7 +209,7 @@ __device__ __forceinline__ bool resolve_quantize_params(const DynamicRange &dyn,
 // memory when `params` is non-null, or (dynamic quantization) from the range partials: then
 // every workgroup folds the same few hundred partials in the same order, derives the same
 // parameters, and workgroup 0 publishes them, which saves the launch of a finalize kernel.
-template <typename OutT, bool DIV, int RND>
+template <typename OutT, int DIV, int RND>
 __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restrict__ x, size_t n, float scale,
                                                            int zp, const hipq_qparams *__restrict__ params,
                                                            DynamicRange dyn, float lo, float hi,
@@ -460,12 +460,13 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     const float zpf = static_cast<float>(zp);
     const float inv = recip_for_div(scale);  // once per row; each element then divides with two FMAs
     uint32_t *q4 = reinterpret_cast<uint32_t *>(qr);
-    auto quant4 = [&](float4 t) {
-        return pack4(quantize_int<true, EVEN>(t.x, scale, inv, zpf, qmin, qmax),
-                     quantize_int<true, EVEN>(t.y, scale, inv, zpf, qmin, qmax),
-                     quantize_int<true, EVEN>(t.z, scale, inv, zpf, qmin, qmax),
-                     quantize_int<true, EVEN>(t.w, scale, inv, zpf, qmin, qmax));
+    // torsh-nn's per-channel weights pass each value through `as i32` before the zero point is added
+    const bool int_cast = flavor >= HIPQ_PARAMS_NN_SYMMETRIC;
+    auto quant1 = [&](float v) {
+        return int_cast ? quantize_int<QFORM_DIV_INT_CAST, EVEN>(v, scale, inv, zpf, qmin, qmax)
+                        : quantize_int<QFORM_DIV, EVEN>(v, scale, inv, zpf, qmin, qmax);
     };
+    auto quant4 = [&](float4 t) { return pack4(quant1(t.x), quant1(t.y), quant1(t.z), quant1(t.w)); };
 #pragma unroll
     for (int i = 0; i < kCache; ++i) {
         const size_t v = size_t(lane) + size_t(i) * TPR;
@@ -473,7 +474,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     }
     for (size_t v = size_t(lane) + size_t(kCache) * TPR; v < nvec; v += TPR) q4[v] = quant4(x4[v]);
     for (size_t c = nvec * 4 + lane; c < cols; c += TPR)
-        qr[c] = static_cast<int8_t>(quantize_int<true, EVEN>(xr[c], scale, inv, zpf, qmin, qmax));
+        qr[c] = static_cast<int8_t>(quant1(xr[c]));
 }
 
 // quantize_per_channel_auto for a channel axis that is not the leading one, and its group-wise
@@ -629,18 +630,32 @@ static int32_t launch_quantize(hipq_ctx *ctx, const float *x, size_t n, float sc
 #define HIPQ_LAUNCH_Q(D, E)                                                                                   \
     hipLaunchKernelGGL((quantize_kernel<OutT, D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, n, scale, zp, \
                        params, dyn, lo, hi, out)
-    if (half_up && div)
-        HIPQ_LAUNCH_Q(true, 2);
+    if (mode & HIPQ_FORM_ZP_BEFORE_ROUND) {  // integer outputs only (checked by the entry points)
+        if constexpr (sizeof(OutT) == 1) {
+            if (even)
+                HIPQ_LAUNCH_Q(QFORM_DIV_ZP_FIRST, 1);
+            else
+                HIPQ_LAUNCH_Q(QFORM_DIV_ZP_FIRST, 0);
+        }
+    } else if (mode & HIPQ_FORM_INT_CAST) {  // carrier output only
+        if constexpr (sizeof(OutT) == 4) {
+            if (even)
+                HIPQ_LAUNCH_Q(QFORM_DIV_INT_CAST, 1);
+            else
+                HIPQ_LAUNCH_Q(QFORM_DIV_INT_CAST, 0);
+        }
+    } else if (half_up && div)
+        HIPQ_LAUNCH_Q(1, 2);
     else if (half_up)
-        HIPQ_LAUNCH_Q(false, 2);
+        HIPQ_LAUNCH_Q(0, 2);
     else if (div && even)
-        HIPQ_LAUNCH_Q(true, 1);
+        HIPQ_LAUNCH_Q(1, 1);
     else if (div)
-        HIPQ_LAUNCH_Q(true, 0);
+        HIPQ_LAUNCH_Q(1, 0);
     else if (even)
-        HIPQ_LAUNCH_Q(false, 1);
+        HIPQ_LAUNCH_Q(0, 1);
     else
-        HIPQ_LAUNCH_Q(false, 0);
+        HIPQ_LAUNCH_Q(0, 0);
 #undef HIPQ_LAUNCH_Q
     return check_launch("quantize");
 }
@@ -704,7 +719,7 @@ int32_t hipq_qparams_from_minmax(hipq_ctx *ctx, const float *minmax, int32_t fla
     HIPQ_ENTER(ctx);
     HIPQ_REQUIRE_PTR(minmax);
     HIPQ_REQUIRE_PTR(out_params);
-    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_NN_ASYMMETRIC)
         return fail(HIPQ_INVALID_ARGUMENT, "hipq_qparams_from_minmax: unknown flavor %d", flavor);
     if (qmin >= qmax) return fail(HIPQ_INVALID_ARGUMENT, "hipq_qparams_from_minmax: qmin %d >= qmax %d", qmin, qmax);
     hipLaunchKernelGGL(qparams_kernel, dim3(1), dim3(64), 0, ctx->stream, minmax, flavor, qmin, qmax, out_params);
@@ -716,9 +731,10 @@ int32_t hipq_quantize_per_tensor_f32_i8(hipq_ctx *ctx, const float *x, size_t n,
     HIPQ_ENTER(ctx);
     int32_t rc = check_scale(__func__, scale);
     if (rc) return rc;
-    // this entry point alone also knows the floor(v + 0.5) rounding of quantize_mobile_optimized
-    if ((rc = check_mode(__func__, mode & ~HIPQ_ROUND_FLOOR_HALF_UP))) return rc;
-    if ((mode & HIPQ_ROUND_FLOOR_HALF_UP) && (mode & HIPQ_ROUND_HALF_EVEN))
+    // this entry point alone also knows the floor(v + 0.5) rounding of quantize_mobile_optimized; the integer
+    // outputs know the zero-point-first form of the scalar quantized types
+    if ((rc = check_mode(__func__, mode & ~(HIPQ_ROUND_FLOOR_HALF_UP | HIPQ_FORM_ZP_BEFORE_ROUND)))) return rc;
+    if ((mode & HIPQ_ROUND_FLOOR_HALF_UP) && (mode & (HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_ZP_BEFORE_ROUND)))
         return fail(HIPQ_INVALID_ARGUMENT, "%s: two rounding modes in mode 0x%x", __func__, mode);
     if (n == 0) return HIPQ_SUCCESS;
     HIPQ_REQUIRE_PTR(x);
@@ -746,7 +762,7 @@ int32_t hipq_quantize_per_tensor_f32_u8(hipq_ctx *ctx, const float *x, size_t n,
     HIPQ_ENTER(ctx);
     int32_t rc = check_scale(__func__, scale);
     if (rc) return rc;
-    if ((rc = check_mode(__func__, mode))) return rc;
+    if ((rc = check_mode(__func__, mode & ~HIPQ_FORM_ZP_BEFORE_ROUND))) return rc;
     if (n == 0) return HIPQ_SUCCESS;
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
@@ -759,7 +775,7 @@ int32_t hipq_quantize_per_tensor_f32_carrier(hipq_ctx *ctx, const float *x, size
     HIPQ_ENTER(ctx);
     int32_t rc = check_scale(__func__, scale);
     if (rc) return rc;
-    if ((rc = check_mode(__func__, mode))) return rc;
+    if ((rc = check_mode(__func__, mode & ~HIPQ_FORM_INT_CAST))) return rc;
     if (qmin > qmax) return fail(HIPQ_INVALID_ARGUMENT, "%s: qmin %d > qmax %d", __func__, qmin, qmax);
     if (n == 0) return HIPQ_SUCCESS;
     HIPQ_REQUIRE_PTR(x);
@@ -810,7 +826,7 @@ int32_t hipq::quantize_dynamic_per_tensor(hipq_ctx *ctx, const float *x, size_t 
     HIPQ_REQUIRE_PTR(out_params);
     int32_t rc = check_mode(fn, mode);
     if (rc) return rc;
-    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_NN_ASYMMETRIC)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", fn, flavor);
     if (dtype != HIPQ_DTYPE_I8 && dtype != HIPQ_DTYPE_U8)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", fn, dtype);
@@ -996,10 +1012,12 @@ int32_t hipq_quantize_per_group_auto_f32_i8(hipq_ctx *ctx, const float *x, size_
                                             int32_t qmax, int32_t mode, int8_t *out, float *out_scales,
                                             int32_t *out_zero_points, int32_t *out_status) {
     HIPQ_ENTER(ctx);
-    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_ZERO_INCLUDED)
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_NN_ASYMMETRIC)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", __func__, flavor);
-    if (qmin < -128 || qmax > 127 || qmin >= qmax)
-        return fail(HIPQ_INVALID_ARGUMENT, "%s: range [%d, %d] must lie inside [-128, 127]", __func__, qmin, qmax);
+    // one byte per code: a signed range is stored as int8, an unsigned one (qmin >= 0) as the same byte read as uint8
+    if (qmin >= qmax || !((qmin >= -128 && qmax <= 127) || (qmin >= 0 && qmax <= 255)))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: range [%d, %d] must lie inside [-128, 127] or [0, 255]", __func__, qmin,
+                    qmax);
     return quantize_channels(__func__, ctx, x, outer, channels, inner, group_size, flavor, true, qmin, qmax, mode, out,
                              out_scales, out_zero_points, out_status);
 }

@@ -88,18 +88,13 @@ __device__ __forceinline__ float div_rn(float a, float b, float y) {
     return (r == r) ? q1 : q0;
 }
 
-// round(x * inv | x / scale) + zp, clamped; result still a float (the carrier).
-// DIV: `inv` is recip_for_div(scale); otherwise 1.0f / scale.
-template <bool DIV, int RND>
-__device__ __forceinline__ float quantize_value(float x, float scale, float inv, float zpf, float lo, float hi) {
-    float t;
-    if constexpr (DIV)
-        t = div_rn(x, scale, inv);
-    else
-        t = x * inv;
-    float q = round_mode<RND>(t) + zpf;
-    return clamp_keep_nan(q, lo, hi);
-}
+// The reference's "quantize one value" formulas differ in where the zero point enters:
+//   FORM 0  round(x * (1/scale)) + zp     crates/torsh-quantization/src/simd_ops.rs:36-46
+//   FORM 1  round(x / scale) + zp         crates/torsh-quantization/src/algorithms.rs:230-233, 302-305
+//   FORM 2  round(x / scale + zp)         crates/torsh-core/src/dtype/quantized.rs:129-134 (QInt8 / QUInt8)
+//   FORM 3  (round(x / scale) as i32) + zp   crates/torsh-nn/src/quantization/ops.rs:153-162 (NaN -> 0 before zp)
+// A bool first argument reads as FORM 0 / 1.  `inv` is recip_for_div(scale) for the division forms, else 1/scale.
+enum { QFORM_MUL = 0, QFORM_DIV = 1, QFORM_DIV_ZP_FIRST = 2, QFORM_DIV_INT_CAST = 3 };
 
 // Saturating f32 -> i32 with NaN -> 0: exactly Rust's `as i32`, and exactly what
 // v_cvt_i32_f32 does.  Inline asm so the conversion is never treated as undefined for
@@ -110,18 +105,44 @@ __device__ __forceinline__ int cvt_i32_sat(float v) {
     return r;
 }
 
+// The quantized value, clamped; result still a float (the carrier).
+template <int FORM, int RND>
+__device__ __forceinline__ float quantize_value(float x, float scale, float inv, float zpf, float lo, float hi) {
+    float t;
+    if constexpr (FORM != QFORM_MUL)
+        t = div_rn(x, scale, inv);
+    else
+        t = x * inv;
+    float q;
+    if constexpr (FORM == QFORM_DIV_ZP_FIRST)
+        q = round_mode<RND>(t + zpf);
+    else if constexpr (FORM == QFORM_DIV_INT_CAST)
+        q = static_cast<float>(cvt_i32_sat(round_mode<RND>(t))) + zpf;  // clamped to a small range next
+    else
+        q = round_mode<RND>(t) + zpf;
+    return clamp_keep_nan(q, lo, hi);
+}
+
 // Integer form of quantize_value for int8/uint8 outputs: the clamp is done after the
 // conversion, on integers (round(..)+zp is integral, so converting first changes nothing;
 // a NaN becomes 0 as `NaN.clamp(..) as i8` does, and +-Inf saturate).  About half the
 // vector instructions of the float-clamp form.
-template <bool DIV, int RND>
+template <int FORM, int RND>
 __device__ __forceinline__ int quantize_int(float x, float scale, float inv, float zpf, int lo, int hi) {
     float t;
-    if constexpr (DIV)
+    if constexpr (FORM != QFORM_MUL)
         t = div_rn(x, scale, inv);
     else
         t = x * inv;
-    const int q = cvt_i32_sat(round_mode<RND>(t) + zpf);
+    int q;
+    if constexpr (FORM == QFORM_DIV_ZP_FIRST) {
+        q = cvt_i32_sat(round_mode<RND>(t + zpf));
+    } else if constexpr (FORM == QFORM_DIV_INT_CAST) {
+        // i32 sum of the reference; the inner clamp keeps it from wrapping and changes nothing after the outer one
+        q = min(max(cvt_i32_sat(round_mode<RND>(t)), -(1 << 30)), 1 << 30) + static_cast<int>(zpf);
+    } else {
+        q = cvt_i32_sat(round_mode<RND>(t) + zpf);
+    }
     return min(max(q, lo), hi);
 }
 
@@ -170,6 +191,8 @@ __device__ __forceinline__ float wave_max(float v) {
 //   HIPQ_PARAMS_BACKEND_SYMMETRIC  crates/torsh-backend/src/quantization/params.rs:323-340
 //   HIPQ_PARAMS_BACKEND_ASYMMETRIC crates/torsh-backend/src/quantization/params.rs:343-363
 //   HIPQ_PARAMS_ZERO_INCLUDED      crates/torsh-quantization/src/observers.rs:263-310, specialized.rs:39-48, 322-335
+//   HIPQ_PARAMS_NN_SYMMETRIC       crates/torsh-nn/src/quantization/ops.rs:322-325 (no guards: a zero range gives scale 0)
+//   HIPQ_PARAMS_NN_ASYMMETRIC      crates/torsh-nn/src/quantization/ops.rs:326-330 (zero point not clamped)
 __device__ __forceinline__ int params_from_minmax(float mn, float mx, int flavor, int qmin_i, int qmax_i,
                                                   float *scale, int *zp) {
     const bool finite = (fabsf(mn) <= FLT_MAX) && (fabsf(mx) <= FLT_MAX);  // false for NaN and Inf
@@ -222,6 +245,16 @@ __device__ __forceinline__ int params_from_minmax(float mn, float mx, int flavor
         if (s == 0.0f) s = 1.0f;
         *scale = s;
         *zp = f32_as_i32(fminf(fmaxf(roundf(qmin - mn / s), qmin), qmax));
+        return HIPQ_SUCCESS;
+    }
+    case HIPQ_PARAMS_NN_SYMMETRIC: {
+        *scale = fmaxf(fabsf(mx), fabsf(mn)) / 127.0f;
+        return HIPQ_SUCCESS;
+    }
+    case HIPQ_PARAMS_NN_ASYMMETRIC: {
+        const float s = (mx - mn) / 255.0f;
+        *scale = s;
+        *zp = f32_as_i32(roundf(-mn / s));
         return HIPQ_SUCCESS;
     }
     default:

@@ -20,8 +20,11 @@ SUCCESS, INVALID_ARGUMENT, SHAPE_ERROR, DIMENSION_MISMATCH, DEVICE_ERROR, ALLOCA
 ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
 ROUND_FLOOR_HALF_UP = 16  # hipq_quantize_per_tensor_f32_i8 only
 FORM_MUL_INV, FORM_DIV = 0, 2
+FORM_ZP_BEFORE_ROUND = 32  # round(x / scale + zp): the scalar quantized types of torsh-core
+FORM_INT_CAST = 64         # (round(x / scale) as i32) + zp: torsh-nn's quantize_value_*; carrier output only
 DTYPE_I8, DTYPE_U8 = 0, 1
 PARAMS_SYMMETRIC, PARAMS_AFFINE, PARAMS_BACKEND_SYMMETRIC, PARAMS_BACKEND_ASYMMETRIC, PARAMS_ZERO_INCLUDED = range(5)
+PARAMS_NN_SYMMETRIC, PARAMS_NN_ASYMMETRIC = 5, 6
 FAKE_INT_CAST = 4
 FAKE_NAN_TO_QMIN = 8
 HISTOGRAM_MAX_BINS = 16384

@@ -16,6 +16,7 @@
 //                     -> bias + requantize to int8 with a calibrated output scale (operations.rs:716-724)
 #pragma once
 
+#include <cmath>
 #include <map>
 
 #include "core.hpp"
@@ -119,6 +120,7 @@ class QuantizedLinear : public Module {
             q.bias_ = std::move(db);
             q.has_bias_ = true;
         }
+        TORSH_CHECK(q.pack());
         return std::move(q);
     }
 
@@ -159,6 +161,7 @@ class QuantizedLinear : public Module {
             q.bias_ = std::move(db);
             q.has_bias_ = true;
         }
+        TORSH_CHECK(q.pack());
         return std::move(q);
     }
     Result<quantization::QuantizedWeights> to_quantized_weights() const {
@@ -193,22 +196,29 @@ class QuantizedLinear : public Module {
         std::vector<size_t> out_dims = d;
         out_dims.back() = out_;
         if (m == 0) return TorshError::invalid_argument("Cannot quantize empty tensor");
+        // The reference refuses a range that is not finite before it quantizes (algorithms.rs:403-407);
+        // min / max skip a NaN (simd_ops.rs:95-108), so only an infinity makes the range non-finite.  The
+        // device call is asynchronous and could only answer with NaN outputs, so the check is made here.
+        for (float v : input.as_slice())
+            if (std::isinf(v)) return TorshError::invalid_argument("Min and max values must be finite");
         TORSH_TRY(dx, hip::DeviceBuffer::from_host(ctx_, input.as_slice().data(), input.numel()));
         TORSH_TRY(dy, hip::DeviceBuffer::alloc(ctx_, m * out_ * sizeof(float)));
         // Activations follow the reference's branch for their size: x*(1/scale) above 64 elements
         // (algorithms.rs:292), x/scale otherwise; per-token always divides (algorithms.rs:230).
         const int32_t mode = (act_ == ActivationQuant::PerTensor && m * in_ > 64) ? HIPQ_FORM_MUL_INV : HIPQ_FORM_DIV;
         if (static_scale_ > 0.0f) {
-            TORSH_CHECK(hip::check(hipq_linear_static_f32(ctx_, dx.as<float>(), static_scale_, w_.as<int8_t>(),
-                                                          sw_.as<float>(), has_bias_ ? bias_.as<float>() : nullptr, m,
-                                                          out_, in_, mode, dy.as<float>())));
+            TORSH_CHECK(hip::check(hipq_linear_static_packed_f32(ctx_, dx.as<float>(), static_scale_,
+                                                                 wp_.as<int8_t>(), sw_.as<float>(),
+                                                                 has_bias_ ? bias_.as<float>() : nullptr, m, out_, in_,
+                                                                 mode, dy.as<float>())));
             TORSH_TRY(ys, dy.to_host<float>(m * out_));
             return Tensor::from_data(std::move(ys), std::move(out_dims));
         }
-        TORSH_CHECK(hip::check(hipq_linear_dynamic_f32(ctx_, dx.as<float>(), act_ == ActivationQuant::PerToken ? 1 : 0,
-                                                       w_.as<int8_t>(), sw_.as<float>(),
-                                                       has_bias_ ? bias_.as<float>() : nullptr, m, out_, in_, mode,
-                                                       dy.as<float>())));
+        TORSH_CHECK(hip::check(hipq_linear_dynamic_packed_f32(ctx_, dx.as<float>(),
+                                                              act_ == ActivationQuant::PerToken ? 1 : 0,
+                                                              wp_.as<int8_t>(), sw_.as<float>(),
+                                                              has_bias_ ? bias_.as<float>() : nullptr, m, out_, in_,
+                                                              mode, dy.as<float>())));
         TORSH_TRY(y, dy.to_host<float>(m * out_));
         return Tensor::from_data(std::move(y), std::move(out_dims));
     }
@@ -247,10 +257,20 @@ class QuantizedLinear : public Module {
 
   private:
     QuantizedLinear() = default;
+    // Weight preparation, once per layer: the int8 rows in the operand order of the matrix cores, which is
+    // what the forward reads; the row-major copy stays for parameters() and save().
+    Result<Unit> pack() {
+        size_t bytes = 0;
+        TORSH_CHECK(hip::check(hipq_packed_size(out_, in_, &bytes)));
+        TORSH_TRY(dp, hip::DeviceBuffer::alloc(ctx_, bytes));
+        TORSH_CHECK(hip::check(hipq_pack_rows_i8(ctx_, w_.as<int8_t>(), out_, in_, dp.as<int8_t>())));
+        wp_ = std::move(dp);
+        return Unit{};
+    }
     hipq_ctx *ctx_ = nullptr;
     size_t in_ = 0, out_ = 0;
     ActivationQuant act_ = ActivationQuant::PerTensor;
-    hip::DeviceBuffer w_, sw_, bias_;
+    hip::DeviceBuffer w_, wp_, sw_, bias_;
     bool has_bias_ = false;
     float static_scale_ = 0.0f;  // > 0: calibrated activation scale
 };

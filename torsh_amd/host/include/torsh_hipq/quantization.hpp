@@ -338,28 +338,6 @@ inline Result<Unit> quantize_with_cache_optimization(const std::vector<float> &i
     return quantize_per_tensor_affine_simd(input, scale, zero_point, output);
 }
 
-// algorithms.rs:677-708 (advice about a CPU's caches; kept for callers that print it).
-inline std::vector<std::string> get_cache_optimization_recommendations(size_t tensor_size, size_t element_size,
-                                                                       const CacheAwareParams &cache_params) {
-    std::vector<std::string> r;
-    const size_t total_bytes = tensor_size * element_size;
-    if (total_bytes <= cache_params.l1_cache_size) {
-        r.push_back("Tensor fits in L1 cache - use simple sequential access");
-    } else if (total_bytes <= cache_params.l2_cache_size) {
-        r.push_back("Tensor fits in L2 cache - consider blocked algorithms");
-    } else if (total_bytes <= cache_params.l3_cache_size) {
-        r.push_back("Tensor fits in L3 cache - use tiled processing with medium blocks");
-    } else {
-        r.push_back("Large tensor - use streaming algorithms with prefetching");
-        r.push_back("Consider parallel processing to utilize multiple cache hierarchies");
-    }
-    const size_t per_line = cache_params.cache_line_size / element_size;
-    if (tensor_size % per_line != 0)
-        r.push_back("Consider padding to align with cache lines (" + std::to_string(cache_params.cache_line_size) +
-                    "B boundaries)");
-    return r;
-}
-
 // simd_ops.rs:264-272
 struct TensorStats {
     float min = 0, max = 0, mean = 0, std_dev = 0, variance = 0;
@@ -429,18 +407,6 @@ inline Result<Unit> quantize_mobile_optimized(const std::vector<float> &input, f
     output = std::move(q);
     return Unit{};
 }
-
-// simd_ops.rs:274-298, 449-471: what the reference reports on its default x86-64 build.
-inline bool is_simd_available() { return detail::is_simd_available(); }
-inline size_t get_simd_width() { return 4; }
-struct MobileOptimizationHints {
-    bool prefer_int8 = true;
-    bool use_reduced_precision = false;
-    size_t optimal_chunk_size = 512;
-    bool enable_fast_math = true;
-    bool prefer_sequential = false;
-};
-inline MobileOptimizationHints get_mobile_optimization_hints() { return MobileOptimizationHints{}; }
 
 // ---- tensor-level functions (algorithms.rs) ----
 

@@ -264,7 +264,9 @@ inline uint64_t fnv1a64(const unsigned char *p, size_t n, uint64_t h = 146959810
     return h;
 }
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
-constexpr char kWeightMagic[8] = {'T', 'Q', 'H', 'I', 'P', 'Q', 'W', '1'};
+constexpr char kWeightMagic[8] = {'T', 'Q', 'H', 'I', 'P', 'Q', 'W', '2'};
+// a * b without wrapping; false when the product does not fit
+inline bool mul_fits(uint64_t a, uint64_t b, uint64_t *out) { return !__builtin_mul_overflow(a, b, out); }
 }  // namespace detail
 
 inline Result<Unit> save_quantized_weights(const QuantizedWeights &w, const std::string &path) {
@@ -287,7 +289,9 @@ inline Result<Unit> save_quantized_weights(const QuantizedWeights &w, const std:
     std::memcpy(buf.data() + off_w, w.weight.data(), w.weight.size());
     std::memcpy(buf.data() + off_s, w.scales.data(), w.scales.size() * sizeof(float));
     if (!w.bias.empty()) std::memcpy(buf.data() + off_b, w.bias.data(), w.bias.size() * sizeof(float));
-    const uint64_t sum = detail::fnv1a64(buf.data() + 256, total - 256);
+    // the checksum covers the header too (its own field counted as zero), so a damaged dimension or offset is
+    // caught before it is used
+    const uint64_t sum = detail::fnv1a64(buf.data(), total);
     std::memcpy(buf.data() + 80, &sum, 8);
     std::ofstream f(path, std::ios::binary | std::ios::trunc);
     if (!f) return TorshError::invalid_argument("Failed to open " + path + " for writing");
@@ -311,17 +315,30 @@ inline Result<QuantizedWeights> load_quantized_weights(const std::string &path) 
     std::memcpy(offs, buf.data() + 48, 32);
     std::memcpy(&sum, buf.data() + 80, 8);
     if (offs[3] != buf.size()) return bad("length field does not match the file (truncated?)");
-    if (detail::fnv1a64(buf.data() + 256, buf.size() - 256) != sum) return bad("checksum mismatch");
+    {
+        std::vector<unsigned char> zeroed(buf.begin(), buf.begin() + 256);
+        std::memset(zeroed.data() + 80, 0, 8);
+        const uint64_t h = detail::fnv1a64(buf.data() + 256, buf.size() - 256, detail::fnv1a64(zeroed.data(), 256));
+        if (h != sum) return bad("checksum mismatch");
+    }
     QuantizedWeights w;
     if (kind != QuantizedWeights::Linear && kind != QuantizedWeights::Conv2d) return bad("unknown weight kind");
     w.kind = static_cast<QuantizedWeights::Kind>(kind);
     const size_t nd = kind == QuantizedWeights::Linear ? 2 : 4;
     for (size_t i = 0; i < nd; ++i) w.dims.push_back(static_cast<size_t>(dims[i]));
-    const size_t rows = w.rows(), len = w.row_len();
-    if (rows == 0 || len == 0 || len > buf.size() / rows) return bad("implausible dims");
+    // every product and sum below is checked: the fields come from the file
+    uint64_t len64 = 1;
+    for (size_t i = 1; i < nd; ++i)
+        if (!detail::mul_fits(len64, dims[i], &len64)) return bad("implausible dims");
+    const uint64_t rows64 = dims[0], size = buf.size();
+    uint64_t wbytes = 0, fbytes = 0;
+    if (rows64 == 0 || len64 == 0 || !detail::mul_fits(rows64, len64, &wbytes) || wbytes > size ||
+        !detail::mul_fits(rows64, sizeof(float), &fbytes) || fbytes > size)
+        return bad("implausible dims");
+    const size_t rows = static_cast<size_t>(rows64), len = static_cast<size_t>(len64);
     const bool has_bias = (flags & 1u) != 0;
-    if (offs[0] + rows * len > buf.size() || offs[1] + rows * sizeof(float) > buf.size() ||
-        (has_bias && offs[2] + rows * sizeof(float) > buf.size()))
+    auto inside = [&](uint64_t off, uint64_t need) { return off >= 256 && off <= size && need <= size - off; };
+    if (!inside(offs[0], wbytes) || !inside(offs[1], fbytes) || (has_bias && !inside(offs[2], fbytes)))
         return bad("section outside the file");
     w.weight.assign(reinterpret_cast<const int8_t *>(buf.data() + offs[0]),
                     reinterpret_cast<const int8_t *>(buf.data() + offs[0]) + rows * len);
