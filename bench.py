@@ -48,10 +48,31 @@ def measured_gemm_traffic():
     return None
 
 
+SPINUP_MS = 40.0  # --spinup-ms
+
+
+def spin_up(fn, ms: float) -> None:
+    """Runs fn() back to back for `ms` milliseconds, untimed.  After an idle period (start of the process, the CPU
+    baseline) the device needs a few tens of milliseconds of sustained work before its clocks reach the level they
+    hold under load: the same GEMM launch takes 17.2 us in the first 5 ms and 14.9 us from ~30 ms on.  Every timed
+    region below starts after such a spin-up, so the figures are the sustained ones a serving loop sees."""
+    import torch
+
+    if ms <= 0:
+        return
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(32):
+            fn()
+        torch.cuda.synchronize()
+
+
 def event_time_ms(fn, reps: int, warmup: int) -> float:
     """Average duration of fn() in ms, HIP events on torch's current stream (the stream the kernels use)."""
     import torch
 
+    spin_up(fn, SPINUP_MS)
     for _ in range(warmup):
         fn()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -102,6 +123,56 @@ def cpu_baseline(m: int, n: int, k: int):
     }
 
 
+def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
+    """Phase budget of the packed GEMM kernel from its own clock stamps (hipq_ctx_set_trace_buffer): 200 launches on
+    rotating operand sets; for every launch the median over its 1024 waves of each phase, then the median and the
+    spread of that over the launches.  Cycles are shader-clock cycles; the clock rate is what the stamps of the
+    constant 100 MHz counter give for the same interval."""
+    import torch
+
+    sets, reps = 32, 200
+    pa = [ctx.pack_rows(torch.randint(-128, 128, (M, K), generator=g, device="cuda", dtype=torch.int8))
+          for _ in range(sets)]
+    pw = [ctx.pack_rows(torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8))
+          for _ in range(sets)]
+    sw = torch.rand(N, generator=g, device="cuda") * 1e-3
+    bias = torch.randn(N, generator=g, device="cuda") * 0.01
+    sa = torch.full((1,), 0.03, device="cuda")
+    outs = [torch.empty(M, N, device="cuda") for _ in range(sets)]
+    waves = ((M + 127) // 128) * ((N + 63) // 64) * 4
+    trace = torch.zeros(reps, waves, 8, dtype=torch.int64, device="cuda")
+    for i in range(20):
+        ctx.linear_packed_i8_f32(pa[i % sets], sa, pw[i % sets], sw, bias, M, N, K, out=outs[i % sets])
+    for i in range(reps):
+        ctx.set_trace_buffer(trace[i])
+        ctx.linear_packed_i8_f32(pa[i % sets], sa, pw[i % sets], sw, bias, M, N, K, out=outs[i % sets])
+    ctx.set_trace_buffer(None)
+    ctx.synchronize()
+    t = trace.cpu().double()
+    names = ["start -> first operands in registers", "K loop (first operands -> last MFMA retired)",
+             "4-way K-split sum through LDS (incl. waiting for the slowest wave)", "convert + issue stores",
+             "stores retired", "whole wave"]
+    spans = [(0, 1), (1, 2), (2, 3), (3, 4), (4, 5), (0, 5)]
+    ghz = (t[:, :, 5] - t[:, :, 0]) / ((t[:, :, 7] - t[:, :, 6]).clamp(min=1) * 10.0) / 1e0  # cycles per ns
+    clock = ghz.median(dim=1).values
+    print(f"packed GEMM M={M} N={N} K={K}: {reps} launches x {waves} waves; shader clock during the kernel "
+          f"{clock.median():.2f} GHz (launch medians {clock.min():.2f} .. {clock.max():.2f})")
+    print(f"{'phase':72s} {'cycles (median of launch medians)':>34s} {'min .. max':>18s} {'us at that clock':>17s}")
+    for name, (a, b) in zip(names, spans):
+        d = (t[:, :, b] - t[:, :, a]).median(dim=1).values
+        print(f"{name:72s} {d.median():34.0f} {d.min():8.0f} .. {d.max():6.0f} {d.median() / clock.median() / 1e3:17.2f}")
+    skew = (t[:, :, 2].view(reps, -1, 4).max(dim=2).values - t[:, :, 2].view(reps, -1, 4).min(dim=2).values)
+    print(f"{'skew between the four waves of a workgroup at the end of the K loop':72s} "
+          f"{skew.median(dim=1).values.median():34.0f}")
+    # Across workgroups only the constant 100 MHz counter is comparable (10 ns steps).
+    first = t[:, :, 6].min(dim=1, keepdim=True).values
+    last_start = (t[:, :, 6] - first).max(dim=1).values * 0.01
+    span = (t[:, :, 7].max(dim=1).values - first[:, 0]) * 0.01
+    print(f"last wave of the grid starts {last_start.median():.2f} us after the first; first wave start -> last wave "
+          f"end {span.median():.2f} us (launches: {span.min():.2f} .. {span.max():.2f})")
+    return 0
+
+
 def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
     """A handful of launches of one kernel on HBM-cold operands, for rocprofv3 --pmc / --kernel-trace passes.
 
@@ -113,6 +184,8 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
 
     g = torch.Generator(device="cuda").manual_seed(2)
     reps = 20
+    if which == "gemm_phases":
+        return gemm_phase_table(ctx, M, N, K, g)
     if which in ("gemm", "gemm_rowmajor"):
         aq = [torch.randint(-128, 128, (M, K), generator=g, device="cuda", dtype=torch.int8) for _ in range(reps)]
         wq = [torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8) for _ in range(reps)]
@@ -245,16 +318,20 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
 
 
 def main() -> int:
+    global SPINUP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--spinup-ms", type=float, default=SPINUP_MS,
+                    help="milliseconds of untimed back-to-back launches before each timed region (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "gemm_rowmajor", "step", "quantize", "calib", "special", "copy",
+    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "gemm_rowmajor", "step", "quantize", "calib", "special", "copy",
                                           "stack", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
+    SPINUP_MS = args.spinup_ms
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (no collectives are part of it).",
               file=sys.stderr)
@@ -294,6 +371,7 @@ def main() -> int:
         it[0] += 1
         ctx.linear_dynamic_packed(xs[i], pw[i], sw[i], bias, per_token=False, mode=hipq.FORM_MUL_INV, out=outs[i])
 
+    spin_up(step, SPINUP_MS)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -339,6 +417,7 @@ def main() -> int:
             "M": M, "N": N, "K": K,
             "rounding": "half-away-from-zero (reference f32::round)",
             "operand_pool": f"{pool} rotating weight/activation/output sets (HBM-cold)",
+            "spinup_ms": SPINUP_MS,
         },
         "roofline": {
             "kernel": "gemm_i8_packed_kernel (int8 MFMA GEMM on fragment-packed operands + dequant/bias epilogue)",

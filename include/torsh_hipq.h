@@ -318,6 +318,14 @@ HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
  * handing back a wrong product silently.  `limit` is the number of polls after the first look
  * (negative = the default, 2^20); 0 lets a test see the error path without hanging anything. */
 HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
+/* Tuning aid with no counterpart in the reference.  While a device buffer is set, hipq_linear_packed_i8_f32
+ * (and the forwards built on it) run a form of the packed GEMM kernel in which every wave records the shader
+ * clock at six points - start, first operands in registers, end of the K loop, partial sums reduced, stores
+ * issued, stores retired - followed by the constant 100 MHz counter at the first and the last point, as uint64
+ * values [workgroup][wave 0..3][8], provided the buffer holds ceil(m/128) * ceil(n/64) * 4 * 8 * 8 bytes
+ * (otherwise the ordinary kernel runs).  The results are the same
+ * bits.  null removes the buffer.  bench.py --profile gemm_phases prints the phase table from it. */
+HIPQ_API int32_t hipq_ctx_set_trace_buffer(hipq_ctx *ctx, void *device_buffer, size_t bytes);
 /* Whole forward of a quantized Linear with a static (calibrated) activation scale: the scale an
  * observer derived beforehand (Observer::calculate_qparams, crates/torsh-quantization/src/observers.rs:263-310,
  * symmetric: zero point 0) instead of a range pass over every input - per-tensor quantize

@@ -173,6 +173,13 @@ int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit) {
     return HIPQ_SUCCESS;
 }
 
+int32_t hipq_ctx_set_trace_buffer(hipq_ctx *ctx, void *device_buffer, size_t bytes) {
+    HIPQ_REQUIRE_PTR(ctx);
+    ctx->trace = device_buffer;
+    ctx->trace_bytes = device_buffer ? bytes : 0;
+    return HIPQ_SUCCESS;
+}
+
 void *hipq_ctx_stream(hipq_ctx *ctx) { return ctx ? static_cast<void *>(ctx->stream) : nullptr; }
 
 int32_t hipq_device_malloc(hipq_ctx *ctx, size_t bytes, void **out_ptr) {

@@ -39,7 +39,15 @@ struct GemmEpilogue {
     // (owned by the context) in which a give-up is recorded.
     int spin_limit = 1 << 20;
     uint32_t *wait_error = nullptr;
+    // Packed kernel, tuning aid: when set, every wave records the shader clock at its phase boundaries
+    // (kTraceWords values per wave, workgroup-major: kTracePoints shader-clock stamps, then the constant
+    // 100 MHz counter at the first and the last of them).
+    unsigned long long *trace = nullptr;
+    // Packed kernel: 1 = the activations were written by the kernel just before this one on the stream
+    // (still in the memory-side cache), so the XCDs need not be kept from reading the same lines at once.
+    int fresh_activations = 0;
 };
+constexpr int kTracePoints = 6, kTraceWords = 8;
 
 // Host-side twin of recip_for_div: the correctly rounded 1/b if it is a normal number, else 0.
 static inline float host_recip_for_div(float b) {
@@ -106,13 +114,28 @@ __device__ __forceinline__ void epilogue_store4(const GemmEpilogue &ep, int m, i
 // N = 4096: all 4 row blocks x 8 weight panels, each weight panel read from HBM by one XCD only;
 // for a tall M x 256 product: 8 row blocks x all 4 panels, instead of every XCD streaming half
 // of the tall operand).
+// a / d and a % d for small non-negative wave-uniform values; a power of two (the usual case) costs a
+// shift instead of the ~25 instructions of an integer division, which sit in front of a kernel's first load.
+__device__ __forceinline__ void divmod_uniform(int a, int d, int *q, int *r) {
+    if ((d & (d - 1)) == 0) {
+        *q = a >> (__builtin_ffs(d) - 1);
+        *r = a & (d - 1);
+    } else {
+        *q = a / d;
+        *r = a % d;
+    }
+}
+
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int gm, int gn, int *tm, int *tn) {
     const int b = blockIdx.x;
     if (gm > 0) {
-        const int x = b % 8, i = b / 8;     // XCD, index within the XCD's rectangle
-        const int blocks_m = tiles_m / gm;  // rectangles along M
-        *tm = (x % blocks_m) * gm + i % gm;
-        *tn = (x / blocks_m) * gn + i / gm;
+        const int x = b % 8, i = b / 8;  // XCD, index within the XCD's rectangle
+        int blocks_m, unused, xq, xr, iq, ir;   // rectangles along M
+        divmod_uniform(tiles_m, gm, &blocks_m, &unused);
+        divmod_uniform(x, blocks_m, &xq, &xr);
+        divmod_uniform(i, gm, &iq, &ir);
+        *tm = xr * gm + ir;
+        *tn = xq * gn + iq;
         return;
     }
     *tm = b % tiles_m;

@@ -17,6 +17,8 @@
 // partial accumulators (through LDS, integer adds, order independent).
 #pragma once
 
+#include <type_traits>
+
 #include "hipq_gemm_kernels.h"
 
 namespace hipq {
@@ -31,6 +33,64 @@ __host__ __device__ inline size_t packed_bytes(size_t rows, size_t k) {
     return packed_row_blocks(rows) * packed_k_blocks(k) * 1024;
 }
 
+// fp32 / int32 epilogue of one 32-row block that lies wholly inside the output (first row `row0`, first
+// column `n0`): the same arithmetic as store_tile, without per-element bounds checks and with buffer
+// stores whose row and column-block offsets are scalar, so that an output costs a convert, a multiply,
+// an add and a store instead of a predicate, a branch and a 64-bit address as well.
+template <int TNB, int EPI>
+__device__ __forceinline__ void store_block_interior(v16i (&own)[1][TNB], const GemmEpilogue &ep, int N, int row0,
+                                                     int n0, int lane, const float (&swv)[TNB],
+                                                     const float (&bv)[TNB], float sa0) {
+    static_assert(EPI == EPI_F32 || EPI == EPI_I32, "interior epilogue: fp32 or int32 output");
+    // 4-byte elements: a row block spans at most (31 * N + 64) * 4 bytes from its first element, far below
+    // the 2 GiB a buffer offset can hold for any N the entry points accept.
+    char *base = static_cast<char *>(ep.out) + (size_t(row0) * N + n0) * 4;
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
+    const int voff = (4 * (lane / 32) * N + lane % 32) * 4;
+    const int row_bytes = N * 4;
+    auto put = [&](int r, int j, int bits) {
+        __builtin_amdgcn_raw_buffer_store_b32(bits, ro, voff, (8 * (r / 4) + (r % 4)) * row_bytes + j * 128, /*nt*/ 2);
+    };
+    if constexpr (EPI == EPI_I32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+            for (int j = 0; j < TNB; ++j) put(r, j, own[0][j][r]);
+    } else {
+        const bool has_bias = ep.bias != nullptr;
+        auto emit = [&](auto scale_of, auto with_bias) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+#pragma unroll
+                for (int j = 0; j < TNB; ++j) {
+                    float v = static_cast<float>(own[0][j][r]) * scale_of(r, j);
+                    if constexpr (decltype(with_bias)::value) v = v + bv[j];
+                    put(r, j, __builtin_bit_cast(int, v));
+                }
+        };
+        if (ep.sa_per_row) {
+            float s_row[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_row[r] = ep.sa[row0 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4)];
+            wait_vmcnt<0>();
+            auto sc = [&](int r, int j) { return s_row[r] * swv[j]; };
+            if (has_bias)
+                emit(sc, std::true_type{});
+            else
+                emit(sc, std::false_type{});
+        } else {
+            float s_comb[TNB];
+#pragma unroll
+            for (int j = 0; j < TNB; ++j) s_comb[j] = sa0 * swv[j];
+            auto sc = [&](int, int j) { return s_comb[j]; };
+            if (has_bias)
+                emit(sc, std::true_type{});
+            else
+                emit(sc, std::false_type{});
+        }
+    }
+}
+
 // TMB x TNB row blocks of 32 per workgroup tile; D register stages of (TMB + TNB) KiB per wave in
 // flight.  Loads are buffer loads with a constant per-lane offset and scalar (SGPR) fragment
 // offsets, so the loop spends no vector instruction on addressing.
@@ -38,8 +98,13 @@ __host__ __device__ inline size_t packed_bytes(size_t rows, size_t k) {
 // Sibling tiles (same weight panel, different tile_m) run on CUs of one XCD at the same time; each
 // starts its K loop a quarter of the way further on (`rot`), so the four of them miss on
 // different weight lines and every line is fetched from HBM by one of them and found in the L2 by
-// the other three, instead of all four waiting on the same miss.
-template <int TMB, int TNB, int D, int EPI, bool EVEN>
+// the other three, instead of all four waiting on the same miss.  The activation rows of a tile_m
+// are read by all 8 XCDs (each has its own L2): every XCD starts a further (steps/8 | 1) steps on, so
+// that the eight do not ask memory for the same lines at the same moment (17.9 -> 16.5 us at
+// M = 512, N = K = 4096 with operands from HBM; with 32 steps every (tile_m, XCD) pair starts on a
+// different step).  Activations that the previous kernel has just written are served by the memory-side
+// cache, where the same stagger costs 0.4 us instead: the fused forwards switch it off.
+template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false>
 __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__restrict__ PA,
                                                              const int8_t *__restrict__ PW, int M, int N, int K,
                                                              GemmEpilogue ep) {
@@ -53,6 +118,14 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     const int m0 = tile_m * TMB * 32, n0 = tile_n * TNB * 32;
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // TRACE: shader-clock stamps at the phase boundaries of this wave (start, first operands in registers,
+    // end of the K loop, partial sums reduced, stores issued, stores retired).
+    unsigned long long stamp[kTraceWords] = {};
+    auto mark = [&](int i) {
+        if constexpr (TRACE) stamp[i] = __builtin_readcyclecounter();
+    };
+    if constexpr (TRACE) stamp[kTracePoints] = __builtin_amdgcn_s_memrealtime();
+    mark(0);
 
     // Epilogue operands first: their latency hides behind the main loop.
     float swv[TNB], bv[TNB], sa0 = 1.0f;
@@ -75,10 +148,14 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     // the matrix repeat the last one: computed and discarded).  Operands are below 2 GiB.
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PA), 0, 0x7fffffff, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PW), 0, 0x7fffffff, 0x00020000);
+    // A wave numbers the tile's row blocks from the one it will own after the K-split sum: its block i is
+    // row block (wave + i) % TMB of the tile.  Every wave then runs the same code on the same registers
+    // (block 0 is kept, blocks 1.. are handed over), with no wave-dependent branch in the epilogue.
+    static_assert(TMB == WK, "one row block per K-split wave");
     int soa[TMB], sow[TNB];
 #pragma unroll
     for (int i = 0; i < TMB; ++i) {
-        int rb = tile_m * TMB + i;
+        int rb = tile_m * TMB + (wave + i) % TMB;
         rb = rb < rbA ? rb : rbA - 1;
         soa[i] = (rb * KB + wave) * 1024;
     }
@@ -89,7 +166,8 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
         sow[j] = (rb * KB + wave) * 1024;
     }
     const int steps = KB / WK;  // k blocks per wave
-    const int rot = (tile_m % 4) * (steps / 4);
+    int rot = (tile_m % 4) * (steps / 4) + (ep.fresh_activations ? 0 : int(blockIdx.x % 8) * ((steps / 8) | 1));
+    while (rot >= steps) rot -= steps;  // at most a few rounds; cheaper than a division in front of the first load
     const int voff = lane * 16;
 
     v4i fa[D][TMB], fb[D][TNB];
@@ -123,6 +201,10 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     // steps is a positive multiple of D (the host picks D so).
 #pragma unroll
     for (int u = 0; u < D; ++u) issue(u, u);
+    if constexpr (TRACE) {
+        wait_vmcnt<(D - 1) * (TMB + TNB)>();  // the first stage has landed
+        mark(1);
+    }
     for (int s0 = D; s0 < steps; s0 += D) {
 #pragma unroll
         for (int u = 0; u < D; ++u) {
@@ -132,10 +214,69 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     }
 #pragma unroll
     for (int u = 0; u < D; ++u) compute(u);
+    if constexpr (TRACE) {
+        // the last MFMA has retired once its result can be read
+        asm volatile("s_nop 15\n\ts_nop 15" ::"v"(acc[TMB - 1][TNB - 1][0]));
+        mark(2);
+    }
 
-    // wave `wave` holds the partial sums of its k blocks for the whole tile
-    ksplit_reduce<TMB, TNB, WK, false>(acc, lds, wave, 0, lane);
-    store_tile<TMB, TNB, WK, EPI, EVEN>(acc, ep, M, N, m0, wave, lane, nn, swv, bv, sa0);
+    // Wave `wave` holds the partial sums of its k blocks for the whole tile.  Block i (i >= 1) goes to its
+    // owner, wave (wave + i) % TMB, through LDS: [owner][slot i-1][column block][4 registers][lane] of 16
+    // bytes; the three writers of one owner use three different slots.  Integer adds: any order, same bits.
+    v4i *red = reinterpret_cast<v4i *>(lds);
+#pragma unroll
+    for (int i = 1; i < TMB; ++i) {
+        const int owner = (wave + i) % TMB;
+        v4i *dst = red + ((owner * (TMB - 1) + (i - 1)) * TNB * 4) * kWave + lane;
+#pragma unroll
+        for (int j = 0; j < TNB; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                dst[(j * 4 + g) * kWave] =
+                    v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+    }
+    __syncthreads();
+    // All reads first (the operand registers of the loop are free), then the adds: the LDS pipe streams
+    // instead of paying its latency once per pair of reads.
+    v4i part[TMB - 1][TNB][4];
+    const v4i *src = red + (wave * (TMB - 1) * TNB * 4) * kWave + lane;
+#pragma unroll
+    for (int sl = 0; sl < TMB - 1; ++sl)
+#pragma unroll
+        for (int j = 0; j < TNB; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) part[sl][j][g] = src[((sl * TNB + j) * 4 + g) * kWave];
+    __builtin_amdgcn_sched_barrier(0);
+    v16i own[1][TNB];
+#pragma unroll
+    for (int j = 0; j < TNB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            int v = acc[0][j][r];
+#pragma unroll
+            for (int sl = 0; sl < TMB - 1; ++sl) v += part[sl][j][r / 4][r % 4];
+            own[0][j][r] = v;
+        }
+    mark(3);
+    const int row0 = m0 + wave * 32;
+    bool interior = false;
+    if constexpr (EPI != EPI_I8) interior = m0 + TMB * 32 <= M && n0 + TNB * 32 <= N && ep.residual == nullptr;
+    if (interior) {
+        if constexpr (EPI != EPI_I8) store_block_interior<TNB, EPI>(own, ep, N, row0, n0, lane, swv, bv, sa0);
+    } else {
+        store_tile<1, TNB, 1, EPI, EVEN>(own, ep, M, N, row0, 0, lane, nn, swv, bv, sa0);
+    }
+    if constexpr (TRACE) {
+        mark(4);
+        wait_vmcnt<0>();
+        mark(5);
+        stamp[kTracePoints + 1] = __builtin_amdgcn_s_memrealtime();
+        if (lane == 0) {
+            unsigned long long *t = ep.trace + (size_t(blockIdx.x) * WK + wave) * kTraceWords;
+#pragma unroll
+            for (int i = 0; i < kTraceWords; ++i) t[i] = stamp[i];
+        }
+    }
 }
 
 // Row-major int8 [rows, k] -> packed.  One wave per fragment: a lane copies the 16 bytes of its
@@ -165,11 +306,11 @@ __global__ __launch_bounds__(256) void pack_rows_i8_kernel(const int8_t *__restr
     }
 }
 
-template <int TMB, int TNB, int D, int EPI, bool EVEN>
+template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false>
 static int32_t launch_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                              const GemmEpilogue &ep) {
     constexpr int kLds = TMB * TNB * 3 * 4096;
-    auto kernel = gemm_i8_packed_kernel<TMB, TNB, D, EPI, EVEN>;
+    auto kernel = gemm_i8_packed_kernel<TMB, TNB, D, EPI, EVEN, TRACE>;
     static bool configured[16] = {false};  // per device: raise the dynamic LDS limit once
     if (ctx->device < 16 && !configured[ctx->device]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -182,6 +323,7 @@ static int32_t launch_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, 
     const int tiles_m = ((M + 31) / 32 + TMB - 1) / TMB, tiles_n = ((N + 31) / 32 + TNB - 1) / TNB;
     GemmEpilogue placed = ep;
     pick_xcd_rectangle(tiles_m, tiles_n, TMB * 32, TNB * 32, &placed.xcd_gm, &placed.xcd_gn);
+    if constexpr (TRACE) placed.trace = static_cast<unsigned long long *>(ctx->trace);
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(256), kLds, ctx->stream, pa, pw, M, N, K, placed);
     return check_launch("gemm_i8 (packed)");
 }
@@ -192,6 +334,13 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
                                   const GemmEpilogue &ep) {
     const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
     const int steps = static_cast<int>(packed_k_blocks(k)) / 4;
+    if constexpr (EPI == EPI_F32 && !EVEN) {
+        // Phase stamps (hipq_ctx_set_trace_buffer): the depth-4 fp32 form only, and only when the buffer holds
+        // every wave's record.
+        const size_t tiles = ((packed_row_blocks(m) + 3) / 4) * ((packed_row_blocks(n) + 1) / 2);
+        if (ctx->trace && steps % 4 == 0 && ctx->trace_bytes >= tiles * 4 * kTraceWords * sizeof(unsigned long long))
+            return launch_packed<4, 2, 4, EPI, EVEN, true>(ctx, pa, pw, M, N, K, ep);
+    }
     if (steps % 4 == 0) return launch_packed<4, 2, 4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     if (steps % 2 == 0) return launch_packed<4, 2, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     return launch_packed<4, 2, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);

@@ -81,6 +81,16 @@ int32_t hipq_gemm_packed_i8_i32(hipq_ctx *ctx, const int8_t *a_packed, const int
     return launch_gemm_packed<EPI_I32, false>(ctx, a_packed, w_packed, m, n, k, ep);
 }
 
+// The GEMM launch of hipq_linear_packed_i8_f32 (arguments already checked); `fresh`: a_packed was written by the
+// kernel launched just before on this stream.
+static int32_t linear_packed_launch(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                    int32_t a_scale_per_row, const int8_t *w_packed, const float *w_scales,
+                                    const float *bias, size_t m, size_t n, size_t k, float *out, bool fresh) {
+    GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, 1.0f, 0, out};
+    ep.fresh_activations = fresh ? 1 : 0;
+    return launch_gemm_packed<EPI_F32, false>(ctx, a_packed, w_packed, m, n, k, ep);
+}
+
 int32_t hipq_linear_packed_i8_f32(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
                                   int32_t a_scale_per_row, const int8_t *w_packed, const float *w_scales,
                                   const float *bias, size_t m, size_t n, size_t k, float *out) {
@@ -94,8 +104,7 @@ int32_t hipq_linear_packed_i8_f32(hipq_ctx *ctx, const int8_t *a_packed, const f
     HIPQ_REQUIRE_PTR(w_scales);
     HIPQ_REQUIRE_PTR(a_packed);
     HIPQ_REQUIRE_PTR(w_packed);
-    GemmEpilogue ep{a_scale, a_scale_per_row ? 1 : 0, w_scales, bias, 1.0f, 0, out};
-    return launch_gemm_packed<EPI_F32, false>(ctx, a_packed, w_packed, m, n, k, ep);
+    return linear_packed_launch(ctx, a_packed, a_scale, a_scale_per_row, w_packed, w_scales, bias, m, n, k, out, false);
 }
 
 int32_t hipq_linear_packed_i8_i8(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale, int32_t a_scale_per_row,
@@ -159,12 +168,12 @@ int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t pe
         rc = quantize_activations_per_row(ctx, x, m, k, mode & HIPQ_ROUND_HALF_EVEN, qa, row_scales);
         if (rc) return rc;
         if ((rc = pack_rows(ctx, qa, m, k, pa))) return rc;
-        return hipq_linear_packed_i8_f32(ctx, pa, row_scales, 1, w_packed, w_scales, bias, m, n, k, out);
+        return linear_packed_launch(ctx, pa, row_scales, 1, w_packed, w_scales, bias, m, n, k, out, true);
     }
     rc = quantize_activations_per_tensor(ctx, x, m, k, true, 1.0f, mode, true, pa, params, base + L.partials,
                                          L.scales - L.partials);
     if (rc) return rc;
-    return hipq_linear_packed_i8_f32(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out);
+    return linear_packed_launch(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out, true);
 }
 
 int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_scale, const int8_t *w_packed,
@@ -188,7 +197,7 @@ int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_sca
     int8_t *pa = reinterpret_cast<int8_t *>(base + L.packed);
     rc = quantize_activations_per_tensor(ctx, x, m, k, false, a_scale, mode, true, pa, params, nullptr, 0);
     if (rc) return rc;
-    return hipq_linear_packed_i8_f32(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out);
+    return linear_packed_launch(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out, true);
 }
 
 }  // extern "C"

@@ -25,6 +25,9 @@ struct hipq_ctx {
     // HIPQ_GEMM_VARIANT environment variable) and the spin limit of the persistent kernel's waits.
     int gemm_variant = -1;
     int wait_spin_limit = 1 << 20;
+    // Tuning aid (hipq_ctx_set_trace_buffer): caller-owned device memory for the packed GEMM's phase stamps.
+    void *trace = nullptr;
+    size_t trace_bytes = 0;
 };
 
 namespace hipq {

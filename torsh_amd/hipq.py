@@ -122,6 +122,7 @@ _SIGNATURES = {
     "hipq_quantize_static_per_tensor_f32_i8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp, _vp],
     "hipq_set_gemm_kernel_variant": [_vp, _i32],
     "hipq_ctx_set_wait_spin_limit": [_vp, _i32],
+    "hipq_ctx_set_trace_buffer": [_vp, _vp, _sz],
     "hipq_linear_static_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_add_layer_norm_quantize_f32_i8": [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
@@ -233,6 +234,13 @@ class Context:
     def set_gemm_kernel_variant(self, variant: int) -> None:
         """Test / tuning hook: force one GEMM kernel form for later calls (0 = automatic)."""
         self.call("hipq_set_gemm_kernel_variant", int(variant))
+
+    def set_trace_buffer(self, buf: Optional[torch.Tensor]) -> None:
+        """Tuning aid: phase stamps of the packed GEMM go to `buf` (int64 device tensor) until None is set."""
+        if buf is None:
+            self.call("hipq_ctx_set_trace_buffer", None, 0)
+        else:
+            self.call("hipq_ctx_set_trace_buffer", _ptr(buf), buf.numel() * buf.element_size())
 
     def set_wait_spin_limit(self, limit: int) -> None:
         """Test hook: polls a bounded wait of the persistent GEMM kernel makes before it gives up (< 0: default)."""
