@@ -141,8 +141,14 @@ def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
     outs = [torch.empty(M, N, device="cuda") for _ in range(sets)]
     waves = ((M + 127) // 128) * ((N + 63) // 64) * 4
     trace = torch.zeros(reps, waves, 8, dtype=torch.int64, device="cuda")
-    for i in range(20):
-        ctx.linear_packed_i8_f32(pa[i % sets], sa, pw[i % sets], sw, bias, M, N, K, out=outs[i % sets])
+    cnt = [0]
+
+    def untraced():
+        i = cnt[0] % sets
+        cnt[0] += 1
+        ctx.linear_packed_i8_f32(pa[i], sa, pw[i], sw, bias, M, N, K, out=outs[i])
+
+    spin_up(untraced, SPINUP_MS)
     for i in range(reps):
         ctx.set_trace_buffer(trace[i])
         ctx.linear_packed_i8_f32(pa[i % sets], sa, pw[i % sets], sw, bias, M, N, K, out=outs[i % sets])

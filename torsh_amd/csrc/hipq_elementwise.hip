@@ -279,8 +279,22 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__
     // The first fragment's floats are requested before the parameters are resolved (a fold of the range
     // partials and two workgroup barriers in a dynamic call): the loads do not depend on the scale, and a
     // launch of this size is bound by latency, not by bandwidth.
+    // frag -> (row block, k block) without a 64-bit division where it can be avoided: it would sit, with
+    // its ~100 instructions, in front of the kernel's first load.
+    const bool kb_pow2 = (KB & (KB - 1)) == 0, frag32 = nfrag + fstep < (size_t(1) << 32);
+    const int kb_shift = __builtin_ffsll(static_cast<long long>(KB)) - 1;
     auto whole = [&](size_t frag, size_t *row, size_t *k0) {
-        const size_t rb = frag / KB, kb = frag % KB;
+        size_t rb, kb;
+        if (kb_pow2) {
+            rb = frag >> kb_shift;
+            kb = frag & (KB - 1);
+        } else if (frag32) {
+            rb = static_cast<uint32_t>(frag) / static_cast<uint32_t>(KB);
+            kb = static_cast<uint32_t>(frag) - static_cast<uint32_t>(rb) * static_cast<uint32_t>(KB);
+        } else {
+            rb = frag / KB;
+            kb = frag % KB;
+        }
         *row = rb * 32 + lane % 32;
         *k0 = kb * 32 + 16 * (lane / 32);
         return vec && frag < nfrag && *row < rows && *k0 + 16 <= cols;
