@@ -241,3 +241,28 @@ def test_packed_argument_errors(ctx, hipq):
         ctx.call("hipq_gemm_packed_i8_i32", a.data_ptr(), a.data_ptr(), 1 << 20, 4, 4096, out.data_ptr())
     assert e.value.code == hipq.SHAPE_ERROR
     ctx.call("hipq_gemm_packed_i8_i32", a.data_ptr(), a.data_ptr(), 0, 4, 16, None)  # empty M: no-op
+
+
+def test_phase_stamps_do_not_change_the_product(ctx, hipq, oracle):
+    """hipq_ctx_set_trace_buffer: the stamped form of the kernel gives the same bits, every wave of the grid
+    writes its record (six increasing shader-clock values, then the 100 MHz counter at the first and the last of
+    them), and a buffer that is too small leaves the ordinary kernel in place."""
+    m, n, k = 256, 192, 1024
+    x, bias, wq, sw, aq, sa, acc, want = _linear_case(oracle, m, n, k, False, 77)
+    pa, pw = ctx.pack_rows(dev(aq)), ctx.pack_rows(dev(wq))
+    plain = host(ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(bias), m, n, k))
+    waves = ((m + 127) // 128) * ((n + 63) // 64) * 4
+    trace = torch.zeros(waves, 8, dtype=torch.int64, device="cuda")
+    ctx.set_trace_buffer(trace)
+    try:
+        stamped = host(ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(bias), m, n, k))
+        ctx.set_trace_buffer(trace[:1])  # too small: ignored
+        small = host(ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(bias), m, n, k))
+    finally:
+        ctx.set_trace_buffer(None)
+    np.testing.assert_array_equal(stamped, plain)
+    np.testing.assert_array_equal(small, plain)
+    t = trace.cpu().numpy()
+    assert (t[:, :6] > 0).all()
+    assert (np.diff(t[:, :6], axis=1) >= 0).all()
+    assert (t[:, 7] >= t[:, 6]).all()
