@@ -123,6 +123,27 @@ def cpu_baseline(m: int, n: int, k: int):
     }
 
 
+def conv_phase_table(ctx, g) -> int:
+    """Phase budget of the convolution's implicit GEMM ([32,256,14,14] x [256,256,3,3]) from the kernel's clock
+    stamps, as gemm_phase_table."""
+    import torch
+
+    xc = [torch.randint(0, 256, (32, 256, 14, 14), generator=g, device="cuda", dtype=torch.uint8) for _ in range(8)]
+    wc = torch.randint(-128, 128, (256, 256, 3, 3), generator=g, device="cuda", dtype=torch.int8)
+    swc = torch.rand(256, generator=g, device="cuda") * 1e-3
+    bc = torch.randn(256, generator=g, device="cuda") * 0.01
+    oc = torch.empty(32, 256, 14, 14, dtype=torch.int8, device="cuda")
+    packed, sums = ctx.conv2d_pack_weights(wc)
+    cnt = [0]
+
+    def forward():
+        cnt[0] += 1
+        ctx.conv2d_i8_packed(xc[cnt[0] % 8], 0, 0.02, packed, sums, (3, 3), swc, bc, 0.05, 0, (1, 1), out=oc)
+
+    waves = 2 * 128 * 4  # 256 filters / 128 x 8192 padded windows / 64 tiles, four waves each
+    return phase_table("conv2d implicit GEMM M=256 N=8192 K=2304", ctx, forward, waves)
+
+
 def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
     """Phase budget of the packed GEMM kernel from its own clock stamps (hipq_ctx_set_trace_buffer): 200 launches on
     rotating operand sets; for every launch the median over its 1024 waves of each phase, then the median and the
@@ -140,18 +161,26 @@ def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
     sa = torch.full((1,), 0.03, device="cuda")
     outs = [torch.empty(M, N, device="cuda") for _ in range(sets)]
     waves = ((M + 127) // 128) * ((N + 63) // 64) * 4
-    trace = torch.zeros(reps, waves, 8, dtype=torch.int64, device="cuda")
     cnt = [0]
 
-    def untraced():
+    def launch():
         i = cnt[0] % sets
         cnt[0] += 1
         ctx.linear_packed_i8_f32(pa[i], sa, pw[i], sw, bias, M, N, K, out=outs[i])
 
-    spin_up(untraced, SPINUP_MS)
+    return phase_table(f"packed GEMM M={M} N={N} K={K}", ctx, launch, waves, reps)
+
+
+def phase_table(title: str, ctx, launch, waves: int, reps: int = 200) -> int:
+    """Runs `launch` (one call = one launch of the packed kernel) `reps` times with the trace buffer set and prints
+    the phase medians."""
+    import torch
+
+    trace = torch.zeros(reps, waves, 8, dtype=torch.int64, device="cuda")
+    spin_up(launch, SPINUP_MS)
     for i in range(reps):
         ctx.set_trace_buffer(trace[i])
-        ctx.linear_packed_i8_f32(pa[i % sets], sa, pw[i % sets], sw, bias, M, N, K, out=outs[i % sets])
+        launch()
     ctx.set_trace_buffer(None)
     ctx.synchronize()
     t = trace.cpu().double()
@@ -161,7 +190,7 @@ def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
     spans = [(0, 1), (1, 2), (2, 3), (3, 4), (4, 5), (0, 5)]
     ghz = (t[:, :, 5] - t[:, :, 0]) / ((t[:, :, 7] - t[:, :, 6]).clamp(min=1) * 10.0) / 1e0  # cycles per ns
     clock = ghz.median(dim=1).values
-    print(f"packed GEMM M={M} N={N} K={K}: {reps} launches x {waves} waves; shader clock during the kernel "
+    print(f"{title}: {reps} launches x {waves} waves; shader clock during the kernel "
           f"{clock.median():.2f} GHz (launch medians {clock.min():.2f} .. {clock.max():.2f})")
     print(f"{'phase':72s} {'cycles (median of launch medians)':>34s} {'min .. max':>18s} {'us at that clock':>17s}")
     for name, (a, b) in zip(names, spans):
@@ -192,6 +221,8 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
     reps = 20
     if which == "gemm_phases":
         return gemm_phase_table(ctx, M, N, K, g)
+    if which == "conv_phases":
+        return conv_phase_table(ctx, g)
     if which in ("gemm", "gemm_rowmajor"):
         aq = [torch.randint(-128, 128, (M, K), generator=g, device="cuda", dtype=torch.int8) for _ in range(reps)]
         wq = [torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8) for _ in range(reps)]
@@ -333,7 +364,7 @@ def main() -> int:
                     help="milliseconds of untimed back-to-back launches before each timed region (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "gemm_rowmajor", "step", "quantize", "calib", "special", "copy",
+    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "conv_phases", "gemm_rowmajor", "step", "quantize", "calib", "special", "copy",
                                           "stack", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()

@@ -426,13 +426,15 @@ HIPQ_API int32_t hipq_conv2d_u8i8_f32(hipq_ctx *ctx, const uint8_t *x, int32_t z
                                       const float *w_scales, const float *bias, size_t nb, size_t c, size_t h, size_t wd,
                                       size_t oc, size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
                                       size_t pad_w, float *out);
-/* One-time filter preparation for the stride-1 fast path: int8 [OC,IC,KH,KW]
- * -> [OC,KH*KW,IC] (same byte count) and the per-filter sums w_sums[oc]
- * (offline weight preparation; no reference counterpart, the reference keeps
- * filters as stored). */
+/* One-time filter preparation for the stride-1 fast path (offline weight preparation; no reference
+ * counterpart, the reference keeps filters as stored): int8 [OC,IC,KH,KW] -> the packed row operand of the
+ * matrix-core GEMM with K ordered (tap, channel), and the per-filter sums w_sums[oc].  `packed` is device
+ * memory of hipq_conv2d_packed_weights_size bytes (>= OC*IC*KH*KW: rows are padded to 32, K to 128),
+ * 16-byte aligned. */
+HIPQ_API int32_t hipq_conv2d_packed_weights_size(size_t oc, size_t ic, size_t kh, size_t kw, size_t *out_bytes);
 HIPQ_API int32_t hipq_conv2d_pack_weights_i8(hipq_ctx *ctx, const int8_t *w, size_t oc, size_t ic, size_t kh, size_t kw,
                                              int8_t *packed, int32_t *w_sums);
-/* hipq_conv2d_u8i8_i8 on prepared filters (stride 1, channels a multiple of 128). */
+/* hipq_conv2d_u8i8_i8 on prepared filters (stride 1, channels a multiple of 32). */
 HIPQ_API int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, float s_in,
                                             const int8_t *w_packed, const int32_t *w_sums, const float *w_scales,
                                             const float *bias, size_t nb, size_t c, size_t h, size_t wd, size_t oc,

@@ -16,8 +16,13 @@ def host(t):
 
 
 GEOMS = [
-    # nb, c, h, w, oc, k, stride, pad, zp      (fast path: stride 1 and c % 128 == 0)
+    # nb, c, h, w, oc, k, stride, pad, zp      (fast path: stride 1 and c % 32 == 0)
     (1, 128, 5, 5, 8, 3, (1, 1), (1, 1), 0),
+    (3, 96, 10, 9, 40, 3, (1, 1), (1, 1), 77),     # three channel blocks: the tap walk wraps on a non-power of two
+    (2, 32, 20, 20, 70, 5, (1, 1), (2, 2), 255),   # one channel block, 25 taps
+    (1, 64, 33, 40, 8, 1, (1, 1), (0, 0), 1),      # 1x1: a plain matrix product over the pixels
+    (1, 32, 70, 60, 33, 3, (1, 1), (1, 0), 128),   # padded rows of 60 pixels: the layout pass works in five bands
+    (2, 160, 6, 5, 129, 2, (1, 1), (0, 1), 60),    # even kernel, k blocks padded up to a multiple of four
     (2, 128, 7, 6, 130, 3, (1, 1), (1, 1), 17),
     (1, 256, 6, 6, 64, 1, (1, 1), (0, 0), 3),
     (2, 128, 9, 8, 40, 5, (1, 1), (2, 2), 200),
@@ -58,7 +63,8 @@ def _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, seed):
     return x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out, out_f
 
 
-@pytest.mark.parametrize("nb,c,h,w,oc,k,pad", [(2, 128, 14, 14, 64, 3, 1), (1, 256, 7, 7, 33, 3, 1), (3, 16, 10, 10, 8, 3, 1)])
+@pytest.mark.parametrize("nb,c,h,w,oc,k,pad", [(2, 128, 14, 14, 64, 3, 1), (1, 256, 7, 7, 33, 3, 1), (3, 16, 10, 10, 8, 3, 1),
+                                               (2, 96, 9, 11, 48, 3, 1)])
 def test_quantized_conv2d_forward(ctx, hipq, oracle, nb, c, h, w, oc, k, pad):
     """The Conv2d configuration ([32,256,14,14], 3x3) at reduced size: asymmetric u8 activations, per-channel int8 filters, fused bias + requant."""
     x, wf, bias, s_in, zp_in, xq, wq, sw, acc2d, s_out, out_f = _quantized_conv_case(oracle, nb, c, h, w, oc, k, pad, c + oc)
@@ -79,7 +85,7 @@ def test_quantized_conv2d_forward(ctx, hipq, oracle, nb, c, h, w, oc, k, pad):
             oracle.set_round_mode(0)
         got = host(ctx.conv2d_i8(dq, zp_in, s_in, dwq, dsw, dev(bias), s_out, -2, (1, 1), (pad, pad), mode))
         np.testing.assert_array_equal(got.reshape(acc2d.shape), want)
-        if c % 128 == 0:
+        if c % 32 == 0:
             packed, sums = ctx.conv2d_pack_weights(dwq)
             got = host(ctx.conv2d_i8_packed(dq, zp_in, s_in, packed, sums, (k, k), dsw, dev(bias), s_out, -2, (pad, pad), mode))
             np.testing.assert_array_equal(got.reshape(acc2d.shape), want)

@@ -1,14 +1,16 @@
 // Quantized Conv2d forward: u8 activations (NCHW) x per-channel int8 filters ->
 // int32 accumulators -> requantized int8 (NCHW), bias fused.
 //
-// Fast path (stride 1, channels a multiple of 128): an im2col-free implicit GEMM
-// on the pipelined MFMA kernel.  The activations are rewritten once as signed
-// bytes (x - 128) in a zero-point-padded NHWC image, so that for every filter tap
-// the K-slice of the "window matrix" is a plain strided matrix (consecutive
-// windows start one pixel apart) and the kernel's global->LDS fills need no
-// gather.  Shifting by 128 lets the signed int8 MFMA multiply unsigned
-// activations; the shift and the zero point are undone in the epilogue with the
-// per-filter weight sum:  sum (x - zp) w = sum (x - 128) w + (128 - zp) sum w,
+// Fast path (stride 1, channels a multiple of 32): an im2col-free implicit GEMM on the
+// fragment-packed MFMA kernel (hipq_gemm_packed.h, CONV).  The activations are rewritten
+// once as signed bytes (x - 128) in a zero-point-padded image stored as
+// [channel block of 32][pixel][32 bytes]: consecutive pixels of one channel block are 32
+// bytes apart, so the 32 windows of an MFMA fragment, shifted by any filter tap, are one
+// contiguous KiB that a wave loads with a single coalesced instruction, straight into the
+// operand registers (no LDS, no gather).  The filters are packed once in the GEMM's
+// fragment order with K = (tap, channel).  Shifting by 128 lets the signed int8 MFMA
+// multiply unsigned activations; the shift and the zero point are undone in the epilogue
+// with the per-filter weight sum:  sum (x - zp) w = sum (x - 128) w + (128 - zp) sum w,
 // and a border pixel holds exactly zp so padded taps contribute nothing.
 // Everything else runs through a direct per-output kernel (correct, not fast).
 #include "hipq_gemm_kernels.h"
@@ -17,43 +19,48 @@ namespace hipq {
 
 constexpr int kConvThreads = 256;
 
-// u8 NCHW -> i8 NHWC with a border of `pad` pixels holding (zp - 128).  One workgroup per
-// padded image row: the C x W source bytes of that row (W-byte runs, one per channel) are
-// transposed through LDS so that the NHWC row is written as 16-byte pieces; one extra
-// workgroup clears the slack behind the last image that the last windows read into.
-// C % 16 == 0.  Dynamic LDS: W * (C + 16) bytes.
-__global__ __launch_bounds__(kConvThreads) void conv_pack_input_kernel(const uint8_t *__restrict__ x, int C, int H, int W,
+// u8 NCHW -> i8 [channel block][padded pixel][32] with a border of `pad` pixels holding (zp - 128); pixel
+// index = (n * hp + y) * wp + x, `pixels` of them per channel block (the real ones, then zeroed slack that
+// the last windows read into).  One thread per (channel block, padded pixel): it reads its pixel's byte from
+// each of the block's 32 channel planes (consecutive lanes are consecutive pixels: consecutive bytes of a
+// plane row), all 32 loads in flight at once, and writes the 32 bytes as two 16-byte stores (a wave writes
+// 2 KiB contiguous).  x - 128 on a byte is a flip of its top bit.  No LDS.  The last cbs workgroups clear
+// the slack.  C % 32 == 0.
+__global__ __launch_bounds__(kConvThreads) void conv_pack_image_kernel(const uint8_t *__restrict__ x, int C, int H, int W,
                                                                          int pad_h, int pad_w, int zp, int nb,
-                                                                         int8_t *__restrict__ out, size_t slack) {
-    extern __shared__ __attribute__((aligned(16))) int8_t tile[];  // [W][C + 16]
-    const int hp_count = H + 2 * pad_h, wp_count = W + 2 * pad_w;
-    const uint32_t border4 = static_cast<uint32_t>(static_cast<uint8_t>(zp - 128)) * 0x01010101u;
-    if (static_cast<int>(blockIdx.x) == nb * hp_count) {
-        int8_t *tail = out + size_t(nb) * hp_count * wp_count * C;
-        for (size_t i = threadIdx.x; i < slack; i += kConvThreads) tail[i] = 0;
+                                                                         int groups_per_cb, int8_t *__restrict__ out,
+                                                                         int pixels) {
+    const int hp = H + 2 * pad_h, wp = W + 2 * pad_w, cbs = C / 32;
+    const int real_pixels = nb * hp * wp;
+    const int work = cbs * groups_per_cb;
+    if (static_cast<int>(blockIdx.x) >= work) {
+        const int cb = blockIdx.x - work;
+        uint4 *tail = reinterpret_cast<uint4 *>(out + (size_t(cb) * pixels + real_pixels) * 32);
+        for (int i = threadIdx.x; i < (pixels - real_pixels) * 2; i += kConvThreads) tail[i] = make_uint4(0, 0, 0, 0);
         return;
     }
-    const int n = blockIdx.x / hp_count, hp = blockIdx.x % hp_count;
-    const int h = hp - pad_h;
-    const bool row_inside = h >= 0 && h < H;
-    const int pitch = C + 16;
-    if (row_inside) {
-        const uint8_t *src = x + (size_t(n) * C * H + h) * W;  // + c * H * W + w
-        for (int e = threadIdx.x; e < C * W; e += kConvThreads) {
-            const int c = e / W, w = e % W;
-            tile[w * pitch + c] = static_cast<int8_t>(static_cast<int>(src[size_t(c) * H * W + w]) - 128);
-        }
+    const int cb = blockIdx.x / groups_per_cb;
+    const int p = (blockIdx.x % groups_per_cb) * kConvThreads + threadIdx.x;  // padded pixel of the whole batch
+    if (p >= real_pixels) return;
+    const int n = p / (hp * wp), rem = p % (hp * wp);
+    const int h = rem / wp - pad_h, w = rem % wp - pad_w;
+    const uint32_t border4 = static_cast<uint32_t>(static_cast<uint8_t>(zp - 128)) * 0x01010101u;
+    uint32_t d[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d[i] = border4;
+    if (h >= 0 && h < H && w >= 0 && w < W) {
+        const size_t plane = size_t(H) * W;
+        const uint8_t *src = x + ((size_t(n) * C + cb * 32) * H + h) * W + w;
+        uint32_t b[32];
+#pragma unroll
+        for (int c = 0; c < 32; ++c) b[c] = src[size_t(c) * plane];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            d[i] = (b[4 * i] | (b[4 * i + 1] << 8) | (b[4 * i + 2] << 16) | (b[4 * i + 3] << 24)) ^ 0x80808080u;
     }
-    __syncthreads();
-    uint4 *orow = reinterpret_cast<uint4 *>(out + (size_t(n) * hp_count + hp) * wp_count * C);
-    const int vec_per_pixel = C / 16;
-    for (int i = threadIdx.x; i < wp_count * vec_per_pixel; i += kConvThreads) {
-        const int wp = i / vec_per_pixel, cv = i % vec_per_pixel;
-        const int w = wp - pad_w;
-        uint4 v = make_uint4(border4, border4, border4, border4);
-        if (row_inside && w >= 0 && w < W) v = *reinterpret_cast<const uint4 *>(tile + w * pitch + cv * 16);
-        orow[i] = v;
-    }
+    uint4 *dst = reinterpret_cast<uint4 *>(out + (size_t(cb) * pixels + p) * 32);
+    dst[0] = make_uint4(d[0], d[1], d[2], d[3]);
+    dst[1] = make_uint4(d[4], d[5], d[6], d[7]);
 }
 
 // int8 [OC, IC, KH*KW] -> [OC, KH*KW, IC] and wsum[oc] = sum of the filter's weights.
@@ -140,36 +147,33 @@ static int32_t check_geom(const char *fn, const ConvGeom &g) {
     return HIPQ_SUCCESS;
 }
 
-static bool fast_path_ok(const ConvGeom &g) {
-    // (the layout pass stages one image row, w * (c + 16) bytes, in the default 64 KiB of LDS)
-    return g.sh == 1 && g.sw == 1 && g.c % 128 == 0 && g.c * g.kh * g.kw >= 256 && g.oc >= 1 &&
-           size_t(g.w) * (g.c + 16) <= 64 * 1024;
+// Pixels per channel block of the packed image: the padded grid, what the last windows' taps reach past it,
+// and the 32 windows of a fragment that starts at the last one.
+static size_t image_pixels(const ConvGeom &g) {
+    const size_t hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw;
+    const size_t reach = size_t(g.kh - 1) * wp + g.kw + 32;
+    return (size_t(g.nb) * hp * wp + reach + 31) / 32 * 32;
 }
 
-// Runs the implicit GEMM on an already packed image / filter pair.
-template <int EPI, bool EVEN>
-static int32_t run_implicit_gemm(hipq_ctx *ctx, const int8_t *ximg, const int8_t *wpacked, const int32_t *wsum,
-                                 int zp_in, const ConvGeom &g, float s_in, const float *sw, const float *bias,
-                                 float s_out, int zp_out, void *out) {
-    const int hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw;
-    GemmEpilogue ep{nullptr, 0, sw, bias, s_out, zp_out, out};
-    ep.s_out_inv = host_recip_for_div(s_out);
-    ep.sa_scalar = s_in;
-    ep.cv_tiles_per_tap = g.c / 128;
-    ep.cv_kw = g.kw;
-    ep.cv_wp = wp;
-    ep.cv_hp = hp;
-    ep.cv_c = g.c;
-    ep.cv_ho = g.ho;
-    ep.cv_wo = g.wo;
-    ep.cv_oc = g.oc;
-    ep.cv_wsum = wsum;
-    ep.cv_corr_mul = 128 - zp_in;
-    const int M = g.oc, N = g.nb * hp * wp, K = g.c * g.kh * g.kw;
-    return launch_pipe<128, 64, 6, 4, 2, 1, 2, EPI, EVEN, 1>(ctx, wpacked, ximg, M, N, K, ep);
+static bool fast_path_ok(const ConvGeom &g) {
+    const size_t k = size_t(g.c) * g.kh * g.kw;
+    // offsets into the packed image and the packed filters are 32-bit
+    return g.sh == 1 && g.sw == 1 && g.c % 32 == 0 && g.oc >= 1 &&
+           size_t(g.c / 32) * image_pixels(g) * 32 < (size_t(1) << 31) &&
+           packed_operand_bytes(g.oc, k) < (size_t(1) << 31);
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+// [OC, IC, taps] filters -> the GEMM's packed row operand with K = (tap, channel), and the per-filter sums.
+// `staging` holds OC * IC * taps bytes.
+static int32_t pack_filters(hipq_ctx *ctx, const int8_t *w, int oc, int ic, int taps, int8_t *staging, int8_t *packed,
+                            int32_t *wsum) {
+    hipLaunchKernelGGL(conv_pack_weights_kernel, dim3(oc), dim3(kConvThreads), 0, ctx->stream, w, ic, taps, staging, wsum);
+    int32_t rc = check_launch("conv_pack_weights");
+    if (rc) return rc;
+    return pack_rows(ctx, staging, size_t(oc), size_t(ic) * taps, packed);
+}
 
 template <int EPI, bool EVEN>
 static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int zp_in, float s_in, const int8_t *w,
@@ -185,29 +189,45 @@ static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int
                            ctx->stream, x, zp_in, w, g, s_in, sw, bias, s_out, zp_out, out);
         return check_launch(fn);
     }
-    const int hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw, taps = g.kh * g.kw;
-    // Windows near the end of the last image read up to (kh-1)*wp + kw-1 pixels past it.
-    const size_t img_bytes = size_t(g.nb) * hp * wp * g.c;
-    const size_t slack = (size_t(g.kh - 1) * wp + g.kw) * g.c + 1024;
-    const size_t w_bytes = size_t(g.oc) * g.c * taps;
+    const int hp = g.h + 2 * g.ph, wp = g.w + 2 * g.pw, taps = g.kh * g.kw, cbs = g.c / 32;
+    const size_t pixels = image_pixels(g);
+    const size_t img_bytes = size_t(cbs) * pixels * 32;
+    const size_t k = size_t(g.c) * taps;
+    const size_t w_bytes = wpacked ? 0 : align256(size_t(g.oc) * k) + align256(packed_operand_bytes(g.oc, k)) +
+                                             align256(size_t(g.oc) * 4);
     void *s = nullptr;
-    int32_t rc = scratch(ctx, kScratchHeader + align256(img_bytes + slack) + align256(w_bytes) + align256(g.oc * 4), &s);
+    int32_t rc = scratch(ctx, kScratchHeader + align256(img_bytes) + w_bytes, &s);
     if (rc) return rc;
     int8_t *ximg = reinterpret_cast<int8_t *>(static_cast<char *>(s) + kScratchHeader);
-    int8_t *wbuf = ximg + align256(img_bytes + slack);
-    int32_t *wsbuf = reinterpret_cast<int32_t *>(wbuf + align256(w_bytes));
-    const size_t pack_lds = size_t(g.w) * (g.c + 16);
-    hipLaunchKernelGGL(conv_pack_input_kernel, dim3(g.nb * hp + 1), dim3(kConvThreads), pack_lds, ctx->stream, x, g.c, g.h,
-                       g.w, g.ph, g.pw, zp_in, g.nb, ximg, slack);
+    const int groups_per_cb = (g.nb * hp * wp + kConvThreads - 1) / kConvThreads;
+    hipLaunchKernelGGL(conv_pack_image_kernel, dim3(cbs * groups_per_cb + cbs), dim3(kConvThreads), 0, ctx->stream, x, g.c,
+                       g.h, g.w, g.ph, g.pw, zp_in, g.nb, groups_per_cb, ximg, static_cast<int>(pixels));
+    if ((rc = check_launch(fn))) return rc;
     if (!wpacked) {
-        hipLaunchKernelGGL(conv_pack_weights_kernel, dim3(g.oc), dim3(kConvThreads), 0, ctx->stream, w, g.c, taps, wbuf,
-                           wsbuf);
-        wpacked = wbuf;
+        int8_t *staging = ximg + align256(img_bytes);
+        int8_t *pbuf = staging + align256(size_t(g.oc) * k);
+        int32_t *wsbuf = reinterpret_cast<int32_t *>(pbuf + align256(packed_operand_bytes(g.oc, k)));
+        if ((rc = pack_filters(ctx, w, g.oc, g.c, taps, staging, pbuf, wsbuf))) return rc;
+        wpacked = pbuf;
         wsum = wsbuf;
     }
-    rc = check_launch(fn);
-    if (rc) return rc;
-    return run_implicit_gemm<EPI, EVEN>(ctx, ximg, wpacked, wsum, zp_in, g, s_in, sw, bias, s_out, zp_out, out);
+    GemmEpilogue ep{nullptr, 0, sw, bias, s_out, zp_out, out};
+    ep.s_out_inv = host_recip_for_div(s_out);
+    ep.sa_scalar = s_in;
+    ep.cv_kw = g.kw;
+    ep.cv_wp = wp;
+    ep.cv_hp = hp;
+    ep.cv_c = g.c;
+    ep.cv_ho = g.ho;
+    ep.cv_wo = g.wo;
+    ep.cv_oc = g.oc;
+    ep.cv_nb = g.nb;
+    ep.cv_wsum = wsum;
+    ep.cv_corr_mul = 128 - zp_in;
+    ep.cv_pixels = static_cast<int>(pixels);
+    ep.cv_kblocks = taps * cbs;
+    ep.fresh_activations = 1;  // the image was written by the kernel just before
+    return conv_gemm_packed(ctx, wpacked, ximg, g.oc, g.nb * hp * wp, static_cast<int>(k), ep, EPI, EVEN);
 }
 
 static int32_t make_geom(const char *fn, size_t nb, size_t c, size_t h, size_t w, size_t oc, size_t kh, size_t kw,
@@ -233,6 +253,14 @@ using namespace hipq;
 
 extern "C" {
 
+int32_t hipq_conv2d_packed_weights_size(size_t oc, size_t ic, size_t kh, size_t kw, size_t *out_bytes) {
+    HIPQ_REQUIRE_PTR(out_bytes);
+    if (oc >> 24 || ic >> 24 || (kh * kw) >> 16 || (ic * kh * kw) >> 24)
+        return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    *out_bytes = packed_operand_bytes(oc, ic * kh * kw);
+    return HIPQ_SUCCESS;
+}
+
 int32_t hipq_conv2d_pack_weights_i8(hipq_ctx *ctx, const int8_t *w, size_t oc, size_t ic, size_t kh, size_t kw,
                                     int8_t *packed, int32_t *wsum) {
     HIPQ_ENTER(ctx);
@@ -240,10 +268,16 @@ int32_t hipq_conv2d_pack_weights_i8(hipq_ctx *ctx, const int8_t *w, size_t oc, s
     HIPQ_REQUIRE_PTR(w);
     HIPQ_REQUIRE_PTR(packed);
     HIPQ_REQUIRE_PTR(wsum);
-    if (oc >> 24 || ic >> 24 || (kh * kw) >> 16) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
-    hipLaunchKernelGGL(conv_pack_weights_kernel, dim3(static_cast<int>(oc)), dim3(kConvThreads), 0, ctx->stream, w,
-                       static_cast<int>(ic), static_cast<int>(kh * kw), packed, wsum);
-    return check_launch(__func__);
+    if (oc >> 24 || ic >> 24 || (kh * kw) >> 16 || (ic * kh * kw) >> 24)
+        return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    if (reinterpret_cast<uintptr_t>(packed) & 15u)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: the packed buffer must be 16-byte aligned", __func__);
+    void *s = nullptr;
+    int32_t rc = scratch(ctx, kScratchHeader + oc * ic * kh * kw, &s);
+    if (rc) return rc;
+    int8_t *staging = reinterpret_cast<int8_t *>(static_cast<char *>(s) + kScratchHeader);
+    return pack_filters(ctx, w, static_cast<int>(oc), static_cast<int>(ic), static_cast<int>(kh * kw), staging, packed,
+                        wsum);
 }
 
 int32_t hipq_conv2d_u8i8_i32(hipq_ctx *ctx, const uint8_t *x, int32_t zp_in, const int8_t *w, size_t nb, size_t c,
@@ -317,7 +351,7 @@ int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int32_t zp_i
     int32_t rc = make_geom(__func__, nb, c, h, wd, oc, kh, kw, 1, 1, pad_h, pad_w, &g);
     if (rc) return rc;
     if (!fast_path_ok(g))
-        return fail(HIPQ_INVALID_ARGUMENT, "%s: packed filters need stride 1 and channels a multiple of 128", __func__);
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: packed filters need stride 1 and channels a multiple of 32", __func__);
     if (nb != 0 && oc != 0) {
         HIPQ_REQUIRE_PTR(w_packed);
         HIPQ_REQUIRE_PTR(w_sums);

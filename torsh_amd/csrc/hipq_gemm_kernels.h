@@ -22,14 +22,15 @@ struct GemmEpilogue {
     int zp_out;
     void *out;  // int32 / float / int8 [M,N]
     const float *residual = nullptr;  // fp32 epilogue only: added after the bias, [M,N]; may alias out
-    // Implicit-GEMM convolution (pipelined kernel, CONV = 1): the column operand is a padded
-    // NHWC int8 image [nb, hp, wp, c]; column q is the window whose top-left tap is padded
-    // pixel q, and K runs over (tap, channel).  The row operand holds the packed filters.
-    int cv_tiles_per_tap = 0;  // c / 128
+    // Implicit-GEMM convolution (packed kernel, CONV): the row operand holds the packed filters, the column
+    // operand is the padded int8 image as [channel block of 32][pixel][32 bytes]; column q is the window whose
+    // top-left tap is padded pixel q = (n * hp + y) * wp + x, and K runs over (tap, channel).
     int cv_kw = 0, cv_wp = 0, cv_hp = 0, cv_c = 0;
-    int cv_ho = 0, cv_wo = 0, cv_oc = 0;
+    int cv_ho = 0, cv_wo = 0, cv_oc = 0, cv_nb = 0;
     const int32_t *cv_wsum = nullptr;  // [oc] sum of the filter's int8 weights
     int cv_corr_mul = 0;               // 128 - zp_in: accumulator += cv_corr_mul * cv_wsum[oc]
+    int cv_pixels = 0;                 // pixels per channel block of the image buffer (with slack)
+    int cv_kblocks = 0;                // taps * (c / 32): the k blocks that hold data
     float sa_scalar = 1.0f;            // activation scale used when sa is null
     float s_out_inv = 0.0f;            // recip_for_div(s_out), or 0 to divide directly (requantize only)
     // Tiles per XCD along M and N (pipelined kernel): the 8 XCDs each take a gm x gn rectangle of
@@ -48,6 +49,15 @@ struct GemmEpilogue {
     int fresh_activations = 0;
 };
 constexpr int kTracePoints = 6, kTraceWords = 8;
+
+// Defined with the packed kernel (hipq_gemm_packed.hip), used by the convolution.
+// Row-major int8 [rows, k] -> fragment-packed operand (packed_operand_bytes(rows, k) bytes at dst).
+int32_t pack_rows(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_t *dst);
+size_t packed_operand_bytes(size_t rows, size_t k);
+// Implicit-GEMM convolution: `filters` packed [M = output channels, K = taps x channels], `image` in
+// [channel block][pixel][32] order, N = padded pixels; ep carries the cv_* geometry.  epi: EPI_I32 / _F32 / _I8.
+int32_t conv_gemm_packed(hipq_ctx *ctx, const int8_t *filters, const int8_t *image, int M, int N, int K,
+                         const GemmEpilogue &ep, int epi, bool even);
 
 // Host-side twin of recip_for_div: the correctly rounded 1/b if it is a normal number, else 0.
 static inline float host_recip_for_div(float b) {
@@ -497,7 +507,7 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[FM][FN], const GemmEpilog
 // wave while the texture path is busy, so mixing fills and MFMAs in one wave
 // serialises the two pipes; with the roles split, MFMA issue never waits behind a
 // memory instruction.  All waves meet at one barrier per K-tile.
-template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN, int CONV = 0>
+template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN>
 __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kernel(const int8_t *__restrict__ A,
                                                                                     const int8_t *__restrict__ W,
                                                                                     int M, int N, int K,
@@ -531,13 +541,11 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     if (wave < PW) {
         // ---------------- producer ----------------
         const int8_t *src[IPW];
-        bool col_side[IPW];
 #pragma unroll
         for (int j = 0; j < IPW; ++j) {
             const int q = wave * IPW + j;
             const int trow = q * RPI + lane / CPR;  // row in the stacked [A rows | W rows] tile
             const int col = (lane % CPR) ^ ((trow >> 1) & 7);
-            col_side[j] = trow >= BM;
             if (trow < BM) {
                 int gm = m0 + trow;
                 gm = gm < M ? gm : M - 1;  // rows past the edge are computed and discarded
@@ -545,22 +553,16 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
             } else {
                 int gn = n0 + (trow - BM);
                 gn = gn < N ? gn : N - 1;
-                // CONV: consecutive windows start one pixel (c bytes) apart.
-                src[j] = W + size_t(gn) * (CONV ? ep.cv_c : K) + col * 16;
+                src[j] = W + size_t(gn) * K + col * 16;
             }
         }
         auto issue_stage = [&](int kt, int buf) {
             int8_t *base = lds + buf * STAGE + wave * (IPW * 1024);
             const size_t koff_row = size_t(kt) * BK;
-            size_t koff_col = koff_row;
-            if constexpr (CONV) {
-                const int tap = kt / ep.cv_tiles_per_tap, sub = kt % ep.cv_tiles_per_tap;
-                koff_col = size_t((tap / ep.cv_kw) * ep.cv_wp + tap % ep.cv_kw) * ep.cv_c + size_t(sub) * BK;
-            }
 #pragma unroll
             for (int j = 0; j < IPW; ++j)
                 __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void *)(src[j] + (col_side[j] ? koff_col : koff_row)),
+                    (const __attribute__((address_space(1))) void *)(src[j] + koff_row),
                     (__attribute__((address_space(3))) void *)(base + j * 1024), 16, 0, 0);
         };
         // Two stages before the first barrier so the consumers start after one memory
@@ -603,46 +605,13 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
         const int nc = nn[j] < N ? nn[j] : N - 1;
         swv[j] = 1.0f;
         bv[j] = 0.0f;
-        if constexpr (EPI != EPI_I32 && !CONV) {
+        if constexpr (EPI != EPI_I32) {
             swv[j] = ep.sw[nc];
             if (ep.bias) bv[j] = ep.bias[nc];
         }
     }
     if constexpr (EPI != EPI_I32)
-        if (CONV || !ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
-    // Convolution: where each window's outputs go and the per-filter operands, also ahead of the
-    // main loop (the index arithmetic and the loads' latency hide behind it).  Rows are output
-    // channels, columns are padded-grid window positions; a lane owns one window.  Lane l of a
-    // row block fetches the operands of row l % 32 (three loads per block instead of three per
-    // accumulator register); the 16 rows a lane needs come back through shuffles in the epilogue.
-    size_t out_base[CONV ? FN : 1];
-    bool valid[CONV ? FN : 1];
-    float s_blk[CONV ? FM : 1], b_blk[CONV ? FM : 1];
-    int c_blk[CONV ? FM : 1];
-    if constexpr (CONV) {
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int q = nn[j];
-            const int per_img = ep.cv_hp * ep.cv_wp;
-            const int img = q / per_img, rem = q % per_img;
-            const int oh = rem / ep.cv_wp, ow = rem % ep.cv_wp;
-            valid[j] = q < N && oh < ep.cv_ho && ow < ep.cv_wo;
-            out_base[j] = (size_t(img) * ep.cv_oc * ep.cv_ho + oh) * ep.cv_wo + ow;  // + oc * ho * wo
-        }
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            const int m = m0 + wm * TM + i * 32 + lane % 32;
-            const int mc = m < M ? m : M - 1;
-            c_blk[i] = ep.cv_corr_mul * ep.cv_wsum[mc];
-            s_blk[i] = 1.0f;
-            b_blk[i] = 0.0f;
-            if constexpr (EPI != EPI_I32) {
-                s_blk[i] = sa0 * ep.sw[mc];
-                if (ep.bias) b_blk[i] = ep.bias[mc];
-            }
-        }
-    }
-
+        if (!ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
     // LDS byte offsets (within a stage) of this lane's fragment reads.
     int offA[FM][KSW], offW[FN][KSW];
 #pragma unroll
@@ -718,60 +687,15 @@ __global__ __launch_bounds__((PW + WM * WN * WK) * kWave) void gemm_i8_pipe_kern
     if (kt < nk) iteration(kt, 0);
 
     if constexpr (WK > 1) ksplit_reduce<FM, FN, WK>(acc, lds, wk, wmn, lane);
-    if constexpr (CONV) {
-        const float zpf = static_cast<float>(ep.zp_out);
-        const bool has_bias = ep.bias != nullptr;
-        // Rows are output channels, columns are padded-grid window positions.  A lane owns one
-        // window; consecutive lanes are consecutive ow, i.e. consecutive bytes of the NCHW output.
-        const size_t plane = size_t(ep.cv_ho) * ep.cv_wo;
-        wait_vmcnt<0>();
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            if (WK > 1 && i % WK != wk) continue;
-            float s_row[16], b_row[16];
-            int c_row[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int src = 8 * (r / 4) + 4 * (lane / 32) + (r % 4);  // row of the block = lane that holds it
-                c_row[r] = __shfl(c_blk[i], src, kWave);
-                s_row[r] = __shfl(s_blk[i], src, kWave);
-                b_row[r] = __shfl(b_blk[i], src, kWave);
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * TM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-                if (m >= M) continue;
-#pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    if (!valid[j]) continue;
-                    const size_t off = out_base[j] + size_t(m) * plane;
-                    const int a = acc[i][j][r] + c_row[r];
-                    if constexpr (EPI == EPI_I32) {
-                        static_cast<int32_t *>(ep.out)[off] = a;
-                    } else {
-                        float v = static_cast<float>(a) * s_row[r];
-                        if (has_bias) v = v + b_row[r];
-                        if constexpr (EPI == EPI_F32) {
-                            static_cast<float *>(ep.out)[off] = v;
-                        } else {
-                            const float qv = clamp_keep_nan(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128.0f, 127.0f);
-                            static_cast<int8_t *>(ep.out)[off] = static_cast<int8_t>(to_int_nan0(qv));
-                        }
-                    }
-                }
-            }
-        }
-    } else {
-        store_tile<FM, FN, WK, EPI, EVEN>(acc, ep, M, N, m0 + wm * TM, wk, lane, nn, swv, bv, sa0);
-    }
+    store_tile<FM, FN, WK, EPI, EVEN>(acc, ep, M, N, m0 + wm * TM, wk, lane, nn, swv, bv, sa0);
 }
 
-template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN, int CONV = 0>
+template <int BM, int BN, int STAGES, int PW, int WM, int WN, int WK, int EPI, bool EVEN>
 static int32_t launch_pipe(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, int N, int K,
                            const GemmEpilogue &ep) {
     constexpr int kLds = STAGES * (BM + BN) * 128;
     constexpr int kThreads = (PW + WM * WN * WK) * kWave;
-    auto kernel = gemm_i8_pipe_kernel<BM, BN, STAGES, PW, WM, WN, WK, EPI, EVEN, CONV>;
+    auto kernel = gemm_i8_pipe_kernel<BM, BN, STAGES, PW, WM, WN, WK, EPI, EVEN>;
     static bool configured[16] = {false};  // per device: raise the dynamic LDS limit once
     if (ctx->device < 16 && !configured[ctx->device]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),

@@ -91,6 +91,111 @@ __device__ __forceinline__ void store_block_interior(v16i (&own)[1][TNB], const 
     }
 }
 
+// Convolution epilogue of one 32-row block (rows = output channels from `row0`, a lane = one window per column
+// block): accumulator + (128 - zp_in) * sum of the filter's weights, then the Linear's dequantize / requantize
+// arithmetic, stored to NCHW (consecutive lanes are consecutive ow: consecutive bytes).  c_l / s_l / b_l: the
+// correction, combined scale and bias of row row0 + lane % 32, handed round by shuffles.
+//
+// With one wave per SIMD the epilogue is bound by instruction issue, so the common case - the whole row block
+// inside the output channels, the output below 2 GiB - has no branch and no 64-bit address per element: the
+// stores are buffer stores whose per-lane offset (the window's place in its image plus the lane half's four
+// rows; beyond the buffer for a window of the padded grid that is not an output, which makes the hardware drop
+// the store) is formed once, and whose row offset is scalar.
+template <int TNB, int EPI, bool EVEN>
+__device__ __forceinline__ void conv_store_block(v16i (&own)[1][TNB], const GemmEpilogue &ep, int M, int row0, int lane,
+                                                 const size_t (&out_base)[TNB], const bool (&valid)[TNB], int c_l,
+                                                 float s_l, float b_l) {
+    constexpr int ES = EPI == EPI_I8 ? 1 : 4;  // bytes per output element
+    const float zpf = static_cast<float>(ep.zp_out);
+    const bool has_bias = ep.bias != nullptr;
+    const size_t plane = size_t(ep.cv_ho) * ep.cv_wo;
+    wait_vmcnt<0>();
+    float s_row[16], b_row[16];
+    int c_row[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int src = 8 * (r / 4) + 4 * (lane / 32) + (r % 4);  // row of the block = lane that holds its operands
+        c_row[r] = __shfl(c_l, src, kWave);
+        s_row[r] = __shfl(s_l, src, kWave);
+        b_row[r] = __shfl(b_l, src, kWave);
+    }
+    // The element's bits (int8 in the low byte for EPI_I8).  FAST_DIV / BIAS are hoisted out of the element loop
+    // so that its body is straight-line code the compiler can interleave across the 32 outputs of a lane.
+    auto value = [&](int r, int j, auto fast_div, auto with_bias) -> int {
+        const int a = own[0][j][r] + c_row[r];
+        if constexpr (EPI == EPI_I32) {
+            return a;
+        } else {
+            float v = static_cast<float>(a) * s_row[r];
+            if constexpr (decltype(with_bias)::value) v = v + b_row[r];
+            if constexpr (EPI == EPI_F32) {
+                return __builtin_bit_cast(int, v);
+            } else {
+                float q;
+                if constexpr (decltype(fast_div)::value) {
+                    const float q0 = v * ep.s_out_inv;  // div_rn with a usable reciprocal
+                    const float rem = fmaf(-q0, ep.s_out, v);
+                    const float q1 = fmaf(rem, ep.s_out_inv, q0);
+                    q = (rem == rem) ? q1 : q0;
+                } else {
+                    q = v / ep.s_out;
+                }
+                return clamp_to_int(round_mode<EVEN>(q) + zpf, -128, 127);  // NaN -> 0, as `as i8` after the clamp
+            }
+        }
+    };
+    const size_t out_bytes = size_t(ep.cv_nb) * ep.cv_oc * plane * ES;
+    const bool whole = row0 + 32 <= M && out_bytes < (size_t(1) << 31);
+    const __amdgpu_buffer_rsrc_t ro =
+        __builtin_amdgcn_make_buffer_rsrc(ep.out, 0, whole ? static_cast<int>(out_bytes) : 0, 0x00020000);
+    int voff[TNB];
+#pragma unroll
+    for (int j = 0; j < TNB; ++j)
+        voff[j] = valid[j] ? static_cast<int>((out_base[j] + size_t(4 * (lane / 32)) * plane) * ES) : 0x7fffffff;
+    const int plane_bytes = static_cast<int>(plane) * ES;
+    auto emit = [&](auto fast_div, auto with_bias) {
+        if (whole) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int soff = (row0 + 8 * (r / 4) + (r % 4)) * plane_bytes;
+#pragma unroll
+                for (int j = 0; j < TNB; ++j) {
+                    const int bits = value(r, j, fast_div, with_bias);
+                    if constexpr (EPI == EPI_I8)
+                        __builtin_amdgcn_raw_buffer_store_b8(static_cast<char>(bits), ro, voff[j], soff, 0);
+                    else
+                        __builtin_amdgcn_raw_buffer_store_b32(bits, ro, voff[j], soff, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = row0 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+                if (m >= M) continue;
+#pragma unroll
+                for (int j = 0; j < TNB; ++j) {
+                    if (!valid[j]) continue;
+                    const size_t off = out_base[j] + size_t(m) * plane;
+                    const int bits = value(r, j, fast_div, with_bias);
+                    if constexpr (EPI == EPI_I8)
+                        static_cast<int8_t *>(ep.out)[off] = static_cast<int8_t>(bits);
+                    else
+                        static_cast<int32_t *>(ep.out)[off] = bits;
+                }
+            }
+        }
+    };
+    const bool fast = ep.s_out_inv != 0.0f;
+    if (fast && has_bias)
+        emit(std::true_type{}, std::true_type{});
+    else if (fast)
+        emit(std::true_type{}, std::false_type{});
+    else if (has_bias)
+        emit(std::false_type{}, std::true_type{});
+    else
+        emit(std::false_type{}, std::false_type{});
+}
+
 // TMB x TNB row blocks of 32 per workgroup tile; D register stages of (TMB + TNB) KiB per wave in
 // flight.  Loads are buffer loads with a constant per-lane offset and scalar (SGPR) fragment
 // offsets, so the loop spends no vector instruction on addressing.
@@ -104,7 +209,13 @@ __device__ __forceinline__ void store_block_interior(v16i (&own)[1][TNB], const 
 // M = 512, N = K = 4096 with operands from HBM; with 32 steps every (tile_m, XCD) pair starts on a
 // different step).  Activations that the previous kernel has just written are served by the memory-side
 // cache, where the same stagger costs 0.4 us instead: the fused forwards switch it off.
-template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false>
+//
+// CONV: implicit-GEMM convolution on the same loop.  The row operand PA holds the packed filters (M = output
+// channels, K = taps x channels, tap-major), the column operand PW is the image as signed bytes in
+// [channel block of 32][padded pixel][32 bytes] order (conv_pack_image_kernel), N = padded pixels = windows:
+// window q's fragment for (tap, channel block) is the 32 pixels from q + tap offset on, 1 KiB contiguous, so a
+// window fragment is one coalesced wave load like a packed one, with no im2col and no gather.
+template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false>
 __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__restrict__ PA,
                                                              const int8_t *__restrict__ PW, int M, int N, int K,
                                                              GemmEpilogue ep) {
@@ -136,13 +247,39 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
         const int nc = nn[j] < N ? nn[j] : N - 1;
         swv[j] = 1.0f;
         bv[j] = 0.0f;
-        if constexpr (EPI != EPI_I32) {
+        if constexpr (EPI != EPI_I32 && !CONV) {
             swv[j] = ep.sw[nc];
             if (ep.bias) bv[j] = ep.bias[nc];
         }
     }
     if constexpr (EPI != EPI_I32)
-        if (!ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
+        if (CONV || !ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
+    // Convolution: where each window's outputs go and the per-filter operands of this wave's row block, also
+    // ahead of the main loop.  Rows are output channels, columns are padded-grid windows; a lane owns one
+    // window per column block.  Lane l fetches the operands of row l % 32 of the block; the 16 rows a lane
+    // needs come back through shuffles in the epilogue.
+    size_t cv_out_base[CONV ? TNB : 1];
+    bool cv_valid[CONV ? TNB : 1];
+    float cv_s = 1.0f, cv_b = 0.0f;
+    int cv_c = 0;
+    if constexpr (CONV) {
+#pragma unroll
+        for (int j = 0; j < TNB; ++j) {
+            const int q = nn[j];
+            const int per_img = ep.cv_hp * ep.cv_wp;
+            const int img = q / per_img, rem = q % per_img;
+            const int oh = rem / ep.cv_wp, ow = rem % ep.cv_wp;
+            cv_valid[j] = q < N && oh < ep.cv_ho && ow < ep.cv_wo;
+            cv_out_base[j] = (size_t(img) * ep.cv_oc * ep.cv_ho + oh) * ep.cv_wo + ow;  // + oc * ho * wo
+        }
+        const int m = m0 + wave * 32 + lane % 32;
+        const int mc = m < M ? m : M - 1;
+        cv_c = ep.cv_corr_mul * ep.cv_wsum[mc];
+        if constexpr (EPI != EPI_I32) {
+            cv_s = sa0 * ep.sw[mc];
+            if (ep.bias) cv_b = ep.bias[mc];
+        }
+    }
 
     // Byte offsets of this wave's first fragment of every row block of the tile (row blocks past
     // the matrix repeat the last one: computed and discarded).  Operands are below 2 GiB.
@@ -163,12 +300,25 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     for (int j = 0; j < TNB; ++j) {
         int rb = tile_n * TNB + j;
         rb = rb < rbW ? rb : rbW - 1;
-        sow[j] = (rb * KB + wave) * 1024;
+        sow[j] = CONV ? rb * 1024 : (rb * KB + wave) * 1024;  // CONV: 32 pixels of 32 bytes per row block
     }
     const int steps = KB / WK;  // k blocks per wave
     int rot = (tile_m % 4) * (steps / 4) + (ep.fresh_activations ? 0 : int(blockIdx.x % 8) * ((steps / 8) | 1));
     while (rot >= steps) rot -= steps;  // at most a few rounds; cheaper than a division in front of the first load
     const int voff = lane * 16;
+    // CONV: lane l reads window l % 32 (pixels are 32 bytes apart), bytes 16 * (l / 32) of the channel block.
+    const int voffw = CONV ? (lane % 32) * 32 + (lane / 32) * 16 : voff;
+    // CONV: this wave's k block as (channel block, tap row, tap column), advanced by 4 k blocks per step with
+    // scalar adds (a division per step would cost more than the step's MFMAs).
+    const int cv_cb_count = CONV ? ep.cv_c / 32 : 1;
+    int cv_kb = 0, cv_cb = 0, cv_ty = 0, cv_tx = 0;
+    auto conv_seek = [&](int sr) {
+        int tap;
+        cv_kb = wave + WK * sr;
+        divmod_uniform(cv_kb, cv_cb_count, &tap, &cv_cb);
+        divmod_uniform(tap, ep.cv_kw, &cv_ty, &cv_tx);
+    };
+    if constexpr (CONV) conv_seek(rot);
 
     v4i fa[D][TMB], fb[D][TNB];
     auto issue = [&](int s, int slot) {
@@ -178,9 +328,24 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
 #pragma unroll
         for (int i = 0; i < TMB; ++i)
             fa[slot][i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, voff, soa[i] + koff, 0));
+        int koffw = koff;
+        if constexpr (CONV) {
+            if (sr == 0 && s != 0) conv_seek(0);  // wrapped round
+            // k blocks past taps x channel blocks are zero in the filters: any valid address will do
+            koffw = cv_kb < ep.cv_kblocks ? (cv_cb * ep.cv_pixels + cv_ty * ep.cv_wp + cv_tx) * 32 : 0;
+            cv_kb += WK;
+            cv_cb += WK;
+            while (cv_cb >= cv_cb_count) {
+                cv_cb -= cv_cb_count;
+                if (++cv_tx == ep.cv_kw) {
+                    cv_tx = 0;
+                    ++cv_ty;
+                }
+            }
+        }
 #pragma unroll
         for (int j = 0; j < TNB; ++j)
-            fb[slot][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, sow[j] + koff, 0));
+            fb[slot][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voffw, sow[j] + koffw, 0));
     };
 
     v16i acc[TMB][TNB];
@@ -259,12 +424,16 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
         }
     mark(3);
     const int row0 = m0 + wave * 32;
-    bool interior = false;
-    if constexpr (EPI != EPI_I8) interior = m0 + TMB * 32 <= M && n0 + TNB * 32 <= N && ep.residual == nullptr;
-    if (interior) {
-        if constexpr (EPI != EPI_I8) store_block_interior<TNB, EPI>(own, ep, N, row0, n0, lane, swv, bv, sa0);
+    if constexpr (CONV) {
+        conv_store_block<TNB, EPI, EVEN>(own, ep, M, row0, lane, cv_out_base, cv_valid, cv_c, cv_s, cv_b);
     } else {
-        store_tile<1, TNB, 1, EPI, EVEN>(own, ep, M, N, row0, 0, lane, nn, swv, bv, sa0);
+        bool interior = false;
+        if constexpr (EPI != EPI_I8) interior = m0 + TMB * 32 <= M && n0 + TNB * 32 <= N && ep.residual == nullptr;
+        if (interior) {
+            if constexpr (EPI != EPI_I8) store_block_interior<TNB, EPI>(own, ep, N, row0, n0, lane, swv, bv, sa0);
+        } else {
+            store_tile<1, TNB, 1, EPI, EVEN>(own, ep, M, N, row0, 0, lane, nn, swv, bv, sa0);
+        }
     }
     if constexpr (TRACE) {
         mark(4);
@@ -306,11 +475,11 @@ __global__ __launch_bounds__(256) void pack_rows_i8_kernel(const int8_t *__restr
     }
 }
 
-template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false>
+template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false>
 static int32_t launch_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                              const GemmEpilogue &ep) {
     constexpr int kLds = TMB * TNB * 3 * 4096;
-    auto kernel = gemm_i8_packed_kernel<TMB, TNB, D, EPI, EVEN, TRACE>;
+    auto kernel = gemm_i8_packed_kernel<TMB, TNB, D, EPI, EVEN, TRACE, CONV>;
     static bool configured[16] = {false};  // per device: raise the dynamic LDS limit once
     if (ctx->device < 16 && !configured[ctx->device]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),

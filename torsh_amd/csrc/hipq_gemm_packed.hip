@@ -17,7 +17,7 @@ static int32_t check_packed_shape(const char *fn, size_t m, size_t n, size_t k) 
     return HIPQ_SUCCESS;
 }
 
-static int32_t pack_rows(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_t *dst) {
+int32_t pack_rows(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_t *dst) {
     const size_t nfrag = packed_row_blocks(rows) * packed_k_blocks(k);
     size_t blocks = (nfrag + 3) / 4;
     const size_t cap = size_t(ctx->num_cus) * 16;
@@ -41,6 +41,35 @@ static PackedScratch packed_scratch_layout(int num_cus, size_t m, size_t k, bool
     L.rowmajor = L.packed + up(packed_bytes(m, k));
     L.total = L.rowmajor + (per_token ? up(m * k) : 0) + 256;
     return L;
+}
+
+size_t packed_operand_bytes(size_t rows, size_t k) { return packed_bytes(rows, k); }
+
+// Implicit-GEMM convolution on the packed kernel: picks the register depth (the largest of 4, 3, 2, 1 that
+// divides the k blocks per wave) and the epilogue.
+template <int EPI, bool EVEN>
+static int32_t launch_conv_packed(hipq_ctx *ctx, const int8_t *filters, const int8_t *image, int M, int N, int K,
+                                  const GemmEpilogue &ep) {
+    const int steps = static_cast<int>(packed_k_blocks(size_t(K))) / 4;
+    if constexpr (EPI == EPI_I8 && !EVEN) {
+        // Phase stamps (hipq_ctx_set_trace_buffer): the depth-3 requantizing form only.
+        const size_t tiles = ((packed_row_blocks(size_t(M)) + 3) / 4) * ((packed_row_blocks(size_t(N)) + 1) / 2);
+        if (ctx->trace && steps % 4 != 0 && steps % 3 == 0 &&
+            ctx->trace_bytes >= tiles * 4 * kTraceWords * sizeof(unsigned long long))
+            return launch_packed<4, 2, 3, EPI, EVEN, true, true>(ctx, filters, image, M, N, K, ep);
+    }
+    if (steps % 4 == 0) return launch_packed<4, 2, 4, EPI, EVEN, false, true>(ctx, filters, image, M, N, K, ep);
+    if (steps % 3 == 0) return launch_packed<4, 2, 3, EPI, EVEN, false, true>(ctx, filters, image, M, N, K, ep);
+    if (steps % 2 == 0) return launch_packed<4, 2, 2, EPI, EVEN, false, true>(ctx, filters, image, M, N, K, ep);
+    return launch_packed<4, 2, 1, EPI, EVEN, false, true>(ctx, filters, image, M, N, K, ep);
+}
+
+int32_t conv_gemm_packed(hipq_ctx *ctx, const int8_t *filters, const int8_t *image, int M, int N, int K,
+                         const GemmEpilogue &ep, int epi, bool even) {
+    if (epi == EPI_I32) return launch_conv_packed<EPI_I32, false>(ctx, filters, image, M, N, K, ep);
+    if (epi == EPI_F32) return launch_conv_packed<EPI_F32, false>(ctx, filters, image, M, N, K, ep);
+    if (even) return launch_conv_packed<EPI_I8, true>(ctx, filters, image, M, N, K, ep);
+    return launch_conv_packed<EPI_I8, false>(ctx, filters, image, M, N, K, ep);
 }
 
 }  // namespace hipq

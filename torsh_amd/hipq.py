@@ -153,6 +153,7 @@ _SPECIAL = {
     "hipq_ctx_stream": (_vp, [_vp]),
     "hipq_transformer_stack_workspace_bytes": (_sz, [_sz, _sz, _sz]),
     "hipq_packed_size": (_i32, [_sz, _sz, C.POINTER(C.c_size_t)]),
+    "hipq_conv2d_packed_weights_size": (_i32, [_sz, _sz, _sz, _sz, C.POINTER(C.c_size_t)]),
 }
 
 
@@ -639,8 +640,11 @@ class Context:
         return out
 
     def conv2d_pack_weights(self, w_i8):
+        """int8 [OC, IC, KH, KW] filters -> (packed row operand of the matrix-core GEMM, per-filter sums)."""
         oc, ic, kh, kw = w_i8.shape
-        packed = torch.empty((oc, kh * kw, ic), dtype=torch.int8, device=self._dev())
+        n = C.c_size_t(0)
+        _check(self._lib.hipq_conv2d_packed_weights_size(oc, ic, kh, kw, C.byref(n)))
+        packed = torch.empty(int(n.value), dtype=torch.int8, device=self._dev())
         sums = torch.empty(oc, dtype=torch.int32, device=self._dev())
         self.call("hipq_conv2d_pack_weights_i8", _ptr(w_i8), oc, ic, kh, kw, _ptr(packed), _ptr(sums))
         return packed, sums
@@ -648,7 +652,7 @@ class Context:
     def conv2d_i8_packed(self, x_u8, zp_in, s_in, w_packed, w_sums, kernel, w_scales, bias, s_out, zp_out,
                          padding=(0, 0), mode=0, out=None):
         nb, c, h, wd = x_u8.shape
-        oc = w_packed.shape[0]
+        oc = w_sums.numel()
         kh, kw = kernel
         ho = h + 2 * padding[0] - kh + 1
         wo = wd + 2 * padding[1] - kw + 1
