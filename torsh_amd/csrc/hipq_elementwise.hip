@@ -265,25 +265,30 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
 // floats of its (row, half k block) as four 16-byte loads and writes its 16 codes as one 16-byte
 // store, so a wave reads 32 whole 128-byte lines and writes 1 KiB contiguous.  Rows and columns
 // past the matrix become code 0 (zero padding along K adds nothing to a dot product).
-template <bool DIV, int RND>
-__global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__restrict__ x, size_t rows,
-                                                                  size_t cols, float scale, int zp,
-                                                                  const hipq_qparams *__restrict__ params,
-                                                                  DynamicRange dyn, int8_t *__restrict__ out) {
-    const size_t KB = ((cols + 31) / 32 + 3) / 4 * 4;
-    const size_t nfrag = ((rows + 31) / 32) * KB;
-    const int lane = threadIdx.x % kWave;
-    const bool vec = (cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
-    const size_t fstep = size_t(gridDim.x) * (kBlock / kWave);
-    size_t f = size_t(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave;
-    // The first fragment's floats are requested before the parameters are resolved (a fold of the range
-    // partials and two workgroup barriers in a dynamic call): the loads do not depend on the scale, and a
-    // launch of this size is bound by latency, not by bandwidth.
-    // frag -> (row block, k block) without a 64-bit division where it can be avoided: it would sit, with
-    // its ~100 instructions, in front of the kernel's first load.
-    const bool kb_pow2 = (KB & (KB - 1)) == 0, frag32 = nfrag + fstep < (size_t(1) << 32);
-    const int kb_shift = __builtin_ffsll(static_cast<long long>(KB)) - 1;
-    auto whole = [&](size_t frag, size_t *row, size_t *k0) {
+// How the packed quantizer's waves walk the matrix: wave w of the grid takes fragments w, w + waves, ...;
+// lane l of a fragment owns row 32 * rb + l % 32, floats 32 * kb + 16 * (l / 32) .. +15.  Shared with the range
+// pass that runs just before it in a dynamic call, so that each workgroup reads the very same lines in both
+// kernels: workgroup ids map to XCDs the same way in both launches, and the second read is served by that
+// XCD's L2 instead of the memory-side cache.
+struct FragmentWalk {
+    size_t rows, cols, KB, nfrag, fstep;
+    int lane, kb_shift;
+    bool vec, kb_pow2, frag32;
+    __device__ FragmentWalk(const float *x, size_t rows_, size_t cols_) : rows(rows_), cols(cols_) {
+        KB = ((cols + 31) / 32 + 3) / 4 * 4;
+        nfrag = ((rows + 31) / 32) * KB;
+        lane = threadIdx.x % kWave;
+        vec = (cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
+        fstep = size_t(gridDim.x) * (kBlock / kWave);
+        // frag -> (row block, k block) without a 64-bit division where it can be avoided: it would sit, with
+        // its ~100 instructions, in front of the kernel's first load.
+        kb_pow2 = (KB & (KB - 1)) == 0;
+        frag32 = nfrag + fstep < (size_t(1) << 32);
+        kb_shift = __builtin_ffsll(static_cast<long long>(KB)) - 1;
+    }
+    __device__ size_t first() const { return size_t(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave; }
+    // The lane's (row, first float) in fragment `frag`; true when its 16 floats can be read as four float4.
+    __device__ bool whole(size_t frag, size_t *row, size_t *k0) const {
         size_t rb, kb;
         if (kb_pow2) {
             rb = frag >> kb_shift;
@@ -298,7 +303,50 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__
         *row = rb * 32 + lane % 32;
         *k0 = kb * 32 + 16 * (lane / 32);
         return vec && frag < nfrag && *row < rows && *k0 + 16 <= cols;
-    };
+    }
+};
+
+// Range pass over a matrix in the packed quantizer's order (see FragmentWalk): one (min, max) partial per
+// workgroup, the same numbers as minmax_partial_kernel's fold whatever the order (min and max are exact).
+__global__ __launch_bounds__(kBlock) void minmax_fragments_kernel(const float *__restrict__ x, size_t rows, size_t cols,
+                                                                   float2 *__restrict__ partials) {
+    __shared__ float lds[2 * kBlock / kWave];
+    const FragmentWalk fw(x, rows, cols);
+    MinMax m{INFINITY, -INFINITY};
+    for (size_t f = fw.first(); f < fw.nfrag; f += fw.fstep) {
+        size_t row, k0;
+        if (fw.whole(f, &row, &k0)) {
+            float4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(x + row * cols + k0)[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                m.mn = fminf(m.mn, fminf(fminf(v[i].x, v[i].y), fminf(v[i].z, v[i].w)));
+                m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
+            }
+        } else if (row < rows && k0 < cols) {
+            const float *p = x + row * cols + k0;
+            for (int b = 0; b < 16; ++b)
+                if (k0 + b < cols) acc_minmax(m, p[b]);
+        }
+    }
+    const MinMax r = block_minmax(m, lds);
+    if (threadIdx.x == 0) partials[blockIdx.x] = make_float2(r.mn, r.mx);
+}
+
+template <bool DIV, int RND>
+__global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__restrict__ x, size_t rows,
+                                                                  size_t cols, float scale, int zp,
+                                                                  const hipq_qparams *__restrict__ params,
+                                                                  DynamicRange dyn, int8_t *__restrict__ out) {
+    const FragmentWalk fw(x, rows, cols);
+    const size_t nfrag = fw.nfrag, fstep = fw.fstep;
+    const int lane = fw.lane;
+    size_t f = fw.first();
+    // The first fragment's floats are requested before the parameters are resolved (a fold of the range
+    // partials and two workgroup barriers in a dynamic call): the loads do not depend on the scale, and a
+    // launch of this size is bound by latency, not by bandwidth.
+    auto whole = [&](size_t frag, size_t *row, size_t *k0) { return fw.whole(frag, row, k0); };
     float4 v[4];
     size_t row, k0;
     bool have = whole(f, &row, &k0);
@@ -961,7 +1009,26 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
     DynamicRange dyn{nullptr, 0, HIPQ_PARAMS_SYMMETRIC, -128, 127, out_params};
     dyn.poison = 1;
     float scale = 1.0f;
-    if (dynamic) {
+    const size_t KB = ((cols + 31) / 32 + 3) / 4 * 4, nfrag = ((rows + 31) / 32) * KB;
+    size_t blocks = (nfrag + 3) / 4;
+    const size_t cap = size_t(ctx->num_cus) * 8;
+    int grid = static_cast<int>(blocks < cap ? blocks : cap);
+    if (dynamic && packed) {
+        // Range pass in the quantizer's own order and with its grid (FragmentWalk): one partial per workgroup.
+        float2 *p = static_cast<float2 *>(partials);
+        if (p) {
+            const size_t room = partials_bytes / sizeof(float2);
+            if (size_t(grid) > room) grid = static_cast<int>(room);
+        } else {
+            void *s = nullptr;
+            if ((rc = scratch(ctx, kScratchHeader + size_t(grid) * sizeof(float2), &s))) return rc;
+            p = reinterpret_cast<float2 *>(static_cast<char *>(s) + kScratchHeader);
+        }
+        hipLaunchKernelGGL(minmax_fragments_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, x, rows, cols, p);
+        if ((rc = check_launch("minmax (fragments)"))) return rc;
+        dyn.partials = p;
+        dyn.nparts = grid;
+    } else if (dynamic) {
         rc = launch_minmax_partials(ctx, x, rows * cols, &dyn, static_cast<float2 *>(partials),
                                     partials_bytes / sizeof(float2));
         if (rc) return rc;
@@ -970,10 +1037,6 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
         scale = static_scale;
     }
     if (!packed) return launch_quantize<int8_t>(ctx, x, rows * cols, scale, 0, nullptr, mode, -128.0f, 127.0f, out, dyn);
-    const size_t KB = ((cols + 31) / 32 + 3) / 4 * 4, nfrag = ((rows + 31) / 32) * KB;
-    size_t blocks = (nfrag + 3) / 4;
-    const size_t cap = size_t(ctx->num_cus) * 8;
-    const int grid = static_cast<int>(blocks < cap ? blocks : cap);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
 #define HIPQ_LAUNCH_QP(D, E)                                                                                       \
     hipLaunchKernelGGL((quantize_packed_kernel<D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, rows, cols, scale, \
