@@ -268,8 +268,8 @@ __global__ __launch_bounds__(kBlock) void quantize_kernel(const float *__restric
 // How the packed quantizer's waves walk the matrix: wave w of the grid takes fragments w, w + waves, ...;
 // lane l of a fragment owns row 32 * rb + l % 32, floats 32 * kb + 16 * (l / 32) .. +15.  Shared with the range
 // pass that runs just before it in a dynamic call, so that each workgroup reads the very same lines in both
-// kernels: workgroup ids map to XCDs the same way in both launches, and the second read is served by that
-// XCD's L2 instead of the memory-side cache.
+// kernels, in the same order: the second read then finds them in the memory-side cache the way they went in
+// (measured: the quantizer takes 5.2 us instead of 5.9 us after a range pass in flat order).
 struct FragmentWalk {
     size_t rows, cols, KB, nfrag, fstep;
     int lane, kb_shift;

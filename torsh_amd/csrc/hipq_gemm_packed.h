@@ -589,7 +589,10 @@ static int32_t launch_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, 
     return check_launch("gemm_i8 (packed)");
 }
 
-// Picks the register depth: the largest of 4, 2, 1 that divides the k blocks per wave.
+// Register depth 2 where it divides the k blocks per wave (else 1): two stages of 6 KiB per wave in flight.  Depth
+// 4 is as fast when the kernel is launched back to back at sustained clocks (14.8 us at M = 512, N = K = 4096) but
+// slower from idle clocks (17.6 against 15.7 us) and inside the Linear step, where the kernel follows the small
+// quantize kernels (24.2 against 23.5 us per step); depth 1 is 2-3 us slower everywhere.
 template <int EPI, bool EVEN>
 static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, size_t m, size_t n, size_t k,
                                   const GemmEpilogue &ep) {
@@ -597,13 +600,12 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
     const int steps = static_cast<int>(packed_k_blocks(k)) / 4;
     if (M <= 32) return launch_gemv_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // one row block of activations
     if constexpr (EPI == EPI_F32 && !EVEN) {
-        // Phase stamps (hipq_ctx_set_trace_buffer): the depth-4 fp32 form only, and only when the buffer holds
+        // Phase stamps (hipq_ctx_set_trace_buffer): the depth-2 fp32 form only, and only when the buffer holds
         // every wave's record.
         const size_t tiles = ((packed_row_blocks(m) + 3) / 4) * ((packed_row_blocks(n) + 1) / 2);
-        if (ctx->trace && steps % 4 == 0 && ctx->trace_bytes >= tiles * 4 * kTraceWords * sizeof(unsigned long long))
-            return launch_packed<4, 2, 4, EPI, EVEN, true>(ctx, pa, pw, M, N, K, ep);
+        if (ctx->trace && steps % 2 == 0 && ctx->trace_bytes >= tiles * 4 * kTraceWords * sizeof(unsigned long long))
+            return launch_packed<4, 2, 2, EPI, EVEN, true>(ctx, pa, pw, M, N, K, ep);
     }
-    if (steps % 4 == 0) return launch_packed<4, 2, 4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     if (steps % 2 == 0) return launch_packed<4, 2, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     return launch_packed<4, 2, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
 }
