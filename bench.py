@@ -517,6 +517,27 @@ def main() -> int:
         extra["linear_step_static_activation_scale"] = {"ms_per_step": ms3, "TOP/s": ops / (ms3 * 1e-3) / 1e12,
                                                         "note": "activation scale from calibration instead of a "
                                                                 "min/max pass per call (two launches, not three)"}
+        # Per-token (per-row) dynamic activation scales instead of one per tensor: one pass over the activations
+        # (each row's range and codes in one kernel, written straight into the packed layout), then the GEMM.
+        pt = [0]
+
+        def step_per_token():
+            i = pt[0] % pool
+            pt[0] += 1
+            ctx.linear_dynamic_packed(xs[i], pw[i], sw[i], bias, per_token=True, mode=hipq.FORM_MUL_INV, out=outs[i])
+
+        spin_up(step_per_token, SPINUP_MS)
+        for _ in range(args.warmup):
+            step_per_token()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_per_token()
+        torch.cuda.synchronize()
+        ms5 = (time.perf_counter() - t0) * 1e3 / args.steps
+        extra["linear_step_per_token_activation_scales"] = {
+            "ms_per_step": ms5, "TOP/s": ops / (ms5 * 1e-3) / 1e12,
+            "note": "dynamic per-row activation quantization (two launches); not the per-tensor scheme `value` is quoted on"}
         # The same step on row-major int8 weights (no weight preparation): LDS-staged kernel.
         pr = [0]
 

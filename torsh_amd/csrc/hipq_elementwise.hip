@@ -446,7 +446,13 @@ __global__ __launch_bounds__(kBlock) void dequantize_kernel(const InT *__restric
 // read it once (rows up to TPR*16 floats stay in registers), reduce min/max
 // across the row with wave shuffles, derive the row's parameters and quantize
 // with the division form.
-template <int TPR, bool EVEN>
+//
+// PACKED: the codes go straight into the fragment-packed operand layout of the packed GEMM
+// ([row block of 32][k block of 32 bytes][1 KiB]; lane l of a fragment = row l % 32, bytes 16 * (l / 32) .. +15)
+// instead of a dense [rows, cols] matrix, so that a per-token Linear forward needs no packing pass.  The grid
+// then covers the rows up to a multiple of 32, and the padding - rows past the matrix, k past cols up to a
+// multiple of 128 - is written as zeros.
+template <int TPR, bool EVEN, bool PACKED = false>
 __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *__restrict__ x, size_t rows,
                                                                    size_t cols, size_t ld, int flavor, int qmin,
                                                                    int qmax,
@@ -462,6 +468,10 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     const bool active = row < rows;
     const float *xr = x + (active ? row : 0) * ld;  // input rows are ld elements apart, output is dense
     int8_t *qr = out + (active ? row : 0) * cols;
+    // PACKED: where the byte of (row, k) lives, and the padded extent of K.
+    const size_t kpad = ((cols + 31) / 32 + 3) / 4 * 4 * 32;
+    int8_t *prow = out + (row / 32) * (kpad / 32) * 1024 + (row % 32) * 16;  // + packed_k(k)
+    auto packed_k = [](size_t k) { return (k / 32) * 1024 + ((k % 32) / 16) * 512 + (k % 16); };
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (cols % 4 == 0) && (ld % 4 == 0) &&
                          ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
     const size_t nvec = aligned ? cols / 4 : 0;
@@ -501,7 +511,14 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
         static_assert(TPR == kBlock, "a row is owned by one wave or by the whole block");
         m = block_minmax(m, lds);
     }
-    if (!active) return;
+    if (!active) {
+        if constexpr (PACKED) {  // a padding row of the last row block
+            if (row < (rows + 31) / 32 * 32)
+                for (size_t k = size_t(lane) * 4; k < kpad; k += size_t(TPR) * 4)
+                    *reinterpret_cast<uint32_t *>(prow + packed_k(k)) = 0u;
+        }
+        return;
+    }
 
     float scale;
     int zp;
@@ -529,14 +546,27 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
                         : quantize_int<QFORM_DIV, EVEN>(v, scale, inv, zpf, qmin, qmax);
     };
     auto quant4 = [&](float4 t) { return pack4(quant1(t.x), quant1(t.y), quant1(t.z), quant1(t.w)); };
+    auto put4 = [&](size_t v, uint32_t w) {
+        if constexpr (PACKED)
+            *reinterpret_cast<uint32_t *>(prow + packed_k(v * 4)) = w;
+        else
+            q4[v] = w;
+    };
+    auto put1 = [&](size_t c, int8_t b) {
+        if constexpr (PACKED)
+            prow[packed_k(c)] = b;
+        else
+            qr[c] = b;
+    };
 #pragma unroll
     for (int i = 0; i < kCache; ++i) {
         const size_t v = size_t(lane) + size_t(i) * TPR;
-        if (v < nvec) q4[v] = quant4(cache[i]);
+        if (v < nvec) put4(v, quant4(cache[i]));
     }
-    for (size_t v = size_t(lane) + size_t(kCache) * TPR; v < nvec; v += TPR) q4[v] = quant4(x4[v]);
-    for (size_t c = nvec * 4 + lane; c < cols; c += TPR)
-        qr[c] = static_cast<int8_t>(quant1(xr[c]));
+    for (size_t v = size_t(lane) + size_t(kCache) * TPR; v < nvec; v += TPR) put4(v, quant4(x4[v]));
+    for (size_t c = nvec * 4 + lane; c < cols; c += TPR) put1(c, static_cast<int8_t>(quant1(xr[c])));
+    if constexpr (PACKED)
+        for (size_t c = cols + lane; c < kpad; c += TPR) put1(c, int8_t(0));  // k padding: zeros add nothing
 }
 
 // quantize_per_channel_auto for a channel axis that is not the leading one, and its group-wise
@@ -935,7 +965,8 @@ int32_t hipq_dequantize_with_params_i8_f32(hipq_ctx *ctx, const int8_t *q, size_
 // HIPQ_PARAMS_* formula (the reference's per-channel function knows two).
 static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
                              int32_t flavor, bool any_flavor, int32_t qmin, int32_t qmax, int32_t mode, int8_t *out,
-                             float *out_scales, int32_t *out_zero_points, int32_t *out_status, int poison = 0) {
+                             float *out_scales, int32_t *out_zero_points, int32_t *out_status, int poison = 0,
+                             bool packed = false) {
     int32_t rc = any_flavor ? HIPQ_SUCCESS : check_row_flavor(fn, flavor);
     if (rc) return rc;
     if ((rc = check_mode(fn, mode))) return rc;
@@ -947,23 +978,37 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
     HIPQ_REQUIRE_PTR(out);
     const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
     if (rows >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many rows", fn);
+    // Packed output: the grid also covers the padding rows of the last row block (they are written as zeros).
+    const size_t grid_rows = packed ? (rows + 31) / 32 * 32 : rows;
+#define HIPQ_LAUNCH_ROWS(TPR, E, P, G)                                                                               \
+    hipLaunchKernelGGL((quantize_per_row_kernel<TPR, E, P>), dim3(G), dim3(kBlock), 0, ctx->stream, x, rows, cols, ld, \
+                       flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison)
     if (cols > 1024) {
-        const int grid = static_cast<int>(rows);
-        if (even)
-            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
-        else
-            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
+        const int grid = static_cast<int>(grid_rows);
+        if (packed) {
+            if (even)
+                HIPQ_LAUNCH_ROWS(kBlock, true, true, grid);
+            else
+                HIPQ_LAUNCH_ROWS(kBlock, false, true, grid);
+        } else if (even) {
+            HIPQ_LAUNCH_ROWS(kBlock, true, false, grid);
+        } else {
+            HIPQ_LAUNCH_ROWS(kBlock, false, false, grid);
+        }
     } else {
-        const int grid = static_cast<int>((rows + 3) / 4);
-        if (even)
-            hipLaunchKernelGGL((quantize_per_row_kernel<kWave, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
-        else
-            hipLaunchKernelGGL((quantize_per_row_kernel<kWave, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                               rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison);
+        const int grid = static_cast<int>((grid_rows + 3) / 4);
+        if (packed) {
+            if (even)
+                HIPQ_LAUNCH_ROWS(kWave, true, true, grid);
+            else
+                HIPQ_LAUNCH_ROWS(kWave, false, true, grid);
+        } else if (even) {
+            HIPQ_LAUNCH_ROWS(kWave, true, false, grid);
+        } else {
+            HIPQ_LAUNCH_ROWS(kWave, false, false, grid);
+        }
     }
+#undef HIPQ_LAUNCH_ROWS
     return check_launch(fn);
 }
 
@@ -1054,9 +1099,9 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
 }
 
 int32_t hipq::quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
-                                           int8_t *out, float *out_scales) {
+                                           int8_t *out, float *out_scales, bool packed) {
     return quantize_rows("hipq_linear (activation quantize)", ctx, x, rows, cols, cols, HIPQ_PARAMS_SYMMETRIC, false,
-                         -128, 127, mode, out, out_scales, nullptr, nullptr, /*poison=*/1);
+                         -128, 127, mode, out, out_scales, nullptr, nullptr, /*poison=*/1, packed);
 }
 
 extern "C" {

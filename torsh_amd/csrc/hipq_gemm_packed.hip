@@ -27,19 +27,17 @@ int32_t pack_rows(hipq_ctx *ctx, const int8_t *src, size_t rows, size_t k, int8_
     return check_launch("pack_rows_i8");
 }
 
-// Scratch of the fused forward: header (hipq_qparams), range partials, per-row scales, the packed
-// activations, and (per token only) the row-major codes the pack pass reads.
+// Scratch of the fused forward: header (hipq_qparams), range partials, per-row scales, the packed activations.
 struct PackedScratch {
-    size_t partials, scales, packed, rowmajor, total;
+    size_t partials, scales, packed, total;
 };
-static PackedScratch packed_scratch_layout(int num_cus, size_t m, size_t k, bool per_token) {
+static PackedScratch packed_scratch_layout(int num_cus, size_t m, size_t k) {
     PackedScratch L;
     auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
     L.partials = kScratchHeader;
     L.scales = L.partials + up(size_t(num_cus) * 16 * sizeof(float2));
     L.packed = L.scales + up(m * sizeof(float));
-    L.rowmajor = L.packed + up(packed_bytes(m, k));
-    L.total = L.rowmajor + (per_token ? up(m * k) : 0) + 256;
+    L.total = L.packed + up(packed_bytes(m, k)) + 256;
     return L;
 }
 
@@ -184,7 +182,7 @@ int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t pe
     HIPQ_REQUIRE_PTR(w_packed);
     HIPQ_REQUIRE_PTR(w_scales);
     HIPQ_REQUIRE_PTR(out);
-    const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k, per_token != 0);
+    const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k);
     void *s = nullptr;
     rc = scratch(ctx, L.total, &s);
     if (rc) return rc;
@@ -193,10 +191,9 @@ int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t pe
     float *row_scales = reinterpret_cast<float *>(base + L.scales);
     int8_t *pa = reinterpret_cast<int8_t *>(base + L.packed);
     if (per_token) {
-        int8_t *qa = reinterpret_cast<int8_t *>(base + L.rowmajor);
-        rc = quantize_activations_per_row(ctx, x, m, k, mode & HIPQ_ROUND_HALF_EVEN, qa, row_scales);
+        // one pass over the activations: the per-row quantizer writes the packed operand itself
+        rc = quantize_activations_per_row(ctx, x, m, k, mode & HIPQ_ROUND_HALF_EVEN, pa, row_scales, /*packed=*/true);
         if (rc) return rc;
-        if ((rc = pack_rows(ctx, qa, m, k, pa))) return rc;
         return linear_packed_launch(ctx, pa, row_scales, 1, w_packed, w_scales, bias, m, n, k, out, true);
     }
     rc = quantize_activations_per_tensor(ctx, x, m, k, true, 1.0f, mode, true, pa, params, base + L.partials,
@@ -217,7 +214,7 @@ int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_sca
     HIPQ_REQUIRE_PTR(w_packed);
     HIPQ_REQUIRE_PTR(w_scales);
     HIPQ_REQUIRE_PTR(out);
-    const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k, false);
+    const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k);
     void *s = nullptr;
     rc = scratch(ctx, L.total, &s);
     if (rc) return rc;

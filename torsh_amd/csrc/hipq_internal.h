@@ -56,7 +56,7 @@ int32_t quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, size_t ro
                                         float static_scale, int32_t mode, bool packed, int8_t *out,
                                         hipq_qparams *out_params, void *partials, size_t partials_bytes);
 int32_t quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
-                                     int8_t *out, float *out_scales);
+                                     int8_t *out, float *out_scales, bool packed = false);
 // Looks up, once per device, the address of the static device array behind
 // hipq_linear_dynamic_f32_noalloc; called by hipq_ctx_create with the device current.
 int32_t linear_noalloc_setup(int device);
