@@ -391,8 +391,15 @@ HIPQ_API int32_t hipq_linear_packed_i8_i8(hipq_ctx *ctx, const int8_t *a_packed,
 HIPQ_API int32_t hipq_quantize_per_tensor_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
                                                         int32_t dynamic, float scale, int32_t mode,
                                                         int8_t *out_packed, hipq_qparams *out_params);
-/* hipq_linear_dynamic_f32 with prepared (packed) weights: range pass, quantize into the packed
- * layout, packed GEMM with the dequantizing epilogue. */
+/* Symmetric per-row (per-token) int8 quantize of fp32 [rows, cols] into the packed layout: each row's range, scale
+ * and codes in one pass (quantize_per_channel_auto over axis 0, algorithms.rs:126-242; the codes and scales of
+ * hipq_quantize_per_row_f32_i8 with HIPQ_PARAMS_SYMMETRIC).  out_scales: rows floats.  A row whose range is
+ * not finite gets a NaN scale and zero codes. */
+HIPQ_API int32_t hipq_quantize_per_row_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
+                                                     int32_t mode, int8_t *out_packed, float *out_scales);
+/* hipq_linear_dynamic_f32 with prepared (packed) weights: per tensor a range pass, the quantizer writing the packed
+ * layout and the packed GEMM with the dequantizing epilogue; per token the per-row quantizer (one pass) and the
+ * GEMM. */
 HIPQ_API int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t per_token,
                                                 const int8_t *w_packed, const float *w_scales, const float *bias,
                                                 size_t m, size_t n, size_t k, int32_t mode, float *out);

@@ -144,6 +144,23 @@ def test_quantize_per_tensor_packed_matches_row_major(ctx, hipq, rows, cols):
         assert ctx.read_qparams(sp).scale == np.float32(0.037)
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 8), (3, 70), (64, 256), (100, 304), (33, 1001), (40, 1500), (512, 4096)])
+def test_quantize_per_row_packed_matches_row_major(ctx, hipq, rows, cols):
+    """Codes and scales of the packed per-row quantizer = those of the row-major one (bit-exact with the oracle,
+    tests/test_gpu_elementwise.py), then packed; the padding of the packed buffer is written as zeros even when
+    the buffer held something else before."""
+    g = torch.Generator(device="cuda").manual_seed(rows * 131 + cols)
+    x = torch.randn(rows, cols, generator=g, device="cuda")
+    x[rows // 2] *= 40.0
+    for mode in (0, hipq.ROUND_HALF_EVEN):
+        q, s, _, _ = ctx.quantize_per_row(x, mode=mode)
+        dirty = torch.full((ctx.packed_size(rows, cols),), 77, dtype=torch.int8, device="cuda")
+        pq, ps = ctx.quantize_per_row_packed(x, mode=mode, out=dirty)
+        torch.cuda.synchronize()
+        assert torch.equal(pq, ctx.pack_rows(q))
+        assert torch.equal(ps, s)
+
+
 def test_linear_static_packed(ctx, hipq):
     g = torch.Generator(device="cuda").manual_seed(3)
     m, n, k = 96, 160, 512

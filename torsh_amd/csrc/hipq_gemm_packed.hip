@@ -170,6 +170,20 @@ int32_t hipq_quantize_per_tensor_packed_f32_i8(hipq_ctx *ctx, const float *x, si
                                            nullptr, 0);
 }
 
+int32_t hipq_quantize_per_row_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
+                                            int8_t *out_packed, float *out_scales) {
+    HIPQ_ENTER(ctx);
+    if ((rows >> 30) || (cols >> 30)) return fail(HIPQ_SHAPE_ERROR, "%s: dimension too large", __func__);
+    if (rows == 0 || cols == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: Cannot quantize empty tensor", __func__);
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(out_packed);
+    HIPQ_REQUIRE_PTR(out_scales);
+    if (reinterpret_cast<uintptr_t>(out_packed) & 15u)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: the packed buffer must be 16-byte aligned", __func__);
+    if (mode & ~HIPQ_ROUND_HALF_EVEN) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", __func__);
+    return quantize_activations_per_row(ctx, x, rows, cols, mode, out_packed, out_scales, /*packed=*/true);
+}
+
 int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t per_token, const int8_t *w_packed,
                                        const float *w_scales, const float *bias, size_t m, size_t n, size_t k,
                                        int32_t mode, float *out) {

@@ -114,6 +114,7 @@ _SIGNATURES = {
     "hipq_linear_packed_i8_f32": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
     "hipq_linear_packed_i8_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _f32, _i32, _i32, _vp],
     "hipq_quantize_per_tensor_packed_f32_i8": [_vp, _vp, _sz, _sz, _i32, _f32, _i32, _vp, _vp],
+    "hipq_quantize_per_row_packed_f32_i8": [_vp, _vp, _sz, _sz, _i32, _vp, _vp],
     "hipq_linear_dynamic_packed_f32": [_vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_linear_static_packed_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_quantize_per_row_strided_f32_i8": [_vp, _vp, _sz, _sz, _sz, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -574,6 +575,15 @@ class Context:
         self.call("hipq_quantize_per_tensor_packed_f32_i8", _ptr(x), rows, cols, int(dynamic), float(scale), mode,
                   _ptr(out), _ptr(params))
         return out, params
+
+    def quantize_per_row_packed(self, x, mode=0, out=None, scales=None):
+        """Symmetric per-row int8 quantize of fp32 [rows, cols] into the packed layout -> (packed, row scales)."""
+        rows, cols = x.shape
+        out = out if out is not None else torch.empty(self.packed_size(rows, cols), dtype=torch.int8,
+                                                      device=self._dev())
+        scales = scales if scales is not None else torch.empty(rows, dtype=torch.float32, device=self._dev())
+        self.call("hipq_quantize_per_row_packed_f32_i8", _ptr(x), rows, cols, mode, _ptr(out), _ptr(scales))
+        return out, scales
 
     def linear_dynamic_packed(self, x, w_packed, w_scales, bias=None, per_token=False, mode=0, out=None):
         m, k = x.shape
