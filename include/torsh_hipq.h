@@ -309,14 +309,19 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
                                         int32_t mode, int8_t *out);
 /* Test and tuning hook with no counterpart in the reference: forces one of the GEMM kernel forms
  * for every later call on this context wherever the shape allows it (0 = automatic choice, the
- * default; 1-3 one-tile-per-workgroup forms, 5-8 persistent forms, 10 register-staged form).
+ * default; 1-3 one-tile-per-workgroup forms, 5-8 persistent forms, 10 register-staged form); 6 also
+ * makes the dynamic per-tensor packed quantizer run as two launches (range partials, then a quantizer that
+ * folds them) where it would run as one.
  * Results do not depend on it; the parity tests use it to run every form on the same inputs. */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
-/* Test hook with no counterpart in the reference.  The persistent GEMM kernel couples its waves
- * through counters and bounds every wait, so that a grid always drains; a wait that gives up
- * marks the context, and the next hipq_ctx_synchronize returns HIPQ_DEVICE_ERROR once instead of
- * handing back a wrong product silently.  `limit` is the number of polls after the first look
- * (negative = the default, 2^20); 0 lets a test see the error path without hanging anything. */
+/* Test hook with no counterpart in the reference.  Two kernels couple their waves through device
+ * memory: the persistent GEMM kernel (counters between producer and consumer waves) and the one-launch
+ * dynamic per-tensor packed quantizer (its workgroups meet to agree on the range).  Both bound every
+ * wait, so that a grid always drains; a wait that gives up marks the context, and the next
+ * hipq_ctx_synchronize returns HIPQ_DEVICE_ERROR once instead of handing back a wrong result silently
+ * (the quantizer also leaves zero codes, a NaN scale and status HIPQ_DEVICE_ERROR in out_params).
+ * `limit` is the number of polls after the first look (negative = the default, 2^20); 0 lets a test see
+ * the error path without hanging anything. */
 HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
 /* Tuning aid with no counterpart in the reference.  While a device buffer is set, hipq_linear_packed_i8_f32
  * (and the forwards built on it) run a form of the packed GEMM kernel in which every wave records the shader
@@ -387,7 +392,12 @@ HIPQ_API int32_t hipq_linear_packed_i8_i8(hipq_ctx *ctx, const int8_t *a_packed,
  * scale comes from the tensor's own range (quantize_tensor_auto, crates/torsh-quantization/src/algorithms.rs:85-123),
  * otherwise `scale` is used (quantize_per_tensor_affine, algorithms.rs:277-315).  Codes are those of
  * hipq_quantize_dynamic_per_tensor_f32 / hipq_quantize_per_tensor_f32_i8; a range that is not finite
- * gives status HIPQ_INVALID_ARGUMENT in out_params, a NaN scale and zero codes. */
+ * gives status HIPQ_INVALID_ARGUMENT in out_params, a NaN scale and zero codes.
+ * A dynamic call on up to 16384 * (compute units) elements (4 Mi on MI355X), cols % 16 == 0, x 16-byte aligned, is
+ * one kernel: every wave holds its 16 x 64 floats in registers while the workgroups agree on the range
+ * through device words of the context (see hipq_ctx_set_wait_spin_limit), so x is read once.  It keeps no
+ * host state per launch and can be captured and replayed.  Two such calls on one context must not overlap
+ * (they cannot: a context has one stream). */
 HIPQ_API int32_t hipq_quantize_per_tensor_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
                                                         int32_t dynamic, float scale, int32_t mode,
                                                         int8_t *out_packed, hipq_qparams *out_params);

@@ -283,3 +283,102 @@ def test_phase_stamps_do_not_change_the_product(ctx, hipq, oracle):
     assert (t[:, :6] > 0).all()
     assert (np.diff(t[:, :6], axis=1) >= 0).all()
     assert (t[:, 7] >= t[:, 6]).all()
+
+
+def test_one_launch_dynamic_quantize_over_many_launches(hipq):
+    """The dynamic per-tensor packed quantizer of matrices up to four workgroups per compute unit is one kernel
+    whose workgroups meet through device words of the context, numbered by a counter in device memory that starts
+    a few launches before its wrap.  A fresh context therefore crosses the wrap here; grids of different sizes
+    follow one another (a small one after a large one leaves the large one's words behind), inputs change between
+    launches, and every launch must give the codes and parameters of the row-major dynamic quantizer (bit-exact
+    with the oracle, tests/test_gpu_elementwise.py), as must the two-launch form (variant 6) it replaces."""
+    c = hipq.Context(0)
+    try:
+        shapes = [(512, 4096), (1, 16), (1000, 1008), (33, 48), (64, 256), (1024, 4096), (100, 304), (31, 4096)]
+        g = torch.Generator(device="cuda").manual_seed(99)
+        for it in range(48):
+            rows, cols = shapes[it % len(shapes)]
+            x = torch.randn(rows, cols, generator=g, device="cuda") * (1.0 + it)
+            mode = (0, hipq.FORM_DIV, hipq.ROUND_HALF_EVEN, hipq.FORM_DIV | hipq.ROUND_HALF_EVEN)[it % 4]
+            q, params = c.quantize_dynamic_per_tensor(x, mode=mode)
+            pq, pparams = c.quantize_per_tensor_packed(x, dynamic=True, mode=mode)
+            c.set_gemm_kernel_variant(6)
+            pq2, pparams2 = c.quantize_per_tensor_packed(x, dynamic=True, mode=mode)
+            c.set_gemm_kernel_variant(0)
+            c.synchronize()
+            want = c.pack_rows(q)
+            assert torch.equal(pq, want) and torch.equal(pq2, want), (it, rows, cols)
+            a, b, b2 = c.read_qparams(params), c.read_qparams(pparams), c.read_qparams(pparams2)
+            for p in (b, b2):
+                assert (a.scale, a.zero_point, a.min_val, a.max_val, a.status) == (p.scale, p.zero_point, p.min_val,
+                                                                                p.max_val, p.status), (it, rows, cols)
+    finally:
+        c.close()
+
+
+def test_one_launch_dynamic_quantize_gives_up_cleanly(hipq):
+    """With the spin limit forced to 0 workgroup 0 polls every other workgroup's words once, which with 512
+    workgroups is certain to come too early for some: the kernel must still drain, leave zero codes and a NaN scale
+    (never codes made with a partial range), and the context must report HIPQ_DEVICE_ERROR at the next
+    synchronize, once, and work normally again afterwards."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(5)
+        x = torch.randn(512, 4096, generator=g, device="cuda")
+        q, params = c.quantize_dynamic_per_tensor(x)
+        want = c.pack_rows(q)
+        c.synchronize()
+        c.set_wait_spin_limit(0)
+        pq, pparams = c.quantize_per_tensor_packed(x, dynamic=True)
+        with pytest.raises(hipq.HipqError) as e:
+            c.synchronize()
+        assert e.value.code == hipq.DEVICE_ERROR and "gave up" in str(e.value)
+        p = c.read_qparams(pparams)
+        assert p.scale != p.scale and p.status == hipq.DEVICE_ERROR
+        assert not pq.any()
+        c.synchronize()  # reported once, then cleared
+        c.set_wait_spin_limit(-1)
+        for _ in range(3):
+            pq, pparams = c.quantize_per_tensor_packed(x, dynamic=True)
+            c.synchronize()
+            assert torch.equal(pq, want)
+            assert c.read_qparams(pparams).scale == c.read_qparams(params).scale
+    finally:
+        c.close()
+
+
+def test_captured_dynamic_linear_replays(hipq):
+    """The one-launch quantizer keeps no host state per launch (its meeting number lives in device memory), so a
+    captured dynamic Linear forward can be replayed: every replay, with new activations in the captured input
+    buffer and eager work on the same context in between, equals the eager forward of the same activations."""
+    m, n, k = 512, 1024, 1024
+    g = torch.Generator(device="cuda").manual_seed(8)
+    wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(n, generator=g, device="cuda")
+    x = torch.randn(m, k, generator=g, device="cuda")
+    out = torch.empty(m, n, device="cuda")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        c = hipq.Context(0)
+        try:
+            pw = c.pack_rows(wq)
+            c.linear_dynamic_packed(x, pw, sw, bias, out=out)  # grows the scratch outside the capture
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                c.linear_dynamic_packed(x, pw, sw, bias, out=out)
+            for rep in range(24):
+                xn = torch.randn(m, k, generator=g, device="cuda") * (rep + 1)
+                x.copy_(xn)
+                side.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                got = out.clone()
+                eager = c.linear_dynamic_packed(xn, pw, sw, bias)
+                side.synchronize()
+                assert torch.equal(got, eager), rep
+        finally:
+            torch.cuda.synchronize()
+            c.close()

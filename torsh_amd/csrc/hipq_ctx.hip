@@ -60,6 +60,14 @@ int32_t check_launch(const char *what) {
     return HIPQ_SUCCESS;
 }
 
+int32_t reset_ctx_words(hipq_ctx *ctx) {
+    hipError_t e = hipMemset(ctx->wait_error, 0, kCtxWordsBytes);
+    const uint32_t epoch = kCtxFirstEpoch;
+    if (e == hipSuccess) e = hipMemcpy(ctx->wait_error + kCtxEpochWord, &epoch, sizeof(epoch), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return fail(HIPQ_DEVICE_ERROR, "status words of the context: %s", hipGetErrorString(e));
+    return HIPQ_SUCCESS;
+}
+
 }  // namespace hipq
 
 extern "C" {
@@ -104,10 +112,11 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
     int32_t rc = hipq::linear_noalloc_setup(device);
     if (rc == HIPQ_SUCCESS) rc = hipq::scratch(ctx, size_t(8) << 20, &p);
     if (rc == HIPQ_SUCCESS) {
-        e = hipMalloc(reinterpret_cast<void **>(&ctx->wait_error), 256);
-        if (e == hipSuccess) e = hipMemset(ctx->wait_error, 0, 256);
+        e = hipMalloc(reinterpret_cast<void **>(&ctx->wait_error), hipq::kCtxWordsBytes);
         if (e != hipSuccess)
-            rc = hipq::fail(HIPQ_ALLOCATION_ERROR, "hipq_ctx_create: status word: %s", hipGetErrorString(e));
+            rc = hipq::fail(HIPQ_ALLOCATION_ERROR, "hipq_ctx_create: status words: %s", hipGetErrorString(e));
+        else
+            rc = hipq::reset_ctx_words(ctx);
     }
     if (rc != HIPQ_SUCCESS) {
         if (ctx->wait_error) (void)hipFree(ctx->wait_error);
@@ -150,10 +159,14 @@ int32_t hipq_ctx_synchronize(hipq_ctx *ctx) {
     uint32_t gave_up = 0;
     HIPQ_HIP(hipMemcpy(&gave_up, ctx->wait_error, sizeof(gave_up), hipMemcpyDeviceToHost));
     if (gave_up) {
-        HIPQ_HIP(hipMemset(ctx->wait_error, 0, sizeof(gave_up)));
+        // Workgroups that ran after their meeting was given up may have left words that a later meeting would
+        // take for its own: start over.
+        const int32_t rc = hipq::reset_ctx_words(ctx);
+        if (rc) return rc;
         return hipq::fail(HIPQ_DEVICE_ERROR,
-                          "hipq_ctx_synchronize: a bounded wait inside the persistent GEMM kernel gave up "
-                          "(spin limit %d); results of the GEMM calls since the last synchronize are invalid",
+                          "hipq_ctx_synchronize: a bounded wait inside a kernel (persistent GEMM or one-launch "
+                          "dynamic quantize) gave up (spin limit %d); results of the calls since the last "
+                          "synchronize are invalid",
                           ctx->wait_spin_limit);
     }
     return HIPQ_SUCCESS;

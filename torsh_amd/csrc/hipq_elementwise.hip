@@ -334,6 +334,134 @@ __global__ __launch_bounds__(kBlock) void minmax_fragments_kernel(const float *_
     if (threadIdx.x == 0) partials[blockIdx.x] = make_float2(r.mn, r.mx);
 }
 
+// Dynamic per-tensor quantize into the packed layout in ONE launch, for matrices of at most one fragment per wave
+// of the grid.  Every wave keeps its fragment in registers across a meeting of the whole grid:
+//   1. each workgroup publishes its (min, max) as two 64-bit words {meeting number, float bits}, each one atomic
+//      store, so a reader can tell a word of this meeting from what an earlier one left;
+//   2. workgroup 0 polls the words of all workgroups, folds them, derives the parameters, publishes them for the
+//      kernels that follow and ends the meeting with one 64-bit word {meeting number, scale bits};
+//   3. thread 0 of every other workgroup polls that word.
+// That is two trips through device-coherent memory on the critical path; tickets counted with atomics need four
+// and measured 1.3 us slower, the two-kernel form (range partials, then a quantizer that folds them) 1.7 us.
+// The meeting number comes from device memory (`words`, see kCtxEpochWord): every workgroup reads it first, and
+// workgroup 0 advances it once all have published, which they do after reading it; so a launch needs no host
+// state and a captured launch can be replayed.  When the number is about to wrap, workgroup 0 wipes the slots.
+// All waits are bounded (`spin_limit` polls): a workgroup that gives up sets the context's flag word and
+// quantizes with an infinite scale (zero codes; NaN scale published), so the grid always drains.  The caller
+// guarantees that the grid can be resident at once: at most two workgroups per compute unit.
+template <bool DIV, int RND>
+__global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(const float *__restrict__ x, size_t rows,
+                                                                             size_t cols, hipq_qparams *out_params,
+                                                                             uint32_t *words, int spin_limit,
+                                                                             int8_t *__restrict__ out) {
+    __shared__ float lds[2 * kBlock / kWave];
+    __shared__ float s_scale;
+    uint32_t *epoch = words + kCtxEpochWord;
+    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
+    unsigned long long *slots = reinterpret_cast<unsigned long long *>(words + kCtxSlotWord);
+    const FragmentWalk fw(x, rows, cols);
+    const size_t f = fw.first();
+    size_t row, k0;
+    const bool have = fw.whole(f, &row, &k0);
+    float4 v[4];
+    MinMax m{INFINITY, -INFINITY};
+    if (have) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(x + row * cols + k0)[i];
+    }
+    // Behind the fragment's loads in program order: memory operations return in order, and the number is not
+    // needed before the fragment has been folded.
+    const uint32_t gen = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+    const unsigned long long tag = static_cast<unsigned long long>(gen) << 32;
+    if (have) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            m.mn = fminf(m.mn, fminf(fminf(v[i].x, v[i].y), fminf(v[i].z, v[i].w)));
+            m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
+        }
+    }
+    const MinMax r = block_minmax(m, lds);
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(slots + 2 * blockIdx.x, tag | __builtin_bit_cast(uint32_t, r.mn), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(slots + 2 * blockIdx.x + 1, tag | __builtin_bit_cast(uint32_t, r.mx), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float scale;
+    if (blockIdx.x == 0) {
+        MinMax t{INFINITY, -INFINITY};
+        bool all = true;
+        for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) {
+            bool got = false;
+            for (int spin = 0; spin <= spin_limit; ++spin) {
+                const unsigned long long lo = __hip_atomic_load(slots + 2 * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const unsigned long long hi =
+                    __hip_atomic_load(slots + 2 * i + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (static_cast<uint32_t>(lo >> 32) == gen && static_cast<uint32_t>(hi >> 32) == gen) {
+                    t.mn = fminf(t.mn, __builtin_bit_cast(float, static_cast<uint32_t>(lo)));
+                    t.mx = fmaxf(t.mx, __builtin_bit_cast(float, static_cast<uint32_t>(hi)));
+                    got = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            all &= got;
+        }
+        const bool gave_up = __syncthreads_or(!all) != 0;
+        t = block_minmax(t, lds);
+        int zp;
+        int st = params_from_minmax(t.mn, t.mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp);
+        if (gave_up) st = HIPQ_DEVICE_ERROR;
+        const bool bad = st != HIPQ_SUCCESS;
+        if (bad) scale = INFINITY;  // x * (1/inf): 0 for finite x, NaN -> code 0 otherwise
+        if (gen == 0xffffffffu) {
+            // Every workgroup has published (or the meeting is lost anyway): nobody writes a slot any more.
+            for (unsigned i = threadIdx.x; i < 2 * kCtxSlots; i += kBlock)
+                __hip_atomic_store(slots + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(ready, tag | __builtin_bit_cast(uint32_t, scale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(epoch, gen == 0xffffffffu ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (gave_up) __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            out_params->scale = bad ? __builtin_nanf("") : scale;
+            out_params->zero_point = 0;
+            out_params->min_val = t.mn;
+            out_params->max_val = t.mx;
+            out_params->status = st;
+        }
+    } else {
+        if (threadIdx.x == 0) {
+            float sc = INFINITY;
+            bool got = false;
+            for (int spin = 0; spin <= spin_limit; ++spin) {
+                const unsigned long long w = __hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (static_cast<uint32_t>(w >> 32) == gen) {
+                    sc = __builtin_bit_cast(float, static_cast<uint32_t>(w));
+                    got = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (!got) __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_scale = sc;
+        }
+        __syncthreads();
+        scale = s_scale;
+    }
+    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    if (have) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, 0.0f, -128, 127),
+                         quantize_int<DIV, RND>(v[i].y, scale, inv, 0.0f, -128, 127),
+                         quantize_int<DIV, RND>(v[i].z, scale, inv, 0.0f, -128, 127),
+                         quantize_int<DIV, RND>(v[i].w, scale, inv, 0.0f, -128, 127));
+    }
+    if (f < fw.nfrag) *reinterpret_cast<uint4 *>(out + f * 1024 + size_t(fw.lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 template <bool DIV, int RND>
 __global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__restrict__ x, size_t rows,
                                                                   size_t cols, float scale, int zp,
@@ -1058,6 +1186,26 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
     size_t blocks = (nfrag + 3) / 4;
     const size_t cap = size_t(ctx->num_cus) * 8;
     int grid = static_cast<int>(blocks < cap ? blocks : cap);
+    const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    size_t one_launch_cap = size_t(ctx->num_cus) * 4;  // half of what an idle device keeps resident
+    if (one_launch_cap > kCtxSlots) one_launch_cap = kCtxSlots;
+    if (dynamic && packed && ctx->gemm_variant != 6 && blocks <= one_launch_cap && cols % 16 == 0 &&
+        (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+        // Every lane's 16 floats are all inside the matrix or all outside it, and four aligned float4.
+#define HIPQ_LAUNCH_Q1(D, E)                                                                                        \
+    hipLaunchKernelGGL((quantize_packed_one_launch_kernel<D, E>), dim3(static_cast<int>(blocks)), dim3(kBlock), 0, \
+                       ctx->stream, x, rows, cols, out_params, ctx->wait_error, ctx->wait_spin_limit, out)
+        if (div && even)
+            HIPQ_LAUNCH_Q1(true, 1);
+        else if (div)
+            HIPQ_LAUNCH_Q1(true, 0);
+        else if (even)
+            HIPQ_LAUNCH_Q1(false, 1);
+        else
+            HIPQ_LAUNCH_Q1(false, 0);
+#undef HIPQ_LAUNCH_Q1
+        return check_launch("quantize (packed, one launch)");
+    }
     if (dynamic && packed) {
         // Range pass in the quantizer's own order and with its grid (FragmentWalk): one partial per workgroup.
         float2 *p = static_cast<float2 *>(partials);
@@ -1082,7 +1230,6 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
         scale = static_scale;
     }
     if (!packed) return launch_quantize<int8_t>(ctx, x, rows * cols, scale, 0, nullptr, mode, -128.0f, 127.0f, out, dyn);
-    const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
 #define HIPQ_LAUNCH_QP(D, E)                                                                                       \
     hipLaunchKernelGGL((quantize_packed_kernel<D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, rows, cols, scale, \
                        0, static_cast<const hipq_qparams *>(nullptr), dyn, out)

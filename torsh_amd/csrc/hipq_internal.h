@@ -19,7 +19,8 @@ struct hipq_ctx {
     void *scratch = nullptr;
     size_t scratch_bytes = 0;
     int num_cus = 256;
-    // Device word set by a kernel whose bounded wait gave up; read and cleared by hipq_ctx_synchronize.
+    // Device words of the context (kCtxWordsBytes of them, laid out as the kCtx* constants below say).  Word 0 is
+    // set by a kernel whose bounded wait gave up; hipq_ctx_synchronize reads and clears it.
     uint32_t *wait_error = nullptr;
     // Test and tuning hooks, per context: forced GEMM kernel form (0 = automatic, -1 = not yet read from the
     // HIPQ_GEMM_VARIANT environment variable) and the spin limit of the persistent kernel's waits.
@@ -31,6 +32,21 @@ struct hipq_ctx {
 };
 
 namespace hipq {
+
+// Layout of hipq_ctx::wait_error, in 32-bit words.  Beyond the give-up flag it holds the meeting point of the
+// one-launch dynamic quantizer (quantize_packed_one_launch_kernel): the number of the last meeting, the 64-bit
+// word {meeting, scale bits} that ends one, and per workgroup two 64-bit words {meeting, min} and {meeting, max}.
+constexpr size_t kCtxFlagWord = 0;
+constexpr size_t kCtxEpochWord = 16;
+constexpr size_t kCtxReadyWord = 32;
+constexpr size_t kCtxSlotWord = 64;
+constexpr size_t kCtxSlots = 2048;  // workgroups that can meet
+constexpr size_t kCtxWordsBytes = kCtxSlotWord * 4 + kCtxSlots * 16;
+// Number the first meeting of a context gets, a few launches before the counter wraps, so that the wrap (which
+// wipes the slots) is a path every context takes early, not once in 2^32 launches.
+constexpr uint32_t kCtxFirstEpoch = 0xfffffff0u;
+// Puts the device words of a context into their initial state (device current, stream idle).
+int32_t reset_ctx_words(hipq_ctx *ctx);
 
 // Records `msg` (printf style) as the calling thread's last error and returns `code`.
 int32_t fail(int32_t code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));

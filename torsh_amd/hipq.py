@@ -245,7 +245,8 @@ class Context:
             self.call("hipq_ctx_set_trace_buffer", _ptr(buf), buf.numel() * buf.element_size())
 
     def set_wait_spin_limit(self, limit: int) -> None:
-        """Test hook: polls a bounded wait of the persistent GEMM kernel makes before it gives up (< 0: default)."""
+        """Test hook: polls a bounded wait (persistent GEMM, one-launch dynamic quantizer) makes before it gives
+        up (< 0: default)."""
         self.call("hipq_ctx_set_wait_spin_limit", int(limit))
 
     def synchronize(self) -> None:
