@@ -407,9 +407,9 @@ HIPQ_API int32_t hipq_quantize_per_tensor_packed_f32_i8(hipq_ctx *ctx, const flo
  * not finite gets a NaN scale and zero codes. */
 HIPQ_API int32_t hipq_quantize_per_row_packed_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols,
                                                      int32_t mode, int8_t *out_packed, float *out_scales);
-/* hipq_linear_dynamic_f32 with prepared (packed) weights: per tensor a range pass, the quantizer writing the packed
- * layout and the packed GEMM with the dequantizing epilogue; per token the per-row quantizer (one pass) and the
- * GEMM. */
+/* hipq_linear_dynamic_f32 with prepared (packed) weights: per tensor the dynamic quantizer of
+ * hipq_quantize_per_tensor_packed_f32_i8 (one launch where its conditions hold, else a range pass and a quantizer)
+ * and the packed GEMM with the dequantizing epilogue; per token the per-row quantizer (one pass) and the GEMM. */
 HIPQ_API int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t per_token,
                                                 const int8_t *w_packed, const float *w_scales, const float *bias,
                                                 size_t m, size_t n, size_t k, int32_t mode, float *out);

@@ -317,10 +317,11 @@ def test_one_launch_dynamic_quantize_over_many_launches(hipq):
 
 
 def test_one_launch_dynamic_quantize_gives_up_cleanly(hipq):
-    """With the spin limit forced to 0 workgroup 0 polls every other workgroup's words once, which with 512
-    workgroups is certain to come too early for some: the kernel must still drain, leave zero codes and a NaN scale
-    (never codes made with a partial range), and the context must report HIPQ_DEVICE_ERROR at the next
-    synchronize, once, and work normally again afterwards."""
+    """With the spin limit forced to 0 every workgroup looks at the other workgroups' range words exactly once,
+    which with 512 workgroups is certain to come too early for some of them: the kernel must still drain, a
+    workgroup that gave up must leave zero codes (never codes made with a partial range), the others the right
+    codes, and the context must report HIPQ_DEVICE_ERROR at the next synchronize, once, and work normally again
+    afterwards."""
     c = hipq.Context(0)
     try:
         g = torch.Generator(device="cuda").manual_seed(5)
@@ -334,8 +335,12 @@ def test_one_launch_dynamic_quantize_gives_up_cleanly(hipq):
             c.synchronize()
         assert e.value.code == hipq.DEVICE_ERROR and "gave up" in str(e.value)
         p = c.read_qparams(pparams)
-        assert p.scale != p.scale and p.status == hipq.DEVICE_ERROR
-        assert not pq.any()
+        if p.status == hipq.DEVICE_ERROR:  # workgroup 0 was among those that gave up
+            assert p.scale != p.scale
+        else:
+            assert p.status == hipq.SUCCESS and p.scale == c.read_qparams(params).scale
+        assert bool(((pq == 0) | (pq == want)).all())
+        assert bool((pq != want).any())  # somebody did give up
         c.synchronize()  # reported once, then cleared
         c.set_wait_spin_limit(-1)
         for _ in range(3):

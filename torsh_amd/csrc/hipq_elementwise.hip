@@ -5,42 +5,12 @@
 // latency, and wave-level shuffles for the reductions.
 #include "hipq_internal.h"
 #include "hipq_math.h"
+#include "hipq_meeting.h"
 
 namespace hipq {
 
-constexpr int kBlock = 256;
 constexpr int kVecPerThread = 4;                         // float4 loads in flight per lane
 constexpr int kTileVec = kBlock * kVecPerThread;         // float4s per block iteration
-
-struct MinMax {
-    float mn, mx;
-};
-
-__device__ __forceinline__ void acc_minmax(MinMax &m, float v) {
-    m.mn = fminf(m.mn, v);
-    m.mx = fmaxf(m.mx, v);
-}
-
-// Block-wide min/max; result valid in every thread.
-__device__ __forceinline__ MinMax block_minmax(MinMax m, float *lds /* 2 * kBlock/kWave + 2 floats */) {
-    m.mn = wave_min(m.mn);
-    m.mx = wave_max(m.mx);
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    constexpr int nw = kBlock / kWave;
-    __syncthreads();
-    if (lane == 0) {
-        lds[wave] = m.mn;
-        lds[nw + wave] = m.mx;
-    }
-    __syncthreads();
-    MinMax r{lds[0], lds[nw]};
-#pragma unroll
-    for (int w = 1; w < nw; ++w) {
-        r.mn = fminf(r.mn, lds[w]);
-        r.mx = fmaxf(r.mx, lds[nw + w]);
-    }
-    return r;
-}
 
 // Stage 1 of the range reduction: each block folds a strided set of 4096-element
 // tiles and writes one (min,max) partial.
@@ -335,30 +305,15 @@ __global__ __launch_bounds__(kBlock) void minmax_fragments_kernel(const float *_
 }
 
 // Dynamic per-tensor quantize into the packed layout in ONE launch, for matrices of at most one fragment per wave
-// of the grid.  Every wave keeps its fragment in registers across a meeting of the whole grid:
-//   1. each workgroup publishes its (min, max) as two 64-bit words {meeting number, float bits}, each one atomic
-//      store, so a reader can tell a word of this meeting from what an earlier one left;
-//   2. workgroup 0 polls the words of all workgroups, folds them, derives the parameters, publishes them for the
-//      kernels that follow and ends the meeting with one 64-bit word {meeting number, scale bits};
-//   3. thread 0 of every other workgroup polls that word.
-// That is two trips through device-coherent memory on the critical path; tickets counted with atomics need four
-// and measured 1.3 us slower, the two-kernel form (range partials, then a quantizer that folds them) 1.7 us.
-// The meeting number comes from device memory (`words`, see kCtxEpochWord): every workgroup reads it first, and
-// workgroup 0 advances it once all have published, which they do after reading it; so a launch needs no host
-// state and a captured launch can be replayed.  When the number is about to wrap, workgroup 0 wipes the slots.
-// All waits are bounded (`spin_limit` polls): a workgroup that gives up sets the context's flag word and
-// quantizes with an infinite scale (zero codes; NaN scale published), so the grid always drains.  The caller
-// guarantees that the grid can be resident at once: at most two workgroups per compute unit.
+// of the grid: every wave keeps its fragment in registers while the grid agrees on the range (hipq_meeting.h), so
+// the matrix is read once.  The two-kernel form (range partials, then a quantizer that folds them) measured 1.7 us
+// more at 512 x 4096 and is what larger matrices use.  The caller guarantees that the grid can be resident at once.
 template <bool DIV, int RND>
 __global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(const float *__restrict__ x, size_t rows,
                                                                              size_t cols, hipq_qparams *out_params,
                                                                              uint32_t *words, int spin_limit,
                                                                              int8_t *__restrict__ out) {
-    __shared__ float lds[2 * kBlock / kWave];
-    __shared__ float s_scale;
-    uint32_t *epoch = words + kCtxEpochWord;
-    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
-    unsigned long long *slots = reinterpret_cast<unsigned long long *>(words + kCtxSlotWord);
+    __shared__ float lds[kMeetingLdsFloats];
     const FragmentWalk fw(x, rows, cols);
     const size_t f = fw.first();
     size_t row, k0;
@@ -371,8 +326,7 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(cons
     }
     // Behind the fragment's loads in program order: memory operations return in order, and the number is not
     // needed before the fragment has been folded.
-    const uint32_t gen = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-    const unsigned long long tag = static_cast<unsigned long long>(gen) << 32;
+    const uint32_t gen = meeting_number(words);
     if (have) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -381,74 +335,8 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(cons
         }
     }
     const MinMax r = block_minmax(m, lds);
-    if (threadIdx.x == 0) {
-        __hip_atomic_store(slots + 2 * blockIdx.x, tag | __builtin_bit_cast(uint32_t, r.mn), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(slots + 2 * blockIdx.x + 1, tag | __builtin_bit_cast(uint32_t, r.mx), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    }
-    float scale;
-    if (blockIdx.x == 0) {
-        MinMax t{INFINITY, -INFINITY};
-        bool all = true;
-        for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) {
-            bool got = false;
-            for (int spin = 0; spin <= spin_limit; ++spin) {
-                const unsigned long long lo = __hip_atomic_load(slots + 2 * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const unsigned long long hi =
-                    __hip_atomic_load(slots + 2 * i + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (static_cast<uint32_t>(lo >> 32) == gen && static_cast<uint32_t>(hi >> 32) == gen) {
-                    t.mn = fminf(t.mn, __builtin_bit_cast(float, static_cast<uint32_t>(lo)));
-                    t.mx = fmaxf(t.mx, __builtin_bit_cast(float, static_cast<uint32_t>(hi)));
-                    got = true;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-            all &= got;
-        }
-        const bool gave_up = __syncthreads_or(!all) != 0;
-        t = block_minmax(t, lds);
-        int zp;
-        int st = params_from_minmax(t.mn, t.mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp);
-        if (gave_up) st = HIPQ_DEVICE_ERROR;
-        const bool bad = st != HIPQ_SUCCESS;
-        if (bad) scale = INFINITY;  // x * (1/inf): 0 for finite x, NaN -> code 0 otherwise
-        if (gen == 0xffffffffu) {
-            // Every workgroup has published (or the meeting is lost anyway): nobody writes a slot any more.
-            for (unsigned i = threadIdx.x; i < 2 * kCtxSlots; i += kBlock)
-                __hip_atomic_store(slots + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-        }
-        if (threadIdx.x == 0) {
-            __hip_atomic_store(ready, tag | __builtin_bit_cast(uint32_t, scale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(epoch, gen == 0xffffffffu ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (gave_up) __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            out_params->scale = bad ? __builtin_nanf("") : scale;
-            out_params->zero_point = 0;
-            out_params->min_val = t.mn;
-            out_params->max_val = t.mx;
-            out_params->status = st;
-        }
-    } else {
-        if (threadIdx.x == 0) {
-            float sc = INFINITY;
-            bool got = false;
-            for (int spin = 0; spin <= spin_limit; ++spin) {
-                const unsigned long long w = __hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (static_cast<uint32_t>(w >> 32) == gen) {
-                    sc = __builtin_bit_cast(float, static_cast<uint32_t>(w));
-                    got = true;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-            if (!got) __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_scale = sc;
-        }
-        __syncthreads();
-        scale = s_scale;
-    }
+    const float published = meet_on_range(words, gen, r, spin_limit, lds, out_params);
+    const float scale = published == published ? published : INFINITY;  // x * (1/inf): 0; NaN -> code 0
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
     if (have) {

@@ -34,14 +34,14 @@ struct hipq_ctx {
 namespace hipq {
 
 // Layout of hipq_ctx::wait_error, in 32-bit words.  Beyond the give-up flag it holds the meeting point of the
-// one-launch dynamic quantizer (quantize_packed_one_launch_kernel): the number of the last meeting, the 64-bit
-// word {meeting, scale bits} that ends one, and per workgroup two 64-bit words {meeting, min} and {meeting, max}.
+// one-launch dynamic quantizer (hipq_meeting.h): the number of the last meeting, the 64-bit word {meeting,
+// scale bits} that ends one, and per workgroup the two 64-bit words {meeting, min}, {meeting, max}.
 constexpr size_t kCtxFlagWord = 0;
 constexpr size_t kCtxEpochWord = 16;
 constexpr size_t kCtxReadyWord = 32;
-constexpr size_t kCtxSlotWord = 64;
+constexpr size_t kCtxRangeWord = 64;
 constexpr size_t kCtxSlots = 2048;  // workgroups that can meet
-constexpr size_t kCtxWordsBytes = kCtxSlotWord * 4 + kCtxSlots * 16;
+constexpr size_t kCtxWordsBytes = (kCtxRangeWord + kCtxSlots * 4) * 4;
 // Number the first meeting of a context gets, a few launches before the counter wraps, so that the wrap (which
 // wipes the slots) is a path every context takes early, not once in 2^32 launches.
 constexpr uint32_t kCtxFirstEpoch = 0xfffffff0u;

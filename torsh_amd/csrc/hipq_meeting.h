@@ -1,0 +1,165 @@
+// A meeting of all workgroups of one launch, through device words of the context: the grid agrees on the
+// (min, max) of a tensor of which every workgroup has seen a part, without ending the kernel.
+//
+// Every word another workgroup waits for is a 64-bit {meeting number, payload} pair written by one atomic
+// store, so a reader can tell a word of this meeting from what an earlier one left behind; nothing is reset
+// between launches.  The number comes from device memory: every workgroup reads it first (meeting_number),
+// and workgroup 0 advances it once all workgroups have published their range, which they do after reading it.
+// A launch therefore needs no host state and a captured launch can be replayed.  When the number is about to
+// wrap, workgroup 0 wipes the range words (nobody reads them any more once all have published), so that none
+// can be taken for a word of a meeting 2^32 launches later.
+//
+// Every workgroup publishes {number, min} and {number, max}; workgroup 0 polls the words of all workgroups,
+// folds them, derives the parameters and publishes {number, scale}; thread 0 of every other workgroup polls
+// that word.  That is two trips through device-coherent memory on the critical path (~1.5 us each).
+// Measured alternatives: arrival counters need four trips and cross-XCD atomics on one address serialise
+// (+1.3 us); every workgroup polling every workgroup's words needs one trip, but 512 workgroups reading the
+// same 64 lines past their L2s round after round cost more than the trip saved (+1.2 us).
+//
+// All waits are bounded: a poll that gives up sets the context's flag word (hipq_ctx_synchronize reports
+// it) and the kernel runs on with defined values, so a grid always drains.  The caller guarantees that the
+// grid can be resident at once; launches that share a context's words must not overlap (they are on the
+// context's one stream).  256 threads per workgroup.
+#pragma once
+
+#include "hipq_internal.h"
+#include "hipq_math.h"
+
+namespace hipq {
+
+constexpr int kBlock = 256;
+
+struct MinMax {
+    float mn, mx;
+};
+
+__device__ __forceinline__ void acc_minmax(MinMax &m, float v) {
+    m.mn = fminf(m.mn, v);
+    m.mx = fmaxf(m.mx, v);
+}
+
+// Block-wide min/max; result valid in every thread.
+__device__ __forceinline__ MinMax block_minmax(MinMax m, float *lds /* 2 * kBlock/kWave floats */) {
+    m.mn = wave_min(m.mn);
+    m.mx = wave_max(m.mx);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    constexpr int nw = kBlock / kWave;
+    __syncthreads();
+    if (lane == 0) {
+        lds[wave] = m.mn;
+        lds[nw + wave] = m.mx;
+    }
+    __syncthreads();
+    MinMax r{lds[0], lds[nw]};
+#pragma unroll
+    for (int w = 1; w < nw; ++w) {
+        r.mn = fminf(r.mn, lds[w]);
+        r.mx = fmaxf(r.mx, lds[nw + w]);
+    }
+    return r;
+}
+
+constexpr int kMeetingLdsFloats = 2 * kBlock / kWave + 1;
+
+// The number of the meeting this launch holds.  Call it before anything of the meeting is published.
+__device__ __forceinline__ uint32_t meeting_number(const uint32_t *words) {
+    return __hip_atomic_load(words + kCtxEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+}
+
+// {number, min}, {number, max} of workgroup `workgroup`.
+__device__ __forceinline__ unsigned long long *meeting_range_slot(uint32_t *words, unsigned workgroup) {
+    return reinterpret_cast<unsigned long long *>(words + kCtxRangeWord) + 2 * size_t(workgroup);
+}
+__device__ __forceinline__ void publish_tagged(unsigned long long *word, uint32_t gen, uint32_t payload) {
+    __hip_atomic_store(word, (static_cast<unsigned long long>(gen) << 32) | payload, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Polls `word` until it carries meeting `gen` (at most spin_limit + 1 looks); false = gave up.
+__device__ __forceinline__ bool poll_tagged(const unsigned long long *word, uint32_t gen, int spin_limit,
+                                            uint32_t *payload) {
+    for (int spin = 0; spin <= spin_limit; ++spin) {
+        const unsigned long long w = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (static_cast<uint32_t>(w >> 32) == gen) {
+            *payload = static_cast<uint32_t>(w);
+            return true;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    return false;
+}
+
+__device__ __forceinline__ void record_give_up(uint32_t *words) {
+    __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The whole grid agrees on the symmetric int8 scale of a tensor: `r` is this workgroup's (min, max), uniform
+// over its threads.  Returns, in every thread of every workgroup, the scale that workgroup 0 also writes to
+// out_params: NaN when the range is not finite or a wait of the meeting was given up (the caller then
+// quantizes with an infinite scale: zero codes).  `lds`: kMeetingLdsFloats floats.
+__device__ __forceinline__ float meet_on_range(uint32_t *words, uint32_t gen, MinMax r, int spin_limit, float *lds,
+                                               hipq_qparams *out_params) {
+    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
+    if (threadIdx.x == 0) {
+        unsigned long long *mine = meeting_range_slot(words, blockIdx.x);
+        publish_tagged(mine, gen, __builtin_bit_cast(uint32_t, r.mn));
+        publish_tagged(mine + 1, gen, __builtin_bit_cast(uint32_t, r.mx));
+    }
+    float published;
+    if (blockIdx.x == 0) {
+        MinMax t{INFINITY, -INFINITY};
+        bool all = true;
+        for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) {
+            uint32_t lo = 0, hi = 0;
+            const unsigned long long *slot = meeting_range_slot(words, i);
+            const bool got = poll_tagged(slot, gen, spin_limit, &lo) && poll_tagged(slot + 1, gen, spin_limit, &hi);
+            if (got) {
+                t.mn = fminf(t.mn, __builtin_bit_cast(float, lo));
+                t.mx = fmaxf(t.mx, __builtin_bit_cast(float, hi));
+            }
+            all &= got;
+        }
+        const bool gave_up = __syncthreads_or(!all) != 0;
+        t = block_minmax(t, lds);
+        float scale;
+        int zp;
+        int st = params_from_minmax(t.mn, t.mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp);
+        if (gave_up) st = HIPQ_DEVICE_ERROR;
+        published = st == HIPQ_SUCCESS ? scale : __builtin_nanf("");
+        const bool wrap = gen == 0xffffffffu;
+        if (wrap) {
+            // Every workgroup has published (or the meeting is lost anyway): nobody writes or reads a range
+            // word any more.
+            unsigned long long *first = meeting_range_slot(words, 0);
+            for (unsigned i = threadIdx.x; i < 2 * kCtxSlots; i += kBlock)
+                __hip_atomic_store(first + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            publish_tagged(ready, gen, __builtin_bit_cast(uint32_t, published));
+            // Every workgroup has published, so every workgroup has read the number.
+            __hip_atomic_store(words + kCtxEpochWord, wrap ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (gave_up) record_give_up(words);
+            out_params->scale = published;
+            out_params->zero_point = 0;
+            out_params->min_val = t.mn;
+            out_params->max_val = t.mx;
+            out_params->status = st;
+        }
+    } else {
+        if (threadIdx.x == 0) {
+            uint32_t bits = 0;
+            if (poll_tagged(ready, gen, spin_limit, &bits)) {
+                lds[kMeetingLdsFloats - 1] = __builtin_bit_cast(float, bits);
+            } else {
+                record_give_up(words);
+                lds[kMeetingLdsFloats - 1] = __builtin_nanf("");
+            }
+        }
+        __syncthreads();
+        published = lds[kMeetingLdsFloats - 1];
+    }
+    return published;
+}
+
+}  // namespace hipq
