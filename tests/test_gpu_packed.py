@@ -50,6 +50,7 @@ SHAPES = [
     (1, 1, 16), (1, 16, 64), (16, 16, 64), (17, 33, 128), (64, 64, 256), (128, 64, 128), (130, 70, 144),
     (127, 129, 4096), (512, 256, 1024), (5, 300, 48), (256, 512, 16), (33, 1000, 2048), (9, 40, 1001), (3, 5, 7),
     (129, 65, 512), (200, 96, 768), (256, 128, 2304), (96, 200, 11008),
+    (2100, 1100, 512), (4100, 600, 272),  # more tiles than compute units: two workgroups per compute unit
 ]
 
 
@@ -159,6 +160,23 @@ def test_quantize_per_row_packed_matches_row_major(ctx, hipq, rows, cols):
         torch.cuda.synchronize()
         assert torch.equal(pq, ctx.pack_rows(q))
         assert torch.equal(ps, s)
+
+
+@pytest.mark.parametrize("m,n,k", [(8192, 768, 768), (4100, 1100, 272)])
+def test_linear_packed_many_tiles_matches_row_major(ctx, hipq, m, n, k):
+    """More tiles than compute units (the packed kernel then runs two workgroups per compute unit and sums its K
+    split one column block at a time), fp32 epilogue with per-row activation scales and bias: the same bits as
+    the row-major entry point, which the oracle tests of tests/test_gpu_gemm.py pin."""
+    g = torch.Generator(device="cuda").manual_seed(m + n + k)
+    a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    sa = torch.rand(m, generator=g, device="cuda") * 1e-2 + 1e-3
+    sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(n, generator=g, device="cuda")
+    want = ctx.linear_i8_f32(a, sa, w, sw, bias)
+    got = ctx.linear_packed_i8_f32(ctx.pack_rows(a), sa, ctx.pack_rows(w), sw, bias, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
 
 
 def test_linear_static_packed(ctx, hipq):

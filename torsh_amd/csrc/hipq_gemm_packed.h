@@ -215,7 +215,7 @@ __device__ __forceinline__ void conv_store_block(v16i (&own)[1][TNB], const Gemm
 // [channel block of 32][padded pixel][32 bytes] order (conv_pack_image_kernel), N = padded pixels = windows:
 // window q's fragment for (tap, channel block) is the 32 pixels from q + tap offset on, 1 KiB contiguous, so a
 // window fragment is one coalesced wave load like a packed one, with no im2col and no gather.
-template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false>
+template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false, bool HALVES = false>
 __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__restrict__ PA,
                                                              const int8_t *__restrict__ PW, int M, int N, int K,
                                                              GemmEpilogue ep) {
@@ -389,6 +389,38 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
     // owner, wave (wave + i) % TMB, through LDS: [owner][slot i-1][column block][4 registers][lane] of 16
     // bytes; the three writers of one owner use three different slots.  Integer adds: any order, same bits.
     v4i *red = reinterpret_cast<v4i *>(lds);
+    v16i own[1][TNB];
+    if constexpr (HALVES) {
+        // One column block at a time: half the LDS (48 KB), so that two workgroups share a compute unit and one
+        // runs its loop while the other sums and stores.  [owner][slot i-1][4 registers][lane] of 16 bytes.
+#pragma unroll
+        for (int j = 0; j < TNB; ++j) {
+            if (j) __syncthreads();  // the previous column block has been read
+#pragma unroll
+            for (int i = 1; i < TMB; ++i) {
+                const int owner = (wave + i) % TMB;
+                v4i *dst = red + ((owner * (TMB - 1) + (i - 1)) * 4) * kWave + lane;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    dst[g * kWave] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+            }
+            __syncthreads();
+            v4i part[TMB - 1][4];
+            const v4i *src = red + (wave * (TMB - 1) * 4) * kWave + lane;
+#pragma unroll
+            for (int sl = 0; sl < TMB - 1; ++sl)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) part[sl][g] = src[(sl * 4 + g) * kWave];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int v = acc[0][j][r];
+#pragma unroll
+                for (int sl = 0; sl < TMB - 1; ++sl) v += part[sl][r / 4][r % 4];
+                own[0][j][r] = v;
+            }
+        }
+    } else {
 #pragma unroll
     for (int i = 1; i < TMB; ++i) {
         const int owner = (wave + i) % TMB;
@@ -412,7 +444,6 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
 #pragma unroll
             for (int g = 0; g < 4; ++g) part[sl][j][g] = src[((sl * TNB + j) * 4 + g) * kWave];
     __builtin_amdgcn_sched_barrier(0);
-    v16i own[1][TNB];
 #pragma unroll
     for (int j = 0; j < TNB; ++j)
 #pragma unroll
@@ -422,6 +453,7 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
             for (int sl = 0; sl < TMB - 1; ++sl) v += part[sl][j][r / 4][r % 4];
             own[0][j][r] = v;
         }
+    }
     mark(3);
     const int row0 = m0 + wave * 32;
     if constexpr (CONV) {
@@ -567,11 +599,11 @@ __global__ __launch_bounds__(256) void pack_rows_i8_kernel(const int8_t *__restr
     }
 }
 
-template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false>
+template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false, bool HALVES = false>
 static int32_t launch_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                              const GemmEpilogue &ep) {
-    constexpr int kLds = TMB * TNB * 3 * 4096;
-    auto kernel = gemm_i8_packed_kernel<TMB, TNB, D, EPI, EVEN, TRACE, CONV>;
+    constexpr int kLds = TMB * (HALVES ? 1 : TNB) * 3 * 4096;
+    auto kernel = gemm_i8_packed_kernel<TMB, TNB, D, EPI, EVEN, TRACE, CONV, HALVES>;
     static bool configured[16] = {false};  // per device: raise the dynamic LDS limit once
     if (ctx->device < 16 && !configured[ctx->device]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -605,6 +637,17 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
         const size_t tiles = ((packed_row_blocks(m) + 3) / 4) * ((packed_row_blocks(n) + 1) / 2);
         if (ctx->trace && steps % 2 == 0 && ctx->trace_bytes >= tiles * 4 * kTraceWords * sizeof(unsigned long long))
             return launch_packed<4, 2, 2, EPI, EVEN, true>(ctx, pa, pw, M, N, K, ep);
+    }
+    if constexpr (EPI != EPI_I8) {
+        // More tiles than compute units: the form that sums one column block at a time (48 KB of LDS), so that two
+        // workgroups share a compute unit and one runs its loop while the other sums and stores (M = 8192, N = 2304,
+        // K = 768: 43.6 -> 31.3 us; M = 2048, N = K = 4096: 50.2 -> 43.2 us).  The int8 epilogue needs more than
+        // half the register file, so two of its workgroups would not fit anyway.
+        const size_t tiles = ((packed_row_blocks(m) + 3) / 4) * ((packed_row_blocks(n) + 1) / 2);
+        if (tiles > size_t(ctx->num_cus) && ctx->gemm_variant != 9) {
+            if (steps % 2 == 0) return launch_packed<4, 2, 2, EPI, EVEN, false, false, true>(ctx, pa, pw, M, N, K, ep);
+            return launch_packed<4, 2, 1, EPI, EVEN, false, false, true>(ctx, pa, pw, M, N, K, ep);
+        }
     }
     if (steps % 2 == 0) return launch_packed<4, 2, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     return launch_packed<4, 2, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
