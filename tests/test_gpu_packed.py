@@ -334,6 +334,33 @@ def test_one_launch_dynamic_quantize_over_many_launches(hipq):
         c.close()
 
 
+def test_flat_one_launch_dynamic_quantize_over_many_launches(hipq):
+    """The same one-launch quantizer with a row-major output, behind hipq_linear_dynamic_f32 (activations of up to
+    4 Mi elements, a multiple of 4): over a fresh context's first 48 launches (across the wrap of the meeting
+    number, grids of changing size, all four modes) the forward equals the one whose quantizer runs as two
+    launches (variant 6), which tests/test_gpu_gemm.py pins to the oracle."""
+    c = hipq.Context(0)
+    try:
+        shapes = [(512, 4096), (1, 4), (1000, 1008), (33, 48), (64, 256), (1024, 4096), (100, 304), (3, 20), (7, 9)]
+        g = torch.Generator(device="cuda").manual_seed(123)
+        n = 40
+        for it in range(48):
+            m, k = shapes[it % len(shapes)]
+            x = torch.randn(m, k, generator=g, device="cuda") * (1.0 + it)
+            wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+            sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+            bias = torch.randn(n, generator=g, device="cuda")
+            mode = (0, hipq.FORM_DIV, hipq.ROUND_HALF_EVEN, hipq.FORM_DIV | hipq.ROUND_HALF_EVEN)[it % 4]
+            got = c.linear_dynamic(x, wq, sw, bias, mode=mode)
+            c.set_gemm_kernel_variant(6)
+            want = c.linear_dynamic(x, wq, sw, bias, mode=mode)
+            c.set_gemm_kernel_variant(0)
+            c.synchronize()
+            assert torch.equal(got, want), (it, m, k, mode)
+    finally:
+        c.close()
+
+
 def test_one_launch_dynamic_quantize_gives_up_cleanly(hipq):
     """With the spin limit forced to 0 every workgroup looks at the other workgroups' range words exactly once,
     which with 512 workgroups is certain to come too early for some of them: the kernel must still drain, a

@@ -350,6 +350,45 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(cons
     if (f < fw.nfrag) *reinterpret_cast<uint4 *>(out + f * 1024 + size_t(fw.lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The same for a flat (row-major) output: a workgroup keeps 4096 consecutive elements in registers (four float4
+// per lane, each load and each store of a wave 1 KiB contiguous).  n is a multiple of 4 and x is 16-byte aligned.
+template <bool DIV, int RND>
+__global__ __launch_bounds__(kBlock) void quantize_flat_one_launch_kernel(const float *__restrict__ x, size_t n,
+                                                                           hipq_qparams *out_params, uint32_t *words,
+                                                                           int spin_limit, int8_t *__restrict__ out) {
+    __shared__ float lds[kMeetingLdsFloats];
+    const size_t nvec = n / 4;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    const size_t base = size_t(blockIdx.x) * kTileVec + threadIdx.x;
+    float4 v[kVecPerThread];
+    bool have[kVecPerThread];
+#pragma unroll
+    for (int i = 0; i < kVecPerThread; ++i) {
+        have[i] = base + size_t(i) * kBlock < nvec;
+        if (have[i]) v[i] = x4[base + size_t(i) * kBlock];
+    }
+    const uint32_t gen = meeting_number(words);  // behind the data in program order: returned after it
+    MinMax m{INFINITY, -INFINITY};
+#pragma unroll
+    for (int i = 0; i < kVecPerThread; ++i)
+        if (have[i]) {
+            m.mn = fminf(m.mn, fminf(fminf(v[i].x, v[i].y), fminf(v[i].z, v[i].w)));
+            m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
+        }
+    const MinMax r = block_minmax(m, lds);
+    const float published = meet_on_range(words, gen, r, spin_limit, lds, out_params);
+    const float scale = published == published ? published : INFINITY;  // x * (1/inf): 0; NaN -> code 0
+    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
+    uint32_t *out4 = reinterpret_cast<uint32_t *>(out);
+#pragma unroll
+    for (int i = 0; i < kVecPerThread; ++i)
+        if (have[i])
+            out4[base + size_t(i) * kBlock] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, 0.0f, -128, 127),
+                                                    quantize_int<DIV, RND>(v[i].y, scale, inv, 0.0f, -128, 127),
+                                                    quantize_int<DIV, RND>(v[i].z, scale, inv, 0.0f, -128, 127),
+                                                    quantize_int<DIV, RND>(v[i].w, scale, inv, 0.0f, -128, 127));
+}
+
 template <bool DIV, int RND>
 __global__ __launch_bounds__(kBlock) void quantize_packed_kernel(const float *__restrict__ x, size_t rows,
                                                                   size_t cols, float scale, int zp,
@@ -1110,7 +1149,24 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
         dyn.partials = p;
         dyn.nparts = grid;
     } else if (dynamic) {
-        rc = launch_minmax_partials(ctx, x, rows * cols, &dyn, static_cast<float2 *>(partials),
+        const size_t n = rows * cols, flat_blocks = (n / 4 + kTileVec - 1) / kTileVec;
+        if (ctx->gemm_variant != 6 && flat_blocks <= one_launch_cap && n % 4 == 0 &&
+            (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(out) & 3u) == 0) {
+#define HIPQ_LAUNCH_Q1F(D, E)                                                                                      \
+    hipLaunchKernelGGL((quantize_flat_one_launch_kernel<D, E>), dim3(static_cast<int>(flat_blocks)), dim3(kBlock), 0, \
+                       ctx->stream, x, n, out_params, ctx->wait_error, ctx->wait_spin_limit, out)
+            if (div && even)
+                HIPQ_LAUNCH_Q1F(true, 1);
+            else if (div)
+                HIPQ_LAUNCH_Q1F(true, 0);
+            else if (even)
+                HIPQ_LAUNCH_Q1F(false, 1);
+            else
+                HIPQ_LAUNCH_Q1F(false, 0);
+#undef HIPQ_LAUNCH_Q1F
+            return check_launch("quantize (flat, one launch)");
+        }
+        rc = launch_minmax_partials(ctx, x, n, &dyn, static_cast<float2 *>(partials),
                                     partials_bytes / sizeof(float2));
         if (rc) return rc;
     } else {
