@@ -186,7 +186,12 @@ HIPQ_API int32_t hipq_quantize_with_params_f32_u8(hipq_ctx *ctx, const float *x,
                                                   const hipq_qparams *params, int32_t mode, uint8_t *out);
 /* quantize_tensor_auto, algorithms.rs:85-123: min/max -> params (`flavor`) ->
  * quantize, all on the device.  dtype is HIPQ_DTYPE_I8 (out is int8_t*) or
- * HIPQ_DTYPE_U8 (out is uint8_t*).  out_params receives the parameters. */
+ * HIPQ_DTYPE_U8 (out is uint8_t*).  out_params receives the parameters.
+ * Up to 65536 * (compute units) elements (16 Mi on MI355X: a 4096 x 4096 tensor), n % 4 == 0, x 16-byte and
+ * out 4-byte aligned, mode within HIPQ_FORM_DIV | HIPQ_ROUND_HALF_EVEN: one kernel that keeps the tensor in
+ * registers between the range and the codes (up to 64 floats a lane, four workgroups per compute unit), so x
+ * is read from memory once; its workgroups agree on the range through device words of the context (see
+ * hipq_ctx_set_wait_spin_limit).  Anything else: a range pass, then a quantizer that folds its partials. */
 HIPQ_API int32_t hipq_quantize_dynamic_per_tensor_f32(hipq_ctx *ctx, const float *x, size_t n, int32_t flavor,
                                                       int32_t dtype, int32_t mode, void *out,
                                                       hipq_qparams *out_params);

@@ -216,12 +216,43 @@ def test_config1_full_size_properties(ctx, hipq):
     assert torch.equal(q, ref)
 
 
-def test_non_finite_range_sets_status_and_skips(ctx, hipq):
-    x = torch.tensor([1.0, float("inf"), 2.0] * 50, device="cuda")
-    out = torch.full((150,), 77, dtype=torch.int8, device="cuda")
+@pytest.mark.parametrize("n", [150, 152, 5 * (1 << 20)])
+def test_non_finite_range_sets_status_and_skips(ctx, hipq, n):
+    """150 elements take the two-launch path (not a multiple of 4), 152 the one-launch path with 4 float4 per
+    lane, 5 Mi the one with 16: each must report the status and leave the output untouched."""
+    x = torch.ones(n, device="cuda")
+    x[n // 3] = float("inf")
+    out = torch.full((n,), 77, dtype=torch.int8, device="cuda")
     _, params = ctx.quantize_dynamic_per_tensor(x, out=out)
-    assert ctx.read_qparams(params).status == hipq.INVALID_ARGUMENT
+    p = ctx.read_qparams(params)
+    assert p.status == hipq.INVALID_ARGUMENT and p.scale == 1.0
     assert bool((out == 77).all())
+
+
+@pytest.mark.parametrize("n", [1000, 6 * (1 << 20) + 4])
+@pytest.mark.parametrize("dtype_name", ["i8", "u8"])
+def test_dynamic_quantize_one_launch_matches_two_launches(hipq, n, dtype_name):
+    """Every parameter flavour and both quantize forms and roundings through the one-launch dynamic quantizer (the
+    tensor stays in registers between the range and the codes; 6 Mi + 4 elements: 16 float4 per lane and a ragged
+    last workgroup) against the two-launch path (variant 6), whose kernels the oracle tests above pin."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(n % 977)
+        x = torch.randn(n, generator=g, device="cuda") * 3.0 + 0.5
+        dtype = hipq.DTYPE_I8 if dtype_name == "i8" else hipq.DTYPE_U8
+        for flavor in range(7):
+            for mode in (0, hipq.FORM_DIV, hipq.ROUND_HALF_EVEN, hipq.FORM_DIV | hipq.ROUND_HALF_EVEN):
+                q, params = c.quantize_dynamic_per_tensor(x, flavor, dtype, mode)
+                c.set_gemm_kernel_variant(6)
+                q2, params2 = c.quantize_dynamic_per_tensor(x, flavor, dtype, mode)
+                c.set_gemm_kernel_variant(0)
+                c.synchronize()
+                a, b = c.read_qparams(params), c.read_qparams(params2)
+                assert (a.scale, a.zero_point, a.min_val, a.max_val, a.status) == (b.scale, b.zero_point, b.min_val,
+                                                                                b.max_val, b.status), (flavor, mode)
+                assert torch.equal(q, q2), (flavor, mode)
+    finally:
+        c.close()
 
 
 @pytest.mark.parametrize("shape", [(1, 8), (3, 33), (16, 4096), (5, 1024), (7, 1025), (4, 4100), (2, 20000), (64, 768)])

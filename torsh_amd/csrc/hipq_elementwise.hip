@@ -335,8 +335,9 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(cons
         }
     }
     const MinMax r = block_minmax(m, lds);
-    const float published = meet_on_range(words, gen, r, spin_limit, lds, out_params);
-    const float scale = published == published ? published : INFINITY;  // x * (1/inf): 0; NaN -> code 0
+    const MeetingParams agreed = meet_on_range(words, gen, r, HIPQ_PARAMS_SYMMETRIC, -128, 127, /*poison=*/true, spin_limit,
+                                               lds, out_params);
+    const float scale = agreed.scale == agreed.scale ? agreed.scale : INFINITY;  // x * (1/inf): 0; NaN -> code 0
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
     if (have) {
@@ -350,43 +351,115 @@ __global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(cons
     if (f < fw.nfrag) *reinterpret_cast<uint4 *>(out + f * 1024 + size_t(fw.lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// The same for a flat (row-major) output: a workgroup keeps 4096 consecutive elements in registers (four float4
-// per lane, each load and each store of a wave 1 KiB contiguous).  n is a multiple of 4 and x is 16-byte aligned.
-template <bool DIV, int RND>
-__global__ __launch_bounds__(kBlock) void quantize_flat_one_launch_kernel(const float *__restrict__ x, size_t n,
-                                                                           hipq_qparams *out_params, uint32_t *words,
-                                                                           int spin_limit, int8_t *__restrict__ out) {
+// The same for a flat output, any parameter flavor and int8 / uint8 codes: a workgroup keeps VPT x 1024 consecutive
+// elements in registers (VPT float4 per lane; each load and each store of a wave 1 KiB contiguous).  VPT = 16 is
+// 64 registers of data per lane: with four workgroups per compute unit the chip's register files hold 16 Mi
+// floats, so even a 4096 x 4096 tensor is read from memory once (29.5 -> ~20 us).  The launch bound keeps the
+// kernel at 128 registers, which is what lets four workgroups share a compute unit: the grid has to be resident
+// at once.  n is a multiple of 4, x is 16-byte and out 4-byte aligned.  `poison`: what a bad range leaves behind,
+// see meet_on_range; without it no code is written, as in the two-launch path.
+template <typename OutT, bool DIV, int RND, int VPT>
+__global__ __launch_bounds__(kBlock, 4) void quantize_flat_one_launch_kernel(const float *__restrict__ x, size_t n,
+                                                                              int flavor, int qmin, int qmax,
+                                                                              int poison, hipq_qparams *out_params,
+                                                                              uint32_t *words, int spin_limit,
+                                                                              OutT *__restrict__ out) {
+    static_assert(sizeof(OutT) == 1, "int8 or uint8 codes");
     __shared__ float lds[kMeetingLdsFloats];
     const size_t nvec = n / 4;
     const float4 *x4 = reinterpret_cast<const float4 *>(x);
-    const size_t base = size_t(blockIdx.x) * kTileVec + threadIdx.x;
-    float4 v[kVecPerThread];
-    bool have[kVecPerThread];
+    const size_t base = size_t(blockIdx.x) * (size_t(kBlock) * VPT) + threadIdx.x;
+    const bool whole = (size_t(blockIdx.x) + 1) * (size_t(kBlock) * VPT) <= nvec;
+    float4 v[VPT];
+    if (whole) {
 #pragma unroll
-    for (int i = 0; i < kVecPerThread; ++i) {
-        have[i] = base + size_t(i) * kBlock < nvec;
-        if (have[i]) v[i] = x4[base + size_t(i) * kBlock];
+        for (int i = 0; i < VPT; ++i) v[i] = load_stream(x4 + base + size_t(i) * kBlock);
+    } else {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            // past the end: a value that changes neither the minimum nor the maximum (NaN is skipped by both)
+            v[i] = make_float4(NAN, NAN, NAN, NAN);
+            if (base + size_t(i) * kBlock < nvec) v[i] = x4[base + size_t(i) * kBlock];
+        }
     }
     const uint32_t gen = meeting_number(words);  // behind the data in program order: returned after it
     MinMax m{INFINITY, -INFINITY};
 #pragma unroll
-    for (int i = 0; i < kVecPerThread; ++i)
-        if (have[i]) {
-            m.mn = fminf(m.mn, fminf(fminf(v[i].x, v[i].y), fminf(v[i].z, v[i].w)));
-            m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
-        }
+    for (int i = 0; i < VPT; ++i) {
+        m.mn = fminf(m.mn, fminf(fminf(v[i].x, v[i].y), fminf(v[i].z, v[i].w)));
+        m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
+    }
     const MinMax r = block_minmax(m, lds);
-    const float published = meet_on_range(words, gen, r, spin_limit, lds, out_params);
-    const float scale = published == published ? published : INFINITY;  // x * (1/inf): 0; NaN -> code 0
+    const MeetingParams agreed = meet_on_range(words, gen, r, flavor, qmin, qmax, poison != 0, spin_limit, lds, out_params);
+    float scale = agreed.scale;
+    if (scale != scale) {
+        if (!poison) return;  // the reference errors before quantizing
+        scale = INFINITY;      // x * (1/inf) and x / inf: 0 for finite x, NaN -> code 0 otherwise
+    }
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
+    const float zpf = static_cast<float>(agreed.zero_point);
     uint32_t *out4 = reinterpret_cast<uint32_t *>(out);
 #pragma unroll
-    for (int i = 0; i < kVecPerThread; ++i)
-        if (have[i])
-            out4[base + size_t(i) * kBlock] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, 0.0f, -128, 127),
-                                                    quantize_int<DIV, RND>(v[i].y, scale, inv, 0.0f, -128, 127),
-                                                    quantize_int<DIV, RND>(v[i].z, scale, inv, 0.0f, -128, 127),
-                                                    quantize_int<DIV, RND>(v[i].w, scale, inv, 0.0f, -128, 127));
+    for (int i = 0; i < VPT; ++i)
+        if (whole || base + size_t(i) * kBlock < nvec)
+            store_stream(out4 + base + size_t(i) * kBlock,
+                         pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, zpf, qmin, qmax),
+                               quantize_int<DIV, RND>(v[i].y, scale, inv, zpf, qmin, qmax),
+                               quantize_int<DIV, RND>(v[i].z, scale, inv, zpf, qmin, qmax),
+                               quantize_int<DIV, RND>(v[i].w, scale, inv, zpf, qmin, qmax)));
+}
+
+// Launches the kernel above when the call qualifies (returns true), else leaves the two-launch path to the caller.
+// The grid must be resident at once: at most four workgroups per compute unit, which the kernel's launch bound
+// makes room for; checked against the runtime's own occupancy figure the first time.
+template <typename OutT>
+static bool launch_flat_one_launch(hipq_ctx *ctx, const float *x, size_t n, int flavor, int qmin, int qmax, int mode,
+                                   bool poison, hipq_qparams *out_params, OutT *out, int32_t *rc) {
+    if (ctx->gemm_variant == 6 || n % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) ||
+        (reinterpret_cast<uintptr_t>(out) & 3u) || (mode & ~(HIPQ_FORM_DIV | HIPQ_ROUND_HALF_EVEN)))
+        return false;
+    size_t cap = size_t(ctx->num_cus) * 4;
+    if (cap > kCtxSlots) cap = kCtxSlots;
+    const size_t nvec = n / 4;
+    const int vpt = nvec <= cap * kBlock * 4 ? 4 : 16;
+    const size_t blocks = (nvec + size_t(kBlock) * vpt - 1) / (size_t(kBlock) * vpt);
+    if (blocks > cap) return false;
+    static int resident[16] = {0};  // per device: workgroups of the widest form per compute unit, 0 = not asked yet
+    if (vpt == 16 && ctx->device < 16) {
+        if (resident[ctx->device] == 0) {
+            int per_cu = 0;
+            const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                &per_cu, reinterpret_cast<const void *>(quantize_flat_one_launch_kernel<int8_t, false, 0, 16>), kBlock, 0);
+            resident[ctx->device] = (e == hipSuccess && per_cu > 0) ? per_cu : -1;
+        }
+        if (resident[ctx->device] < 4) return false;
+    } else if (vpt == 16) {
+        return false;
+    }
+    const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+#define HIPQ_LAUNCH_Q1F(D, E, V)                                                                                       \
+    hipLaunchKernelGGL((quantize_flat_one_launch_kernel<OutT, D, E, V>), dim3(static_cast<int>(blocks)), dim3(kBlock), 0, \
+                       ctx->stream, x, n, flavor, qmin, qmax, poison ? 1 : 0, out_params, ctx->wait_error,             \
+                       ctx->wait_spin_limit, out)
+#define HIPQ_LAUNCH_Q1F_MODE(V)          \
+    do {                                 \
+        if (div && even)                 \
+            HIPQ_LAUNCH_Q1F(true, 1, V); \
+        else if (div)                    \
+            HIPQ_LAUNCH_Q1F(true, 0, V); \
+        else if (even)                   \
+            HIPQ_LAUNCH_Q1F(false, 1, V); \
+        else                             \
+            HIPQ_LAUNCH_Q1F(false, 0, V); \
+    } while (0)
+    if (vpt == 4)
+        HIPQ_LAUNCH_Q1F_MODE(4);
+    else
+        HIPQ_LAUNCH_Q1F_MODE(16);
+#undef HIPQ_LAUNCH_Q1F_MODE
+#undef HIPQ_LAUNCH_Q1F
+    *rc = check_launch("quantize (flat, one launch)");
+    return true;
 }
 
 template <bool DIV, int RND>
@@ -978,6 +1051,14 @@ int32_t hipq::quantize_dynamic_per_tensor(hipq_ctx *ctx, const float *x, size_t 
     if (dtype != HIPQ_DTYPE_I8 && dtype != HIPQ_DTYPE_U8)
         return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown dtype %d", fn, dtype);
     const int qmin = dtype == HIPQ_DTYPE_I8 ? -128 : 0, qmax = dtype == HIPQ_DTYPE_I8 ? 127 : 255;
+    if (dtype == HIPQ_DTYPE_I8) {
+        if (launch_flat_one_launch<int8_t>(ctx, x, n, flavor, qmin, qmax, mode, false, out_params,
+                                           static_cast<int8_t *>(out), &rc))
+            return rc;
+    } else if (launch_flat_one_launch<uint8_t>(ctx, x, n, flavor, qmin, qmax, mode, false, out_params,
+                                               static_cast<uint8_t *>(out), &rc)) {
+        return rc;
+    }
     DynamicRange dyn{nullptr, 0, flavor, qmin, qmax, out_params};
     rc = launch_minmax_partials(ctx, x, n, &dyn, static_cast<float2 *>(partials), partials_cap / sizeof(float2));
     if (rc) return rc;
@@ -1149,23 +1230,10 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
         dyn.partials = p;
         dyn.nparts = grid;
     } else if (dynamic) {
-        const size_t n = rows * cols, flat_blocks = (n / 4 + kTileVec - 1) / kTileVec;
-        if (ctx->gemm_variant != 6 && flat_blocks <= one_launch_cap && n % 4 == 0 &&
-            (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(out) & 3u) == 0) {
-#define HIPQ_LAUNCH_Q1F(D, E)                                                                                      \
-    hipLaunchKernelGGL((quantize_flat_one_launch_kernel<D, E>), dim3(static_cast<int>(flat_blocks)), dim3(kBlock), 0, \
-                       ctx->stream, x, n, out_params, ctx->wait_error, ctx->wait_spin_limit, out)
-            if (div && even)
-                HIPQ_LAUNCH_Q1F(true, 1);
-            else if (div)
-                HIPQ_LAUNCH_Q1F(true, 0);
-            else if (even)
-                HIPQ_LAUNCH_Q1F(false, 1);
-            else
-                HIPQ_LAUNCH_Q1F(false, 0);
-#undef HIPQ_LAUNCH_Q1F
-            return check_launch("quantize (flat, one launch)");
-        }
+        const size_t n = rows * cols;
+        if (launch_flat_one_launch<int8_t>(ctx, x, n, HIPQ_PARAMS_SYMMETRIC, -128, 127, mode, /*poison=*/true, out_params,
+                                           out, &rc))
+            return rc;
         rc = launch_minmax_partials(ctx, x, n, &dyn, static_cast<float2 *>(partials),
                                     partials_bytes / sizeof(float2));
         if (rc) return rc;

@@ -34,8 +34,8 @@ struct hipq_ctx {
 namespace hipq {
 
 // Layout of hipq_ctx::wait_error, in 32-bit words.  Beyond the give-up flag it holds the meeting point of the
-// one-launch dynamic quantizer (hipq_meeting.h): the number of the last meeting, the 64-bit word {meeting,
-// scale bits} that ends one, and per workgroup the two 64-bit words {meeting, min}, {meeting, max}.
+// one-launch dynamic quantizer (hipq_meeting.h): the number of the last meeting, the two 64-bit words {meeting,
+// scale bits}, {meeting, zero point} that end one, and per workgroup the two 64-bit words {meeting, min}, {meeting, max}.
 constexpr size_t kCtxFlagWord = 0;
 constexpr size_t kCtxEpochWord = 16;
 constexpr size_t kCtxReadyWord = 32;

@@ -10,8 +10,8 @@
 // can be taken for a word of a meeting 2^32 launches later.
 //
 // Every workgroup publishes {number, min} and {number, max}; workgroup 0 polls the words of all workgroups,
-// folds them, derives the parameters and publishes {number, scale}; thread 0 of every other workgroup polls
-// that word.  That is two trips through device-coherent memory on the critical path (~1.5 us each).
+// folds them, derives the parameters and publishes {number, scale} and {number, zero point}; thread 0 of every
+// other workgroup polls those two words.  That is two trips through device-coherent memory on the critical path (~1.5 us each).
 // Measured alternatives: arrival counters need four trips and cross-XCD atomics on one address serialise
 // (+1.3 us); every workgroup polling every workgroup's words needs one trip, but 512 workgroups reading the
 // same 64 lines past their L2s round after round cost more than the trip saved (+1.2 us).
@@ -59,7 +59,7 @@ __device__ __forceinline__ MinMax block_minmax(MinMax m, float *lds /* 2 * kBloc
     return r;
 }
 
-constexpr int kMeetingLdsFloats = 2 * kBlock / kWave + 1;
+constexpr int kMeetingLdsFloats = 2 * kBlock / kWave + 2;
 
 // The number of the meeting this launch holds.  Call it before anything of the meeting is published.
 __device__ __forceinline__ uint32_t meeting_number(const uint32_t *words) {
@@ -93,19 +93,28 @@ __device__ __forceinline__ void record_give_up(uint32_t *words) {
     __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// The whole grid agrees on the symmetric int8 scale of a tensor: `r` is this workgroup's (min, max), uniform
-// over its threads.  Returns, in every thread of every workgroup, the scale that workgroup 0 also writes to
-// out_params: NaN when the range is not finite or a wait of the meeting was given up (the caller then
-// quantizes with an infinite scale: zero codes).  `lds`: kMeetingLdsFloats floats.
-__device__ __forceinline__ float meet_on_range(uint32_t *words, uint32_t gen, MinMax r, int spin_limit, float *lds,
-                                               hipq_qparams *out_params) {
-    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
+// What a meeting agrees on: the parameters workgroup 0 derives from the folded range.  scale is NaN when the
+// range is not acceptable to the flavor (not finite, ...) or a wait of the meeting was given up.
+struct MeetingParams {
+    float scale;
+    int zero_point;
+};
+
+// The whole grid agrees on the quantization parameters of a tensor: `r` is this workgroup's (min, max), uniform
+// over its threads; flavor / qmin / qmax as for params_from_minmax.  Returns the same parameters in every thread of
+// every workgroup.  Workgroup 0 also writes them to out_params, with the status; for a bad range it records a
+// NaN scale if `poison` is set (the fused Linear forwards, whose GEMM must then produce NaN) and the neutral 1.0 of
+// the two-launch path otherwise.  `lds`: kMeetingLdsFloats floats.
+__device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t gen, MinMax r, int flavor, int qmin,
+                                                       int qmax, bool poison, int spin_limit, float *lds,
+                                                       hipq_qparams *out_params) {
+    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);  // scale, then zp
     if (threadIdx.x == 0) {
         unsigned long long *mine = meeting_range_slot(words, blockIdx.x);
         publish_tagged(mine, gen, __builtin_bit_cast(uint32_t, r.mn));
         publish_tagged(mine + 1, gen, __builtin_bit_cast(uint32_t, r.mx));
     }
-    float published;
+    MeetingParams p;
     if (blockIdx.x == 0) {
         MinMax t{INFINITY, -INFINITY};
         bool all = true;
@@ -123,9 +132,11 @@ __device__ __forceinline__ float meet_on_range(uint32_t *words, uint32_t gen, Mi
         t = block_minmax(t, lds);
         float scale;
         int zp;
-        int st = params_from_minmax(t.mn, t.mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp);
+        int st = params_from_minmax(t.mn, t.mx, flavor, qmin, qmax, &scale, &zp);
         if (gave_up) st = HIPQ_DEVICE_ERROR;
-        published = st == HIPQ_SUCCESS ? scale : __builtin_nanf("");
+        const bool bad = st != HIPQ_SUCCESS;
+        p.scale = bad ? __builtin_nanf("") : scale;
+        p.zero_point = bad ? 0 : zp;
         const bool wrap = gen == 0xffffffffu;
         if (wrap) {
             // Every workgroup has published (or the meeting is lost anyway): nobody writes or reads a range
@@ -136,30 +147,34 @@ __device__ __forceinline__ float meet_on_range(uint32_t *words, uint32_t gen, Mi
             __syncthreads();
         }
         if (threadIdx.x == 0) {
-            publish_tagged(ready, gen, __builtin_bit_cast(uint32_t, published));
+            publish_tagged(ready, gen, __builtin_bit_cast(uint32_t, p.scale));
+            publish_tagged(ready + 1, gen, static_cast<uint32_t>(p.zero_point));
             // Every workgroup has published, so every workgroup has read the number.
             __hip_atomic_store(words + kCtxEpochWord, wrap ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (gave_up) record_give_up(words);
-            out_params->scale = published;
-            out_params->zero_point = 0;
+            out_params->scale = (bad && !poison) ? scale : p.scale;
+            out_params->zero_point = bad ? zp : p.zero_point;
             out_params->min_val = t.mn;
             out_params->max_val = t.mx;
             out_params->status = st;
         }
     } else {
         if (threadIdx.x == 0) {
-            uint32_t bits = 0;
-            if (poll_tagged(ready, gen, spin_limit, &bits)) {
-                lds[kMeetingLdsFloats - 1] = __builtin_bit_cast(float, bits);
+            uint32_t bits = 0, zbits = 0;
+            if (poll_tagged(ready, gen, spin_limit, &bits) && poll_tagged(ready + 1, gen, spin_limit, &zbits)) {
+                lds[kMeetingLdsFloats - 2] = __builtin_bit_cast(float, bits);
+                lds[kMeetingLdsFloats - 1] = __builtin_bit_cast(float, zbits);
             } else {
                 record_give_up(words);
-                lds[kMeetingLdsFloats - 1] = __builtin_nanf("");
+                lds[kMeetingLdsFloats - 2] = __builtin_nanf("");
+                lds[kMeetingLdsFloats - 1] = 0.0f;
             }
         }
         __syncthreads();
-        published = lds[kMeetingLdsFloats - 1];
+        p.scale = lds[kMeetingLdsFloats - 2];
+        p.zero_point = __builtin_bit_cast(int, lds[kMeetingLdsFloats - 1]);
     }
-    return published;
+    return p;
 }
 
 }  // namespace hipq
