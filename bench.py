@@ -481,6 +481,8 @@ def main() -> int:
         # `value`, which stays the one-stream figure.
         ctx2 = hipq.Context(0, own_stream=True)
         ctx3 = hipq.Context(0, own_stream=True)
+        ctx2.set_resident_share(2)
+        ctx3.set_resident_share(2)
         pt = [0]
 
         def step_two_streams():

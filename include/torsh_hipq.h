@@ -328,6 +328,13 @@ HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
  * `limit` is the number of polls after the first look (negative = the default, 2^20); 0 lets a test see
  * the error path without hanging anything. */
 HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
+/* No counterpart in the reference.  The one-launch dynamic quantizers need their whole grid resident on the device
+ * at once and size it for the device being theirs: up to half of it (four light workgroups per compute unit) for
+ * tensors of up to 4 Mi elements, all of its register files above that.  When `contexts` contexts launch such
+ * work concurrently (one per serving thread, say), tell each of them so: it then sizes those grids for 1 / contexts
+ * of the device and takes the two-launch path for what does not fit, instead of two half-resident grids waiting
+ * for each other until their bounded waits give up.  Default 1; 1..64. */
+HIPQ_API int32_t hipq_ctx_set_resident_share(hipq_ctx *ctx, int32_t contexts);
 /* Tuning aid with no counterpart in the reference.  While a device buffer is set, hipq_linear_packed_i8_f32
  * (and the forwards built on it) run a form of the packed GEMM kernel in which every wave records the shader
  * clock at six points - start, first operands in registers, end of the K loop, partial sums reduced, stores
@@ -398,8 +405,8 @@ HIPQ_API int32_t hipq_linear_packed_i8_i8(hipq_ctx *ctx, const int8_t *a_packed,
  * otherwise `scale` is used (quantize_per_tensor_affine, algorithms.rs:277-315).  Codes are those of
  * hipq_quantize_dynamic_per_tensor_f32 / hipq_quantize_per_tensor_f32_i8; a range that is not finite
  * gives status HIPQ_INVALID_ARGUMENT in out_params, a NaN scale and zero codes.
- * A dynamic call on up to 16384 * (compute units) elements (4 Mi on MI355X), cols % 16 == 0, x 16-byte aligned, is
- * one kernel: every wave holds its 16 x 64 floats in registers while the workgroups agree on the range
+ * A dynamic call on up to 65536 * (compute units) elements (16 Mi on MI355X), cols % 16 == 0, x 16-byte aligned, is
+ * one kernel: every wave holds its one or four fragments of 16 x 64 floats in registers while the workgroups agree on the range
  * through device words of the context (see hipq_ctx_set_wait_spin_limit), so x is read once.  It keeps no
  * host state per launch and can be captured and replayed.  Two such calls on one context must not overlap
  * (they cannot: a context has one stream). */

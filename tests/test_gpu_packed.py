@@ -304,15 +304,17 @@ def test_phase_stamps_do_not_change_the_product(ctx, hipq, oracle):
 
 
 def test_one_launch_dynamic_quantize_over_many_launches(hipq):
-    """The dynamic per-tensor packed quantizer of matrices up to four workgroups per compute unit is one kernel
-    whose workgroups meet through device words of the context, numbered by a counter in device memory that starts
+    """The dynamic per-tensor packed quantizer of matrices of up to 16 Mi elements is one kernel (one or four
+    fragments per wave, at most four workgroups per compute unit) whose workgroups meet through device words of the
+    context, numbered by a counter in device memory that starts
     a few launches before its wrap.  A fresh context therefore crosses the wrap here; grids of different sizes
     follow one another (a small one after a large one leaves the large one's words behind), inputs change between
     launches, and every launch must give the codes and parameters of the row-major dynamic quantizer (bit-exact
     with the oracle, tests/test_gpu_elementwise.py), as must the two-launch form (variant 6) it replaces."""
     c = hipq.Context(0)
     try:
-        shapes = [(512, 4096), (1, 16), (1000, 1008), (33, 48), (64, 256), (1024, 4096), (100, 304), (31, 4096)]
+        shapes = [(512, 4096), (1, 16), (1000, 1008), (33, 48), (64, 256), (1024, 4096), (100, 304), (31, 4096),
+                  (2048, 4096), (5000, 1008)]  # the last two: four fragments per wave
         g = torch.Generator(device="cuda").manual_seed(99)
         for it in range(48):
             rows, cols = shapes[it % len(shapes)]
@@ -357,6 +359,32 @@ def test_flat_one_launch_dynamic_quantize_over_many_launches(hipq):
             c.set_gemm_kernel_variant(0)
             c.synchronize()
             assert torch.equal(got, want), (it, m, k, mode)
+    finally:
+        c.close()
+
+
+def test_resident_share_changes_the_path_not_the_result(hipq):
+    """hipq_ctx_set_resident_share(ctx, n) tells a context that n contexts launch concurrently: the one-launch
+    quantizers then size their grids for 1 / n of the device and what does not fit takes two launches.  The codes
+    and parameters are the same whatever the share; out-of-range shares are refused."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(21)
+        for rows, cols in ((512, 4096), (2048, 4096), (4096, 4096)):
+            x = torch.randn(rows, cols, generator=g, device="cuda")
+            want = None
+            for share in (1, 2, 4, 8, 64):
+                c.set_resident_share(share)
+                pq, pparams = c.quantize_per_tensor_packed(x, dynamic=True)
+                q, params = c.quantize_dynamic_per_tensor(x.reshape(-1))
+                c.synchronize()
+                got = (pq.clone(), q.clone(), c.read_qparams(pparams).scale, c.read_qparams(params).scale)
+                if want is None:
+                    want = got
+                assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]) and got[2:] == want[2:], (rows, share)
+        for bad in (0, -1, 65):
+            with pytest.raises(hipq.HipqError):
+                c.set_resident_share(bad)
     finally:
         c.close()
 

@@ -180,6 +180,14 @@ int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant) {
     return HIPQ_SUCCESS;
 }
 
+int32_t hipq_ctx_set_resident_share(hipq_ctx *ctx, int32_t contexts) {
+    HIPQ_REQUIRE_PTR(ctx);
+    if (contexts < 1 || contexts > 64)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: %d is not in 1..64", __func__, contexts);
+    ctx->resident_share = contexts;
+    return HIPQ_SUCCESS;
+}
+
 int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit) {
     HIPQ_REQUIRE_PTR(ctx);
     ctx->wait_spin_limit = limit < 0 ? (1 << 20) : limit;

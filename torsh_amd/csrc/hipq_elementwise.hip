@@ -304,51 +304,65 @@ __global__ __launch_bounds__(kBlock) void minmax_fragments_kernel(const float *_
     if (threadIdx.x == 0) partials[blockIdx.x] = make_float2(r.mn, r.mx);
 }
 
-// Dynamic per-tensor quantize into the packed layout in ONE launch, for matrices of at most one fragment per wave
-// of the grid: every wave keeps its fragment in registers while the grid agrees on the range (hipq_meeting.h), so
-// the matrix is read once.  The two-kernel form (range partials, then a quantizer that folds them) measured 1.7 us
-// more at 512 x 4096 and is what larger matrices use.  The caller guarantees that the grid can be resident at once.
-template <bool DIV, int RND>
-__global__ __launch_bounds__(kBlock) void quantize_packed_one_launch_kernel(const float *__restrict__ x, size_t rows,
-                                                                             size_t cols, hipq_qparams *out_params,
-                                                                             uint32_t *words, int spin_limit,
-                                                                             int8_t *__restrict__ out) {
+// Dynamic per-tensor quantize into the packed layout in ONE launch, for matrices of at most FPW fragments per wave
+// of the grid: every wave keeps its fragments in registers (16 floats a lane each) while the grid agrees on the
+// range (hipq_meeting.h), so the matrix is read once.  The two-kernel form (range partials, then a quantizer that
+// folds them) measured 1.7 us more at 512 x 4096 with FPW = 1; FPW = 4 with four workgroups per compute unit
+// covers 16 Mi elements.  The launch bound keeps the kernel at 128 registers, so that four workgroups fit a
+// compute unit: the caller relies on the grid being resident at once.  Wave w of the grid takes fragments
+// w, w + waves, ...
+template <bool DIV, int RND, int FPW>
+__global__ __launch_bounds__(kBlock, 4) void quantize_packed_one_launch_kernel(const float *__restrict__ x, size_t rows,
+                                                                                size_t cols, hipq_qparams *out_params,
+                                                                                uint32_t *words, int spin_limit,
+                                                                                int8_t *__restrict__ out) {
     __shared__ float lds[kMeetingLdsFloats];
     const FragmentWalk fw(x, rows, cols);
-    const size_t f = fw.first();
-    size_t row, k0;
-    const bool have = fw.whole(f, &row, &k0);
-    float4 v[4];
-    MinMax m{INFINITY, -INFINITY};
-    if (have) {
+    size_t f[FPW];
+    bool have[FPW];
+    float4 v[FPW][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<const float4 *>(x + row * cols + k0)[i];
-    }
-    // Behind the fragment's loads in program order: memory operations return in order, and the number is not
-    // needed before the fragment has been folded.
-    const uint32_t gen = meeting_number(words);
-    if (have) {
+    for (int u = 0; u < FPW; ++u) {
+        f[u] = fw.first() + u * fw.fstep;
+        size_t row, k0;
+        have[u] = fw.whole(f[u], &row, &k0);
+        if (have[u]) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            m.mn = fminf(m.mn, fminf(fminf(v[i].x, v[i].y), fminf(v[i].z, v[i].w)));
-            m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
+            for (int i = 0; i < 4; ++i) v[u][i] = reinterpret_cast<const float4 *>(x + row * cols + k0)[i];
         }
     }
+    // Behind the fragments' loads in program order: memory operations return in order, and the number is not
+    // needed before the fragments have been folded.
+    const uint32_t gen = meeting_number(words);
+    MinMax m{INFINITY, -INFINITY};
+#pragma unroll
+    for (int u = 0; u < FPW; ++u)
+        if (have[u]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                m.mn = fminf(m.mn, fminf(fminf(v[u][i].x, v[u][i].y), fminf(v[u][i].z, v[u][i].w)));
+                m.mx = fmaxf(m.mx, fmaxf(fmaxf(v[u][i].x, v[u][i].y), fmaxf(v[u][i].z, v[u][i].w)));
+            }
+        }
     const MinMax r = block_minmax(m, lds);
     const MeetingParams agreed = meet_on_range(words, gen, r, HIPQ_PARAMS_SYMMETRIC, -128, 127, /*poison=*/true, spin_limit,
                                                lds, out_params);
     const float scale = agreed.scale == agreed.scale ? agreed.scale : INFINITY;  // x * (1/inf): 0; NaN -> code 0
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
-    uint32_t w[4] = {0u, 0u, 0u, 0u};
-    if (have) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            w[i] = pack4(quantize_int<DIV, RND>(v[i].x, scale, inv, 0.0f, -128, 127),
-                         quantize_int<DIV, RND>(v[i].y, scale, inv, 0.0f, -128, 127),
-                         quantize_int<DIV, RND>(v[i].z, scale, inv, 0.0f, -128, 127),
-                         quantize_int<DIV, RND>(v[i].w, scale, inv, 0.0f, -128, 127));
+    for (int u = 0; u < FPW; ++u) {
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (have[u]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = pack4(quantize_int<DIV, RND>(v[u][i].x, scale, inv, 0.0f, -128, 127),
+                             quantize_int<DIV, RND>(v[u][i].y, scale, inv, 0.0f, -128, 127),
+                             quantize_int<DIV, RND>(v[u][i].z, scale, inv, 0.0f, -128, 127),
+                             quantize_int<DIV, RND>(v[u][i].w, scale, inv, 0.0f, -128, 127));
+        }
+        if (f[u] < fw.nfrag)
+            *reinterpret_cast<uint4 *>(out + f[u] * 1024 + size_t(fw.lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
     }
-    if (f < fw.nfrag) *reinterpret_cast<uint4 *>(out + f * 1024 + size_t(fw.lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
 // The same for a flat output, any parameter flavor and int8 / uint8 codes: a workgroup keeps VPT x 1024 consecutive
@@ -409,6 +423,22 @@ __global__ __launch_bounds__(kBlock, 4) void quantize_flat_one_launch_kernel(con
                                quantize_int<DIV, RND>(v[i].w, scale, inv, zpf, qmin, qmax)));
 }
 
+// The one-launch quantizers that hold 64 floats a lane need four workgroups per compute unit resident: what the
+// runtime says about the widest flat form (the packed one has the same launch bound), asked once per device.
+static bool four_wide_workgroups_fit(const hipq_ctx *ctx) {
+    static int resident[16] = {0};  // workgroups per compute unit; 0 = not asked yet, -1 = the query failed
+    if (ctx->device < 0 || ctx->device >= 16) return false;
+    if (resident[ctx->device] == 0) {
+        int a = 0, b = 0;
+        const hipError_t ea = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &a, reinterpret_cast<const void *>(quantize_flat_one_launch_kernel<int8_t, false, 0, 16>), kBlock, 0);
+        const hipError_t eb = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &b, reinterpret_cast<const void *>(quantize_packed_one_launch_kernel<false, 0, 4>), kBlock, 0);
+        resident[ctx->device] = (ea == hipSuccess && eb == hipSuccess && a > 0 && b > 0) ? (a < b ? a : b) : -1;
+    }
+    return resident[ctx->device] >= 4;
+}
+
 // Launches the kernel above when the call qualifies (returns true), else leaves the two-launch path to the caller.
 // The grid must be resident at once: at most four workgroups per compute unit, which the kernel's launch bound
 // makes room for; checked against the runtime's own occupancy figure the first time.
@@ -418,24 +448,11 @@ static bool launch_flat_one_launch(hipq_ctx *ctx, const float *x, size_t n, int 
     if (ctx->gemm_variant == 6 || n % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) ||
         (reinterpret_cast<uintptr_t>(out) & 3u) || (mode & ~(HIPQ_FORM_DIV | HIPQ_ROUND_HALF_EVEN)))
         return false;
-    size_t cap = size_t(ctx->num_cus) * 4;
-    if (cap > kCtxSlots) cap = kCtxSlots;
     const size_t nvec = n / 4;
-    const int vpt = nvec <= cap * kBlock * 4 ? 4 : 16;
+    const int vpt = nvec <= resident_workgroups(ctx, false) * kBlock * 4 ? 4 : 16;
     const size_t blocks = (nvec + size_t(kBlock) * vpt - 1) / (size_t(kBlock) * vpt);
-    if (blocks > cap) return false;
-    static int resident[16] = {0};  // per device: workgroups of the widest form per compute unit, 0 = not asked yet
-    if (vpt == 16 && ctx->device < 16) {
-        if (resident[ctx->device] == 0) {
-            int per_cu = 0;
-            const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                &per_cu, reinterpret_cast<const void *>(quantize_flat_one_launch_kernel<int8_t, false, 0, 16>), kBlock, 0);
-            resident[ctx->device] = (e == hipSuccess && per_cu > 0) ? per_cu : -1;
-        }
-        if (resident[ctx->device] < 4) return false;
-    } else if (vpt == 16) {
-        return false;
-    }
+    if (blocks > resident_workgroups(ctx, vpt == 16)) return false;
+    if (vpt == 16 && !four_wide_workgroups_fit(ctx)) return false;
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
 #define HIPQ_LAUNCH_Q1F(D, E, V)                                                                                       \
     hipLaunchKernelGGL((quantize_flat_one_launch_kernel<OutT, D, E, V>), dim3(static_cast<int>(blocks)), dim3(kBlock), 0, \
@@ -1195,22 +1212,30 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
     const size_t cap = size_t(ctx->num_cus) * 8;
     int grid = static_cast<int>(blocks < cap ? blocks : cap);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
-    size_t one_launch_cap = size_t(ctx->num_cus) * 4;  // half of what an idle device keeps resident
-    if (one_launch_cap > kCtxSlots) one_launch_cap = kCtxSlots;
-    if (dynamic && packed && ctx->gemm_variant != 6 && blocks <= one_launch_cap && cols % 16 == 0 &&
-        (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    const int fpw = blocks <= resident_workgroups(ctx, false) ? 1 : 4;
+    const size_t q1_blocks = (blocks + fpw - 1) / fpw;
+    if (dynamic && packed && ctx->gemm_variant != 6 && q1_blocks <= resident_workgroups(ctx, fpw == 4) && cols % 16 == 0 &&
+        (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (fpw == 1 || four_wide_workgroups_fit(ctx))) {
         // Every lane's 16 floats are all inside the matrix or all outside it, and four aligned float4.
-#define HIPQ_LAUNCH_Q1(D, E)                                                                                        \
-    hipLaunchKernelGGL((quantize_packed_one_launch_kernel<D, E>), dim3(static_cast<int>(blocks)), dim3(kBlock), 0, \
+#define HIPQ_LAUNCH_Q1(D, E, F)                                                                                           \
+    hipLaunchKernelGGL((quantize_packed_one_launch_kernel<D, E, F>), dim3(static_cast<int>(q1_blocks)), dim3(kBlock), 0, \
                        ctx->stream, x, rows, cols, out_params, ctx->wait_error, ctx->wait_spin_limit, out)
-        if (div && even)
-            HIPQ_LAUNCH_Q1(true, 1);
-        else if (div)
-            HIPQ_LAUNCH_Q1(true, 0);
-        else if (even)
-            HIPQ_LAUNCH_Q1(false, 1);
+#define HIPQ_LAUNCH_Q1_MODE(F)          \
+    do {                                \
+        if (div && even)                \
+            HIPQ_LAUNCH_Q1(true, 1, F); \
+        else if (div)                   \
+            HIPQ_LAUNCH_Q1(true, 0, F); \
+        else if (even)                  \
+            HIPQ_LAUNCH_Q1(false, 1, F); \
+        else                            \
+            HIPQ_LAUNCH_Q1(false, 0, F); \
+    } while (0)
+        if (fpw == 1)
+            HIPQ_LAUNCH_Q1_MODE(1);
         else
-            HIPQ_LAUNCH_Q1(false, 0);
+            HIPQ_LAUNCH_Q1_MODE(4);
+#undef HIPQ_LAUNCH_Q1_MODE
 #undef HIPQ_LAUNCH_Q1
         return check_launch("quantize (packed, one launch)");
     }

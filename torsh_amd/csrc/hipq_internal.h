@@ -26,6 +26,9 @@ struct hipq_ctx {
     // HIPQ_GEMM_VARIANT environment variable) and the spin limit of the persistent kernel's waits.
     int gemm_variant = -1;
     int wait_spin_limit = 1 << 20;
+    // How many contexts launch concurrently on this device (hipq_ctx_set_resident_share): kernels whose grid has to
+    // be resident at once size it for 1 / resident_share of the device.
+    int resident_share = 1;
     // Tuning aid (hipq_ctx_set_trace_buffer): caller-owned device memory for the packed GEMM's phase stamps.
     void *trace = nullptr;
     size_t trace_bytes = 0;
@@ -34,8 +37,8 @@ struct hipq_ctx {
 namespace hipq {
 
 // Layout of hipq_ctx::wait_error, in 32-bit words.  Beyond the give-up flag it holds the meeting point of the
-// one-launch dynamic quantizer (hipq_meeting.h): the number of the last meeting, the two 64-bit words {meeting,
-// scale bits}, {meeting, zero point} that end one, and per workgroup the two 64-bit words {meeting, min}, {meeting, max}.
+// one-launch dynamic quantizer (hipq_meeting.h): the number of the last meeting, the 64-bit word {tag, zero
+// point, scale bits} that ends one, and per workgroup the two 64-bit words {meeting, min}, {meeting, max}.
 constexpr size_t kCtxFlagWord = 0;
 constexpr size_t kCtxEpochWord = 16;
 constexpr size_t kCtxReadyWord = 32;
@@ -47,6 +50,17 @@ constexpr size_t kCtxWordsBytes = (kCtxRangeWord + kCtxSlots * 4) * 4;
 constexpr uint32_t kCtxFirstEpoch = 0xfffffff0u;
 // Puts the device words of a context into their initial state (device current, stream idle).
 int32_t reset_ctx_words(hipq_ctx *ctx);
+// Workgroups of 256 threads per compute unit that a kernel of this context may count on being resident together
+// with the rest of its grid, for a kernel of at most 64 (light) or at most 128 (wide) registers: a compute unit
+// holds 8 resp. 4 such workgroups, and the context's share of that is 1 / resident_share.  A light kernel takes
+// at most half of the device.
+inline size_t resident_workgroups(const hipq_ctx *ctx, bool wide) {
+    const int share = ctx->resident_share > 0 ? ctx->resident_share : 1;
+    int per_cu = (wide ? 4 : 8) / share;
+    if (!wide && per_cu > 4) per_cu = 4;
+    size_t total = size_t(ctx->num_cus) * static_cast<size_t>(per_cu);
+    return total < kCtxSlots ? total : kCtxSlots;
+}
 
 // Records `msg` (printf style) as the calling thread's last error and returns `code`.
 int32_t fail(int32_t code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));

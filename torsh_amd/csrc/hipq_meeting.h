@@ -10,8 +10,8 @@
 // can be taken for a word of a meeting 2^32 launches later.
 //
 // Every workgroup publishes {number, min} and {number, max}; workgroup 0 polls the words of all workgroups,
-// folds them, derives the parameters and publishes {number, scale} and {number, zero point}; thread 0 of every
-// other workgroup polls those two words.  That is two trips through device-coherent memory on the critical path (~1.5 us each).
+// folds them, derives the parameters and publishes them in one word (ready_word); thread 0 of every other
+// workgroup polls that word.  That is two trips through device-coherent memory on the critical path (~1.5 us each).
 // Measured alternatives: arrival counters need four trips and cross-XCD atomics on one address serialise
 // (+1.3 us); every workgroup polling every workgroup's words needs one trip, but 512 workgroups reading the
 // same 64 lines past their L2s round after round cost more than the trip saved (+1.2 us).
@@ -93,12 +93,24 @@ __device__ __forceinline__ void record_give_up(uint32_t *words) {
     __hip_atomic_store(words + kCtxFlagWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The word that ends the range part of a meeting carries the scale, the zero point and a tag in 64 bits, so that
+// one look suffices: {meeting number mod 2^22, zero point + 128 in 10 bits, scale bits}.  The short tag is enough
+// here because this word, unlike the range words, is rewritten by every meeting: it only has to differ from the
+// one before (and from the all-zero initial state, which the first numbers of a context do).
+constexpr uint32_t kReadyTagMask = 0x3fffffu;
+
 // What a meeting agrees on: the parameters workgroup 0 derives from the folded range.  scale is NaN when the
 // range is not acceptable to the flavor (not finite, ...) or a wait of the meeting was given up.
 struct MeetingParams {
     float scale;
     int zero_point;
 };
+
+__device__ __forceinline__ unsigned long long ready_word(uint32_t gen, const MeetingParams &p) {
+    return (static_cast<unsigned long long>(gen & kReadyTagMask) << 42) |
+           (static_cast<unsigned long long>(static_cast<uint32_t>(p.zero_point + 128) & 0x3ffu) << 32) |
+           __builtin_bit_cast(uint32_t, p.scale);
+}
 
 // The whole grid agrees on the quantization parameters of a tensor: `r` is this workgroup's (min, max), uniform
 // over its threads; flavor / qmin / qmax as for params_from_minmax.  Returns the same parameters in every thread of
@@ -108,7 +120,7 @@ struct MeetingParams {
 __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t gen, MinMax r, int flavor, int qmin,
                                                        int qmax, bool poison, int spin_limit, float *lds,
                                                        hipq_qparams *out_params) {
-    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);  // scale, then zp
+    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
     if (threadIdx.x == 0) {
         unsigned long long *mine = meeting_range_slot(words, blockIdx.x);
         publish_tagged(mine, gen, __builtin_bit_cast(uint32_t, r.mn));
@@ -134,6 +146,7 @@ __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t
         int zp;
         int st = params_from_minmax(t.mn, t.mx, flavor, qmin, qmax, &scale, &zp);
         if (gave_up) st = HIPQ_DEVICE_ERROR;
+        if (st == HIPQ_SUCCESS && (zp < -128 || zp > 895)) st = HIPQ_INVALID_ARGUMENT;  // not a code of an 8-bit type
         const bool bad = st != HIPQ_SUCCESS;
         p.scale = bad ? __builtin_nanf("") : scale;
         p.zero_point = bad ? 0 : zp;
@@ -147,8 +160,7 @@ __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t
             __syncthreads();
         }
         if (threadIdx.x == 0) {
-            publish_tagged(ready, gen, __builtin_bit_cast(uint32_t, p.scale));
-            publish_tagged(ready + 1, gen, static_cast<uint32_t>(p.zero_point));
+            __hip_atomic_store(ready, ready_word(gen, p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             // Every workgroup has published, so every workgroup has read the number.
             __hip_atomic_store(words + kCtxEpochWord, wrap ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (gave_up) record_give_up(words);
@@ -160,11 +172,18 @@ __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t
         }
     } else {
         if (threadIdx.x == 0) {
-            uint32_t bits = 0, zbits = 0;
-            if (poll_tagged(ready, gen, spin_limit, &bits) && poll_tagged(ready + 1, gen, spin_limit, &zbits)) {
-                lds[kMeetingLdsFloats - 2] = __builtin_bit_cast(float, bits);
-                lds[kMeetingLdsFloats - 1] = __builtin_bit_cast(float, zbits);
-            } else {
+            bool got = false;
+            for (int spin = 0; spin <= spin_limit; ++spin) {
+                const unsigned long long w = __hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((w >> 42) == (gen & kReadyTagMask)) {
+                    lds[kMeetingLdsFloats - 2] = __builtin_bit_cast(float, static_cast<uint32_t>(w));
+                    lds[kMeetingLdsFloats - 1] = __builtin_bit_cast(float, static_cast<int>((w >> 32) & 0x3ffu) - 128);
+                    got = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (!got) {
                 record_give_up(words);
                 lds[kMeetingLdsFloats - 2] = __builtin_nanf("");
                 lds[kMeetingLdsFloats - 1] = 0.0f;

@@ -123,6 +123,7 @@ _SIGNATURES = {
     "hipq_quantize_static_per_tensor_f32_i8": [_vp, _vp, _sz, _f32, _i32, _i32, _vp, _vp],
     "hipq_set_gemm_kernel_variant": [_vp, _i32],
     "hipq_ctx_set_wait_spin_limit": [_vp, _i32],
+    "hipq_ctx_set_resident_share": [_vp, _i32],
     "hipq_ctx_set_trace_buffer": [_vp, _vp, _sz],
     "hipq_linear_static_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
@@ -243,6 +244,11 @@ class Context:
             self.call("hipq_ctx_set_trace_buffer", None, 0)
         else:
             self.call("hipq_ctx_set_trace_buffer", _ptr(buf), buf.numel() * buf.element_size())
+
+    def set_resident_share(self, contexts: int) -> None:
+        """How many contexts launch concurrently on this device: the one-launch dynamic quantizers, whose grid has
+        to be resident at once, then size it for 1 / contexts of the device."""
+        self.call("hipq_ctx_set_resident_share", int(contexts))
 
     def set_wait_spin_limit(self, limit: int) -> None:
         """Test hook: polls a bounded wait (persistent GEMM, one-launch dynamic quantizer) makes before it gives
