@@ -216,6 +216,39 @@ def test_config1_full_size_properties(ctx, hipq):
     assert torch.equal(q, ref)
 
 
+def test_minmax_one_launch_and_its_bounded_wait(hipq):
+    """hipq_minmax_f32 is one launch: every workgroup publishes its partial as tagged words of the context and
+    workgroup 0 collects them.  Over a fresh context's first 40 calls (across the wrap of the meeting number,
+    grids of different sizes) it equals the two-launch form (variant 6) and torch; with the spin limit forced to 0
+    workgroup 0 looks once, too early for some of 512 partials: the outputs must then be NaN (never a range made of
+    some of the partials) and the context reports HIPQ_DEVICE_ERROR once."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(31)
+        sizes = [1 << 22, 7, 4096, 1 << 24, 100003, 1 << 12]
+        for it in range(40):
+            x = torch.randn(sizes[it % len(sizes)], generator=g, device="cuda") * (it + 1)
+            got = c.minmax(x)
+            c.set_gemm_kernel_variant(6)
+            want = c.minmax(x)
+            c.set_gemm_kernel_variant(0)
+            c.synchronize()
+            assert torch.equal(got, want) and got[0].item() == x.min().item() and got[1].item() == x.max().item(), it
+        x = torch.randn(1 << 24, generator=g, device="cuda")
+        c.set_wait_spin_limit(0)
+        got = c.minmax(x)
+        with pytest.raises(hipq.HipqError) as e:
+            c.synchronize()
+        assert e.value.code == hipq.DEVICE_ERROR
+        assert bool(torch.isnan(got).all())
+        c.set_wait_spin_limit(-1)
+        got = c.minmax(x)
+        c.synchronize()
+        assert got[0].item() == x.min().item() and got[1].item() == x.max().item()
+    finally:
+        c.close()
+
+
 @pytest.mark.parametrize("n", [150, 152, 5 * (1 << 20)])
 def test_non_finite_range_sets_status_and_skips(ctx, hipq, n):
     """150 elements take the two-launch path (not a multiple of 4), 152 the one-launch path with 4 float4 per

@@ -117,31 +117,61 @@ __device__ __forceinline__ unsigned long long ready_word(uint32_t gen, const Mee
 // every workgroup.  Workgroup 0 also writes them to out_params, with the status; for a bad range it records a
 // NaN scale if `poison` is set (the fused Linear forwards, whose GEMM must then produce NaN) and the neutral 1.0 of
 // the two-launch path otherwise.  `lds`: kMeetingLdsFloats floats.
-__device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t gen, MinMax r, int flavor, int qmin,
-                                                       int qmax, bool poison, int spin_limit, float *lds,
-                                                       hipq_qparams *out_params) {
-    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
+__device__ __forceinline__ void meeting_publish_range(uint32_t *words, uint32_t gen, MinMax r) {
     if (threadIdx.x == 0) {
         unsigned long long *mine = meeting_range_slot(words, blockIdx.x);
         publish_tagged(mine, gen, __builtin_bit_cast(uint32_t, r.mn));
         publish_tagged(mine + 1, gen, __builtin_bit_cast(uint32_t, r.mx));
     }
+}
+
+// Workgroup 0, all threads: waits for the range words of every workgroup of the grid and folds them; the result
+// is valid in every thread.  Returns true if a wait was given up.
+__device__ __forceinline__ bool meeting_collect_range(uint32_t *words, uint32_t gen, int spin_limit, float *lds,
+                                                      MinMax *folded) {
+    MinMax t{INFINITY, -INFINITY};
+    bool all = true;
+    for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) {
+        uint32_t lo = 0, hi = 0;
+        const unsigned long long *slot = meeting_range_slot(words, i);
+        const bool got = poll_tagged(slot, gen, spin_limit, &lo) && poll_tagged(slot + 1, gen, spin_limit, &hi);
+        if (got) {
+            t.mn = fminf(t.mn, __builtin_bit_cast(float, lo));
+            t.mx = fmaxf(t.mx, __builtin_bit_cast(float, hi));
+        }
+        all &= got;
+    }
+    const bool gave_up = __syncthreads_or(!all) != 0;
+    *folded = block_minmax(t, lds);
+    return gave_up;
+}
+
+// Workgroup 0, all threads, after meeting_collect_range: every workgroup has published, so every workgroup has
+// read the number, and nobody writes or reads a range word any more (or the meeting is lost anyway): advances the
+// number, and at its wrap wipes the range words first.
+__device__ __forceinline__ void meeting_close(uint32_t *words, uint32_t gen, bool gave_up) {
+    const bool wrap = gen == 0xffffffffu;
+    if (wrap) {
+        unsigned long long *first = meeting_range_slot(words, 0);
+        for (unsigned i = threadIdx.x; i < 2 * kCtxSlots; i += kBlock)
+            __hip_atomic_store(first + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(words + kCtxEpochWord, wrap ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (gave_up) record_give_up(words);
+    }
+}
+
+__device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t gen, MinMax r, int flavor, int qmin,
+                                                       int qmax, bool poison, int spin_limit, float *lds,
+                                                       hipq_qparams *out_params) {
+    unsigned long long *ready = reinterpret_cast<unsigned long long *>(words + kCtxReadyWord);
+    meeting_publish_range(words, gen, r);
     MeetingParams p;
     if (blockIdx.x == 0) {
-        MinMax t{INFINITY, -INFINITY};
-        bool all = true;
-        for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) {
-            uint32_t lo = 0, hi = 0;
-            const unsigned long long *slot = meeting_range_slot(words, i);
-            const bool got = poll_tagged(slot, gen, spin_limit, &lo) && poll_tagged(slot + 1, gen, spin_limit, &hi);
-            if (got) {
-                t.mn = fminf(t.mn, __builtin_bit_cast(float, lo));
-                t.mx = fmaxf(t.mx, __builtin_bit_cast(float, hi));
-            }
-            all &= got;
-        }
-        const bool gave_up = __syncthreads_or(!all) != 0;
-        t = block_minmax(t, lds);
+        MinMax t;
+        const bool gave_up = meeting_collect_range(words, gen, spin_limit, lds, &t);
         float scale;
         int zp;
         int st = params_from_minmax(t.mn, t.mx, flavor, qmin, qmax, &scale, &zp);
@@ -150,20 +180,9 @@ __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t
         const bool bad = st != HIPQ_SUCCESS;
         p.scale = bad ? __builtin_nanf("") : scale;
         p.zero_point = bad ? 0 : zp;
-        const bool wrap = gen == 0xffffffffu;
-        if (wrap) {
-            // Every workgroup has published (or the meeting is lost anyway): nobody writes or reads a range
-            // word any more.
-            unsigned long long *first = meeting_range_slot(words, 0);
-            for (unsigned i = threadIdx.x; i < 2 * kCtxSlots; i += kBlock)
-                __hip_atomic_store(first + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-        }
+        meeting_close(words, gen, gave_up);
         if (threadIdx.x == 0) {
             __hip_atomic_store(ready, ready_word(gen, p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            // Every workgroup has published, so every workgroup has read the number.
-            __hip_atomic_store(words + kCtxEpochWord, wrap ? 0u : gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (gave_up) record_give_up(words);
             out_params->scale = (bad && !poison) ? scale : p.scale;
             out_params->zero_point = bad ? zp : p.zero_point;
             out_params->min_val = t.mn;
