@@ -674,8 +674,16 @@ def main() -> int:
                 ct[0] += 1
                 ctx.linear_packed_i8_f32(pa3, sa3, pw3[ct[0] % len(pw3)], sw3, None, m3, n3, k3, out=o3)
 
+            x3 = torch.randn(m3, k3, generator=g, device="cuda")
+
+            def run_gemv_forward():
+                # configs[2] as specified: fp32 activations in, per-token dynamic int8 quantize, then the product
+                ct[0] += 1
+                ctx.linear_dynamic_packed(x3, pw3[ct[0] % len(pw3)], sw3, None, per_token=True, out=o3)
+
             nbytes = n3 * k3 + m3 * k3 + 4 * m3 * n3 + 4 * n3
             for name, fn in ((f"gemv_m{m3}_n11008_k4096", run_gemv_prepared),
+                             (f"gemv_m{m3}_n11008_k4096_forward_from_f32", run_gemv_forward),
                              (f"gemv_m{m3}_n11008_k4096_row_major_weights", run_gemv)):
                 ms = event_time_ms(fn, reps=100, warmup=10)
                 extra[name] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9,
@@ -695,8 +703,23 @@ def main() -> int:
             cc[0] += 1
             ctx.conv2d_i8_packed(xc[cc[0] % len(xc)], 0, 0.02, packed, sums, (3, 3), swc, bc, 0.05, 0, (1, 1), out=oc)
 
-        ms = event_time_ms(run_conv, reps=100, warmup=10)
+        xcf = [torch.relu(torch.randn(32, 256, 14, 14, generator=g, device="cuda")) for _ in range(8)]
+        conv_params = ctx.new_qparams()
+
+        def run_conv_forward():
+            # configs[3] as specified: fp32 activations in, dynamic per-tensor asymmetric uint8 quantize on the device
+            # (fused into the image-layout pass), convolution, fused bias + requantize to int8
+            cc[0] += 1
+            ctx.conv2d_dynamic_packed(xcf[cc[0] % len(xcf)], packed, sums, (3, 3), swc, bc, 0.05, 0, (1, 1),
+                                      quant_mode=hipq.FORM_DIV, out=oc, params=conv_params)
+
         conv_ops = 2.0 * 6272 * 256 * 2304
+        ms = event_time_ms(run_conv_forward, reps=100, warmup=10)
+        extra["conv2d_32x256x14x14_k3_forward_from_f32"] = {
+            "us": ms * 1e3, "TOP/s": conv_ops / (ms * 1e-3) / 1e12,
+            "frac_mfma_peak": conv_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, "ops": conv_ops,
+            "note": "dynamic uint8 quantize fused into the layout pass + implicit GEMM + fused requant"}
+        ms = event_time_ms(run_conv, reps=100, warmup=10)
         extra["conv2d_32x256x14x14_k3"] = {"us": ms * 1e3, "TOP/s": conv_ops / (ms * 1e-3) / 1e12,
                                            "frac_mfma_peak": conv_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
                                            "ops": conv_ops, "note": "layout pass + implicit GEMM + fused requant"}

@@ -469,6 +469,21 @@ HIPQ_API int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int
                                             const float *bias, size_t nb, size_t c, size_t h, size_t wd, size_t oc,
                                             size_t kh, size_t kw, size_t pad_h, size_t pad_w, float out_scale,
                                             int32_t out_zero_point, int32_t mode, int8_t *out);
+/* The whole quantized Conv2d forward from fp32 activations, on the device: x [nb, c, h, w] fp32 is quantized per
+ * tensor to uint8 with parameters from its own range (`flavor`, e.g. HIPQ_PARAMS_BACKEND_ASYMMETRIC as
+ * QuantizationParams::from_statistics derives them, crates/torsh-backend/src/quantization/params.rs; quant_mode:
+ * HIPQ_FORM_DIV / HIPQ_ROUND_HALF_EVEN bits of that quantize) and convolved as by hipq_conv2d_u8i8_i8_packed -
+ * the codes, the parameters and the outputs are those of hipq_quantize_dynamic_per_tensor_f32 followed by
+ * hipq_conv2d_u8i8_i8_packed, without the uint8 copy of the input and without reading the parameters back to the
+ * host.  in_params (device) receives the input parameters; a range that is not finite leaves status
+ * HIPQ_INVALID_ARGUMENT and a NaN scale there and outputs that carry no information.  Inputs whose image-layout
+ * pass fits the device at once (the usual case) are quantized inside that pass, in one launch. */
+HIPQ_API int32_t hipq_conv2d_dynamic_f32_i8_packed(hipq_ctx *ctx, const float *x, int32_t flavor, int32_t quant_mode,
+                                                   const int8_t *w_packed, const int32_t *w_sums,
+                                                   const float *w_scales, const float *bias, size_t nb, size_t c,
+                                                   size_t h, size_t wd, size_t oc, size_t kh, size_t kw, size_t pad_h,
+                                                   size_t pad_w, float out_scale, int32_t out_zero_point, int32_t mode,
+                                                   int8_t *out, hipq_qparams *in_params);
 
 /* ---- fp32 helpers of the int8 transformer stack ------------------------- */
 /* LayerNorm over the last dimension (biased variance, eps inside the square

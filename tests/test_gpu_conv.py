@@ -159,3 +159,48 @@ def test_conv_error_cases(ctx, hipq):
         ctx.conv2d_i8(x, 0, -1.0, w, sw, None, 1.0, 0)
     with pytest.raises(hipq.HipqError):
         ctx.conv2d_i8(x, 300, 1.0, w, sw, None, 1.0, 0)
+
+
+@pytest.mark.parametrize("nb,c,h,w,oc,k,pad", [
+    (2, 32, 5, 5, 16, (3, 3), (1, 1)), (1, 64, 7, 9, 40, (3, 2), (1, 0)), (3, 96, 12, 10, 33, (1, 1), (0, 0)),
+    (32, 256, 14, 14, 256, (3, 3), (1, 1)),   # configs[3] at full size, as specified: fp32 in, int8 out
+    (64, 128, 30, 30, 32, (3, 3), (1, 1)),    # image pass too large to be resident at once: quantized in a pass of its own
+])
+def test_conv2d_forward_from_fp32_equals_quantize_then_conv(ctx, hipq, nb, c, h, w, oc, k, pad):
+    """hipq_conv2d_dynamic_f32_i8_packed (dynamic per-tensor uint8 quantize of the fp32 input fused into the image
+    pass, parameters kept on the device) must give the parameters and the output bytes of
+    hipq_quantize_dynamic_per_tensor_f32 followed by hipq_conv2d_u8i8_i8_packed with those parameters passed by
+    value - the composition the oracle tests above pin - for both quantize forms and roundings."""
+    g = torch.Generator(device="cuda").manual_seed(nb * 131 + c + h)
+    x = torch.relu(torch.randn(nb, c, h, w, generator=g, device="cuda")) * 1.7
+    wq = torch.randint(-128, 128, (oc, c) + k, generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(oc, generator=g, device="cuda") * 1e-3 + 1e-4
+    bias = torch.randn(oc, generator=g, device="cuda") * 0.05
+    packed, sums = ctx.conv2d_pack_weights(wq)
+    for qmode in (0, hipq.FORM_DIV, hipq.ROUND_HALF_EVEN | hipq.FORM_DIV):
+        q, params = ctx.quantize_dynamic_per_tensor(x, hipq.PARAMS_BACKEND_ASYMMETRIC, hipq.DTYPE_U8, qmode)
+        p = ctx.read_qparams(params)
+        want = ctx.conv2d_i8_packed(q, p.zero_point, p.scale, packed, sums, k, sw, bias, 0.05, 3, pad,
+                                    mode=hipq.ROUND_HALF_EVEN)
+        got, gparams = ctx.conv2d_dynamic_packed(x, packed, sums, k, sw, bias, 0.05, 3, pad, quant_mode=qmode,
+                                                 mode=hipq.ROUND_HALF_EVEN)
+        torch.cuda.synchronize()
+        gp = ctx.read_qparams(gparams)
+        assert (gp.scale, gp.zero_point, gp.min_val, gp.max_val, gp.status) == (p.scale, p.zero_point, p.min_val,
+                                                                                p.max_val, p.status)
+        assert torch.equal(got, want), qmode
+
+
+def test_conv2d_forward_from_fp32_reports_a_bad_range(ctx, hipq):
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x = torch.randn(2, 32, 6, 6, generator=g, device="cuda")
+    x[1, 3, 2, 2] = float("inf")
+    wq = torch.randint(-128, 128, (8, 32, 3, 3), generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(8, generator=g, device="cuda") * 1e-3 + 1e-4
+    packed, sums = ctx.conv2d_pack_weights(wq)
+    out, params = ctx.conv2d_dynamic_packed(x, packed, sums, (3, 3), sw, None, 0.05, 0, (1, 1))
+    torch.cuda.synchronize()
+    p = ctx.read_qparams(params)
+    assert p.status == hipq.INVALID_ARGUMENT and p.scale != p.scale
+    with pytest.raises(hipq.HipqError):
+        ctx.conv2d_dynamic_packed(x[:, :31].contiguous(), packed, sums, (3, 3), sw, None, 0.05, 0, (1, 1))

@@ -14,6 +14,7 @@
 // and a border pixel holds exactly zp so padded taps contribute nothing.
 // Everything else runs through a direct per-output kernel (correct, not fast).
 #include "hipq_gemm_kernels.h"
+#include "hipq_meeting.h"
 
 namespace hipq {
 
@@ -27,9 +28,11 @@ constexpr int kConvThreads = 256;
 // 2 KiB contiguous).  x - 128 on a byte is a flip of its top bit.  No LDS.  The last cbs workgroups clear
 // the slack.  C % 32 == 0.
 __global__ __launch_bounds__(kConvThreads) void conv_pack_image_kernel(const uint8_t *__restrict__ x, int C, int H, int W,
-                                                                         int pad_h, int pad_w, int zp, int nb,
+                                                                         int pad_h, int pad_w, int zp,
+                                                                         const int32_t *__restrict__ zp_dev, int nb,
                                                                          int groups_per_cb, int8_t *__restrict__ out,
                                                                          int pixels) {
+    if (zp_dev) zp = *zp_dev;  // the zero point a dynamic quantize has left on the device
     const int hp = H + 2 * pad_h, wp = W + 2 * pad_w, cbs = C / 32;
     const int real_pixels = nb * hp * wp;
     const int work = cbs * groups_per_cb;
@@ -57,6 +60,79 @@ __global__ __launch_bounds__(kConvThreads) void conv_pack_image_kernel(const uin
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             d[i] = (b[4 * i] | (b[4 * i + 1] << 8) | (b[4 * i + 2] << 16) | (b[4 * i + 3] << 24)) ^ 0x80808080u;
+    }
+    uint4 *dst = reinterpret_cast<uint4 *>(out + (size_t(cb) * pixels + p) * 32);
+    dst[0] = make_uint4(d[0], d[1], d[2], d[3]);
+    dst[1] = make_uint4(d[4], d[5], d[6], d[7]);
+}
+
+// The same image from fp32 activations, quantized on the way: per-tensor uint8 with parameters from the
+// tensor's own range (flavor; codes 0..255).  A thread keeps the 32 channel values of its pixel in registers
+// while the grid agrees on the range (hipq_meeting.h), quantizes them, and writes the 32 bytes; the border holds
+// zp - 128 with the zero point just agreed on.  The input is read once and no uint8 copy of it is ever written.
+// Workgroup 0 publishes the parameters in out_params for the convolution kernel that follows.  The caller
+// guarantees that the grid can be resident at once.
+template <bool DIV, int RND>
+__global__ __launch_bounds__(kConvThreads, 4) void conv_quantize_pack_image_kernel(
+    const float *__restrict__ x, int C, int H, int W, int pad_h, int pad_w, int flavor, int nb, int groups_per_cb,
+    hipq_qparams *out_params, uint32_t *words, int spin_limit, int8_t *__restrict__ out, int pixels) {
+    __shared__ float lds[kMeetingLdsFloats];
+    const int hp = H + 2 * pad_h, wp = W + 2 * pad_w, cbs = C / 32;
+    const int real_pixels = nb * hp * wp;
+    const int work = cbs * groups_per_cb;
+    const bool slack = static_cast<int>(blockIdx.x) >= work;
+    const int cb = slack ? blockIdx.x - work : blockIdx.x / groups_per_cb;
+    const int p = (blockIdx.x % groups_per_cb) * kConvThreads + threadIdx.x;  // padded pixel of the whole batch
+    bool inside = false;
+    float v[32];
+    if (!slack && p < real_pixels) {
+        const int n = p / (hp * wp), rem = p % (hp * wp);
+        const int h = rem / wp - pad_h, w = rem % wp - pad_w;
+        if (h >= 0 && h < H && w >= 0 && w < W) {
+            inside = true;
+            const size_t plane = size_t(H) * W;
+            const float *src = x + ((size_t(n) * C + cb * 32) * H + h) * W + w;
+#pragma unroll
+            for (int c = 0; c < 32; ++c) v[c] = src[size_t(c) * plane];
+        }
+    }
+    const uint32_t gen = meeting_number(words);  // behind the data in program order: returned after it
+    MinMax m{INFINITY, -INFINITY};
+    if (inside) {
+#pragma unroll
+        for (int c = 0; c < 32; ++c) {
+            m.mn = fminf(m.mn, v[c]);
+            m.mx = fmaxf(m.mx, v[c]);
+        }
+    }
+    const MinMax r = block_minmax(m, lds);
+    if (slack) {
+        // These workgroups only clear the slack behind the image: they take part in the meeting with a range
+        // that changes nothing and do not wait for its result.
+        meeting_publish_range(words, gen, r);
+        uint4 *tail = reinterpret_cast<uint4 *>(out + (size_t(cb) * pixels + real_pixels) * 32);
+        for (int i = threadIdx.x; i < (pixels - real_pixels) * 2; i += kConvThreads) tail[i] = make_uint4(0, 0, 0, 0);
+        return;
+    }
+    const MeetingParams agreed = meet_on_range(words, gen, r, flavor, 0, 255, /*poison=*/true, spin_limit, lds, out_params);
+    if (p >= real_pixels) return;
+    const bool bad = agreed.scale != agreed.scale;
+    const float scale = bad ? INFINITY : agreed.scale;  // x / inf: every code is the zero point
+    const int zp = agreed.zero_point;
+    const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
+    const float zpf = static_cast<float>(zp);
+    const uint32_t border4 = static_cast<uint32_t>(static_cast<uint8_t>(zp - 128)) * 0x01010101u;
+    uint32_t d[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d[i] = border4;
+    if (inside) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            d[i] = pack4(quantize_int<DIV, RND>(v[4 * i], scale, inv, zpf, 0, 255),
+                         quantize_int<DIV, RND>(v[4 * i + 1], scale, inv, zpf, 0, 255),
+                         quantize_int<DIV, RND>(v[4 * i + 2], scale, inv, zpf, 0, 255),
+                         quantize_int<DIV, RND>(v[4 * i + 3], scale, inv, zpf, 0, 255)) ^
+                   0x80808080u;
     }
     uint4 *dst = reinterpret_cast<uint4 *>(out + (size_t(cb) * pixels + p) * 32);
     dst[0] = make_uint4(d[0], d[1], d[2], d[3]);
@@ -175,11 +251,21 @@ static int32_t pack_filters(hipq_ctx *ctx, const int8_t *w, int oc, int ic, int 
     return pack_rows(ctx, staging, size_t(oc), size_t(ic) * taps, packed);
 }
 
+// Dynamic input of a convolution: fp32 activations to be quantized to uint8 on the device (flavor, quantize mode
+// bits), and where the parameters go.  x null: the input is already uint8.
+struct ConvDynamicInput {
+    const float *x = nullptr;
+    int flavor = 0, quant_mode = 0;
+    hipq_qparams *params = nullptr;
+};
+
 template <int EPI, bool EVEN>
 static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int zp_in, float s_in, const int8_t *w,
                             const int8_t *wpacked, const int32_t *wsum, const float *sw, const float *bias,
-                            const ConvGeom &g, float s_out, int zp_out, void *out) {
+                            const ConvGeom &g, float s_out, int zp_out, void *out,
+                            const ConvDynamicInput &dyn = ConvDynamicInput{}) {
     if (!fast_path_ok(g)) {
+        if (dyn.x) return fail(HIPQ_INVALID_ARGUMENT, "%s: needs stride 1 and channels a multiple of 32", fn);
         if (!w) return fail(HIPQ_INVALID_ARGUMENT, "%s: this geometry needs the unpacked filters", fn);
         const size_t total = size_t(g.nb) * g.oc * g.ho * g.wo;
         size_t blocks = (total + kConvThreads - 1) / kConvThreads;
@@ -195,13 +281,47 @@ static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int
     const size_t k = size_t(g.c) * taps;
     const size_t w_bytes = wpacked ? 0 : align256(size_t(g.oc) * k) + align256(packed_operand_bytes(g.oc, k)) +
                                              align256(size_t(g.oc) * 4);
+    const int groups_per_cb = (g.nb * hp * wp + kConvThreads - 1) / kConvThreads;
+    const size_t pack_grid = size_t(cbs) * groups_per_cb + cbs;
+    // Dynamic input: in one launch with the image pack when its grid can be resident at once (the kernel holds 32
+    // floats a lane: four workgroups per compute unit), else quantized to a uint8 copy first.
+    const bool fused_input = dyn.x && ctx->gemm_variant != 6 && pack_grid <= resident_workgroups(ctx, true);
+    const size_t u8_bytes = (dyn.x && !fused_input) ? align256(size_t(g.nb) * g.c * g.h * g.w) : 0;
     void *s = nullptr;
-    int32_t rc = scratch(ctx, kScratchHeader + align256(img_bytes) + w_bytes, &s);
+    int32_t rc = scratch(ctx, kScratchHeader + align256(img_bytes) + w_bytes + u8_bytes, &s);
     if (rc) return rc;
     int8_t *ximg = reinterpret_cast<int8_t *>(static_cast<char *>(s) + kScratchHeader);
-    const int groups_per_cb = (g.nb * hp * wp + kConvThreads - 1) / kConvThreads;
-    hipLaunchKernelGGL(conv_pack_image_kernel, dim3(cbs * groups_per_cb + cbs), dim3(kConvThreads), 0, ctx->stream, x, g.c,
-                       g.h, g.w, g.ph, g.pw, zp_in, g.nb, groups_per_cb, ximg, static_cast<int>(pixels));
+    if (fused_input) {
+        const bool qdiv = (dyn.quant_mode & HIPQ_FORM_DIV) != 0, qeven = (dyn.quant_mode & HIPQ_ROUND_HALF_EVEN) != 0;
+#define HIPQ_LAUNCH_CQ(D, E)                                                                                          \
+    hipLaunchKernelGGL((conv_quantize_pack_image_kernel<D, E>), dim3(static_cast<int>(pack_grid)), dim3(kConvThreads), 0, \
+                       ctx->stream, dyn.x, g.c, g.h, g.w, g.ph, g.pw, dyn.flavor, g.nb, groups_per_cb, dyn.params,    \
+                       ctx->wait_error, ctx->wait_spin_limit, ximg, static_cast<int>(pixels))
+        if (qdiv && qeven)
+            HIPQ_LAUNCH_CQ(true, 1);
+        else if (qdiv)
+            HIPQ_LAUNCH_CQ(true, 0);
+        else if (qeven)
+            HIPQ_LAUNCH_CQ(false, 1);
+        else
+            HIPQ_LAUNCH_CQ(false, 0);
+#undef HIPQ_LAUNCH_CQ
+    } else {
+        if (dyn.x) {
+            uint8_t *xq = reinterpret_cast<uint8_t *>(ximg + align256(img_bytes) + w_bytes);
+            rc = quantize_dynamic_per_tensor(ctx, dyn.x, size_t(g.nb) * g.c * g.h * g.w, dyn.flavor, HIPQ_DTYPE_U8,
+                                             dyn.quant_mode, xq, dyn.params, nullptr, 0);
+            if (rc) return rc;
+            // the call above may have grown (moved) the scratch
+            if ((rc = scratch(ctx, kScratchHeader + align256(img_bytes) + w_bytes + u8_bytes, &s))) return rc;
+            if (static_cast<char *>(s) + kScratchHeader != reinterpret_cast<char *>(ximg))
+                return fail(HIPQ_DEVICE_ERROR, "%s: scratch moved under a pending kernel", fn);
+            x = xq;
+        }
+        hipLaunchKernelGGL(conv_pack_image_kernel, dim3(static_cast<int>(pack_grid)), dim3(kConvThreads), 0, ctx->stream,
+                           x, g.c, g.h, g.w, g.ph, g.pw, zp_in, dyn.x ? &dyn.params->zero_point : nullptr, g.nb,
+                           groups_per_cb, ximg, static_cast<int>(pixels));
+    }
     if ((rc = check_launch(fn))) return rc;
     if (!wpacked) {
         int8_t *staging = ximg + align256(img_bytes);
@@ -224,6 +344,10 @@ static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int
     ep.cv_nb = g.nb;
     ep.cv_wsum = wsum;
     ep.cv_corr_mul = 128 - zp_in;
+    if (dyn.x) {
+        ep.sa = &dyn.params->scale;  // NaN for a range that is not finite: the outputs then carry no information
+        ep.cv_zp_in = &dyn.params->zero_point;
+    }
     ep.cv_pixels = static_cast<int>(pixels);
     ep.cv_kblocks = taps * cbs;
     ep.fresh_activations = 1;  // the image was written by the kernel just before
@@ -358,6 +482,42 @@ int32_t hipq_conv2d_u8i8_i8_packed(hipq_ctx *ctx, const uint8_t *x, int32_t zp_i
     }
     return conv_i8_common(__func__, ctx, x, zp_in, s_in, nullptr, w_packed, w_sums, w_scales, bias, g, out_scale,
                           out_zero_point, mode, out);
+}
+
+int32_t hipq_conv2d_dynamic_f32_i8_packed(hipq_ctx *ctx, const float *x, int32_t flavor, int32_t quant_mode,
+                                          const int8_t *w_packed, const int32_t *w_sums, const float *w_scales,
+                                          const float *bias, size_t nb, size_t c, size_t h, size_t wd, size_t oc,
+                                          size_t kh, size_t kw, size_t pad_h, size_t pad_w, float out_scale,
+                                          int32_t out_zero_point, int32_t mode, int8_t *out, hipq_qparams *in_params) {
+    HIPQ_ENTER(ctx);
+    ConvGeom g;
+    int32_t rc = make_geom(__func__, nb, c, h, wd, oc, kh, kw, 1, 1, pad_h, pad_w, &g);
+    if (rc) return rc;
+    if (!fast_path_ok(g))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: packed filters need stride 1 and channels a multiple of 32", __func__);
+    if (flavor < HIPQ_PARAMS_SYMMETRIC || flavor > HIPQ_PARAMS_NN_ASYMMETRIC)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown flavor %d", __func__, flavor);
+    if (quant_mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV))
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown quantize mode bits", __func__);
+    if (mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV)) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", __func__);
+    if (out_scale <= 0.0f) return fail(HIPQ_INVALID_ARGUMENT, "%s: Scale must be positive", __func__);
+    if (nb == 0 || oc == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(x);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_sums);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    HIPQ_REQUIRE_PTR(in_params);
+    ConvDynamicInput dyn;
+    dyn.x = x;
+    dyn.flavor = flavor;
+    dyn.quant_mode = quant_mode;
+    dyn.params = in_params;
+    if (mode & HIPQ_ROUND_HALF_EVEN)
+        return conv_forward<EPI_I8, true>(__func__, ctx, nullptr, 0, 1.0f, nullptr, w_packed, w_sums, w_scales, bias, g,
+                                          out_scale, out_zero_point, out, dyn);
+    return conv_forward<EPI_I8, false>(__func__, ctx, nullptr, 0, 1.0f, nullptr, w_packed, w_sums, w_scales, bias, g,
+                                       out_scale, out_zero_point, out, dyn);
 }
 
 }  // extern "C"

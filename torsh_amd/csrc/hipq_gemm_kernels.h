@@ -29,6 +29,7 @@ struct GemmEpilogue {
     int cv_ho = 0, cv_wo = 0, cv_oc = 0, cv_nb = 0;
     const int32_t *cv_wsum = nullptr;  // [oc] sum of the filter's int8 weights
     int cv_corr_mul = 0;               // 128 - zp_in: accumulator += cv_corr_mul * cv_wsum[oc]
+    const int32_t *cv_zp_in = nullptr; // when set: the input zero point on the device, used instead of cv_corr_mul
     int cv_pixels = 0;                 // pixels per channel block of the image buffer (with slack)
     int cv_kblocks = 0;                // taps * (c / 32): the k blocks that hold data
     float sa_scalar = 1.0f;            // activation scale used when sa is null

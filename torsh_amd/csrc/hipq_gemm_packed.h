@@ -274,7 +274,7 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
         }
         const int m = m0 + wave * 32 + lane % 32;
         const int mc = m < M ? m : M - 1;
-        cv_c = ep.cv_corr_mul * ep.cv_wsum[mc];
+        cv_c = (ep.cv_zp_in ? 128 - *ep.cv_zp_in : ep.cv_corr_mul) * ep.cv_wsum[mc];
         if constexpr (EPI != EPI_I32) {
             cv_s = sa0 * ep.sw[mc];
             if (ep.bias) cv_b = ep.bias[mc];

@@ -145,6 +145,8 @@ _SIGNATURES = {
     "hipq_conv2d_u8i8_f32": [_vp, _vp, _i32, _f32, _vp, _vp, _vp] + [_sz] * 11 + [_vp],
     "hipq_conv2d_pack_weights_i8": [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp],
     "hipq_conv2d_u8i8_i8_packed": [_vp, _vp, _i32, _f32, _vp, _vp, _vp, _vp] + [_sz] * 9 + [_f32, _i32, _i32, _vp],
+    "hipq_conv2d_dynamic_f32_i8_packed": [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp] + [_sz] * 9 +
+                                         [_f32, _i32, _i32, _vp, _vp],
 }
 
 _SPECIAL = {
@@ -678,6 +680,22 @@ class Context:
                   _ptr(w_scales), _ptr(bias), nb, c, h, wd, oc, kh, kw, padding[0], padding[1], float(s_out),
                   int(zp_out), mode, _ptr(out))
         return out
+
+    def conv2d_dynamic_packed(self, x, w_packed, w_sums, kernel, w_scales, bias, s_out, zp_out, padding=(0, 0),
+                              flavor=PARAMS_BACKEND_ASYMMETRIC, quant_mode=0, mode=0, out=None, params=None):
+        """Conv2d forward from fp32 activations: dynamic per-tensor uint8 quantize of x on the device, then the
+        convolution on prepared filters -> (int8 output, device hipq_qparams of the input)."""
+        nb, c, h, wd = x.shape
+        oc = w_sums.numel()
+        kh, kw = kernel
+        ho = h + 2 * padding[0] - kh + 1
+        wo = wd + 2 * padding[1] - kw + 1
+        out = out if out is not None else torch.empty((nb, oc, ho, wo), dtype=torch.int8, device=self._dev())
+        params = params if params is not None else self.new_qparams()
+        self.call("hipq_conv2d_dynamic_f32_i8_packed", _ptr(x), flavor, quant_mode, _ptr(w_packed), _ptr(w_sums),
+                  _ptr(w_scales), _ptr(bias), nb, c, h, wd, oc, kh, kw, padding[0], padding[1], float(s_out),
+                  int(zp_out), mode, _ptr(out), _ptr(params))
+        return out, params
 
     def quantize_per_row_strided(self, x_base, rows, cols, ld, elem_offset=0, flavor=PARAMS_SYMMETRIC, mode=0):
         out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
