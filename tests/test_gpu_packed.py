@@ -179,6 +179,40 @@ def test_linear_packed_many_tiles_matches_row_major(ctx, hipq, m, n, k):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 64, 16), (1, 11008, 4096), (4, 11008, 4096), (16, 11008, 4096), (32, 1024, 1040),
+                                   (7, 300, 11008), (3, 96, 16384), (5, 4096, 272)])
+def test_decode_forward_per_token(hipq, m, n, k):
+    """Per-token dynamic forward with M <= 32 rows (the decode shapes of configs[2] among them), from fp32
+    activations: same bits as the per-row quantizer followed by the product on its output (both pinned to the oracle
+    elsewhere), for both roundings; a row with an infinite value gives a NaN row and leaves the others."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(m * 7 + n + k)
+        wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+        pw = c.pack_rows(wq)
+        sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+        bias = torch.randn(n, generator=g, device="cuda")
+        for it in range(20):
+            x = torch.randn(m, k, generator=g, device="cuda") * (it + 1)
+            x[m // 2, k // 3] *= 30.0
+            mode = hipq.ROUND_HALF_EVEN if it % 2 else 0
+            got = c.linear_dynamic_packed(x, pw, sw, bias, per_token=True, mode=mode)
+            pq, ps = c.quantize_per_row_packed(x, mode=mode)
+            want = c.linear_packed_i8_f32(pq, ps, pw, sw, bias, m, n, k)
+            c.synchronize()
+            assert torch.equal(got, want), it
+        xb = x.clone()
+        xb[m - 1, 5] = float("inf")
+        got = c.linear_dynamic_packed(xb, pw, sw, bias, per_token=True)
+        good = c.linear_dynamic_packed(x, pw, sw, bias, per_token=True)
+        c.synchronize()
+        assert torch.isnan(got[m - 1]).all()
+        if m > 1:
+            assert torch.equal(got[: m - 1], good[: m - 1])
+    finally:
+        c.close()
+
+
 def test_linear_static_packed(ctx, hipq):
     g = torch.Generator(device="cuda").manual_seed(3)
     m, n, k = 96, 160, 512
