@@ -125,6 +125,7 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
         delete ctx;
         return rc;
     }
+    (void)hipq::four_wide_workgroups_fit(ctx);  // asked here so that no later call is the first
     *out_ctx = ctx;
     return HIPQ_SUCCESS;
 }

@@ -459,8 +459,9 @@ __global__ __launch_bounds__(kBlock, 4) void quantize_flat_one_launch_kernel(con
 }
 
 // The one-launch quantizers that hold 64 floats a lane need four workgroups per compute unit resident: what the
-// runtime says about the widest flat form (the packed one has the same launch bound), asked once per device.
-static bool four_wide_workgroups_fit(const hipq_ctx *ctx) {
+// runtime says about the widest flat form (the packed one has the same launch bound), asked once per device -
+// hipq_ctx_create does, so that no later call (one under stream capture, say) is the first to ask.
+bool four_wide_workgroups_fit(const hipq_ctx *ctx) {
     static int resident[16] = {0};  // workgroups per compute unit; 0 = not asked yet, -1 = the query failed
     if (ctx->device < 0 || ctx->device >= 16) return false;
     if (resident[ctx->device] == 0) {

@@ -90,6 +90,9 @@ int32_t quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t rows,
 // Looks up, once per device, the address of the static device array behind
 // hipq_linear_dynamic_f32_noalloc; called by hipq_ctx_create with the device current.
 int32_t linear_noalloc_setup(int device);
+// Whether four workgroups of the widest one-launch quantizers fit a compute unit of the context's device (asked of
+// the runtime once per device and remembered).
+bool four_wide_workgroups_fit(const hipq_ctx *ctx);
 
 // Bytes reserved at the head of the context scratch for small device records
 // (hipq_qparams, min/max pairs, status words); bulk scratch starts after it.
