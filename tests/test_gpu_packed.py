@@ -423,6 +423,44 @@ def test_resident_share_changes_the_path_not_the_result(hipq):
         c.close()
 
 
+def test_two_contexts_meet_side_by_side(hipq):
+    """Two contexts on two streams, each told that two contexts launch concurrently (hipq_ctx_set_resident_share),
+    run their one-launch quantizers and Linear steps at the same time for a few hundred launches: each has its own
+    meeting words, the grids of both fit the device together, and every result equals the one the same context
+    computes alone afterwards."""
+    a, b = hipq.Context(0, own_stream=True), hipq.Context(0, own_stream=True)
+    try:
+        a.set_resident_share(2)
+        b.set_resident_share(2)
+        g = torch.Generator(device="cuda").manual_seed(77)
+        m, n, k = 512, 1024, 4096
+        pw = a.pack_rows(torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8))
+        sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+        xs = [torch.randn(m, k, generator=g, device="cuda") * (i + 1) for i in range(6)]
+        big = [torch.randn(2048 * 4096, generator=g, device="cuda") * (i + 1) for i in range(2)]
+        a.synchronize()
+        torch.cuda.synchronize()  # the inputs were made on torch's stream, the contexts have their own
+        outs = {}
+        for it in range(240):
+            c = a if it % 2 == 0 else b
+            if it % 8 < 6:
+                outs[it] = c.linear_dynamic_packed(xs[it % 6], pw, sw, None)
+            else:
+                outs[it] = c.quantize_dynamic_per_tensor(big[it % 2])[0]
+        a.synchronize()
+        b.synchronize()
+        for it in range(0, 240, 7):
+            if it % 8 < 6:
+                want = a.linear_dynamic_packed(xs[it % 6], pw, sw, None)
+            else:
+                want = a.quantize_dynamic_per_tensor(big[it % 2])[0]
+            a.synchronize()
+            assert torch.equal(outs[it], want), it
+    finally:
+        a.close()
+        b.close()
+
+
 def test_one_launch_dynamic_quantize_gives_up_cleanly(hipq):
     """With the spin limit forced to 0 every workgroup looks at the other workgroups' range words exactly once,
     which with 512 workgroups is certain to come too early for some of them: the kernel must still drain, a
