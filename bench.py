@@ -591,6 +591,13 @@ def main() -> int:
             i = rot()
             ctx.quantize_dynamic_per_tensor(fx[i], out=fq[i], params=params)
 
+        def run_round_trip():
+            # configs[0] as it is specified: quantize_tensor_auto (scale from max|x|) then dequantize with the
+            # parameters it left on the device
+            i = rot()
+            ctx.quantize_dynamic_per_tensor(fx[i], out=fq[i], params=params)
+            ctx.dequantize_with_params(fq[i], params, out=fy[i])
+
         # calibration / quality kernels on the same 16 Mi-element tensors
         metrics_rec = ctx.quantization_metrics(fx[0], fy[0])
         observe_rec = ctx.observe(fx[0])
@@ -634,6 +641,7 @@ def main() -> int:
         for name, fn, bytes_per in (("hbm_copy_reference_f32", run_copy, 8),
                                     ("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
                                     ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9),
+                                    ("round_trip_dynamic_quantize_dequantize_f32", run_round_trip, 14),
                                     ("quality_metrics_two_tensors_f32", run_metrics, 8),
                                     ("fake_quantize_metrics_fused_f32", run_fused_metrics, 4),
                                     ("fake_quantize_f32", run_fake_quant, 8),
@@ -648,10 +656,11 @@ def main() -> int:
         # The dynamic quantize is priced at the two passes of the algorithm (9 B per element), but a tensor of this
         # size runs as one launch that holds it in registers between the range and the codes, so only 5 B per
         # element cross the memory interface: both rates, so that neither is mistaken for the other.
-        dq = extra["dynamic_quantize_f32_i8"]
-        dq["bytes_moved_per_elem"] = 5
-        dq["GB/s_moved"] = 5 * n / (dq["us"] * 1e-6) / 1e9
-        dq["frac_hbm_peak_moved"] = dq["GB/s_moved"] / PEAK_HBM_GBPS
+        for key, moved in (("dynamic_quantize_f32_i8", 5), ("round_trip_dynamic_quantize_dequantize_f32", 10)):
+            dq = extra[key]
+            dq["bytes_moved_per_elem"] = moved
+            dq["GB/s_moved"] = moved * n / (dq["us"] * 1e-6) / 1e9
+            dq["frac_hbm_peak_moved"] = dq["GB/s_moved"] / PEAK_HBM_GBPS
         del fx, fq, fy
 
         # configs[2]: decode-shaped skinny GEMM, weight streaming (N=11008, K=4096)
