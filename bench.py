@@ -591,6 +591,19 @@ def main() -> int:
             i = rot()
             ctx.quantize_dynamic_per_tensor(fx[i], out=fq[i], params=params)
 
+        racc = [torch.randint(-(1 << 20), 1 << 20, (4096, 4096), generator=g, device="cuda", dtype=torch.int32)
+                for _ in range(4)]
+        rsa = torch.full((1,), 0.03, device="cuda")
+        rsw = torch.rand(4096, generator=g, device="cuda") * 1e-3 + 1e-4
+        rbias = torch.randn(4096, generator=g, device="cuda") * 0.01
+        rout = torch.empty((4096, 4096), dtype=torch.int8, device="cuda")
+
+        def run_requant():
+            # the stand-alone requantize of int32 accumulators [4096, 4096]: 4 B read + 1 B written per element
+            i = rot()
+            ctx.call("hipq_requantize_i32_i8", racc[i % 4].data_ptr(), 4096, 4096, rsa.data_ptr(), 0, rsw.data_ptr(),
+                     rbias.data_ptr(), 0.05, 0, 0, rout.data_ptr())
+
         def run_round_trip():
             # configs[0] as it is specified: quantize_tensor_auto (scale from max|x|) then dequantize with the
             # parameters it left on the device
@@ -640,6 +653,7 @@ def main() -> int:
 
         for name, fn, bytes_per in (("hbm_copy_reference_f32", run_copy, 8),
                                     ("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
+                                    ("requantize_i32_i8", run_requant, 5),
                                     ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9),
                                     ("round_trip_dynamic_quantize_dequantize_f32", run_round_trip, 14),
                                     ("quality_metrics_two_tensors_f32", run_metrics, 8),
@@ -661,7 +675,7 @@ def main() -> int:
             dq["bytes_moved_per_elem"] = moved
             dq["GB/s_moved"] = moved * n / (dq["us"] * 1e-6) / 1e9
             dq["frac_hbm_peak_moved"] = dq["GB/s_moved"] / PEAK_HBM_GBPS
-        del fx, fq, fy
+        del fx, fq, fy, racc
 
         # configs[2]: decode-shaped skinny GEMM, weight streaming (N=11008, K=4096)
         n3, k3 = 11008, 4096
