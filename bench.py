@@ -604,6 +604,25 @@ def main() -> int:
             ctx.call("hipq_requantize_i32_i8", racc[i % 4].data_ptr(), 4096, 4096, rsa.data_ptr(), 0, rsw.data_ptr(),
                      rbias.data_ptr(), 0.05, 0, 0, rout.data_ptr())
 
+        pc_scales = torch.rand(4096, generator=g, device="cuda") * 0.05 + 0.01
+        pc_zps = torch.zeros(4096, dtype=torch.int32, device="cuda")
+
+        def run_pc_quant():
+            # per-channel quantize with given parameters, channels = the 4096 rows of a [4096, 4096] weight
+            i = rot()
+            ctx.call("hipq_quantize_per_channel_f32_i8", fx[i].data_ptr(), 1, 4096, 4096, pc_scales.data_ptr(),
+                     pc_zps.data_ptr(), hipq.FORM_DIV, fq[i].data_ptr())
+
+        def run_pc_dequant():
+            i = rot()
+            ctx.call("hipq_dequantize_per_channel_i8_f32", fq[i].data_ptr(), 1, 4096, 4096, pc_scales.data_ptr(),
+                     pc_zps.data_ptr(), fy[i].data_ptr())
+
+        def run_pc_auto():
+            # quantize_per_channel_auto over axis 0: each row's range, scale and codes in one pass
+            i = rot()
+            ctx.quantize_per_row(fx[i].view(4096, 4096))
+
         def run_round_trip():
             # configs[0] as it is specified: quantize_tensor_auto (scale from max|x|) then dequantize with the
             # parameters it left on the device
@@ -654,6 +673,9 @@ def main() -> int:
         for name, fn, bytes_per in (("hbm_copy_reference_f32", run_copy, 8),
                                     ("quantize_f32_i8", run_quant, 5), ("dequantize_i8_f32", run_dequant, 5),
                                     ("requantize_i32_i8", run_requant, 5),
+                                    ("quantize_per_channel_f32_i8", run_pc_quant, 5),
+                                    ("dequantize_per_channel_i8_f32", run_pc_dequant, 5),
+                                    ("quantize_per_channel_auto_f32_i8", run_pc_auto, 5),
                                     ("minmax_f32", run_minmax, 4), ("dynamic_quantize_f32_i8", run_dynamic, 9),
                                     ("round_trip_dynamic_quantize_dequantize_f32", run_round_trip, 14),
                                     ("quality_metrics_two_tensors_f32", run_metrics, 8),

@@ -331,6 +331,39 @@ def test_per_channel_any_axis(ctx, hipq, oracle, axis):
         np.testing.assert_array_equal(got, want.astype(np.int8))
 
 
+@pytest.mark.parametrize("shape,axis", [((3, 8, 12), 0), ((3, 8, 12), 1), ((7, 5, 2048), 1), ((6, 1000), 0),
+                                        ((300, 64, 36), 1), ((1, 1, 4), 2), ((257, 4100), 0), ((16, 4096), 1)])
+def test_per_channel_vector_forms(ctx, hipq, oracle, shape, axis):
+    """Explicit-parameter per-channel quantize / dequantize where the run of one channel is a multiple of four
+    elements (the kernels then work on vectors of four): power-of-two and other run lengths and channel counts,
+    whole tiles and ragged tails, both rounding forms; and the same data one element off alignment, which takes
+    the element-wise kernels and must give the same bytes."""
+    x = normal(77 + axis, shape) * 3
+    ch = shape[axis]
+    rng = np.random.default_rng(9)
+    scales = rng.uniform(0.01, 0.05, ch).astype(np.float32)
+    zps = rng.integers(-7, 8, ch).astype(np.int32)
+    want = oracle.quantize_per_channel_affine(x, scales, zps, axis).astype(np.int8)
+    got = ctx.quantize_per_channel(dev(x), dev(scales), dev(zps), axis, hipq.FORM_DIV)
+    np.testing.assert_array_equal(host(got), want)
+    want_y = oracle.dequantize_per_channel_affine(want.astype(np.float32), scales, zps, axis)
+    np.testing.assert_array_equal(host(ctx.dequantize_per_channel(got, dev(scales), dev(zps), axis)), want_y)
+    for mode in (hipq.FORM_MUL_INV, hipq.FORM_DIV | hipq.ROUND_HALF_EVEN):
+        # off alignment: the same elements at an address one element past a 16-byte boundary
+        n = x.size
+        pad = torch.empty(n + 4, dtype=torch.float32, device="cuda")
+        pad[1:n + 1] = dev(x).reshape(-1)
+        off = pad[1:n + 1].view(shape)
+        assert off.data_ptr() % 16 == 4
+        a = ctx.quantize_per_channel(dev(x), dev(scales), dev(zps), axis, mode)
+        b = ctx.quantize_per_channel(off, dev(scales), dev(zps), axis, mode)
+        assert torch.equal(a, b)
+    if axis == 0 and len(shape) == 2:
+        want = oracle.quantize_per_channel_simd(x, scales, zps, shape[1])
+        got = ctx.quantize_per_channel(dev(x), dev(scales), dev(zps), 0, hipq.FORM_MUL_INV)
+        np.testing.assert_array_equal(host(got), want.astype(np.int8))
+
+
 @pytest.mark.parametrize("shape", [(1, 1), (5, 9), (64, 256), (100, 333)])
 def test_requantize(ctx, hipq, oracle, shape):
     rng = np.random.default_rng(shape[1])

@@ -816,6 +816,105 @@ __global__ __launch_bounds__(kBlock) void dequantize_per_channel_kernel(const in
     }
 }
 
+// The channel of vector j (four consecutive elements) of a dense [outer, channels, inner] view with inner % 4 == 0,
+// so that a vector never straddles channels: (j / (inner / 4)) % channels, by shifts where the counts are powers
+// of two and by 32-bit divisions where the index fits.
+struct ChannelOfVector {
+    size_t vpc, channels;  // vectors per channel run
+    int vpc_shift, ch_shift;
+    bool vpc_pow2, ch_pow2, small;
+    __device__ ChannelOfVector(size_t inner, size_t channels_, size_t nvec) : vpc(inner / 4), channels(channels_) {
+        vpc_pow2 = (vpc & (vpc - 1)) == 0;
+        ch_pow2 = (channels & (channels - 1)) == 0;
+        vpc_shift = __builtin_ffsll(static_cast<long long>(vpc)) - 1;
+        ch_shift = __builtin_ffsll(static_cast<long long>(channels)) - 1;
+        small = nvec < (size_t(1) << 32);
+    }
+    __device__ size_t operator()(size_t j) const {
+        size_t run;
+        if (vpc_pow2)
+            run = j >> vpc_shift;
+        else if (small)
+            run = static_cast<uint32_t>(j) / static_cast<uint32_t>(vpc);
+        else
+            run = j / vpc;
+        if (ch_pow2) return run & (channels - 1);
+        if (small) return static_cast<uint32_t>(run) % static_cast<uint32_t>(channels);
+        return run % channels;
+    }
+};
+
+// quantize_per_channel_kernel / dequantize_per_channel_kernel on vectors of four: 16-byte loads (4-byte for codes),
+// 4-byte (16-byte) stores, four in flight per lane on whole tiles, the streams that are touched once past the
+// caches; the element arithmetic is the scalar kernels'.  inner % 4 == 0, x / out aligned to their vector size.
+template <bool DIV, bool EVEN>
+__global__ __launch_bounds__(kBlock) void quantize_per_channel_vec_kernel(const float *__restrict__ x, size_t nvec,
+                                                                           size_t channels, size_t inner,
+                                                                           const float *__restrict__ scales,
+                                                                           const int32_t *__restrict__ zps,
+                                                                           int8_t *__restrict__ out) {
+    const ChannelOfVector channel_of(inner, channels, nvec);
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    uint32_t *out4 = reinterpret_cast<uint32_t *>(out);
+    auto emit = [&](size_t j, const float4 &t) {
+        const size_t c = channel_of(j);
+        const float s = scales[c], zpf = static_cast<float>(zps[c]);
+        const float inv = DIV ? 0.0f : 1.0f / s;  // the division form divides directly, as the scalar kernel does
+        auto one = [&](float v) { return to_int_nan0(quantize_value<DIV, EVEN>(v, s, inv, zpf, -128.0f, 127.0f)); };
+        store_stream(out4 + j, pack4(one(t.x), one(t.y), one(t.z), one(t.w)));
+    };
+    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * kTileVec + threadIdx.x;
+        if ((t + 1) * kTileVec <= nvec) {
+            float4 v[kVecPerThread];
+#pragma unroll
+            for (int i = 0; i < kVecPerThread; ++i) v[i] = load_stream(x4 + base + size_t(i) * kBlock);
+#pragma unroll
+            for (int i = 0; i < kVecPerThread; ++i) emit(base + size_t(i) * kBlock, v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kVecPerThread; ++i) {
+                const size_t j = base + size_t(i) * kBlock;
+                if (j < nvec) emit(j, x4[j]);
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void dequantize_per_channel_vec_kernel(const int8_t *__restrict__ q, size_t nvec,
+                                                                             size_t channels, size_t inner,
+                                                                             const float *__restrict__ scales,
+                                                                             const int32_t *__restrict__ zps,
+                                                                             float *__restrict__ out) {
+    const ChannelOfVector channel_of(inner, channels, nvec);
+    const uint32_t *q4 = reinterpret_cast<const uint32_t *>(q);
+    float4 *out4 = reinterpret_cast<float4 *>(out);
+    auto emit = [&](size_t j, uint32_t w) {
+        const size_t c = channel_of(j);
+        const float s = scales[c], zpf = static_cast<float>(zps[c]);
+        auto one = [&](int shift) { return s * (static_cast<float>(static_cast<int8_t>(w >> shift)) - zpf); };
+        store_stream(out4 + j, make_float4(one(0), one(8), one(16), one(24)));
+    };
+    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * kTileVec + threadIdx.x;
+        if ((t + 1) * kTileVec <= nvec) {
+            uint32_t w[kVecPerThread];
+#pragma unroll
+            for (int i = 0; i < kVecPerThread; ++i) w[i] = q4[base + size_t(i) * kBlock];
+#pragma unroll
+            for (int i = 0; i < kVecPerThread; ++i) emit(base + size_t(i) * kBlock, w[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kVecPerThread; ++i) {
+                const size_t j = base + size_t(i) * kBlock;
+                if (j < nvec) emit(j, q4[j]);
+            }
+        }
+    }
+}
+
 // int32 accumulators -> int8: v = acc*(s_a*s_w[c]) (+bias[c]); q = clamp(round(v/s_out)+zp_out).
 template <bool EVEN>
 __global__ __launch_bounds__(kBlock) void requantize_kernel(const int32_t *__restrict__ acc, size_t rows, size_t cols,
@@ -1450,8 +1549,24 @@ int32_t hipq_quantize_per_channel_f32_i8(hipq_ctx *ctx, const float *x, size_t o
     HIPQ_REQUIRE_PTR(scales);
     HIPQ_REQUIRE_PTR(zero_points);
     HIPQ_REQUIRE_PTR(out);
-    const int grid = grid_for_elems(ctx, total);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    if (inner % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(out) & 3u) == 0) {
+        const int vgrid = grid_for_tiles(ctx, total);
+#define HIPQ_LAUNCH_PCV(D, E)                                                                                          \
+    hipLaunchKernelGGL((quantize_per_channel_vec_kernel<D, E>), dim3(vgrid), dim3(kBlock), 0, ctx->stream, x, total / 4, \
+                       channels, inner, scales, zero_points, out)
+        if (div && even)
+            HIPQ_LAUNCH_PCV(true, true);
+        else if (div)
+            HIPQ_LAUNCH_PCV(true, false);
+        else if (even)
+            HIPQ_LAUNCH_PCV(false, true);
+        else
+            HIPQ_LAUNCH_PCV(false, false);
+#undef HIPQ_LAUNCH_PCV
+        return check_launch(__func__);
+    }
+    const int grid = grid_for_elems(ctx, total);
 #define HIPQ_LAUNCH_PC(D, E)                                                                                       \
     hipLaunchKernelGGL((quantize_per_channel_kernel<D, E>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, total,     \
                        channels, inner, scales, zero_points, out)
@@ -1477,6 +1592,11 @@ int32_t hipq_dequantize_per_channel_i8_f32(hipq_ctx *ctx, const int8_t *q, size_
     HIPQ_REQUIRE_PTR(scales);
     HIPQ_REQUIRE_PTR(zero_points);
     HIPQ_REQUIRE_PTR(out);
+    if (inner % 4 == 0 && (reinterpret_cast<uintptr_t>(q) & 3u) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+        hipLaunchKernelGGL(dequantize_per_channel_vec_kernel, dim3(grid_for_tiles(ctx, total)), dim3(kBlock), 0,
+                           ctx->stream, q, total / 4, channels, inner, scales, zero_points, out);
+        return check_launch(__func__);
+    }
     const int grid = grid_for_elems(ctx, total);
     hipLaunchKernelGGL(dequantize_per_channel_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, q, total, channels,
                        inner, scales, zero_points, out);
