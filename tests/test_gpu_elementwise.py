@@ -331,6 +331,75 @@ def test_per_channel_any_axis(ctx, hipq, oracle, axis):
         np.testing.assert_array_equal(got, want.astype(np.int8))
 
 
+SPREAD_SHAPES = [((8, 64, 28, 28), 1, 1), ((300, 1000), 1, 1), ((64, 33, 130), 1, 4), ((5, 12, 4400), 1, 5),
+                 ((20000, 16), 1, 1), ((9000, 8, 4), 1, 1), ((3, 700, 129), 2, 1), ((2, 3, 50000), 1, 1),
+                 ((1025, 257), 1, 1), ((40, 2000, 4), 1, 3)]
+
+
+@pytest.mark.parametrize("shape,axis,group", SPREAD_SHAPES)
+def test_per_channel_auto_spread_over_columns(ctx, hipq, oracle, shape, axis, group):
+    """Ranges, parameters and codes per channel / per group of channels over a channel axis that is not the leading one,
+    at sizes where the work is spread over many workgroups by columns (few groups, or short runs per channel):
+    vectors of four and single elements, column tiles narrower than a workgroup, a last group that is shorter."""
+    x = normal(sum(shape) + axis, shape) * np.linspace(0.2, 3.0, shape[axis], dtype=np.float32).reshape(
+        [-1 if i == axis else 1 for i in range(len(shape))])
+    assert x.size >= 1 << 18
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    for qmin, qmax in ((-128, 127), (-8, 7)):
+        q, s, z, status = ctx.quantize_per_group_auto(dev(x), outer, shape[axis], inner, group,
+                                                      hipq.PARAMS_ZERO_INCLUDED, qmin, qmax, hipq.FORM_DIV)
+        want, ws, wz, _, _ = oracle.quantize_group_wise(x, axis, group, qmin, qmax)
+        assert int(host(status)[0]) == 0
+        np.testing.assert_array_equal(host(s), ws)
+        np.testing.assert_array_equal(host(z), wz)
+        np.testing.assert_array_equal(host(q).astype(np.float32), want)
+    if group == 1:
+        for scheme, flavor in ((oracle.PER_CHANNEL_SYMMETRIC, hipq.PARAMS_SYMMETRIC),
+                               (oracle.PER_CHANNEL_AFFINE, hipq.PARAMS_AFFINE)):
+            want_q, want_s, want_z = oracle.quantize_per_channel_auto(x, axis, 0, scheme)
+            q, s, z, status = ctx.quantize_per_channel_auto(dev(x), axis, flavor)
+            assert host(status)[0] == 0
+            np.testing.assert_array_equal(host(s), want_s)
+            np.testing.assert_array_equal(host(z), want_z)
+            np.testing.assert_array_equal(host(q), want_q.astype(np.int8))
+
+
+def test_per_channel_auto_spread_half_even_and_bad_groups(ctx, hipq, oracle):
+    """Round-half-even over columns equals the per-row kernel on the transposed matrix; a channel holding an infinity
+    sets the status word and keeps its codes untouched while the other channels get theirs; NaNs are left out of a
+    channel's range and become code 0."""
+    x = np.round(normal(5, (600, 500)) * 8) / 16  # many exact .5 ties after the division
+    xd = dev(x)
+    q, s, z, status = ctx.quantize_per_channel_auto(xd, 1, hipq.PARAMS_AFFINE, hipq.ROUND_HALF_EVEN)
+    qr, sr, zr, _ = ctx.quantize_per_row(xd.t().contiguous(), hipq.PARAMS_AFFINE, hipq.ROUND_HALF_EVEN)
+    assert host(status)[0] == 0
+    assert torch.equal(s, sr) and torch.equal(z, zr) and torch.equal(q, qr.t())
+    q0, _, _, _ = ctx.quantize_per_channel_auto(xd, 1, hipq.PARAMS_AFFINE, 0)
+    assert not torch.equal(q, q0)  # the ties do round differently
+    bad = x.copy()
+    bad[17, 3] = np.inf
+    bad[5, 9] = np.nan
+    out = torch.full((600, 500), 77, dtype=torch.int8, device="cuda")
+    scales = torch.empty(500, dtype=torch.float32, device="cuda")
+    zps = torch.empty(500, dtype=torch.int32, device="cuda")
+    status = torch.empty(1, dtype=torch.int32, device="cuda")
+    ctx.call("hipq_quantize_per_channel_auto_f32_i8", dev(bad).data_ptr(), 600, 500, 1, hipq.PARAMS_AFFINE, 0,
+             out.data_ptr(), scales.data_ptr(), zps.data_ptr(), status.data_ptr())
+    assert host(status)[0] == hipq.INVALID_ARGUMENT
+    got = host(out)
+    assert (got[:, 3] == 77).all()
+    keep = np.ones(500, bool)
+    keep[3] = False
+    ref_in = bad.copy()
+    ref_in[17, 3] = x[17, 3]
+    want_q, want_s, want_z = oracle.quantize_per_channel_auto(ref_in, 1, 0, oracle.PER_CHANNEL_AFFINE)
+    assert np.isnan(want_q[5, 9]) and got[5, 9] == 0  # the float carrier keeps the NaN; as an int8 code it is 0
+    np.testing.assert_array_equal(got[:, keep], np.nan_to_num(want_q, nan=0.0).astype(np.int8)[:, keep])
+    np.testing.assert_array_equal(host(scales)[keep], want_s[keep])
+    np.testing.assert_array_equal(host(zps)[keep], want_z[keep])
+
+
 @pytest.mark.parametrize("shape,axis", [((3, 8, 12), 0), ((3, 8, 12), 1), ((7, 5, 2048), 1), ((6, 1000), 0),
                                         ((300, 64, 36), 1), ((1, 1, 4), 2), ((257, 4100), 0), ((16, 4096), 1)])
 def test_per_channel_vector_forms(ctx, hipq, oracle, shape, axis):

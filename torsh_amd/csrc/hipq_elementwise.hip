@@ -788,6 +788,199 @@ __global__ __launch_bounds__(kBlock) void quantize_per_channel_auto_kernel(
     }
 }
 
+// ---- the same over many workgroups: [outer, channels, inner] read as the matrix [outer, period = channels * inner],
+// whose column j belongs to group j / (inner * group).  A thread owns one column unit (V = 4 consecutive columns
+// where a channel's run is a multiple of four and the base is aligned, else 1) of a tile of `col_lanes` units and walks
+// a share of the rows, so its group never changes; the workgroup's other threads (256 / col_lanes row lanes) walk other
+// rows of the same tile.  Two passes after the keys are set: ranges by atomic min / max on order-preserving integer
+// keys, then parameters (per thread, from its group's keys) and codes.  A workgroup per group, as above, leaves most of the chip idle when the groups are few or their
+// runs short.
+struct ChannelColumns {
+    size_t outer, period, units, span;  // rows; elements per row; column units per row (period / V); inner * group
+    unsigned col_tiles, slices;         // grid = col_tiles * slices
+    int col_lanes_log2;
+    int key_shift;  // a group's two keys start at keys[group << key_shift]: a 64-byte line of its own while that is cheap
+};
+
+// Floats as integers of the same order (-0 below +0), for atomicMin / atomicMax; its own inverse.
+__device__ __forceinline__ int32_t ordered_key(int32_t bits) { return bits ^ ((bits >> 31) & 0x7fffffff); }
+
+__global__ void channel_keys_init_kernel(int32_t *keys, uint32_t groups, int key_shift, int32_t *status) {
+    const uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g < groups) {
+        keys[size_t(g) << key_shift] = ordered_key(__float_as_int(INFINITY));
+        keys[(size_t(g) << key_shift) + 1] = ordered_key(__float_as_int(-INFINITY));
+    }
+    if (g == 0 && status) *status = 0;
+}
+
+constexpr uint32_t kNoGroup = 0xffffffffu;
+
+// Where thread `tid` of workgroup `block` starts: its column unit, first row and row step; false if it has no column.
+struct ChannelWalk {
+    size_t unit, row, row_step;
+    __device__ bool start(const ChannelColumns &cc, unsigned block, unsigned tid) {
+        const unsigned tile = block % cc.col_tiles, slice = block / cc.col_tiles;
+        const unsigned col_lane = tid & ((1u << cc.col_lanes_log2) - 1), row_lane = tid >> cc.col_lanes_log2;
+        const unsigned row_lanes = kBlock >> cc.col_lanes_log2;
+        unit = (size_t(tile) << cc.col_lanes_log2) + col_lane;
+        row = size_t(slice) * row_lanes + row_lane;
+        row_step = size_t(cc.slices) * row_lanes;
+        return unit < cc.units;
+    }
+};
+
+template <int V>
+__global__ __launch_bounds__(kBlock) void channel_range_kernel(const float *__restrict__ x, ChannelColumns cc,
+                                                                int32_t *__restrict__ keys) {
+    ChannelWalk w;
+    const bool live = w.start(cc, blockIdx.x, threadIdx.x);
+    uint32_t g = kNoGroup;
+    MinMax m{INFINITY, -INFINITY};
+    if (live) {
+        g = static_cast<uint32_t>(w.unit * V / cc.span);
+        auto take = [&](size_t row) {
+            const float *p = x + row * cc.period + w.unit * V;
+            if constexpr (V == 4) {
+                const float4 t = *reinterpret_cast<const float4 *>(p);
+                acc_minmax(m, t.x);
+                acc_minmax(m, t.y);
+                acc_minmax(m, t.z);
+                acc_minmax(m, t.w);
+            } else {
+                acc_minmax(m, *p);
+            }
+        };
+        size_t row = w.row;
+        for (; row < cc.outer && cc.outer - row > 3 * w.row_step; row += 4 * w.row_step) {
+            take(row);
+            take(row + w.row_step);
+            take(row + 2 * w.row_step);
+            take(row + 3 * w.row_step);
+        }
+        for (; row < cc.outer; row += w.row_step) take(row);
+    }
+    // Column tiles of a wave's width or less: the workgroup's waves hold the same columns lane by lane (other rows),
+    // so they combine through the LDS and the first wave alone goes on.
+    if (cc.col_lanes_log2 <= 6) {
+        __shared__ float lds_mn[kBlock], lds_mx[kBlock];
+        lds_mn[threadIdx.x] = m.mn;
+        lds_mx[threadIdx.x] = m.mx;
+        __syncthreads();
+        if (threadIdx.x >= kWave) return;
+#pragma unroll
+        for (int wv = 1; wv < kBlock / kWave; ++wv) {
+            m.mn = fminf(m.mn, lds_mn[wv * kWave + threadIdx.x]);
+            m.mx = fmaxf(m.mx, lds_mx[wv * kWave + threadIdx.x]);
+        }
+    }
+    // Lanes of one group combine first (a wave's columns are consecutive, so a group's lanes are neighbours; where
+    // equal groups are not neighbours the extra combination is of the same group and changes nothing), then the
+    // first lane of every run of equal groups adds the run to the group's keys.
+    const int lane = threadIdx.x % kWave;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const float omn = __shfl_down(m.mn, d), omx = __shfl_down(m.mx, d);
+        const uint32_t og = __shfl_down(g, d);
+        if (lane + d < kWave && og == g) {
+            m.mn = fminf(m.mn, omn);
+            m.mx = fmaxf(m.mx, omx);
+        }
+    }
+    const uint32_t before = __shfl_up(g, 1);
+    const bool head = g != kNoGroup && (lane == 0 || before != g);
+    auto add_to_keys = [&](uint32_t group, float mn, float mx) {
+        if (!(mn <= mx)) return;  // no finite or infinite value seen
+        atomicMin(&keys[size_t(group) << cc.key_shift], ordered_key(__float_as_int(mn)));
+        atomicMax(&keys[(size_t(group) << cc.key_shift) + 1], ordered_key(__float_as_int(mx)));
+    };
+    if (cc.col_lanes_log2 > 6) {
+        // Wide tiles over long runs: mostly the four waves hold one group, the same one; then one thread adds for
+        // all four.  (Atomics of many workgroups on a few keys queue up behind each other.)
+        constexpr int nw = kBlock / kWave;
+        constexpr uint32_t kMixed = kNoGroup - 1;
+        __shared__ float wave_mn[nw], wave_mx[nw];
+        __shared__ uint32_t wave_group[nw];
+        const unsigned long long heads = __ballot(head);
+        if (lane == 0) {
+            wave_group[threadIdx.x / kWave] = heads == 1ull ? g : kMixed;
+            wave_mn[threadIdx.x / kWave] = m.mn;
+            wave_mx[threadIdx.x / kWave] = m.mx;
+        }
+        __syncthreads();
+        bool same = wave_group[0] < kMixed;
+#pragma unroll
+        for (int wv = 1; wv < nw; ++wv) same = same && wave_group[wv] == wave_group[0];
+        if (same) {
+            if (threadIdx.x == 0) {
+                MinMax all{wave_mn[0], wave_mx[0]};
+#pragma unroll
+                for (int wv = 1; wv < nw; ++wv) {
+                    all.mn = fminf(all.mn, wave_mn[wv]);
+                    all.mx = fmaxf(all.mx, wave_mx[wv]);
+                }
+                add_to_keys(wave_group[0], all.mn, all.mx);
+            }
+            return;
+        }
+    }
+    if (head) add_to_keys(g, m.mn, m.mx);
+}
+
+// Parameters of the thread's group from the group's keys, then the codes of the thread's column.  The thread that
+// owns a group's first column on the first row writes the group's parameters and, for a range that gives none, the
+// status; such a group keeps what `out` held, as with a workgroup per group.
+template <bool EVEN, int V>
+__global__ __launch_bounds__(kBlock) void channel_quantize_kernel(const float *__restrict__ x, ChannelColumns cc,
+                                                                   const int32_t *__restrict__ keys, int flavor, int qmin,
+                                                                   int qmax, int8_t *__restrict__ out,
+                                                                   float *__restrict__ out_scales,
+                                                                   int32_t *__restrict__ out_zps,
+                                                                   int32_t *__restrict__ out_status) {
+    ChannelWalk w;
+    if (!w.start(cc, blockIdx.x, threadIdx.x)) return;
+    const size_t g = w.unit * V / cc.span;
+    const float mn = __int_as_float(ordered_key(keys[g << cc.key_shift]));
+    const float mx = __int_as_float(ordered_key(keys[(g << cc.key_shift) + 1]));
+    float scale;
+    int zp;
+    const int st = params_from_minmax(mn, mx, flavor, qmin, qmax, &scale, &zp);
+    if (w.row == 0 && w.unit * V == g * cc.span) {
+        if (out_scales) out_scales[g] = scale;
+        if (out_zps) out_zps[g] = zp;
+        if (st != HIPQ_SUCCESS && out_status) *out_status = st;
+    }
+    if (st != HIPQ_SUCCESS) return;
+    const float inv = recip_for_div(scale), zpf = static_cast<float>(zp);
+    const float lo = static_cast<float>(qmin), hi = static_cast<float>(qmax);
+    auto one = [&](float v) { return to_int_nan0(quantize_value<true, EVEN>(v, scale, inv, zpf, lo, hi)); };
+    using Vec = typename std::conditional<V == 4, float4, float>::type;
+    auto load = [&](size_t row) {
+        const Vec *p = reinterpret_cast<const Vec *>(x + row * cc.period + w.unit * V);
+        if constexpr (V == 4)
+            return load_stream(p);
+        else
+            return *p;
+    };
+    auto store = [&](size_t row, const Vec &t) {
+        int8_t *q = out + row * cc.period + w.unit * V;
+        if constexpr (V == 4)
+            store_stream(reinterpret_cast<uint32_t *>(q), pack4(one(t.x), one(t.y), one(t.z), one(t.w)));
+        else
+            *q = static_cast<int8_t>(one(t));
+    };
+    size_t row = w.row;
+    for (; row < cc.outer && cc.outer - row > 3 * w.row_step; row += 4 * w.row_step) {
+        const Vec a = load(row), b = load(row + w.row_step), c = load(row + 2 * w.row_step),
+                  d = load(row + 3 * w.row_step);
+        store(row, a);
+        store(row + w.row_step, b);
+        store(row + 2 * w.row_step, c);
+        store(row + 3 * w.row_step, d);
+    }
+    for (; row < cc.outer; row += w.row_step) store(row, load(row));
+}
+
 // Explicit per-channel parameters over a dense [outer, channels, inner] view.
 template <bool DIV, bool EVEN>
 __global__ __launch_bounds__(kBlock) void quantize_per_channel_kernel(const float *__restrict__ x, size_t total,
@@ -1374,6 +1567,9 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
     return check_launch(fn);
 }
 
+// Below this many elements the per-group workgroups' one launch beats the three of the form spread over columns.
+constexpr size_t kSpreadMinElems = size_t(1) << 18;
+
 // quantize_per_channel_auto over a dense [outer, channels, inner] view with groups of `group`
 // consecutive channels sharing their parameters (1 = per channel), integer range [qmin, qmax].
 static int32_t quantize_channels(const char *fn, hipq_ctx *ctx, const float *x, size_t outer, size_t channels,
@@ -1387,15 +1583,73 @@ static int32_t quantize_channels(const char *fn, hipq_ctx *ctx, const float *x, 
     int32_t rc = any_flavor ? HIPQ_SUCCESS : check_row_flavor(fn, flavor);
     if (rc) return rc;
     if ((rc = check_mode(fn, mode))) return rc;
-    if (out_status) hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
+    const size_t groups = (channels + group - 1) / group;
+    const size_t period = channels * inner;
+    // Many workgroups over the columns: a workgroup per group leaves the chip idle where the groups are few, reads
+    // with a stride where their runs are short, and works element by element.  Small tensors stay with its one launch.
+    const bool spread = x && out && !(groups >> 31) && outer * period >= kSpreadMinElems && period >= 16;
+    // (the spread form clears the status word in its first kernel)
+    if (out_status && !spread)
+        hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, ctx->stream, out_status, 0, size_t(1));
     if (channels == 0) return check_launch(fn);
     if (outer == 0 || inner == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: channels of zero length have no range", fn);
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
-    const size_t groups = (channels + group - 1) / group;
     if (groups >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many channels", fn);
+    const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    if (spread) {
+        const bool vec = inner % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 &&
+                         (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+        ChannelColumns cc;
+        cc.outer = outer;
+        cc.period = period;
+        cc.units = vec ? period / 4 : period;
+        cc.span = inner * group;
+        // Groups narrower than a wave's columns: every lane, or every few, ends in atomics of its own (they go past
+        // the per-die caches and cost accordingly).  Tiles one wave wide then let the four waves combine first, and
+        // at least eight rows per thread keep the atomics under one per 32 elements.
+        const bool narrow = cc.span / (vec ? 4 : 1) < size_t(kWave);
+        const int widest = narrow ? 6 : 8;
+        cc.col_lanes_log2 = 0;
+        while (cc.col_lanes_log2 < widest && (size_t(1) << cc.col_lanes_log2) < cc.units) ++cc.col_lanes_log2;
+        const size_t col_lanes = size_t(1) << cc.col_lanes_log2, row_lanes = kBlock / col_lanes;
+        const size_t col_tiles = (cc.units + col_lanes - 1) / col_lanes;
+        const size_t row_sets = (outer + row_lanes - 1) / row_lanes;
+        const size_t most = narrow ? (row_sets + 7) / 8 : row_sets;
+        size_t slices = (size_t(ctx->num_cus) * 8 + col_tiles - 1) / col_tiles;
+        if (slices > most) slices = most;
+        if (col_tiles * slices >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many columns", fn);
+        cc.col_tiles = static_cast<unsigned>(col_tiles);
+        cc.slices = static_cast<unsigned>(slices);
+        void *s = nullptr;
+        // (narrow groups: a wave's atomics go to neighbouring keys, which travel together when they share lines)
+        cc.key_shift = (!narrow && groups <= 65536) ? 4 : 1;
+        if ((rc = scratch(ctx, kScratchHeader + (groups << cc.key_shift) * sizeof(int32_t), &s))) return rc;
+        int32_t *keys = reinterpret_cast<int32_t *>(static_cast<char *>(s) + kScratchHeader);
+        const unsigned ngroups = static_cast<unsigned>(groups), gblocks = (ngroups + kBlock - 1) / kBlock;
+        const dim3 grid(cc.col_tiles * cc.slices);
+        hipLaunchKernelGGL(channel_keys_init_kernel, dim3(gblocks), dim3(kBlock), 0, ctx->stream, keys, ngroups,
+                           cc.key_shift, out_status);
+        if (vec)
+            hipLaunchKernelGGL(channel_range_kernel<4>, grid, dim3(kBlock), 0, ctx->stream, x, cc, keys);
+        else
+            hipLaunchKernelGGL(channel_range_kernel<1>, grid, dim3(kBlock), 0, ctx->stream, x, cc, keys);
+#define HIPQ_LAUNCH_CQ(E, V)                                                                                         \
+    hipLaunchKernelGGL((channel_quantize_kernel<E, V>), grid, dim3(kBlock), 0, ctx->stream, x, cc, keys, flavor, qmin, \
+                       qmax, out, out_scales, out_zero_points, out_status)
+        if (even && vec)
+            HIPQ_LAUNCH_CQ(true, 4);
+        else if (even)
+            HIPQ_LAUNCH_CQ(true, 1);
+        else if (vec)
+            HIPQ_LAUNCH_CQ(false, 4);
+        else
+            HIPQ_LAUNCH_CQ(false, 1);
+#undef HIPQ_LAUNCH_CQ
+        return check_launch(fn);
+    }
     const int grid = static_cast<int>(groups);
-    if (mode & HIPQ_ROUND_HALF_EVEN)
+    if (even)
         hipLaunchKernelGGL((quantize_per_channel_auto_kernel<true>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, outer,
                            channels, inner, group, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status);
     else
