@@ -224,7 +224,11 @@ HIPQ_API int32_t hipq_quantize_per_row_strided_f32_i8(hipq_ctx *ctx, const float
                                                       float *out_scales, int32_t *out_zero_points,
                                                       int32_t *out_status);
 /* quantize_per_channel_auto for any axis of a dense tensor viewed as
- * [outer, channels, inner] (algorithms.rs:126-242). */
+ * [outer, channels, inner] (algorithms.rs:126-242).  A channel whose range is
+ * not finite sets *out_status and keeps what `out` held for it.  From 256 Ki
+ * elements on, a channel axis that is not the leading one takes two range keys
+ * per channel from the context's scratch memory (grown on first use), so calls
+ * on one context must not overlap, as for every entry point that uses it. */
 HIPQ_API int32_t hipq_quantize_per_channel_auto_f32_i8(hipq_ctx *ctx, const float *x, size_t outer,
                                                        size_t channels, size_t inner, int32_t flavor,
                                                        int32_t mode, int8_t *out, float *out_scales,
