@@ -233,7 +233,16 @@ __global__ __launch_bounds__(kRowBlock) void row_op_kernel(const float *x, const
 }
 
 __global__ __launch_bounds__(256) void gelu_kernel(const float *__restrict__ x, size_t n, float *__restrict__ out) {
-    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += size_t(gridDim.x) * 256) out[i] = gelu_tanh(x[i]);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    const size_t nvec = aligned ? n / 4 : 0;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < nvec; i += size_t(gridDim.x) * 256) {
+        const float4 p = x4[i];
+        o4[i] = make_float4(gelu_tanh(p.x), gelu_tanh(p.y), gelu_tanh(p.z), gelu_tanh(p.w));
+    }
+    for (size_t i = nvec * 4 + size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += size_t(gridDim.x) * 256)
+        out[i] = gelu_tanh(x[i]);
 }
 
 __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, const float *__restrict__ b, size_t n,
@@ -350,7 +359,7 @@ int32_t hipq_gelu_tanh_f32(hipq_ctx *ctx, const float *x, size_t n, float *out) 
     if (n == 0) return HIPQ_SUCCESS;
     HIPQ_REQUIRE_PTR(x);
     HIPQ_REQUIRE_PTR(out);
-    size_t blocks = (n + 255) / 256;
+    size_t blocks = (n / 4 + 255) / 256 + 1;
     const size_t cap = size_t(ctx->num_cus) * 16;
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL(gelu_kernel, dim3(static_cast<int>(blocks)), dim3(256), 0, ctx->stream, x, n, out);
