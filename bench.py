@@ -289,6 +289,35 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
         prm = ctx.new_qparams()
         for i in range(reps):  # quantize_tensor_auto at the same size: one launch, the tensor held in registers
             ctx.quantize_dynamic_per_tensor(xs[i % 8], out=qs[i % 8], params=prm)
+    elif which == "per_channel":
+        # per-channel forms: given parameters (quantize, dequantize) over [4096 channels, 4096]; ranges per row; ranges
+        # over a channel axis that is not the leading one (an NCHW activation per channel, a matrix per column)
+        xs = [torch.randn(4096, 4096, generator=g, device="cuda") for _ in range(8)]
+        qs = [torch.empty((4096, 4096), dtype=torch.int8, device="cuda") for _ in range(8)]
+        ys = [torch.empty((4096, 4096), device="cuda") for _ in range(8)]
+        sc = torch.rand(4096, generator=g, device="cuda") * 0.05 + 0.01
+        zp = torch.zeros(4096, dtype=torch.int32, device="cuda")
+        osc = torch.empty(4096, device="cuda")
+        ozp = torch.empty(4096, dtype=torch.int32, device="cuda")
+        st = torch.empty(1, dtype=torch.int32, device="cuda")
+        act = [torch.randn(64, 256, 56, 56, generator=g, device="cuda") for _ in range(2)]
+        qact = torch.empty((64, 256, 56, 56), dtype=torch.int8, device="cuda")
+        torch.cuda.synchronize()
+        for i in range(reps):
+            ctx.call("hipq_quantize_per_channel_f32_i8", xs[i % 8].data_ptr(), 1, 4096, 4096, sc.data_ptr(),
+                     zp.data_ptr(), hipq.FORM_DIV, qs[i % 8].data_ptr())
+        for i in range(reps):
+            ctx.call("hipq_dequantize_per_channel_i8_f32", qs[i % 8].data_ptr(), 1, 4096, 4096, sc.data_ptr(),
+                     zp.data_ptr(), ys[i % 8].data_ptr())
+        for i in range(reps):
+            ctx.call("hipq_quantize_per_row_f32_i8", xs[i % 8].data_ptr(), 4096, 4096, hipq.PARAMS_SYMMETRIC, 0,
+                     qs[i % 8].data_ptr(), osc.data_ptr(), ozp.data_ptr(), st.data_ptr())
+        for i in range(reps):  # per column of a [4096, 4096] matrix
+            ctx.call("hipq_quantize_per_channel_auto_f32_i8", xs[i % 8].data_ptr(), 4096, 4096, 1,
+                     hipq.PARAMS_SYMMETRIC, 0, qs[i % 8].data_ptr(), osc.data_ptr(), ozp.data_ptr(), st.data_ptr())
+        for i in range(reps):  # per channel of a [64, 256, 56, 56] activation
+            ctx.call("hipq_quantize_per_channel_auto_f32_i8", act[i % 2].data_ptr(), 64, 256, 56 * 56,
+                     hipq.PARAMS_SYMMETRIC, 0, qact.data_ptr(), osc.data_ptr(), ozp.data_ptr(), st.data_ptr())
     elif which == "calib":
         n = 4096 * 4096
         xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
@@ -368,7 +397,7 @@ def main() -> int:
                     help="milliseconds of untimed back-to-back launches before each timed region (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "conv_phases", "gemm_rowmajor", "step", "quantize", "calib", "special", "copy",
+    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "conv_phases", "gemm_rowmajor", "step", "quantize", "per_channel", "calib", "special", "copy",
                                           "stack", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
