@@ -179,6 +179,40 @@ def test_linear_packed_many_tiles_matches_row_major(ctx, hipq, m, n, k):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (256, 4096, 1024), (128, 2048, 4096), (384, 1024, 8192),
+                                   (500, 4096, 4096), (512, 4032, 4096), (512, 4096, 4000), (64, 512, 1024)])
+def test_dynamic_forward_with_and_without_weight_line_touching(hipq, m, n, k):
+    """The dynamic per-tensor forward on prepared weights lets its activation quantizer touch weight lines for the
+    GEMM while the grid waits for the range (shapes whose tiles make one round over the compute units and split into
+    one rectangle per die; the last four shapes here do not qualify or are ragged).  Values read that way are not
+    used: outputs and parameters are the same bits with the touching switched off (variant 11), call after call on
+    rotating weights."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(m + n + k)
+        sets = []
+        for _ in range(3):
+            wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+            sets.append((c.pack_rows(wq), torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4,
+                         torch.randn(n, generator=g, device="cuda")))
+        xs = [torch.randn(m, k, generator=g, device="cuda") * (i + 1) for i in range(6)]
+        got = {}
+        for variant in (0, 11):
+            c.set_gemm_kernel_variant(variant)
+            got[variant] = [c.linear_dynamic_packed(x, *sets[i % 3]).clone() for i, x in enumerate(xs)]
+            c.synchronize()
+        for a, b in zip(got[0], got[11]):
+            assert torch.equal(a, b)
+        # and against the separate calls: quantize into the packed layout, then the product
+        pw, sw, bias = sets[0]
+        pa, params = c.quantize_per_tensor_packed(xs[0])
+        want = c.linear_packed_i8_f32(pa, params.view(torch.float32)[:1], pw, sw, bias, m, n, k)  # scale: first field
+        c.synchronize()
+        assert torch.equal(got[0][0], want)
+    finally:
+        c.close()
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 64, 16), (1, 11008, 4096), (4, 11008, 4096), (16, 11008, 4096), (32, 1024, 1040),
                                    (7, 300, 11008), (3, 96, 16384), (5, 4096, 272)])
 def test_decode_forward_per_token(hipq, m, n, k):

@@ -126,6 +126,10 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
         return rc;
     }
     (void)hipq::four_wide_workgroups_fit(ctx);  // asked here so that no later call is the first
+    if (const char *e = getenv("HIPQ_GEMM_VARIANT")) {
+        const int v = atoi(e);
+        if (v >= 0 && v <= 11) ctx->gemm_variant = v;
+    }
     *out_ctx = ctx;
     return HIPQ_SUCCESS;
 }
@@ -175,8 +179,8 @@ int32_t hipq_ctx_synchronize(hipq_ctx *ctx) {
 
 int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant) {
     HIPQ_REQUIRE_PTR(ctx);
-    if (variant < 0 || variant > 10)
-        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..10", __func__, variant);
+    if (variant < 0 || variant > 11)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..11", __func__, variant);
     ctx->gemm_variant = variant;
     return HIPQ_SUCCESS;
 }

@@ -350,7 +350,8 @@ template <bool DIV, int RND, int FPW>
 __global__ __launch_bounds__(kBlock, 4) void quantize_packed_one_launch_kernel(const float *__restrict__ x, size_t rows,
                                                                                 size_t cols, hipq_qparams *out_params,
                                                                                 uint32_t *words, int spin_limit,
-                                                                                int8_t *__restrict__ out) {
+                                                                                int8_t *__restrict__ out,
+                                                                                WarmLines warm) {
     __shared__ float lds[kMeetingLdsFloats];
     const FragmentWalk fw(x, rows, cols);
     size_t f[FPW];
@@ -380,8 +381,27 @@ __global__ __launch_bounds__(kBlock, 4) void quantize_packed_one_launch_kernel(c
             }
         }
     const MinMax r = block_minmax(m, lds);
+    // While the grid agrees on the range the memory system is idle: touch the lines of the next kernel's operand
+    // that the workgroups of this die (workgroups are dealt to the dies in turn) will read first thing, one load
+    // per line, so that they wait in this die's L2.  The values are not used.
+    uint32_t touched = 0;
+    // Not by the waves that poll (the first of every workgroup, all of workgroup 0): loads return in order, so a
+    // poll issued behind such a load would not be seen before it.
+    if (warm.lines && threadIdx.x >= kWave && blockIdx.x != 0) {
+        constexpr uint32_t kWarmers = kBlock - kWave;
+        const uint32_t die = blockIdx.x % 8, slot = blockIdx.x / 8, sharers = (gridDim.x + 7 - die) / 8;
+        const uint32_t *base = warm.base + size_t(die) * warm.die_stride_lines * 32;
+        for (uint32_t i = slot * kWarmers + (threadIdx.x - kWave); i < warm.lines; i += sharers * kWarmers) {
+            // i counts the lines wanted: per row block, `starts` runs of `run_lines`, `start_step_lines` apart
+            const uint32_t rb = i / (warm.starts * warm.run_lines), rem = i % (warm.starts * warm.run_lines);
+            const uint32_t line = rb * warm.row_block_lines + (rem / warm.run_lines) * warm.start_step_lines +
+                                  rem % warm.run_lines;
+            touched ^= base[size_t(line) * 32];
+        }
+    }
     const MeetingParams agreed = meet_on_range(words, gen, r, HIPQ_PARAMS_SYMMETRIC, -128, 127, /*poison=*/true, spin_limit,
                                                lds, out_params);
+    asm volatile("" ::"v"(touched));
     const float scale = agreed.scale == agreed.scale ? agreed.scale : INFINITY;  // x * (1/inf): 0; NaN -> code 0
     const float inv = DIV ? recip_for_div(scale) : 1.0f / scale;
 #pragma unroll
@@ -1682,7 +1702,8 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
         // Every lane's 16 floats are all inside the matrix or all outside it, and four aligned float4.
 #define HIPQ_LAUNCH_Q1(D, E, F)                                                                                           \
     hipLaunchKernelGGL((quantize_packed_one_launch_kernel<D, E, F>), dim3(static_cast<int>(q1_blocks)), dim3(kBlock), 0, \
-                       ctx->stream, x, rows, cols, out_params, ctx->wait_error, ctx->wait_spin_limit, out)
+                       ctx->stream, x, rows, cols, out_params, ctx->wait_error, ctx->wait_spin_limit, out,              \
+                       ctx->warm)
 #define HIPQ_LAUNCH_Q1_MODE(F)          \
     do {                                \
         if (div && even)                \

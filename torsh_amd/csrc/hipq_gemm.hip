@@ -287,17 +287,10 @@ static void launch_tile(hipq_ctx *ctx, const int8_t *a, const int8_t *w, int M, 
                        ctx->stream, a, w, M, N, K, placed);
 }
 
-// Tuning and test hook, per context: HIPQ_GEMM_VARIANT=<n> in the environment (read when a context first
-// runs a GEMM), or hipq_set_gemm_kernel_variant(ctx, n), forces one kernel configuration wherever the shape
+// Tuning and test hook, per context: HIPQ_GEMM_VARIANT=<n> in the environment (read when the context is
+// created), or hipq_set_gemm_kernel_variant(ctx, n), forces one kernel configuration wherever the shape
 // allows it (0 = automatic).
-static int gemm_variant_override(hipq_ctx *ctx) {
-    if (ctx->gemm_variant < 0) {
-        const char *e = getenv("HIPQ_GEMM_VARIANT");
-        const int v = e ? atoi(e) : 0;
-        ctx->gemm_variant = (v >= 0 && v <= 10) ? v : 0;
-    }
-    return ctx->gemm_variant;
-}
+static int gemm_variant_override(hipq_ctx *ctx) { return ctx->gemm_variant; }
 
 template <int EPI, bool EVEN>
 static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size_t m, size_t n, size_t k,
@@ -316,6 +309,7 @@ static int32_t launch_gemm(hipq_ctx *ctx, const int8_t *a, const int8_t *w, size
     const size_t cus = static_cast<size_t>(ctx->num_cus);
     auto tiles = [&](size_t bm, size_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     int variant = gemm_variant_override(ctx);
+    if (variant == 9 || variant == 11) variant = 0;  // switches of the packed forms only
     if (variant == 0 && M <= 16 && K % 256 == 0) return launch_gemv<EPI, EVEN>(ctx, a, w, M, N, K, ep);
     const bool pipe_ok = (K % 128 == 0) && K >= 256;
     if (variant == 0 && pipe_ok) {

@@ -9,6 +9,14 @@
 
 #include "torsh_hipq.h"
 
+// Lines (128 bytes) of a packed operand wanted in the L2 of the die whose workgroups will read them: die d's share
+// starts die_stride_lines * d lines after base; within it, per row block (row_block_lines apart), `starts` runs of
+// run_lines lines, start_step_lines apart; `lines` of them per die in all.
+struct WarmLines {
+    const uint32_t *base = nullptr;
+    uint32_t lines = 0, die_stride_lines = 0, row_block_lines = 0, starts = 1, run_lines = 0, start_step_lines = 0;
+};
+
 struct hipq_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -22,13 +30,16 @@ struct hipq_ctx {
     // Device words of the context (kCtxWordsBytes of them, laid out as the kCtx* constants below say).  Word 0 is
     // set by a kernel whose bounded wait gave up; hipq_ctx_synchronize reads and clears it.
     uint32_t *wait_error = nullptr;
-    // Test and tuning hooks, per context: forced GEMM kernel form (0 = automatic, -1 = not yet read from the
-    // HIPQ_GEMM_VARIANT environment variable) and the spin limit of the persistent kernel's waits.
-    int gemm_variant = -1;
+    // Test and tuning hooks, per context: forced GEMM kernel form (0 = automatic; hipq_ctx_create takes it from the
+    // HIPQ_GEMM_VARIANT environment variable when that is set) and the spin limit of the persistent kernel's waits.
+    int gemm_variant = 0;
     int wait_spin_limit = 1 << 20;
     // How many contexts launch concurrently on this device (hipq_ctx_set_resident_share): kernels whose grid has to
     // be resident at once size it for 1 / resident_share of the device.
     int resident_share = 1;
+    // Set by a fused forward around its activation-quantize launch: lines of the operand that the next kernel reads
+    // first, for the quantizer's workgroups to touch while they wait for the grid's range.  lines = 0: none.
+    WarmLines warm;
     // Tuning aid (hipq_ctx_set_trace_buffer): caller-owned device memory for the packed GEMM's phase stamps.
     void *trace = nullptr;
     size_t trace_bytes = 0;
