@@ -322,8 +322,8 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
  * makes the dynamic per-tensor activation quantizer of the Linear forwards run as two launches (range
  * partials, then a quantizer that folds them) where it would run as one; 9 and 11 leave the choice
  * automatic and switch off, on prepared operands, the two-workgroups-per-compute-unit form of the
- * GEMM (9) and the touching of weight lines by the one-launch activation quantizer while its grid
- * waits for the range (11).
+ * GEMM (9) and the touching of weight / filter lines by the one-launch activation quantizers of the
+ * dynamic Linear and Conv2d forwards while their grids wait for the range (11).
  * Results do not depend on it; the parity tests use it to run every form on the same inputs. */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
 /* Test hook with no counterpart in the reference.  Two kernels couple their waves through device

@@ -189,6 +189,14 @@ def test_conv2d_forward_from_fp32_equals_quantize_then_conv(ctx, hipq, nb, c, h,
         assert (gp.scale, gp.zero_point, gp.min_val, gp.max_val, gp.status) == (p.scale, p.zero_point, p.min_val,
                                                                                 p.max_val, p.status)
         assert torch.equal(got, want), qmode
+        ctx.set_gemm_kernel_variant(11)  # the same without the filter lines touched while the quantizer's grid waits
+        try:
+            off, _ = ctx.conv2d_dynamic_packed(x, packed, sums, k, sw, bias, 0.05, 3, pad, quant_mode=qmode,
+                                               mode=hipq.ROUND_HALF_EVEN)
+            torch.cuda.synchronize()
+        finally:
+            ctx.set_gemm_kernel_variant(0)
+        assert torch.equal(off, want), qmode
 
 
 def test_conv2d_forward_from_fp32_reports_a_bad_range(ctx, hipq):

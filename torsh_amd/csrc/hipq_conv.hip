@@ -75,7 +75,8 @@ __global__ __launch_bounds__(kConvThreads) void conv_pack_image_kernel(const uin
 template <bool DIV, int RND>
 __global__ __launch_bounds__(kConvThreads, 4) void conv_quantize_pack_image_kernel(
     const float *__restrict__ x, int C, int H, int W, int pad_h, int pad_w, int flavor, int nb, int groups_per_cb,
-    hipq_qparams *out_params, uint32_t *words, int spin_limit, int8_t *__restrict__ out, int pixels) {
+    hipq_qparams *out_params, uint32_t *words, int spin_limit, int8_t *__restrict__ out, int pixels,
+    const uint32_t *__restrict__ touch, uint32_t touch_lines) {
     __shared__ float lds[kMeetingLdsFloats];
     const int hp = H + 2 * pad_h, wp = W + 2 * pad_w, cbs = C / 32;
     const int real_pixels = nb * hp * wp;
@@ -114,7 +115,17 @@ __global__ __launch_bounds__(kConvThreads, 4) void conv_quantize_pack_image_kern
         for (int i = threadIdx.x; i < (pixels - real_pixels) * 2; i += kConvThreads) tail[i] = make_uint4(0, 0, 0, 0);
         return;
     }
+    // While the grid agrees on the range: one load per 128-byte line of the prepared filters, which every die's
+    // workgroups of the convolution kernel read first thing (workgroups are dealt to the dies in turn, there as
+    // here), by the waves that do not poll.  The values are not used.
+    uint32_t touched = 0;
+    if (touch_lines && threadIdx.x >= kWave && blockIdx.x != 0) {
+        const uint32_t sharers = (work + 7 - blockIdx.x % 8) / 8, warmers = kConvThreads - kWave;
+        for (uint32_t i = (blockIdx.x / 8) * warmers + (threadIdx.x - kWave); i < touch_lines; i += sharers * warmers)
+            touched ^= touch[size_t(i) * 32];
+    }
     const MeetingParams agreed = meet_on_range(words, gen, r, flavor, 0, 255, /*poison=*/true, spin_limit, lds, out_params);
+    asm volatile("" ::"v"(touched));
     if (p >= real_pixels) return;
     const bool bad = agreed.scale != agreed.scale;
     const float scale = bad ? INFINITY : agreed.scale;  // x / inf: every code is the zero point
@@ -293,10 +304,15 @@ static int32_t conv_forward(const char *fn, hipq_ctx *ctx, const uint8_t *x, int
     int8_t *ximg = reinterpret_cast<int8_t *>(static_cast<char *>(s) + kScratchHeader);
     if (fused_input) {
         const bool qdiv = (dyn.quant_mode & HIPQ_FORM_DIV) != 0, qeven = (dyn.quant_mode & HIPQ_ROUND_HALF_EVEN) != 0;
+        // Prepared filters of at most 1 MiB: touched by the quantizer while it waits (variant 11 switches it off).
+        const size_t filter_bytes = packed_operand_bytes(g.oc, k);
+        const bool touching = wpacked && ctx->gemm_variant != 11 && filter_bytes <= (size_t(1) << 20);
+        const uint32_t *touch = touching ? reinterpret_cast<const uint32_t *>(wpacked) : nullptr;
+        const uint32_t touch_lines = touching ? static_cast<uint32_t>(filter_bytes / 128) : 0u;
 #define HIPQ_LAUNCH_CQ(D, E)                                                                                          \
     hipLaunchKernelGGL((conv_quantize_pack_image_kernel<D, E>), dim3(static_cast<int>(pack_grid)), dim3(kConvThreads), 0, \
                        ctx->stream, dyn.x, g.c, g.h, g.w, g.ph, g.pw, dyn.flavor, g.nb, groups_per_cb, dyn.params,    \
-                       ctx->wait_error, ctx->wait_spin_limit, ximg, static_cast<int>(pixels))
+                       ctx->wait_error, ctx->wait_spin_limit, ximg, static_cast<int>(pixels), touch, touch_lines)
         if (qdiv && qeven)
             HIPQ_LAUNCH_CQ(true, 1);
         else if (qdiv)
