@@ -764,6 +764,35 @@ def main() -> int:
                                "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "algorithmic_bytes": nbytes}
         del w3, pw3
 
+        # the transposed decode shape (N=4096, K=11008: a down projection): 128 weight row blocks only, the case the
+        # skinny kernel's depth rule is for
+        n5, k5 = 4096, 11008
+        pw5 = [ctx.pack_rows(torch.randint(-128, 128, (n5, k5), generator=g, device="cuda", dtype=torch.int8))
+               for _ in range(8)]
+        sw5 = torch.rand(n5, generator=g, device="cuda") * 1e-3
+        for m5 in (1, 4):
+            pa5 = ctx.pack_rows(torch.randint(-128, 128, (m5, k5), generator=g, device="cuda", dtype=torch.int8))
+            sa5 = torch.rand(m5, generator=g, device="cuda") * 0.05 + 0.01
+            x5 = torch.randn(m5, k5, generator=g, device="cuda")
+            o5 = torch.empty(m5, n5, device="cuda")
+            c5 = [0]
+
+            def run_down_prepared():
+                c5[0] += 1
+                ctx.linear_packed_i8_f32(pa5, sa5, pw5[c5[0] % len(pw5)], sw5, None, m5, n5, k5, out=o5)
+
+            def run_down_forward():
+                c5[0] += 1
+                ctx.linear_dynamic_packed(x5, pw5[c5[0] % len(pw5)], sw5, None, per_token=True, out=o5)
+
+            nbytes = n5 * k5 + m5 * k5 + 4 * m5 * n5 + 4 * n5
+            for name, fn in ((f"gemv_m{m5}_n4096_k11008", run_down_prepared),
+                             (f"gemv_m{m5}_n4096_k11008_forward_from_f32", run_down_forward)):
+                ms = event_time_ms(fn, reps=100, warmup=10)
+                extra[name] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9,
+                               "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "algorithmic_bytes": nbytes}
+        del pw5
+
         # configs[3]: quantized Conv2d [32,256,14,14] (*) [256,256,3,3], stride 1, pad 1, fused bias + requant
         xc = [torch.randint(0, 256, (32, 256, 14, 14), generator=g, device="cuda", dtype=torch.uint8) for _ in range(8)]
         wc = torch.randint(-128, 128, (256, 256, 3, 3), generator=g, device="cuda", dtype=torch.int8)

@@ -214,7 +214,10 @@ def test_dynamic_forward_with_and_without_weight_line_touching(hipq, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 64, 16), (1, 11008, 4096), (4, 11008, 4096), (16, 11008, 4096), (32, 1024, 1040),
-                                   (7, 300, 11008), (3, 96, 16384), (5, 4096, 272)])
+                                   (7, 300, 11008), (3, 96, 16384), (5, 4096, 272),
+                                   # up to four rows in one launch (every workgroup quantizes the rows itself):
+                                   (2, 512, 8192), (1, 768, 16384), (3, 1000, 4608), (1, 4096, 11008), (2, 100, 2048),
+                                   (4, 33, 256), (2, 4096, 4096), (1, 64, 1024)])
 def test_decode_forward_per_token(hipq, m, n, k):
     """Per-token dynamic forward with M <= 32 rows (the decode shapes of configs[2] among them), from fp32
     activations: same bits as the per-row quantizer followed by the product on its output (both pinned to the oracle
@@ -235,6 +238,11 @@ def test_decode_forward_per_token(hipq, m, n, k):
             want = c.linear_packed_i8_f32(pq, ps, pw, sw, bias, m, n, k)
             c.synchronize()
             assert torch.equal(got, want), it
+            if it == 0:  # and without a bias
+                got = c.linear_dynamic_packed(x, pw, sw, None, per_token=True, mode=mode)
+                want = c.linear_packed_i8_f32(pq, ps, pw, sw, None, m, n, k)
+                c.synchronize()
+                assert torch.equal(got, want)
         xb = x.clone()
         xb[m - 1, 5] = float("inf")
         got = c.linear_dynamic_packed(xb, pw, sw, bias, per_token=True)

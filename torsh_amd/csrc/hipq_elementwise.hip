@@ -653,7 +653,11 @@ __global__ __launch_bounds__(kBlock) void dequantize_kernel(const InT *__restric
 // instead of a dense [rows, cols] matrix, so that a per-token Linear forward needs no packing pass.  The grid
 // then covers the rows up to a multiple of 32, and the padding - rows past the matrix, k past cols up to a
 // multiple of 128 - is written as zeros.
-template <int TPR, bool EVEN, bool PACKED = false>
+// KC: float4 per lane that stay in registers between the two phases (4: rows up to 4096 floats with a workgroup
+// per row; 16: up to 16384).  What does not fit is read again, one dependent round trip per 1024 floats in each phase,
+// which is what a long row costs (a single row of 11008 floats: 7.3 us with KC = 4, a round trip less per 4096 floats
+// with 16).
+template <int TPR, bool EVEN, bool PACKED = false, int KC = 4>
 __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *__restrict__ x, size_t rows,
                                                                    size_t cols, size_t ld, int flavor, int qmin,
                                                                    int qmax,
@@ -662,7 +666,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
                                                                    int32_t *__restrict__ out_zps,
                                                                    int32_t *__restrict__ out_status, int poison) {
     constexpr int kRowsPerBlock = kBlock / TPR;
-    constexpr int kCache = 4;
+    constexpr int kCache = KC;
     __shared__ float lds[2 * kBlock / kWave];
     const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
     const size_t row = size_t(blockIdx.x) * kRowsPerBlock + sub;
@@ -1558,7 +1562,22 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
 #define HIPQ_LAUNCH_ROWS(TPR, E, P, G)                                                                               \
     hipLaunchKernelGGL((quantize_per_row_kernel<TPR, E, P>), dim3(G), dim3(kBlock), 0, ctx->stream, x, rows, cols, ld, \
                        flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison)
-    if (cols > 1024) {
+    if (cols > 4096 && ld % 4 == 0) {
+        // long rows: four times the registers, so that up to 16384 floats are read once and all requested up front
+        const int grid = static_cast<int>(grid_rows);
+#define HIPQ_LAUNCH_LONG_ROWS(E, P)                                                                                   \
+    hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, E, P, 16>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, rows,   \
+                       cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison)
+        if (packed && even)
+            HIPQ_LAUNCH_LONG_ROWS(true, true);
+        else if (packed)
+            HIPQ_LAUNCH_LONG_ROWS(false, true);
+        else if (even)
+            HIPQ_LAUNCH_LONG_ROWS(true, false);
+        else
+            HIPQ_LAUNCH_LONG_ROWS(false, false);
+#undef HIPQ_LAUNCH_LONG_ROWS
+    } else if (cols > 1024) {
         const int grid = static_cast<int>(grid_rows);
         if (packed) {
             if (even)

@@ -484,6 +484,9 @@ __global__ __launch_bounds__(256) void gemm_i8_packed_kernel(const int8_t *__res
 // nothing else matters: one 32-row block of weights per workgroup, K split between the four waves, D stages of
 // one weight fragment (1 KiB, contiguous in HBM) and one activation fragment (L2 resident) per wave in flight.
 // The four partial 32x32 blocks are summed through LDS by wave 0, which runs the ordinary checked epilogue.
+// The loop runs in rounds of D stages for any number of k steps: stages past the last ask for an offset beyond the
+// buffers, which returns zeros without touching memory and adds nothing.  D is the host's choice by how many
+// workgroups there are (see launch_gemv_packed).
 template <int D, int EPI, bool EVEN>
 __global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__restrict__ PA, const int8_t *__restrict__ PW,
                                                              int M, int N, int K, GemmEpilogue ep) {
@@ -515,18 +518,21 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__res
     const int steps = KB / WK, voff = lane * 16;
     const int voffa = lane % 32 < M ? voff : 0x7fffffff;
     v4i fa[D], fb[D];
+    const int rounds_end = (steps + D - 1) / D * D;
     auto issue = [&](int s, int slot) {
         const int koff = s * (WK * 1024);
-        fa[slot] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, voffa, soa + koff, 0));
-        fb[slot] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, sow + koff, 0));
+        const bool real = s < steps;
+        fa[slot] = __builtin_bit_cast(
+            v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, real ? voffa : 0x7fffffff, real ? soa + koff : 0, 0));
+        fb[slot] = __builtin_bit_cast(
+            v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, real ? voff : 0x7fffffff, real ? sow + koff : 0, 0));
     };
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0;
-    // steps is a positive multiple of D (the host picks D so).
 #pragma unroll
     for (int u = 0; u < D; ++u) issue(u, u);
-    for (int s0 = D; s0 < steps; s0 += D) {
+    for (int s0 = D; s0 < rounds_end; s0 += D) {
 #pragma unroll
         for (int u = 0; u < D; ++u) {
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u], fb[u], acc, 0, 0, 0);
@@ -551,6 +557,190 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__res
     store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, 0, 0, lane, nn, swv, bv, sa0);
 }
 
+// The same product straight from fp32 activations of at most four rows (decode), per-row dynamic int8: one launch
+// instead of a quantizer and the product.  No workgroup depends on another: each one requests its first weight
+// fragments, then reads the rows itself (they are 16 KiB each and come out of the L2 for all but the first
+// workgroups), finds every row's range (waves by shuffles, the four waves through LDS), quantizes with the per-row
+// quantizer's own arithmetic (params_from_minmax, symmetric; division form; a row whose range is not finite gets a
+// NaN scale and zero codes) and leaves the codes in LDS in fragment order: [k block][half][row], 16 bytes each.
+// The main loop takes its activation fragments from there.  A thread holds 16 consecutive floats per row and chunk
+// of 4096 columns: MROWS * CH <= 4 chunks, i.e. at most 64 registers of data.  K % 16 == 0, x 16-byte aligned.
+// Rounds of D stages as in gemv_i8_packed_kernel.  fp32 output: out = acc * (s_a[m] * s_w[n]) (+ bias[n]), as
+// store_tile does it.  Every workgroup repeats the quantize arithmetic of all rows (16 values a thread and row at
+// K = 4096), which is why this pays for one or two rows only: N = 11008, K = 4096 from fp32, one launch against
+// the quantizer and the product: M = 1 11.7 / 14.7 us, M = 2 13.3 / 14.7, M = 3 15.4 / 14.8, M = 4 17.3 / 15.0.
+template <int D, bool EVEN, int MROWS, int CH>
+__global__ __launch_bounds__(256) void gemv_i8_packed_from_f32_kernel(const float *__restrict__ x,
+                                                                      const int8_t *__restrict__ PW, int M, int N, int K,
+                                                                      GemmEpilogue ep) {
+    static_assert(MROWS * CH <= 4, "at most 64 data registers per thread");
+    __shared__ __attribute__((aligned(16))) v4i red[3][4][kWave];
+    __shared__ __attribute__((aligned(16))) v4i codes[MROWS * CH * 256];
+    __shared__ float wave_mn[4][MROWS], wave_mx[4][MROWS];
+    constexpr int WK = 4;
+    const int KB = static_cast<int>(packed_k_blocks(K));
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int n = blockIdx.x * 32 + lane % 32;
+    // Weights first: nothing below depends on them, and they are what the launch waits for.
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PW), 0, 0x7fffffff, 0x00020000);
+    const int sow = (static_cast<int>(blockIdx.x) * KB + wave) * 1024, steps = KB / WK, voff = lane * 16;
+    const int rounds_end = (steps + D - 1) / D * D;
+    v4i fb[D];
+    auto issue = [&](int s, int slot) {
+        const bool real = s < steps;
+        fb[slot] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, real ? voff : 0x7fffffff,
+                                                                                 real ? sow + s * (WK * 1024) : 0, 0));
+    };
+#pragma unroll
+    for (int u = 0; u < D; ++u) issue(u, u);
+    float sw = 1.0f, b = 0.0f;
+    if (wave == 0) {
+        const int nc = n < N ? n : N - 1;
+        sw = ep.sw[nc];
+        if (ep.bias) b = ep.bias[nc];
+    }
+    // The rows: thread t holds floats [16 g, 16 g + 16) of every row for g = t + 256 c.
+    float4 v[MROWS][CH][4];
+    bool have[MROWS][CH];
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m)
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int k0 = (static_cast<int>(threadIdx.x) + 256 * c) * 16;
+            have[m][c] = m < M && k0 < K;
+            if (have[m][c]) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[m][c][i] = reinterpret_cast<const float4 *>(x + size_t(m) * K + k0)[i];
+            }
+        }
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+        float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            if (have[m][c]) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    mn = fminf(mn, fminf(fminf(v[m][c][i].x, v[m][c][i].y), fminf(v[m][c][i].z, v[m][c][i].w)));
+                    mx = fmaxf(mx, fmaxf(fmaxf(v[m][c][i].x, v[m][c][i].y), fmaxf(v[m][c][i].z, v[m][c][i].w)));
+                }
+            }
+        mn = wave_min(mn);
+        mx = wave_max(mx);
+        if (lane == 0) {
+            wave_mn[wave][m] = mn;
+            wave_mx[wave][m] = mx;
+        }
+    }
+    __syncthreads();
+    float sa[MROWS];
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+        const float mn = fminf(fminf(wave_mn[0][m], wave_mn[1][m]), fminf(wave_mn[2][m], wave_mn[3][m]));
+        const float mx = fmaxf(fmaxf(wave_mx[0][m], wave_mx[1][m]), fmaxf(wave_mx[2][m], wave_mx[3][m]));
+        float scale;
+        int zp;
+        const bool bad = params_from_minmax(mn, mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp) != HIPQ_SUCCESS;
+        sa[m] = bad ? __builtin_nanf("") : scale;
+        if (bad) scale = INFINITY;  // x / inf: 0 for finite x, NaN -> code 0 otherwise
+        const float inv = recip_for_div(scale), zpf = static_cast<float>(bad ? 0 : zp);
+        auto q = [&](float f) { return quantize_int<QFORM_DIV, EVEN>(f, scale, inv, zpf, -128, 127); };
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int g = static_cast<int>(threadIdx.x) + 256 * c;
+            if (m < M && g < KB * 2) {  // k past K up to the padded extent: zeros
+                v4i w = v4i{0, 0, 0, 0};
+                if (have[m][c]) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        w[i] = static_cast<int>(pack4(q(v[m][c][i].x), q(v[m][c][i].y), q(v[m][c][i].z), q(v[m][c][i].w)));
+                }
+                codes[g * MROWS + m] = w;
+            }
+        }
+    }
+    __syncthreads();
+    // Lane l of an activation fragment: row l % 32, bytes 16 * (l / 32) .. +15 of the k block; rows past M are zero.
+    const int row = lane % 32, half = lane / 32;
+    auto fragment = [&](int s) {
+        const int kb = wave + WK * s;
+        return (row < M && s < steps) ? codes[(kb * 2 + half) * MROWS + row] : v4i{0, 0, 0, 0};
+    };
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
+    for (int s0 = D; s0 < rounds_end; s0 += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fragment(s0 - D + u), fb[u], acc, 0, 0, 0);
+            issue(s0 + u, u);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < D; ++u)
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fragment(rounds_end - D + u), fb[u], acc, 0, 0, 0);
+    if (wave > 0) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) red[wave - 1][g][lane] = v4i{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    // Rows 0..3 of the block are registers 0..3 of lanes 0..31 (lane = output column).
+    const v4i t = red[0][0][lane] + red[1][0][lane] + red[2][0][lane];
+    if (lane < 32 && n < N) {
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) {
+            if (m >= M) continue;
+            float o = static_cast<float>(acc[m] + t[m]) * (sa[m] * sw);
+            if (ep.bias) o = o + b;
+            __builtin_nontemporal_store(o, static_cast<float *>(ep.out) + size_t(m) * N + n);
+        }
+    }
+}
+
+// Whether the decode forward from fp32 can take the kernel above, and its launch.  Returns false when the shape is
+// left to the two launches (per-row quantizer into the packed layout, then gemv_i8_packed_kernel).
+template <bool EVEN>
+static bool launch_gemv_packed_from_f32(hipq_ctx *ctx, const float *x, const int8_t *pw, size_t m, size_t n, size_t k,
+                                        const GemmEpilogue &ep, int32_t *rc) {
+    const size_t KB = packed_k_blocks(k);
+    const size_t chunks = (KB * 2 + 255) / 256;  // 16-float groups per thread and row
+    if (m == 0 || m > 2 || k % 16 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) != 0 || KB < 16) return false;
+    const int mrows = static_cast<int>(m), ch = chunks <= 1 ? 1 : (chunks == 2 ? 2 : 4);
+    if (chunks > 4 || mrows * ch > 4) return false;
+    const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
+    const int row_blocks = (N + 31) / 32;
+    const int depth = row_blocks >= 200 ? 4 : (row_blocks >= 100 ? 8 : 16);  // as launch_gemv_packed
+    const dim3 grid(row_blocks);
+#define HIPQ_LAUNCH_GFD(DEPTH, MR, C)                                                                              \
+    hipLaunchKernelGGL((gemv_i8_packed_from_f32_kernel<DEPTH, EVEN, MR, C>), grid, dim3(256), 0, ctx->stream, x, pw, M, N, \
+                       K, ep)
+#define HIPQ_LAUNCH_GF(MR, C)              \
+    do {                                   \
+        if (depth == 4)                    \
+            HIPQ_LAUNCH_GFD(4, MR, C);     \
+        else if (depth == 8)               \
+            HIPQ_LAUNCH_GFD(8, MR, C);     \
+        else                               \
+            HIPQ_LAUNCH_GFD(16, MR, C);    \
+    } while (0)
+    if (mrows == 1 && ch == 1)
+        HIPQ_LAUNCH_GF(1, 1);
+    else if (mrows == 1 && ch == 2)
+        HIPQ_LAUNCH_GF(1, 2);
+    else if (mrows == 1)
+        HIPQ_LAUNCH_GF(1, 4);
+    else if (ch == 1)
+        HIPQ_LAUNCH_GF(2, 1);
+    else
+        HIPQ_LAUNCH_GF(2, 2);
+#undef HIPQ_LAUNCH_GF
+#undef HIPQ_LAUNCH_GFD
+    *rc = check_launch("gemv_i8 (packed, from fp32)");
+    return true;
+}
+
 template <int D, int EPI, bool EVEN>
 static int32_t launch_gemv_packed_d(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                                     const GemmEpilogue &ep) {
@@ -559,17 +749,31 @@ static int32_t launch_gemv_packed_d(hipq_ctx *ctx, const int8_t *pa, const int8_
     return check_launch("gemv_i8 (packed)");
 }
 
-// Register depth 4 where it divides the k blocks per wave (else 2 or 1).  Measured at N = 11008, K = 4096: depth
-// 4 gives 10.2 us, 2 11.9, 8 10.9, 16 11.0, 32 12.3 - with more in flight the workgroups' streams through their
-// 128 KiB row blocks interleave more finely in memory and the stream as a whole gets slower, not faster.  Starting
-// the workgroups on different K steps does not help either (10.7 against 10.5 us).
+// Stages in flight per wave (1 KiB of weights each) by the number of workgroups, i.e. weight row blocks.  What
+// streams well is 5-6 MB in flight over the chip.  Measured (M = 4, us; depth 2 / 4 / 8 / 16):
+//   N = 11008, K = 4096  (344 workgroups):  13.0 / 10.9 / 11.7 / 11.9 - with more in flight the workgroups' streams
+//     through their 128 KiB row blocks interleave more finely in memory and the stream as a whole gets slower;
+//   N = 8192,  K = 2048  (256):   5.6 /  5.5 /  5.7 /  5.6
+//   N = 4096,  K = 11008 (128):  24.2 / 16.3 / 12.5 / 12.7   (depth 2 was all that divided its 86 steps: 33.8 us)
+//   N = 4096,  K = 4096  (128):   7.5 /  6.0 /  5.5 /  5.4
+//   N = 2048,  K = 8192  (64):   11.8 /  8.4 /  6.8 /  6.5
+// Splitting K over several workgroups per row block instead (partials written through to memory, a ticket per row
+// block, the last to arrive sums and stores) was built and measured: level with depth 8 at N = 4096, K = 11008
+// (12.3 us), 1.5-2 us slower at 16.8 MB of weights - the hand-over costs two trips through device-coherent memory.
+// Starting the workgroups on different K steps does not help either (10.7 against 10.5 us).
 template <int EPI, bool EVEN>
 static int32_t launch_gemv_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                                   const GemmEpilogue &ep) {
-    const int steps = static_cast<int>(packed_k_blocks(size_t(K))) / 4;
-    if (steps % 4 == 0) return launch_gemv_packed_d<4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-    if (steps % 2 == 0) return launch_gemv_packed_d<2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-    return launch_gemv_packed_d<1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    const int steps = static_cast<int>(packed_k_blocks(size_t(K))) / 4, row_blocks = (N + 31) / 32;
+    int depth = row_blocks >= 200 ? 4 : (row_blocks >= 100 ? 8 : 16);
+    while (depth > 1 && depth > steps) depth /= 2;
+    switch (depth) {
+    case 16: return launch_gemv_packed_d<16, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    case 8: return launch_gemv_packed_d<8, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    case 4: return launch_gemv_packed_d<4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    case 2: return launch_gemv_packed_d<2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    default: return launch_gemv_packed_d<1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    }
 }
 
 // Row-major int8 [rows, k] -> packed.  One wave per fragment: a lane copies the 16 bytes of its

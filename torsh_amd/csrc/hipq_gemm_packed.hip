@@ -235,6 +235,14 @@ int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t pe
     float *row_scales = reinterpret_cast<float *>(base + L.scales);
     int8_t *pa = reinterpret_cast<int8_t *>(base + L.packed);
     if (per_token) {
+        // Decode, one or two rows: one launch, every workgroup quantizes the rows itself (variant 6 keeps the two).
+        if (m <= 2 && ctx->gemm_variant != 6) {
+            GemmEpilogue ep{nullptr, 1, w_scales, bias, 1.0f, 0, out};
+            const bool fused = (mode & HIPQ_ROUND_HALF_EVEN)
+                                   ? launch_gemv_packed_from_f32<true>(ctx, x, w_packed, m, n, k, ep, &rc)
+                                   : launch_gemv_packed_from_f32<false>(ctx, x, w_packed, m, n, k, ep, &rc);
+            if (fused) return rc;
+        }
         // one pass over the activations: the per-row quantizer writes the packed operand itself
         rc = quantize_activations_per_row(ctx, x, m, k, mode & HIPQ_ROUND_HALF_EVEN, pa, row_scales, /*packed=*/true);
         if (rc) return rc;
