@@ -788,7 +788,7 @@ def main() -> int:
             nbytes = n5 * k5 + m5 * k5 + 4 * m5 * n5 + 4 * n5
             for name, fn in ((f"gemv_m{m5}_n4096_k11008", run_down_prepared),
                              (f"gemv_m{m5}_n4096_k11008_forward_from_f32", run_down_forward)):
-                ms = event_time_ms(fn, reps=100, warmup=10)
+                ms = event_time_ms(fn, reps=100, warmup=40)
                 extra[name] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9,
                                "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "algorithmic_bytes": nbytes}
         del pw5
