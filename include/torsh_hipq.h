@@ -320,10 +320,12 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
  * for every later call on this context wherever the shape allows it (0 = automatic choice, the
  * default; 1-3 one-tile-per-workgroup forms, 5-8 persistent forms, 10 register-staged form); 6 also
  * makes the dynamic per-tensor activation quantizer of the Linear forwards run as two launches (range
- * partials, then a quantizer that folds them) where it would run as one; 9 and 11 leave the choice
- * automatic and switch off, on prepared operands, the two-workgroups-per-compute-unit form of the
- * GEMM (9) and the touching of weight / filter lines by the one-launch activation quantizers of the
- * dynamic Linear and Conv2d forwards while their grids wait for the range (11).
+ * partials, then a quantizer that folds them) where it would run as one, and the per-token forward
+ * of one or two rows as a quantizer and a product where it would be one kernel; 9 and 11 leave the
+ * choice automatic and switch off, on prepared operands, the forms of the GEMM that are picked by
+ * occupancy - two workgroups per compute unit, the weight-streaming kernel for 33..128 rows - (9)
+ * and the touching of weight / filter lines by the one-launch activation quantizers of the dynamic
+ * Linear and Conv2d forwards while their grids wait for the range (11).
  * Results do not depend on it; the parity tests use it to run every form on the same inputs. */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
 /* Test hook with no counterpart in the reference.  Two kernels couple their waves through device

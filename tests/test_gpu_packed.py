@@ -51,6 +51,7 @@ SHAPES = [
     (127, 129, 4096), (512, 256, 1024), (5, 300, 48), (256, 512, 16), (33, 1000, 2048), (9, 40, 1001), (3, 5, 7),
     (129, 65, 512), (200, 96, 768), (256, 128, 2304), (96, 200, 11008),
     (2100, 1100, 512), (4100, 600, 272),  # more tiles than compute units: two workgroups per compute unit
+    (65, 4096, 4096), (50, 300, 1040), (100, 7000, 512), (128, 96, 80),  # 33..128 rows: the skinny kernel's 2..4 row blocks
 ]
 
 
@@ -177,6 +178,37 @@ def test_linear_packed_many_tiles_matches_row_major(ctx, hipq, m, n, k):
     got = ctx.linear_packed_i8_f32(ctx.pack_rows(a), sa, ctx.pack_rows(w), sw, bias, m, n, k)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 4096, 4096), (128, 2048, 8192), (96, 1000, 4096), (33, 11008, 512), (64, 300, 11008),
+                                   (40, 64, 48)])
+def test_weight_streaming_kernel_for_33_to_128_rows_matches_tiled(hipq, m, n, k):
+    """33..128 activation rows on prepared operands take a kernel that streams one 32-row block of weights per
+    workgroup against two to four activation row blocks; variant 9 keeps the 128 x 64 tiles.  Same bits for the
+    fp32 epilogue (per-row scales, bias), the requantizing one (both roundings) and the raw accumulators."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(m * 3 + n + k)
+        a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+        w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+        pa, pw = c.pack_rows(a), c.pack_rows(w)
+        sa = torch.rand(m, generator=g, device="cuda") * 1e-2 + 1e-3
+        sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+        bias = torch.randn(n, generator=g, device="cuda")
+        got = {}
+        for variant in (0, 9):
+            c.set_gemm_kernel_variant(variant)
+            got[variant] = (c.linear_packed_i8_f32(pa, sa, pw, sw, bias, m, n, k),
+                            c.linear_packed_i8_i8(pa, sa, pw, sw, bias, m, n, k, 0.31, -3),
+                            c.linear_packed_i8_i8(pa, sa[:1], pw, sw, None, m, n, k, 0.05, 7, mode=hipq.ROUND_HALF_EVEN),
+                            c.gemm_packed_i8_i32(pa, pw, m, n, k))
+            c.synchronize()
+        for x, y in zip(got[0], got[9]):
+            assert torch.equal(x, y)
+        want = a.double() @ w.double().T  # exact: |acc| < 2^53
+        assert torch.equal(got[0][3], want.to(torch.int32))
+    finally:
+        c.close()
 
 
 @pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (256, 4096, 1024), (128, 2048, 4096), (384, 1024, 8192),

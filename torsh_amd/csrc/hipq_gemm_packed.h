@@ -557,6 +557,101 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__res
     store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, 0, 0, lane, nn, swv, bv, sa0);
 }
 
+// The same for 33 to 128 activation rows (RB = 2..4 row blocks; a batch of decodes, a short prefill): still one
+// 32-row block of weights per workgroup and K split between the four waves, each of which multiplies its weight
+// fragment with the RB activation fragments of the k block (L2 resident: RB KiB a step against 1 KiB from HBM).
+// The weights are the only operand that comes from memory, and they are read once; the 128 x 64 tiles of the general
+// kernel give such shapes 64-170 workgroups with 786 KB of operands each, and take as long for 64 rows as for 512.
+// Wave b ends up owning row block b: the others park their partials of it in LDS.
+template <int D, int RB, int EPI, bool EVEN>
+__global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__restrict__ PA, const int8_t *__restrict__ PW,
+                                                               int M, int N, int K, GemmEpilogue ep) {
+    static_assert(RB >= 2 && RB <= 4, "two to four activation row blocks");
+    __shared__ __attribute__((aligned(16))) v4i red[3][RB][4][kWave];
+    constexpr int WK = 4;
+    const int KB = static_cast<int>(packed_k_blocks(K));
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    float swv[1], bv[1], sa0 = 1.0f;
+    int nn[1];
+    nn[0] = static_cast<int>(blockIdx.x) * 32 + lane % 32;
+    swv[0] = 1.0f;
+    bv[0] = 0.0f;
+    if constexpr (EPI != EPI_I32) {
+        if (wave < RB) {
+            const int nc = nn[0] < N ? nn[0] : N - 1;
+            swv[0] = ep.sw[nc];
+            if (ep.bias) bv[0] = ep.bias[nc];
+            if (!ep.sa_per_row) sa0 = ep.sa ? ep.sa[0] : ep.sa_scalar;
+        }
+    }
+    const __amdgpu_buffer_rsrc_t ra =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PA), 0, RB * KB * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PW), 0, 0x7fffffff, 0x00020000);
+    const int sow = (static_cast<int>(blockIdx.x) * KB + wave) * 1024;
+    const int steps = KB / WK, voff = lane * 16;
+    int soa[RB], voffa[RB];  // rows past M read zeros without touching memory
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+        soa[i] = (i * KB + wave) * 1024;
+        voffa[i] = i * 32 + lane % 32 < M ? voff : 0x7fffffff;
+    }
+    v4i fa[D][RB], fb[D];
+    const int rounds_end = (steps + D - 1) / D * D;
+    auto issue = [&](int s, int slot) {
+        const int koff = s * (WK * 1024);
+        const bool real = s < steps;
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+            fa[slot][i] = __builtin_bit_cast(
+                v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, real ? voffa[i] : 0x7fffffff, real ? soa[i] + koff : 0, 0));
+        fb[slot] = __builtin_bit_cast(
+            v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, real ? voff : 0x7fffffff, real ? sow + koff : 0, 0));
+    };
+    v16i acc[RB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+#pragma unroll
+    for (int u = 0; u < D; ++u) issue(u, u);
+    for (int s0 = D; s0 < rounds_end; s0 += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+#pragma unroll
+            for (int i = 0; i < RB; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u][i], fb[u], acc[i], 0, 0, 0);
+            issue(s0 + u, u);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < D; ++u)
+#pragma unroll
+        for (int i = 0; i < RB; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u][i], fb[u], acc[i], 0, 0, 0);
+    // Row block b goes to wave b; wave w parks its partial of it in slot (w - b - 1) mod 4 of the three.
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        if (b == wave) continue;
+        const int slot = (wave - b + 3) % 4;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            red[slot][b][g][lane] = v4i{acc[b][4 * g], acc[b][4 * g + 1], acc[b][4 * g + 2], acc[b][4 * g + 3]};
+    }
+    __syncthreads();
+    if (wave >= RB) return;
+    v16i own[1][1];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        if (b != wave) continue;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const v4i t = red[0][b][g][lane] + red[1][b][g][lane] + red[2][b][g][lane];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) own[0][0][4 * g + c] = acc[b][4 * g + c] + t[c];
+        }
+    }
+    store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, wave * 32, 0, lane, nn, swv, bv, sa0);
+}
+
 // The same product straight from fp32 activations of at most four rows (decode), per-row dynamic int8: one launch
 // instead of a quantizer and the product.  No workgroup depends on another: each one requests its first weight
 // fragments, then reads the rows itself (they are 16 KiB each and come out of the L2 for all but the first
@@ -761,6 +856,28 @@ static int32_t launch_gemv_packed_d(hipq_ctx *ctx, const int8_t *pa, const int8_
 // block, the last to arrive sums and stores) was built and measured: level with depth 8 at N = 4096, K = 11008
 // (12.3 us), 1.5-2 us slower at 16.8 MB of weights - the hand-over costs two trips through device-coherent memory.
 // Starting the workgroups on different K steps does not help either (10.7 against 10.5 us).
+template <int RB, int EPI, bool EVEN>
+static int32_t launch_skinny_packed_rb(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
+                                       const GemmEpilogue &ep) {
+    const int row_blocks = (N + 31) / 32;
+    const dim3 grid(row_blocks);
+    // (depth 8 at most: a stage is RB + 1 fragments of four registers)
+    if (row_blocks >= 200)
+        hipLaunchKernelGGL((skinny_i8_packed_kernel<4, RB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K, ep);
+    else
+        hipLaunchKernelGGL((skinny_i8_packed_kernel<8, RB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K, ep);
+    return check_launch("skinny_i8 (packed)");
+}
+
+// 33..128 activation rows.
+template <int EPI, bool EVEN>
+static int32_t launch_skinny_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
+                                    const GemmEpilogue &ep) {
+    if (M <= 64) return launch_skinny_packed_rb<2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    if (M <= 96) return launch_skinny_packed_rb<3, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    return launch_skinny_packed_rb<4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+}
+
 template <int EPI, bool EVEN>
 static int32_t launch_gemv_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                                   const GemmEpilogue &ep) {
@@ -835,6 +952,20 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
     const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
     const int steps = static_cast<int>(packed_k_blocks(k)) / 4;
     if (M <= 32) return launch_gemv_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // one row block of activations
+    // Up to four: the weights streamed once per 32-row block, as above, where that beats the tiled kernel (variant
+    // 9: the tiled kernel always).  Every workgroup pulls all activation fragments through its compute unit's
+    // vector-memory path, RB KiB for each KiB of weights, so the more row blocks of either operand, the less it
+    // pays.  Measured, skinny / tiled in us:   N = K = 4096          N = 11008, K = 4096    N = 4096, K = 11264
+    //                                 M = 48    8.4 / 12.1            15.6 / 17.0            19.2 / 30.6
+    //                                 M = 64    9.1 / 11.8            17.5 / 16.9            21.2 / 30.5
+    //                                 M = 96   11.5 / 12.6            21.4 / 18.4            25.9 / 34.7
+    //                                 M = 128  13.4 / 12.2            25.6 / 19.0            30.4 / 36.9
+    // (the tiled kernel's depth makes no difference at these shapes: 2 / 4 / 8 stages within 0.5 us.)
+    if (M <= 128 && ctx->gemm_variant != 9) {
+        const int row_blocks = (N + 31) / 32;
+        if (M <= 64 || (row_blocks <= 200 && (M <= 96 || steps >= 64)))
+            return launch_skinny_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    }
     if constexpr (EPI == EPI_F32 && !EVEN) {
         // Phase stamps (hipq_ctx_set_trace_buffer): the depth-2 fp32 form only, and only when the buffer holds
         // every wave's record.
