@@ -1714,7 +1714,11 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
     const size_t cap = size_t(ctx->num_cus) * 8;
     int grid = static_cast<int>(blocks < cap ? blocks : cap);
     const bool div = (mode & HIPQ_FORM_DIV) != 0, even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
-    const int fpw = blocks <= resident_workgroups(ctx, false) ? 1 : 4;
+    // Fragments per wave of the one-launch form: one while that gives a workgroup per compute unit at most, two up to
+    // four times that (fewer workgroups to meet: 512 x 4096 7.36 -> 7.27 us, 1024 x 4096 9.74 -> 9.18 us, the Linear
+    // step at 512 rows -0.3 us), else four; more where the grid would not be resident otherwise.
+    int fpw = blocks <= size_t(ctx->num_cus) ? 1 : (blocks <= size_t(ctx->num_cus) * 4 ? 2 : 4);
+    while (fpw < 4 && (blocks + fpw - 1) / fpw > resident_workgroups(ctx, false)) fpw *= 2;
     const size_t q1_blocks = (blocks + fpw - 1) / fpw;
     if (dynamic && packed && ctx->gemm_variant != 6 && q1_blocks <= resident_workgroups(ctx, fpw == 4) && cols % 16 == 0 &&
         (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (fpw == 1 || four_wide_workgroups_fit(ctx))) {
@@ -1736,6 +1740,8 @@ int32_t hipq::quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, siz
     } while (0)
         if (fpw == 1)
             HIPQ_LAUNCH_Q1_MODE(1);
+        else if (fpw == 2)
+            HIPQ_LAUNCH_Q1_MODE(2);
         else
             HIPQ_LAUNCH_Q1_MODE(4);
 #undef HIPQ_LAUNCH_Q1_MODE
