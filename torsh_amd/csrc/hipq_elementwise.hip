@@ -1038,13 +1038,12 @@ __global__ __launch_bounds__(kBlock) void dequantize_per_channel_kernel(const in
 // of two and by 32-bit divisions where the index fits.
 struct ChannelOfVector {
     size_t vpc, channels;  // vectors per channel run
-    int vpc_shift, ch_shift;
+    int vpc_shift;
     bool vpc_pow2, ch_pow2, small;
     __device__ ChannelOfVector(size_t inner, size_t channels_, size_t nvec) : vpc(inner / 4), channels(channels_) {
         vpc_pow2 = (vpc & (vpc - 1)) == 0;
         ch_pow2 = (channels & (channels - 1)) == 0;
         vpc_shift = __builtin_ffsll(static_cast<long long>(vpc)) - 1;
-        ch_shift = __builtin_ffsll(static_cast<long long>(channels)) - 1;
         small = nvec < (size_t(1) << 32);
     }
     __device__ size_t operator()(size_t j) const {
