@@ -52,6 +52,7 @@ SHAPES = [
     (129, 65, 512), (200, 96, 768), (256, 128, 2304), (96, 200, 11008),
     (2100, 1100, 512), (4100, 600, 272),  # more tiles than compute units: two workgroups per compute unit
     (65, 4096, 4096), (50, 300, 1040), (100, 7000, 512), (128, 96, 80),  # 33..128 rows: the skinny kernel's 2..4 row blocks
+    (17, 9700, 96), (40, 10000, 272), (64, 9632, 1040), (1, 10016, 64),  # >= 300 weight row blocks: two per workgroup (odd counts too)
 ]
 
 

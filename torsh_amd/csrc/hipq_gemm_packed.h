@@ -557,28 +557,31 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__res
     store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, 0, 0, lane, nn, swv, bv, sa0);
 }
 
-// The same for 33 to 128 activation rows (RB = 2..4 row blocks; a batch of decodes, a short prefill): still one
-// 32-row block of weights per workgroup and K split between the four waves, each of which multiplies its weight
-// fragment with the RB activation fragments of the k block (L2 resident: RB KiB a step against 1 KiB from HBM).
-// The weights are the only operand that comes from memory, and they are read once; the 128 x 64 tiles of the general
-// kernel give such shapes 64-170 workgroups with 786 KB of operands each, and take as long for 64 rows as for 512.
-// Wave b ends up owning row block b: the others park their partials of it in LDS.
-template <int D, int RB, int EPI, bool EVEN>
+// The same for up to 128 activation rows (RB = 1..4 row blocks; a batch of decodes, a short prefill) and TNB = 1 or 2
+// 32-row blocks of weights per workgroup, RB * TNB <= 4 output blocks: K split between the four waves, each of which
+// multiplies its TNB weight fragments with the RB activation fragments of the k block (L2 resident: RB KiB a step
+// against TNB KiB from HBM).  The weights are the only operand that comes from memory, and they are read once; the
+// 128 x 64 tiles of the general kernel give such shapes 64-170 workgroups with 786 KB of operands each, and take as
+// long for 64 rows as for 512.  Wave b ends up owning output block b: the others park their partials of it in LDS.
+template <int D, int RB, int TNB, int EPI, bool EVEN>
 __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__restrict__ PA, const int8_t *__restrict__ PW,
                                                                int M, int N, int K, GemmEpilogue ep) {
-    static_assert(RB >= 2 && RB <= 4, "two to four activation row blocks");
-    __shared__ __attribute__((aligned(16))) v4i red[3][RB][4][kWave];
+    constexpr int NBLK = RB * TNB;  // 32 x 32 output blocks of the workgroup: block b = (row block b / TNB, column block b % TNB)
+    static_assert(NBLK >= 2 && NBLK <= 4, "at most one output block per wave");
+    __shared__ __attribute__((aligned(16))) v4i red[3][NBLK][4][kWave];
     constexpr int WK = 4;
     const int KB = static_cast<int>(packed_k_blocks(K));
+    const int rbW = (N + 31) / 32;
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // Epilogue operands of the block this wave will own.
     float swv[1], bv[1], sa0 = 1.0f;
     int nn[1];
-    nn[0] = static_cast<int>(blockIdx.x) * 32 + lane % 32;
+    nn[0] = (static_cast<int>(blockIdx.x) * TNB + wave % TNB) * 32 + lane % 32;
     swv[0] = 1.0f;
     bv[0] = 0.0f;
     if constexpr (EPI != EPI_I32) {
-        if (wave < RB) {
+        if (wave < NBLK) {
             const int nc = nn[0] < N ? nn[0] : N - 1;
             swv[0] = ep.sw[nc];
             if (ep.bias) bv[0] = ep.bias[nc];
@@ -588,15 +591,20 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
     const __amdgpu_buffer_rsrc_t ra =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PA), 0, RB * KB * 1024, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PW), 0, 0x7fffffff, 0x00020000);
-    const int sow = (static_cast<int>(blockIdx.x) * KB + wave) * 1024;
     const int steps = KB / WK, voff = lane * 16;
-    int soa[RB], voffa[RB];  // rows past M read zeros without touching memory
+    int soa[RB], voffa[RB], sow[TNB];  // rows past M read zeros without touching memory
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
         soa[i] = (i * KB + wave) * 1024;
         voffa[i] = i * 32 + lane % 32 < M ? voff : 0x7fffffff;
     }
-    v4i fa[D][RB], fb[D];
+#pragma unroll
+    for (int j = 0; j < TNB; ++j) {
+        int rb = static_cast<int>(blockIdx.x) * TNB + j;
+        rb = rb < rbW ? rb : rbW - 1;  // a column block past the matrix repeats the last one; its outputs are not stored
+        sow[j] = (rb * KB + wave) * 1024;
+    }
+    v4i fa[D][RB], fb[D][TNB];
     const int rounds_end = (steps + D - 1) / D * D;
     auto issue = [&](int s, int slot) {
         const int koff = s * (WK * 1024);
@@ -605,31 +613,37 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
         for (int i = 0; i < RB; ++i)
             fa[slot][i] = __builtin_bit_cast(
                 v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, real ? voffa[i] : 0x7fffffff, real ? soa[i] + koff : 0, 0));
-        fb[slot] = __builtin_bit_cast(
-            v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, real ? voff : 0x7fffffff, real ? sow + koff : 0, 0));
+#pragma unroll
+        for (int j = 0; j < TNB; ++j)
+            fb[slot][j] = __builtin_bit_cast(
+                v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, real ? voff : 0x7fffffff, real ? sow[j] + koff : 0, 0));
     };
-    v16i acc[RB];
+    v16i acc[NBLK];
 #pragma unroll
-    for (int i = 0; i < RB; ++i)
+    for (int b = 0; b < NBLK; ++b)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+        for (int r = 0; r < 16; ++r) acc[b][r] = 0;
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int j = 0; j < TNB; ++j)
+                acc[i * TNB + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[slot][i], fb[slot][j], acc[i * TNB + j], 0, 0, 0);
+    };
 #pragma unroll
     for (int u = 0; u < D; ++u) issue(u, u);
     for (int s0 = D; s0 < rounds_end; s0 += D) {
 #pragma unroll
         for (int u = 0; u < D; ++u) {
-#pragma unroll
-            for (int i = 0; i < RB; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u][i], fb[u], acc[i], 0, 0, 0);
+            multiply(u);
             issue(s0 + u, u);
         }
     }
 #pragma unroll
-    for (int u = 0; u < D; ++u)
+    for (int u = 0; u < D; ++u) multiply(u);
+    // Output block b goes to wave b; wave w parks its partial of it in slot (w - b - 1) mod 4 of the three.
 #pragma unroll
-        for (int i = 0; i < RB; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u][i], fb[u], acc[i], 0, 0, 0);
-    // Row block b goes to wave b; wave w parks its partial of it in slot (w - b - 1) mod 4 of the three.
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
+    for (int b = 0; b < NBLK; ++b) {
         if (b == wave) continue;
         const int slot = (wave - b + 3) % 4;
 #pragma unroll
@@ -637,10 +651,10 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
             red[slot][b][g][lane] = v4i{acc[b][4 * g], acc[b][4 * g + 1], acc[b][4 * g + 2], acc[b][4 * g + 3]};
     }
     __syncthreads();
-    if (wave >= RB) return;
+    if (wave >= NBLK) return;
     v16i own[1][1];
 #pragma unroll
-    for (int b = 0; b < RB; ++b) {
+    for (int b = 0; b < NBLK; ++b) {
         if (b != wave) continue;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -649,7 +663,7 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
             for (int c = 0; c < 4; ++c) own[0][0][4 * g + c] = acc[b][4 * g + c] + t[c];
         }
     }
-    store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, wave * 32, 0, lane, nn, swv, bv, sa0);
+    store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, (wave / TNB) * 32, 0, lane, nn, swv, bv, sa0);
 }
 
 // The same product straight from fp32 activations of at most four rows (decode), per-row dynamic int8: one launch
@@ -856,26 +870,40 @@ static int32_t launch_gemv_packed_d(hipq_ctx *ctx, const int8_t *pa, const int8_
 // block, the last to arrive sums and stores) was built and measured: level with depth 8 at N = 4096, K = 11008
 // (12.3 us), 1.5-2 us slower at 16.8 MB of weights - the hand-over costs two trips through device-coherent memory.
 // Starting the workgroups on different K steps does not help either (10.7 against 10.5 us).
-template <int RB, int EPI, bool EVEN>
+template <int RB, int TNB, int EPI, bool EVEN>
 static int32_t launch_skinny_packed_rb(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                                        const GemmEpilogue &ep) {
-    const int row_blocks = (N + 31) / 32;
-    const dim3 grid(row_blocks);
-    // (depth 8 at most: a stage is RB + 1 fragments of four registers)
-    if (row_blocks >= 200)
-        hipLaunchKernelGGL((skinny_i8_packed_kernel<4, RB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K, ep);
+    const int groups = ((N + 31) / 32 + TNB - 1) / TNB;
+    const dim3 grid(groups);
+    // (depth 8 at most: a stage is RB + TNB fragments of four registers)
+    if (groups >= 200)
+        hipLaunchKernelGGL((skinny_i8_packed_kernel<4, RB, TNB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K,
+                           ep);
     else
-        hipLaunchKernelGGL((skinny_i8_packed_kernel<8, RB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K, ep);
+        hipLaunchKernelGGL((skinny_i8_packed_kernel<8, RB, TNB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K,
+                           ep);
     return check_launch("skinny_i8 (packed)");
 }
 
-// 33..128 activation rows.
+// Up to 128 activation rows on the weight-streaming kernel.  From 300 weight row blocks on a workgroup takes two of
+// them (up to two activation row blocks): half the activation traffic per weight byte, and still more than one
+// workgroup per compute unit.  One / two weight row blocks per workgroup, us:
+//   N = 11008, K = 4096: M = 1 10.4 / 10.25, 16 11.3 / 10.9, 32 13.4 / 12.0, 33 14.9 / 12.9, 64 17.5 / 14.2
+//   N = 32000, K = 4096: M = 1 26.6 / 24.0 (5.5 TB/s), 32 28.5 / 25.6, 64 35.9 / 28.6;   N = 128256: M = 1 87.6 / 86.1
+//   N = 8192,  K = 2048: M = 1 4.7 / 5.1, 32 5.4 / 6.2, 64 7.3 / 7.9 (and the same below that); four per workgroup: slower.
+constexpr int kTwoBlockRowBlocks = 300;
+
 template <int EPI, bool EVEN>
 static int32_t launch_skinny_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                                     const GemmEpilogue &ep) {
-    if (M <= 64) return launch_skinny_packed_rb<2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-    if (M <= 96) return launch_skinny_packed_rb<3, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-    return launch_skinny_packed_rb<4, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    const bool two = (N + 31) / 32 >= kTwoBlockRowBlocks;
+    if (M <= 32) return launch_skinny_packed_rb<1, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // (callers: `two` only)
+    if (M <= 64) {
+        if (two) return launch_skinny_packed_rb<2, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+        return launch_skinny_packed_rb<2, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    }
+    if (M <= 96) return launch_skinny_packed_rb<3, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    return launch_skinny_packed_rb<4, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
 }
 
 template <int EPI, bool EVEN>
@@ -951,7 +979,11 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
                                   const GemmEpilogue &ep) {
     const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
     const int steps = static_cast<int>(packed_k_blocks(k)) / 4;
-    if (M <= 32) return launch_gemv_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // one row block of activations
+    if (M <= 32) {  // one row block of activations
+        if ((N + 31) / 32 >= kTwoBlockRowBlocks && ctx->gemm_variant != 9)
+            return launch_skinny_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+        return launch_gemv_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    }
     // Up to four: the weights streamed once per 32-row block, as above, where that beats the tiled kernel (variant
     // 9: the tiled kernel always).  Every workgroup pulls all activation fragments through its compute unit's
     // vector-memory path, RB KiB for each KiB of weights, so the more row blocks of either operand, the less it
