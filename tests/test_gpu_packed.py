@@ -182,11 +182,13 @@ def test_linear_packed_many_tiles_matches_row_major(ctx, hipq, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(65, 4096, 4096), (128, 2048, 8192), (96, 1000, 4096), (33, 11008, 512), (64, 300, 11008),
-                                   (40, 64, 48)])
-def test_weight_streaming_kernel_for_33_to_128_rows_matches_tiled(hipq, m, n, k):
-    """33..128 activation rows on prepared operands take a kernel that streams one 32-row block of weights per
-    workgroup against two to four activation row blocks; variant 9 keeps the 128 x 64 tiles.  Same bits for the
-    fp32 epilogue (per-row scales, bias), the requantizing one (both roundings) and the raw accumulators."""
+                                   (40, 64, 48), (160, 1024, 512), (256, 4096, 256), (384, 2304, 768), (130, 100, 1040)])
+def test_weight_streaming_kernel_matches_tiled(hipq, m, n, k):
+    """From 33 activation rows up to as many as make one round of 64 x 64 tiles over the compute units, prepared
+    operands take the weight-streaming kernel (one or two 32-row blocks of weights per workgroup against two
+    activation row blocks, the row-block pair picked by the grid's second dimension); variant 9 keeps the 128 x 64
+    tiles.  Same bits for the fp32 epilogue (per-row scales, bias), the requantizing one (both roundings) and the raw
+    accumulators."""
     c = hipq.Context(0)
     try:
         g = torch.Generator(device="cuda").manual_seed(m * 3 + n + k)

@@ -557,12 +557,13 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_kernel(const int8_t *__res
     store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, 0, 0, lane, nn, swv, bv, sa0);
 }
 
-// The same for up to 128 activation rows (RB = 1..4 row blocks; a batch of decodes, a short prefill) and TNB = 1 or 2
-// 32-row blocks of weights per workgroup, RB * TNB <= 4 output blocks: K split between the four waves, each of which
-// multiplies its TNB weight fragments with the RB activation fragments of the k block (L2 resident: RB KiB a step
-// against TNB KiB from HBM).  The weights are the only operand that comes from memory, and they are read once; the
-// 128 x 64 tiles of the general kernel give such shapes 64-170 workgroups with 786 KB of operands each, and take as
-// long for 64 rows as for 512.  Wave b ends up owning output block b: the others park their partials of it in LDS.
+// The same with RB = 1 or 2 activation row blocks and TNB = 1 or 2 32-row blocks of weights per workgroup (a batch of
+// decodes, a short prefill): K split between the four waves, each of which multiplies its TNB weight fragments with
+// the RB activation fragments of the k block (L2 resident: RB KiB a step against TNB KiB from HBM).  Up to 64
+// activation rows one row of workgroups covers the matrix and the weights are read from memory once; with more rows,
+// blockIdx.y picks the pair of row blocks and the grid is one of 64 x 64 tiles.  The 128 x 64 tiles of the general
+// kernel give such shapes 64-170 workgroups with 786 KB of operands each, and take as long for 64 rows as for 512.
+// Wave b ends up owning output block b: the others park their partials of it in LDS.
 template <int D, int RB, int TNB, int EPI, bool EVEN>
 __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__restrict__ PA, const int8_t *__restrict__ PW,
                                                                int M, int N, int K, GemmEpilogue ep) {
@@ -589,14 +590,16 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
         }
     }
     const __amdgpu_buffer_rsrc_t ra =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PA), 0, RB * KB * 1024, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PA), 0, 0x7ffffffe, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(PW), 0, 0x7fffffff, 0x00020000);
     const int steps = KB / WK, voff = lane * 16;
+    // blockIdx.y: which group of RB activation row blocks (more than RB of them: a grid of RB*32 x TNB*32 tiles)
+    const int rb0 = static_cast<int>(blockIdx.y) * RB;
     int soa[RB], voffa[RB], sow[TNB];  // rows past M read zeros without touching memory
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-        soa[i] = (i * KB + wave) * 1024;
-        voffa[i] = i * 32 + lane % 32 < M ? voff : 0x7fffffff;
+        soa[i] = ((rb0 + i) * KB + wave) * 1024;
+        voffa[i] = (rb0 + i) * 32 + lane % 32 < M ? voff : 0x7fffffff;
     }
 #pragma unroll
     for (int j = 0; j < TNB; ++j) {
@@ -663,7 +666,7 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
             for (int c = 0; c < 4; ++c) own[0][0][4 * g + c] = acc[b][4 * g + c] + t[c];
         }
     }
-    store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, (wave / TNB) * 32, 0, lane, nn, swv, bv, sa0);
+    store_tile<1, 1, 1, EPI, EVEN>(own, ep, M, N, (rb0 + wave / TNB) * 32, 0, lane, nn, swv, bv, sa0);
 }
 
 // The same product straight from fp32 activations of at most four rows (decode), per-row dynamic int8: one launch
@@ -874,7 +877,7 @@ template <int RB, int TNB, int EPI, bool EVEN>
 static int32_t launch_skinny_packed_rb(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                                        const GemmEpilogue &ep) {
     const int groups = ((N + 31) / 32 + TNB - 1) / TNB;
-    const dim3 grid(groups);
+    const dim3 grid(groups, ((M + 31) / 32 + RB - 1) / RB);
     // (depth 8 at most: a stage is RB + TNB fragments of four registers)
     if (groups >= 200)
         hipLaunchKernelGGL((skinny_i8_packed_kernel<4, RB, TNB, EPI, EVEN>), grid, dim3(256), 0, ctx->stream, pa, pw, M, N, K,
@@ -885,9 +888,9 @@ static int32_t launch_skinny_packed_rb(hipq_ctx *ctx, const int8_t *pa, const in
     return check_launch("skinny_i8 (packed)");
 }
 
-// Up to 128 activation rows on the weight-streaming kernel.  From 300 weight row blocks on a workgroup takes two of
-// them (up to two activation row blocks): half the activation traffic per weight byte, and still more than one
-// workgroup per compute unit.  One / two weight row blocks per workgroup, us:
+// The weight-streaming kernel's forms.  Up to 64 activation rows: from 300 weight row blocks on a workgroup takes two
+// of them: half the activation traffic per weight byte, and still more than one workgroup per compute unit.  One /
+// two weight row blocks per workgroup, us:
 //   N = 11008, K = 4096: M = 1 10.4 / 10.25, 16 11.3 / 10.9, 32 13.4 / 12.0, 33 14.9 / 12.9, 64 17.5 / 14.2
 //   N = 32000, K = 4096: M = 1 26.6 / 24.0 (5.5 TB/s), 32 28.5 / 25.6, 64 35.9 / 28.6;   N = 128256: M = 1 87.6 / 86.1
 //   N = 8192,  K = 2048: M = 1 4.7 / 5.1, 32 5.4 / 6.2, 64 7.3 / 7.9 (and the same below that); four per workgroup: slower.
@@ -898,12 +901,8 @@ static int32_t launch_skinny_packed(hipq_ctx *ctx, const int8_t *pa, const int8_
                                     const GemmEpilogue &ep) {
     const bool two = (N + 31) / 32 >= kTwoBlockRowBlocks;
     if (M <= 32) return launch_skinny_packed_rb<1, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // (callers: `two` only)
-    if (M <= 64) {
-        if (two) return launch_skinny_packed_rb<2, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-        return launch_skinny_packed_rb<2, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-    }
-    if (M <= 96) return launch_skinny_packed_rb<3, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
-    return launch_skinny_packed_rb<4, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    if (M <= 64 && !two) return launch_skinny_packed_rb<2, 1, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    return launch_skinny_packed_rb<2, 2, EPI, EVEN>(ctx, pa, pw, M, N, K, ep);  // more than 64 rows: a grid of 64 x 64 tiles
 }
 
 template <int EPI, bool EVEN>
@@ -984,19 +983,17 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
             return launch_skinny_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
         return launch_gemv_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     }
-    // Up to four: the weights streamed once per 32-row block, as above, where that beats the tiled kernel (variant
-    // 9: the tiled kernel always).  Every workgroup pulls all activation fragments through its compute unit's
-    // vector-memory path, RB KiB for each KiB of weights, so the more row blocks of either operand, the less it
-    // pays.  Measured, skinny / tiled in us:   N = K = 4096          N = 11008, K = 4096    N = 4096, K = 11264
-    //                                 M = 48    8.4 / 12.1            15.6 / 17.0            19.2 / 30.6
-    //                                 M = 64    9.1 / 11.8            17.5 / 16.9            21.2 / 30.5
-    //                                 M = 96   11.5 / 12.6            21.4 / 18.4            25.9 / 34.7
-    //                                 M = 128  13.4 / 12.2            25.6 / 19.0            30.4 / 36.9
-    // (the tiled kernel's depth makes no difference at these shapes: 2 / 4 / 8 stages within 0.5 us.)
-    if (M <= 128 && ctx->gemm_variant != 9) {
-        const int row_blocks = (N + 31) / 32;
-        if (M <= 64 || (row_blocks <= 200 && (M <= 96 || steps >= 64)))
-            return launch_skinny_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
+    // Up to 64 rows: the weight-streaming kernel.  More rows: the same kernel as a grid of 64 x 64 tiles, while those
+    // make one round over the compute units at most - half the operand bytes per workgroup of a 128 x 64 tile
+    // (512 KB against 786 KB at K = 4096), and twice the workgroups where the 128 x 64 tiles leave compute units idle
+    // (variant 9: the 128 x 64 tiles always).  128 x 64 / 64 x 64 in us:
+    //   N = K = 4096:        M = 96 12.6 / 8.5   128 12.2 / 8.9   192 13.7 / 9.0   256 13.4 / 9.3   384 13.2 / 15.0
+    //   N = 4096, K = 11264: M = 128 36.9 / 26.3  256 34.0 / 25.4  384 32.9 / 38.3
+    //   N = 8192, K = 2048:  M = 128  8.8 / 7.9;  N = 2304, K = 768: M = 384 6.0 / 5.3, 512 6.0 / 6.2
+    //   N = 11008, K = 4096: M = 128 18.8 / 20.5  256 30.0 / 31.2  512 39.4 / 58.6   (344 and more 64 x 64 tiles)
+    if (ctx->gemm_variant != 9 && !ctx->trace) {  // (the phase stamps are the 128 x 64 kernel's)
+        const size_t tiles64 = ((packed_row_blocks(m) + 1) / 2) * ((packed_row_blocks(n) + 1) / 2);
+        if (M <= 64 || tiles64 <= size_t(ctx->num_cus)) return launch_skinny_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);
     }
     if constexpr (EPI == EPI_F32 && !EVEN) {
         // Phase stamps (hipq_ctx_set_trace_buffer): the depth-2 fp32 form only, and only when the buffer holds

@@ -194,8 +194,10 @@ int32_t hipq_quantize_per_row_packed_f32_i8(hipq_ctx *ctx, const float *x, size_
 // most half of its 4 MiB L2 and the tiles make one round over the compute units; variant 11 switches it off.
 static void set_weight_warming(hipq_ctx *ctx, const int8_t *w_packed, size_t m, size_t n, size_t k) {
     ctx->warm = WarmLines{};
-    if (ctx->gemm_variant == 11 || m <= 128) return;  // (up to 128 rows mostly go to the skinny kernels)
     const size_t rbW = packed_row_blocks(n), KB = packed_k_blocks(k);
+    // (few rows, or few 64 x 64 tiles: the weight-streaming kernel runs, not the 128 x 64 tiles this is laid out for)
+    if (ctx->gemm_variant == 11 || m <= 64 || ((packed_row_blocks(m) + 1) / 2) * ((rbW + 1) / 2) <= size_t(ctx->num_cus))
+        return;
     const size_t tiles_m = (packed_row_blocks(m) + 3) / 4, tiles_n = (rbW + 1) / 2;
     if (tiles_m * tiles_n > size_t(ctx->num_cus) || rbW % 2 != 0 || KB % 32 != 0) return;
     int gm = 0, gn = 0;
