@@ -755,9 +755,15 @@ def main() -> int:
                 ct[0] += 1
                 ctx.linear_dynamic_packed(x3, pw3[ct[0] % len(pw3)], sw3, None, per_token=True, out=o3)
 
+            def run_gemv_forward_static():
+                # the same forward with a calibrated (static) per-tensor activation scale
+                ct[0] += 1
+                ctx.linear_static_packed(x3, 0.03, pw3[ct[0] % len(pw3)], sw3, None, out=o3)
+
             nbytes = n3 * k3 + m3 * k3 + 4 * m3 * n3 + 4 * n3
             for name, fn in ((f"gemv_m{m3}_n11008_k4096", run_gemv_prepared),
                              (f"gemv_m{m3}_n11008_k4096_forward_from_f32", run_gemv_forward),
+                             (f"gemv_m{m3}_n11008_k4096_forward_from_f32_static_scale", run_gemv_forward_static),
                              (f"gemv_m{m3}_n11008_k4096_row_major_weights", run_gemv)):
                 ms = event_time_ms(fn, reps=100, warmup=10)
                 extra[name] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9,

@@ -290,6 +290,38 @@ def test_decode_forward_per_token(hipq, m, n, k):
         c.close()
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 11008, 4096), (4, 11008, 4096), (3, 1000, 4096), (2, 512, 8192), (1, 300, 16384),
+                                   (4, 96, 512), (2, 4096, 11008), (4, 64, 8192)])
+def test_decode_forward_with_a_static_scale(hipq, m, n, k):
+    """hipq_linear_static_packed_f32 with up to four rows runs as one launch where the rows fit a thread's registers
+    (the last two shapes do not): same bits as the two launches (variant 6) for both quantize forms and roundings,
+    with values that saturate, a NaN and an infinity among them."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(m * 11 + n + k)
+        wq = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+        pw = c.pack_rows(wq)
+        sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+        bias = torch.randn(n, generator=g, device="cuda")
+        x = torch.randn(m, k, generator=g, device="cuda") * 2.0
+        x[0, 3] = 1e6
+        x[m - 1, 7] = float("nan")
+        x[m // 2, 11] = float("-inf")
+        for mode in (hipq.FORM_MUL_INV, hipq.FORM_DIV, hipq.FORM_DIV | hipq.ROUND_HALF_EVEN, hipq.ROUND_HALF_EVEN):
+            for b in (bias, None):
+                c.set_gemm_kernel_variant(0)
+                got = c.linear_static_packed(x, 0.037, pw, sw, b, mode=mode)
+                c.set_gemm_kernel_variant(6)
+                want = c.linear_static_packed(x, 0.037, pw, sw, b, mode=mode)
+                c.synchronize()
+                assert torch.equal(got, want), mode
+        c.set_gemm_kernel_variant(0)
+        with pytest.raises(hipq.HipqError):
+            c.linear_static_packed(x, 0.0, pw, sw, bias)
+    finally:
+        c.close()
+
+
 def test_linear_static_packed(ctx, hipq):
     g = torch.Generator(device="cuda").manual_seed(3)
     m, n, k = 96, 160, 512

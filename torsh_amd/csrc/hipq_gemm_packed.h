@@ -681,10 +681,10 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
 // store_tile does it.  Every workgroup repeats the quantize arithmetic of all rows (16 values a thread and row at
 // K = 4096), which is why this pays for one or two rows only: N = 11008, K = 4096 from fp32, one launch against
 // the quantizer and the product: M = 1 11.7 / 14.7 us, M = 2 13.3 / 14.7, M = 3 15.4 / 14.8, M = 4 17.3 / 15.0.
-template <int D, bool EVEN, int MROWS, int CH>
+template <int D, bool EVEN, int MROWS, int CH, bool STATIC = false>
 __global__ __launch_bounds__(256) void gemv_i8_packed_from_f32_kernel(const float *__restrict__ x,
                                                                       const int8_t *__restrict__ PW, int M, int N, int K,
-                                                                      GemmEpilogue ep) {
+                                                                      GemmEpilogue ep, int static_div) {
     static_assert(MROWS * CH <= 4, "at most 64 data registers per thread");
     __shared__ __attribute__((aligned(16))) v4i red[3][4][kWave];
     __shared__ __attribute__((aligned(16))) v4i codes[MROWS * CH * 256];
@@ -726,38 +726,55 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_from_f32_kernel(const floa
                 for (int i = 0; i < 4; ++i) v[m][c][i] = reinterpret_cast<const float4 *>(x + size_t(m) * K + k0)[i];
             }
         }
+    if constexpr (!STATIC) {
 #pragma unroll
-    for (int m = 0; m < MROWS; ++m) {
-        float mn = INFINITY, mx = -INFINITY;
+        for (int m = 0; m < MROWS; ++m) {
+            float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
-        for (int c = 0; c < CH; ++c)
-            if (have[m][c]) {
+            for (int c = 0; c < CH; ++c)
+                if (have[m][c]) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    mn = fminf(mn, fminf(fminf(v[m][c][i].x, v[m][c][i].y), fminf(v[m][c][i].z, v[m][c][i].w)));
-                    mx = fmaxf(mx, fmaxf(fmaxf(v[m][c][i].x, v[m][c][i].y), fmaxf(v[m][c][i].z, v[m][c][i].w)));
+                    for (int i = 0; i < 4; ++i) {
+                        mn = fminf(mn, fminf(fminf(v[m][c][i].x, v[m][c][i].y), fminf(v[m][c][i].z, v[m][c][i].w)));
+                        mx = fmaxf(mx, fmaxf(fmaxf(v[m][c][i].x, v[m][c][i].y), fmaxf(v[m][c][i].z, v[m][c][i].w)));
+                    }
                 }
+            mn = wave_min(mn);
+            mx = wave_max(mx);
+            if (lane == 0) {
+                wave_mn[wave][m] = mn;
+                wave_mx[wave][m] = mx;
             }
-        mn = wave_min(mn);
-        mx = wave_max(mx);
-        if (lane == 0) {
-            wave_mn[wave][m] = mn;
-            wave_mx[wave][m] = mx;
         }
+        __syncthreads();
     }
-    __syncthreads();
     float sa[MROWS];
 #pragma unroll
     for (int m = 0; m < MROWS; ++m) {
-        const float mn = fminf(fminf(wave_mn[0][m], wave_mn[1][m]), fminf(wave_mn[2][m], wave_mn[3][m]));
-        const float mx = fmaxf(fmaxf(wave_mx[0][m], wave_mx[1][m]), fmaxf(wave_mx[2][m], wave_mx[3][m]));
-        float scale;
-        int zp;
-        const bool bad = params_from_minmax(mn, mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp) != HIPQ_SUCCESS;
-        sa[m] = bad ? __builtin_nanf("") : scale;
-        if (bad) scale = INFINITY;  // x / inf: 0 for finite x, NaN -> code 0 otherwise
-        const float inv = recip_for_div(scale), zpf = static_cast<float>(bad ? 0 : zp);
-        auto q = [&](float f) { return quantize_int<QFORM_DIV, EVEN>(f, scale, inv, zpf, -128, 127); };
+        float scale, inv, zpf = 0.0f;
+        if constexpr (STATIC) {
+            // a given per-tensor scale: the packed quantizer's arithmetic in the caller's form (quantize_packed_kernel)
+            scale = ep.sa_scalar;
+            sa[m] = scale;
+            inv = static_div ? recip_for_div(scale) : 1.0f / scale;
+        } else {
+            const float mn = fminf(fminf(wave_mn[0][m], wave_mn[1][m]), fminf(wave_mn[2][m], wave_mn[3][m]));
+            const float mx = fmaxf(fmaxf(wave_mx[0][m], wave_mx[1][m]), fmaxf(wave_mx[2][m], wave_mx[3][m]));
+            int zp;
+            const bool bad = params_from_minmax(mn, mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp) != HIPQ_SUCCESS;
+            sa[m] = bad ? __builtin_nanf("") : scale;
+            if (bad) scale = INFINITY;  // x / inf: 0 for finite x, NaN -> code 0 otherwise
+            inv = recip_for_div(scale);
+            zpf = static_cast<float>(bad ? 0 : zp);
+        }
+        auto q = [&](float f) {
+            if constexpr (STATIC) {
+                return static_div ? quantize_int<true, EVEN>(f, scale, inv, zpf, -128, 127)
+                                  : quantize_int<false, EVEN>(f, scale, inv, zpf, -128, 127);
+            } else {
+                return quantize_int<QFORM_DIV, EVEN>(f, scale, inv, zpf, -128, 127);
+            }
+        };
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int g = static_cast<int>(threadIdx.x) + 256 * c;
@@ -812,22 +829,25 @@ __global__ __launch_bounds__(256) void gemv_i8_packed_from_f32_kernel(const floa
 }
 
 // Whether the decode forward from fp32 can take the kernel above, and its launch.  Returns false when the shape is
-// left to the two launches (per-row quantizer into the packed layout, then gemv_i8_packed_kernel).
-template <bool EVEN>
+// left to the two launches (quantizer into the packed layout, then the product).  STATIC: a given per-tensor scale
+// (ep.sa_scalar; `static_div`: the division form) instead of per-row dynamic scales; without the range pass and its
+// barrier the prologue is cheap enough for four rows.
+template <bool EVEN, bool STATIC>
 static bool launch_gemv_packed_from_f32(hipq_ctx *ctx, const float *x, const int8_t *pw, size_t m, size_t n, size_t k,
-                                        const GemmEpilogue &ep, int32_t *rc) {
+                                        const GemmEpilogue &ep, int static_div, int32_t *rc) {
     const size_t KB = packed_k_blocks(k);
     const size_t chunks = (KB * 2 + 255) / 256;  // 16-float groups per thread and row
-    if (m == 0 || m > 2 || k % 16 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) != 0 || KB < 16) return false;
-    const int mrows = static_cast<int>(m), ch = chunks <= 1 ? 1 : (chunks == 2 ? 2 : 4);
+    const size_t most_rows = STATIC ? 4 : 2;
+    if (m == 0 || m > most_rows || k % 16 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) != 0 || KB < 16) return false;
+    const int mrows = m <= 2 ? static_cast<int>(m) : 4, ch = chunks <= 1 ? 1 : (chunks == 2 ? 2 : 4);
     if (chunks > 4 || mrows * ch > 4) return false;
     const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
     const int row_blocks = (N + 31) / 32;
     const int depth = row_blocks >= 200 ? 4 : (row_blocks >= 100 ? 8 : 16);  // as launch_gemv_packed
     const dim3 grid(row_blocks);
-#define HIPQ_LAUNCH_GFD(DEPTH, MR, C)                                                                              \
-    hipLaunchKernelGGL((gemv_i8_packed_from_f32_kernel<DEPTH, EVEN, MR, C>), grid, dim3(256), 0, ctx->stream, x, pw, M, N, \
-                       K, ep)
+#define HIPQ_LAUNCH_GFD(DEPTH, MR, C)                                                                                  \
+    hipLaunchKernelGGL((gemv_i8_packed_from_f32_kernel<DEPTH, EVEN, MR, C, STATIC>), grid, dim3(256), 0, ctx->stream, x, pw, \
+                       M, N, K, ep, static_div)
 #define HIPQ_LAUNCH_GF(MR, C)              \
     do {                                   \
         if (depth == 4)                    \
@@ -843,10 +863,12 @@ static bool launch_gemv_packed_from_f32(hipq_ctx *ctx, const float *x, const int
         HIPQ_LAUNCH_GF(1, 2);
     else if (mrows == 1)
         HIPQ_LAUNCH_GF(1, 4);
-    else if (ch == 1)
+    else if (mrows == 2 && ch == 1)
         HIPQ_LAUNCH_GF(2, 1);
-    else
+    else if (mrows == 2)
         HIPQ_LAUNCH_GF(2, 2);
+    else if constexpr (STATIC)
+        HIPQ_LAUNCH_GF(4, 1);
 #undef HIPQ_LAUNCH_GF
 #undef HIPQ_LAUNCH_GFD
     *rc = check_launch("gemv_i8 (packed, from fp32)");

@@ -241,8 +241,8 @@ int32_t hipq_linear_dynamic_packed_f32(hipq_ctx *ctx, const float *x, int32_t pe
         if (m <= 2 && ctx->gemm_variant != 6) {
             GemmEpilogue ep{nullptr, 1, w_scales, bias, 1.0f, 0, out};
             const bool fused = (mode & HIPQ_ROUND_HALF_EVEN)
-                                   ? launch_gemv_packed_from_f32<true>(ctx, x, w_packed, m, n, k, ep, &rc)
-                                   : launch_gemv_packed_from_f32<false>(ctx, x, w_packed, m, n, k, ep, &rc);
+                                   ? launch_gemv_packed_from_f32<true, false>(ctx, x, w_packed, m, n, k, ep, 0, &rc)
+                                   : launch_gemv_packed_from_f32<false, false>(ctx, x, w_packed, m, n, k, ep, 0, &rc);
             if (fused) return rc;
         }
         // one pass over the activations: the per-row quantizer writes the packed operand itself
@@ -270,6 +270,17 @@ int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_sca
     HIPQ_REQUIRE_PTR(w_packed);
     HIPQ_REQUIRE_PTR(w_scales);
     HIPQ_REQUIRE_PTR(out);
+    // Decode, up to four rows: one launch, every workgroup quantizes the rows itself (variant 6 keeps the two).  A
+    // scale or mode that is not valid goes on to the quantizer below, which says so.
+    if (m <= 4 && ctx->gemm_variant != 6 && a_scale > 0.0f && !(mode & ~(HIPQ_ROUND_HALF_EVEN | HIPQ_FORM_DIV))) {
+        GemmEpilogue ep{nullptr, 0, w_scales, bias, 1.0f, 0, out};
+        ep.sa_scalar = a_scale;
+        const int div = (mode & HIPQ_FORM_DIV) ? 1 : 0;
+        const bool fused = (mode & HIPQ_ROUND_HALF_EVEN)
+                               ? launch_gemv_packed_from_f32<true, true>(ctx, x, w_packed, m, n, k, ep, div, &rc)
+                               : launch_gemv_packed_from_f32<false, true>(ctx, x, w_packed, m, n, k, ep, div, &rc);
+        if (fused) return rc;
+    }
     const PackedScratch L = packed_scratch_layout(ctx->num_cus, m, k);
     void *s = nullptr;
     rc = scratch(ctx, L.total, &s);
