@@ -316,27 +316,6 @@ HIPQ_API int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_
                                         const float *a_scale, int32_t a_scale_per_row, const float *w_scales,
                                         const float *bias, float out_scale, int32_t out_zero_point,
                                         int32_t mode, int8_t *out);
-/* Test and tuning hook with no counterpart in the reference: forces one of the GEMM kernel forms
- * for every later call on this context wherever the shape allows it (0 = automatic choice, the
- * default; 1-3 one-tile-per-workgroup forms, 5-8 persistent forms, 10 register-staged form); 6 also
- * makes the dynamic per-tensor activation quantizer of the Linear forwards run as two launches (range
- * partials, then a quantizer that folds them) where it would run as one, and the per-token forward
- * of one or two rows as a quantizer and a product where it would be one kernel; 9 and 11 leave the
- * choice automatic and switch off, on prepared operands, the forms of the GEMM that are picked by
- * occupancy - two workgroups per compute unit, the weight-streaming kernel for 33..128 rows - (9)
- * and the touching of weight / filter lines by the one-launch activation quantizers of the dynamic
- * Linear and Conv2d forwards while their grids wait for the range (11).
- * Results do not depend on it; the parity tests use it to run every form on the same inputs. */
-HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
-/* Test hook with no counterpart in the reference.  Two kernels couple their waves through device
- * memory: the persistent GEMM kernel (counters between producer and consumer waves) and the one-launch
- * dynamic per-tensor packed quantizer (its workgroups meet to agree on the range).  Both bound every
- * wait, so that a grid always drains; a wait that gives up marks the context, and the next
- * hipq_ctx_synchronize returns HIPQ_DEVICE_ERROR once instead of handing back a wrong result silently
- * (the quantizer also leaves zero codes, a NaN scale and status HIPQ_DEVICE_ERROR in out_params).
- * `limit` is the number of polls after the first look (negative = the default, 2^20); 0 lets a test see
- * the error path without hanging anything. */
-HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
 /* No counterpart in the reference.  The one-launch dynamic quantizers need their whole grid resident on the device
  * at once and size it for the device being theirs: up to half of it (four light workgroups per compute unit) for
  * tensors of up to 4 Mi elements, all of its register files above that.  When `contexts` contexts launch such
@@ -344,14 +323,6 @@ HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
  * of the device and takes the two-launch path for what does not fit, instead of two half-resident grids waiting
  * for each other until their bounded waits give up.  Default 1; 1..64. */
 HIPQ_API int32_t hipq_ctx_set_resident_share(hipq_ctx *ctx, int32_t contexts);
-/* Tuning aid with no counterpart in the reference.  While a device buffer is set, hipq_linear_packed_i8_f32
- * (and the forwards built on it) run a form of the packed GEMM kernel in which every wave records the shader
- * clock at six points - start, first operands in registers, end of the K loop, partial sums reduced, stores
- * issued, stores retired - followed by the constant 100 MHz counter at the first and the last point, as uint64
- * values [workgroup][wave 0..3][8], provided the buffer holds ceil(m/128) * ceil(n/64) * 4 * 8 * 8 bytes
- * (otherwise the ordinary kernel runs).  The results are the same
- * bits.  null removes the buffer.  bench.py --profile gemm_phases prints the phase table from it. */
-HIPQ_API int32_t hipq_ctx_set_trace_buffer(hipq_ctx *ctx, void *device_buffer, size_t bytes);
 /* Whole forward of a quantized Linear with a static (calibrated) activation scale: the scale an
  * observer derived beforehand (Observer::calculate_qparams, crates/torsh-quantization/src/observers.rs:263-310,
  * symmetric: zero point 0) instead of a range pass over every input - per-tensor quantize

@@ -1,0 +1,52 @@
+/*
+ * torsh_hipq - test and tuning hooks of the library.  None of them has a counterpart in the
+ * reference and none belongs to the surface a binding exposes: a maintainer's FFI crate binds
+ * include/torsh_hipq.h only (the generated Rust declarations leave this file out).  They exist so
+ * that the parity tests can run every kernel form on the same inputs, see the error path of a
+ * bounded wait without hanging anything, and read the kernels' own phase stamps.  Results never
+ * depend on them.  No environment variable changes which kernels run.
+ */
+#ifndef TORSH_HIPQ_TESTING_H
+#define TORSH_HIPQ_TESTING_H
+
+#include "torsh_hipq.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Forces one of the GEMM kernel forms for every later call on this context wherever the shape
+ * allows it (0 = automatic choice, the default; 1-3 one-tile-per-workgroup forms, 5-8 persistent
+ * forms, 10 register-staged form); 6 also makes the dynamic per-tensor activation quantizer of the
+ * Linear forwards run as two launches (range partials, then a quantizer that folds them) where it
+ * would run as one, and the per-token forward of one or two rows as a quantizer and a product where
+ * it would be one kernel; 9 and 11 leave the choice automatic and switch off, on prepared operands,
+ * the forms of the GEMM that are picked by occupancy - two workgroups per compute unit, the
+ * weight-streaming kernel for 33..128 rows - (9) and the touching of weight / filter lines by the
+ * one-launch activation quantizers of the dynamic Linear and Conv2d forwards while their grids wait
+ * for the range (11); 12 keeps the headline shape on the one-tile-per-compute-unit form where the
+ * K-split-across-compute-units form would be picked. */
+HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
+/* Some kernels couple their waves through device memory: the persistent GEMM kernel (counters
+ * between producer and consumer waves), the one-launch dynamic quantizers (their workgroups meet to
+ * agree on the range) and the GEMM form whose workgroup pairs exchange partial sums.  All bound
+ * every wait, so that a grid always drains; a wait that gives up marks the context, and the next
+ * hipq_ctx_synchronize returns HIPQ_DEVICE_ERROR once instead of handing back a wrong result
+ * silently (the quantizers also leave zero codes, a NaN scale and status HIPQ_DEVICE_ERROR in
+ * out_params).  `limit` is the number of polls after the first look (negative = the default, 2^20);
+ * 0 lets a test see the error path without hanging anything. */
+HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
+/* While a device buffer is set, hipq_linear_packed_i8_f32 (and the forwards built on it) run a
+ * form of the packed GEMM kernel in which every wave records the shader clock at six points -
+ * start, first operands in registers, end of the K loop, partial sums reduced, stores issued,
+ * stores retired - followed by the constant 100 MHz counter at the first and the last point, as
+ * uint64 values [workgroup][wave 0..3][8], provided the buffer holds one such record per wave of
+ * the grid (otherwise the ordinary kernel runs).  The results are the same bits.  null removes the
+ * buffer.  bench.py --profile gemm_phases prints the phase table from it. */
+HIPQ_API int32_t hipq_ctx_set_trace_buffer(hipq_ctx *ctx, void *device_buffer, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TORSH_HIPQ_TESTING_H */

@@ -59,3 +59,9 @@ def test_json_line_has_the_contract_fields():
     r = d["roofline"]
     assert r["bound"] in ("hbm", "mfma") and r["frac"] == pytest.approx(r["achieved"] / r["peak"])
     assert d["value"] > 0 and d["ms_per_step"] > 0
+    # the metric's second half (quantize GB/s) travels inside `roofline`, on the bytes that move
+    for key, nbytes in (("quantize", 5 << 24), ("dequantize", 5 << 24), ("minmax", 4 << 24)):
+        h = r["hbm"][key]
+        assert h["bytes"] == nbytes and h["peak"] == 8000.0 and h["unit"] == "GB/s"
+        assert h["achieved"] == pytest.approx(nbytes / (h["us"] * 1e-6) / 1e9)
+        assert h["frac"] == pytest.approx(h["achieved"] / h["peak"]) and 0 < h["frac"] < 1

@@ -288,6 +288,31 @@ def test_dynamic_quantize_one_launch_matches_two_launches(hipq, n, dtype_name):
         c.close()
 
 
+@pytest.mark.parametrize("lo,hi", [(2.0, 5.0), (-100.0, -99.0)])
+@pytest.mark.parametrize("n", [4096, 4099, 1 << 20])
+def test_dynamic_quantize_with_a_zero_point_outside_the_code_range(ctx, hipq, lo, hi, n):
+    """The torsh-nn asymmetric rule does not clamp its zero point: an all-positive tensor in [2, 5] gives -170, an
+    all-negative one in [-100, -99] gives 25500.  Such a zero point must not depend on which path a size and
+    alignment select (sizes that qualify for the one-launch quantizer and one that does not): status SUCCESS, the
+    parameters of the formula ((max - min) / 255, round(-min / scale)), and the codes
+    clamp(round(x / scale) + zp, 0, 255), from numpy in float32."""
+    rng = np.random.default_rng(n)
+    x = (rng.random(n, dtype=np.float32) * np.float32(hi - lo) + np.float32(lo)).astype(np.float32)
+    x[0], x[-1] = lo, hi
+    q, params = ctx.quantize_dynamic_per_tensor(dev(x), hipq.PARAMS_NN_ASYMMETRIC, hipq.DTYPE_U8, hipq.FORM_DIV)
+    ctx.synchronize()
+    p = ctx.read_qparams(params)
+    scale = np.float32(np.float32(hi) - np.float32(lo)) / np.float32(255.0)
+    t = -np.float32(lo) / scale
+    zp = int(np.trunc(t + np.copysign(np.float32(0.5), t)))  # f32::round of a value that is no tie
+    assert p.status == hipq.SUCCESS and p.scale == scale and p.zero_point == zp
+    assert zp == {2.0: -170, -100.0: 25500}[lo]
+    v = x / scale
+    r = np.trunc(v + np.copysign(np.float32(0.49999997), v))  # f32::round (tests/host/round_away_check.c)
+    want = np.clip(r + np.float32(zp), 0, 255).astype(np.uint8)
+    np.testing.assert_array_equal(host(q), want)
+
+
 @pytest.mark.parametrize("shape", [(1, 8), (3, 33), (16, 4096), (5, 1024), (7, 1025), (4, 4100), (2, 20000), (64, 768)])
 @pytest.mark.parametrize("flavor_name", ["symmetric", "affine"])
 def test_per_row_quantize(ctx, hipq, oracle, shape, flavor_name):

@@ -207,6 +207,37 @@ def test_config3_full_size_weight_streaming(ctx, hipq, m):
     want = ref.float() * (sa[:, None] * sw[None, :]) + bias[None, :]  # same individually rounded f32 ops
     torch.cuda.synchronize()
     assert torch.equal(out, want)
+    # The kernels the benchmark times at this shape run on prepared (fragment-packed) operands: the one-row-block
+    # kernel and both forms of the weight-streaming kernel, at 344 weight row blocks x 128 k blocks, against the
+    # same exact product and the same f32 expression.
+    pa, pw = ctx.pack_rows(a), ctx.pack_rows(w)
+    assert torch.equal(ctx.gemm_packed_i8_i32(pa, pw, m, n, k), ref)
+    assert torch.equal(ctx.linear_packed_i8_f32(pa, sa, pw, sw, bias, m, n, k), want)
+    assert torch.equal(ctx.linear_packed_i8_f32(pa, sa[:1], pw, sw, None, m, n, k),
+                       ref.float() * (sa[0] * sw[None, :]))  # one scale for the tensor, no bias
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 16])
+def test_config3_full_size_forward_from_fp32_against_the_oracle(ctx, hipq, oracle, m):
+    """configs[2] as specified, at its own size (N=11008, K=4096): fp32 activations, per-token dynamic int8, prepared
+    per-channel weights, fp32 out.  One or two rows take the one-launch kernel in which every workgroup quantizes
+    the rows itself, more rows the per-row quantizer and the product; both against the oracle's per-channel
+    quantize (axis 0) + int32 GEMM + dequantize epilogue, bit for bit."""
+    rng = np.random.default_rng(500 + m)
+    n, k = 11008, 4096
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wq = rand_i8(rng, (n, k))
+    sw = (rng.random(n) * 0.002 + 0.0001).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    aq, sa, _ = oracle.quantize_per_channel_auto(x, 0, oracle.DTYPE_I8, oracle.PER_CHANNEL_SYMMETRIC)
+    acc = oracle.gemm_i8_nk(aq.astype(np.int8), wq)
+    want = oracle.linear_dequant_epilogue(acc, sa, sw, bias)
+    pw = ctx.pack_rows(dev(wq))
+    got = host(ctx.linear_dynamic_packed(dev(x), pw, dev(sw), dev(bias), per_token=True))
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=0)
+    np.testing.assert_array_equal(got, want)
+    want_nb = oracle.linear_dequant_epilogue(acc, sa, sw, None)
+    np.testing.assert_array_equal(host(ctx.linear_dynamic_packed(dev(x), pw, dev(sw), None, per_token=True)), want_nb)
 
 
 @pytest.mark.parametrize("n,k", [(2304, 768), (768, 768), (3072, 768), (768, 3072)])

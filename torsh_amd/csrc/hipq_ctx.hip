@@ -33,21 +33,34 @@ int32_t enter(hipq_ctx *ctx) {
 }
 
 int32_t scratch(hipq_ctx *ctx, size_t bytes, void **out) {
+    // Kernels recorded under stream capture keep pointers into the block of that moment.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(ctx->stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
+    if (capturing) ctx->scratch_captured = true;
     if (bytes > ctx->scratch_bytes) {
+        if (capturing)
+            return fail(HIPQ_ALLOCATION_ERROR,
+                        "scratch: this call needs %zu bytes of context scratch and the context holds %zu; memory cannot "
+                        "be allocated while the stream is capturing - run the same call once before the capture",
+                        bytes, ctx->scratch_bytes);
         // Round up so a sequence of slightly growing requests reallocates rarely.
         size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        void *grown = nullptr;
+        hipError_t e = hipMalloc(&grown, want);
+        if (e != hipSuccess) return fail(HIPQ_ALLOCATION_ERROR, "scratch: hipMalloc(%zu): %s", want, hipGetErrorString(e));
         if (ctx->scratch) {
-            hipError_t e = hipStreamSynchronize(ctx->stream);
-            if (e != hipSuccess) return fail(HIPQ_SYNCHRONIZATION_ERROR, "scratch: %s", hipGetErrorString(e));
-            (void)hipFree(ctx->scratch);
-            ctx->scratch = nullptr;
-            ctx->scratch_bytes = 0;
+            if (ctx->scratch_captured) {
+                ctx->retired.push_back(ctx->scratch);  // a captured graph may still be replayed on it
+            } else {
+                e = hipStreamSynchronize(ctx->stream);
+                if (e != hipSuccess) {
+                    (void)hipFree(grown);
+                    return fail(HIPQ_SYNCHRONIZATION_ERROR, "scratch: %s", hipGetErrorString(e));
+                }
+                (void)hipFree(ctx->scratch);
+            }
         }
-        hipError_t e = hipMalloc(&ctx->scratch, want);
-        if (e != hipSuccess) {
-            ctx->scratch = nullptr;
-            return fail(HIPQ_ALLOCATION_ERROR, "scratch: hipMalloc(%zu): %s", want, hipGetErrorString(e));
-        }
+        ctx->scratch = grown;
         ctx->scratch_bytes = want;
     }
     *out = ctx->scratch;
@@ -126,10 +139,6 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
         return rc;
     }
     (void)hipq::four_wide_workgroups_fit(ctx);  // asked here so that no later call is the first
-    if (const char *e = getenv("HIPQ_GEMM_VARIANT")) {
-        const int v = atoi(e);
-        if (v >= 0 && v <= 11) ctx->gemm_variant = v;
-    }
     *out_ctx = ctx;
     return HIPQ_SUCCESS;
 }
@@ -148,6 +157,7 @@ int32_t hipq_ctx_destroy(hipq_ctx *ctx) {
     HIPQ_ENTER(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    for (void *p : ctx->retired) (void)hipFree(p);
     if (ctx->wait_error) (void)hipFree(ctx->wait_error);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -179,8 +189,8 @@ int32_t hipq_ctx_synchronize(hipq_ctx *ctx) {
 
 int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant) {
     HIPQ_REQUIRE_PTR(ctx);
-    if (variant < 0 || variant > 11)
-        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..11", __func__, variant);
+    if (variant < 0 || variant > 12)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not in 0..12", __func__, variant);
     ctx->gemm_variant = variant;
     return HIPQ_SUCCESS;
 }

@@ -102,6 +102,7 @@ __global__ __launch_bounds__(kBlock) void minmax_one_launch_kernel(const float *
     const bool gave_up = meeting_collect_range(words, gen, spin_limit, lds, &t);
     meeting_close(words, gen, gave_up);
     if (threadIdx.x == 0) {
+        meeting_mark_ready(words, gen);
         if (gave_up) t = MinMax{__builtin_nanf(""), __builtin_nanf("")};  // never a range made of some of the partials
         write_range_outputs(outs, t);
     }
@@ -504,6 +505,9 @@ static bool launch_flat_one_launch(hipq_ctx *ctx, const float *x, size_t n, int 
     if (ctx->gemm_variant == 6 || n % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) ||
         (reinterpret_cast<uintptr_t>(out) & 3u) || (mode & ~(HIPQ_FORM_DIV | HIPQ_ROUND_HALF_EVEN)))
         return false;
+    // The torsh-nn flavours do not clamp their zero point to the code range (min = 2, max = 5 gives -170), and the
+    // word the meeting ends with has room for -128..895 only: they take the two launches, whatever the size.
+    if (flavor > HIPQ_PARAMS_ZERO_INCLUDED) return false;
     const size_t nvec = n / 4;
     const int vpt = nvec <= resident_workgroups(ctx, false) * kBlock * 4 ? 4 : 16;
     const size_t blocks = (nvec + size_t(kBlock) * vpt - 1) / (size_t(kBlock) * vpt);

@@ -7,7 +7,10 @@
 #include <cstddef>
 #include <cstdint>
 
+#include <vector>
+
 #include "torsh_hipq.h"
+#include "torsh_hipq_testing.h"
 
 // Lines (128 bytes) of a packed operand wanted in the L2 of the die whose workgroups will read them: die d's share
 // starts die_stride_lines * d lines after base; within it, per row block (row_block_lines apart), `starts` runs of
@@ -26,12 +29,17 @@ struct hipq_ctx {
     // the context.
     void *scratch = nullptr;
     size_t scratch_bytes = 0;
+    // Set once a call that uses the scratch was recorded under stream capture: the recorded kernels hold pointers
+    // into the block of that moment, so from then on a block that is outgrown is kept (in `retired`, freed with
+    // the context) instead of freed, and a replay of the graph still finds its memory.
+    bool scratch_captured = false;
+    std::vector<void *> retired;
     int num_cus = 256;
     // Device words of the context (kCtxWordsBytes of them, laid out as the kCtx* constants below say).  Word 0 is
     // set by a kernel whose bounded wait gave up; hipq_ctx_synchronize reads and clears it.
     uint32_t *wait_error = nullptr;
-    // Test and tuning hooks, per context: forced GEMM kernel form (0 = automatic; hipq_ctx_create takes it from the
-    // HIPQ_GEMM_VARIANT environment variable when that is set) and the spin limit of the persistent kernel's waits.
+    // Test and tuning hooks, per context (torsh_hipq_testing.h): forced GEMM kernel form (0 = automatic) and the
+    // spin limit of the kernels' bounded waits.
     int gemm_variant = 0;
     int wait_spin_limit = 1 << 20;
     // How many contexts launch concurrently on this device (hipq_ctx_set_resident_share): kernels whose grid has to
@@ -62,13 +70,12 @@ constexpr uint32_t kCtxFirstEpoch = 0xfffffff0u;
 // Puts the device words of a context into their initial state (device current, stream idle).
 int32_t reset_ctx_words(hipq_ctx *ctx);
 // Workgroups of 256 threads per compute unit that a kernel of this context may count on being resident together
-// with the rest of its grid, for a kernel of at most 64 (light) or at most 128 (wide) registers: a compute unit
-// holds 8 resp. 4 such workgroups, and the context's share of that is 1 / resident_share.  A light kernel takes
-// at most half of the device.
-inline size_t resident_workgroups(const hipq_ctx *ctx, bool wide) {
+// with the rest of its grid.  The one-launch kernels, light or wide, are built with a launch bound of four
+// workgroups per compute unit (at most 128 registers), so four is what the bound guarantees whatever the compiler
+// made of a kernel, and the context's share of that is 1 / resident_share.
+inline size_t resident_workgroups(const hipq_ctx *ctx, bool /*wide*/) {
     const int share = ctx->resident_share > 0 ? ctx->resident_share : 1;
-    int per_cu = (wide ? 4 : 8) / share;
-    if (!wide && per_cu > 4) per_cu = 4;
+    const int per_cu = 4 / share;
     size_t total = size_t(ctx->num_cus) * static_cast<size_t>(per_cu);
     return total < kCtxSlots ? total : kCtxSlots;
 }

@@ -95,8 +95,9 @@ __device__ __forceinline__ void record_give_up(uint32_t *words) {
 
 // The word that ends the range part of a meeting carries the scale, the zero point and a tag in 64 bits, so that
 // one look suffices: {meeting number mod 2^22, zero point + 128 in 10 bits, scale bits}.  The short tag is enough
-// here because this word, unlike the range words, is rewritten by every meeting: it only has to differ from the
-// one before (and from the all-zero initial state, which the first numbers of a context do).
+// here because this word, unlike the range words, is rewritten by every meeting - also by those that only collect
+// a range and have nobody waiting for it (meeting_mark_ready) - so it only has to differ from the one before (and
+// from the all-zero initial state, which the first numbers of a context do).
 constexpr uint32_t kReadyTagMask = 0x3fffffu;
 
 // What a meeting agrees on: the parameters workgroup 0 derives from the folded range.  scale is NaN when the
@@ -110,6 +111,13 @@ __device__ __forceinline__ unsigned long long ready_word(uint32_t gen, const Mee
     return (static_cast<unsigned long long>(gen & kReadyTagMask) << 42) |
            (static_cast<unsigned long long>(static_cast<uint32_t>(p.zero_point + 128) & 0x3ffu) << 32) |
            __builtin_bit_cast(uint32_t, p.scale);
+}
+
+// Workgroup 0, thread 0, of a meeting in which nobody waits for parameters: leaves this meeting's tag in the ready
+// word (NaN scale), so that the word always carries the number of the last meeting held.
+__device__ __forceinline__ void meeting_mark_ready(uint32_t *words, uint32_t gen) {
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(words + kCtxReadyWord),
+                       ready_word(gen, MeetingParams{__builtin_nanf(""), 0}), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The whole grid agrees on the quantization parameters of a tensor: `r` is this workgroup's (min, max), uniform
@@ -187,7 +195,11 @@ __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t
             out_params->zero_point = bad ? zp : p.zero_point;
             out_params->min_val = t.mn;
             out_params->max_val = t.mx;
-            out_params->status = st;
+            // A workgroup that stopped waiting for the word above has marked the context; the record says so as
+            // well (it writes the status itself too, in case this store is the later one).
+            const bool lost = __hip_atomic_load(words + kCtxFlagWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+            __hip_atomic_store(&out_params->status, lost ? HIPQ_DEVICE_ERROR : st, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
         }
     } else {
         if (threadIdx.x == 0) {
@@ -204,6 +216,7 @@ __device__ __forceinline__ MeetingParams meet_on_range(uint32_t *words, uint32_t
             }
             if (!got) {
                 record_give_up(words);
+                __hip_atomic_store(&out_params->status, HIPQ_DEVICE_ERROR, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 lds[kMeetingLdsFloats - 2] = __builtin_nanf("");
                 lds[kMeetingLdsFloats - 1] = 0.0f;
             }
