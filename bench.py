@@ -186,7 +186,7 @@ def conv_phase_table(ctx, g) -> int:
     return phase_table("conv2d implicit GEMM M=256 N=8192 K=2304", ctx, forward, waves)
 
 
-def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
+def gemm_phase_table(ctx, M: int, N: int, K: int, g, pairs: bool = False) -> int:
     """Phase budget of the packed GEMM kernel from its own clock stamps (hipq_ctx_set_trace_buffer): 200 launches on
     rotating operand sets; for every launch the median over its 1024 waves of each phase, then the median and the
     spread of that over the launches.  Cycles are shader-clock cycles; the clock rate is what the stamps of the
@@ -210,10 +210,31 @@ def gemm_phase_table(ctx, M: int, N: int, K: int, g) -> int:
         cnt[0] += 1
         ctx.linear_packed_i8_f32(pa[i], sa, pw[i], sw, bias, M, N, K, out=outs[i])
 
-    return phase_table(f"packed GEMM M={M} N={N} K={K}", ctx, launch, waves, reps)
+    if pairs:  # one 128 x 128 tile per pair of compute units (test hook 12): two workgroups per tile
+        ctx.set_gemm_kernel_variant(12)
+        waves = (M // 128) * (N // 128) * 2 * 4
+        rc = phase_table(f"packed GEMM M={M} N={N} K={K}, one 128x128 tile per pair of compute units", ctx, launch,
+                         waves, reps, PHASES_PAIR)
+        ms = event_time_ms(launch, reps=400, warmup=20)
+        print(f"launch to launch without the stamps (HIP events): {ms * 1e3:.2f} us")
+        ctx.set_gemm_kernel_variant(0)
+        return rc
+    rc = phase_table(f"packed GEMM M={M} N={N} K={K}", ctx, launch, waves, reps)
+    ms = event_time_ms(launch, reps=400, warmup=20)
+    print(f"launch to launch without the stamps (HIP events): {ms * 1e3:.2f} us")
+    return rc
 
 
-def phase_table(title: str, ctx, launch, waves: int, reps: int = 200) -> int:
+PHASES_TILE = ["start -> first operands in registers", "K loop (first operands -> last MFMA retired)",
+               "4-way K-split sum through LDS (incl. waiting for the slowest wave)", "convert + issue stores",
+               "stores retired", "whole wave"]
+PHASES_PAIR = ["start -> first operands in registers", "K loop (first operands -> last MFMA retired)",
+               "4-way K-split sum through LDS in two rounds; partials for the partner stored",
+               "partner's flag seen, its partials read (past the L1) and added", "convert + stores issued and retired",
+               "whole wave"]
+
+
+def phase_table(title: str, ctx, launch, waves: int, reps: int = 200, names=None) -> int:
     """Runs `launch` (one call = one launch of the packed kernel) `reps` times with the trace buffer set and prints
     the phase medians."""
     import torch
@@ -226,9 +247,7 @@ def phase_table(title: str, ctx, launch, waves: int, reps: int = 200) -> int:
     ctx.set_trace_buffer(None)
     ctx.synchronize()
     t = trace.cpu().double()
-    names = ["start -> first operands in registers", "K loop (first operands -> last MFMA retired)",
-             "4-way K-split sum through LDS (incl. waiting for the slowest wave)", "convert + issue stores",
-             "stores retired", "whole wave"]
+    names = names or PHASES_TILE
     spans = [(0, 1), (1, 2), (2, 3), (3, 4), (4, 5), (0, 5)]
     ghz = (t[:, :, 5] - t[:, :, 0]) / ((t[:, :, 7] - t[:, :, 6]).clamp(min=1) * 10.0) / 1e0  # cycles per ns
     clock = ghz.median(dim=1).values
@@ -250,6 +269,63 @@ def phase_table(title: str, ctx, launch, waves: int, reps: int = 200) -> int:
     return 0
 
 
+def vector_memory_path_table(ctx) -> int:
+    """What the vector-memory path of a compute unit and the matrix pipes deliver on this device, by the probe
+    kernel's own clocks (hipq_probe_vector_memory_path): 1 KiB fragment loads as the packed GEMM issues them, alone,
+    with MFMAs, and MFMAs alone; 8 workgroups (one per XCD: a compute unit with the XCD's L2 to itself) or one per
+    compute unit; lines private to a compute unit or shared by four of an XCD; out of the L2 (64 KiB regions walked many times; the last of three runs) or from memory (2 MiB regions
+    walked once, a part of a 1 GiB buffer that no earlier run has touched)."""
+    import torch
+
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    buf = torch.randint(-128, 128, (1 << 30,), device="cuda", dtype=torch.int8)
+    print(f"device: {cus} compute units.  A step = `loads` coalesced 1 KiB loads and `MFMAs` v_mfma_i32_32x32x32_i8 per "
+          f"wave, four waves per workgroup.  B/clk/CU = bytes requested per shader-clock cycle and compute unit (median "
+          f"over workgroups, times workgroups per compute unit); GHz = shader cycles per 10 ns tick of the constant "
+          f"counter (median); TB/s and POP/s are chip-wide, from the slowest workgroup's wall time.")
+    print(f"{'workgroups':>10s} {'source':>22s} {'share':>5s} {'loads':>5s} {'MFMAs':>5s} {'steps':>5s} {'cycles/step':>11s} "
+          f"{'ns/step':>8s} {'B/clk/CU':>9s} {'GHz':>5s} {'TB/s':>6s} {'POP/s':>6s}")
+    l2, mem = 64 << 10, 2 << 20
+    rows = []
+    for wgs in (8, cus):
+        for share in (1, 4):
+            for loads, mfmas in ((6, 0), (8, 0), (0, 8), (0, 16), (6, 8), (8, 16), (4, 8)):
+                if loads == 0 and share != 1:
+                    continue
+                rows.append((wgs, "L2 (64 KiB regions)", l2, 512, share, loads, mfmas))
+        for loads, mfmas in ((6, 0), (6, 8)):
+            rows.append((wgs, "memory (2 MiB regions)", mem, 64, 1, loads, mfmas))
+    # the same work in a burst as short as the GEMM's main loop (32 steps), launched back to back
+    rows.append((cus, "L2 (64 KiB regions)", l2, 32, 4, 6, 8))
+    rows.append((cus, "L2 (64 KiB regions)", l2, 32, 4, 4, 8))
+    out = torch.zeros(2 * cus, 3, dtype=torch.int64, device="cuda")
+    fresh = 0  # bytes of `buf` the memory rows have used up
+    for wgs, source, region, steps, share, loads, mfmas in rows:
+        base = buf
+        runs = 3 if steps > 32 else 50
+        if region == mem:
+            need = 8 * ((wgs + 7) // 8 + 2) * region
+            if fresh + need > buf.numel():
+                continue
+            base, fresh, runs = buf[fresh:], fresh + need, 1
+        for _ in range(runs):
+            ctx.call("hipq_probe_vector_memory_path", base.data_ptr(), base.numel(), wgs, region, share, loads, mfmas,
+                     steps, out.data_ptr())
+        ctx.synchronize()
+        o = out[:wgs].cpu().double()
+        cyc, ticks = o[:, 0], o[:, 1]
+        per_cu = max(1, wgs // cus)
+        nbytes = loads * 1024 * 4 * steps
+        bpc = nbytes / cyc.median().item() * per_cu
+        ghz = (cyc / (ticks * 10.0)).median().item()
+        wall = ticks.max().item() * 1e-8
+        tbs = nbytes * wgs / wall / 1e12
+        pops = mfmas * 65536.0 * 4 * steps * wgs / wall / 1e15
+        print(f"{wgs:10d} {source:>22s} {share:5d} {loads:5d} {mfmas:5d} {steps:5d} {cyc.median().item() / steps:11.1f} "
+              f"{ticks.median().item() * 10.0 / steps:8.1f} {bpc:9.1f} {ghz:5.2f} {tbs:6.2f} {pops:6.2f}")
+    return 0
+
+
 def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
     """A handful of launches of one kernel on HBM-cold operands, for rocprofv3 --pmc / --kernel-trace passes.
 
@@ -261,8 +337,12 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
 
     g = torch.Generator(device="cuda").manual_seed(2)
     reps = 20
+    if which == "vmem_path":
+        return vector_memory_path_table(ctx)
     if which == "gemm_phases":
         return gemm_phase_table(ctx, M, N, K, g)
+    if which == "gemm_pair_phases":
+        return gemm_phase_table(ctx, M, N, K, g, pairs=True)
     if which == "conv_phases":
         return conv_phase_table(ctx, g)
     if which in ("gemm", "gemm_rowmajor"):
@@ -439,7 +519,7 @@ def main() -> int:
                     help="milliseconds of untimed back-to-back launches before each timed region (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "conv_phases", "gemm_rowmajor", "step", "quantize", "per_channel", "calib", "special", "copy",
+    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "gemm_pair_phases", "vmem_path", "conv_phases", "gemm_rowmajor", "step", "quantize", "per_channel", "calib", "special", "copy",
                                           "stack", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()

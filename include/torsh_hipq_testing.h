@@ -24,8 +24,9 @@ extern "C" {
  * the forms of the GEMM that are picked by occupancy - two workgroups per compute unit, the
  * weight-streaming kernel for 33..128 rows - (9) and the touching of weight / filter lines by the
  * one-launch activation quantizers of the dynamic Linear and Conv2d forwards while their grids wait
- * for the range (11); 12 keeps the headline shape on the one-tile-per-compute-unit form where the
- * K-split-across-compute-units form would be picked. */
+ * for the range (11); 12 runs shapes of whole 128 x 128 tiles that fill the device once as one tile
+ * per PAIR of compute units, K halved between the two, partial sums exchanged through their XCD's L2
+ * (measured slower than the default forms; kept as a measured alternative). */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
 /* Some kernels couple their waves through device memory: the persistent GEMM kernel (counters
  * between producer and consumer waves), the one-launch dynamic quantizers (their workgroups meet to
@@ -44,6 +45,17 @@ HIPQ_API int32_t hipq_ctx_set_wait_spin_limit(hipq_ctx *ctx, int32_t limit);
  * the grid (otherwise the ordinary kernel runs).  The results are the same bits.  null removes the
  * buffer.  bench.py --profile gemm_phases prints the phase table from it. */
 HIPQ_API int32_t hipq_ctx_set_trace_buffer(hipq_ctx *ctx, void *device_buffer, size_t bytes);
+
+/* Machine probe: what a compute unit's vector-memory path and matrix pipes deliver, by the kernel's own clocks.
+ * `workgroups` workgroups of four waves; every step a wave requests `loads_per_step` fragments of 1 KiB (one
+ * coalesced 16-byte-per-lane load each, as the packed GEMM does) and issues `mfmas_per_step`
+ * v_mfma_i32_32x32x32_i8; (loads, MFMAs) one of (6,0) (8,0) (0,8) (0,16) (6,8) (8,16) (4,8); `steps` even.  The
+ * workgroups walk regions of `region_bytes` (a power of two) of `buf` round and round, `share` workgroups of one XCD
+ * per region.  out (device): per workgroup {shader-clock cycles, 100 MHz ticks, checksum} as uint64.
+ * bench.py --profile vmem_path prints the table. */
+HIPQ_API int32_t hipq_probe_vector_memory_path(hipq_ctx *ctx, const int8_t *buf, size_t buf_bytes, int32_t workgroups,
+                                               int32_t region_bytes, int32_t share, int32_t loads_per_step,
+                                               int32_t mfmas_per_step, int32_t steps, uint64_t *out);
 
 #ifdef __cplusplus
 }

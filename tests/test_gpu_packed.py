@@ -64,6 +64,42 @@ def test_gemm_packed_bit_exact(ctx, oracle, m, n, k):
     np.testing.assert_array_equal(got, oracle.gemm_i8_nk(a, w))
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (512, 4096, 512), (1024, 2048, 1024), (256, 8192, 1536), (128, 16384, 512)])
+def test_gemm_one_tile_per_pair_of_compute_units(hipq, oracle, m, n, k):
+    """Test hook 12: one 128 x 128 tile per pair of compute units, K halved between the two workgroups, which exchange
+    partial sums through the L2 of the XCD they share (shapes of whole tiles that fill the device once).  int32
+    accumulators against an exact float64 product (and the oracle where it finishes in a second), the fp32
+    epilogue with per-tensor and per-row activation scales against the same individually rounded f32 expression,
+    and the same bits as the default form; twice in a row, since the exchange flags must be back at zero."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(m + n + k)
+        a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+        w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+        ref = torch.empty((m, n), dtype=torch.int32, device="cuda")
+        wd = w.double().T.contiguous()
+        for r0 in range(0, m, 128):
+            ref[r0:r0 + 128] = (a[r0:r0 + 128].double() @ wd).to(torch.int32)  # exact: |acc| < 2^53
+        if m * n * k <= 512 * 4096 * 512:
+            np.testing.assert_array_equal(host(ref), oracle.gemm_i8_nk(host(a), host(w)))
+        pa, pw = c.pack_rows(a), c.pack_rows(w)
+        sa = torch.rand(m, generator=g, device="cuda") * 0.05 + 0.01
+        sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+        bias = torch.randn(n, generator=g, device="cuda") * 0.01
+        default = c.linear_packed_i8_f32(pa, sa, pw, sw, bias, m, n, k)
+        c.set_gemm_kernel_variant(12)
+        for _ in range(2):
+            assert torch.equal(c.gemm_packed_i8_i32(pa, pw, m, n, k), ref)
+            got = c.linear_packed_i8_f32(pa, sa, pw, sw, bias, m, n, k)
+            assert torch.equal(got, ref.float() * (sa[:, None] * sw[None, :]) + bias[None, :])
+            assert torch.equal(got, default)
+            got = c.linear_packed_i8_f32(pa, sa[:1], pw, sw, None, m, n, k)
+            assert torch.equal(got, ref.float() * (sa[0] * sw[None, :]))
+        c.synchronize()  # no wait of the exchange gave up
+    finally:
+        c.close()
+
+
 def test_gemm_packed_extreme_values(ctx):
     a = np.full((32, 4096), -128, np.int8)
     pa = ctx.pack_rows(dev(a))

@@ -67,6 +67,44 @@ int32_t scratch(hipq_ctx *ctx, size_t bytes, void **out) {
     return HIPQ_SUCCESS;
 }
 
+int32_t pair_area(hipq_ctx *ctx, size_t flag_bytes, size_t buf_bytes, uint32_t **flags, int8_t **buf) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(ctx->stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
+    if (capturing) ctx->scratch_captured = true;
+    const size_t flags_up = (flag_bytes + 255) & ~size_t(255);
+    if (flags_up > ctx->pair_flag_bytes || flags_up + buf_bytes > ctx->pair_bytes) {
+        if (capturing)
+            return fail(HIPQ_ALLOCATION_ERROR,
+                        "pair exchange area: memory cannot be allocated while the stream is capturing - run the same "
+                        "call once before the capture");
+        // The flags of a larger area start further on, and flags must be zero: a fresh, zeroed block (the stream is
+        // drained first, so no launch is using the old one).
+        hipError_t e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return fail(HIPQ_SYNCHRONIZATION_ERROR, "pair exchange area: %s", hipGetErrorString(e));
+        const size_t fl = flags_up > ctx->pair_flag_bytes ? flags_up : ctx->pair_flag_bytes;
+        const size_t want = (fl + buf_bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        void *grown = nullptr;
+        e = hipMalloc(&grown, want);
+        if (e == hipSuccess) e = hipMemset(grown, 0, fl);
+        if (e != hipSuccess) {
+            if (grown) (void)hipFree(grown);
+            return fail(HIPQ_ALLOCATION_ERROR, "pair exchange area: %zu bytes: %s", want, hipGetErrorString(e));
+        }
+        if (ctx->pair_area) {
+            if (ctx->scratch_captured)
+                ctx->retired.push_back(ctx->pair_area);
+            else
+                (void)hipFree(ctx->pair_area);
+        }
+        ctx->pair_area = grown;
+        ctx->pair_flag_bytes = fl;
+        ctx->pair_bytes = want;
+    }
+    *flags = static_cast<uint32_t *>(ctx->pair_area);
+    *buf = static_cast<int8_t *>(ctx->pair_area) + ctx->pair_flag_bytes;
+    return HIPQ_SUCCESS;
+}
+
 int32_t check_launch(const char *what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HIPQ_DEVICE_ERROR, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
@@ -77,6 +115,8 @@ int32_t reset_ctx_words(hipq_ctx *ctx) {
     hipError_t e = hipMemset(ctx->wait_error, 0, kCtxWordsBytes);
     const uint32_t epoch = kCtxFirstEpoch;
     if (e == hipSuccess) e = hipMemcpy(ctx->wait_error + kCtxEpochWord, &epoch, sizeof(epoch), hipMemcpyHostToDevice);
+    // (flags of the pair exchange: a launch that gave up may have left some set)
+    if (e == hipSuccess && ctx->pair_area) e = hipMemset(ctx->pair_area, 0, ctx->pair_flag_bytes);
     if (e != hipSuccess) return fail(HIPQ_DEVICE_ERROR, "status words of the context: %s", hipGetErrorString(e));
     return HIPQ_SUCCESS;
 }
@@ -139,6 +179,7 @@ static int32_t ctx_new(int32_t device, hipStream_t stream, bool own, hipq_ctx **
         return rc;
     }
     (void)hipq::four_wide_workgroups_fit(ctx);  // asked here so that no later call is the first
+    ctx->pair_ok = hipq::pairs_share_an_xcd(ctx);
     *out_ctx = ctx;
     return HIPQ_SUCCESS;
 }
@@ -157,6 +198,7 @@ int32_t hipq_ctx_destroy(hipq_ctx *ctx) {
     HIPQ_ENTER(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->pair_area) (void)hipFree(ctx->pair_area);
     for (void *p : ctx->retired) (void)hipFree(p);
     if (ctx->wait_error) (void)hipFree(ctx->wait_error);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);

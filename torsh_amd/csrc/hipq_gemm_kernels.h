@@ -137,10 +137,11 @@ __device__ __forceinline__ void divmod_uniform(int a, int d, int *q, int *r) {
     }
 }
 
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int gm, int gn, int *tm, int *tn) {
-    const int b = blockIdx.x;
+// Tile of slot i (0, 1, ...) of XCD x: with a rectangle (gm > 0) the i-th tile of the XCD's rectangle, column
+// major; without one, tile x + 8 * i in id order.
+__device__ __forceinline__ void tile_of_xcd_slot(int tiles_m, int tiles_n, int gm, int gn, int x, int i, int *tm,
+                                                 int *tn) {
     if (gm > 0) {
-        const int x = b % 8, i = b / 8;  // XCD, index within the XCD's rectangle
         int blocks_m, unused, xq, xr, iq, ir;   // rectangles along M
         divmod_uniform(tiles_m, gm, &blocks_m, &unused);
         divmod_uniform(x, blocks_m, &xq, &xr);
@@ -149,8 +150,14 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int gm, 
         *tn = xq * gn + iq;
         return;
     }
+    const int b = x + 8 * i;
     *tm = b % tiles_m;
     *tn = b / tiles_m;
+}
+
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int gm, int gn, int *tm, int *tn) {
+    const int b = blockIdx.x;
+    tile_of_xcd_slot(tiles_m, tiles_n, gm, gn, b % 8, b / 8, tm, tn);  // XCD, index within the XCD's rectangle
 }
 
 // Host side: the rectangle for tile_of_block, or (0, 0) when the tile grid does not split into 8

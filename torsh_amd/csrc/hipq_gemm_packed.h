@@ -210,6 +210,10 @@ __device__ __forceinline__ void conv_store_block(v16i (&own)[1][TNB], const Gemm
 // different step).  Activations that the previous kernel has just written are served by the memory-side
 // cache, where the same stagger costs 0.4 us instead: the fused forwards switch it off.
 //
+// Issuing the loads of a stage between the MFMAs of the stage being multiplied (a third register slot, one load
+// behind each of the first six MFMAs, the order pinned with sched_group_barrier) instead of behind all eight was
+// measured: K loop 19.6 k -> 18.4 k cycles under the stamps, 14.7 us from launch to launch either way.  Not kept.
+//
 // CONV: implicit-GEMM convolution on the same loop.  The row operand PA holds the packed filters (M = output
 // channels, K = taps x channels, tap-major), the column operand PW is the image as signed bytes in
 // [channel block of 32][padded pixel][32 bytes] order (conv_pack_image_kernel), N = padded pixels = windows:
@@ -969,6 +973,12 @@ __global__ __launch_bounds__(256) void pack_rows_i8_kernel(const int8_t *__restr
     }
 }
 
+}  // namespace hipq
+
+#include "hipq_gemm_pair.h"
+
+namespace hipq {
+
 template <int TMB, int TNB, int D, int EPI, bool EVEN, bool TRACE = false, bool CONV = false, bool HALVES = false>
 static int32_t launch_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t *pw, int M, int N, int K,
                              const GemmEpilogue &ep) {
@@ -1013,6 +1023,12 @@ static int32_t launch_gemm_packed(hipq_ctx *ctx, const int8_t *pa, const int8_t 
     //   N = 4096, K = 11264: M = 128 36.9 / 26.3  256 34.0 / 25.4  384 32.9 / 38.3
     //   N = 8192, K = 2048:  M = 128  8.8 / 7.9;  N = 2304, K = 768: M = 384 6.0 / 5.3, 512 6.0 / 6.2
     //   N = 11008, K = 4096: M = 128 18.8 / 20.5  256 30.0 / 31.2  512 39.4 / 58.6   (344 and more 64 x 64 tiles)
+    if (ctx->gemm_variant == 12) {
+        // Test hook: one 128 x 128 tile per pair of compute units, K halved between them (hipq_gemm_pair.h), where
+        // the shape allows it.  Measured slower than the forms below at every shape tried, so never the default.
+        int32_t rc = HIPQ_SUCCESS;
+        if (launch_pair_if_fits<EPI, EVEN>(ctx, pa, pw, m, n, k, ep, &rc)) return rc;
+    }
     if (ctx->gemm_variant != 9 && !ctx->trace) {  // (the phase stamps are the 128 x 64 kernel's)
         const size_t tiles64 = ((packed_row_blocks(m) + 1) / 2) * ((packed_row_blocks(n) + 1) / 2);
         if (M <= 64 || tiles64 <= size_t(ctx->num_cus)) return launch_skinny_packed<EPI, EVEN>(ctx, pa, pw, M, N, K, ep);

@@ -43,6 +43,31 @@ static PackedScratch packed_scratch_layout(int num_cus, size_t m, size_t k) {
 
 size_t packed_operand_bytes(size_t rows, size_t k) { return packed_bytes(rows, k); }
 
+// The pair form relies on the dispatcher handing workgroup ids b and b + 8 to one XCD.  Asked of the device once:
+// a grid of one workgroup per compute unit records the XCD each workgroup ran on.
+bool pairs_share_an_xcd(hipq_ctx *ctx) {
+    static int known[16] = {0};  // 1 = yes, -1 = no
+    if (ctx->device < 0 || ctx->device >= 16) return false;
+    if (known[ctx->device] == 0) {
+        int verdict = -1;
+        const int n = ctx->num_cus;
+        uint32_t *dev = nullptr;
+        if (n >= 16 && n <= 4096 && hipMalloc(reinterpret_cast<void **>(&dev), size_t(n) * 4) == hipSuccess) {
+            uint32_t host[4096];
+            hipLaunchKernelGGL(xcc_probe_kernel, dim3(n), dim3(64), 0, ctx->stream, dev);
+            if (hipGetLastError() == hipSuccess && hipStreamSynchronize(ctx->stream) == hipSuccess &&
+                hipMemcpy(host, dev, size_t(n) * 4, hipMemcpyDeviceToHost) == hipSuccess) {
+                verdict = 1;
+                for (int b = 8; b < n; ++b)
+                    if (host[b] != host[b - 8]) verdict = -1;
+            }
+            (void)hipFree(dev);
+        }
+        known[ctx->device] = verdict;
+    }
+    return known[ctx->device] > 0;
+}
+
 // Implicit-GEMM convolution on the packed kernel: picks the register depth (the largest of 4, 3, 2, 1 that
 // divides the k blocks per wave) and the epilogue.
 template <int EPI, bool EVEN>

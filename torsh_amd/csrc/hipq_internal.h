@@ -35,6 +35,12 @@ struct hipq_ctx {
     bool scratch_captured = false;
     std::vector<void *> retired;
     int num_cus = 256;
+    // Exchange area of the GEMM form whose workgroup pairs hand partial sums to each other (hipq_gemm_pair.h):
+    // flag words (zero between launches), then the buffer.  Grown like the scratch; pair_ok: the device hands
+    // workgroup ids b and b + 8 to the same XCD (checked by hipq_ctx_create).
+    void *pair_area = nullptr;
+    size_t pair_flag_bytes = 0, pair_bytes = 0;
+    bool pair_ok = false;
     // Device words of the context (kCtxWordsBytes of them, laid out as the kCtx* constants below say).  Word 0 is
     // set by a kernel whose bounded wait gave up; hipq_ctx_synchronize reads and clears it.
     uint32_t *wait_error = nullptr;
@@ -88,6 +94,11 @@ void clear_error();
 int32_t enter(hipq_ctx *ctx);
 // Ensures ctx->scratch holds at least `bytes`; returns pointer via out.
 int32_t scratch(hipq_ctx *ctx, size_t bytes, void **out);
+// Ensures the pair-exchange area holds `flag_bytes` of zeroed flag words followed (256-byte aligned) by
+// `buf_bytes`; returns both pointers.  Same rules under stream capture as the scratch.
+int32_t pair_area(hipq_ctx *ctx, size_t flag_bytes, size_t buf_bytes, uint32_t **flags, int8_t **buf);
+// Whether workgroup ids 8 apart run on one XCD on this device (asked of the device once, remembered).
+bool pairs_share_an_xcd(hipq_ctx *ctx);
 // Checks the sticky launch error after a kernel launch.
 int32_t check_launch(const char *what);
 
