@@ -326,6 +326,43 @@ def vector_memory_path_table(ctx) -> int:
     return 0
 
 
+def quantize_sweep_table(ctx) -> int:
+    """The streaming kernels of configs[0] against tensor size: how much of a 16 Mi-element launch is ramp and tail,
+    and what the stream itself reaches once it is long.  Operands rotate through at least 1 GiB (more than the
+    memory-side cache holds); HIP events around back-to-back launches on the launch stream."""
+    import torch
+
+    from torsh_amd import hipq
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    mm = torch.empty(2, device="cuda")
+    params = ctx.new_qparams()
+    print(f"{'elements':>10s} {'kernel':>34s} {'us':>9s} {'GB/s':>8s} {'of 8 TB/s':>9s}   (bytes that move per element)")
+    for mi in (1, 4, 16, 64, 256):
+        n = mi << 20
+        sets = max(2, min(16, (1 << 30) // (4 * n)))
+        xs = [torch.randn(n, generator=g, device="cuda") for _ in range(sets)]
+        qs = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(sets)]
+        ys = [torch.empty(n, device="cuda") for _ in range(min(sets, 4) if mi >= 64 else sets)]
+        k = [0]
+
+        def rot(pool):
+            k[0] += 1
+            return pool[k[0] % len(pool)]
+
+        runs = (("quantize f32 -> i8 (given scale)", 5, lambda: ctx.quantize_per_tensor_i8(rot(xs), 0.04, 0, hipq.FORM_MUL_INV, out=rot(qs))),
+                ("dequantize i8 -> f32", 5, lambda: ctx.dequantize(rot(qs), 0.04, 0, out=rot(ys))),
+                ("min/max of f32", 4, lambda: ctx.call("hipq_minmax_f32", rot(xs).data_ptr(), n, mm.data_ptr())),
+                ("dynamic quantize (range + codes)", 5 if mi <= 16 else 9,
+                 lambda: ctx.quantize_dynamic_per_tensor(rot(xs), out=rot(qs), params=params)))
+        for name, bytes_per, fn in runs:
+            ms = event_time_ms(fn, reps=max(10, 400 // mi), warmup=3)
+            gbps = bytes_per * n / (ms * 1e-3) / 1e9
+            print(f"{n:10d} {name:>34s} {ms * 1e3:9.2f} {gbps:8.0f} {gbps / PEAK_HBM_GBPS:9.3f}   ({bytes_per})")
+        del xs, qs, ys
+    return 0
+
+
 def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
     """A handful of launches of one kernel on HBM-cold operands, for rocprofv3 --pmc / --kernel-trace passes.
 
@@ -339,6 +376,8 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
     reps = 20
     if which == "vmem_path":
         return vector_memory_path_table(ctx)
+    if which == "quantize_sweep":
+        return quantize_sweep_table(ctx)
     if which == "gemm_phases":
         return gemm_phase_table(ctx, M, N, K, g)
     if which == "gemm_pair_phases":
@@ -519,7 +558,7 @@ def main() -> int:
                     help="milliseconds of untimed back-to-back launches before each timed region (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "gemm_pair_phases", "vmem_path", "conv_phases", "gemm_rowmajor", "step", "quantize", "per_channel", "calib", "special", "copy",
+    ap.add_argument("--profile", choices=["gemm", "gemm_phases", "gemm_pair_phases", "vmem_path", "quantize_sweep", "conv_phases", "gemm_rowmajor", "step", "quantize", "per_channel", "calib", "special", "copy",
                                           "stack", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()

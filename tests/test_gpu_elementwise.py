@@ -426,13 +426,15 @@ def test_per_channel_auto_spread_half_even_and_bad_groups(ctx, hipq, oracle):
 
 
 @pytest.mark.parametrize("shape,axis", [((3, 8, 12), 0), ((3, 8, 12), 1), ((7, 5, 2048), 1), ((6, 1000), 0),
-                                        ((300, 64, 36), 1), ((1, 1, 4), 2), ((257, 4100), 0), ((16, 4096), 1)])
+                                        ((300, 64, 36), 1), ((1, 1, 4), 2), ((257, 4100), 0), ((16, 4096), 1),
+                                        ((8, 16384), 0), ((2, 64, 1024), 1)])
 def test_per_channel_vector_forms(ctx, hipq, oracle, shape, axis):
     """Explicit-parameter per-channel quantize / dequantize where the run of one channel is a multiple of four
     elements (the kernels then work on vectors of four): power-of-two and other run lengths and channel counts,
     whole tiles and ragged tails, both rounding forms; and the same data one element off alignment, which takes
     the element-wise kernels and must give the same bytes."""
     x = normal(77 + axis, shape) * 3
+    x.reshape(-1)[:4] = [np.nan, np.inf, -np.inf, 1e30]  # NaN -> the zero point's code; infinities saturate
     ch = shape[axis]
     rng = np.random.default_rng(9)
     scales = rng.uniform(0.01, 0.05, ch).astype(np.float32)
@@ -455,7 +457,8 @@ def test_per_channel_vector_forms(ctx, hipq, oracle, shape, axis):
     if axis == 0 and len(shape) == 2:
         want = oracle.quantize_per_channel_simd(x, scales, zps, shape[1])
         got = ctx.quantize_per_channel(dev(x), dev(scales), dev(zps), 0, hipq.FORM_MUL_INV)
-        np.testing.assert_array_equal(host(got), want.astype(np.int8))
+        # (the reference's f32 carrier keeps a NaN; as an int8 code it is 0, Rust's `NaN as i8`)
+        np.testing.assert_array_equal(host(got), np.nan_to_num(want, nan=0.0).astype(np.int8))
 
 
 @pytest.mark.parametrize("shape", [(1, 1), (5, 9), (64, 256), (100, 333)])
@@ -471,6 +474,34 @@ def test_requantize(ctx, hipq, oracle, shape):
     want = oracle.requantize_epilogue(acc, sa, sw, None, 0.31, 0)
     got = host(ctx.requantize(dev(acc), dev(sa), dev(sw), None, 0.31, 0))
     np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("rows,cols", [(2304, 4096), (3000, 3072), (800, 11008), (4100, 2052), (16384, 768)])
+def test_requantize_large_tensors_with_columns_fixed_per_thread(ctx, hipq, oracle, rows, cols):
+    """Tensors of several tiles per workgroup take the form of the requantize kernel in which a thread meets the
+    same column vectors in every tile and loads their weight scales and biases once (the grid is then a multiple of
+    a period that depends on cols: 1, 3, 43, 513, 3 here).  One block of rows repeated, expected bytes from the
+    oracle on the block; one activation scale and one per row, with and without bias, both roundings."""
+    brows = 37
+    reps = -(-rows // brows)
+    rng = np.random.default_rng(rows + cols)
+    acc0 = rng.integers(-3_000_000, 3_000_000, size=(brows, cols), dtype=np.int32)
+    acc0[0, :8] = [2**31 - 1, -2**31, 0, 1, -1, 2_000_000_000, -2_000_000_000, 77]  # saturation either side
+    sw = rng.uniform(1e-4, 1e-3, cols).astype(np.float32)
+    bias = (rng.standard_normal(cols) * 0.01).astype(np.float32)
+    acc = dev(acc0).repeat(reps, 1)[:rows].contiguous()
+    for sa0 in (np.array([0.02], np.float32), rng.uniform(0.01, 0.03, brows).astype(np.float32)):
+        sa = dev(sa0) if sa0.size == 1 else dev(sa0).repeat(reps)[:rows].contiguous()
+        for b in (bias, None):
+            for mode, rm in ((hipq.ROUND_HALF_AWAY, 0), (hipq.ROUND_HALF_EVEN, 1)):
+                oracle.set_round_mode(rm)
+                try:
+                    want = oracle.requantize_epilogue(acc0, sa0, sw, b, 0.31, -3)
+                finally:
+                    oracle.set_round_mode(0)
+                got = ctx.requantize(acc, sa, dev(sw), None if b is None else dev(b), 0.31, -3, mode)
+                torch.cuda.synchronize()
+                assert torch.equal(got, dev(want).repeat(reps, 1)[:rows]), (sa0.size, b is None, mode)
 
 
 @pytest.mark.parametrize("n", [4, 1024, 8192, 8196, 1 << 20, 4096 * 4096, 4096 * 4096 + 8192])

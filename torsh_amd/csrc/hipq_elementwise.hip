@@ -5,6 +5,8 @@
 // latency, and wave-level shuffles for the reductions.
 #include "hipq_internal.h"
 #include "hipq_math.h"
+#include <type_traits>
+
 #include "hipq_meeting.h"
 
 namespace hipq {
@@ -661,7 +663,9 @@ __global__ __launch_bounds__(kBlock) void dequantize_kernel(const InT *__restric
 // per row; 16: up to 16384).  What does not fit is read again, one dependent round trip per 1024 floats in each phase,
 // which is what a long row costs (a single row of 11008 floats: 7.3 us with KC = 4, a round trip less per 4096 floats
 // with 16).
-template <int TPR, bool EVEN, bool PACKED = false, int KC = 4>
+// STREAM: a large dense tensor that is read and written once goes past the caches (non-temporal accesses), as in
+// the per-tensor quantizer.
+template <int TPR, bool EVEN, bool PACKED = false, int KC = 4, bool STREAM = false>
 __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *__restrict__ x, size_t rows,
                                                                    size_t cols, size_t ld, int flavor, int qmin,
                                                                    int qmax,
@@ -692,7 +696,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
 #pragma unroll
         for (int i = 0; i < kCache; ++i) {
             const size_t v = size_t(lane) + size_t(i) * TPR;
-            if (v < nvec) cache[i] = x4[v];
+            if (v < nvec) cache[i] = STREAM ? load_stream(x4 + v) : x4[v];
         }
 #pragma unroll
         for (int i = 0; i < kCache; ++i) {
@@ -758,6 +762,8 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     auto put4 = [&](size_t v, uint32_t w) {
         if constexpr (PACKED)
             *reinterpret_cast<uint32_t *>(prow + packed_k(v * 4)) = w;
+        else if constexpr (STREAM)
+            store_stream(q4 + v, w);
         else
             q4[v] = w;
     };
@@ -1076,30 +1082,68 @@ __global__ __launch_bounds__(kBlock) void quantize_per_channel_vec_kernel(const 
     const ChannelOfVector channel_of(inner, channels, nvec);
     const float4 *x4 = reinterpret_cast<const float4 *>(x);
     uint32_t *out4 = reinterpret_cast<uint32_t *>(out);
-    auto emit = [&](size_t j, const float4 &t) {
-        const size_t c = channel_of(j);
-        const float s = scales[c], zpf = static_cast<float>(zps[c]);
-        const float inv = DIV ? 0.0f : 1.0f / s;  // the division form divides directly, as the scalar kernel does
-        auto one = [&](float v) { return to_int_nan0(quantize_value<DIV, EVEN>(v, s, inv, zpf, -128.0f, 127.0f)); };
-        store_stream(out4 + j, pack4(one(t.x), one(t.y), one(t.z), one(t.w)));
-    };
-    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
-    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const size_t base = t * kTileVec + threadIdx.x;
-        if ((t + 1) * kTileVec <= nvec) {
-            float4 v[kVecPerThread];
+    // How a vector's channel is found (shifts / 32-bit divisions / 64-bit divisions) is decided once, outside the
+    // loop: inside it the choice would be three branches per vector between the loads and the stores.
+    auto run = [&](auto shifts, auto small) {
+        auto channel = [&](size_t j) -> size_t {
+            if constexpr (decltype(shifts)::value)
+                return (j >> channel_of.vpc_shift) & (channels - 1);
+            else if constexpr (decltype(small)::value)
+                return (static_cast<uint32_t>(j) / static_cast<uint32_t>(channel_of.vpc)) % static_cast<uint32_t>(channels);
+            else
+                return channel_of(j);
+        };
+        auto emit = [&](size_t j, const float4 &t) {
+            const size_t c = channel(j);
+            const float s = scales[c], zpf = static_cast<float>(zps[c]);
+            // One reciprocal per vector: the division form then gets the correctly rounded quotient from two FMAs
+            // (div_rn: the same bits as the scalar kernel's x / s), the other form multiplies by it.
+            const float inv = DIV ? recip_for_div(s) : 1.0f / s;
+            auto one = [&](float v) { return quantize_int<DIV ? QFORM_DIV : QFORM_MUL, EVEN>(v, s, inv, zpf, -128, 127); };
+            store_stream(out4 + j, pack4(one(t.x), one(t.y), one(t.z), one(t.w)));
+        };
+        const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+        for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+            const size_t base = t * kTileVec + threadIdx.x;
+            if ((t + 1) * kTileVec <= nvec) {
+                float4 v[kVecPerThread];
 #pragma unroll
-            for (int i = 0; i < kVecPerThread; ++i) v[i] = load_stream(x4 + base + size_t(i) * kBlock);
+                for (int i = 0; i < kVecPerThread; ++i) v[i] = load_stream(x4 + base + size_t(i) * kBlock);
+                // The usual case - runs of a channel much longer than a tile - has the thread's vectors in one
+                // channel: its scale, zero point and reciprocal then once, not once per vector.
+                size_t c[kVecPerThread];
+                bool same = true;
 #pragma unroll
-            for (int i = 0; i < kVecPerThread; ++i) emit(base + size_t(i) * kBlock, v[i]);
-        } else {
+                for (int i = 0; i < kVecPerThread; ++i) {
+                    c[i] = channel(base + size_t(i) * kBlock);
+                    same = same && c[i] == c[0];
+                }
+                if (same) {
+                    const float s = scales[c[0]], zpf = static_cast<float>(zps[c[0]]);
+                    const float inv = DIV ? recip_for_div(s) : 1.0f / s;
+                    auto one = [&](float f) { return quantize_int<DIV ? QFORM_DIV : QFORM_MUL, EVEN>(f, s, inv, zpf, -128, 127); };
 #pragma unroll
-            for (int i = 0; i < kVecPerThread; ++i) {
-                const size_t j = base + size_t(i) * kBlock;
-                if (j < nvec) emit(j, x4[j]);
+                    for (int i = 0; i < kVecPerThread; ++i)
+                        store_stream(out4 + base + size_t(i) * kBlock, pack4(one(v[i].x), one(v[i].y), one(v[i].z), one(v[i].w)));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < kVecPerThread; ++i) emit(base + size_t(i) * kBlock, v[i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < kVecPerThread; ++i) {
+                    const size_t j = base + size_t(i) * kBlock;
+                    if (j < nvec) emit(j, x4[j]);
+                }
             }
         }
-    }
+    };
+    if (channel_of.vpc_pow2 && channel_of.ch_pow2)
+        run(std::true_type{}, std::true_type{});
+    else if (channel_of.small)
+        run(std::false_type{}, std::true_type{});
+    else
+        run(std::false_type{}, std::false_type{});
 }
 
 __global__ __launch_bounds__(kBlock) void dequantize_per_channel_vec_kernel(const int8_t *__restrict__ q, size_t nvec,
@@ -1161,7 +1205,10 @@ __global__ __launch_bounds__(kBlock) void requantize_kernel(const int32_t *__res
 // arithmetic is the scalar kernel's.  cols % 4 == 0; acc, sw, bias 16-byte and out 4-byte aligned.  A vector's
 // row and column come from a shift when cols / 4 is a power of two, else from one 32- or 64-bit division per
 // four elements.
-template <bool EVEN>
+// FIXED_COLUMNS: the grid is sized so that a thread meets the same four column vectors in every tile it takes
+// ((gridDim.x * kTileVec) % (cols / 4) == 0, see requantize_grid): their weight scales and biases are loaded once,
+// ahead of the accumulators, instead of with every vector.
+template <bool EVEN, bool FIXED_COLUMNS>
 __global__ __launch_bounds__(kBlock) void requantize_vec_kernel(const int32_t *__restrict__ acc, size_t rows, size_t cols,
                                                                  const float *__restrict__ sa, int sa_per_row,
                                                                  const float *__restrict__ sw,
@@ -1177,51 +1224,112 @@ __global__ __launch_bounds__(kBlock) void requantize_vec_kernel(const int32_t *_
     const float4 *sw4 = reinterpret_cast<const float4 *>(sw);
     const float4 *bias4 = reinterpret_cast<const float4 *>(bias);
     uint32_t *out4 = reinterpret_cast<uint32_t *>(out);
-    auto one = [&](int a, float s_w, float b, float s_a) {
-        float v = static_cast<float>(a) * (s_a * s_w);
-        if (bias) v = v + b;
-        // saturating conversion (NaN -> 0), then the clamp on integers: the scalar kernel's clamp-then-convert
-        return clamp_to_int(round_mode<EVEN>(div_rn(v, s_out, inv_out)) + zpf, -128, 127);
-    };
-    auto emit = [&](size_t j, const int4 &a) {
-        size_t r, cv;
-        if (pow2) {
-            r = j >> shift;
-            cv = j & (vpr - 1);
-        } else if (small) {
-            r = static_cast<uint32_t>(j) / static_cast<uint32_t>(vpr);
-            cv = static_cast<uint32_t>(j) - static_cast<uint32_t>(r) * static_cast<uint32_t>(vpr);
-        } else {
-            r = j / vpr;
-            cv = j % vpr;
-        }
-        const float s_a = sa_per_row ? sa[r] : sa0;
-        const float4 w = sw4[cv];
-        const float4 b = bias ? bias4[cv] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        store_stream(out4 + j, pack4(one(a.x, w.x, b.x, s_a), one(a.y, w.y, b.y, s_a), one(a.z, w.z, b.z, s_a),
-                                     one(a.w, w.w, b.w, s_a)));
-    };
-    const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
-    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const size_t base = t * kTileVec + threadIdx.x;
-        if ((t + 1) * kTileVec <= nvec) {  // whole tile: unguarded loads issue back to back
-            int4 a[kVecPerThread];
+    // The uniform choices (how a vector's row and column are found, bias or none, one activation scale or one per
+    // row) are made once, outside the loop: inside it they would be branches between the loads and the stores.
+    auto run = [&](auto shifts, auto small32, auto with_bias, auto per_row) {
+        auto row_col = [&](size_t j, size_t *r, size_t *cv) {
+            if constexpr (decltype(shifts)::value) {
+                *r = j >> shift;
+                *cv = j & (vpr - 1);
+            } else if constexpr (decltype(small32)::value) {
+                *r = static_cast<uint32_t>(j) / static_cast<uint32_t>(vpr);
+                *cv = static_cast<uint32_t>(j) - static_cast<uint32_t>(*r) * static_cast<uint32_t>(vpr);
+            } else {
+                *r = j / vpr;
+                *cv = j % vpr;
+            }
+        };
+        auto one = [&](int a, float s_w, float b, float s_a) {
+            float v = static_cast<float>(a) * (s_a * s_w);
+            if constexpr (decltype(with_bias)::value) v = v + b;
+            // saturating conversion (NaN -> 0), then the clamp on integers: the scalar kernel's clamp-then-convert
+            return clamp_to_int(round_mode<EVEN>(div_rn(v, s_out, inv_out)) + zpf, -128, 127);
+        };
+        const float4 none = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        auto emit4 = [&](size_t j, size_t r, const int4 &a, const float4 &w, const float4 &b) {
+            float s_a = sa0;
+            if constexpr (decltype(per_row)::value) s_a = sa[r];
+            store_stream(out4 + j, pack4(one(a.x, w.x, b.x, s_a), one(a.y, w.y, b.y, s_a), one(a.z, w.z, b.z, s_a),
+                                         one(a.w, w.w, b.w, s_a)));
+        };
+        auto emit = [&](size_t j, const int4 &a) {
+            size_t r, cv;
+            row_col(j, &r, &cv);
+            emit4(j, r, a, sw4[cv], decltype(with_bias)::value ? bias4[cv] : none);
+        };
+        auto load_acc = [&](size_t j) {
+            typedef int vi4 __attribute__((ext_vector_type(4)));
+            const vi4 t = __builtin_nontemporal_load(reinterpret_cast<const vi4 *>(acc4 + j));
+            return make_int4(t.x, t.y, t.z, t.w);
+        };
+        const size_t ntiles = (nvec + kTileVec - 1) / kTileVec;
+        float4 w_fixed[kVecPerThread], b_fixed[kVecPerThread];
+        if constexpr (FIXED_COLUMNS) {
 #pragma unroll
             for (int i = 0; i < kVecPerThread; ++i) {
-                typedef int vi4 __attribute__((ext_vector_type(4)));
-                const vi4 t = __builtin_nontemporal_load(reinterpret_cast<const vi4 *>(acc4 + base + size_t(i) * kBlock));
-                a[i] = make_int4(t.x, t.y, t.z, t.w);
-            }
-#pragma unroll
-            for (int i = 0; i < kVecPerThread; ++i) emit(base + size_t(i) * kBlock, a[i]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < kVecPerThread; ++i) {
-                const size_t j = base + size_t(i) * kBlock;
-                if (j < nvec) emit(j, acc4[j]);
+                size_t r, cv;  // (a first vector past nvec still has a valid column)
+                row_col(size_t(blockIdx.x) * kTileVec + threadIdx.x + size_t(i) * kBlock, &r, &cv);
+                w_fixed[i] = sw4[cv];
+                b_fixed[i] = decltype(with_bias)::value ? bias4[cv] : none;
+                if constexpr (!decltype(per_row)::value) {  // s_a * s_w once (the same product, rounded the same)
+                    w_fixed[i].x = sa0 * w_fixed[i].x;
+                    w_fixed[i].y = sa0 * w_fixed[i].y;
+                    w_fixed[i].z = sa0 * w_fixed[i].z;
+                    w_fixed[i].w = sa0 * w_fixed[i].w;
+                }
             }
         }
-    }
+        auto one_combined = [&](int a, float sc, float b) {
+            float v = static_cast<float>(a) * sc;
+            if constexpr (decltype(with_bias)::value) v = v + b;
+            return clamp_to_int(round_mode<EVEN>(div_rn(v, s_out, inv_out)) + zpf, -128, 127);
+        };
+        for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+            const size_t base = t * kTileVec + threadIdx.x;
+            if ((t + 1) * kTileVec <= nvec) {  // whole tile: unguarded loads issue back to back
+                int4 a[kVecPerThread];
+#pragma unroll
+                for (int i = 0; i < kVecPerThread; ++i) a[i] = load_acc(base + size_t(i) * kBlock);
+#pragma unroll
+                for (int i = 0; i < kVecPerThread; ++i) {
+                    const size_t j = base + size_t(i) * kBlock;
+                    if constexpr (FIXED_COLUMNS && !decltype(per_row)::value) {
+                        const float4 &w = w_fixed[i], &b = b_fixed[i];
+                        store_stream(out4 + j, pack4(one_combined(a[i].x, w.x, b.x), one_combined(a[i].y, w.y, b.y),
+                                                     one_combined(a[i].z, w.z, b.z), one_combined(a[i].w, w.w, b.w)));
+                    } else if constexpr (FIXED_COLUMNS) {
+                        size_t r, cv;
+                        row_col(j, &r, &cv);
+                        emit4(j, r, a[i], w_fixed[i], b_fixed[i]);
+                    } else {
+                        emit(j, a[i]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < kVecPerThread; ++i) {
+                    const size_t j = base + size_t(i) * kBlock;
+                    if (j < nvec) emit(j, acc4[j]);
+                }
+            }
+        }
+    };
+    auto with_index = [&](auto with_bias, auto per_row) {
+        if (pow2)
+            run(std::true_type{}, std::true_type{}, with_bias, per_row);
+        else if (small)
+            run(std::false_type{}, std::true_type{}, with_bias, per_row);
+        else
+            run(std::false_type{}, std::false_type{}, with_bias, per_row);
+    };
+    if (bias && sa_per_row)
+        with_index(std::true_type{}, std::true_type{});
+    else if (bias)
+        with_index(std::true_type{}, std::false_type{});
+    else if (sa_per_row)
+        with_index(std::false_type{}, std::true_type{});
+    else
+        with_index(std::false_type{}, std::false_type{});
 }
 
 static inline int grid_for_tiles(hipq_ctx *ctx, size_t n) {
@@ -1562,6 +1670,9 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
     if (rows >> 31) return fail(HIPQ_INVALID_ARGUMENT, "%s: too many rows", fn);
     // Packed output: the grid also covers the padding rows of the last row block (they are written as zeros).
     const size_t grid_rows = packed ? (rows + 31) / 32 * 32 : rows;
+    // A large dense tensor is read and written once: past the caches, as the per-tensor quantizer does it
+    // (4096 x 4096: 19.9 -> 17.3 us).  Packed output is an operand of the GEMM that follows: it stays cached.
+    const bool stream = !packed && rows * cols >= (size_t(1) << 22);
 #define HIPQ_LAUNCH_ROWS(TPR, E, P, G)                                                                               \
     hipLaunchKernelGGL((quantize_per_row_kernel<TPR, E, P>), dim3(G), dim3(kBlock), 0, ctx->stream, x, rows, cols, ld, \
                        flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison)
@@ -1571,7 +1682,15 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
 #define HIPQ_LAUNCH_LONG_ROWS(E, P)                                                                                   \
     hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, E, P, 16>), dim3(grid), dim3(kBlock), 0, ctx->stream, x, rows,   \
                        cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points, out_status, poison)
-        if (packed && even)
+        if (stream && even)
+            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true, false, 16, true>), dim3(grid), dim3(kBlock), 0,
+                               ctx->stream, x, rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                               out_status, poison);
+        else if (stream)
+            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false, false, 16, true>), dim3(grid), dim3(kBlock), 0,
+                               ctx->stream, x, rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                               out_status, poison);
+        else if (packed && even)
             HIPQ_LAUNCH_LONG_ROWS(true, true);
         else if (packed)
             HIPQ_LAUNCH_LONG_ROWS(false, true);
@@ -1580,6 +1699,16 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
         else
             HIPQ_LAUNCH_LONG_ROWS(false, false);
 #undef HIPQ_LAUNCH_LONG_ROWS
+    } else if (cols > 1024 && stream) {
+        const int grid = static_cast<int>(grid_rows);
+        if (even)
+            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, true, false, 4, true>), dim3(grid), dim3(kBlock), 0,
+                               ctx->stream, x, rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                               out_status, poison);
+        else
+            hipLaunchKernelGGL((quantize_per_row_kernel<kBlock, false, false, 4, true>), dim3(grid), dim3(kBlock), 0,
+                               ctx->stream, x, rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                               out_status, poison);
     } else if (cols > 1024) {
         const int grid = static_cast<int>(grid_rows);
         if (packed) {
@@ -1592,6 +1721,16 @@ static int32_t quantize_rows(const char *fn, hipq_ctx *ctx, const float *x, size
         } else {
             HIPQ_LAUNCH_ROWS(kBlock, false, false, grid);
         }
+    } else if (stream) {
+        const int grid = static_cast<int>((grid_rows + 3) / 4);
+        if (even)
+            hipLaunchKernelGGL((quantize_per_row_kernel<kWave, true, false, 4, true>), dim3(grid), dim3(kBlock), 0,
+                               ctx->stream, x, rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                               out_status, poison);
+        else
+            hipLaunchKernelGGL((quantize_per_row_kernel<kWave, false, false, 4, true>), dim3(grid), dim3(kBlock), 0,
+                               ctx->stream, x, rows, cols, ld, flavor, qmin, qmax, out, out_scales, out_zero_points,
+                               out_status, poison);
     } else {
         const int grid = static_cast<int>((grid_rows + 3) / 4);
         if (packed) {
@@ -1922,13 +2061,35 @@ int32_t hipq_requantize_i32_i8(hipq_ctx *ctx, const int32_t *acc, size_t rows, s
                      (reinterpret_cast<uintptr_t>(w_scales) & 15u) == 0 && (reinterpret_cast<uintptr_t>(bias) & 15u) == 0 &&
                      (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
     if (vec) {
-        const int vgrid = grid_for_tiles(ctx, rows * cols);
-        if (mode & HIPQ_ROUND_HALF_EVEN)
-            hipLaunchKernelGGL((requantize_vec_kernel<true>), dim3(vgrid), dim3(kBlock), 0, ctx->stream, acc, rows, cols,
-                               a_scale, a_scale_per_row, w_scales, bias, out_scale, out_zero_point, out);
-        else
-            hipLaunchKernelGGL((requantize_vec_kernel<false>), dim3(vgrid), dim3(kBlock), 0, ctx->stream, acc, rows, cols,
-                               a_scale, a_scale_per_row, w_scales, bias, out_scale, out_zero_point, out);
+        // A grid of g workgroups hands a thread the vectors j, j + g * kTileVec, ...: the same column vector every
+        // time when g * kTileVec is a multiple of the vectors per row.  With several tiles per workgroup that pays
+        // (weight scales and biases loaded once per thread); g = the multiple of the period nearest 4 per compute unit (eight was slower: 17.1 against 16.4 us for 16 Mi).
+        const size_t vpr = cols / 4, tiles = (rows * vpr + kTileVec - 1) / kTileVec;
+        size_t a = vpr, b = kTileVec;
+        while (b) {
+            const size_t t = a % b;
+            a = b;
+            b = t;
+        }
+        const size_t period = vpr / a, want = size_t(ctx->num_cus) * 4;
+        const size_t fixed_grid = period <= want ? want / period * period : 0;
+        const bool fixed = fixed_grid && tiles >= 2 * fixed_grid;
+        const int vgrid = fixed ? static_cast<int>(fixed_grid) : grid_for_tiles(ctx, rows * cols);
+#define HIPQ_LAUNCH_RQ(E, F)                                                                                         \
+    hipLaunchKernelGGL((requantize_vec_kernel<E, F>), dim3(vgrid), dim3(kBlock), 0, ctx->stream, acc, rows, cols, a_scale, \
+                       a_scale_per_row, w_scales, bias, out_scale, out_zero_point, out)
+        if (mode & HIPQ_ROUND_HALF_EVEN) {
+            if (fixed)
+                HIPQ_LAUNCH_RQ(true, true);
+            else
+                HIPQ_LAUNCH_RQ(true, false);
+        } else {
+            if (fixed)
+                HIPQ_LAUNCH_RQ(false, true);
+            else
+                HIPQ_LAUNCH_RQ(false, false);
+        }
+#undef HIPQ_LAUNCH_RQ
         return check_launch(__func__);
     }
     const int grid = grid_for_elems(ctx, rows * cols);
