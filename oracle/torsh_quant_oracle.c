@@ -431,6 +431,78 @@ int tq_nn_per_channel_quantize_weights_asym_u8(const float *w, size_t channels, 
     return TQ_OK;
 }
 
+/* One carrier value of a torsh-nn quantized tensor back to f32: dequantize_from_int8 / _int16
+ * (crates/torsh-nn/src/quantization/ops.rs:110-125, 146-150: the zero point is not used) or
+ * dequantize_from_uint8 (ops.rs:128-143). */
+static inline float nn_dequantize_carrier(float v, float scale, int32_t zp, int is_u8) {
+    const int32_t q = f32_as_i32(roundf(v));
+    return is_u8 ? (float)(q - zp) * scale : (float)q * scale;
+}
+/* quantize_tensor (ops.rs:11-24) on one value: int8 / int16 take the symmetric formula, uint8 the asymmetric. */
+static inline float nn_quantize_carrier(float v, float scale, int32_t zp, int is_u8, int32_t qmin, int32_t qmax) {
+    return (float)(is_u8 ? tq_nn_quantize_value_asymmetric(v, scale, zp, qmin, qmax)
+                         : tq_nn_quantize_value_symmetric(v, scale, qmin, qmax));
+}
+
+/* quantized_matmul_int8, crates/torsh-nn/src/quantization/ops.rs:175-194: dequantize both operands, multiply in
+ * f32, quantize the product with the caller's output parameters.  a [m,k], b [k,n], f32 carriers.  The f32 product
+ * is a plain i, j, l loop here; the reference's Tensor::matmul picks among several f32 kernels
+ * (crates/torsh-tensor/src/ops/matrix.rs:83-160) whose order of summation is not fixed, so results are comparable
+ * to within the f32 summation error, i.e. one output code. */
+int tq_nn_quantized_matmul_int8(const float *a, const float *b, size_t m, size_t k, size_t n, float sa, int32_t zpa,
+                                int a_u8, float sb, int32_t zpb, int b_u8, float so, int32_t zpo, int o_u8,
+                                int32_t qmin, int32_t qmax, float *out) {
+    for (size_t i = 0; i < m; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            float acc = 0.0f;
+            for (size_t l = 0; l < k; ++l)
+                acc += nn_dequantize_carrier(a[i * k + l], sa, zpa, a_u8) * nn_dequantize_carrier(b[l * n + j], sb, zpb, b_u8);
+            out[i * n + j] = nn_quantize_carrier(acc, so, zpo, o_u8, qmin, qmax);
+        }
+    return TQ_OK;
+}
+
+/* quantized_conv2d_int8, ops.rs:197-237: dequantize input, weight and (optional) bias, f32 convolution (dilation 1,
+ * one group; padded taps are the real value 0), quantize with the caller's output parameters.  Summation order:
+ * kh, kw, ic (the same caveat as for the product above). */
+int tq_nn_quantized_conv2d_int8(const float *x, const float *w, const float *bias, size_t nb, size_t c_in, size_t h,
+                                size_t wd, size_t c_out, size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                size_t pad_h, size_t pad_w, float sx, int32_t zpx, int x_u8, float sw, int32_t zpw,
+                                int w_u8, float sbias, int32_t zpb, int b_u8, float so, int32_t zpo, int o_u8,
+                                int32_t qmin, int32_t qmax, float *out) {
+    if (stride_h == 0 || stride_w == 0) return TQ_ERR_INVALID_ARGUMENT;
+    if (h + 2 * pad_h < kh || wd + 2 * pad_w < kw) return TQ_ERR_INVALID_ARGUMENT;
+    const size_t ho = (h + 2 * pad_h - kh) / stride_h + 1, wo = (wd + 2 * pad_w - kw) / stride_w + 1;
+    for (size_t b = 0; b < nb; ++b)
+        for (size_t oc = 0; oc < c_out; ++oc)
+            for (size_t oh = 0; oh < ho; ++oh)
+                for (size_t ow = 0; ow < wo; ++ow) {
+                    float acc = 0.0f;
+                    for (size_t r = 0; r < kh; ++r)
+                        for (size_t s = 0; s < kw; ++s)
+                            for (size_t ic = 0; ic < c_in; ++ic) {
+                                size_t ih = oh * stride_h + r, iw = ow * stride_w + s;
+                                if (ih < pad_h || iw < pad_w) continue;
+                                ih -= pad_h;
+                                iw -= pad_w;
+                                if (ih >= h || iw >= wd) continue;
+                                acc += nn_dequantize_carrier(x[((b * c_in + ic) * h + ih) * wd + iw], sx, zpx, x_u8) *
+                                       nn_dequantize_carrier(w[((oc * c_in + ic) * kh + r) * kw + s], sw, zpw, w_u8);
+                            }
+                    if (bias) acc += nn_dequantize_carrier(bias[oc], sbias, zpb, b_u8);
+                    out[((b * c_out + oc) * ho + oh) * wo + ow] = nn_quantize_carrier(acc, so, zpo, o_u8, qmin, qmax);
+                }
+    return TQ_OK;
+}
+
+/* quantized_relu_int8, ops.rs:261-294: the code of the real value 0 by the asymmetric formula (whatever the
+ * dtype), then max on the carrier: `(value as i32) > zero ? value : zero as f32`. */
+int tq_nn_quantized_relu_int8(const float *x, size_t n, float scale, int32_t zp, int32_t qmin, int32_t qmax, float *out) {
+    const int32_t zero_q = tq_nn_quantize_value_asymmetric(0.0f, scale, zp, qmin, qmax);
+    for (size_t i = 0; i < n; ++i) out[i] = f32_as_i32(x[i]) > zero_q ? x[i] : (float)zero_q;
+    return TQ_OK;
+}
+
 /* crates/torsh-backend/src/quantization/ops.rs:185-195 */
 int32_t tq_backend_quantize_value(float v, float scale, int32_t zp, int32_t qmin, int32_t qmax) {
     float q = rnd(v / scale) + (float)zp;

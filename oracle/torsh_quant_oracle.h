@@ -90,6 +90,18 @@ int tq_nn_per_channel_quantize_weights_sym_i8(const float *w, size_t channels, s
 int tq_nn_per_channel_quantize_weights_asym_u8(const float *w, size_t channels, size_t channel_size,
                                                float *out_carrier, float *scales, int32_t *zps);
 
+/* quantized_matmul_int8 / quantized_conv2d_int8 / quantized_relu_int8 (crates/torsh-nn/src/quantization/ops.rs:175-294)
+ * on f32 carriers; *_u8 = 1 selects the uint8 (asymmetric) value formulas, 0 the int8 / int16 (symmetric) ones. */
+int tq_nn_quantized_matmul_int8(const float *a, const float *b, size_t m, size_t k, size_t n, float sa, int32_t zpa,
+                                int a_u8, float sb, int32_t zpb, int b_u8, float so, int32_t zpo, int o_u8,
+                                int32_t qmin, int32_t qmax, float *out);
+int tq_nn_quantized_conv2d_int8(const float *x, const float *w, const float *bias, size_t nb, size_t c_in, size_t h,
+                                size_t wd, size_t c_out, size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                size_t pad_h, size_t pad_w, float sx, int32_t zpx, int x_u8, float sw, int32_t zpw,
+                                int w_u8, float sbias, int32_t zpb, int b_u8, float so, int32_t zpo, int o_u8,
+                                int32_t qmin, int32_t qmax, float *out);
+int tq_nn_quantized_relu_int8(const float *x, size_t n, float scale, int32_t zp, int32_t qmin, int32_t qmax, float *out);
+
 /* ---- torsh-backend::quantization -------------------------------------- */
 int32_t tq_backend_quantize_value(float v, float scale, int32_t zp, int32_t qmin, int32_t qmax);
 float tq_backend_dequantize_value(int32_t q, float scale, int32_t zp);

@@ -1241,6 +1241,37 @@ GPU_TEST(test_quantized_modules_survive_a_weight_file) {
     for (size_t i = 0; i < n * k; ++i) CHECK(static_cast<float>(file.weight[i]) == carrier[i]);
     check_same(file.bias, b.as_slice(), __LINE__);
     std::remove(path.c_str());
+    // The prepared blob: the rows in the operand order of the matrix cores.  The file's payload is the layout
+    // written out on the host from the row-major codes (ragged shape: 96 rows are three row blocks, K = 304 pads
+    // to 12 k blocks), a layer loaded from it forwards the same bits without a packing pass, and its row-major
+    // view (rebuilt from the prepared bytes) is the row-major file's.
+    {
+        const size_t n2 = 70, k2 = 304;
+        const Tensor w2 = Tensor::from_data(normal(n2 * k2, 66, 0.03f), {n2, k2}).unwrap();
+        const Tensor x2 = Tensor::from_data(normal(m * k2, 67), {m, k2}).unwrap();
+        auto lin2 = nn::QuantizedLinear::from_weight_nk(w2, nullptr, nn::ActivationQuant::PerTensor).unwrap();
+        CHECK(lin2.save_prepared(path).is_ok());
+        const QuantizedWeights prepared = load_quantized_weights(path).unwrap();
+        const QuantizedWeights plain = lin2.to_quantized_weights().unwrap();
+        CHECK(prepared.packed.size() == packed_layout::bytes(n2, k2) && prepared.packed.size() == 3 * 12 * 1024);
+        CHECK_SAME(prepared.weight, plain.weight);
+        std::vector<int8_t> want(prepared.packed.size(), 0);
+        for (size_t r = 0; r < n2; ++r)
+            for (size_t kk = 0; kk < k2; ++kk) want[packed_layout::offset(r, kk, k2)] = plain.weight[r * k2 + kk];
+        CHECK_SAME(prepared.packed, want);
+        auto back2 = nn::QuantizedLinear::load(path).unwrap();
+        check_same(back2.forward(x2).unwrap().as_slice(), lin2.forward(x2).unwrap().as_slice(), __LINE__);
+        CHECK_SAME(back2.to_quantized_weights(true).unwrap().packed, want);
+        // a damaged prepared section is caught by the checksum
+        {
+            std::fstream f(path, std::ios::in | std::ios::out | std::ios::binary);
+            f.seekp(256 + 1000);
+            const char flip = 0x55;
+            f.write(&flip, 1);
+        }
+        CHECK(load_quantized_weights(path).is_err());
+        std::remove(path.c_str());
+    }
     // conv: same round trip
     const Tensor cw = Tensor::from_data(normal(8 * 4 * 3 * 3, 64, 0.1f), {8, 4, 3, 3}).unwrap();
     const Tensor cx = Tensor::from_data(normal(2 * 4 * 6 * 6, 65, 1.0f, true), {2, 4, 6, 6}).unwrap();
@@ -1677,6 +1708,118 @@ GPU_TEST(parity_torsh_nn_quantizer_and_qtype_slices) {
         for (size_t i = 0; i < x.size(); ++i) CHECK(q[i] == tq_qint8_quantize(x[i], 0.1f, 5));
         const auto u = torsh::dtype::quantized::quantize_slice_quint8(x, 0.1f, 130).unwrap();
         for (size_t i = 0; i < x.size(); ++i) CHECK(u[i] == tq_quint8_quantize(x[i], 0.1f, 130));
+    }
+}
+
+// quantized_matmul_int8 / quantized_conv2d_int8 / quantized_relu_int8 (crates/torsh-nn/src/quantization/ops.rs:175-294)
+// with caller-supplied output parameters.  The device result is bit-identical to the exact int32 composition
+// (oracle GEMM / conv accumulators, acc * (s_a * s_b) (+ bias), then the reference's own value formulas) and within
+// one output code of the oracle's restatement of the reference's f32 path (dequantize, f32 product, quantize),
+// whose summation order the reference does not fix.  The ReLU is exact.
+GPU_TEST(parity_torsh_nn_quantized_helpers) {
+    namespace nq = torsh::nn::quantization;
+    std::mt19937 rng(77);
+    std::uniform_int_distribution<int> d8(-128, 127), du8(0, 255);
+    for (auto [m, k, n] : {std::make_tuple(size_t(5), size_t(7), size_t(3)), std::make_tuple(size_t(33), size_t(256), size_t(70)),
+                           std::make_tuple(size_t(64), size_t(512), size_t(48))}) {
+        std::vector<float> a(m * k), b(k * n);
+        std::vector<int8_t> a8(m * k), bt8(n * k);
+        for (size_t i = 0; i < m * k; ++i) a[i] = float(a8[i] = int8_t(d8(rng)));
+        for (size_t l = 0; l < k; ++l)
+            for (size_t j = 0; j < n; ++j) b[l * n + j] = float(bt8[j * k + l] = int8_t(d8(rng)));
+        const Tensor ta = Tensor::from_data(a, {m, k}).unwrap(), tb = Tensor::from_data(b, {k, n}).unwrap();
+        const auto pa = nq::QuantizationParams::symmetric(0.031f, DType::F32, DType::I8).unwrap();
+        const auto pb = nq::QuantizationParams::symmetric(0.0007f, DType::F32, DType::I8).unwrap();
+        std::vector<int32_t> acc(m * n);
+        CHECK_EQ(tq_gemm_i8_nk(a8.data(), bt8.data(), m, n, k, acc.data()), 0);
+        const float sab = pa.scale * pb.scale;
+        for (const auto &po : {nq::QuantizationParams::symmetric(0.05f, DType::F32, DType::I8).unwrap(),
+                               nq::QuantizationParams::asymmetric(0.03f, 131, DType::F32, DType::U8).unwrap(),
+                               nq::QuantizationParams::symmetric(0.0004f, DType::F32, DType::I16).unwrap()}) {
+            const bool o_u8 = po.dst_dtype == DType::U8;
+            const Tensor got = nq::quantized_matmul_int8(ta, tb, pa, pb, po).unwrap();
+            CHECK(got.shape().dims() == (std::vector<size_t>{m, n}));
+            std::vector<float> ref(m * n);
+            CHECK_EQ(tq_nn_quantized_matmul_int8(a.data(), b.data(), m, k, n, pa.scale, 0, 0, pb.scale, 0, 0, po.scale,
+                                                 po.zero_point, o_u8, po.qmin, po.qmax, ref.data()), 0);
+            for (size_t i = 0; i < m * n; ++i) {
+                const float v = float(acc[i]) * sab;
+                const float want = float(o_u8 ? tq_nn_quantize_value_asymmetric(v, po.scale, po.zero_point, po.qmin, po.qmax)
+                                              : tq_nn_quantize_value_symmetric(v, po.scale, po.qmin, po.qmax));
+                CHECK(got.as_slice()[i] == want);
+                CHECK(std::fabs(got.as_slice()[i] - ref[i]) <= 1.0f);
+            }
+        }
+    }
+    {
+        const Tensor ta = Tensor::from_data(std::vector<float>(6, 1.0f), {2, 3}).unwrap();
+        const Tensor tb = Tensor::from_data(std::vector<float>(8, 1.0f), {4, 2}).unwrap();
+        const auto p = nq::QuantizationParams::symmetric(0.1f, DType::F32, DType::I8).unwrap();
+        CHECK(nq::quantized_matmul_int8(ta, tb, p, p, p).is_err());  // K mismatch
+        const Tensor big = Tensor::from_data(std::vector<float>(6, 300.0f), {3, 2}).unwrap();
+        CHECK(nq::quantized_matmul_int8(ta, big, p, p, p).is_err());  // not an int8 carrier
+        const auto pu = nq::QuantizationParams::asymmetric(0.1f, 3, DType::F32, DType::U8).unwrap();
+        CHECK(nq::quantized_matmul_int8(ta, Tensor::from_data(std::vector<float>(6, 1.0f), {3, 2}).unwrap(), pu, p, p)
+                  .unwrap_err().kind == TorshError::NotImplemented);
+    }
+    struct G { size_t nb, c, h, w, oc, k, stride, pad; bool in_u8, with_bias; };
+    for (G g : {G{2, 3, 8, 8, 4, 3, 1, 1, true, true}, G{1, 32, 7, 7, 16, 3, 1, 1, false, true}, G{1, 16, 9, 9, 6, 3, 2, 1, true, false},
+                G{2, 64, 6, 6, 32, 3, 1, 1, true, true}}) {
+        const size_t nx = g.nb * g.c * g.h * g.w, nw = g.oc * g.c * g.k * g.k;
+        std::vector<float> x(nx), w(nw), bias(g.oc);
+        std::vector<uint8_t> xq(nx);
+        std::vector<int8_t> wq(nw);
+        for (size_t i = 0; i < nx; ++i) {
+            const int q = g.in_u8 ? du8(rng) : d8(rng);
+            x[i] = float(q);
+            xq[i] = uint8_t(g.in_u8 ? q : int8_t(q));
+        }
+        for (size_t i = 0; i < nw; ++i) w[i] = float(wq[i] = int8_t(d8(rng)));
+        for (size_t i = 0; i < g.oc; ++i) bias[i] = float(d8(rng));
+        const auto px = g.in_u8 ? nq::QuantizationParams::asymmetric(0.02f, 117, DType::F32, DType::U8).unwrap()
+                                : nq::QuantizationParams::symmetric(0.02f, DType::F32, DType::I8).unwrap();
+        const auto pw = nq::QuantizationParams::symmetric(0.0009f, DType::F32, DType::I8).unwrap();
+        const auto pbias = nq::QuantizationParams::symmetric(0.0005f, DType::F32, DType::I8).unwrap();
+        const Tensor tx = Tensor::from_data(x, {g.nb, g.c, g.h, g.w}).unwrap();
+        const Tensor tw = Tensor::from_data(w, {g.oc, g.c, g.k, g.k}).unwrap();
+        const Tensor tbias = Tensor::from_data(bias, {g.oc}).unwrap();
+        const size_t ho = (g.h + 2 * g.pad - g.k) / g.stride + 1, wo = (g.w + 2 * g.pad - g.k) / g.stride + 1;
+        std::vector<int32_t> acc(g.nb * g.oc * ho * wo);
+        CHECK_EQ(tq_backend_conv2d_i32(xq.data(), g.in_u8 ? 0 : 1, g.in_u8 ? px.zero_point : 0, wq.data(), g.nb, g.c, g.h,
+                                       g.w, g.oc, g.k, g.k, g.stride, g.stride, g.pad, g.pad, acc.data()), 0);
+        for (const auto &po : {nq::QuantizationParams::symmetric(0.04f, DType::F32, DType::I8).unwrap(),
+                               nq::QuantizationParams::asymmetric(0.03f, 120, DType::F32, DType::U8).unwrap()}) {
+            const bool o_u8 = po.dst_dtype == DType::U8;
+            const Tensor got = nq::quantized_conv2d_int8(tx, tw, g.with_bias ? &tbias : nullptr, px, pw,
+                                                         g.with_bias ? &pbias : nullptr, po, {g.stride, g.stride},
+                                                         {g.pad, g.pad}).unwrap();
+            CHECK(got.shape().dims() == (std::vector<size_t>{g.nb, g.oc, ho, wo}));
+            std::vector<float> ref(acc.size());
+            CHECK_EQ(tq_nn_quantized_conv2d_int8(x.data(), w.data(), g.with_bias ? bias.data() : nullptr, g.nb, g.c, g.h, g.w,
+                                                 g.oc, g.k, g.k, g.stride, g.stride, g.pad, g.pad, px.scale, px.zero_point,
+                                                 g.in_u8, pw.scale, 0, 0, pbias.scale, 0, 0, po.scale, po.zero_point, o_u8,
+                                                 po.qmin, po.qmax, ref.data()), 0);
+            for (size_t i = 0; i < acc.size(); ++i) {
+                const size_t oc = (i / (ho * wo)) % g.oc;
+                float v = float(acc[i]) * (px.scale * pw.scale);
+                if (g.with_bias) v = v + bias[oc] * pbias.scale;
+                const float want = float(o_u8 ? tq_nn_quantize_value_asymmetric(v, po.scale, po.zero_point, po.qmin, po.qmax)
+                                              : tq_nn_quantize_value_symmetric(v, po.scale, po.qmin, po.qmax));
+                CHECK(got.as_slice()[i] == want);
+                CHECK(std::fabs(got.as_slice()[i] - ref[i]) <= 1.0f);
+            }
+        }
+    }
+    for (const auto &p : {nq::QuantizationParams::asymmetric(0.05f, 77, DType::F32, DType::U8).unwrap(),
+                          nq::QuantizationParams::symmetric(0.05f, DType::F32, DType::I8).unwrap(),
+                          nq::QuantizationParams::asymmetric(0.05f, 300, DType::F32, DType::U8).unwrap()}) {
+        std::vector<float> x(5000);
+        for (float &v : x) v = float(p.dst_dtype == DType::U8 ? du8(rng) : d8(rng));
+        const Tensor t = tensor_1d(x).unwrap();
+        const Tensor got = nq::quantized_relu_int8(t, p, p).unwrap();
+        std::vector<float> want(x.size());
+        CHECK_EQ(tq_nn_quantized_relu_int8(x.data(), x.size(), p.scale, p.zero_point, p.qmin, p.qmax, want.data()), 0);
+        check_same(got.as_slice(), want, __LINE__);
     }
 }
 

@@ -606,6 +606,51 @@ def test_two_contexts_meet_side_by_side(hipq):
         b.close()
 
 
+def test_one_launch_forms_beside_unrelated_work_on_the_device(hipq):
+    """Co-tenancy: a plain torch stream that knows nothing of the library keeps the device busy (long elementwise
+    kernels over a 256 MiB tensor, back to back, on a side stream) while a context runs the forms whose workgroups
+    wait for each other - the dynamic Linear forward on prepared weights, the 16 Mi-element dynamic quantize (four
+    workgroups per compute unit, all of which must be resident), the convolution from fp32 - a few hundred times.
+    Every result must equal the quiet-device result and no wait may give up (hipq_ctx_synchronize would say so).
+    The other tenant's workgroups finish on their own, so every wait ends normally; nothing is made to hang."""
+    c = hipq.Context(0)
+    side = torch.cuda.Stream()
+    try:
+        g = torch.Generator(device="cuda").manual_seed(77)
+        m, n, k = 512, 1024, 4096
+        xs = [torch.randn(m, k, generator=g, device="cuda") * (i + 1) for i in range(4)]
+        pw = c.pack_rows(torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8))
+        sw = torch.rand(n, generator=g, device="cuda") * 1e-3 + 1e-4
+        bias = torch.randn(n, generator=g, device="cuda")
+        big = torch.randn(4096 * 4096, generator=g, device="cuda")
+        want_lin = [c.linear_dynamic_packed(x, pw, sw, bias) for x in xs]
+        want_q, want_p = c.quantize_dynamic_per_tensor(big)
+        c.synchronize()
+        want_scale = c.read_qparams(want_p).scale
+        noise_a = torch.randn(64 << 20, device="cuda")
+        noise_b = torch.empty_like(noise_a)
+        torch.cuda.synchronize()
+        outs, qs = [], []
+        for it in range(240):
+            with torch.cuda.stream(side):  # the other tenant: enqueued ahead, so that it is running throughout
+                for _ in range(2):
+                    torch.mul(noise_a, 1.0001, out=noise_b)
+                    torch.add(noise_b, 0.5, out=noise_a)
+            outs.append(c.linear_dynamic_packed(xs[it % 4], pw, sw, bias))
+            if it % 8 == 0:
+                qs.append(c.quantize_dynamic_per_tensor(big))
+        c.synchronize()  # raises if a bounded wait gave up
+        side.synchronize()
+        for it, o in enumerate(outs):
+            assert torch.equal(o, want_lin[it % 4]), it
+        for q, p in qs:
+            assert torch.equal(q, want_q) and c.read_qparams(p).scale == want_scale
+            assert c.read_qparams(p).status == hipq.SUCCESS
+    finally:
+        torch.cuda.synchronize()
+        c.close()
+
+
 def test_one_launch_dynamic_quantize_gives_up_cleanly(hipq):
     """With the spin limit forced to 0 every workgroup looks at the other workgroups' range words exactly once,
     which with hundreds of workgroups is certain to come too early for some of them: the kernel must still drain, a

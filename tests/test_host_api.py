@@ -31,6 +31,7 @@ CPU_CASES = [
 ]
 GPU_CASES = [
     "parity_torsh_nn_quantizer_and_qtype_slices",
+    "parity_torsh_nn_quantized_helpers",
     "test_quantize_per_tensor_affine",
     "test_dequantize_per_tensor_affine",
     "test_quantize_tensor_auto",

@@ -161,10 +161,17 @@ class QuantizedLinear : public Module {
             q.bias_ = std::move(db);
             q.has_bias_ = true;
         }
-        TORSH_CHECK(q.pack());
+        if (!w.packed.empty()) {
+            // the file held the operand in tile order: it is what the forward reads, uploaded as it is
+            TORSH_TRY(dp, hip::DeviceBuffer::from_host(ctx, w.packed.data(), w.packed.size()));
+            q.wp_ = std::move(dp);
+        } else {
+            TORSH_CHECK(q.pack());
+        }
         return std::move(q);
     }
-    Result<quantization::QuantizedWeights> to_quantized_weights() const {
+    // prepared: also the rows in the operand order of the matrix cores, as the device holds them.
+    Result<quantization::QuantizedWeights> to_quantized_weights(bool prepared = false) const {
         quantization::QuantizedWeights w;
         w.kind = quantization::QuantizedWeights::Linear;
         w.dims = {out_, in_};
@@ -176,10 +183,19 @@ class QuantizedLinear : public Module {
             TORSH_TRY(b, bias_.to_host<float>(out_));
             w.bias = std::move(b);
         }
+        if (prepared) {
+            TORSH_TRY(wp, wp_.to_host<int8_t>(wp_.bytes()));
+            w.packed = std::move(wp);
+        }
         return w;
     }
     Result<Unit> save(const std::string &path) const {
         TORSH_TRY(w, to_quantized_weights());
+        return quantization::save_quantized_weights(w, path);
+    }
+    // The prepared-weight blob: int8 rows in tile order, scales, bias.  load() of it needs no packing pass.
+    Result<Unit> save_prepared(const std::string &path) const {
+        TORSH_TRY(w, to_quantized_weights(/*prepared=*/true));
         return quantization::save_quantized_weights(w, path);
     }
     static Result<QuantizedLinear> load(const std::string &path, ActivationQuant act = ActivationQuant::PerTensor) {

@@ -233,6 +233,23 @@ inline Result<QuantConfig> import_config_from_json(const std::string &json) {
 
 // ---- prepared int8 weights on disk -------------------------------------------------------------
 
+// Where byte (row, k) of an int8 matrix [rows, K] lives in the operand order of the matrix cores (the layout
+// hipq_pack_rows_i8 writes): [row block of 32][k block of 32 bytes, padded to a multiple of 4][1 KiB], and inside a
+// fragment slot l = row % 32 + 32 * ((k % 32) / 16) of 16 bytes.  Padding rows and k are zero.
+namespace packed_layout {
+inline size_t k_blocks(size_t k) { return ((k + 31) / 32 + 3) / 4 * 4; }
+inline size_t bytes(size_t rows, size_t k) { return ((rows + 31) / 32) * k_blocks(k) * 1024; }
+inline size_t offset(size_t row, size_t kk, size_t k) {
+    return ((row / 32) * k_blocks(k) + kk / 32) * 1024 + ((kk % 32) / 16) * 512 + (row % 32) * 16 + kk % 16;
+}
+inline std::vector<int8_t> unpack(const std::vector<int8_t> &packed, size_t rows, size_t k) {
+    std::vector<int8_t> out(rows * k);
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t kk = 0; kk < k; ++kk) out[r * k + kk] = packed[offset(r, kk, k)];
+    return out;
+}
+}  // namespace packed_layout
+
 struct QuantizedWeights {
     enum Kind : uint32_t { Linear = 1, Conv2d = 2 };
     Kind kind = Linear;
@@ -240,6 +257,10 @@ struct QuantizedWeights {
     std::vector<int8_t> weight;  // rows() x row_len(), row-major
     std::vector<float> scales;   // one per row
     std::vector<float> bias;     // empty or one per row
+    // Linear only, optional: the same rows already in the operand order of the matrix cores
+    // (packed_layout::bytes(N, K) bytes).  A file saved with it holds the prepared operand instead of the
+    // row-major rows, and a layer loaded from such a file uploads it as it is: no packing pass on the device.
+    std::vector<int8_t> packed;
 
     size_t rows() const { return dims.empty() ? 0 : dims[0]; }
     size_t row_len() const {
@@ -254,6 +275,8 @@ struct QuantizedWeights {
         if (kind != Linear && kind != Conv2d) return TorshError::invalid_argument("unknown weight kind");
         if (weight.size() != rows() * row_len() || scales.size() != rows() || (!bias.empty() && bias.size() != rows()))
             return TorshError::invalid_argument("quantized weight sections do not match dims");
+        if (!packed.empty() && (kind != Linear || packed.size() != packed_layout::bytes(rows(), row_len())))
+            return TorshError::invalid_argument("prepared weight section does not match dims");
         return Unit{};
     }
 };
@@ -272,13 +295,15 @@ inline bool mul_fits(uint64_t a, uint64_t b, uint64_t *out) { return !__builtin_
 inline Result<Unit> save_quantized_weights(const QuantizedWeights &w, const std::string &path) {
     TORSH_CHECK(w.validate());
     const size_t off_w = 256;
-    const size_t off_s = detail::align256(off_w + w.weight.size());
+    // flag 2: the weight section is the prepared operand (tile order), not the row-major rows
+    const std::vector<int8_t> &payload = w.packed.empty() ? w.weight : w.packed;
+    const size_t off_s = detail::align256(off_w + payload.size());
     const size_t off_b = w.bias.empty() ? 0 : detail::align256(off_s + w.scales.size() * sizeof(float));
     const size_t total = detail::align256(w.bias.empty() ? off_s + w.scales.size() * sizeof(float)
                                                          : off_b + w.bias.size() * sizeof(float));
     std::vector<unsigned char> buf(total, 0);
     std::memcpy(buf.data(), detail::kWeightMagic, 8);
-    const uint32_t kind = w.kind, flags = w.bias.empty() ? 0u : 1u;
+    const uint32_t kind = w.kind, flags = (w.bias.empty() ? 0u : 1u) | (w.packed.empty() ? 0u : 2u);
     std::memcpy(buf.data() + 8, &kind, 4);
     std::memcpy(buf.data() + 12, &flags, 4);
     uint64_t dims[4] = {0, 0, 0, 0};
@@ -286,7 +311,7 @@ inline Result<Unit> save_quantized_weights(const QuantizedWeights &w, const std:
     std::memcpy(buf.data() + 16, dims, 32);
     const uint64_t offs[4] = {off_w, off_s, off_b, total};
     std::memcpy(buf.data() + 48, offs, 32);
-    std::memcpy(buf.data() + off_w, w.weight.data(), w.weight.size());
+    std::memcpy(buf.data() + off_w, payload.data(), payload.size());
     std::memcpy(buf.data() + off_s, w.scales.data(), w.scales.size() * sizeof(float));
     if (!w.bias.empty()) std::memcpy(buf.data() + off_b, w.bias.data(), w.bias.size() * sizeof(float));
     // the checksum covers the header too (its own field counted as zero), so a damaged dimension or offset is
@@ -305,6 +330,7 @@ inline Result<QuantizedWeights> load_quantized_weights(const std::string &path) 
     if (!f) return TorshError::invalid_argument("Failed to open " + path);
     std::vector<unsigned char> buf((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
     auto bad = [&](const char *why) { return TorshError::invalid_argument(path + ": " + why); };
+    // (the row / length extraction below needs them before the sections are read)
     if (buf.size() < 256 || std::memcmp(buf.data(), detail::kWeightMagic, 8) != 0)
         return bad("not a quantized-weight file");
     uint32_t kind, flags;
@@ -336,12 +362,20 @@ inline Result<QuantizedWeights> load_quantized_weights(const std::string &path) 
         !detail::mul_fits(rows64, sizeof(float), &fbytes) || fbytes > size)
         return bad("implausible dims");
     const size_t rows = static_cast<size_t>(rows64), len = static_cast<size_t>(len64);
-    const bool has_bias = (flags & 1u) != 0;
+    const bool has_bias = (flags & 1u) != 0, prepared = (flags & 2u) != 0;
+    if (flags & ~3u) return bad("unknown flags");
+    if (prepared && kind != QuantizedWeights::Linear) return bad("a prepared operand belongs to linear weights");
     auto inside = [&](uint64_t off, uint64_t need) { return off >= 256 && off <= size && need <= size - off; };
-    if (!inside(offs[0], wbytes) || !inside(offs[1], fbytes) || (has_bias && !inside(offs[2], fbytes)))
+    const uint64_t payload_bytes = prepared ? packed_layout::bytes(rows, len) : wbytes;  // (rows * len fits: wbytes does)
+    if (!inside(offs[0], payload_bytes) || !inside(offs[1], fbytes) || (has_bias && !inside(offs[2], fbytes)))
         return bad("section outside the file");
-    w.weight.assign(reinterpret_cast<const int8_t *>(buf.data() + offs[0]),
-                    reinterpret_cast<const int8_t *>(buf.data() + offs[0]) + rows * len);
+    const int8_t *payload = reinterpret_cast<const int8_t *>(buf.data() + offs[0]);
+    if (prepared) {
+        w.packed.assign(payload, payload + payload_bytes);
+        w.weight = packed_layout::unpack(w.packed, rows, len);  // the row-major view, for parameters() and checks
+    } else {
+        w.weight.assign(payload, payload + rows * len);
+    }
     w.scales.resize(rows);
     std::memcpy(w.scales.data(), buf.data() + offs[1], rows * sizeof(float));
     if (has_bias) {
