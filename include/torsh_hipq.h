@@ -490,6 +490,35 @@ HIPQ_API int32_t hipq_gelu_tanh_quantize_f32_i8(hipq_ctx *ctx, const float *x, s
 /* out = a + b (skip connection; Tensor::add). */
 HIPQ_API int32_t hipq_add_f32(hipq_ctx *ctx, const float *a, const float *b, size_t n, float *out);
 
+/* ---- Linear forward with the row operation that follows it in one kernel ---- */
+/* In a transformer block every int8 product feeds an operation over whole rows (a per-token quantizer, a
+ * LayerNorm).  These forms give a workgroup 32 whole rows of the output (all n columns, the accumulators in
+ * registers), so that operation runs on the accumulators and the fp32 product never goes to memory.  Operands
+ * are packed (above); n % 32 == 0 and n <= 3072 (outputs that are packed int8: n % 128 == 0); m, k any.
+ * Results are those of the separate calls named with each: the same f32 operations per element in the same
+ * order.  Only a LayerNorm's row sums are folded in another order, which moves its mean and variance in their
+ * last bits (tests bound the effect: codes differ by at most one step where a value sits on a rounding edge). */
+/* hipq_linear_packed_i8_f32 (operations.rs:669,722; ops.rs:561): same bits, fp32 row-major [m, n]. */
+HIPQ_API int32_t hipq_linear_rows_packed_i8_f32(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                                int32_t a_scale_per_row, const int8_t *w_packed,
+                                                const float *w_scales, const float *bias, size_t m, size_t n,
+                                                size_t k, float *out);
+/* hipq_linear_packed_i8_f32, then hipq_gelu_tanh_quantize_f32_i8 (GELU: modern.rs:124-136; per-token
+ * quantizer: quantize_per_channel_auto on axis 0, algorithms.rs:126-242), the codes written as the packed
+ * operand [m, n] of the next product: same bits as those two calls and hipq_pack_rows_i8. */
+HIPQ_API int32_t hipq_linear_gelu_quantize_packed_i8(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                                     int32_t a_scale_per_row, const int8_t *w_packed,
+                                                     const float *w_scales, const float *bias, size_t m, size_t n,
+                                                     size_t k, int32_t mode, int8_t *out_packed, float *out_scales);
+/* x[m, n] += the product (hipq_linear_i8_f32_residual: Tensor::add on the Linear's output), then, when
+ * out_packed is not NULL, LayerNorm of the new rows (layer_group/mod.rs:130-166) and the per-token quantizer,
+ * packed: hipq_add_layer_norm_quantize_f32_i8 and hipq_pack_rows_i8 on the same operands.  x is bit-identical
+ * to the separate calls'.  gamma / beta [n] may be NULL. */
+HIPQ_API int32_t hipq_linear_residual_layer_norm_quantize_packed_i8(
+    hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale, int32_t a_scale_per_row, const int8_t *w_packed,
+    const float *w_scales, const float *bias, size_t m, size_t n, size_t k, float *x, const float *gamma,
+    const float *beta, float eps, int32_t mode, int8_t *out_packed, float *out_scales);
+
 /* ---- quantized elementwise operators of the backend trait --------------- */
 /* CpuQuantizationOps::qadd, crates/torsh-backend/src/quantization/ops.rs:582-606:
  * out = quantize(dequantize(a) + dequantize(b)) with output parameters derived
@@ -618,6 +647,17 @@ HIPQ_API size_t hipq_transformer_stack_workspace_bytes(size_t tokens, size_t d_m
 HIPQ_API int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_block_weights *blocks, size_t n_layers,
                                                     size_t tokens, size_t d_model, size_t d_ff, float eps,
                                                     int32_t mode, float *x, void *workspace, size_t workspace_bytes);
+/* The same forward on PREPARED weights: every w_* of `blocks` points to the packed form of the [out, in] matrix
+ * (hipq_pack_rows_i8, once, when the model is converted).  Five kernels per layer: each Linear that feeds a row
+ * operation applies it in its epilogue (hipq_linear_residual_layer_norm_quantize_packed_i8,
+ * hipq_linear_gelu_quantize_packed_i8), and int8 activations stay packed between them.  x is what
+ * hipq_transformer_stack_forward_f32 computes up to the fold order of the LayerNorm sums (see those entry
+ * points).  d_model and d_ff: multiples of 128, at most 3072 (else HIPQ_SHAPE_ERROR: use the form above). */
+HIPQ_API size_t hipq_transformer_stack_prepared_workspace_bytes(size_t tokens, size_t d_model, size_t d_ff);
+HIPQ_API int32_t hipq_transformer_stack_forward_prepared_f32(hipq_ctx *ctx, const hipq_block_weights *blocks,
+                                                             size_t n_layers, size_t tokens, size_t d_model,
+                                                             size_t d_ff, float eps, int32_t mode, float *x,
+                                                             void *workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

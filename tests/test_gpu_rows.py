@@ -1,0 +1,248 @@
+"""Parity of the row-panel Linear forwards (a workgroup owns 32 whole rows of the output and applies the row
+operation that follows the Linear - per-token quantizer, GELU, skip connection, LayerNorm - to its accumulators)
+and of the projection stack built from them.
+
+What is bit-exact and what is not:
+  * the fp32 product, the skip connection and GELU + per-token int8 perform, per element, the f32 operations of
+    the separate entry points in their order: outputs are compared bit for bit with those entry points, which
+    the other test files hold against the CPU oracle;
+  * a LayerNorm folds its row sums in another order than the row kernel (any two orders differ in the last bits
+    of mean and variance), so its per-token scales are held to 1e-6 relative and its codes to one step, on at most
+    1e-5 of the elements; the oracle's LayerNorm of the device's own x gives a second, independent bound.
+"""
+import numpy as np
+import pytest
+import torch
+
+from test_gpu_packed import dev, host, pack_reference, rand_i8
+
+pytestmark = pytest.mark.gpu
+
+
+def unpack_reference(p: np.ndarray, rows: int, k: int) -> np.ndarray:
+    """Inverse of pack_reference: packed bytes -> int8 [rows, k]."""
+    rb, kb = (rows + 31) // 32, ((k + 31) // 32 + 3) // 4 * 4
+    t = p.reshape(rb, kb, 2, 32, 16).transpose(0, 3, 1, 2, 4).reshape(rb * 32, kb * 32)
+    return np.ascontiguousarray(t[:rows, :k])
+
+
+def operands(rng, m, n, k, per_row=True, bias=True):
+    a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+    sa = (rng.uniform(0.001, 0.02, m if per_row else 1)).astype(np.float32)
+    sw = rng.uniform(1e-4, 2e-3, n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32) if bias else None
+    return a, w, sa, sw, b
+
+
+def bits(t):
+    return host(t).view(np.int32)
+
+
+# m ragged and whole; n: every instantiation (<= 768, <= 1536, <= 2304, <= 3072) and widths that leave waves
+# without columns; k ragged, one stage of the activation panel (768), several (1600, 3072)
+F32_SHAPES = [(1, 32, 16), (100, 256, 96), (33, 96, 70), (64, 160, 768), (257, 768, 800), (40, 1536, 1600),
+              (130, 2304, 768), (96, 3072, 768), (65, 800, 3072), (32, 2080, 64)]
+
+
+@pytest.mark.parametrize("m,n,k", F32_SHAPES)
+@pytest.mark.parametrize("per_row,bias", [(True, True), (False, False)])
+def test_linear_rows_f32_equals_the_tiled_form(ctx, oracle, m, n, k, per_row, bias):
+    rng = np.random.default_rng(m * 31 + n * 7 + k)
+    a, w, sa, sw, b = operands(rng, m, n, k, per_row, bias)
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    bd = dev(b) if bias else None
+    got = ctx.linear_rows_packed_i8_f32(pa, dev(sa), pw, dev(sw), bd, m, n, k)
+    want = ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), bd, m, n, k)
+    np.testing.assert_array_equal(bits(got), bits(want))
+    if m * n * k <= 1 << 24:  # and the oracle itself where it is quick
+        acc = oracle.gemm_i8_nk(a, w)
+        ref = oracle.linear_dequant_epilogue(acc, np.broadcast_to(sa, (m,)).copy(), sw, b)
+        np.testing.assert_array_equal(host(got), ref)
+
+
+Q_SHAPES = [(1, 128, 32), (100, 256, 96), (33, 128, 70), (257, 768, 800), (40, 1536, 1600), (130, 2304, 768),
+            (96, 3072, 768), (65, 768, 3072), (70, 1024, 200)]
+
+
+@pytest.mark.parametrize("m,n,k", Q_SHAPES)
+@pytest.mark.parametrize("mode", [0, 1])
+def test_linear_gelu_quantize_equals_its_parts(ctx, hipq, m, n, k, mode):
+    rng = np.random.default_rng(m * 13 + n * 5 + k + mode)
+    a, w, sa, sw, b = operands(rng, m, n, k)
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    rmode = hipq.ROUND_HALF_EVEN if mode else 0
+    f = ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    q, s = ctx.gelu_tanh_quantize(f, mode=rmode)
+    got_q, got_s = ctx.linear_gelu_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), m, n, k, mode=rmode)
+    np.testing.assert_array_equal(bits(got_s), bits(s))
+    np.testing.assert_array_equal(host(got_q), pack_reference(host(q)))  # (padding rows and k blocks: zeros)
+
+
+def test_linear_gelu_quantize_rows_that_are_not_finite(ctx):
+    """A row whose GELU output holds an infinity gets a NaN scale and zero codes, a NaN element is code 0 and does
+    not enter the row's maximum: as the row kernel has it."""
+    rng = np.random.default_rng(5)
+    m, n, k = 40, 256, 64
+    a, w, sa, sw, b = operands(rng, m, n, k)
+    b[3] = np.inf
+    sa[7] = np.nan  # a whole row of NaN
+    sw[9] = np.nan  # one NaN per row
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    f = ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    q, s = ctx.gelu_tanh_quantize(f)
+    got_q, got_s = ctx.linear_gelu_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    assert np.isnan(host(got_s)).sum() >= m - 1  # (column 3 is +inf in every row; row 7 is NaN throughout)
+    np.testing.assert_array_equal(np.isnan(host(got_s)), np.isnan(host(s)))
+    np.testing.assert_array_equal(host(got_q), pack_reference(host(q)))
+    b[3] = 0.5
+    f = ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    q, s = ctx.gelu_tanh_quantize(f)
+    got_q, got_s = ctx.linear_gelu_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    np.testing.assert_array_equal(bits(got_s), bits(s))
+    np.testing.assert_array_equal(host(got_q), pack_reference(host(q)))
+
+
+LN_SHAPES = [(1, 128, 32), (100, 256, 96), (257, 768, 800), (65, 768, 3072), (40, 1536, 160), (48, 3072, 64)]
+
+
+@pytest.mark.parametrize("m,n,k", LN_SHAPES)
+@pytest.mark.parametrize("affine", [True, False])
+def test_linear_residual_layer_norm_quantize(ctx, oracle, m, n, k, affine):
+    rng = np.random.default_rng(m * 3 + n + k)
+    a, w, sa, sw, b = operands(rng, m, n, k)
+    x0 = rng.standard_normal((m, n)).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, n).astype(np.float32) if affine else None
+    beta = (rng.standard_normal(n) * 0.1).astype(np.float32) if affine else None
+    gd, bd = (dev(gamma), dev(beta)) if affine else (None, None)
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    # the separate entry points
+    f = ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    x_parts = dev(x0)
+    q, s = ctx.add_layer_norm_quantize(x_parts, f, gd, bd)
+    # one kernel
+    x_one = dev(x0)
+    got_q, got_s = ctx.linear_residual_layer_norm_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), m, n, k, x_one, gd, bd)
+    np.testing.assert_array_equal(bits(x_one), bits(x_parts))  # the stream: bit for bit
+    np.testing.assert_allclose(host(got_s), host(s), rtol=1e-6, atol=0)
+    codes = unpack_reference(host(got_q), m, n).astype(np.int16)
+    diff = np.abs(codes - host(q).astype(np.int16))
+    assert diff.max() <= 1
+    assert (diff != 0).mean() <= 1e-5 + 2.0 / diff.size
+    # against the oracle's LayerNorm of the device's own stream (f32 sums in yet another order): every code
+    # within one step of the oracle's quantization of its own LayerNorm output
+    h = oracle.layer_norm(host(x_one), gamma, beta, 1e-5)
+    oq, osc, _ = oracle.quantize_per_channel_auto(h, 0, 0, oracle.PER_CHANNEL_SYMMETRIC)
+    np.testing.assert_allclose(host(got_s), osc, rtol=2e-6, atol=0)
+    assert np.abs(codes - oq.astype(np.int16)).max() <= 1
+    # padding of the packed output is zero
+    full = host(got_q)
+    np.testing.assert_array_equal(full, pack_reference(codes.astype(np.int8)))
+    # without the LayerNorm: only the skip connection
+    x_res = dev(x0)
+    ctx.linear_residual_layer_norm_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), m, n, k, x_res, normalize=False)
+    np.testing.assert_array_equal(bits(x_res), bits(x_parts))
+
+
+def test_row_panel_shapes_that_are_refused(ctx, hipq):
+    rng = np.random.default_rng(1)
+    a, w, sa, sw, b = operands(rng, 8, 3104, 32)
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    with pytest.raises(hipq.HipqError) as e:  # wider than a workgroup's registers hold
+        ctx.linear_rows_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), 8, 3104, 32)
+    assert e.value.code == hipq.SHAPE_ERROR
+    a, w, sa, sw, b = operands(rng, 8, 96, 32)
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    with pytest.raises(hipq.HipqError) as e:  # a packed int8 output is the K of the next product: whole groups of 4 k blocks
+        ctx.linear_gelu_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), 8, 96, 32)
+    assert e.value.code == hipq.SHAPE_ERROR
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.linear_rows_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), 8, 90, 32)
+    assert e.value.code == hipq.SHAPE_ERROR
+    # nothing to do
+    ctx.linear_rows_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), 0, 96, 32, out=torch.empty((0, 96), device="cuda"))
+
+
+# ---- the projection stack on prepared weights ---------------------------------------------------------------
+
+from test_gpu_stack import _make_blocks, _oracle_stack  # noqa: E402
+
+
+@pytest.mark.parametrize("tokens,d,dff,layers", [(48, 128, 512, 2), (130, 256, 1024, 3)])
+def test_prepared_stack_small_against_the_oracle(ctx, oracle, tokens, d, dff, layers):
+    rng = np.random.default_rng(tokens + d)
+    blocks_h = _make_blocks(rng, layers, d, dff, oracle)
+    for blk in blocks_h:
+        for ln in ("ln1", "ln2"):
+            blk[ln + "_gamma"] = rng.uniform(0.5, 1.5, d).astype(np.float32)
+            blk[ln + "_beta"] = (rng.standard_normal(d) * 0.1).astype(np.float32)
+    x = rng.standard_normal((tokens, d)).astype(np.float32)
+    want = _oracle_stack(oracle, blocks_h, x, d)
+    blocks_d = [{k: dev(v) for k, v in blk.items()} for blk in blocks_h]
+    prepared = ctx.stack_prepare(blocks_d)
+    got = host(ctx.stack_forward(prepared, dev(x), dff, ctx.stack_workspace_prepared(tokens, d, dff), prepared=True))
+    plain = host(ctx.stack_forward(blocks_d, dev(x), dff, ctx.stack_workspace(tokens, d, dff)))
+    # fp32 LayerNorm / GELU rounding feeds re-quantization (an occasional code flips by one level); the same loose
+    # bound as for the unprepared stack, and the two device forms as close to each other as to the oracle
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want)
+    rel_plain = np.linalg.norm(got - plain) / np.linalg.norm(plain)
+    print(f"prepared stack tokens={tokens} d={d} layers={layers}: rel L2 vs oracle {rel:.3e}, vs the plain stack {rel_plain:.3e}")
+    assert rel < 2e-3
+    assert rel_plain < 2e-3
+
+
+def test_prepared_stack_full_size_equals_its_parts(ctx, hipq):
+    """Config 5 at its real size (8192 tokens, d = 768, d_ff = 3072; 3 layers keep the test short): the one call is
+    bit-identical to the same layers composed from the entry points tested above, and stays within the drift bound
+    of the stack on row-major weights."""
+    tokens, d, dff, layers = 8192, 768, 3072, 3
+    g = torch.Generator(device="cuda").manual_seed(11)
+    blocks = []
+    for _ in range(layers):
+        blk = {}
+        for name, (o, i) in {"qkv": (3 * d, d), "out": (d, d), "fc1": (dff, d), "fc2": (d, dff)}.items():
+            wf = torch.randn(o, i, generator=g, device="cuda") * 0.02
+            q, sc, _, _ = ctx.quantize_per_row(wf)
+            blk["w_" + name], blk["s_" + name] = q, sc
+            blk["b_" + name] = torch.randn(o, generator=g, device="cuda") * 0.01
+        for ln in ("ln1", "ln2"):
+            blk[ln + "_gamma"] = torch.rand(d, generator=g, device="cuda") + 0.5
+            blk[ln + "_beta"] = torch.randn(d, generator=g, device="cuda") * 0.1
+        blocks.append(blk)
+    prepared = ctx.stack_prepare(blocks)
+    x0 = torch.randn(tokens, d, generator=g, device="cuda")
+    got = ctx.stack_forward(prepared, x0.clone(), dff, ctx.stack_workspace_prepared(tokens, d, dff), prepared=True)
+    x = x0.clone()
+    q, s = ctx.layer_norm_quantize(x, blocks[0]["ln1_gamma"], blocks[0]["ln1_beta"], 1e-5)
+    qa = ctx.pack_rows(q)
+    for i, blk in enumerate(prepared):
+        qkv = ctx.linear_packed_i8_f32(qa, s, blk["w_qkv"], blk["s_qkv"], blk["b_qkv"], tokens, 3 * d, d)
+        q, s = ctx.quantize_per_row_strided(qkv, tokens, d, 3 * d, elem_offset=2 * d)
+        qa, s = ctx.linear_residual_layer_norm_quantize_packed(ctx.pack_rows(q), s, blk["w_out"], blk["s_out"], blk["b_out"],
+                                                               tokens, d, d, x, blk["ln2_gamma"], blk["ln2_beta"])
+        qb, sb = ctx.linear_gelu_quantize_packed(qa, s, blk["w_fc1"], blk["s_fc1"], blk["b_fc1"], tokens, dff, d)
+        last = i + 1 == layers
+        nxt = None if last else prepared[i + 1]
+        qa, s = ctx.linear_residual_layer_norm_quantize_packed(
+            qb, sb, blk["w_fc2"], blk["s_fc2"], blk["b_fc2"], tokens, d, dff, x,
+            None if last else nxt["ln1_gamma"], None if last else nxt["ln1_beta"], normalize=not last)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all()
+    assert torch.equal(got, x)
+    plain = ctx.stack_forward(blocks, x0.clone(), dff, ctx.stack_workspace(tokens, d, dff))
+    rel = float((got - plain).norm() / plain.norm())
+    print(f"prepared vs plain stack at full size, {layers} layers: rel L2 {rel:.3e}")
+    assert rel < 2e-3
+
+
+def test_prepared_stack_arguments(ctx, hipq):
+    x = torch.zeros((8, 128), device="cuda")
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.stack_forward([{}], x, 512, torch.empty(1024, dtype=torch.uint8, device="cuda"), prepared=True)
+    assert e.value.code == hipq.INVALID_ARGUMENT
+    with pytest.raises(hipq.HipqError) as e:  # d_ff beyond what a workgroup's registers hold
+        ctx.stack_forward([{}], x, 4096, ctx.stack_workspace_prepared(8, 128, 4096), prepared=True)
+    assert e.value.code == hipq.SHAPE_ERROR
+    with pytest.raises(hipq.HipqError) as e:
+        ctx.stack_forward([{}], torch.zeros((8, 96), device="cuda"), 512, ctx.stack_workspace_prepared(8, 96, 512),
+                          prepared=True)
+    assert e.value.code == hipq.SHAPE_ERROR

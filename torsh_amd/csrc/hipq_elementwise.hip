@@ -1939,6 +1939,12 @@ int32_t hipq::quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t
                          -128, 127, mode, out, out_scales, nullptr, nullptr, /*poison=*/1, packed);
 }
 
+int32_t hipq::quantize_activations_per_row_strided(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
+                                                   int32_t mode, int8_t *out, float *out_scales, bool packed) {
+    return quantize_rows("hipq_linear (activation quantize)", ctx, x, rows, cols, ld, HIPQ_PARAMS_SYMMETRIC, false,
+                         -128, 127, mode, out, out_scales, nullptr, nullptr, /*poison=*/1, packed);
+}
+
 extern "C" {
 
 int32_t hipq_quantize_per_row_strided_f32_i8(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,

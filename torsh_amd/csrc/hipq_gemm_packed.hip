@@ -4,6 +4,7 @@
 // order" of a prepared weight blob); activations are written in the packed layout by the quantize
 // pass itself, so the forward costs no extra pass over either operand.
 #include "hipq_gemm_packed.h"
+#include "hipq_gemm_rows.h"
 
 namespace hipq {
 
@@ -316,6 +317,76 @@ int32_t hipq_linear_static_packed_f32(hipq_ctx *ctx, const float *x, float a_sca
     rc = quantize_activations_per_tensor(ctx, x, m, k, false, a_scale, mode, true, pa, params, nullptr, 0);
     if (rc) return rc;
     return linear_packed_launch(ctx, pa, &params->scale, 0, w_packed, w_scales, bias, m, n, k, out, true);
+}
+
+// ---- row-panel forms: a workgroup owns 32 whole rows of the output (hipq_gemm_rows.h) -------------------------
+
+static int32_t check_rows_args(const char *fn, hipq_ctx *ctx, size_t m, size_t n, size_t k) {
+    int32_t rc = check_packed_shape(fn, m, n, k);
+    if (rc) return rc;
+    if (k == 0) return fail(HIPQ_INVALID_ARGUMENT, "%s: K must be positive", fn);
+    (void)ctx;
+    return HIPQ_SUCCESS;
+}
+
+int32_t hipq_linear_rows_packed_i8_f32(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale, int32_t a_scale_per_row,
+                                       const int8_t *w_packed, const float *w_scales, const float *bias, size_t m,
+                                       size_t n, size_t k, float *out) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_rows_args(__func__, ctx, m, n, k);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(a_packed);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out);
+    RowPanel p{a_packed, a_scale, a_scale_per_row ? 1 : 0, w_packed, w_scales, bias, static_cast<int>(m),
+               static_cast<int>(n), static_cast<int>(k), out, nullptr, nullptr, nullptr, nullptr, 0.0f};
+    return launch_rows<RP_F32>(ctx, p, false);
+}
+
+int32_t hipq_linear_gelu_quantize_packed_i8(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                            int32_t a_scale_per_row, const int8_t *w_packed, const float *w_scales,
+                                            const float *bias, size_t m, size_t n, size_t k, int32_t mode,
+                                            int8_t *out_packed, float *out_scales) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_rows_args(__func__, ctx, m, n, k);
+    if (rc) return rc;
+    if (mode & ~HIPQ_ROUND_HALF_EVEN) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", __func__);
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(a_packed);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(out_packed);
+    HIPQ_REQUIRE_PTR(out_scales);
+    RowPanel p{a_packed, a_scale, a_scale_per_row ? 1 : 0, w_packed, w_scales, bias, static_cast<int>(m),
+               static_cast<int>(n), static_cast<int>(k), nullptr, out_packed, out_scales, nullptr, nullptr, 0.0f};
+    return launch_rows<RP_GELU_Q>(ctx, p, (mode & HIPQ_ROUND_HALF_EVEN) != 0);
+}
+
+int32_t hipq_linear_residual_layer_norm_quantize_packed_i8(hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale,
+                                                           int32_t a_scale_per_row, const int8_t *w_packed,
+                                                           const float *w_scales, const float *bias, size_t m, size_t n,
+                                                           size_t k, float *x, const float *gamma, const float *beta,
+                                                           float eps, int32_t mode, int8_t *out_packed,
+                                                           float *out_scales) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_rows_args(__func__, ctx, m, n, k);
+    if (rc) return rc;
+    if (mode & ~HIPQ_ROUND_HALF_EVEN) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", __func__);
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(a_packed);
+    HIPQ_REQUIRE_PTR(a_scale);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(x);
+    RowPanel p{a_packed, a_scale, a_scale_per_row ? 1 : 0, w_packed, w_scales, bias, static_cast<int>(m),
+               static_cast<int>(n), static_cast<int>(k), x, out_packed, out_scales, gamma, beta, eps};
+    if (!out_packed) return launch_rows<RP_RESID_F32>(ctx, p, false);  // no LayerNorm to feed: x += product only
+    HIPQ_REQUIRE_PTR(out_scales);
+    return launch_rows<RP_RESID_LN_Q>(ctx, p, (mode & HIPQ_ROUND_HALF_EVEN) != 0);
 }
 
 }  // extern "C"

@@ -1,0 +1,437 @@
+// int8 GEMM on fragment-packed operands with one PANEL OF ROWS per workgroup: 32 rows of the activations against
+// ALL columns of the weights, the whole panel of accumulators in registers (N / 32 blocks of 32 x 32, an eighth of
+// them per wave: up to 192 registers).
+//
+// Why.  In a transformer block the products are tall and short in K (8192 x 2304 x 768, 8192 x 3072 x 768, ...)
+// and every one of them feeds an operation that needs whole rows: a per-token quantizer (the row's maximum), a
+// LayerNorm (the row's mean and variance).  Tiles of 128 or 256 columns cannot apply those, so the fp32 product
+// goes to memory and comes back through a row kernel: 100 MB out and 100 MB in for fc1 alone, more time than the
+// multiply.  A workgroup that owns whole rows applies them in its epilogue, on the accumulators:
+//   RP_F32         out = acc * (s_a[m] * s_w[n]) + bias[n]                                   (qkv)
+//   RP_GELU_Q      per-token int8 of GELU(that), written as the packed operand of the next product      (fc1)
+//   RP_RESID_F32   x += that                                                                 (the last fc2)
+//   RP_RESID_LN_Q  x += that, then per-token int8 of LayerNorm(x), packed                     (out-proj, fc2)
+// Every f32 operation is the one the separate kernels perform (same functions, same order per element); only the
+// order in which a LayerNorm's row sums are folded differs (here: over a lane's column blocks, the 32 lanes of a
+// half wave, the eight waves), which moves the mean and variance in their last bits, as any other order does.
+//
+// The price is operand traffic: every workgroup streams the whole weight matrix (out of its XCD's L2, which holds
+// it), one 1 KiB fragment per MFMA - 128 bytes per clock and compute unit wanted, ~57 delivered - so the main loop
+// runs at the vector-memory path's pace, N * K / 57 cycles.  The activations stay off that path: the panel's
+// fragments go through LDS, 24 k blocks at a time (two buffers, one barrier per 24 k blocks), and every wave
+// reads the fragment of a k block from there.  Weight fragments go from L2 straight into registers, D in flight
+// per wave (48 KiB or more per compute unit: what the path needs to stay busy at its latency).
+//
+// M any; K any; N a multiple of 32 and at most 3072 (the *_Q forms: a multiple of 128, since their output is the
+// K of the next product).  Included by hipq_gemm_packed.hip.
+#pragma once
+
+#include "hipq_gemm_packed.h"
+
+namespace hipq {
+
+enum { RP_F32 = 0, RP_GELU_Q = 1, RP_RESID_F32 = 2, RP_RESID_LN_Q = 3 };
+
+struct RowPanel {
+    const int8_t *pa;   // packed activations [M, K]
+    const float *sa;    // activation scales: [M] (sa_per_row) or one
+    int sa_per_row;
+    const int8_t *pw;   // packed weights [N, K]
+    const float *sw;    // [N]
+    const float *bias;  // [N] or null
+    int M, N, K;
+    float *out_f;       // RP_F32: [M, N]; RP_RESID_*: the stream x [M, N], read and written
+    int8_t *out_q;      // *_Q: packed int8 [M, N]
+    float *out_scales;  // *_Q: [M]
+    const float *gamma, *beta;  // RP_RESID_LN_Q: [N] or null
+    float eps;
+};
+
+constexpr int kRowsWaves = 8;
+constexpr int kRowsThreads = kRowsWaves * kWave;
+constexpr int kRowsStage = 24;  // k blocks of the activation panel per LDS buffer (24 KiB)
+
+// tanh-form GELU as the row kernels evaluate it (gelu_tanh in hipq_fp32.hip: the same three lines).
+__device__ __forceinline__ float rp_gelu_tanh(float x) {
+    constexpr float K = -2.8853900817779268f * 0.7978845608028654f;
+    const float arg = x * fmaf(x * x, K * 0.044715f, K);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(arg));
+}
+
+// Maximum or sum over the 32 lanes of a half wave, the result in every lane: four steps inside a row of 16 lanes
+// on the data-parallel path (quad swaps, then the mirrors of 8 and 16 lanes: after each step the groups that were
+// combined hold one value), one swizzle across the two rows.  Both partners of a step add the same two numbers,
+// so all lanes end with the same bits.  MAX is for non-negative values that are no NaN: those order as their bit
+// patterns do, and an integer maximum needs no quieting of its operands.
+template <bool MAX>
+__device__ __forceinline__ float half_wave_fold(float v) {
+    auto combine = [](float a, float b) {
+        if constexpr (MAX) {
+            const uint32_t x = __builtin_bit_cast(uint32_t, a), y = __builtin_bit_cast(uint32_t, b);
+            const uint32_t m = x > y ? x : y;
+            return __builtin_bit_cast(float, m);
+        } else {
+            return a + b;
+        }
+    };
+    auto dpp = [](float x, auto ctrl) {
+        const int bits = __builtin_bit_cast(int, x);
+        const int moved = __builtin_amdgcn_update_dpp(0, bits, decltype(ctrl)::value, 0xf, 0xf, false);
+        return __builtin_bit_cast(float, moved);
+    };
+    v = combine(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1, 0, 3, 2]
+    v = combine(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2, 3, 0, 1]
+    v = combine(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror
+    v = combine(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror
+    const int bits = __builtin_bit_cast(int, v);
+    const int other = __builtin_amdgcn_ds_swizzle(bits, 0x401F);  // lane ^ 16 (and 0x1f, or 0, xor 0x10)
+    return combine(v, __builtin_bit_cast(float, other));
+}
+
+constexpr int rows_gcd(int a, int b) { return b == 0 ? a : rows_gcd(b, a % b); }
+
+template <int NBW, int EPI, bool EVEN>
+__global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) {
+    constexpr int D = NBW <= 6 ? 12 : (NBW == 9 ? 9 : 6);  // weight fragments in flight per wave
+    constexpr int U = D / rows_gcd(NBW, D);  // k blocks per trip of the main loop: U * NBW is a multiple of D
+    static_assert((U * NBW) % D == 0 && kRowsStage % U == 0, "ring slots must be static");
+    constexpr bool QUANT = EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q;
+    constexpr bool RESID = EPI == RP_RESID_F32 || EPI == RP_RESID_LN_Q;
+    // The epilogue handles GS groups of four accumulator registers (= 4 rows per half wave) at a time: all 16 rows
+    // where registers allow, else one group after the other (the row statistics then take a barrier per group).
+    constexpr int GS = NBW <= 6 ? 4 : 1;
+    constexpr int NR = 4 * GS;
+    __shared__ __attribute__((aligned(1024))) int8_t apanel[2][kRowsStage * 1024];
+    __shared__ __attribute__((aligned(16))) float red[3][kRowsWaves][32];  // [statistic][wave][row]: partial sums / maxima
+    __shared__ __attribute__((aligned(16))) float fin[4][32];              // per row: mean, 1 / std, scale, 1 / scale
+    const int tid = threadIdx.x, lane = tid % kWave, half = lane / 32, cin = lane % 32;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int rb = blockIdx.x, m0 = rb * 32;
+    const int KB = static_cast<int>(packed_k_blocks(p.K));  // (a multiple of 4)
+    const int nblocks = p.N / 32;
+    const int jb0 = wave * NBW;  // this wave's column blocks: jb0 .. jb0 + NBW - 1 (those past nblocks: no data)
+    // Exact extents: a fragment past the operand (column blocks past N, k blocks past the last) reads as zeros
+    // without touching memory, or as data of the next column block that no MFMA consumes.
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t *>(p.pa) + size_t(rb) * KB * 1024, 0, KB * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(p.pw), 0, nblocks * KB * 1024, 0x00020000);
+    const int voff = lane * 16;
+    const int wstride = KB * 1024;  // bytes between the column blocks of one k block
+    const int wbase = jb0 * wstride;
+    auto load_w = [&](int kb, int jj) {
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, wbase + jj * wstride + kb * 1024, 0));
+    };
+    // one stage of the activation panel: 24 KiB = three 16-byte pieces per thread
+    auto load_stage = [&](int s, v4i(&t)[3]) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+            t[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                               ra, tid * 16, s * (kRowsStage * 1024) + i * (kRowsThreads * 16), 0));
+    };
+
+    // fp32 rows of this panel (output, or the stream that is read and written): rows past M lie beyond the buffer
+    // and are dropped by the hardware.
+    const int rows_here = p.M - m0 < 32 ? p.M - m0 : 32;
+    const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(
+        p.out_f ? reinterpret_cast<char *>(p.out_f) + size_t(m0) * p.N * 4 : nullptr, 0, p.out_f ? rows_here * p.N * 4 : 0,
+        0x00020000);
+    const int row_bytes = p.N * 4;
+    auto load_x = [&](int jj, int r) {
+        return __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(rf, (4 * half * p.N + (jb0 + jj) * 32 + cin) * 4,
+                                                        (8 * (r / 4) + (r % 4)) * row_bytes, 0));
+    };
+
+    // The weights are new to this XCD's L2 when the kernel starts (the previous layer used others), and all its
+    // workgroups walk them in the same order at the same time: every fragment would be a miss for all of them at
+    // once, and the walk would move at memory latency.  So each workgroup first touches its own thirty-second of
+    // the matrix (workgroups b, b + 8, b + 16, ... share an XCD), one dword per 128-byte line: the whole matrix is
+    // on its way into the L2 within one memory latency, and the walk below meets lines that are there or coming.
+    {
+        const int wbytes = nblocks * KB * 1024;
+        const int chunk = ((wbytes + 31) / 32 + 127) & ~127;
+        const int part = (blockIdx.x / 8) % 32;
+        int touched = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int off = (tid + i * kRowsThreads) * 128;
+            if (off < chunk) touched ^= __builtin_amdgcn_raw_buffer_load_b32(rw, off, part * chunk, 0);
+        }
+        // (keeps the loads alive; never true: p.M is positive)
+        if (touched == 0x5a5a5a5a && p.M < 0) red[0][0][0] = 1.0f;
+    }
+    v4i wf[D];
+#pragma unroll
+    for (int u = 0; u < D; ++u) wf[u] = load_w(u / NBW, u % NBW);
+    v4i astage[3];
+    load_stage(0, astage);
+    // Residual values: with few column blocks per wave all of them are requested here, ahead of the main loop,
+    // which hides them completely (and keeps loads from queueing behind the epilogue's stores: one counter).
+    constexpr bool RES_EARLY = RESID && GS == 4;
+    float res_all[RES_EARLY ? NBW : 1][16];
+    if constexpr (RES_EARLY) {
+#pragma unroll
+        for (int jj = 0; jj < NBW; ++jj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) res_all[jj][r] = load_x(jj, r);
+    }
+
+    v16i acc[NBW];
+#pragma unroll
+    for (int j = 0; j < NBW; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+
+    const int stages = (KB + kRowsStage - 1) / kRowsStage;
+    for (int s = 0; s < stages; ++s) {
+        int8_t *buf = apanel[s & 1];
+        // (the last reads of this buffer, two stages ago, lie before the previous stage's barrier)
+#pragma unroll
+        for (int i = 0; i < 3; ++i) *reinterpret_cast<v4i *>(buf + i * (kRowsThreads * 16) + tid * 16) = astage[i];
+        __syncthreads();
+        if (s + 1 < stages) load_stage(s + 1, astage);
+        const int kb_first = s * kRowsStage;
+        const int len = KB - kb_first < kRowsStage ? KB - kb_first : kRowsStage;  // (a multiple of 4)
+        v4i a_cur = *reinterpret_cast<const v4i *>(buf + voff);
+        for (int kl = 0; kl < len; kl += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int nxt = kl + u + 1 < kRowsStage ? kl + u + 1 : kRowsStage - 1;
+                const v4i a_nxt = *reinterpret_cast<const v4i *>(buf + nxt * 1024 + voff);
+                const int kb = kb_first + kl + u;
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    const int slot = (u * NBW + jj) % D;
+                    acc[jj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_cur, wf[slot], acc[jj], 0, 0, 0);
+                    wf[slot] = load_w(kb + (jj + D) / NBW, (jj + D) % NBW);
+                }
+                a_cur = a_nxt;
+            }
+        }
+    }
+
+    // ---- epilogue: a 32 x 32 block has lane = column cin and register r = row 8 * (r / 4) + 4 * half + r % 4 ----
+    // Instructions are what this part costs (the matrix pipe idles meanwhile), so everything that belongs to a row
+    // rather than an element - the divisions of the mean, the variance, the scale and its reciprocal - is done by
+    // ONE thread per row between two barriers, and handed to the row's lanes through LDS.
+    auto row_of = [&](int r) { return 8 * (r / 4) + 4 * half + (r % 4); };
+    // (through a copy: a bit cast applied to the element expression itself reads element 0 of the vector)
+    auto value = [&](int jj, int r) {
+        const int bits = acc[jj][r];
+        return __builtin_bit_cast(float, bits);
+    };
+    // max(a, |b|) as fmaxf gives it for values that come out of arithmetic (a NaN b leaves a), in one instruction
+    auto max_abs = [](float a, float b) {
+        float o;
+        asm("v_max_f32_e64 %0, %1, |%2|" : "=v"(o) : "v"(a), "v"(b));
+        return o;
+    };
+    // Per-lane statistics of the rows of a pass -> one partial per wave and row in LDS.  MAX: non-negative values
+    // that are no NaN, which order as their bit patterns do.
+    auto partials_to_lds = [&](float(&t)[NR], int which, int g0, auto is_max) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) t[i] = half_wave_fold<decltype(is_max)::value>(t[i]);
+        if (cin == 0) {
+#pragma unroll
+            for (int i = 0; i < NR; ++i) red[which][wave][row_of(4 * g0 + i)] = t[i];
+        }
+        __syncthreads();
+    };
+    // (one thread per row: tid < 8 * GS owns row 8 * g0 + tid of the panel)
+    auto row_total = [&](int which, int row, auto is_max) {
+        float w[kRowsWaves];
+#pragma unroll
+        for (int k = 0; k < kRowsWaves; ++k) w[k] = red[which][k][row];
+        if constexpr (decltype(is_max)::value)
+            return fmaxf(fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])), fmaxf(fmaxf(w[4], w[5]), fmaxf(w[6], w[7])));
+        else
+            return ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
+    };
+    auto from_lds = [&](float(&t)[NR], int which, int g0) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) t[i] = fin[which][row_of(4 * g0 + i)];
+    };
+    const int KBo = p.N / 32;  // k blocks of the packed output (a multiple of 4 for the *_Q forms)
+    const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
+        QUANT ? p.out_q + size_t(rb) * KBo * 1024 : nullptr, 0, QUANT ? KBo * 1024 : 0, 0x00020000);
+    const int qd = lane % 4;
+    const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
+    const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+    // after the byte exchange below a lane holds row 8 g + 4 half + qd, columns 4 * (cin / 4) .. + 3 of a block
+    const int qoff = (4 * half + qd + 32 * (cin / 16)) * 16 + 4 * ((cin / 4) % 4);
+    const float cols_f = static_cast<float>(p.N);
+
+#pragma unroll
+    for (int g0 = 0; g0 < 4; g0 += GS) {
+        // rows of this pass: registers r = 4 * g0 + i, i < NR
+        float s_row[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const int m = m0 + row_of(4 * g0 + i);
+            s_row[i] = p.sa[p.sa_per_row ? (m < p.M ? m : p.M - 1) : 0];
+        }
+        // v = acc * (s_a * s_w) + bias (+ residual) (GELU), in place: the accumulator registers then hold float bits
+        float sum[NR], am[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) sum[i] = am[i] = 0.0f;
+#pragma unroll
+        for (int jj = 0; jj < NBW; ++jj) {
+            if (jb0 + jj >= nblocks) continue;  // (wave-uniform)
+            const int col = (jb0 + jj) * 32 + cin;
+            const float swv = p.sw[col];
+            const float bv = p.bias ? p.bias[col] : -0.0f;  // (v + -0.0f is v, bit for bit)
+            float res[NR];
+            if constexpr (RESID) {
+#pragma unroll
+                for (int i = 0; i < NR; ++i) {
+                    if constexpr (RES_EARLY)
+                        res[i] = res_all[jj][4 * g0 + i];
+                    else
+                        res[i] = load_x(jj, 4 * g0 + i);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int r = 4 * g0 + i;
+                float v = static_cast<float>(acc[jj][r]) * (s_row[i] * swv) + bv;
+                if constexpr (RESID) v = v + res[i];
+                if constexpr (EPI == RP_GELU_Q) {
+                    v = rp_gelu_tanh(v);
+                    am[i] = max_abs(am[i], v);
+                }
+                if constexpr (EPI == RP_F32 || RESID)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v), rf, (4 * half * p.N + col) * 4,
+                                                          (8 * (r / 4) + (r % 4)) * row_bytes, EPI == RP_F32 ? 2 : 0);
+                if constexpr (EPI == RP_RESID_LN_Q) sum[i] += v;
+                acc[jj][r] = __builtin_bit_cast(int, v);
+            }
+        }
+        if constexpr (QUANT) {
+            if constexpr (EPI == RP_RESID_LN_Q) {
+                // LayerNorm over the row (biased variance, eps inside the square root): passes over the registers
+                partials_to_lds(sum, 0, g0, std::false_type{});
+                if (tid < 8 * GS) fin[0][8 * g0 + tid] = row_total(0, 8 * g0 + tid, std::false_type{}) / cols_f;
+                __syncthreads();
+                float mean[NR], sq[NR];
+                from_lds(mean, 0, g0);
+#pragma unroll
+                for (int i = 0; i < NR; ++i) sq[i] = 0.0f;
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    if (jb0 + jj >= nblocks) continue;
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) {
+                        const float d = value(jj, 4 * g0 + i) - mean[i];
+                        sq[i] += d * d;
+                    }
+                }
+                partials_to_lds(sq, 1, g0, std::false_type{});
+                if (tid < 8 * GS)
+                    fin[1][8 * g0 + tid] = 1.0f / sqrtf(row_total(1, 8 * g0 + tid, std::false_type{}) / cols_f + p.eps);
+                __syncthreads();
+                float rstd[NR];
+                from_lds(rstd, 1, g0);
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    if (jb0 + jj >= nblocks) continue;
+                    const int col = (jb0 + jj) * 32 + cin;
+                    // (y * 1.0f and y + -0.0f are y, bit for bit)
+                    const float g = p.gamma ? p.gamma[col] : 1.0f, b = p.beta ? p.beta[col] : -0.0f;
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) {
+                        const float y = (value(jj, 4 * g0 + i) - mean[i]) * rstd[i] * g + b;
+                        am[i] = max_abs(am[i], y);
+                        acc[jj][4 * g0 + i] = __builtin_bit_cast(int, y);
+                    }
+                }
+            }
+            // per-token symmetric int8: scale = max|v| / 127 (1 for an all-zero row, NaN for a row that is not
+            // finite), q = clamp(round(v / scale)) with the row's reciprocal (calculate_symmetric_quantization_params
+            // and the division form of quantize_per_channel_auto, as the row kernels apply them).  1 / scale is a
+            // normal number for every scale this rule can give, or NaN with it; rows past M get a NaN scale here,
+            // which makes their codes 0, as a NaN element's code is.
+            partials_to_lds(am, 2, g0, std::true_type{});
+            if (tid < 8 * GS) {
+                const int row = 8 * g0 + tid;
+                const float a = row_total(2, row, std::true_type{});
+                float sc = a < FLT_EPSILON ? 1.0f : a / 127.0f;
+                if (!(fabsf(a) <= FLT_MAX)) sc = NAN;
+                if (m0 + row < p.M)
+                    p.out_scales[m0 + row] = sc;
+                else
+                    sc = NAN;
+                fin[2][row] = sc;
+                fin[3][row] = 1.0f / sc;
+            }
+            __syncthreads();
+            float scale[NR], inv[NR];
+            from_lds(scale, 2, g0);
+            from_lds(inv, 3, g0);
+            // The codes, in the packed layout of the next product's activations: row block rb, k block = column
+            // block, and inside the 1 KiB fragment slot (row + 32 * (column / 16)) of 16 bytes.  A lane holds one
+            // column of four consecutive rows per register group; the four lanes of a quad exchange bytes (four
+            // quad broadcasts, two byte permutes) so that each holds four consecutive columns of ONE row: a dword.
+#pragma unroll
+            for (int jj = 0; jj < NBW; ++jj) {
+                if (jb0 + jj >= nblocks) continue;
+#pragma unroll
+                for (int gi = 0; gi < GS; ++gi) {
+                    int q[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int i = 4 * gi + k;
+                        // x / scale, correctly rounded, from the reciprocal (div_rn without its special cases: see above)
+                        const float x = value(jj, 4 * g0 + i);
+                        const float q0 = x * inv[i];
+                        const float t = fmaf(fmaf(-q0, scale[i], x), inv[i], q0);
+                        q[k] = min(max(cvt_i32_sat(round_mode<EVEN>(t)), -128), 127);
+                    }
+                    const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));  // byte k = row 8 g + 4 half + k
+                    const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
+                    const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
+                    const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
+                    const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
+                    const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                    __builtin_amdgcn_raw_buffer_store_b32(static_cast<int>(word), rq, qoff,
+                                                          (jb0 + jj) * 1024 + (g0 + gi) * 128, 0);
+                }
+            }
+        }
+    }
+}
+
+// Launch of the row-panel kernel: one workgroup of eight waves per 32 rows.  Returns HIPQ_SHAPE_ERROR for what it
+// does not take (N not a multiple of 32 or above 3072; the *_Q forms: N not a multiple of 128).
+template <int EPI>
+static int32_t launch_rows(hipq_ctx *ctx, const RowPanel &p, bool even) {
+    if (p.N % 32 != 0 || p.N > 3072 || p.N <= 0 || p.M <= 0 || p.K <= 0)
+        return fail(HIPQ_SHAPE_ERROR, "row-panel GEMM: N = %d must be a multiple of 32 and at most 3072", p.N);
+    constexpr bool QUANT = EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q;
+    if (QUANT && p.N % 128 != 0)
+        return fail(HIPQ_SHAPE_ERROR, "row-panel GEMM: N = %d must be a multiple of 128 for a packed int8 output", p.N);
+    // (offsets of column blocks past N, which read as zeros, are still computed: price the widest panel)
+    if (packed_bytes(size_t(3072), size_t(p.K)) >= (size_t(1) << 31))
+        return fail(HIPQ_SHAPE_ERROR, "row-panel GEMM: K = %d is too large (32-bit offsets into the weights)", p.K);
+    const dim3 grid((p.M + 31) / 32);
+    const int nbw = (p.N / 32 + kRowsWaves - 1) / kRowsWaves;
+#define HIPQ_LAUNCH_ROWS_NBW(NBW)                                                                                     \
+    do {                                                                                                              \
+        if (even)                                                                                                     \
+            hipLaunchKernelGGL((gemm_i8_rows_kernel<NBW, EPI, true>), grid, dim3(kRowsThreads), 0, ctx->stream, p);  \
+        else                                                                                                          \
+            hipLaunchKernelGGL((gemm_i8_rows_kernel<NBW, EPI, false>), grid, dim3(kRowsThreads), 0, ctx->stream, p); \
+    } while (0)
+    if (nbw <= 3)
+        HIPQ_LAUNCH_ROWS_NBW(3);
+    else if (nbw <= 6)
+        HIPQ_LAUNCH_ROWS_NBW(6);
+    else if (nbw <= 9)
+        HIPQ_LAUNCH_ROWS_NBW(9);
+    else
+        HIPQ_LAUNCH_ROWS_NBW(12);
+#undef HIPQ_LAUNCH_ROWS_NBW
+    return check_launch("gemm_i8 (row panels)");
+}
+
+}  // namespace hipq

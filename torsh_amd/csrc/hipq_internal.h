@@ -116,6 +116,9 @@ int32_t quantize_activations_per_tensor(hipq_ctx *ctx, const float *x, size_t ro
                                         hipq_qparams *out_params, void *partials, size_t partials_bytes);
 int32_t quantize_activations_per_row(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, int32_t mode,
                                      int8_t *out, float *out_scales, bool packed = false);
+// The same for rows that lie `ld` floats apart (a column slice of a wider matrix).
+int32_t quantize_activations_per_row_strided(hipq_ctx *ctx, const float *x, size_t rows, size_t cols, size_t ld,
+                                             int32_t mode, int8_t *out, float *out_scales, bool packed);
 // Looks up, once per device, the address of the static device array behind
 // hipq_linear_dynamic_f32_noalloc; called by hipq_ctx_create with the device current.
 int32_t linear_noalloc_setup(int device);

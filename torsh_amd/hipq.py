@@ -132,7 +132,12 @@ _SIGNATURES = {
     "hipq_gelu_tanh_f32": [_vp, _vp, _sz, _vp],
     "hipq_gelu_tanh_quantize_f32_i8": [_vp, _vp, _sz, _sz, _i32, _vp, _vp],
     "hipq_add_f32": [_vp, _vp, _vp, _sz, _vp],
+    "hipq_linear_rows_packed_i8_f32": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _vp],
+    "hipq_linear_gelu_quantize_packed_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp, _vp],
+    "hipq_linear_residual_layer_norm_quantize_packed_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp,
+                                                           _vp, _f32, _i32, _vp, _vp],
     "hipq_transformer_stack_forward_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
+    "hipq_transformer_stack_forward_prepared_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
     "hipq_qadd_u8": [_vp, _vp, _i32, _f32, _i32, _vp, _i32, _f32, _i32, _sz, _i32, _i32, _vp, _vp],
     "hipq_qrelu_u8": [_vp, _vp, _i32, _f32, _i32, _sz, _i32, _i32, _vp, _vp],
     "hipq_quantization_metrics_f32": [_vp, _vp, _vp, _sz, C.c_uint32, C.c_uint32, _vp],
@@ -157,6 +162,7 @@ _SPECIAL = {
     "hipq_has_error": (_i32, []),
     "hipq_ctx_stream": (_vp, [_vp]),
     "hipq_transformer_stack_workspace_bytes": (_sz, [_sz, _sz, _sz]),
+    "hipq_transformer_stack_prepared_workspace_bytes": (_sz, [_sz, _sz, _sz]),
     "hipq_packed_size": (_i32, [_sz, _sz, C.POINTER(C.c_size_t)]),
     "hipq_conv2d_packed_weights_size": (_i32, [_sz, _sz, _sz, _sz, C.POINTER(C.c_size_t)]),
 }
@@ -611,6 +617,37 @@ class Context:
                   m, n, k, mode, _ptr(out))
         return out
 
+    # ---- a panel of whole rows per workgroup: the Linear and the row operation after it ----
+    def linear_rows_packed_i8_f32(self, a_packed, a_scale, w_packed, w_scales, bias, m, n, k, out=None):
+        out = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_rows_packed_i8_f32", _ptr(a_packed), _ptr(a_scale), int(a_scale.numel() > 1),
+                  _ptr(w_packed), _ptr(w_scales), _ptr(bias), m, n, k, _ptr(out))
+        return out
+
+    def linear_gelu_quantize_packed(self, a_packed, a_scale, w_packed, w_scales, bias, m, n, k, mode=0, out=None,
+                                    scales=None):
+        """-> (packed int8 [m, n] of GELU(linear), row scales [m])"""
+        out = out if out is not None else torch.empty(self.packed_size(m, n), dtype=torch.int8, device=self._dev())
+        scales = scales if scales is not None else torch.empty(m, dtype=torch.float32, device=self._dev())
+        self.call("hipq_linear_gelu_quantize_packed_i8", _ptr(a_packed), _ptr(a_scale), int(a_scale.numel() > 1),
+                  _ptr(w_packed), _ptr(w_scales), _ptr(bias), m, n, k, mode, _ptr(out), _ptr(scales))
+        return out, scales
+
+    def linear_residual_layer_norm_quantize_packed(self, a_packed, a_scale, w_packed, w_scales, bias, m, n, k, x,
+                                                   gamma=None, beta=None, eps=1e-5, mode=0, normalize=True, out=None,
+                                                   scales=None):
+        """x += linear (in place); with `normalize` -> (packed int8 [m, n] of LayerNorm(x), row scales [m])"""
+        if normalize:
+            out = out if out is not None else torch.empty(self.packed_size(m, n), dtype=torch.int8,
+                                                          device=self._dev())
+            scales = scales if scales is not None else torch.empty(m, dtype=torch.float32, device=self._dev())
+        else:
+            out = scales = None
+        self.call("hipq_linear_residual_layer_norm_quantize_packed_i8", _ptr(a_packed), _ptr(a_scale),
+                  int(a_scale.numel() > 1), _ptr(w_packed), _ptr(w_scales), _ptr(bias), m, n, k, _ptr(x), _ptr(gamma),
+                  _ptr(beta), float(eps), mode, _ptr(out), _ptr(scales))
+        return out, scales
+
     def linear_dynamic_noalloc(self, x, w, w_scales, bias=None, per_token=False, mode=0, out=None):
         """hipq_linear_dynamic_f32_noalloc: the same forward on the library's static device scratch.  `out`
         should be given by callers that must not allocate; it is created here only as a convenience."""
@@ -757,14 +794,24 @@ class Context:
         nbytes = self._lib.hipq_transformer_stack_workspace_bytes(tokens, d_model, d_ff)
         return torch.empty(nbytes, dtype=torch.uint8, device=self._dev())
 
-    def stack_forward(self, blocks, x, d_ff, workspace, eps=1e-5, mode=0):
-        """blocks: list of dicts of device tensors keyed like BlockWeights; x [tokens, d_model] is updated in place."""
+    def stack_prepare(self, blocks):
+        """The blocks with every int8 weight matrix in packed order (done once per model)."""
+        return [{k: (self.pack_rows(v) if k.startswith("w_") else v) for k, v in blk.items()} for blk in blocks]
+
+    def stack_workspace_prepared(self, tokens, d_model, d_ff):
+        nbytes = self._lib.hipq_transformer_stack_prepared_workspace_bytes(tokens, d_model, d_ff)
+        return torch.empty(nbytes, dtype=torch.uint8, device=self._dev())
+
+    def stack_forward(self, blocks, x, d_ff, workspace, eps=1e-5, mode=0, prepared=False):
+        """blocks: list of dicts of device tensors keyed like BlockWeights; x [tokens, d_model] is updated in place.
+        prepared: the blocks come from stack_prepare and the workspace from stack_workspace_prepared."""
         arr = (BlockWeights * len(blocks))()
         for rec, blk in zip(arr, blocks):
             for name, _ in BlockWeights._fields_:
                 t = blk.get(name)
                 setattr(rec, name, None if t is None else t.data_ptr())
         tokens, d_model = x.shape
-        self.call("hipq_transformer_stack_forward_f32", C.cast(arr, C.c_void_p), len(blocks), tokens, d_model, d_ff,
-                  float(eps), mode, _ptr(x), _ptr(workspace), workspace.numel())
+        self.call("hipq_transformer_stack_forward_prepared_f32" if prepared else "hipq_transformer_stack_forward_f32",
+                  C.cast(arr, C.c_void_p), len(blocks), tokens, d_model, d_ff, float(eps), mode, _ptr(x),
+                  _ptr(workspace), workspace.numel())
         return x
