@@ -516,7 +516,8 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
         for i in range(reps):
             ctx.quantize_ternary_adaptive(xs[i % 8])
     elif which == "stack":
-        # configs[4]: three forwards of the 12-layer int8 projection stack (8192 tokens, d 768, d_ff 3072)
+        # configs[4]: three forwards of the 12-layer int8 projection stack (8192 tokens, d 768, d_ff 3072) on
+        # prepared weights
         tokens, d, dff, layers = 8192, 768, 3072, 12
         blocks = []
         for _ in range(layers):
@@ -532,11 +533,12 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
             blocks.append(blk)
         x0 = torch.randn(tokens, d, generator=g, device="cuda")
         x = x0.clone()
-        ws = ctx.stack_workspace(tokens, d, dff)
+        prepared = ctx.stack_prepare(blocks)  # weights in packed order: once per model
+        ws = ctx.stack_workspace_prepared(tokens, d, dff)
         torch.cuda.synchronize()
         for _ in range(3):
             x.copy_(x0)
-            ctx.stack_forward(blocks, x, dff, ws)
+            ctx.stack_forward(prepared, x, dff, ws, prepared=True)
     else:
         n = 4096 * 4096
         xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
@@ -1015,17 +1017,25 @@ def main() -> int:
         x0 = torch.randn(tokens, d, generator=g, device="cuda")
         xs5 = x0.clone()
         ws = ctx.stack_workspace(tokens, d, dff)
+        prepared = ctx.stack_prepare(blocks)  # weights in packed order: once per model
+        wsp = ctx.stack_workspace_prepared(tokens, d, dff)
 
         def run_stack():
+            xs5.copy_(x0)
+            ctx.stack_forward(prepared, xs5, dff, wsp, prepared=True)
+
+        def run_stack_row_major():
             xs5.copy_(x0)
             ctx.stack_forward(blocks, xs5, dff, ws)
 
         ms = event_time_ms(run_stack, reps=5, warmup=2)
+        ms_rm = event_time_ms(run_stack_row_major, reps=5, warmup=2)
         stack_ops = 2.0 * tokens * d * (3 * d + d + dff + dff) * layers
         extra["stack_12x768x3072_8192tok"] = {"ms": ms, "tokens/s": tokens / (ms * 1e-3),
                                               "TOP/s": stack_ops / (ms * 1e-3) / 1e12,
                                               "frac_mfma_peak": stack_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
-                                              "ops": stack_ops}
+                                              "ops": stack_ops, "weights": "prepared (packed order)",
+                                              "ms_row_major_weights": ms_rm}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(M, N, K)
         result["speedup_vs_cpu_baseline"] = value / result["cpu_baseline"]["value"]
