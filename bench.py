@@ -183,7 +183,14 @@ def conv_phase_table(ctx, g) -> int:
         ctx.conv2d_i8_packed(xc[cnt[0] % 8], 0, 0.02, packed, sums, (3, 3), swc, bc, 0.05, 0, (1, 1), out=oc)
 
     waves = 2 * 128 * 4  # 256 filters / 128 x 8192 padded windows / 64 tiles, four waves each
-    return phase_table("conv2d implicit GEMM M=256 N=8192 K=2304", ctx, forward, waves)
+    rc = phase_table("conv2d implicit GEMM M=256 N=8192 K=2304", ctx, forward, waves)
+    print(f"launch to launch without the stamps (HIP events, layout pass + GEMM): {event_time_ms(forward, reps=400, warmup=20) * 1e3:.2f} us")
+    print("measured alternative (test hook 14): one launch, the workgroups gather their own patches of the image")
+    ctx.set_gemm_kernel_variant(14)
+    rc |= phase_table("conv2d patch kernel M=256 N=8192 K=2304", ctx, forward, waves, names=PHASES_PATCH)
+    print(f"launch to launch without the stamps (HIP events): {event_time_ms(forward, reps=400, warmup=20) * 1e3:.2f} us")
+    ctx.set_gemm_kernel_variant(0)
+    return rc
 
 
 def gemm_phase_table(ctx, M: int, N: int, K: int, g, pairs: bool = False) -> int:
@@ -228,6 +235,9 @@ def gemm_phase_table(ctx, M: int, N: int, K: int, g, pairs: bool = False) -> int
 PHASES_TILE = ["start -> first operands in registers", "K loop (first operands -> last MFMA retired)",
                "4-way K-split sum through LDS (incl. waiting for the slowest wave)", "convert + issue stores",
                "stores retired", "whole wave"]
+PHASES_PATCH = ["start -> raw rows of the patch in LDS (dword loads, barrier)",
+                "raw rows -> patch in fragment order (LDS byte reads, barrier)",
+                "K loop (patch built -> last MFMA retired)", "convert + issue stores", "stores retired", "whole wave"]
 PHASES_PAIR = ["start -> first operands in registers", "K loop (first operands -> last MFMA retired)",
                "4-way K-split sum through LDS in two rounds; partials for the partner stored",
                "partner's flag seen, its partials read (past the L1) and added", "convert + stores issued and retired",

@@ -26,7 +26,10 @@ extern "C" {
  * one-launch activation quantizers of the dynamic Linear and Conv2d forwards while their grids wait
  * for the range (11); 12 runs shapes of whole 128 x 128 tiles that fill the device once as one tile
  * per PAIR of compute units, K halved between the two, partial sums exchanged through their XCD's L2
- * (measured slower than the default forms; kept as a measured alternative). */
+ * (measured slower than the default forms; kept as a measured alternative); 14 runs a Conv2d
+ * forward on a uint8 input of 128 or 256 channels and small planes as ONE launch whose workgroups
+ * gather their own patches of the image into LDS (measured no faster than the layout pass + implicit
+ * GEMM it would replace; kept as a measured alternative). */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
 /* Some kernels couple their waves through device memory: the persistent GEMM kernel (counters
  * between producer and consumer waves), the one-launch dynamic quantizers (their workgroups meet to

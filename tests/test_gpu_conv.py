@@ -143,6 +143,50 @@ def test_config4_full_size_packed_requant_forward(ctx, hipq):
             assert torch.equal(ctx.conv2d_i8(x, zp_in, s_in, wq, sw, bias, s_out, zp_out, (1, 1), (1, 1), mode), want)
 
 
+PATCH_GEOMS = [
+    # nb, c, h, w, oc, k, pad, zp: 128 or 256 channels, planes of a multiple of 4 bytes, raw rows within 128 bytes
+    (3, 128, 14, 14, 40, 3, 1, 77),    # three images: patches that run from one image into the next
+    (2, 256, 14, 14, 256, 3, 1, 0),
+    (1, 256, 14, 14, 130, 3, 0, 128),  # no padding; a last filter block of two
+    (5, 128, 8, 8, 64, 3, 1, 255),     # small planes: most patches span two images
+    (2, 256, 10, 10, 33, 1, 0, 9),     # 1 x 1
+    (2, 128, 12, 12, 70, 5, 2, 60),    # 25 taps
+    (1, 128, 16, 12, 32, 2, 1, 3),     # even kernel, taps x channel blocks not a multiple of the loop's trip
+]
+
+
+@pytest.mark.parametrize("nb,c,h,w,oc,k,pad,zp", PATCH_GEOMS)
+def test_conv_one_launch_patch_form(ctx, hipq, oracle, nb, c, h, w, oc, k, pad, zp):
+    """The measured alternative behind test hook 14 (the workgroups gather their own patches of the image; no
+    layout pass): int32 accumulators against the oracle, and the int8 / fp32 forwards bit for bit against the
+    default two-launch form."""
+    rng = np.random.default_rng(nb + c + h * 5 + oc + k)
+    x = rng.integers(0, 256, size=(nb, c, h, w), dtype=np.uint8)
+    wq = rng.integers(-128, 128, size=(oc, c, k, k), dtype=np.int8)
+    sw = rng.uniform(1e-4, 1e-3, oc).astype(np.float32)
+    bias = (rng.standard_normal(oc) * 0.01).astype(np.float32)
+    want = oracle.backend_conv2d_i32(x, zp, wq, (1, 1), (pad, pad))
+    xd, wd, swd, bd = dev(x), dev(wq), dev(sw), dev(bias)
+    packed, sums = ctx.conv2d_pack_weights(wd)
+    outs = {}
+    try:
+        for variant in (0, 14):
+            ctx.set_gemm_kernel_variant(variant)
+            outs[variant] = (
+                host(ctx.conv2d_i32(xd, zp, wd, (1, 1), (pad, pad))),
+                host(ctx.conv2d_i8_packed(xd, zp, 0.02, packed, sums, (k, k), swd, bd, 0.3, -4, (pad, pad))),
+                host(ctx.conv2d_i8_packed(xd, zp, 0.02, packed, sums, (k, k), swd, bd, 0.3, -4, (pad, pad),
+                                          hipq.ROUND_HALF_EVEN)),
+                host(ctx.conv2d_f32(xd, zp, 0.02, wd, swd, bd, (1, 1), (pad, pad))),
+            )
+    finally:
+        ctx.set_gemm_kernel_variant(0)
+    np.testing.assert_array_equal(outs[14][0], want)
+    for a, b in zip(outs[14], outs[0]):
+        np.testing.assert_array_equal(a.view(np.uint8) if a.dtype == np.int8 else a.view(np.int32),
+                                      b.view(np.uint8) if b.dtype == np.int8 else b.view(np.int32))
+
+
 def test_conv_error_cases(ctx, hipq):
     x = torch.zeros((1, 4, 5, 5), dtype=torch.uint8, device="cuda")
     w = torch.zeros((2, 3, 3, 3), dtype=torch.int8, device="cuda")

@@ -59,6 +59,11 @@ size_t packed_operand_bytes(size_t rows, size_t k);
 // [channel block][pixel][32] order, N = padded pixels; ep carries the cv_* geometry.  epi: EPI_I32 / _F32 / _I8.
 int32_t conv_gemm_packed(hipq_ctx *ctx, const int8_t *filters, const int8_t *image, int M, int N, int K,
                          const GemmEpilogue &ep, int epi, bool even);
+// The same convolution in one launch, from the u8 NCHW input itself (hipq_conv_patch.h): `fits` says whether
+// that form takes the geometry (c channels, padded width wp, kh x kw taps).
+bool conv_patch_applicable(int nb, int c, int h, int w, int hp, int wp, int kh, int kw);
+int32_t conv_gemm_patch(hipq_ctx *ctx, const int8_t *filters, const uint8_t *x, size_t x_bytes, int zp_in, int h, int w,
+                        int ph, int pw, int kh, int M, int N, int K, const GemmEpilogue &ep, int epi, bool even);
 
 // Host-side twin of recip_for_div: the correctly rounded 1/b if it is a normal number, else 0.
 static inline float host_recip_for_div(float b) {

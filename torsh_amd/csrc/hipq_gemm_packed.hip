@@ -5,6 +5,7 @@
 // pass itself, so the forward costs no extra pass over either operand.
 #include "hipq_gemm_packed.h"
 #include "hipq_gemm_rows.h"
+#include "hipq_conv_patch.h"
 
 namespace hipq {
 
@@ -94,6 +95,34 @@ int32_t conv_gemm_packed(hipq_ctx *ctx, const int8_t *filters, const int8_t *ima
     if (epi == EPI_F32) return launch_conv_packed<EPI_F32, false>(ctx, filters, image, M, N, K, ep);
     if (even) return launch_conv_packed<EPI_I8, true>(ctx, filters, image, M, N, K, ep);
     return launch_conv_packed<EPI_I8, false>(ctx, filters, image, M, N, K, ep);
+}
+
+bool conv_patch_applicable(int nb, int c, int h, int w, int hp, int wp, int kh, int kw) {
+    int patch = 0, lds_bytes = 0;
+    return conv_patch_fits(c, h, w, hp, wp, kh, kw, static_cast<long long>(nb) * hp * wp, &patch, &lds_bytes);
+}
+
+template <int CBS>
+static int32_t conv_patch_dispatch(hipq_ctx *ctx, const int8_t *filters, int M, int N, int K, const GemmEpilogue &ep,
+                                   const ConvPatch &cp, int lds_bytes, int epi, bool even) {
+    if (epi == EPI_I32) return launch_conv_patch<CBS, EPI_I32, false>(ctx, filters, M, N, K, ep, cp, lds_bytes);
+    if (epi == EPI_F32) return launch_conv_patch<CBS, EPI_F32, false>(ctx, filters, M, N, K, ep, cp, lds_bytes);
+    if (even) return launch_conv_patch<CBS, EPI_I8, true>(ctx, filters, M, N, K, ep, cp, lds_bytes);
+    if (ctx->trace) return launch_conv_patch<CBS, EPI_I8, false, true>(ctx, filters, M, N, K, ep, cp, lds_bytes);
+    return launch_conv_patch<CBS, EPI_I8, false>(ctx, filters, M, N, K, ep, cp, lds_bytes);
+}
+
+int32_t conv_gemm_patch(hipq_ctx *ctx, const int8_t *filters, const uint8_t *x, size_t x_bytes, int zp_in, int h, int w,
+                        int ph, int pw, int kh, int M, int N, int K, const GemmEpilogue &ep, int epi, bool even) {
+    int patch = 0, lds_bytes = 0;
+    if (!conv_patch_fits(ep.cv_c, h, w, ep.cv_hp, ep.cv_wp, kh, ep.cv_kw, N, &patch, &lds_bytes) ||
+        x_bytes >= (size_t(1) << 31) || (reinterpret_cast<uintptr_t>(x) & 3u))
+        return fail(HIPQ_SHAPE_ERROR, "conv2d (patch): geometry not taken by this form");
+    const uint32_t b = static_cast<uint32_t>(zp_in ^ 0x80) & 0xffu;
+    const ConvPatch cp{x, h, w, ph, pw, kh, patch, b * 0x01010101u, static_cast<int>(x_bytes),
+                       1.0f / static_cast<float>(ep.cv_hp * ep.cv_wp), 1.0f / static_cast<float>(ep.cv_wp)};
+    if (ep.cv_c == 128) return conv_patch_dispatch<4>(ctx, filters, M, N, K, ep, cp, lds_bytes, epi, even);
+    return conv_patch_dispatch<8>(ctx, filters, M, N, K, ep, cp, lds_bytes, epi, even);
 }
 
 }  // namespace hipq
