@@ -715,3 +715,29 @@ def test_torsh_nn_flavour(ctx, hipq, oracle):
     np.testing.assert_array_equal(host(s), want_s)
     np.testing.assert_array_equal(host(z), want_z)
     np.testing.assert_array_equal(host(q).view(np.uint8).astype(np.float32), want_carrier)
+    # a NaN weight becomes the code clamp(zero point) (`NaN as i32` is 0, then the zero point is added), in every
+    # kernel form the entry point has: a channel per row, channels that are not the leading dimension (one workgroup
+    # per channel), and the same spread over many workgroups
+    w3 = (rng.standard_normal((7, 130)) * 0.5 + 0.3).astype(np.float32)
+    w3[1, 5] = np.nan
+    w3[4, 0] = np.nan
+    w3[3] = 1.5   # constant channels: scale 0 (no guard), a zero point at the end of the i32 range
+    w3[5] = -0.25
+    want_carrier, want_s, want_z = oracle.nn_per_channel_quantize_weights_asym_u8(w3)
+    q, s, z, st = ctx.quantize_per_group_auto(dev(w3), 1, 7, 130, 1, hipq.PARAMS_NN_ASYMMETRIC, 0, 255, hipq.FORM_DIV)
+    np.testing.assert_array_equal(host(s), want_s)
+    np.testing.assert_array_equal(host(z), want_z)
+    np.testing.assert_array_equal(host(q).view(np.uint8).astype(np.float32), want_carrier)
+    assert host(q).view(np.uint8)[1, 5] == np.clip(want_z[1], 0, 255) and host(q).view(np.uint8)[4, 0] == np.clip(want_z[4], 0, 255)
+    for outer, inner in ((5, 26), (160, 832)):  # [outer, 7, inner]: 130 and 133120 values per channel
+        wc = (rng.standard_normal((7, outer * inner)) * 0.5 + 0.3).astype(np.float32)
+        wc[1, 5] = np.nan
+        wc[6, outer * inner - 1] = np.nan
+        want_carrier, want_s, want_z = oracle.nn_per_channel_quantize_weights_asym_u8(wc)
+        x3 = np.ascontiguousarray(wc.reshape(7, outer, inner).transpose(1, 0, 2))
+        q, s, z, st = ctx.quantize_per_group_auto(dev(x3), outer, 7, inner, 1, hipq.PARAMS_NN_ASYMMETRIC, 0, 255,
+                                                  hipq.FORM_DIV)
+        np.testing.assert_array_equal(host(s), want_s)
+        np.testing.assert_array_equal(host(z), want_z)
+        got = host(q).view(np.uint8).transpose(1, 0, 2).reshape(7, outer * inner).astype(np.float32)
+        np.testing.assert_array_equal(got, want_carrier)

@@ -755,7 +755,7 @@ __global__ __launch_bounds__(kBlock) void quantize_per_row_kernel(const float *_
     // torsh-nn's per-channel weights pass each value through `as i32` before the zero point is added
     const bool int_cast = flavor >= HIPQ_PARAMS_NN_SYMMETRIC;
     auto quant1 = [&](float v) {
-        return int_cast ? quantize_int<QFORM_DIV_INT_CAST, EVEN>(v, scale, inv, zpf, qmin, qmax)
+        return int_cast ? quantize_int_cast<EVEN>(v, scale, inv, zp, qmin, qmax)
                         : quantize_int<QFORM_DIV, EVEN>(v, scale, inv, zpf, qmin, qmax);
     };
     auto quant4 = [&](float4 t) { return pack4(quant1(t.x), quant1(t.y), quant1(t.z), quant1(t.w)); };
@@ -818,7 +818,10 @@ __global__ __launch_bounds__(kBlock) void quantize_per_channel_auto_kernel(
     for (size_t i = threadIdx.x; i < per; i += kBlock) {
         const size_t o = i / run, r = i % run;
         const size_t idx = (o * channels + c0) * inner + r;
-        out[idx] = static_cast<int8_t>(to_int_nan0(quantize_value<true, EVEN>(x[idx], scale, inv, zpf, lo, hi)));
+        // (torsh-nn's flavours: `as i32` before the zero point is added, as in the row kernel)
+        out[idx] = static_cast<int8_t>(flavor >= HIPQ_PARAMS_NN_SYMMETRIC
+                                           ? quantize_int_cast<EVEN>(x[idx], scale, inv, zp, qmin, qmax)
+                                           : to_int_nan0(quantize_value<true, EVEN>(x[idx], scale, inv, zpf, lo, hi)));
     }
 }
 
@@ -987,7 +990,13 @@ __global__ __launch_bounds__(kBlock) void channel_quantize_kernel(const float *_
     if (st != HIPQ_SUCCESS) return;
     const float inv = recip_for_div(scale), zpf = static_cast<float>(zp);
     const float lo = static_cast<float>(qmin), hi = static_cast<float>(qmax);
-    auto one = [&](float v) { return to_int_nan0(quantize_value<true, EVEN>(v, scale, inv, zpf, lo, hi)); };
+    // torsh-nn's per-channel weights pass each value through `as i32` before the zero point is added
+    // (crates/torsh-nn/src/quantization/ops.rs:153-162): a NaN becomes the code clamp(zero point).
+    const bool int_cast = flavor >= HIPQ_PARAMS_NN_SYMMETRIC;
+    auto one = [&](float v) {
+        return int_cast ? quantize_int_cast<EVEN>(v, scale, inv, zp, qmin, qmax)
+                        : to_int_nan0(quantize_value<true, EVEN>(v, scale, inv, zpf, lo, hi));
+    };
     using Vec = typename std::conditional<V == 4, float4, float>::type;
     auto load = [&](size_t row) {
         const Vec *p = reinterpret_cast<const Vec *>(x + row * cc.period + w.unit * V);

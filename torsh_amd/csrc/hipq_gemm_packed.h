@@ -685,6 +685,14 @@ __global__ __launch_bounds__(256) void skinny_i8_packed_kernel(const int8_t *__r
 // store_tile does it.  Every workgroup repeats the quantize arithmetic of all rows (16 values a thread and row at
 // K = 4096), which is why this pays for one or two rows only: N = 11008, K = 4096 from fp32, one launch against
 // the quantizer and the product: M = 1 11.7 / 14.7 us, M = 2 13.3 / 14.7, M = 3 15.4 / 14.8, M = 4 17.3 / 15.0.
+// For more rows a hand-over inside one launch was built and measured (workgroup r quantizes row r into the packed
+// scratch, fences at device scope and raises a flag word; every workgroup requests its first weight fragments,
+// waits for the M flags, passes a device-scope acquire, then runs the product; an arrival counter lets the last
+// workgroup clear the flags for the next launch).  Bit-identical, and slower: M = 4 27.6 us, M = 16 34.9 us against
+// 13.9 / 14.9 us for the two launches (same shape); of that the acquire (an L2 invalidate per workgroup) costs
+// 8.5 us, the arrival atomics on one word 4.4 us, the producers' fence 1.2 us - and with all three taken out
+// (13.5 us, no longer correct) it only equals the two launches, because the chain "read the row, reduce, quantize,
+// write through, flag seen by the other dies" is as long as the quantizer's launch and ramp.  Not kept.
 template <int D, bool EVEN, int MROWS, int CH, bool STATIC = false>
 __global__ __launch_bounds__(256) void gemv_i8_packed_from_f32_kernel(const float *__restrict__ x,
                                                                       const int8_t *__restrict__ PW, int M, int N, int K,

@@ -146,6 +146,15 @@ __device__ __forceinline__ int quantize_int(float x, float scale, float inv, flo
     return min(max(q, lo), hi);
 }
 
+// FORM 3 with the zero point as the integer it is: (round(x / scale) as i32) + zp, the sum taken in 64 bits (the
+// reference's i32 sum never wraps where it does not panic), then the clamp.  A constant channel of torsh-nn's
+// per-channel weights has scale 0 and a zero point at an end of the i32 range, which a float cannot carry.
+template <int RND>
+__device__ __forceinline__ int quantize_int_cast(float x, float scale, float inv, int zp, int lo, int hi) {
+    const long long q = static_cast<long long>(cvt_i32_sat(round_mode<RND>(div_rn(x, scale, inv)))) + zp;
+    return static_cast<int>(q < lo ? lo : (q > hi ? hi : q));
+}
+
 // quantize_int for a symmetric per-row quantizer (zero point 0, int8 range) whose scale was derived
 // from the row's own finite maximum, scale = max|x| / 127: then |x * y| stays near 127, the
 // remainder of div_rn is never NaN for a finite x, and the select that guards it can go; a NaN
