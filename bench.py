@@ -525,9 +525,9 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
             ctx.quantize_binary_learned_threshold(xs[i % 8])
         for i in range(reps):
             ctx.quantize_ternary_adaptive(xs[i % 8])
-    elif which == "stack":
+    elif which in ("stack", "stack_row_major"):
         # configs[4]: three forwards of the 12-layer int8 projection stack (8192 tokens, d 768, d_ff 3072) on
-        # prepared weights
+        # prepared weights ("stack") or on row-major weights (eight kernels per layer)
         tokens, d, dff, layers = 8192, 768, 3072, 12
         blocks = []
         for _ in range(layers):
@@ -543,12 +543,18 @@ def profile_target(ctx, which: str, M: int, N: int, K: int) -> int:
             blocks.append(blk)
         x0 = torch.randn(tokens, d, generator=g, device="cuda")
         x = x0.clone()
-        prepared = ctx.stack_prepare(blocks)  # weights in packed order: once per model
-        ws = ctx.stack_workspace_prepared(tokens, d, dff)
+        if which == "stack":
+            prepared = ctx.stack_prepare(blocks)  # weights in packed order: once per model
+            ws = ctx.stack_workspace_prepared(tokens, d, dff)
+        else:
+            ws = ctx.stack_workspace(tokens, d, dff)
         torch.cuda.synchronize()
         for _ in range(3):
             x.copy_(x0)
-            ctx.stack_forward(prepared, x, dff, ws, prepared=True)
+            if which == "stack":
+                ctx.stack_forward(prepared, x, dff, ws, prepared=True)
+            else:
+                ctx.stack_forward(blocks, x, dff, ws)
     else:
         n = 4096 * 4096
         xs = [torch.randn(n, generator=g, device="cuda") for _ in range(8)]
@@ -571,7 +577,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--profile", choices=["gemm", "gemm_phases", "gemm_pair_phases", "vmem_path", "quantize_sweep", "conv_phases", "gemm_rowmajor", "step", "quantize", "per_channel", "calib", "special", "copy",
-                                          "stack", "gemv", "conv"], default=None,
+                                          "stack", "stack_row_major", "gemv", "conv"], default=None,
                     help="run only a few launches of one kernel (for rocprofv3 counter passes) and exit")
     args = ap.parse_args()
     SPINUP_MS = args.spinup_ms
