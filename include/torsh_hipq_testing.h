@@ -29,11 +29,14 @@ extern "C" {
  * (measured slower than the default forms; kept as a measured alternative); 14 runs a Conv2d
  * forward on a uint8 input of 128 or 256 channels and small planes as ONE launch whose workgroups
  * gather their own patches of the image into LDS (measured no faster than the layout pass + implicit
- * GEMM it would replace; kept as a measured alternative). */
+ * GEMM it would replace; kept as a measured alternative); 15 makes the row-panel forwards (the
+ * Linear forwards with a row operation in their epilogue) keep one workgroup per 32 rows where they
+ * would let two workgroups of an XCD share 64 rows and half of the columns each. */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
 /* Some kernels couple their waves through device memory: the persistent GEMM kernel (counters
  * between producer and consumer waves), the one-launch dynamic quantizers (their workgroups meet to
- * agree on the range) and the GEMM form whose workgroup pairs exchange partial sums.  All bound
+ * agree on the range), the GEMM form whose workgroup pairs exchange partial sums and the row-panel
+ * forwards whose workgroup pairs exchange row maxima and sums.  All bound
  * every wait, so that a grid always drains; a wait that gives up marks the context, and the next
  * hipq_ctx_synchronize returns HIPQ_DEVICE_ERROR once instead of handing back a wrong result
  * silently (the quantizers also leave zero codes, a NaN scale and status HIPQ_DEVICE_ERROR in

@@ -78,11 +78,11 @@ def test_linear_gelu_quantize_equals_its_parts(ctx, hipq, m, n, k, mode):
     np.testing.assert_array_equal(host(got_q), pack_reference(host(q)))  # (padding rows and k blocks: zeros)
 
 
-def test_linear_gelu_quantize_rows_that_are_not_finite(ctx):
+@pytest.mark.parametrize("m,n,k", [(40, 256, 64), (72, 1536, 64)])
+def test_linear_gelu_quantize_rows_that_are_not_finite(ctx, m, n, k):
     """A row whose GELU output holds an infinity gets a NaN scale and zero codes, a NaN element is code 0 and does
-    not enter the row's maximum: as the row kernel has it."""
+    not enter the row's maximum: as the row kernel has it (in a panel of one workgroup and in one of a pair)."""
     rng = np.random.default_rng(5)
-    m, n, k = 40, 256, 64
     a, w, sa, sw, b = operands(rng, m, n, k)
     b[3] = np.inf
     sa[7] = np.nan  # a whole row of NaN
@@ -102,7 +102,8 @@ def test_linear_gelu_quantize_rows_that_are_not_finite(ctx):
     np.testing.assert_array_equal(host(got_q), pack_reference(host(q)))
 
 
-LN_SHAPES = [(1, 128, 32), (100, 256, 96), (257, 768, 800), (65, 768, 3072), (40, 1536, 160), (48, 3072, 64)]
+LN_SHAPES = [(1, 128, 32), (100, 256, 96), (257, 768, 800), (65, 768, 3072), (40, 1536, 160), (48, 3072, 64),
+             (97, 3072, 768), (70, 1536, 1600)]  # (the last two: panels of 64 rows shared by two compute units)
 
 
 @pytest.mark.parametrize("m,n,k", LN_SHAPES)
@@ -160,6 +161,92 @@ def test_row_panel_shapes_that_are_refused(ctx, hipq):
     assert e.value.code == hipq.SHAPE_ERROR
     # nothing to do
     ctx.linear_rows_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), 0, 96, 32, out=torch.empty((0, 96), device="cuda"))
+
+
+# ---- panels of 64 rows shared by a pair of compute units ------------------------------------------------------
+
+PAIR_SHAPES = [(8192, 3072, 768), (97, 3072, 768), (70, 1536, 1600), (40, 2048, 1056), (200, 2304, 1024), (33, 1664, 96)]
+
+
+@pytest.mark.parametrize("m,n,k", PAIR_SHAPES)
+def test_pair_panels_equal_single_panels(hipq, m, n, k):
+    """The row-panel kernels in their pair form (two workgroups of one XCD share 64 rows and take half of the columns
+    each; row maxima and sums cross through the XCD's L2) against the single-workgroup panels (test hook 15): the fp32
+    product, the skip connection, GELU + per-token int8 bit for bit, the LayerNorm form within the bound that holds
+    between any two orders of its sums.  Twice in a row: the exchange flags must be back at zero."""
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(m + n + k)
+        a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+        w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+        sa = torch.rand(m, generator=g, device="cuda") * 0.02 + 0.001
+        sw = torch.rand(n, generator=g, device="cuda") * 2e-3 + 1e-4
+        b = torch.randn(n, generator=g, device="cuda")
+        gamma = torch.rand(n, generator=g, device="cuda") + 0.5
+        beta = torch.randn(n, generator=g, device="cuda") * 0.1
+        x0 = torch.randn(m, n, generator=g, device="cuda")
+        pa, pw = c.pack_rows(a), c.pack_rows(w)
+
+        def forms():
+            f = c.linear_rows_packed_i8_f32(pa, sa, pw, sw, b, m, n, k)
+            gq, gs = c.linear_gelu_quantize_packed(pa, sa, pw, sw, b, m, n, k)
+            x_ln, x_res = x0.clone(), x0.clone()
+            lq, ls = c.linear_residual_layer_norm_quantize_packed(pa, sa, pw, sw, b, m, n, k, x_ln, gamma, beta)
+            c.linear_residual_layer_norm_quantize_packed(pa, sa, pw, sw, b, m, n, k, x_res, normalize=False)
+            c.synchronize()  # (would report an exchange that gave up)
+            return f, gq, gs, x_ln, lq, ls, x_res
+
+        c.set_gemm_kernel_variant(15)
+        single = forms()
+        c.set_gemm_kernel_variant(0)
+        for _ in range(2):
+            pair = forms()
+            for i in (0, 1, 2, 3, 6):
+                assert torch.equal(pair[i].view(torch.int32) if pair[i].dtype == torch.float32 else pair[i],
+                                   single[i].view(torch.int32) if single[i].dtype == torch.float32 else single[i]), i
+            np.testing.assert_allclose(host(pair[5]), host(single[5]), rtol=1e-6, atol=0)
+            diff = (pair[4].to(torch.int16) - single[4].to(torch.int16)).abs()
+            assert int(diff.max()) <= 1
+            assert float((diff != 0).float().mean()) <= 1e-5 + 2.0 / diff.numel()
+    finally:
+        c.close()
+
+
+def test_pair_panels_give_up_cleanly(hipq):
+    """With the spin limit forced to 0 a workgroup looks for its partner's row maxima exactly once, which is too early
+    for some of the 128 pairs: the kernel must drain all the same, the context reports HIPQ_DEVICE_ERROR at the next
+    synchronize, once, and the same call is right again afterwards (flags that a given-up exchange left set have
+    been cleared).  The single-workgroup panels wait for nothing."""
+    m, n, k = 8192, 3072, 768
+    c = hipq.Context(0)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(2)
+        a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+        w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+        sa = torch.rand(m, generator=g, device="cuda") * 0.02 + 0.001
+        sw = torch.rand(n, generator=g, device="cuda") * 2e-3 + 1e-4
+        b = torch.randn(n, generator=g, device="cuda")
+        pa, pw = c.pack_rows(a), c.pack_rows(w)
+        want_q, want_s = c.linear_gelu_quantize_packed(pa, sa, pw, sw, b, m, n, k)
+        c.synchronize()
+        c.set_wait_spin_limit(0)
+        c.linear_gelu_quantize_packed(pa, sa, pw, sw, b, m, n, k)
+        with pytest.raises(hipq.HipqError) as e:
+            c.synchronize()
+        assert e.value.code == hipq.DEVICE_ERROR and "gave up" in str(e.value)
+        c.synchronize()  # reported once
+        c.set_gemm_kernel_variant(15)
+        q, s_ = c.linear_gelu_quantize_packed(pa, sa, pw, sw, b, m, n, k)
+        c.synchronize()
+        assert torch.equal(q, want_q) and torch.equal(s_, want_s)
+        c.set_gemm_kernel_variant(0)
+        c.set_wait_spin_limit(-1)
+        for _ in range(2):
+            q, s_ = c.linear_gelu_quantize_packed(pa, sa, pw, sw, b, m, n, k)
+            c.synchronize()
+            assert torch.equal(q, want_q) and torch.equal(s_, want_s)
+    finally:
+        c.close()
 
 
 # ---- the projection stack on prepared weights ---------------------------------------------------------------

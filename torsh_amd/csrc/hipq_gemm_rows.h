@@ -401,6 +401,401 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
     }
 }
 
+// ---- the same with a panel of 64 rows shared by a PAIR of compute units ----------------------------------------
+// Every workgroup of gemm_i8_rows_kernel streams the whole weight matrix, which is what bounds its main loop
+// (N * K bytes through a 57 B/clk path).  Here two workgroups on one XCD (ids b and b + 8, see hipq_gemm_pair.h)
+// share 64 rows and take half of the columns each: a weight fragment feeds two MFMAs (one per row block), so the
+// same matrix work needs half the weight stream per compute unit, and loop and MFMA time come level.  What the two
+// halves of a row have to agree on - its maximum, its sum, its sum of squares - crosses through their XCD's L2 in
+// one small exchange per statistic (64 floats each way, plain stores, then a flag word; the reader polls the flag
+// past its L1, reads the partner's partials past its L1 and clears the flag, so every launch finds the flags zero
+// and a captured launch can be replayed; a flag that does not come within the spin limit, or comes from another
+// XCD, marks the context and the kernel runs on with defined values).  Both halves add the partials in the same
+// order (columns' lower half first), so they hold the same bits.
+// Results: the fp32 product, the skip connection, GELU and the per-token maxima are exactly those of the other
+// forms; a LayerNorm's sums are folded in yet another order.
+struct RowPairExchange {
+    uint32_t *flags;  // four words per workgroup (three used: one per statistic)
+    float *buf;       // three inboxes of 64 floats per workgroup
+    uint32_t *wait_error;
+    int spin_limit;
+};
+
+constexpr int kRowsPairStage = kRowsStage / 2;  // k blocks per LDS buffer and row block
+
+template <int NBW, int EPI, bool EVEN>
+__global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPanel p, RowPairExchange px) {
+    constexpr int RB = 2;
+    constexpr int D = NBW == 2 ? 8 : (NBW == 3 ? 12 : 6);  // weight fragments in flight per wave
+    constexpr int U = D / rows_gcd(NBW, D);                // k blocks per trip of the main loop
+    static_assert((U * NBW) % D == 0 && 4 % U == 0, "ring slots must be static; stages are multiples of 4 k blocks");
+    constexpr bool QUANT = EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q;
+    constexpr bool RESID = EPI == RP_RESID_F32 || EPI == RP_RESID_LN_Q;
+    __shared__ __attribute__((aligned(1024))) int8_t apanel[2][kRowsStage * 1024];  // [buffer][row block][k block]
+    __shared__ __attribute__((aligned(16))) float red[3][kRowsWaves][64];           // [statistic][wave][row]
+    __shared__ __attribute__((aligned(16))) float fin[4][64];  // per row: mean, 1 / std, scale, 1 / scale
+    const int tid = threadIdx.x, lane = tid % kWave, half = lane / 32, cin = lane % 32;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int grp = blockIdx.x / 8;
+    const int pair = (grp / 2) * 8 + blockIdx.x % 8, h = grp % 2;
+    const int m0 = pair * 64;
+    if (m0 >= p.M) return;  // (both workgroups of a pair)
+    const int KB = static_cast<int>(packed_k_blocks(p.K));  // (a multiple of 4)
+    const int nblocks = p.N / 32, nb2 = nblocks / 2;
+    const int rbA = (p.M + 31) / 32, rb0 = pair * 2;
+    const int jl0 = wave * NBW;         // this wave's column blocks within the half: jl0 .. jl0 + NBW - 1
+    const int jb0 = h * nb2 + jl0;      // ... and within the matrix
+    auto mine_block = [&](int jj) { return jl0 + jj < nb2; };
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t *>(p.pa) + size_t(rb0) * KB * 1024, 0, (rbA - rb0 < 2 ? 1 : 2) * KB * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(p.pw), 0, nblocks * KB * 1024, 0x00020000);
+    const int voff = lane * 16;
+    const int wstride = KB * 1024;
+    // (a wave without columns asks beyond the matrix: zeros, no memory access)
+    const int wbase = jl0 < nb2 ? jb0 * wstride : 0x7fffffff - 64 * 1024 * 1024;
+    auto load_w = [&](int kb, int jj) {
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, wbase + jj * wstride + kb * 1024, 0));
+    };
+    // one stage of the activation panel: 12 k blocks of both row blocks, three 16-byte pieces per thread
+    int aoff[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const int c = tid + i * kRowsThreads;  // 16-byte piece 0 .. 1535: row block c / 768
+        aoff[i] = (c / 768) * KB * 1024 + (c % 768) * 16;
+    }
+    auto load_stage = [&](int s, v4i(&t)[3]) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+            t[i] = __builtin_bit_cast(
+                v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, aoff[i], s * (kRowsPairStage * 1024), 0));
+    };
+    const int rows_here = p.M - m0 < 64 ? p.M - m0 : 64;
+    const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(
+        p.out_f ? reinterpret_cast<char *>(p.out_f) + size_t(m0) * p.N * 4 : nullptr, 0, p.out_f ? rows_here * p.N * 4 : 0,
+        0x00020000);
+    const int row_bytes = p.N * 4;
+    auto load_x = [&](int rbk, int jj, int r) {
+        return __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(rf, (4 * half * p.N + (jb0 + jj) * 32 + cin) * 4,
+                                                        (32 * rbk + 8 * (r / 4) + (r % 4)) * row_bytes, 0));
+    };
+    // touch this workgroup's thirty-second of the weights (see gemm_i8_rows_kernel)
+    {
+        const int wbytes = nblocks * KB * 1024;
+        const int chunk = ((wbytes + 31) / 32 + 127) & ~127;
+        const int part = (blockIdx.x / 8) % 32;
+        int touched = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int off = (tid + i * kRowsThreads) * 128;
+            if (off < chunk) touched ^= __builtin_amdgcn_raw_buffer_load_b32(rw, off, part * chunk, 0);
+        }
+        if (touched == 0x5a5a5a5a && p.M < 0) red[0][0][0] = 1.0f;  // (keeps the loads alive; never true)
+    }
+    v4i wf[D];
+#pragma unroll
+    for (int u = 0; u < D; ++u) wf[u] = load_w(u / NBW, u % NBW);
+    v4i astage[3];
+    load_stage(0, astage);
+    constexpr bool RES_EARLY = RESID && NBW <= 3;
+    float res_all[RES_EARLY ? RB : 1][RES_EARLY ? NBW : 1][16];
+    if constexpr (RES_EARLY) {
+#pragma unroll
+        for (int rbk = 0; rbk < RB; ++rbk)
+#pragma unroll
+            for (int jj = 0; jj < NBW; ++jj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) res_all[rbk][jj][r] = load_x(rbk, jj, r);
+    }
+
+    v16i acc[RB][NBW];
+#pragma unroll
+    for (int rbk = 0; rbk < RB; ++rbk)
+#pragma unroll
+        for (int j = 0; j < NBW; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rbk][j][r] = 0;
+
+    const int stages = (KB + kRowsPairStage - 1) / kRowsPairStage;
+    for (int s = 0; s < stages; ++s) {
+        int8_t *buf = apanel[s & 1];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) *reinterpret_cast<v4i *>(buf + i * (kRowsThreads * 16) + tid * 16) = astage[i];
+        __syncthreads();
+        if (s + 1 < stages) load_stage(s + 1, astage);
+        const int kb_first = s * kRowsPairStage;
+        const int len = KB - kb_first < kRowsPairStage ? KB - kb_first : kRowsPairStage;  // (a multiple of 4)
+        v4i a0 = *reinterpret_cast<const v4i *>(buf + voff);
+        v4i a1 = *reinterpret_cast<const v4i *>(buf + kRowsPairStage * 1024 + voff);
+        for (int kl = 0; kl < len; kl += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int nxt = kl + u + 1 < kRowsPairStage ? kl + u + 1 : kRowsPairStage - 1;
+                const v4i n0 = *reinterpret_cast<const v4i *>(buf + nxt * 1024 + voff);
+                const v4i n1 = *reinterpret_cast<const v4i *>(buf + (kRowsPairStage + nxt) * 1024 + voff);
+                const int kb = kb_first + kl + u;
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    const int slot = (u * NBW + jj) % D;
+                    acc[0][jj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, wf[slot], acc[0][jj], 0, 0, 0);
+                    acc[1][jj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, wf[slot], acc[1][jj], 0, 0, 0);
+                    wf[slot] = load_w(kb + (jj + D) / NBW, (jj + D) % NBW);
+                }
+                a0 = n0;
+                a1 = n1;
+            }
+        }
+    }
+
+    // ---- epilogue (see gemm_i8_rows_kernel; rows 32 * rbk + row_of(r), statistics for all 64 rows at once) ----
+    auto row_of = [&](int r) { return 8 * (r / 4) + 4 * half + (r % 4); };
+    auto value = [&](int rbk, int jj, int r) {
+        const int bits = acc[rbk][jj][r];
+        return __builtin_bit_cast(float, bits);
+    };
+    auto max_abs = [](float a, float b) {
+        float o;
+        asm("v_max_f32_e64 %0, %1, |%2|" : "=v"(o) : "v"(a), "v"(b));
+        return o;
+    };
+    auto partials_to_lds = [&](float(&t)[RB][16], int which, auto is_max) {
+#pragma unroll
+        for (int rbk = 0; rbk < RB; ++rbk)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) t[rbk][r] = half_wave_fold<decltype(is_max)::value>(t[rbk][r]);
+        if (cin == 0) {
+#pragma unroll
+            for (int rbk = 0; rbk < RB; ++rbk)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) red[which][wave][32 * rbk + row_of(r)] = t[rbk][r];
+        }
+        __syncthreads();
+    };
+    // Wave 0, one lane per row: this half's statistic of the row, then the pair's.
+    auto row_total = [&](int which, int round, auto is_max) {
+        constexpr bool MAX = decltype(is_max)::value;
+        float w[kRowsWaves];
+#pragma unroll
+        for (int k = 0; k < kRowsWaves; ++k) w[k] = red[which][k][tid];
+        const float local = MAX ? fmaxf(fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])), fmaxf(fmaxf(w[4], w[5]), fmaxf(w[6], w[7])))
+                                : ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
+        const size_t me = size_t(pair) * 2 + h, partner = size_t(pair) * 2 + (1 - h);
+        px.buf[(partner * 3 + round) * 64 + tid] = local;  // (a plain store: it lands in the XCD's L2)
+        asm volatile("" ::: "memory");
+        wait_vmcnt<0>();
+        asm volatile("" ::: "memory");
+        const uint32_t mine = 0x100u | xcc_id();
+        if (lane == 0) __hip_atomic_store(px.flags + partner * 4 + round, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t *flag = px.flags + me * 4 + round;
+        uint32_t seen = 0;
+        for (int spin = 0; spin <= px.spin_limit; ++spin) {
+            seen = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (seen != 0) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        seen = __builtin_amdgcn_readfirstlane(seen);
+        float other = MAX ? 0.0f : 0.0f;
+        if (seen == mine) {
+            asm volatile("" ::: "memory");
+            const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+                px.buf + (me * 3 + round) * 64, 0, 64 * 4, 0x00020000);
+            other = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, tid * 4, 0, /*sc1*/ 16));
+        } else if (lane == 0) {
+            // nothing came within the limit, or it came from another XCD, whose stores this L2 does not hold
+            __hip_atomic_store(px.wait_error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0 && seen != 0) __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if constexpr (MAX) return fmaxf(local, other);
+        return h == 0 ? local + other : other + local;
+    };
+    auto from_lds = [&](float(&t)[16], int which, int rbk) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) t[r] = fin[which][32 * rbk + row_of(r)];
+    };
+    const int KBo = p.N / 32;
+    const int qd = lane % 4;
+    const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
+    const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+    const int qoff = (4 * half + qd + 32 * (cin / 16)) * 16 + 4 * ((cin / 4) % 4);
+    const float cols_f = static_cast<float>(p.N);
+
+    // v = acc * (s_a * s_w) + bias (+ residual) (GELU), in place
+    float sum[RB][16], am[RB][16];
+#pragma unroll
+    for (int rbk = 0; rbk < RB; ++rbk) {
+        float s_row[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + 32 * rbk + row_of(r);
+            s_row[r] = p.sa[p.sa_per_row ? (m < p.M ? m : p.M - 1) : 0];
+            sum[rbk][r] = am[rbk][r] = 0.0f;
+        }
+#pragma unroll
+        for (int jj = 0; jj < NBW; ++jj) {
+            if (!mine_block(jj)) continue;  // (wave-uniform)
+            const int col = (jb0 + jj) * 32 + cin;
+            const float swv = p.sw[col];
+            const float bv = p.bias ? p.bias[col] : -0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = static_cast<float>(acc[rbk][jj][r]) * (s_row[r] * swv) + bv;
+                if constexpr (RESID) {
+                    if constexpr (RES_EARLY)
+                        v = v + res_all[rbk][jj][r];
+                    else
+                        v = v + load_x(rbk, jj, r);
+                }
+                if constexpr (EPI == RP_GELU_Q) {
+                    v = rp_gelu_tanh(v);
+                    am[rbk][r] = max_abs(am[rbk][r], v);
+                }
+                if constexpr (EPI == RP_F32 || RESID)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v), rf, (4 * half * p.N + col) * 4,
+                                                          (32 * rbk + 8 * (r / 4) + (r % 4)) * row_bytes,
+                                                          EPI == RP_F32 ? 2 : 0);
+                if constexpr (EPI == RP_RESID_LN_Q) sum[rbk][r] += v;
+                acc[rbk][jj][r] = __builtin_bit_cast(int, v);
+            }
+        }
+    }
+    if constexpr (QUANT) {
+        if constexpr (EPI == RP_RESID_LN_Q) {
+            partials_to_lds(sum, 0, std::false_type{});
+            if (wave == 0) fin[0][tid] = row_total(0, 0, std::false_type{}) / cols_f;
+            __syncthreads();
+            float sq[RB][16];
+#pragma unroll
+            for (int rbk = 0; rbk < RB; ++rbk) {
+                float mean[16];
+                from_lds(mean, 0, rbk);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sq[rbk][r] = 0.0f;
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    if (!mine_block(jj)) continue;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float d = value(rbk, jj, r) - mean[r];
+                        sq[rbk][r] += d * d;
+                    }
+                }
+            }
+            partials_to_lds(sq, 1, std::false_type{});
+            if (wave == 0) fin[1][tid] = 1.0f / sqrtf(row_total(1, 1, std::false_type{}) / cols_f + p.eps);
+            __syncthreads();
+#pragma unroll
+            for (int rbk = 0; rbk < RB; ++rbk) {
+                float mean[16], rstd[16];
+                from_lds(mean, 0, rbk);
+                from_lds(rstd, 1, rbk);
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    if (!mine_block(jj)) continue;
+                    const int col = (jb0 + jj) * 32 + cin;
+                    const float g = p.gamma ? p.gamma[col] : 1.0f, b = p.beta ? p.beta[col] : -0.0f;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float y = (value(rbk, jj, r) - mean[r]) * rstd[r] * g + b;
+                        am[rbk][r] = max_abs(am[rbk][r], y);
+                        acc[rbk][jj][r] = __builtin_bit_cast(int, y);
+                    }
+                }
+            }
+        }
+        partials_to_lds(am, 2, std::true_type{});
+        if (wave == 0) {
+            const float a = row_total(2, 2, std::true_type{});
+            float sc = a < FLT_EPSILON ? 1.0f : a / 127.0f;
+            if (!(fabsf(a) <= FLT_MAX)) sc = NAN;
+            if (m0 + tid < p.M) {
+                if (h == 0) p.out_scales[m0 + tid] = sc;
+            } else {
+                sc = NAN;  // rows past M: codes 0
+            }
+            fin[2][tid] = sc;
+            fin[3][tid] = 1.0f / sc;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int rbk = 0; rbk < RB; ++rbk) {
+            float scale[16], inv[16];
+            from_lds(scale, 2, rbk);
+            from_lds(inv, 3, rbk);
+            const bool there = rb0 + rbk < rbA;  // (the packed output has no row block past the matrix)
+            const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
+                p.out_q + size_t(there ? rb0 + rbk : 0) * KBo * 1024, 0, there ? KBo * 1024 : 0, 0x00020000);
+#pragma unroll
+            for (int jj = 0; jj < NBW; ++jj) {
+                if (!mine_block(jj)) continue;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    int q[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int r = 4 * g + k;
+                        const float x = value(rbk, jj, r);
+                        const float q0 = x * inv[r];
+                        const float t = fmaf(fmaf(-q0, scale[r], x), inv[r], q0);
+                        q[k] = min(max(cvt_i32_sat(round_mode<EVEN>(t)), -128), 127);
+                    }
+                    const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));
+                    const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
+                    const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
+                    const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
+                    const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
+                    const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                    __builtin_amdgcn_raw_buffer_store_b32(static_cast<int>(word), rq, qoff, (jb0 + jj) * 1024 + g * 128, 0);
+                }
+            }
+        }
+    }
+}
+
+// The pair form where it applies and pays: the device's workgroup pairs share an XCD, the whole grid is resident at
+// once (one workgroup per compute unit of the context's share), N a multiple of 64 and at most 3072.  An exchange
+// of row statistics costs about 5 us (the partners meet, so it includes their skew), which the halved weight stream
+// pays back when all eight waves have columns to work on (N >= 1536) and, for the three exchanges of a LayerNorm,
+// when the matrix is large (N * K >= 2 Mi).  At M = 8192, K = 768 (3072 for N = 768), pairs against single panels,
+// in us: fp32 11.0 / 11.7 (N = 768), 18.3 / 21.9 (1536), 28.9 / 32.1 (2304), 35.9 / 43.6 (3072), 26.1 / 29.8
+// (768 x 3072); GELU + quantize 15.8 / 13.8, 22.4 / 24.0, 37.9 / 37.2, 40.1 / 48.4, 33.3 / 31.8; skip + LayerNorm +
+// quantize 38.4 / 38.1 (1536), 60.8 / 60.7 (2304), 95.3 / 112.9 (3072), 43.6 / 41.2 (768 x 3072).
+// Test hook 15 keeps the single-workgroup panels.  Returns false when the caller should launch those.
+template <int EPI>
+static bool launch_rows_pair(hipq_ctx *ctx, const RowPanel &p, bool even, int32_t *rc) {
+    const int share = ctx->resident_share > 0 ? ctx->resident_share : 1;
+    const int pairs = (p.M + 63) / 64, grid = (pairs + 7) / 8 * 16;
+    if (!ctx->pair_ok || ctx->gemm_variant == 15 || p.N % 64 != 0 || p.M <= 32 || grid > ctx->num_cus / share) return false;
+    if ((EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q) && p.N < 1536) return false;
+    if (EPI == RP_RESID_LN_Q && size_t(p.N) * p.K < (size_t(2) << 20)) return false;
+    RowPairExchange px;
+    int8_t *buf = nullptr;
+    *rc = pair_area(ctx, size_t(grid) * 4 * sizeof(uint32_t), size_t(grid) * 3 * 64 * sizeof(float), &px.flags, &buf);
+    if (*rc) return true;
+    px.buf = reinterpret_cast<float *>(buf);
+    px.wait_error = ctx->wait_error;
+    px.spin_limit = ctx->wait_spin_limit;
+    const int nbw = (p.N / 64 + kRowsWaves - 1) / kRowsWaves;
+#define HIPQ_LAUNCH_ROWS_PAIR(NBW)                                                                                        \
+    do {                                                                                                                  \
+        if (even)                                                                                                         \
+            hipLaunchKernelGGL((gemm_i8_rows_pair_kernel<NBW, EPI, true>), dim3(grid), dim3(kRowsThreads), 0, ctx->stream, \
+                               p, px);                                                                                    \
+        else                                                                                                              \
+            hipLaunchKernelGGL((gemm_i8_rows_pair_kernel<NBW, EPI, false>), dim3(grid), dim3(kRowsThreads), 0,            \
+                               ctx->stream, p, px);                                                                       \
+    } while (0)
+    if (nbw <= 2)
+        HIPQ_LAUNCH_ROWS_PAIR(2);
+    else if (nbw <= 3)
+        HIPQ_LAUNCH_ROWS_PAIR(3);
+    else
+        HIPQ_LAUNCH_ROWS_PAIR(6);
+#undef HIPQ_LAUNCH_ROWS_PAIR
+    *rc = check_launch("gemm_i8 (row panels, pairs)");
+    return true;
+}
+
 // Launch of the row-panel kernel: one workgroup of eight waves per 32 rows.  Returns HIPQ_SHAPE_ERROR for what it
 // does not take (N not a multiple of 32 or above 3072; the *_Q forms: N not a multiple of 128).
 template <int EPI>
@@ -413,6 +808,10 @@ static int32_t launch_rows(hipq_ctx *ctx, const RowPanel &p, bool even) {
     // (offsets of column blocks past N, which read as zeros, are still computed: price the widest panel)
     if (packed_bytes(size_t(3072), size_t(p.K)) >= (size_t(1) << 31))
         return fail(HIPQ_SHAPE_ERROR, "row-panel GEMM: K = %d is too large (32-bit offsets into the weights)", p.K);
+    {
+        int32_t rc = HIPQ_SUCCESS;
+        if (launch_rows_pair<EPI>(ctx, p, even, &rc)) return rc;
+    }
     const dim3 grid((p.M + 31) / 32);
     const int nbw = (p.N / 32 + kRowsWaves - 1) / kRowsWaves;
 #define HIPQ_LAUNCH_ROWS_NBW(NBW)                                                                                     \
