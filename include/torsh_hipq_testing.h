@@ -31,7 +31,8 @@ extern "C" {
  * gather their own patches of the image into LDS (measured no faster than the layout pass + implicit
  * GEMM it would replace; kept as a measured alternative); 15 makes the row-panel forwards (the
  * Linear forwards with a row operation in their epilogue) keep one workgroup per 32 rows where they
- * would let two workgroups of an XCD share 64 rows and half of the columns each. */
+ * would let two workgroups of an XCD share 64 rows and half of the columns each; 16 makes them take
+ * such pairs wherever the shape allows it, also where the single panels were measured faster. */
 HIPQ_API int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant);
 /* Some kernels couple their waves through device memory: the persistent GEMM kernel (counters
  * between producer and consumer waves), the one-launch dynamic quantizers (their workgroups meet to

@@ -168,8 +168,13 @@ def test_row_panel_shapes_that_are_refused(ctx, hipq):
 PAIR_SHAPES = [(8192, 3072, 768), (97, 3072, 768), (70, 1536, 1600), (40, 2048, 1056), (200, 2304, 1024), (33, 1664, 96)]
 
 
-@pytest.mark.parametrize("m,n,k", PAIR_SHAPES)
-def test_pair_panels_equal_single_panels(hipq, m, n, k):
+# shapes whose quantizing forms keep single panels by default (narrow outputs: waves without columns), with the
+# pair form forced (test hook 16)
+FORCED_PAIR_SHAPES = [(100, 256, 96), (257, 768, 800), (65, 768, 3072), (130, 1280, 64), (8192, 768, 768)]
+
+
+@pytest.mark.parametrize("m,n,k,pairs", [s + (0,) for s in PAIR_SHAPES] + [s + (16,) for s in FORCED_PAIR_SHAPES])
+def test_pair_panels_equal_single_panels(hipq, m, n, k, pairs):
     """The row-panel kernels in their pair form (two workgroups of one XCD share 64 rows and take half of the columns
     each; row maxima and sums cross through the XCD's L2) against the single-workgroup panels (test hook 15): the fp32
     product, the skip connection, GELU + per-token int8 bit for bit, the LayerNorm form within the bound that holds
@@ -198,7 +203,7 @@ def test_pair_panels_equal_single_panels(hipq, m, n, k):
 
         c.set_gemm_kernel_variant(15)
         single = forms()
-        c.set_gemm_kernel_variant(0)
+        c.set_gemm_kernel_variant(pairs)
         for _ in range(2):
             pair = forms()
             for i in (0, 1, 2, 3, 6):

@@ -231,8 +231,8 @@ int32_t hipq_ctx_synchronize(hipq_ctx *ctx) {
 
 int32_t hipq_set_gemm_kernel_variant(hipq_ctx *ctx, int32_t variant) {
     HIPQ_REQUIRE_PTR(ctx);
-    if (variant < 0 || variant > 15 || variant == 13)
-        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not one of 0..12, 14, 15", __func__, variant);
+    if (variant < 0 || variant > 16 || variant == 13)
+        return hipq::fail(HIPQ_INVALID_ARGUMENT, "%s: variant %d is not one of 0..12, 14..16", __func__, variant);
     ctx->gemm_variant = variant;
     return HIPQ_SUCCESS;
 }

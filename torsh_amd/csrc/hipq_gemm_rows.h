@@ -754,20 +754,30 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
 
 // The pair form where it applies and pays: the device's workgroup pairs share an XCD, the whole grid is resident at
 // once (one workgroup per compute unit of the context's share), N a multiple of 64 and at most 3072.  An exchange
-// of row statistics costs about 5 us (the partners meet, so it includes their skew), which the halved weight stream
-// pays back when all eight waves have columns to work on (N >= 1536) and, for the three exchanges of a LayerNorm,
+// of row statistics costs about 2 us, and a workgroup's epilogue handles twice the rows, which the halved weight
+// stream pays back when all eight waves have columns to work on (N >= 1536) and, for the three exchanges of a LayerNorm,
 // when the matrix is large (N * K >= 2 Mi).  At M = 8192, K = 768 (3072 for N = 768), pairs against single panels,
 // in us: fp32 11.0 / 11.7 (N = 768), 18.3 / 21.9 (1536), 28.9 / 32.1 (2304), 35.9 / 43.6 (3072), 26.1 / 29.8
 // (768 x 3072); GELU + quantize 15.8 / 13.8, 22.4 / 24.0, 37.9 / 37.2, 40.1 / 48.4, 33.3 / 31.8; skip + LayerNorm +
-// quantize 38.4 / 38.1 (1536), 60.8 / 60.7 (2304), 95.3 / 112.9 (3072), 43.6 / 41.2 (768 x 3072).
-// Test hook 15 keeps the single-workgroup panels.  Returns false when the caller should launch those.
+// quantize 38.4 / 38.1 (1536), 60.8 / 60.7 (2304), 95.3 / 112.9 (3072), 43.6 / 41.2 (768 x 3072); skip alone 14.8 /
+// 15.8 (768), 32.8 / 36.1 (768 x 3072), 76.2 / 57.0 (3072: the stream is then read inside the epilogue, value by
+// value, by waves that hold twice the rows).  With the waits switched off (spin limit 0) the times are the same to
+// 0.5 us: what an exchange costs is its own chain of L2 trips (store, acknowledge, flag, poll, read), not the
+// partners' skew.  Raising the issue priority of one of the two waves of every SIMD during the main loop, so that
+// its epilogue would overlap the other's loads and MFMAs, changes nothing (41.6 / 41.7 us at N = 3072 with GELU +
+// quantize): the waves advance at the rate their loads return.
+// Test hook 15 keeps the single-workgroup panels, 16 takes pairs wherever the shape allows them.  Returns false
+// when the caller should launch the single panels.
 template <int EPI>
 static bool launch_rows_pair(hipq_ctx *ctx, const RowPanel &p, bool even, int32_t *rc) {
     const int share = ctx->resident_share > 0 ? ctx->resident_share : 1;
     const int pairs = (p.M + 63) / 64, grid = (pairs + 7) / 8 * 16;
     if (!ctx->pair_ok || ctx->gemm_variant == 15 || p.N % 64 != 0 || p.M <= 32 || grid > ctx->num_cus / share) return false;
-    if ((EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q) && p.N < 1536) return false;
-    if (EPI == RP_RESID_LN_Q && size_t(p.N) * p.K < (size_t(2) << 20)) return false;
+    if (ctx->gemm_variant != 16) {
+        if ((EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q) && p.N < 1536) return false;
+        if (EPI == RP_RESID_F32 && p.N > 1536) return false;
+        if (EPI == RP_RESID_LN_Q && size_t(p.N) * p.K < (size_t(2) << 20)) return false;
+    }
     RowPairExchange px;
     int8_t *buf = nullptr;
     *rc = pair_area(ctx, size_t(grid) * 4 * sizeof(uint32_t), size_t(grid) * 3 * 64 * sizeof(float), &px.flags, &buf);
