@@ -254,6 +254,64 @@ def test_pair_panels_give_up_cleanly(hipq):
         c.close()
 
 
+def test_captured_pair_panels_replay(hipq):
+    """The exchange between the two workgroups of a panel keeps no host state per launch and leaves its flags at
+    zero, so a captured MLP (fc1 + GELU + quantizer, fc2 + skip + LayerNorm + quantizer, both as pairs) can be
+    replayed: every replay, with new inputs in the captured buffers and eager work on the same context in between,
+    equals the eager forwards of the same inputs."""
+    m, d, dff = 200, 256, 1024
+    g = torch.Generator(device="cuda").manual_seed(21)
+    w1 = torch.randint(-128, 128, (dff, d), generator=g, device="cuda", dtype=torch.int8)
+    w2 = torch.randint(-128, 128, (d, dff), generator=g, device="cuda", dtype=torch.int8)
+    s1 = torch.rand(dff, generator=g, device="cuda") * 2e-3 + 1e-4
+    s2 = torch.rand(d, generator=g, device="cuda") * 2e-3 + 1e-4
+    b1 = torch.randn(dff, generator=g, device="cuda")
+    b2 = torch.randn(d, generator=g, device="cuda")
+    gamma = torch.rand(d, generator=g, device="cuda") + 0.5
+    beta = torch.randn(d, generator=g, device="cuda") * 0.1
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        c = hipq.Context(0)
+        try:
+            c.set_gemm_kernel_variant(16)
+            p1, p2 = c.pack_rows(w1), c.pack_rows(w2)
+            a = torch.randint(-128, 128, (m, d), generator=g, device="cuda", dtype=torch.int8)
+            pa = c.pack_rows(a)
+            sa = torch.rand(m, generator=g, device="cuda") * 0.02 + 0.001
+            x = torch.randn(m, d, generator=g, device="cuda")
+
+            def mlp(pa_, sa_, x_, hq=None, hs=None, oq=None, os_=None):
+                hq, hs = c.linear_gelu_quantize_packed(pa_, sa_, p1, s1, b1, m, dff, d, out=hq, scales=hs)
+                return (hq, hs) + tuple(c.linear_residual_layer_norm_quantize_packed(
+                    hq, hs, p2, s2, b2, m, d, dff, x_, gamma, beta, out=oq, scales=os_))
+
+            bufs = mlp(pa, sa, x.clone())  # allocates the exchange area outside the capture
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                mlp(pa, sa, x, *bufs)
+            for rep in range(6):
+                an = torch.randint(-128, 128, (m, d), generator=g, device="cuda", dtype=torch.int8)
+                xn = torch.randn(m, d, generator=g, device="cuda") * (rep + 1)
+                pa.copy_(c.pack_rows(an))
+                x.copy_(xn)
+                side.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                got = [t.clone() for t in bufs] + [x.clone()]
+                xe = xn.clone()
+                eager = list(mlp(c.pack_rows(an), sa, xe)) + [xe]
+                side.synchronize()
+                for i, (u, v) in enumerate(zip(got, eager)):
+                    assert torch.equal(u.view(torch.int32) if u.dtype == torch.float32 else u,
+                                       v.view(torch.int32) if v.dtype == torch.float32 else v), (rep, i)
+            c.synchronize()  # no exchange gave up
+        finally:
+            torch.cuda.synchronize()
+            c.close()
+
+
 # ---- the projection stack on prepared weights ---------------------------------------------------------------
 
 from test_gpu_stack import _make_blocks, _oracle_stack  # noqa: E402
