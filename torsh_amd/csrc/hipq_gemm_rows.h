@@ -766,6 +766,12 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
 // partners' skew.  Raising the issue priority of one of the two waves of every SIMD during the main loop, so that
 // its epilogue would overlap the other's loads and MFMAs, changes nothing (41.6 / 41.7 us at N = 3072 with GELU +
 // quantize): the waves advance at the rate their loads return.
+// Halving K instead of the columns between the partners (each multiplies both row blocks by its half of the weights,
+// then every wave hands the partial sums of the partner's row block - 12 KiB a wave, 96 KiB a workgroup - to the
+// partner's wave of the same columns and adds what it receives; integer sums, so bit-identical whatever the
+// epilogue) was built for N <= 768 and measured: 36.7 against 32.9 us (fp32) and 44.2 against 43.0 us (skip +
+// LayerNorm + quantize) at 768 x 3072, 21.6 against 12.8 us at 768 x 768.  The exchange of 24 MB through the L2s
+// costs ~9 us, more than the halved weight stream saves (~5 us at K = 3072).
 // Test hook 15 keeps the single-workgroup panels, 16 takes pairs wherever the shape allows them.  Returns false
 // when the caller should launch the single panels.
 template <int EPI>
