@@ -333,6 +333,20 @@ def vector_memory_path_table(ctx) -> int:
         pops = mfmas * 65536.0 * 4 * steps * wgs / wall / 1e15
         print(f"{wgs:10d} {source:>22s} {share:5d} {loads:5d} {mfmas:5d} {steps:5d} {cyc.median().item() / steps:11.1f} "
               f"{ticks.median().item() * 10.0 / steps:8.1f} {bpc:9.1f} {ghz:5.2f} {tbs:6.2f} {pops:6.2f}")
+    # Range check of raw buffer accesses (hipq_probe_buffer_range_check): lane l of one wave loads the dword at byte
+    # 4 l + soffset of a descriptor of 4096 bytes, then stores a marker there; the memory behind is 1 MiB of 0x11.
+    print("\nraw buffer descriptor of 4096 bytes, lane l at byte 4 l + scalar offset: lanes whose load saw memory / "
+          "whose store landed")
+    mem = torch.empty(1 << 18, dtype=torch.int32, device="cuda")
+    loaded = torch.empty(64, dtype=torch.int32, device="cuda")
+    for soff in (0, 3968, 4096, 8192, 65536, (1 << 20) - 256):
+        mem.fill_(0x11111111)
+        ctx.call("hipq_probe_buffer_range_check", mem.data_ptr(), mem.numel() * 4, 4096, soff, loaded.data_ptr())
+        ctx.synchronize()
+        seen = int((loaded == 0x11111111).sum())
+        zeros = int((loaded == 0).sum())
+        landed = int((mem[soff // 4:soff // 4 + 64] == 0x7777).sum())
+        print(f"  scalar offset {soff:8d}: loads {seen:2d} of 64 saw memory, {zeros:2d} read zero; stores {landed:2d} of 64 landed")
     return 0
 
 

@@ -64,6 +64,14 @@ HIPQ_API int32_t hipq_probe_vector_memory_path(hipq_ctx *ctx, const int8_t *buf,
                                                int32_t region_bytes, int32_t share, int32_t loads_per_step,
                                                int32_t mfmas_per_step, int32_t steps, uint64_t *out);
 
+/* Machine probe: one wave accesses a raw buffer descriptor of `extent` bytes over `mem` with the scalar offset
+ * `soffset`: lane l loads the dword at byte 4 l + soffset into loaded[l] (64 x int32, device), then stores 0x7777
+ * there.  The row-panel GEMM kernels rely on accesses past the extent reading as zero and being dropped, scalar
+ * offset included; every address the wave could reach must lie inside mem (soffset + 256 <= mem_bytes), so the
+ * probe is safe whatever the hardware does. */
+HIPQ_API int32_t hipq_probe_buffer_range_check(hipq_ctx *ctx, int32_t *mem, size_t mem_bytes, int32_t extent,
+                                               int32_t soffset, int32_t *loaded);
+
 #ifdef __cplusplus
 }
 #endif

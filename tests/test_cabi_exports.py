@@ -38,7 +38,8 @@ def test_python_binding_covers_the_header():
 
     assert sorted(hipq.exported_symbols()) == sorted(_declared_symbols() + _test_hooks())
     assert _test_hooks() == ["hipq_ctx_set_trace_buffer", "hipq_ctx_set_wait_spin_limit",
-                             "hipq_probe_vector_memory_path", "hipq_set_gemm_kernel_variant"]
+                             "hipq_probe_buffer_range_check", "hipq_probe_vector_memory_path",
+                             "hipq_set_gemm_kernel_variant"]
     assert not set(_test_hooks()) & set(_declared_symbols())
 
 

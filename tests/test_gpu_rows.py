@@ -163,6 +163,25 @@ def test_row_panel_shapes_that_are_refused(ctx, hipq):
     ctx.linear_rows_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), 0, 96, 32, out=torch.empty((0, 96), device="cuda"))
 
 
+def test_buffer_accesses_past_the_extent_are_checked_with_the_scalar_offset(ctx):
+    """The row-panel kernels give their buffer descriptors exact extents and rely on the hardware for what lies past
+    them (column blocks past N, k blocks past K, rows past M), with the distance in the SCALAR offset of the access:
+    such loads must give zeros and such stores must be dropped, lane by lane.  The probe keeps every address it could
+    reach inside one allocation, so it is safe on hardware that checked less."""
+    mem = torch.empty(1 << 18, dtype=torch.int32, device="cuda")
+    loaded = torch.empty(64, dtype=torch.int32, device="cuda")
+    for soff, inside in ((0, 64), (3968, 32), (4096, 0), (8192, 0), (65536, 0), ((1 << 20) - 256, 0)):
+        mem.fill_(0x11111111)
+        ctx.call("hipq_probe_buffer_range_check", mem.data_ptr(), mem.numel() * 4, 4096, soff, loaded.data_ptr())
+        ctx.synchronize()
+        got = host(loaded)
+        assert (got[:inside] == 0x11111111).all() and (got[inside:] == 0).all(), (soff, got)
+        window = host(mem[soff // 4:soff // 4 + 64])
+        assert (window[:inside] == 0x7777).all() and (window[inside:] == 0x11111111).all(), (soff, window)
+    with pytest.raises(Exception):  # an access the allocation would not cover is refused by the host
+        ctx.call("hipq_probe_buffer_range_check", mem.data_ptr(), mem.numel() * 4, 4096, 1 << 20, loaded.data_ptr())
+
+
 # ---- panels of 64 rows shared by a pair of compute units ------------------------------------------------------
 
 PAIR_SHAPES = [(8192, 3072, 768), (97, 3072, 768), (70, 1536, 1600), (40, 2048, 1056), (200, 2304, 1024), (33, 1664, 96)]

@@ -81,9 +81,34 @@ __global__ __launch_bounds__(256, 2) void probe_vector_memory_kernel(const int8_
     }
 }
 
+// What the hardware does with a raw buffer access whose scalar offset, alone or together with the lane's offset,
+// reaches past the descriptor's extent.  The row-panel GEMM kernels give their descriptors exact extents and lean on
+// the answer (loads give zeros and touch no memory, stores are dropped) for column blocks past N, k blocks past K and
+// rows past M, so a test holds the device at hand to it.  One wave: lane l loads the dword at byte 4 l + soffset of a
+// descriptor of `extent` bytes over `mem`, then stores 0x7777 there.
+__global__ __launch_bounds__(kWave) void probe_range_check_kernel(int *mem, int extent, int soffset, int *loaded) {
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(mem, 0, extent, 0x00020000);
+    const int lane = threadIdx.x;
+    loaded[lane] = __builtin_amdgcn_raw_buffer_load_b32(r, lane * 4, soffset, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(0x7777, r, lane * 4, soffset, 0);
+}
+
 }  // namespace hipq
 
 using namespace hipq;
+
+extern "C" int32_t hipq_probe_buffer_range_check(hipq_ctx *ctx, int32_t *mem, size_t mem_bytes, int32_t extent,
+                                                 int32_t soffset, int32_t *loaded) {
+    HIPQ_ENTER(ctx);
+    HIPQ_REQUIRE_PTR(mem);
+    HIPQ_REQUIRE_PTR(loaded);
+    // every address the wave could reach if nothing were checked lies inside the caller's allocation
+    if (extent < 0 || soffset < 0 || size_t(extent) > mem_bytes || size_t(soffset) + kWave * 4 > mem_bytes)
+        return fail(HIPQ_INVALID_ARGUMENT, "%s: extent and soffset + 256 must lie within the %zu bytes of mem", __func__,
+                    mem_bytes);
+    hipLaunchKernelGGL(probe_range_check_kernel, dim3(1), dim3(kWave), 0, ctx->stream, mem, extent, soffset, loaded);
+    return check_launch("probe_range_check");
+}
 
 extern "C" int32_t hipq_probe_vector_memory_path(hipq_ctx *ctx, const int8_t *buf, size_t buf_bytes, int32_t workgroups,
                                                  int32_t region_bytes, int32_t share, int32_t loads_per_step,

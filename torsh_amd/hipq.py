@@ -126,6 +126,7 @@ _SIGNATURES = {
     "hipq_ctx_set_resident_share": [_vp, _i32],
     "hipq_ctx_set_trace_buffer": [_vp, _vp, _sz],
     "hipq_probe_vector_memory_path": [_vp, _vp, _sz, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+    "hipq_probe_buffer_range_check": [_vp, _vp, _sz, _i32, _i32, _vp],
     "hipq_linear_static_f32": [_vp, _vp, _f32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp],
     "hipq_layer_norm_quantize_f32_i8": [_vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
     "hipq_add_layer_norm_quantize_f32_i8": [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _f32, _i32, _vp, _vp],
