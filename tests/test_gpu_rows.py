@@ -144,6 +144,25 @@ def test_linear_residual_layer_norm_quantize(ctx, oracle, m, n, k, affine):
     np.testing.assert_array_equal(bits(x_res), bits(x_parts))
 
 
+@pytest.mark.parametrize("m,n,k", [(65, 768, 3072), (97, 3072, 768)])
+def test_linear_residual_layer_norm_quantize_half_even(ctx, hipq, m, n, k):
+    """The same comparison with codes rounded half to even (single panels and pairs)."""
+    rng = np.random.default_rng(m + n + k)
+    a, w, sa, sw, b = operands(rng, m, n, k)
+    x0 = rng.standard_normal((m, n)).astype(np.float32)
+    gamma, beta = rng.uniform(0.5, 1.5, n).astype(np.float32), (rng.standard_normal(n) * 0.1).astype(np.float32)
+    pa, pw = ctx.pack_rows(dev(a)), ctx.pack_rows(dev(w))
+    f = ctx.linear_packed_i8_f32(pa, dev(sa), pw, dev(sw), dev(b), m, n, k)
+    x_parts, x_one = dev(x0), dev(x0)
+    q, s = ctx.add_layer_norm_quantize(x_parts, f, dev(gamma), dev(beta), mode=hipq.ROUND_HALF_EVEN)
+    got_q, got_s = ctx.linear_residual_layer_norm_quantize_packed(pa, dev(sa), pw, dev(sw), dev(b), m, n, k, x_one,
+                                                                  dev(gamma), dev(beta), mode=hipq.ROUND_HALF_EVEN)
+    np.testing.assert_array_equal(bits(x_one), bits(x_parts))
+    np.testing.assert_allclose(host(got_s), host(s), rtol=1e-6, atol=0)
+    diff = np.abs(unpack_reference(host(got_q), m, n).astype(np.int16) - host(q).astype(np.int16))
+    assert diff.max() <= 1 and (diff != 0).mean() <= 1e-5 + 2.0 / diff.size
+
+
 def test_row_panel_shapes_that_are_refused(ctx, hipq):
     rng = np.random.default_rng(1)
     a, w, sa, sw, b = operands(rng, 8, 3104, 32)

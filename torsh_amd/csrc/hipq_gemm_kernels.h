@@ -455,13 +455,12 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[FM][FN], const GemmEpilog
         if constexpr (EPI == EPI_I8) {
             // int8 output as dwords.  A lane holds one column of 16 rows; the four lanes of a quad
             // hold four consecutive columns.  Per group of four rows each lane packs its four
-            // bytes, the quad transposes the 4x4 bytes (four quad broadcasts + two byte
+            // bytes, the quad transposes the 4x4 bytes (quad_byte_transpose: two lane swaps, two byte
             // permutes), and every lane stores one dword = four consecutive columns of one row:
             // a quarter of the store instructions of the byte form, none of them sub-dword.
             if (N % 4 == 0 && (reinterpret_cast<uintptr_t>(ep.out) & 3u) == 0) {
                 const int qd = lane % 4;
-                const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
-                const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+                const uint32_t sel1 = (qd & 1) ? 0x03070105u : 0x06020400u, sel2 = (qd & 2) ? 0x03020706u : 0x05040100u;
 #pragma unroll
                 for (int j = 0; j < FN; ++j) {
                     const int col = nn[j] - qd;  // first column of the quad; N % 4 == 0 keeps quads whole
@@ -474,12 +473,8 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[FM][FN], const GemmEpilog
                             if (has_bias) v = v + bv[j];
                             q[k] = clamp_to_int(round_mode<EVEN>(div_rn(v, ep.s_out, ep.s_out_inv)) + zpf, -128, 127);
                         }
-                        const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));  // byte k = row 8t + 4*(lane/32) + k
-                        const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
-                        const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
-                        const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
-                        const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
-                        const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                        // byte k of the packed dword = row 8t + 4*(lane/32) + k
+                        const uint32_t word = quad_byte_transpose(pack4(q[0], q[1], q[2], q[3]), sel1, sel2);
                         const int m = mrow0 + i * 32 + 8 * t + 4 * (lane / 32) + qd;
                         if (m < M && col < N)
                             __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(static_cast<int8_t *>(ep.out) +

@@ -88,6 +88,18 @@ __device__ __forceinline__ float half_wave_fold(float v) {
     return combine(v, __builtin_bit_cast(float, other));
 }
 
+// The code of a value t = x / scale whose scale is its own row's max|x| / 127: round (ties away from zero, or to
+// even) and convert.  v_cvt_i32_f32 truncates, so the ties-away form round_mode<0> = truncf(t + copysign(pred(0.5), t))
+// needs no truncf of its own; |t| <= 127 (1 + 2^-22), so the result lies in [-127, 127] without a clamp; a NaN (a NaN
+// element, or any element of a row whose scale is NaN: an infinity in the row, a row past M) converts to 0.
+template <bool EVEN>
+__device__ __forceinline__ int row_code(float t) {
+    if constexpr (EVEN)
+        return cvt_i32_sat(rintf(t));
+    else
+        return cvt_i32_sat(t + copysignf(0x1.fffffep-2f, t));
+}
+
 constexpr int rows_gcd(int a, int b) { return b == 0 ? a : rows_gcd(b, a % b); }
 
 template <int NBW, int EPI, bool EVEN>
@@ -256,8 +268,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
     const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
         QUANT ? p.out_q + size_t(rb) * KBo * 1024 : nullptr, 0, QUANT ? KBo * 1024 : 0, 0x00020000);
     const int qd = lane % 4;
-    const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
-    const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+    const uint32_t sel1 = (qd & 1) ? 0x03070105u : 0x06020400u, sel2 = (qd & 2) ? 0x03020706u : 0x05040100u;
     // after the byte exchange below a lane holds row 8 g + 4 half + qd, columns 4 * (cin / 4) .. + 3 of a block
     const int qoff = (4 * half + qd + 32 * (cin / 16)) * 16 + 4 * ((cin / 4) % 4);
     const float cols_f = static_cast<float>(p.N);
@@ -370,8 +381,8 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
             from_lds(inv, 3, g0);
             // The codes, in the packed layout of the next product's activations: row block rb, k block = column
             // block, and inside the 1 KiB fragment slot (row + 32 * (column / 16)) of 16 bytes.  A lane holds one
-            // column of four consecutive rows per register group; the four lanes of a quad exchange bytes (four
-            // quad broadcasts, two byte permutes) so that each holds four consecutive columns of ONE row: a dword.
+            // column of four consecutive rows per register group; the four lanes of a quad transpose their 4 x 4
+            // bytes (quad_byte_transpose) so that each holds four consecutive columns of ONE row: a dword.
 #pragma unroll
             for (int jj = 0; jj < NBW; ++jj) {
                 if (jb0 + jj >= nblocks) continue;
@@ -385,14 +396,10 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
                         const float x = value(jj, 4 * g0 + i);
                         const float q0 = x * inv[i];
                         const float t = fmaf(fmaf(-q0, scale[i], x), inv[i], q0);
-                        q[k] = min(max(cvt_i32_sat(round_mode<EVEN>(t)), -128), 127);
+                        q[k] = row_code<EVEN>(t);
                     }
-                    const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));  // byte k = row 8 g + 4 half + k
-                    const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
-                    const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
-                    const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
-                    const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
-                    const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                    // byte k of the packed dword = row 8 g + 4 half + k; after the transpose: this lane's row, 4 columns
+                    const uint32_t word = quad_byte_transpose(pack4(q[0], q[1], q[2], q[3]), sel1, sel2);
                     __builtin_amdgcn_raw_buffer_store_b32(static_cast<int>(word), rq, qoff,
                                                           (jb0 + jj) * 1024 + (g0 + gi) * 128, 0);
                 }
@@ -615,8 +622,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
     };
     const int KBo = p.N / 32;
     const int qd = lane % 4;
-    const uint32_t sel_lo = 0x0c0c0000u | (uint32_t(4 + qd) << 8) | uint32_t(qd);
-    const uint32_t sel_hi = (uint32_t(4 + qd) << 24) | (uint32_t(qd) << 16) | 0x0c0cu;
+    const uint32_t sel1 = (qd & 1) ? 0x03070105u : 0x06020400u, sel2 = (qd & 2) ? 0x03020706u : 0x05040100u;
     const int qoff = (4 * half + qd + 32 * (cin / 16)) * 16 + 4 * ((cin / 4) % 4);
     const float cols_f = static_cast<float>(p.N);
 
@@ -737,14 +743,9 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
                         const float x = value(rbk, jj, r);
                         const float q0 = x * inv[r];
                         const float t = fmaf(fmaf(-q0, scale[r], x), inv[r], q0);
-                        q[k] = min(max(cvt_i32_sat(round_mode<EVEN>(t)), -128), 127);
+                        q[k] = row_code<EVEN>(t);
                     }
-                    const int d = static_cast<int>(pack4(q[0], q[1], q[2], q[3]));
-                    const uint32_t x0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x00, 0xf, 0xf, false));
-                    const uint32_t x1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0x55, 0xf, 0xf, false));
-                    const uint32_t x2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xaa, 0xf, 0xf, false));
-                    const uint32_t x3 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, d, 0xff, 0xf, 0xf, false));
-                    const uint32_t word = __builtin_amdgcn_perm(x1, x0, sel_lo) | __builtin_amdgcn_perm(x3, x2, sel_hi);
+                    const uint32_t word = quad_byte_transpose(pack4(q[0], q[1], q[2], q[3]), sel1, sel2);
                     __builtin_amdgcn_raw_buffer_store_b32(static_cast<int>(word), rq, qoff, (jb0 + jj) * 1024 + g * 128, 0);
                 }
             }

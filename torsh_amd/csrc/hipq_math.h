@@ -181,6 +181,17 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
     return lo | hi;
 }
 
+// 4 x 4 byte transpose inside a quad of lanes: lane q holds bytes (row 0..3) of column q and ends with the bytes
+// (column 0..3) of row q.  Two butterfly steps - swap with lane q ^ 1 and interleave bytes, swap with lane q ^ 2 and
+// interleave halves - each a data-parallel move and a byte permute whose selector depends on the lane:
+// sel1 = q & 1 ? 0x03070105 : 0x06020400, sel2 = q & 2 ? 0x03020706 : 0x05040100.
+__device__ __forceinline__ uint32_t quad_byte_transpose(uint32_t d, uint32_t sel1, uint32_t sel2) {
+    const uint32_t p1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(d), 0xB1, 0xf, 0xf, true));
+    const uint32_t t = __builtin_amdgcn_perm(p1, d, sel1);
+    const uint32_t p2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(t), 0x4E, 0xf, 0xf, true));
+    return __builtin_amdgcn_perm(p2, t, sel2);
+}
+
 __device__ __forceinline__ float wave_min(float v) {
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
