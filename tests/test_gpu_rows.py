@@ -1,6 +1,6 @@
-"""Parity of the row-panel Linear forwards (a workgroup owns 32 whole rows of the output and applies the row
-operation that follows the Linear - per-token quantizer, GELU, skip connection, LayerNorm - to its accumulators)
-and of the projection stack built from them.
+"""Parity of the row-panel Linear forwards (a workgroup owns 32 whole rows of the output - or two workgroups of one
+XCD share 64 rows, half of the columns each - and applies the row operation that follows the Linear - per-token
+quantizer, GELU, skip connection, LayerNorm - to its accumulators) and of the projection stack built from them.
 
 What is bit-exact and what is not:
   * the fp32 product, the skip connection and GELU + per-token int8 perform, per element, the f32 operations of
