@@ -113,7 +113,7 @@ def test_config4_full_size_against_direct_kernel_and_torch(ctx, hipq):
 
 
 def test_config4_full_size_packed_requant_forward(ctx, hipq):
-    """BASELINE configs[3] at full size through the entry point the bench times (layout pass, packed filters,
+    """The Conv2d benchmark configuration at full size through the entry point the bench times (layout pass, packed filters,
     implicit GEMM, fused bias + requantize): every int8 output against the bytes re-derived, with torch's
     individually rounded f32 operations, from exact accumulators (float64 convolution, |acc| < 2^53); both
     roundings, a zero and a non-zero input zero point."""

@@ -408,7 +408,7 @@ def test_non_finite_activations_give_nan_outputs_not_stale_scratch(ctx, hipq, pa
 
 
 def test_config2_full_size_packed_forward(ctx, hipq):
-    """BASELINE configs[1] at full size through the packed forward the bench times: M=512, K=N=4096.  int8
+    """The headline Linear benchmark configuration at full size through the packed forward the bench times: M=512, K=N=4096.  int8
     activations against torch's formulation of clamp(round_half_away(x * (1/s))), accumulators against an exact
     float64 product, fp32 output against the same individually rounded f32 expression (1e-5 relative stated;
     equal in practice), and the row-major entry point against the packed one."""
