@@ -433,7 +433,7 @@ constexpr int kRowsPairStage = kRowsStage / 2;  // k blocks per LDS buffer and r
 template <int NBW, int EPI, bool EVEN>
 __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPanel p, RowPairExchange px) {
     constexpr int RB = 2;
-    constexpr int D = NBW == 2 ? 8 : (NBW == 3 ? 12 : 6);  // weight fragments in flight per wave
+    constexpr int D = NBW == 2 || NBW == 4 ? 8 : (NBW == 3 ? 12 : (NBW == 5 ? 10 : 6));  // weight fragments in flight per wave
     constexpr int U = D / rows_gcd(NBW, D);                // k blocks per trip of the main loop
     static_assert((U * NBW) % D == 0 && 4 % U == 0, "ring slots must be static; stages are multiples of 4 k blocks");
     constexpr bool QUANT = EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q;
@@ -450,19 +450,22 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
     const int KB = static_cast<int>(packed_k_blocks(p.K));  // (a multiple of 4)
     const int nblocks = p.N / 32, nb2 = nblocks / 2;
     const int rbA = (p.M + 31) / 32, rb0 = pair * 2;
-    const int jl0 = wave * NBW;         // this wave's column blocks within the half: jl0 .. jl0 + NBW - 1
-    const int jb0 = h * nb2 + jl0;      // ... and within the matrix
-    auto mine_block = [&](int jj) { return jl0 + jj < nb2; };
+    // This wave's column blocks within the half: wave, wave + 8, wave + 16, ... (dealt round the waves, so that a
+    // width that is no multiple of eight blocks leaves no wave idle), and within the matrix: jb(jj).
+    auto mine_block = [&](int jj) { return wave + kRowsWaves * jj < nb2; };
+    auto jb = [&](int jj) { return h * nb2 + wave + kRowsWaves * jj; };
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t *>(p.pa) + size_t(rb0) * KB * 1024, 0, (rbA - rb0 < 2 ? 1 : 2) * KB * 1024, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(p.pw), 0, nblocks * KB * 1024, 0x00020000);
     const int voff = lane * 16;
     const int wstride = KB * 1024;
-    // (a wave without columns asks beyond the matrix: zeros, no memory access)
-    const int wbase = jl0 < nb2 ? jb0 * wstride : 0x7fffffff - 64 * 1024 * 1024;
+    // (a block this wave does not have asks beyond the matrix: zeros, no memory access)
+    int woff[NBW];
+#pragma unroll
+    for (int jj = 0; jj < NBW; ++jj) woff[jj] = mine_block(jj) ? jb(jj) * wstride : 0x7fffffff - 64 * 1024 * 1024;
     auto load_w = [&](int kb, int jj) {
-        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, wbase + jj * wstride + kb * 1024, 0));
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, woff[jj] + kb * 1024, 0));
     };
     // one stage of the activation panel: 12 k blocks of both row blocks, three 16-byte pieces per thread
     int aoff[3];
@@ -484,7 +487,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
     const int row_bytes = p.N * 4;
     auto load_x = [&](int rbk, int jj, int r) {
         return __builtin_bit_cast(
-            float, __builtin_amdgcn_raw_buffer_load_b32(rf, (4 * half * p.N + (jb0 + jj) * 32 + cin) * 4,
+            float, __builtin_amdgcn_raw_buffer_load_b32(rf, (4 * half * p.N + jb(jj) * 32 + cin) * 4,
                                                         (32 * rbk + 8 * (r / 4) + (r % 4)) * row_bytes, 0));
     };
     // touch this workgroup's thirty-second of the weights (see gemm_i8_rows_kernel)
@@ -640,7 +643,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
 #pragma unroll
         for (int jj = 0; jj < NBW; ++jj) {
             if (!mine_block(jj)) continue;  // (wave-uniform)
-            const int col = (jb0 + jj) * 32 + cin;
+            const int col = jb(jj) * 32 + cin;
             const float swv = p.sw[col];
             const float bv = p.bias ? p.bias[col] : -0.0f;
 #pragma unroll
@@ -698,7 +701,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
 #pragma unroll
                 for (int jj = 0; jj < NBW; ++jj) {
                     if (!mine_block(jj)) continue;
-                    const int col = (jb0 + jj) * 32 + cin;
+                    const int col = jb(jj) * 32 + cin;
                     const float g = p.gamma ? p.gamma[col] : 1.0f, b = p.beta ? p.beta[col] : -0.0f;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
@@ -746,7 +749,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
                         q[k] = row_code<EVEN>(t);
                     }
                     const uint32_t word = quad_byte_transpose(pack4(q[0], q[1], q[2], q[3]), sel1, sel2);
-                    __builtin_amdgcn_raw_buffer_store_b32(static_cast<int>(word), rq, qoff, (jb0 + jj) * 1024 + g * 128, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(static_cast<int>(word), rq, qoff, jb(jj) * 1024 + g * 128, 0);
                 }
             }
         }
@@ -758,7 +761,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_pair_kernel(RowPane
 // of row statistics costs about 2 us, and a workgroup's epilogue handles twice the rows, which the halved weight
 // stream pays back when all eight waves have columns to work on (N >= 1536) and, for the three exchanges of a LayerNorm,
 // when the matrix is large (N * K >= 2 Mi).  At M = 8192, K = 768 (3072 for N = 768), pairs against single panels,
-// in us: fp32 11.0 / 11.7 (N = 768), 18.3 / 21.9 (1536), 28.9 / 32.1 (2304), 35.9 / 43.6 (3072), 26.1 / 29.8
+// in us: fp32 11.0 / 11.7 (N = 768), 18.3 / 21.9 (1536), 26.6 / 32.1 (2304), 35.9 / 43.6 (3072), 26.1 / 29.8
 // (768 x 3072); GELU + quantize 15.8 / 13.8, 22.4 / 24.0, 37.9 / 37.2, 40.1 / 48.4, 33.3 / 31.8; skip + LayerNorm +
 // quantize 38.4 / 38.1 (1536), 60.8 / 60.7 (2304), 95.3 / 112.9 (3072), 43.6 / 41.2 (768 x 3072); skip alone 14.8 /
 // 15.8 (768), 32.8 / 36.1 (768 x 3072), 76.2 / 57.0 (3072: the stream is then read inside the epilogue, value by
@@ -802,12 +805,21 @@ static bool launch_rows_pair(hipq_ctx *ctx, const RowPanel &p, bool even, int32_
             hipLaunchKernelGGL((gemm_i8_rows_pair_kernel<NBW, EPI, false>), dim3(grid), dim3(kRowsThreads), 0,            \
                                ctx->stream, p, px);                                                                       \
     } while (0)
-    if (nbw <= 2)
+    constexpr bool QUANT = EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q;
+    if (nbw <= 2) {
         HIPQ_LAUNCH_ROWS_PAIR(2);
-    else if (nbw <= 3)
+    } else if (nbw <= 3) {
         HIPQ_LAUNCH_ROWS_PAIR(3);
-    else
+    } else if (nbw <= 5 && !QUANT) {  // (the quantizing forms of these widths run with six, one or two blocks of zeros)
+        if constexpr (!QUANT) {
+            if (nbw == 4)
+                HIPQ_LAUNCH_ROWS_PAIR(4);
+            else
+                HIPQ_LAUNCH_ROWS_PAIR(5);
+        }
+    } else {
         HIPQ_LAUNCH_ROWS_PAIR(6);
+    }
 #undef HIPQ_LAUNCH_ROWS_PAIR
     *rc = check_launch("gemm_i8 (row panels, pairs)");
     return true;
