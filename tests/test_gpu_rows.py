@@ -350,6 +350,54 @@ def test_captured_pair_panels_replay(hipq):
             c.close()
 
 
+def test_pair_panels_on_two_contexts_that_share_the_device(hipq):
+    """Two contexts that were told about each other (hipq_ctx_set_resident_share(ctx, 2)) size the shared panels for
+    half of the device each: 4096 rows take the pair form on both at once (both grids are resident together, so no
+    exchange waits for a workgroup that cannot start), 8192 rows no longer fit a context's share and take single
+    panels.  Same bits as one context alone; no wait gives up."""
+    m, n, k = 4096, 3072, 768
+    g = torch.Generator(device="cuda").manual_seed(31)
+    a = torch.randint(-128, 128, (2 * m, k), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    sa = torch.rand(2 * m, generator=g, device="cuda") * 0.02 + 0.001
+    sw = torch.rand(n, generator=g, device="cuda") * 2e-3 + 1e-4
+    b = torch.randn(n, generator=g, device="cuda")
+    alone = hipq.Context(0)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ctxs = []
+    try:
+        pw = alone.pack_rows(w)
+        pas = [alone.pack_rows(a[i * m:(i + 1) * m]) for i in range(2)]
+        want = [alone.linear_gelu_quantize_packed(pas[i], sa[i * m:(i + 1) * m], pw, sw, b, m, n, k) for i in range(2)]
+        pa_all = alone.pack_rows(a)
+        want_all = alone.linear_gelu_quantize_packed(pa_all, sa, pw, sw, b, 2 * m, n, k)
+        alone.synchronize()
+        torch.cuda.synchronize()
+        for s_ in streams:
+            with torch.cuda.stream(s_):
+                c = hipq.Context(0)
+                c.call("hipq_ctx_set_resident_share", 2)
+                ctxs.append(c)
+        for rep in range(5):
+            got = []
+            for i, (c, s_) in enumerate(zip(ctxs, streams)):
+                with torch.cuda.stream(s_):
+                    got.append(c.linear_gelu_quantize_packed(pas[i], sa[i * m:(i + 1) * m], pw, sw, b, m, n, k))
+            for c in ctxs:
+                c.synchronize()  # (would report an exchange that gave up)
+            for i in range(2):
+                assert torch.equal(got[i][0], want[i][0]) and torch.equal(got[i][1], want[i][1]), (rep, i)
+        with torch.cuda.stream(streams[0]):
+            big = ctxs[0].linear_gelu_quantize_packed(pa_all, sa, pw, sw, b, 2 * m, n, k)
+        ctxs[0].synchronize()
+        assert torch.equal(big[0], want_all[0]) and torch.equal(big[1], want_all[1])
+    finally:
+        torch.cuda.synchronize()
+        for c in ctxs:
+            c.close()
+        alone.close()
+
+
 # ---- the projection stack on prepared weights ---------------------------------------------------------------
 
 from test_gpu_stack import _make_blocks, _oracle_stack  # noqa: E402
