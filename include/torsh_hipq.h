@@ -518,6 +518,17 @@ HIPQ_API int32_t hipq_linear_residual_layer_norm_quantize_packed_i8(
     hipq_ctx *ctx, const int8_t *a_packed, const float *a_scale, int32_t a_scale_per_row, const int8_t *w_packed,
     const float *w_scales, const float *bias, size_t m, size_t n, size_t k, float *x, const float *gamma,
     const float *beta, float eps, int32_t mode, int8_t *out_packed, float *out_scales);
+/* The same forward from fp32 activations a [m, k] (rows lda floats apart, 16-byte aligned, k and lda multiples of
+ * 4): every workgroup first quantizes its own 32 rows per token, symmetric int8 (quantize_per_channel_auto on axis
+ * 0, algorithms.rs:126-242: hipq_quantize_per_row_packed_f32_i8 with HIPQ_PARAMS_SYMMETRIC; `mode` rounds these
+ * codes and the output's alike) and keeps the codes on chip, so the quantizer's launch and its packed output are
+ * gone.  Same bits as hipq_quantize_per_row_packed_f32_i8 (on the rows, dense) followed by the entry point above.
+ * k <= 1536 and n <= 1536 (the panel of codes and the accumulators of a workgroup), n % 32 == 0 (% 128 with
+ * out_packed); other shapes: HIPQ_SHAPE_ERROR, use the two calls. */
+HIPQ_API int32_t hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8(
+    hipq_ctx *ctx, const float *a, size_t lda, const int8_t *w_packed, const float *w_scales, const float *bias,
+    size_t m, size_t n, size_t k, float *x, const float *gamma, const float *beta, float eps, int32_t mode,
+    int8_t *out_packed, float *out_scales);
 
 /* ---- quantized elementwise operators of the backend trait --------------- */
 /* CpuQuantizationOps::qadd, crates/torsh-backend/src/quantization/ops.rs:582-606:
@@ -648,9 +659,10 @@ HIPQ_API int32_t hipq_transformer_stack_forward_f32(hipq_ctx *ctx, const hipq_bl
                                                     size_t tokens, size_t d_model, size_t d_ff, float eps,
                                                     int32_t mode, float *x, void *workspace, size_t workspace_bytes);
 /* The same forward on PREPARED weights: every w_* of `blocks` points to the packed form of the [out, in] matrix
- * (hipq_pack_rows_i8, once, when the model is converted).  Five kernels per layer: each Linear that feeds a row
+ * (hipq_pack_rows_i8, once, when the model is converted).  Four kernels per layer: each Linear that feeds a row
  * operation applies it in its epilogue (hipq_linear_residual_layer_norm_quantize_packed_i8,
- * hipq_linear_gelu_quantize_packed_i8), and int8 activations stay packed between them.  x is what
+ * hipq_linear_gelu_quantize_packed_i8), the out-projection quantizes the fp32 value slice itself
+ * (hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8), and int8 activations stay packed between them.  x is what
  * hipq_transformer_stack_forward_f32 computes up to the fold order of the LayerNorm sums (see those entry
  * points).  d_model and d_ff: multiples of 128, at most 3072 (else HIPQ_SHAPE_ERROR: use the form above). */
 HIPQ_API size_t hipq_transformer_stack_prepared_workspace_bytes(size_t tokens, size_t d_model, size_t d_ff);

@@ -201,6 +201,70 @@ def test_buffer_accesses_past_the_extent_are_checked_with_the_scalar_offset(ctx)
         ctx.call("hipq_probe_buffer_range_check", mem.data_ptr(), mem.numel() * 4, 4096, 1 << 20, loaded.data_ptr())
 
 
+# ---- the same forward from fp32 rows: the per-token quantizer inside the kernel -------------------------------
+
+FROM_F32_SHAPES = [(8192, 768, 768, 2304), (100, 256, 96, 96), (33, 128, 1536, 1600), (257, 1536, 800, 2400),
+                   (40, 1024, 64, 64), (1, 128, 4, 8)]  # m, n, k, row pitch of the activations
+
+
+@pytest.mark.parametrize("m,n,k,lda", FROM_F32_SHAPES)
+@pytest.mark.parametrize("mode", [0, 1])
+def test_linear_from_f32_rows_equals_the_quantizer_then_the_linear(ctx, hipq, m, n, k, lda, mode):
+    """hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8 (every workgroup quantizes its own 32 fp32 rows per
+    token and keeps the codes on chip) against hipq_quantize_per_row_packed_f32_i8 on a dense copy of the rows and
+    the forward on packed activations: the stream, the codes and the scales bit for bit, with and without the
+    LayerNorm.  Rows that are a slice of a wider matrix; a NaN element; a row holding an infinity (NaN scale, zero
+    codes: its outputs are NaN in both)."""
+    g = torch.Generator(device="cuda").manual_seed(m * 7 + n + k + mode)
+    rmode = hipq.ROUND_HALF_EVEN if mode else 0
+    a_full = torch.randn(m, lda, generator=g, device="cuda") * 1.7
+    a = a_full[:, lda - k:]
+    a[m // 2, k // 3] = float("nan")
+    if m > 8:
+        a[5, k - 1] = float("inf")
+    w = torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    sw = torch.rand(n, generator=g, device="cuda") * 2e-3 + 1e-4
+    b = torch.randn(n, generator=g, device="cuda")
+    gamma = torch.rand(n, generator=g, device="cuda") + 0.5
+    beta = torch.randn(n, generator=g, device="cuda") * 0.1
+    x0 = torch.randn(m, n, generator=g, device="cuda")
+    pw = ctx.pack_rows(w)
+    try:
+        ctx.set_gemm_kernel_variant(15)  # (the packed-activation forward on single panels, like the kernel under test)
+        qa, sa = ctx.quantize_per_row_packed(a.contiguous(), mode=rmode)
+        x_parts, x_res_parts = x0.clone(), x0.clone()
+        want_q, want_s = ctx.linear_residual_layer_norm_quantize_packed(qa, sa, pw, sw, b, m, n, k, x_parts, gamma, beta,
+                                                                        mode=rmode)
+        ctx.linear_residual_layer_norm_quantize_packed(qa, sa, pw, sw, b, m, n, k, x_res_parts, normalize=False)
+    finally:
+        ctx.set_gemm_kernel_variant(0)
+    x_one, x_res = x0.clone(), x0.clone()
+    got_q, got_s = ctx.linear_from_f32_residual_layer_norm_quantize_packed(a, pw, sw, b, n, x_one, gamma, beta,
+                                                                           mode=rmode)
+    ctx.linear_from_f32_residual_layer_norm_quantize_packed(a, pw, sw, b, n, x_res, mode=rmode, normalize=False)
+    np.testing.assert_array_equal(bits(x_one), bits(x_parts))
+    np.testing.assert_array_equal(bits(x_res), bits(x_res_parts))
+    np.testing.assert_array_equal(bits(got_s), bits(want_s))
+    np.testing.assert_array_equal(host(got_q), host(want_q))
+
+
+def test_linear_from_f32_rows_shapes_that_are_refused(ctx, hipq):
+    g = torch.Generator(device="cuda").manual_seed(4)
+    def call(m, n, k, lda, off=0):
+        a = torch.randn(m * lda + 8, generator=g, device="cuda")[off:off + m * lda].view(m, lda)[:, :k]
+        w = ctx.pack_rows(torch.randint(-128, 128, (n, k), generator=g, device="cuda", dtype=torch.int8))
+        sw = torch.rand(n, generator=g, device="cuda")
+        x = torch.zeros(m, n, device="cuda")
+        return ctx.linear_from_f32_residual_layer_norm_quantize_packed(a, w, sw, None, n, x)
+    for args in ((8, 128, 1540, 1540), (8, 1664, 64, 64), (8, 128, 62, 64), (8, 128, 64, 66), (8, 128, 64, 64, 1),
+                 (8, 96, 64, 64)):
+        with pytest.raises(hipq.HipqError) as e:
+            call(*args)
+        assert e.value.code == hipq.SHAPE_ERROR, args
+    call(8, 128, 64, 64)
+    ctx.synchronize()
+
+
 # ---- panels of 64 rows shared by a pair of compute units ------------------------------------------------------
 
 PAIR_SHAPES = [(8192, 3072, 768), (97, 3072, 768), (70, 1536, 1600), (40, 2048, 1056), (200, 2304, 1024), (33, 1664, 96)]

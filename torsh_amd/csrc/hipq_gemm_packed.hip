@@ -418,4 +418,28 @@ int32_t hipq_linear_residual_layer_norm_quantize_packed_i8(hipq_ctx *ctx, const 
     return launch_rows<RP_RESID_LN_Q>(ctx, p, (mode & HIPQ_ROUND_HALF_EVEN) != 0);
 }
 
+int32_t hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8(hipq_ctx *ctx, const float *a, size_t lda,
+                                                                    const int8_t *w_packed, const float *w_scales,
+                                                                    const float *bias, size_t m, size_t n, size_t k,
+                                                                    float *x, const float *gamma, const float *beta,
+                                                                    float eps, int32_t mode, int8_t *out_packed,
+                                                                    float *out_scales) {
+    HIPQ_ENTER(ctx);
+    int32_t rc = check_rows_args(__func__, ctx, m, n, k);
+    if (rc) return rc;
+    if (mode & ~HIPQ_ROUND_HALF_EVEN) return fail(HIPQ_INVALID_ARGUMENT, "%s: unknown mode bits", __func__);
+    if (lda >= (size_t(1) << 31)) return fail(HIPQ_SHAPE_ERROR, "%s: row pitch %zu is too large", __func__, lda);
+    if (m == 0 || n == 0) return HIPQ_SUCCESS;
+    HIPQ_REQUIRE_PTR(a);
+    HIPQ_REQUIRE_PTR(w_packed);
+    HIPQ_REQUIRE_PTR(w_scales);
+    HIPQ_REQUIRE_PTR(x);
+    RowPanel p{nullptr, nullptr, 1, w_packed, w_scales, bias, static_cast<int>(m), static_cast<int>(n),
+               static_cast<int>(k), x, out_packed, out_scales, gamma, beta, eps, a, static_cast<int>(lda)};
+    const bool even = (mode & HIPQ_ROUND_HALF_EVEN) != 0;
+    if (!out_packed) return launch_rows_from_f32<RP_RESID_F32>(ctx, p, even);
+    HIPQ_REQUIRE_PTR(out_scales);
+    return launch_rows_from_f32<RP_RESID_LN_Q>(ctx, p, even);
+}
+
 }  // extern "C"

@@ -45,6 +45,8 @@ struct RowPanel {
     float *out_scales;  // *_Q: [M]
     const float *gamma, *beta;  // RP_RESID_LN_Q: [N] or null
     float eps;
+    const float *af;    // fp32 activations [M, K], rows lda floats apart (the kernels that quantize them themselves)
+    int lda;
 };
 
 constexpr int kRowsWaves = 8;
@@ -102,7 +104,13 @@ __device__ __forceinline__ int row_code(float t) {
 
 constexpr int rows_gcd(int a, int b) { return b == 0 ? a : rows_gcd(b, a % b); }
 
-template <int NBW, int EPI, bool EVEN>
+// AF32: the activations are fp32 rows (p.af, p.lda) and the workgroup quantizes its own 32 of them first, per token
+// and symmetric, with the per-row quantizer's arithmetic (quantize_per_row_kernel: range by NaN-skipping min / max,
+// params_from_minmax, division form; a row whose range is not finite gets a NaN scale and zero codes): a wave reads
+// four rows, finds their ranges by shuffles, and writes the codes into LDS in fragment order, where the whole panel
+// stays (K <= 1536) and the main loop reads it.  The quantizer's launch, its packed output and its scales are gone;
+// the results are those of the two calls, bit for bit.
+template <int NBW, int EPI, bool EVEN, bool AF32 = false>
 __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) {
     constexpr int D = NBW <= 6 ? 12 : (NBW == 9 ? 9 : 6);  // weight fragments in flight per wave
     constexpr int U = D / rows_gcd(NBW, D);  // k blocks per trip of the main loop: U * NBW is a multiple of D
@@ -116,6 +124,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
     __shared__ __attribute__((aligned(1024))) int8_t apanel[2][kRowsStage * 1024];
     __shared__ __attribute__((aligned(16))) float red[3][kRowsWaves][32];  // [statistic][wave][row]: partial sums / maxima
     __shared__ __attribute__((aligned(16))) float fin[4][32];              // per row: mean, 1 / std, scale, 1 / scale
+    __shared__ float sa_own[AF32 ? 32 : 1];                                // AF32: the rows' activation scales
     const int tid = threadIdx.x, lane = tid % kWave, half = lane / 32, cin = lane % 32;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int rb = blockIdx.x, m0 = rb * 32;
@@ -177,7 +186,57 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
 #pragma unroll
     for (int u = 0; u < D; ++u) wf[u] = load_w(u / NBW, u % NBW);
     v4i astage[3];
-    load_stage(0, astage);
+    if constexpr (!AF32) load_stage(0, astage);
+    if constexpr (AF32) {
+        // rows 4 wave .. 4 wave + 3 of the panel: lane l holds floats 4 (l + 64 i) .. + 3 of each
+        constexpr int kMaxVec = 6;  // K <= 1536
+        int8_t *panel = &apanel[0][0];
+        const int kpad = KB * 32;
+        float4 v[4][kMaxVec];
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int m = m0 + 4 * wave + rr;
+            const float4 *row = reinterpret_cast<const float4 *>(p.af + size_t(m < p.M ? m : 0) * p.lda);
+#pragma unroll
+            for (int i = 0; i < kMaxVec; ++i) {
+                const int k = 4 * (lane + kWave * i);
+                if (m < p.M && k < p.K) v[rr][i] = row[lane + kWave * i];
+            }
+        }
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int m = m0 + 4 * wave + rr;
+            float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < kMaxVec; ++i) {
+                const int k = 4 * (lane + kWave * i);
+                if (m < p.M && k < p.K) {
+                    mn = fminf(mn, fminf(fminf(v[rr][i].x, v[rr][i].y), fminf(v[rr][i].z, v[rr][i].w)));
+                    mx = fmaxf(mx, fmaxf(fmaxf(v[rr][i].x, v[rr][i].y), fmaxf(v[rr][i].z, v[rr][i].w)));
+                }
+            }
+            mn = wave_min(mn);
+            mx = wave_max(mx);
+            float scale;
+            int zp;
+            const bool bad = params_from_minmax(mn, mx, HIPQ_PARAMS_SYMMETRIC, -128, 127, &scale, &zp) != HIPQ_SUCCESS;
+            if (lane == 0) sa_own[4 * wave + rr] = bad ? __builtin_nanf("") : scale;
+            if (bad) scale = INFINITY;  // x / inf: 0 for finite x, NaN -> code 0 otherwise
+            const float inv = recip_for_div(scale);
+            auto q = [&](float f) { return quantize_int<QFORM_DIV, EVEN>(f, scale, inv, 0.0f, -128, 127); };
+#pragma unroll
+            for (int i = 0; i < kMaxVec; ++i) {
+                const int k = 4 * (lane + kWave * i);
+                if (k < kpad) {  // (k past K up to the padded extent, rows past M: zeros)
+                    uint32_t w4 = 0u;
+                    if (m < p.M && k < p.K) w4 = pack4(q(v[rr][i].x), q(v[rr][i].y), q(v[rr][i].z), q(v[rr][i].w));
+                    *reinterpret_cast<uint32_t *>(panel + (k / 32) * 1024 + ((k % 32) / 16) * 512 + (4 * wave + rr) * 16 +
+                                                  (k % 16)) = w4;
+                }
+            }
+        }
+        __syncthreads();
+    }
     // Residual values: with few column blocks per wave all of them are requested here, ahead of the main loop,
     // which hides them completely (and keeps loads from queueing behind the epilogue's stores: one counter).
     constexpr bool RES_EARLY = RESID && GS == 4;
@@ -195,7 +254,25 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[j][r] = 0;
 
-    const int stages = (KB + kRowsStage - 1) / kRowsStage;
+    if constexpr (AF32) {
+        const int8_t *panel = &apanel[0][0];
+        v4i a_cur = *reinterpret_cast<const v4i *>(panel + voff);
+        for (int kl = 0; kl < KB; kl += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int nxt = kl + u + 1 < KB ? kl + u + 1 : KB - 1;
+                const v4i a_nxt = *reinterpret_cast<const v4i *>(panel + nxt * 1024 + voff);
+#pragma unroll
+                for (int jj = 0; jj < NBW; ++jj) {
+                    const int slot = (u * NBW + jj) % D;
+                    acc[jj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_cur, wf[slot], acc[jj], 0, 0, 0);
+                    wf[slot] = load_w(kl + u + (jj + D) / NBW, (jj + D) % NBW);
+                }
+                a_cur = a_nxt;
+            }
+        }
+    }
+    const int stages = AF32 ? 0 : (KB + kRowsStage - 1) / kRowsStage;
     for (int s = 0; s < stages; ++s) {
         int8_t *buf = apanel[s & 1];
         // (the last reads of this buffer, two stages ago, lie before the previous stage's barrier)
@@ -280,7 +357,10 @@ __global__ __launch_bounds__(kRowsThreads) void gemm_i8_rows_kernel(RowPanel p) 
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             const int m = m0 + row_of(4 * g0 + i);
-            s_row[i] = p.sa[p.sa_per_row ? (m < p.M ? m : p.M - 1) : 0];
+            if constexpr (AF32)
+                s_row[i] = sa_own[row_of(4 * g0 + i)];
+            else
+                s_row[i] = p.sa[p.sa_per_row ? (m < p.M ? m : p.M - 1) : 0];
         }
         // v = acc * (s_a * s_w) + bias (+ residual) (GELU), in place: the accumulator registers then hold float bits
         float sum[NR], am[NR];
@@ -823,6 +903,37 @@ static bool launch_rows_pair(hipq_ctx *ctx, const RowPanel &p, bool even, int32_
 #undef HIPQ_LAUNCH_ROWS_PAIR
     *rc = check_launch("gemm_i8 (row panels, pairs)");
     return true;
+}
+
+// Launch of the row-panel kernel that quantizes its own fp32 activations (gemm_i8_rows_kernel<.., AF32>): single
+// panels, the whole panel of codes resident in LDS.
+template <int EPI>
+static int32_t launch_rows_from_f32(hipq_ctx *ctx, const RowPanel &p, bool even) {
+    constexpr bool QUANT = EPI == RP_GELU_Q || EPI == RP_RESID_LN_Q;
+    if (p.N % 32 != 0 || p.N > 1536 || p.N <= 0 || p.M <= 0 || p.K <= 0 || (QUANT && p.N % 128 != 0))
+        return fail(HIPQ_SHAPE_ERROR,
+                    "row-panel GEMM from fp32 rows: N = %d must be a multiple of 32 (of 128 for a packed int8 output) "
+                    "and at most 1536", p.N);
+    if (p.K > 1536 || p.K % 4 != 0 || p.lda % 4 != 0 || p.lda < p.K || (reinterpret_cast<uintptr_t>(p.af) & 15u))
+        return fail(HIPQ_SHAPE_ERROR,
+                    "row-panel GEMM from fp32 rows: K = %d (at most 1536) and the row pitch %d must be multiples of 4, "
+                    "the rows 16-byte aligned", p.K, p.lda);
+    const dim3 grid((p.M + 31) / 32);
+    const int nbw = (p.N / 32 + kRowsWaves - 1) / kRowsWaves;
+#define HIPQ_LAUNCH_ROWS_F32(NBW)                                                                                         \
+    do {                                                                                                                  \
+        if (even)                                                                                                         \
+            hipLaunchKernelGGL((gemm_i8_rows_kernel<NBW, EPI, true, true>), grid, dim3(kRowsThreads), 0, ctx->stream, p); \
+        else                                                                                                              \
+            hipLaunchKernelGGL((gemm_i8_rows_kernel<NBW, EPI, false, true>), grid, dim3(kRowsThreads), 0, ctx->stream,    \
+                               p);                                                                                        \
+    } while (0)
+    if (nbw <= 3)
+        HIPQ_LAUNCH_ROWS_F32(3);
+    else
+        HIPQ_LAUNCH_ROWS_F32(6);
+#undef HIPQ_LAUNCH_ROWS_F32
+    return check_launch("gemm_i8 (row panels, fp32 activations)");
 }
 
 // Launch of the row-panel kernel: one workgroup of eight waves per 32 rows.  Returns HIPQ_SHAPE_ERROR for what it

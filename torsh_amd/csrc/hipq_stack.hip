@@ -155,13 +155,20 @@ int32_t hipq_transformer_stack_forward_prepared_f32(hipq_ctx *ctx, const hipq_bl
         else
             rc = hipq_linear_packed_i8_f32(ctx, qa, sa, 1, b.w_qkv, b.s_qkv, b.b_qkv, tokens, 3 * d_model, d_model, qkv);
         if (rc) return rc;
-        // Stand-in for the attention mixing, which is outside this path: the value slice passes through.
-        rc = hipq::quantize_activations_per_row_strided(ctx, qkv + 2 * d_model, tokens, d_model, 3 * d_model, round_bits,
-                                                        qb, sb, /*packed=*/true);
-        if (rc) return rc;
-        rc = hipq_linear_residual_layer_norm_quantize_packed_i8(ctx, qb, sb, 1, b.w_out, b.s_out, b.b_out, tokens,
-                                                                d_model, d_model, x, b.ln2_gamma, b.ln2_beta, eps,
-                                                                round_bits, qa, sa);
+        // Stand-in for the attention mixing, which is outside this path: the value slice passes through.  Its
+        // per-token quantizer runs inside the out-projection where a workgroup can hold its rows' codes on chip.
+        if (d_model <= 1536 && ctx->gemm_variant != 6) {
+            rc = hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8(
+                ctx, qkv + 2 * d_model, 3 * d_model, b.w_out, b.s_out, b.b_out, tokens, d_model, d_model, x, b.ln2_gamma,
+                b.ln2_beta, eps, round_bits, qa, sa);
+        } else {
+            rc = hipq::quantize_activations_per_row_strided(ctx, qkv + 2 * d_model, tokens, d_model, 3 * d_model,
+                                                            round_bits, qb, sb, /*packed=*/true);
+            if (rc) return rc;
+            rc = hipq_linear_residual_layer_norm_quantize_packed_i8(ctx, qb, sb, 1, b.w_out, b.s_out, b.b_out, tokens,
+                                                                    d_model, d_model, x, b.ln2_gamma, b.ln2_beta, eps,
+                                                                    round_bits, qa, sa);
+        }
         if (rc) return rc;
         // MLP half: x += W_fc2 * quant(GELU(W_fc1 * quant(LN2(x)))), then the next layer's quant(LN1(x))
         rc = hipq_linear_gelu_quantize_packed_i8(ctx, qa, sa, 1, b.w_fc1, b.s_fc1, b.b_fc1, tokens, d_ff, d_model,

@@ -137,6 +137,8 @@ _SIGNATURES = {
     "hipq_linear_gelu_quantize_packed_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _i32, _vp, _vp],
     "hipq_linear_residual_layer_norm_quantize_packed_i8": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp,
                                                            _vp, _f32, _i32, _vp, _vp],
+    "hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8": [_vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp,
+                                                                    _vp, _f32, _i32, _vp, _vp],
     "hipq_transformer_stack_forward_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
     "hipq_transformer_stack_forward_prepared_f32": [_vp, _vp, _sz, _sz, _sz, _sz, _f32, _i32, _vp, _vp, _sz],
     "hipq_qadd_u8": [_vp, _vp, _i32, _f32, _i32, _vp, _i32, _f32, _i32, _sz, _i32, _i32, _vp, _vp],
@@ -762,6 +764,24 @@ class Context:
         out = torch.empty((rows, cols), dtype=torch.int8, device=self._dev())
         scales = torch.empty(rows, dtype=torch.float32, device=self._dev())
         self.call("hipq_layer_norm_quantize_f32_i8", _ptr(x), rows, cols, _ptr(gamma), _ptr(beta), float(eps), mode,
+                  _ptr(out), _ptr(scales))
+        return out, scales
+
+    def linear_from_f32_residual_layer_norm_quantize_packed(self, a, w_packed, w_scales, bias, n, x, gamma=None,
+                                                            beta=None, eps=1e-5, mode=0, normalize=True, out=None,
+                                                            scales=None):
+        """The same from fp32 activations a [m, k] (a view whose rows may be further apart than k): the per-token
+        int8 quantizer of a runs inside the kernel."""
+        m, k = a.shape
+        assert a.stride(1) == 1
+        if normalize:
+            out = out if out is not None else torch.empty(self.packed_size(m, n), dtype=torch.int8,
+                                                          device=self._dev())
+            scales = scales if scales is not None else torch.empty(m, dtype=torch.float32, device=self._dev())
+        else:
+            out = scales = None
+        self.call("hipq_linear_from_f32_residual_layer_norm_quantize_packed_i8", a.data_ptr(), a.stride(0),
+                  _ptr(w_packed), _ptr(w_scales), _ptr(bias), m, n, k, _ptr(x), _ptr(gamma), _ptr(beta), float(eps), mode,
                   _ptr(out), _ptr(scales))
         return out, scales
 
